@@ -1,0 +1,136 @@
+/*
+ * kernl_hip.h — C ABI of libkernl_hip.so: hand-written gfx950 (CDNA4) kernels for the three fused
+ * transformer ops that kernl's graph rewriting swaps into a model.
+ *
+ * The reference (ELS-RD/kernl) has no FFI: its operator boundary is three Python callables that launch
+ * Triton kernels.  Each entry point below replaces the *launch* inside one of those callables; the Python
+ * host layer (kernl_amd/implementations/) keeps the reference's signatures, asserts and allocation
+ * rules and forwards raw pointers, sizes, strides and the current HIP stream to these functions.
+ *
+ * Common rules for every entry point
+ *   - plain pointers and integers only; all pointers are device pointers unless stated otherwise;
+ *   - asynchronous: work is enqueued on `stream` (a hipStream_t passed as void*; NULL = default stream)
+ *     and the call returns immediately — safe under hipGraph stream capture;
+ *   - no allocation, no host synchronisation, no retained pointers; re-entrant;
+ *   - returns KERNL_OK (0) or a negative kernl_status; kernl_last_error_string() gives the reason
+ *     (thread-local);
+ *   - strides are in ELEMENTS, not bytes.
+ */
+#ifndef KERNL_HIP_H
+#define KERNL_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    KERNL_OK = 0,
+    KERNL_ERR_INVALID_ARG = -1, /* NULL pointer, non-positive size, inconsistent broadcast sizes ... */
+    KERNL_ERR_UNSUPPORTED = -2, /* dtype / shape outside what the kernels implement                   */
+    KERNL_ERR_LAUNCH = -3       /* hipLaunchKernel reported an error                                   */
+} kernl_status;
+
+typedef enum { KERNL_F16 = 0, KERNL_BF16 = 1, KERNL_F32 = 2 } kernl_dtype;
+
+/* Epilogues of the fused linear layer.  Reference: src/kernl/implementations/activation_func.py:28-49
+ * ("tanh", "relu", "fast_gelu" = tanh approximation, "gelu" = erf form).  SILU is new (SwiGLU gate). */
+typedef enum {
+    KERNL_ACT_NONE = 0,
+    KERNL_ACT_RELU = 1,
+    KERNL_ACT_TANH = 2,
+    KERNL_ACT_GELU_ERF = 3,
+    KERNL_ACT_GELU_TANH = 4,
+    KERNL_ACT_SILU = 5
+} kernl_activation;
+
+/* Library version, MAJOR*10000 + MINOR*100 + PATCH. */
+int kernl_version(void);
+
+/* Reason for the last non-zero status returned on the calling thread ("" if none). */
+const char *kernl_last_error_string(void);
+
+/*
+ * Flash-attention forward:  out = softmax(q·kᵀ·sm_scale + causal + mask) · v, never materialising q·kᵀ.
+ * Replaces the `_fwd_kernel[grid](...)` launch of src/kernl/implementations/attention.py:499-528
+ * (kernel body :122-435).
+ *
+ *   q   [B,H,M,D]   k,v [B,H,N,D]   out [B,H,M,D]   — any strides (q_strides etc. = {batch, head, row, col});
+ *                    the MFMA path needs col stride 1 and 16-byte aligned rows, other layouts take a slower
+ *                    scalar kernel with identical semantics.
+ *   dtype           KERNL_F16 or KERNL_BF16 for q,k,v,out (reference asserts the same, attention.py:471-474).
+ *   mask            NULL, or an ADDITIVE mask of mask_dtype with sizes mask_sizes = {B|1, H|1, M|1, N}
+ *                   (size-1 batch/head dims broadcast; third size 1 = one value per key, else a full matrix;
+ *                   attention.py:311-323,349-385).  -inf entries are replaced by mask_min_clamp before the add
+ *                   (attention.py:380; the host passes finfo(mask dtype).min as the reference does, :516).
+ *   is_causal       non-zero: key n contributes to query m only if n <= m (top-left aligned, attention.py:346-347).
+ *   Softmax statistics and both accumulators are fp32; P is rounded to `dtype` before P·V (attention.py:424).
+ */
+int kernl_attention_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
+                        int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
+                        const int64_t q_strides[4], const int64_t k_strides[4],
+                        const int64_t v_strides[4], const int64_t o_strides[4],
+                        const int64_t mask_sizes[4], const int64_t mask_strides[4], int mask_dtype,
+                        float sm_scale, int is_causal, float mask_min_clamp, int dtype, void *stream);
+
+/*
+ * Fused linear layer:  out[M,N] = act(x[M,K] · w[N,K]ᵀ + bias[N]).
+ * Replaces the `kernel_fma[grid](...)` launch of src/kernl/implementations/linear_layer.py:254-278
+ * (kernel body :92-210).
+ *
+ *   x        [M,K] with strides x_strides = {row, col}; w [N,K] contiguous and bias [N] contiguous
+ *            (the reference asserts both, linear_layer.py:242-244); out [M,N] with out_strides.
+ *   act_in   NULL, or an [M,N] buffer with strides act_in_strides that receives x·wᵀ + bias BEFORE the
+ *            activation (linear_layer.py:193-195).
+ *   dtype    KERNL_F16 / KERNL_BF16 (MFMA path when x col stride is 1, K % 8 == 0 and rows are 16-byte
+ *            aligned) or KERNL_F32 (FMA path).  Accumulation is fp32; the activation is applied to the
+ *            fp32 accumulator (linear_layer.py:198-205).
+ */
+int kernl_linear_fwd(const void *x, const void *w, const void *bias, void *out, void *act_in,
+                     int64_t M, int64_t N, int64_t K,
+                     const int64_t x_strides[2], const int64_t out_strides[2],
+                     const int64_t act_in_strides[2], int activation, int dtype, void *stream);
+
+/*
+ * LayerNorm / RMSNorm forward over the last dimension of a 2-D view x[M,N].
+ * Replaces the `implementation[(M,)](...)` launch of src/kernl/implementations/layer_norm.py:314-331
+ * (kernel body :115-205).
+ *
+ *   LayerNorm: out = (x - mean) * rstd * w (+ bias),  rstd = 1/sqrt(biased_var + eps)
+ *   RMSNorm  (is_rms != 0): out = x * rstd * w (+ bias), rstd = 1/sqrt(mean(x²) + eps); mean is written as 0.
+ *   mean, rstd  NULL or fp32 [M] side outputs (layer_norm.py:186-187).
+ *   eps is used as given: the fp16 clamp max(eps, 1.6e-5) of layer_norm.py:295-296 is host-side policy.
+ *   Statistics are fp32; x is read from HBM once when a row fits the register-resident path
+ *   (col strides 1, N a multiple of 16 bytes / element size, N <= 8192 elements).
+ */
+int kernl_layernorm_fwd(const void *x, const void *w, const void *bias, void *out, float *mean,
+                        float *rstd, int64_t M, int64_t N, int64_t x_row_stride, int64_t x_col_stride,
+                        int64_t out_row_stride, int64_t out_col_stride, float eps, int is_rms, int dtype,
+                        void *stream);
+
+/*
+ * LayerNorm / RMSNorm of (x + residual), same arguments as kernl_layernorm_fwd plus `residual` [M,N]
+ * (strides res_row_stride/res_col_stride).  The sum is formed in fp32 and is not written back.
+ * No counterpart kernel in the reference, which leaves `x + residual` as a separate eager op in front of
+ * every LayerNorm (e.g. the graph in docs/how-to-guides/support-new-model.md:481-520).
+ */
+int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, const void *bias,
+                            void *out, float *mean, float *rstd, int64_t M, int64_t N,
+                            int64_t x_row_stride, int64_t x_col_stride, int64_t res_row_stride,
+                            int64_t res_col_stride, int64_t out_row_stride, int64_t out_col_stride,
+                            float eps, int is_rms, int dtype, void *stream);
+
+/*
+ * Test and tuning hooks (process-wide, not thread-safe; no counterpart in the reference).
+ *   kernl_linear_force_tile      0 = heuristic (default), 1 = 256x256, 2 = 256x192, 3 = 128x128 output tile
+ *                                of the MFMA linear kernel.
+ *   kernl_attention_force_scalar non-zero routes every attention call through the strided scalar kernel.
+ */
+void kernl_linear_force_tile(int which);
+void kernl_attention_force_scalar(int on);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KERNL_HIP_H */

@@ -1,0 +1,154 @@
+"""ctypes binding of libkernl_hip.so (C ABI: include/kernl_hip.h).
+
+The library is built in-tree by `kernl_amd/csrc/Makefile` (see `kernl_amd.build`).  There is no fallback:
+if the shared object is missing or a call fails, the error is raised to the caller.
+"""
+import ctypes
+import os
+from typing import Optional, Sequence
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libkernl_hip.so")
+_lib: Optional[ctypes.CDLL] = None
+
+KERNL_F16, KERNL_BF16, KERNL_F32 = 0, 1, 2
+DTYPE_CODE = {torch.float16: KERNL_F16, torch.bfloat16: KERNL_BF16, torch.float32: KERNL_F32}
+
+ACT_NONE, ACT_RELU, ACT_TANH, ACT_GELU_ERF, ACT_GELU_TANH, ACT_SILU = range(6)
+
+# every symbol declared in include/kernl_hip.h
+EXPORTED_SYMBOLS = (
+    "kernl_version",
+    "kernl_last_error_string",
+    "kernl_attention_fwd",
+    "kernl_linear_fwd",
+    "kernl_layernorm_fwd",
+    "kernl_add_layernorm_fwd",
+    "kernl_linear_force_tile",
+    "kernl_attention_force_scalar",
+)
+
+_i64 = ctypes.c_int64
+_vp = ctypes.c_void_p
+_i64p = ctypes.POINTER(ctypes.c_int64)
+
+
+class KernlLibraryError(RuntimeError):
+    pass
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Load (once) and return the shared library; raises KernlLibraryError if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise KernlLibraryError(
+            f"{_LIB_PATH} not found: build it with `python -m kernl_amd.build` (needs hipcc, targets gfx950)"
+        )
+    lib = ctypes.CDLL(_LIB_PATH)
+    lib.kernl_version.restype = ctypes.c_int
+    lib.kernl_version.argtypes = []
+    lib.kernl_last_error_string.restype = ctypes.c_char_p
+    lib.kernl_last_error_string.argtypes = []
+    lib.kernl_attention_fwd.restype = ctypes.c_int
+    lib.kernl_attention_fwd.argtypes = (
+        [_vp] * 5 + [_i64] * 5 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, _vp]
+    )
+    lib.kernl_linear_fwd.restype = ctypes.c_int
+    lib.kernl_linear_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
+    lib.kernl_layernorm_fwd.restype = ctypes.c_int
+    lib.kernl_layernorm_fwd.argtypes = [_vp] * 6 + [_i64] * 6 + [ctypes.c_float, ctypes.c_int, ctypes.c_int, _vp]
+    lib.kernl_add_layernorm_fwd.restype = ctypes.c_int
+    lib.kernl_add_layernorm_fwd.argtypes = [_vp] * 7 + [_i64] * 8 + [ctypes.c_float, ctypes.c_int, ctypes.c_int, _vp]
+    lib.kernl_linear_force_tile.restype = None
+    lib.kernl_linear_force_tile.argtypes = [ctypes.c_int]
+    lib.kernl_attention_force_scalar.restype = None
+    lib.kernl_attention_force_scalar.argtypes = [ctypes.c_int]
+    _lib = lib
+    return lib
+
+
+def _arr(values: Sequence[int]):
+    return (ctypes.c_int64 * len(values))(*values)
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        msg = load().kernl_last_error_string().decode("utf-8", "replace")
+        raise KernlLibraryError(f"{what} failed with status {status}: {msg}")
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernlLibraryError("kernl_amd kernels need tensors on a GPU device (there is no CPU path)")
+
+
+def attention_fwd(q, k, v, out, mask, sm_scale: float, is_causal: bool, mask_min_clamp: float) -> None:
+    _require_gpu(q, k, v, out, mask)
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    lib = load()
+    if mask is not None:
+        msizes, mstrides, mdtype, mptr = _arr(mask.shape), _arr(mask.stride()), DTYPE_CODE[mask.dtype], mask.data_ptr()
+    else:
+        msizes, mstrides, mdtype, mptr = None, None, KERNL_F32, None
+    with torch.cuda.device(q.device):
+        st = lib.kernl_attention_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), mptr,
+            B, H, M, N, D,
+            _arr(q.stride()), _arr(k.stride()), _arr(v.stride()), _arr(out.stride()),
+            msizes, mstrides, mdtype,
+            float(sm_scale), int(bool(is_causal)), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
+        )
+    _check(st, "kernl_attention_fwd")
+
+
+def linear_fwd(x2d, weight, bias, out2d, act_in2d, activation: int) -> None:
+    _require_gpu(x2d, weight, bias, out2d, act_in2d)
+    M, K = x2d.shape
+    N = weight.shape[0]
+    lib = load()
+    with torch.cuda.device(x2d.device):
+        st = lib.kernl_linear_fwd(
+            x2d.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(), out2d.data_ptr(),
+            None if act_in2d is None else act_in2d.data_ptr(),
+            M, N, K,
+            _arr(x2d.stride()), _arr(out2d.stride()), None if act_in2d is None else _arr(act_in2d.stride()),
+            int(activation), DTYPE_CODE[x2d.dtype], _stream(x2d),
+        )
+    _check(st, "kernl_linear_fwd")
+
+
+def layernorm_fwd(x2d, weight, bias, out2d, mean, rstd, eps: float, is_rms: bool, residual2d=None) -> None:
+    _require_gpu(x2d, weight, bias, out2d, mean, rstd, residual2d)
+    M, N = x2d.shape
+    lib = load()
+    with torch.cuda.device(x2d.device):
+        if residual2d is None:
+            st = lib.kernl_layernorm_fwd(
+                x2d.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(), out2d.data_ptr(),
+                None if mean is None else mean.data_ptr(), None if rstd is None else rstd.data_ptr(),
+                M, N, x2d.stride(0), x2d.stride(1), out2d.stride(0), out2d.stride(1),
+                float(eps), int(bool(is_rms)), DTYPE_CODE[x2d.dtype], _stream(x2d),
+            )
+            _check(st, "kernl_layernorm_fwd")
+        else:
+            st = lib.kernl_add_layernorm_fwd(
+                x2d.data_ptr(), residual2d.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(),
+                out2d.data_ptr(), None if mean is None else mean.data_ptr(), None if rstd is None else rstd.data_ptr(),
+                M, N, x2d.stride(0), x2d.stride(1), residual2d.stride(0), residual2d.stride(1),
+                out2d.stride(0), out2d.stride(1),
+                float(eps), int(bool(is_rms)), DTYPE_CODE[x2d.dtype], _stream(x2d),
+            )
+            _check(st, "kernl_add_layernorm_fwd")

@@ -1,0 +1,150 @@
+// Shared device/host helpers for the gfx950 kernels: vector types, MFMA wrappers, wave64 reductions,
+// LDS swizzles and the thread-local error slot behind kernl_last_error_string().
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/kernl_hip.h"
+
+namespace kernl {
+
+// ----------------------------------------------------------------------------------------------------
+// vector types
+// ----------------------------------------------------------------------------------------------------
+typedef _Float16 f16;
+typedef __bf16 bf16;
+typedef f16 f16x2 __attribute__((ext_vector_type(2)));
+typedef f16 f16x4 __attribute__((ext_vector_type(4)));
+typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+typedef bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+static constexpr int kWave = 64;
+
+// 16-bit storage types map to their 8-wide MFMA operand vector.
+template <typename T>
+struct Vec8;
+template <>
+struct Vec8<f16> {
+    typedef f16x8 type;
+};
+template <>
+struct Vec8<bf16> {
+    typedef bf16x8 type;
+};
+
+// D[32x32] += A[32x16] * B[16x32], fp32 accumulate (v_mfma_f32_32x32x16_{f16,bf16}, 8 passes).
+// Operand layout, lane l of the wave: A holds row (l % 32), k = 8*(l/32) .. +7; B holds column (l % 32),
+// same k range; D element v (0..15) of lane l is row 8*(v/4) + 4*(l/32) + (v%4), column (l % 32).
+__device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// Because of the D layout above, feeding MFMA row i with logical row rowperm16(i) makes every lane end up
+// with 16 CONSECUTIVE logical rows: lane half h holds logical rows 16*h + v for v = 0..15.
+__device__ __forceinline__ int rowperm16(int i) { return 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3); }
+
+// ----------------------------------------------------------------------------------------------------
+// conversions
+// ----------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float to_float(f16 x) { return (float)x; }
+__device__ __forceinline__ float to_float(bf16 x) { return (float)x; }
+__device__ __forceinline__ float to_float(float x) { return x; }
+
+template <typename T>
+__device__ __forceinline__ T from_float(float x);
+template <>
+__device__ __forceinline__ f16 from_float<f16>(float x) {
+    return (f16)x;
+}
+template <>
+__device__ __forceinline__ bf16 from_float<bf16>(float x) {
+    return (bf16)x;
+}
+template <>
+__device__ __forceinline__ float from_float<float>(float x) {
+    return x;
+}
+
+// Two fp32 -> packed pair of 16-bit values in one 32-bit register (round to nearest even).
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <>
+__device__ __forceinline__ uint32_t pack2<f16>(float lo, float hi) {
+    f16x2 p = {(f16)lo, (f16)hi};
+    return __builtin_bit_cast(uint32_t, p);
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<bf16>(float lo, float hi) {
+    bf16x2 p = {(bf16)lo, (bf16)hi};
+    return __builtin_bit_cast(uint32_t, p);
+}
+
+// ----------------------------------------------------------------------------------------------------
+// wave64 reductions: quad permutes and row mirrors on DPP, the last two steps through scalar lane reads.
+// Every lane receives the full result.
+// ----------------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_mov<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_mov<0x141>(v);  // row_half_mirror
+    v += dpp_mov<0x140>(v);  // row_mirror
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// Value held by the lane 32 positions away (lane l <-> lane l ^ 32).
+__device__ __forceinline__ float swap32(float v) {
+    return __shfl_xor(v, 32, 64);
+}
+
+// ----------------------------------------------------------------------------------------------------
+// LDS swizzle for tiles whose rows are ROW_BYTES long (64, 128 or 256) and are read as 16-byte chunks by the
+// 32 rows x 2 k-halves pattern of an MFMA operand fetch: 16 consecutive rows reading the same logical chunk
+// land in 16 different 16-byte bank groups.
+// ----------------------------------------------------------------------------------------------------
+template <int ROW_BYTES>
+__device__ __forceinline__ int swz_chunk(int row, int chunk) {
+    static_assert(ROW_BYTES == 64 || ROW_BYTES == 128 || ROW_BYTES == 256, "row must span 4, 8 or 16 chunks");
+    if (ROW_BYTES == 64) return chunk ^ ((row >> 2) & 3);
+    if (ROW_BYTES == 128) return chunk ^ ((row >> 1) & 7);
+    return chunk ^ (row & 15);
+}
+template <int ROW_BYTES>
+__device__ __forceinline__ int swz_offset(int row, int chunk) {  // byte offset inside the tile
+    return row * ROW_BYTES + swz_chunk<ROW_BYTES>(row, chunk) * 16;
+}
+
+// ----------------------------------------------------------------------------------------------------
+// host side
+// ----------------------------------------------------------------------------------------------------
+int set_error(int status, const char *fmt, ...);
+int check_launch(const char *what);
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace kernl

@@ -1,0 +1,291 @@
+// LayerNorm / RMSNorm forward for gfx950, with an optional fused residual add.
+//
+// Memory-bound: the register-resident kernel reads every row from HBM exactly once (16-byte loads, one
+// wave per row, the row stays in VGPRs between the statistics and the normalisation), reduces with DPP
+// inside the wave, and writes 16-byte stores.  Semantics follow the reference kernel
+// src/kernl/implementations/layer_norm.py:115-205: fp32 statistics, biased variance, rstd = 1/sqrt(var+eps),
+// RMS branch keeps mean = 0 and uses mean(x^2).  The variance is the exact two-pass form Σ(x-mean)²/N on the
+// register copy, which is at least as accurate as the reference's chunked Welford merge (:159-180).
+#include "common.h"
+
+namespace kernl {
+
+template <typename T>
+struct Row16 {  // one 16-byte chunk of a row
+    static constexpr int kElems = 16 / sizeof(T);
+    T v[kElems];
+};
+
+// One wave per row; lane l owns chunks l, l+64, ... (CHUNKS of them at most).
+template <typename T, int CHUNKS, bool RMS, bool HAS_RES>
+__global__ void __launch_bounds__(256)
+layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const T *__restrict__ w,
+                      const T *__restrict__ b, T *__restrict__ out, float *__restrict__ mean_out,
+                      float *__restrict__ rstd_out, int M, int N, int64_t x_rs, int64_t res_rs,
+                      int64_t out_rs, float eps) {
+    constexpr int E = Row16<T>::kElems;
+    typedef Row16<T> chunk_t;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int waves_per_block = blockDim.x >> 6;
+    const int nchunks = N / E;
+    const float inv_n = 1.0f / (float)N;
+
+    // gamma / beta stay in registers (as 16-bit pairs) for every row this wave visits.
+    chunk_t wv[CHUNKS], bv[CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int ci = lane + c * 64;
+        if (ci < nchunks) {
+            wv[c] = *reinterpret_cast<const chunk_t *>(w + (int64_t)ci * E);
+            if (b != nullptr) bv[c] = *reinterpret_cast<const chunk_t *>(b + (int64_t)ci * E);
+        }
+    }
+
+    for (int row = blockIdx.x * waves_per_block + wave; row < M; row += gridDim.x * waves_per_block) {
+        float v[CHUNKS][E];
+        const T *xr = x + (int64_t)row * x_rs;
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) {
+            const int ci = lane + c * 64;
+            if (ci < nchunks) {
+                chunk_t t = *reinterpret_cast<const chunk_t *>(xr + (int64_t)ci * E);
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[c][e] = to_float(t.v[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) v[c][e] = 0.0f;
+            }
+        }
+        if (HAS_RES) {
+            const T *rr = res + (int64_t)row * res_rs;
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c) {
+                const int ci = lane + c * 64;
+                if (ci < nchunks) {
+                    chunk_t t = *reinterpret_cast<const chunk_t *>(rr + (int64_t)ci * E);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) v[c][e] += to_float(t.v[e]);
+                }
+            }
+        }
+
+        float mean = 0.0f, var;
+        if (RMS) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+                for (int e = 0; e < E; ++e) ss += v[c][e] * v[c][e];
+            var = wave_sum(ss) * inv_n;
+        } else {
+            float s = 0.0f;
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+                for (int e = 0; e < E; ++e) s += v[c][e];
+            mean = wave_sum(s) * inv_n;
+            float ss = 0.0f;
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c) {
+                const int ci = lane + c * 64;
+                if (ci < nchunks) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) {
+                        const float d = v[c][e] - mean;
+                        ss += d * d;
+                    }
+                }
+            }
+            var = wave_sum(ss) * inv_n;
+        }
+        const float rstd = 1.0f / sqrtf(var + eps);
+        if (lane == 0) {
+            if (mean_out != nullptr) mean_out[row] = mean;
+            if (rstd_out != nullptr) rstd_out[row] = rstd;
+        }
+
+        T *orow = out + (int64_t)row * out_rs;
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) {
+            const int ci = lane + c * 64;
+            if (ci < nchunks) {
+                chunk_t o;
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    float y = (v[c][e] - mean) * rstd * to_float(wv[c].v[e]);
+                    if (b != nullptr) y += to_float(bv[c].v[e]);
+                    o.v[e] = from_float<T>(y);
+                }
+                *reinterpret_cast<chunk_t *>(orow + (int64_t)ci * E) = o;
+            }
+        }
+    }
+}
+
+// Any strides, any N: one 256-thread block per row, three passes over the (cache-resident) row.
+template <typename T, bool RMS, bool HAS_RES>
+__global__ void __launch_bounds__(256)
+layernorm_strided_kernel(const T *__restrict__ x, const T *__restrict__ res, const T *__restrict__ w,
+                         const T *__restrict__ b, T *__restrict__ out, float *__restrict__ mean_out,
+                         float *__restrict__ rstd_out, int M, int N, int64_t x_rs, int64_t x_cs,
+                         int64_t res_rs, int64_t res_cs, int64_t out_rs, int64_t out_cs, float eps) {
+    __shared__ float red[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float inv_n = 1.0f / (float)N;
+    for (int row = blockIdx.x; row < M; row += gridDim.x) {
+        const T *xr = x + (int64_t)row * x_rs;
+        const T *rr = HAS_RES ? res + (int64_t)row * res_rs : nullptr;
+        auto load = [&](int i) -> float {
+            float a = to_float(xr[(int64_t)i * x_cs]);
+            if (HAS_RES) a += to_float(rr[(int64_t)i * res_cs]);
+            return a;
+        };
+        auto block_sum = [&](float s) -> float {
+            s = wave_sum(s);
+            __syncthreads();
+            if (lane == 0) red[wave] = s;
+            __syncthreads();
+            return (red[0] + red[1]) + (red[2] + red[3]);
+        };
+        float mean = 0.0f;
+        if (!RMS) {
+            float s = 0.0f;
+            for (int i = threadIdx.x; i < N; i += blockDim.x) s += load(i);
+            mean = block_sum(s) * inv_n;
+        }
+        float ss = 0.0f;
+        for (int i = threadIdx.x; i < N; i += blockDim.x) {
+            const float d = load(i) - mean;
+            ss += d * d;
+        }
+        const float var = block_sum(ss) * inv_n;
+        const float rstd = 1.0f / sqrtf(var + eps);
+        if (threadIdx.x == 0) {
+            if (mean_out != nullptr) mean_out[row] = mean;
+            if (rstd_out != nullptr) rstd_out[row] = rstd;
+        }
+        T *orow = out + (int64_t)row * out_rs;
+        for (int i = threadIdx.x; i < N; i += blockDim.x) {
+            float y = (load(i) - mean) * rstd * to_float(w[i]);
+            if (b != nullptr) y += to_float(b[i]);
+            orow[(int64_t)i * out_cs] = from_float<T>(y);
+        }
+    }
+}
+
+template <typename T, int CHUNKS>
+static void launch_rows(bool rms, bool has_res, dim3 grid, hipStream_t st, const T *x, const T *res,
+                        const T *w, const T *b, T *out, float *mean, float *rstd, int M, int N, int64_t x_rs,
+                        int64_t res_rs, int64_t out_rs, float eps) {
+#define KERNL_LN_LAUNCH(R, H)                                                                          \
+    hipLaunchKernelGGL((layernorm_rows_kernel<T, CHUNKS, R, H>), grid, dim3(256), 0, st, x, res, w, b, \
+                       out, mean, rstd, M, N, x_rs, res_rs, out_rs, eps)
+    if (rms) {
+        if (has_res) KERNL_LN_LAUNCH(true, true);
+        else KERNL_LN_LAUNCH(true, false);
+    } else {
+        if (has_res) KERNL_LN_LAUNCH(false, true);
+        else KERNL_LN_LAUNCH(false, false);
+    }
+#undef KERNL_LN_LAUNCH
+}
+
+template <typename T>
+static int layernorm_dispatch(const void *x_, const void *res_, const void *w_, const void *b_, void *out_,
+                              float *mean, float *rstd, int64_t M, int64_t N, int64_t x_rs, int64_t x_cs,
+                              int64_t res_rs, int64_t res_cs, int64_t out_rs, int64_t out_cs, float eps,
+                              bool rms, hipStream_t st) {
+    const T *x = static_cast<const T *>(x_);
+    const T *res = static_cast<const T *>(res_);
+    const T *w = static_cast<const T *>(w_);
+    const T *b = static_cast<const T *>(b_);
+    T *out = static_cast<T *>(out_);
+    const bool has_res = res != nullptr;
+    constexpr int E = 16 / sizeof(T);
+    const int64_t row_chunks = N / E;
+    const bool vec_ok = (N % E == 0) && x_cs == 1 && out_cs == 1 && (!has_res || res_cs == 1) &&
+                        (x_rs % E == 0) && (out_rs % E == 0) && (!has_res || res_rs % E == 0) &&
+                        aligned16(x) && aligned16(out) && aligned16(w) && (b == nullptr || aligned16(b)) &&
+                        (!has_res || aligned16(res)) && row_chunks <= 64 * 16;
+    if (vec_ok) {
+        // 4 rows per 256-thread block; enough blocks to cover the rows, capped so that gamma/beta loads
+        // amortise over several rows on large inputs.
+        const int64_t blocks_needed = (M + 3) / 4;
+        const int grid = (int)(blocks_needed < 8192 ? blocks_needed : 8192);
+        const int chunks = (int)((row_chunks + 63) / 64);
+#define KERNL_LN_CASE(C)                                                                                   \
+    launch_rows<T, C>(rms, has_res, dim3(grid), st, x, res, w, b, out, mean, rstd, (int)M, (int)N, x_rs, \
+                      res_rs, out_rs, eps)
+        if (chunks <= 1) KERNL_LN_CASE(1);
+        else if (chunks <= 2) KERNL_LN_CASE(2);
+        else if (chunks <= 4) KERNL_LN_CASE(4);
+        else if (chunks <= 8) KERNL_LN_CASE(8);
+        else KERNL_LN_CASE(16);
+#undef KERNL_LN_CASE
+    } else {
+        const int grid = (int)(M < 65535 ? M : 65535);
+#define KERNL_LN_LAUNCH(R, H)                                                                             \
+    hipLaunchKernelGGL((layernorm_strided_kernel<T, R, H>), dim3(grid), dim3(256), 0, st, x, res, w, b, \
+                       out, mean, rstd, (int)M, (int)N, x_rs, x_cs, res_rs, res_cs, out_rs, out_cs, eps)
+        if (rms) {
+            if (has_res) KERNL_LN_LAUNCH(true, true);
+            else KERNL_LN_LAUNCH(true, false);
+        } else {
+            if (has_res) KERNL_LN_LAUNCH(false, true);
+            else KERNL_LN_LAUNCH(false, false);
+        }
+#undef KERNL_LN_LAUNCH
+    }
+    return check_launch("layernorm");
+}
+
+static int layernorm_entry(const void *x, const void *res, const void *w, const void *b, void *out,
+                           float *mean, float *rstd, int64_t M, int64_t N, int64_t x_rs, int64_t x_cs,
+                           int64_t res_rs, int64_t res_cs, int64_t out_rs, int64_t out_cs, float eps,
+                           int is_rms, int dtype, void *stream) {
+    if (x == nullptr || w == nullptr || out == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "layernorm: x, w and out must not be NULL");
+    if (M < 0 || N <= 0) return set_error(KERNL_ERR_INVALID_ARG, "layernorm: bad sizes M=%lld N=%lld",
+                                          (long long)M, (long long)N);
+    if (M > INT32_MAX || N > INT32_MAX)
+        return set_error(KERNL_ERR_UNSUPPORTED, "layernorm: M and N must fit in 31 bits");
+    if (M == 0) return KERNL_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case KERNL_F16:
+            return layernorm_dispatch<f16>(x, res, w, b, out, mean, rstd, M, N, x_rs, x_cs, res_rs, res_cs,
+                                           out_rs, out_cs, eps, is_rms != 0, st);
+        case KERNL_BF16:
+            return layernorm_dispatch<bf16>(x, res, w, b, out, mean, rstd, M, N, x_rs, x_cs, res_rs, res_cs,
+                                            out_rs, out_cs, eps, is_rms != 0, st);
+        case KERNL_F32:
+            return layernorm_dispatch<float>(x, res, w, b, out, mean, rstd, M, N, x_rs, x_cs, res_rs,
+                                             res_cs, out_rs, out_cs, eps, is_rms != 0, st);
+        default:
+            return set_error(KERNL_ERR_UNSUPPORTED, "layernorm: unknown dtype %d", dtype);
+    }
+}
+
+}  // namespace kernl
+
+extern "C" int kernl_layernorm_fwd(const void *x, const void *w, const void *bias, void *out, float *mean,
+                                   float *rstd, int64_t M, int64_t N, int64_t x_row_stride,
+                                   int64_t x_col_stride, int64_t out_row_stride, int64_t out_col_stride,
+                                   float eps, int is_rms, int dtype, void *stream) {
+    return kernl::layernorm_entry(x, nullptr, w, bias, out, mean, rstd, M, N, x_row_stride, x_col_stride,
+                                  0, 0, out_row_stride, out_col_stride, eps, is_rms, dtype, stream);
+}
+
+extern "C" int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, const void *bias,
+                                       void *out, float *mean, float *rstd, int64_t M, int64_t N,
+                                       int64_t x_row_stride, int64_t x_col_stride, int64_t res_row_stride,
+                                       int64_t res_col_stride, int64_t out_row_stride,
+                                       int64_t out_col_stride, float eps, int is_rms, int dtype,
+                                       void *stream) {
+    if (residual == nullptr)
+        return kernl::set_error(KERNL_ERR_INVALID_ARG, "add_layernorm: residual must not be NULL");
+    return kernl::layernorm_entry(x, residual, w, bias, out, mean, rstd, M, N, x_row_stride, x_col_stride,
+                                  res_row_stride, res_col_stride, out_row_stride, out_col_stride, eps,
+                                  is_rms, dtype, stream);
+}

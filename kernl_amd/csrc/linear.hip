@@ -1,0 +1,452 @@
+// Fused linear layer for gfx950:  out[M,N] = act(x[M,K] · w[N,K]ᵀ + bias[N]).
+//
+// Semantics follow the reference kernel src/kernl/implementations/linear_layer.py:92-210: fp32 accumulation,
+// bias added in fp32, optional store of the pre-activation, activation applied to the fp32 accumulator, one
+// rounding to the output dtype.
+//
+// MFMA path (16-bit inputs, K-contiguous x): both operands are K-major, which is exactly what
+// v_mfma_f32_32x32x16 wants (each lane supplies 8 consecutive k of one row), so tiles go HBM -> VGPR -> LDS
+// with 16-byte accesses and no transposition.  The weight rows feed the MFMA "A" side and the activations the
+// "B" side, i.e. the instruction produces a 32(n) x 32(m) block of outᵀ; together with the row permutation
+// rowperm16 on the weight tile this leaves every lane holding 16 consecutive output columns of one output
+// row, so bias loads and output stores are 16-byte vectors without any shuffle through LDS.
+#include "common.h"
+
+namespace kernl {
+
+// ----------------------------------------------------------------------------------------------------
+// activations on the fp32 accumulator (reference: src/kernl/implementations/activation_func.py:28-49)
+// ----------------------------------------------------------------------------------------------------
+static constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ float act_tanh(float x) {
+    // tanh(x) = 1 - 2 / (exp(2x) + 1); saturates correctly through exp2 -> inf / 0.
+    const float t = __builtin_amdgcn_exp2f(x * (2.0f * kLog2e));
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(t + 1.0f);
+}
+__device__ __forceinline__ float act_sigmoid(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-kLog2e * x));
+}
+__device__ __forceinline__ float act_gelu_tanh(float x) {
+    // 0.5 x (1 + tanh(u)) = x * sigmoid(2u),  u = sqrt(2/pi) (x + 0.044715 x^3)
+    const float u2 = x * (1.5957691216057308f + 0.07135481627f * x * x);
+    return x * act_sigmoid(u2);
+}
+__device__ __forceinline__ float act_gelu_erf(float x) {
+    // 0.5 x (1 + erf(x / sqrt 2)) with erf from Abramowitz & Stegun 7.1.26 (|error| <= 1.5e-7):
+    // erf(z) = 1 - (a1 t + ... + a5 t^5) exp(-z^2),  t = 1 / (1 + p z),  z >= 0.
+    const float ax = fabsf(x);
+    const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * 0.7071067811865476f * ax);
+    float poly = 1.061405429f;
+    poly = poly * t - 1.453152027f;
+    poly = poly * t + 1.421413741f;
+    poly = poly * t - 0.284496736f;
+    poly = poly * t + 0.254829592f;
+    poly *= t;
+    const float e = __builtin_amdgcn_exp2f(-0.5f * kLog2e * x * x);
+    const float erf_abs = 1.0f - poly * e;
+    return 0.5f * (x + ax * erf_abs);
+}
+
+__device__ __forceinline__ float apply_act(float x, int act) {
+    switch (act) {
+        case KERNL_ACT_RELU: return fmaxf(x, 0.0f);
+        case KERNL_ACT_TANH: return act_tanh(x);
+        case KERNL_ACT_GELU_ERF: return act_gelu_erf(x);
+        case KERNL_ACT_GELU_TANH: return act_gelu_tanh(x);
+        case KERNL_ACT_SILU: return x * act_sigmoid(x);
+        default: return x;
+    }
+}
+
+// ----------------------------------------------------------------------------------------------------
+// MFMA kernel
+// ----------------------------------------------------------------------------------------------------
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int MIN_BLOCKS_>
+struct LinearTile {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int MIN_BLOCKS = MIN_BLOCKS_;
+    static constexpr int THREADS = 64 * WAVES_M * WAVES_N;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // per-wave output tile
+    static constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 MFMA blocks per wave
+    static constexpr int ROW_BYTES = BK * 2;
+    static constexpr int CPR = BK / 8;  // 16-byte chunks per tile row
+    static constexpr int X_BYTES = BM * ROW_BYTES, W_BYTES = BN * ROW_BYTES;
+    static constexpr int STAGE_BYTES = X_BYTES + W_BYTES;
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+    static constexpr int XI = BM * CPR / THREADS, WI = BN * CPR / THREADS;  // chunks per thread per stage
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32 blocks");
+    static_assert(BM * CPR % THREADS == 0 && BN * CPR % THREADS == 0, "tile rows must split over threads");
+    static constexpr int GROUP_M = 4;  // m-tiles walked together so one XCD's L2 sees a compact block
+};
+
+template <typename T, typename Cfg, int ACT>
+__global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_BLOCKS)
+linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
+                   T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx,
+                   int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n,
+                   int out_vec_ok, int ai_vec_ok, int bias_vec_ok) {
+    typedef typename Vec8<T>::type vec8;
+    const bool HAS_BIAS = bias != nullptr, SAVE_ACT_IN = act_in != nullptr;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, CPR = Cfg::CPR, RB = Cfg::ROW_BYTES;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    // ---- tile assignment: workgroup ids are dealt round-robin to the 8 XCDs, so give each XCD a
+    // contiguous run of the (grouped) tile order; its private L2 then sees neighbouring tiles.
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) >> 3;
+    const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || t >= total) return;
+    const int group_span = Cfg::GROUP_M * tiles_n;
+    const int group = t / group_span;
+    const int first_m = group * Cfg::GROUP_M;
+    const int gsize = min(tiles_m - first_m, Cfg::GROUP_M);
+    const int in_group = t - group * group_span;
+    const int tile_m = first_m + in_group % gsize;
+    const int tile_n = in_group / gsize;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave % Cfg::WAVES_M, wave_n = wave / Cfg::WAVES_M;
+    const int lr = lane & 31, lh = lane >> 5;
+
+    // ---- global -> register staging: thread owns chunks q = tid + THREADS*i, row q / CPR, chunk q % CPR
+    const T *xg[Cfg::XI];
+    const T *wg[Cfg::WI];
+    int xl[Cfg::XI], wl[Cfg::WI];  // LDS byte offsets inside a stage
+#pragma unroll
+    for (int i = 0; i < Cfg::XI; ++i) {
+        const int q = tid + Cfg::THREADS * i;
+        const int row = q / CPR, c = q % CPR;
+        const int gm = min(m0 + row, M - 1);
+        xg[i] = X + (int64_t)gm * ldx + c * 8;
+        xl[i] = swz_offset<RB>(row, c);
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::WI; ++i) {
+        const int q = tid + Cfg::THREADS * i;
+        const int row = q / CPR, c = q % CPR;
+        // LDS row `row` feeds MFMA row (row % 32) of its 32-block and carries weight row rowperm16(row % 32).
+        const int gn = min(n0 + (row & ~31) + rowperm16(row & 31), N - 1);
+        wg[i] = W + (int64_t)gn * K + c * 8;
+        wl[i] = Cfg::X_BYTES + swz_offset<RB>(row, c);
+    }
+    const int kchunk = (tid % CPR) * 8;  // same for every i because THREADS % CPR == 0
+
+    vec8 xs[Cfg::XI], ws[Cfg::WI];
+    auto gload = [&](int k0) {
+        const bool in = (k0 + kchunk) < K;  // K % 8 == 0: a chunk is entirely inside or outside
+#pragma unroll
+        for (int i = 0; i < Cfg::XI; ++i) {
+            vec8 z = {};
+            xs[i] = in ? *reinterpret_cast<const vec8 *>(xg[i] + k0) : z;
+        }
+#pragma unroll
+        for (int i = 0; i < Cfg::WI; ++i) {
+            vec8 z = {};
+            ws[i] = in ? *reinterpret_cast<const vec8 *>(wg[i] + k0) : z;
+        }
+    };
+    auto lstore = [&](int stage) {
+        unsigned char *base = smem + stage * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < Cfg::XI; ++i) *reinterpret_cast<vec8 *>(base + xl[i]) = xs[i];
+#pragma unroll
+        for (int i = 0; i < Cfg::WI; ++i) *reinterpret_cast<vec8 *>(base + wl[i]) = ws[i];
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // LDS rows this lane reads for its operand fragments
+    int xrow[TM], wrow[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) xrow[i] = wave_m * Cfg::WM + i * 32 + lr;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) wrow[j] = wave_n * Cfg::WN + j * 32 + lr;
+
+    const int nk = (K + BK - 1) / BK;
+    gload(0);
+    lstore(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+        if (kt + 1 < nk) gload((kt + 1) * BK);
+        const unsigned char *sx = smem + (kt & 1) * Cfg::STAGE_BYTES;
+        const unsigned char *sw = sx + Cfg::X_BYTES;
+#pragma unroll
+        for (int s = 0; s < BK / 16; ++s) {
+            vec8 a[TN], b[TM];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                a[j] = *reinterpret_cast<const vec8 *>(sw + swz_offset<RB>(wrow[j], 2 * s + lh));
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                b[i] = *reinterpret_cast<const vec8 *>(sx + swz_offset<RB>(xrow[i], 2 * s + lh));
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma32(a[j], b[i], acc[i][j]);
+        }
+        if (kt + 1 < nk) lstore((kt + 1) & 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane (lr, lh) holds, for block (i, j), output row m0 + WM*wave_m + 32 i + lr and the 16
+    // consecutive columns starting at n0 + WN*wave_n + 32 j + 16 lh.
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int n = n0 + wave_n * Cfg::WN + j * 32 + lh * 16;
+        float bv[16];
+        if (HAS_BIAS) {
+            if (bias_vec_ok && n + 16 <= N) {
+                const vec8 b0 = *reinterpret_cast<const vec8 *>(bias + n);
+                const vec8 b1 = *reinterpret_cast<const vec8 *>(bias + n + 8);
+#pragma unroll
+                for (int v = 0; v < 8; ++v) {
+                    bv[v] = to_float(b0[v]);
+                    bv[8 + v] = to_float(b1[v]);
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) bv[v] = (n + v < N) ? to_float(bias[n + v]) : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int m = m0 + wave_m * Cfg::WM + i * 32 + lr;
+            if (m >= M || n >= N) continue;
+            float r[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) r[v] = HAS_BIAS ? acc[i][j][v] + bv[v] : acc[i][j][v];
+            if (SAVE_ACT_IN) {
+                if (ai_vec_ok && n + 16 <= N) {
+                    u32x4 p0, p1;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
+                        p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
+                    }
+                    T *p = act_in + (int64_t)m * ai_rs + n;
+                    *reinterpret_cast<u32x4 *>(p) = p0;
+                    *reinterpret_cast<u32x4 *>(p + 8) = p1;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        if (n + v < N) act_in[(int64_t)m * ai_rs + (int64_t)(n + v) * ai_cs] = from_float<T>(r[v]);
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) r[v] = apply_act(r[v], ACT);
+            if (out_vec_ok && n + 16 <= N) {
+                u32x4 p0, p1;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
+                    p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
+                }
+                T *p = out + (int64_t)m * out_rs + n;
+                *reinterpret_cast<u32x4 *>(p) = p0;
+                *reinterpret_cast<u32x4 *>(p + 8) = p1;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (n + v < N) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
+            }
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------------
+// FMA kernel: any dtype, any strides.  64x64 output tile, 16x16 threads, 4x4 outputs per thread, fp32 LDS tiles.
+// ----------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+linear_fma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
+                  T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t x_rs, int64_t x_cs,
+                  int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int act) {
+    __shared__ float xs[16][64 + 1];
+    __shared__ float ws[16][64 + 1];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        for (int e = threadIdx.x; e < 64 * 16; e += 256) {
+            const int r = e >> 4, kk = e & 15;
+            const int gm = m0 + r, gn = n0 + r, gk = k0 + kk;
+            xs[kk][r] = (gm < M && gk < K) ? to_float(X[(int64_t)gm * x_rs + (int64_t)gk * x_cs]) : 0.0f;
+            ws[kk][r] = (gn < N && gk < K) ? to_float(W[(int64_t)gn * K + gk]) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = xs[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = ws[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += a[i] * b[j];
+        }
+        __syncthreads();
+    }
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= N) continue;
+            float r = acc[i][j];
+            if (bias != nullptr) r += to_float(bias[n]);
+            if (act_in != nullptr) act_in[(int64_t)m * ai_rs + (int64_t)n * ai_cs] = from_float<T>(r);
+            out[(int64_t)m * out_rs + (int64_t)n * out_cs] = from_float<T>(apply_act(r, act));
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------------
+// host dispatch
+// ----------------------------------------------------------------------------------------------------
+struct LinearArgs {
+    const void *x, *w, *bias;
+    void *out, *act_in;
+    int M, N, K;
+    int64_t x_rs, x_cs, out_rs, out_cs, ai_rs, ai_cs;
+    int act;
+    hipStream_t st;
+};
+
+template <typename T, typename Cfg, int ACT>
+static void launch_mfma_act(const LinearArgs &a) {
+    auto kern = linear_mfma_kernel<T, Cfg, ACT>;
+    static bool attr_done = false;  // benign race: the attribute call is idempotent
+    if (!attr_done) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+        attr_done = true;
+    }
+    const int tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
+    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+    const T *x = static_cast<const T *>(a.x);
+    const T *w = static_cast<const T *>(a.w);
+    const T *bias = static_cast<const T *>(a.bias);
+    T *out = static_cast<T *>(a.out);
+    T *act_in = static_cast<T *>(a.act_in);
+    const int out_vec_ok = a.out_cs == 1 && a.out_rs % 8 == 0 && aligned16(out);
+    const int ai_vec_ok = act_in != nullptr && a.ai_cs == 1 && a.ai_rs % 8 == 0 && aligned16(act_in);
+    const int bias_vec_ok = bias != nullptr && aligned16(bias);
+    hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(Cfg::THREADS), Cfg::LDS_BYTES, a.st, x, w, bias, out,
+                       act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs, a.ai_cs, tiles_m, tiles_n,
+                       out_vec_ok, ai_vec_ok, bias_vec_ok);
+}
+
+template <typename T, typename Cfg>
+static void launch_mfma_cfg(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_mfma_act<T, Cfg, KERNL_ACT_RELU>(a); break;
+        case KERNL_ACT_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_TANH>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_ERF>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_TANH>(a); break;
+        case KERNL_ACT_SILU: launch_mfma_act<T, Cfg, KERNL_ACT_SILU>(a); break;
+        default: launch_mfma_act<T, Cfg, KERNL_ACT_NONE>(a); break;
+    }
+}
+
+//                         BM   BN  BK  WAVES_M WAVES_N  MIN_BLOCKS
+typedef LinearTile<256, 256, 64, 2, 4, 1> Tile256x256;
+typedef LinearTile<256, 192, 64, 4, 2, 1> Tile256x192;
+typedef LinearTile<128, 128, 64, 2, 2, 2> Tile128x128;
+
+// Number of "rounds" a tile shape needs on 256 CUs times the work of one tile: a proxy for run time.
+static double tile_cost(int M, int N, int bm, int bn, int blocks_per_cu) {
+    const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    const int64_t slots = 256 * blocks_per_cu;
+    const int64_t rounds = (tiles + slots - 1) / slots;
+    // larger tiles move fewer operand bytes per flop; weigh that in mildly.
+    const double eff = 1.0 / (1.0 + 48.0 / bm + 48.0 / bn);
+    return (double)rounds * bm * bn * blocks_per_cu / eff;
+}
+
+int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128
+
+template <typename T>
+static int linear_mfma_dispatch(const LinearArgs &a) {
+    int pick = g_linear_force_tile;
+    if (pick == 0) {
+        const double c1 = tile_cost(a.M, a.N, 256, 256, 1);
+        const double c2 = tile_cost(a.M, a.N, 256, 192, 1);
+        const double c3 = tile_cost(a.M, a.N, 128, 128, 2);
+        pick = 1;
+        double best = c1;
+        if (c2 < best) { best = c2; pick = 2; }
+        if (c3 < best) { best = c3; pick = 3; }
+    }
+    if (pick == 1) launch_mfma_cfg<T, Tile256x256>(a);
+    else if (pick == 2) launch_mfma_cfg<T, Tile256x192>(a);
+    else launch_mfma_cfg<T, Tile128x128>(a);
+    return check_launch("linear (mfma)");
+}
+
+template <typename T>
+static int linear_fma_dispatch(const LinearArgs &a) {
+    dim3 grid((a.N + 63) / 64, (a.M + 63) / 64);
+    hipLaunchKernelGGL((linear_fma_kernel<T>), grid, dim3(256), 0, a.st, static_cast<const T *>(a.x),
+                       static_cast<const T *>(a.w), static_cast<const T *>(a.bias), static_cast<T *>(a.out),
+                       static_cast<T *>(a.act_in), a.M, a.N, a.K, a.x_rs, a.x_cs, a.out_rs, a.out_cs, a.ai_rs,
+                       a.ai_cs, a.act);
+    return check_launch("linear (fma)");
+}
+
+}  // namespace kernl
+
+// Tuning hook used by the sweep tests: force a tile shape (0 restores the heuristic).
+extern "C" void kernl_linear_force_tile(int which) { kernl::g_linear_force_tile = which; }
+
+extern "C" int kernl_linear_fwd(const void *x, const void *w, const void *bias, void *out, void *act_in,
+                                int64_t M, int64_t N, int64_t K, const int64_t x_strides[2],
+                                const int64_t out_strides[2], const int64_t act_in_strides[2], int activation,
+                                int dtype, void *stream) {
+    using namespace kernl;
+    if (x == nullptr || w == nullptr || out == nullptr || x_strides == nullptr || out_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear: x, w, out and their strides must not be NULL");
+    if (act_in != nullptr && act_in_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear: act_in given without strides");
+    if (M < 0 || N <= 0 || K <= 0)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear: bad sizes M=%lld N=%lld K=%lld", (long long)M,
+                         (long long)N, (long long)K);
+    if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear: sizes must fit in 31 bits");
+    if (activation < KERNL_ACT_NONE || activation > KERNL_ACT_SILU)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear: unknown activation %d", activation);
+    if (M == 0) return KERNL_OK;
+
+    LinearArgs a;
+    a.x = x; a.w = w; a.bias = bias; a.out = out; a.act_in = act_in;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.x_rs = x_strides[0]; a.x_cs = x_strides[1];
+    a.out_rs = out_strides[0]; a.out_cs = out_strides[1];
+    a.ai_rs = act_in ? act_in_strides[0] : 0; a.ai_cs = act_in ? act_in_strides[1] : 0;
+    a.act = activation;
+    a.st = static_cast<hipStream_t>(stream);
+
+    if (dtype == KERNL_F16 || dtype == KERNL_BF16) {
+        const bool mfma_ok = a.x_cs == 1 && K % 8 == 0 && a.x_rs % 8 == 0 && aligned16(x) && aligned16(w);
+        if (mfma_ok) return dtype == KERNL_F16 ? linear_mfma_dispatch<f16>(a) : linear_mfma_dispatch<bf16>(a);
+        if ((M + 63) / 64 > 65535) return set_error(KERNL_ERR_UNSUPPORTED, "linear: M too large for the strided path");
+        return dtype == KERNL_F16 ? linear_fma_dispatch<f16>(a) : linear_fma_dispatch<bf16>(a);
+    }
+    if (dtype == KERNL_F32) {
+        if ((M + 63) / 64 > 65535) return set_error(KERNL_ERR_UNSUPPORTED, "linear: M too large for the fp32 path");
+        return linear_fma_dispatch<float>(a);
+    }
+    return set_error(KERNL_ERR_UNSUPPORTED, "linear: unknown dtype %d", dtype);
+}

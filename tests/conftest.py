@@ -1,0 +1,40 @@
+import os
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: test needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(autouse=True)
+def set_seed():
+    torch.manual_seed(0)
+    yield
+
+
+# Tolerance of the fp16/bf16 kernels against the fp32 oracle on the same (already rounded) inputs:
+# max-abs-error <= 1e-2 and mean relative error <= 1e-3 for fp16 outputs of unit scale.  bf16 has 3 fewer mantissa
+# bits than fp16, so its bounds are 8x wider.  Outputs of larger magnitude scale the absolute bound.
+def check_close(actual: torch.Tensor, expected: torch.Tensor, dtype=torch.float16, scale: float = 1.0, what: str = ""):
+    a = actual.detach().float().cpu()
+    e = expected.detach().float().cpu()
+    assert a.shape == e.shape, f"{what}: shape {tuple(a.shape)} != {tuple(e.shape)}"
+    assert torch.isfinite(a).all(), f"{what}: non-finite values in the kernel output"
+    widen = 8.0 if dtype == torch.bfloat16 else 1.0
+    max_abs = (a - e).abs().max().item()
+    mean_rel = ((a - e).abs().mean() / e.abs().mean().clamp_min(1e-12)).item()
+    assert max_abs <= 1e-2 * widen * scale, f"{what}: max abs error {max_abs:.3e} > {1e-2 * widen * scale:.1e}"
+    assert mean_rel <= 1e-3 * widen, f"{what}: mean relative error {mean_rel:.3e} > {1e-3 * widen:.1e}"
+    return max_abs, mean_rel
+
+
+@pytest.fixture
+def close():
+    return check_close

@@ -1,0 +1,177 @@
+"""GPU parity of the fused attention kernel against the CPU oracle.
+
+Shapes, mask kinds and stride cases follow the reference's test/test_attention.py:62-145 (tile-edge sequence lengths
+8..512 and 1500, broadcast padding mask, full bias mask, mixed strides, cross-attention), sized so the fp32 oracle
+finishes in seconds; BASELINE config 1 ([32,12,512,64] with padding lengths in [256,512]) runs at full size.
+"""
+import pytest
+import torch
+
+from kernl_amd import _lib
+from kernl_amd.implementations.attention import attention_forward
+from oracle import attention_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _mk(shape, dtype, gen, lo=None):
+    if lo is None:
+        t = torch.randn(shape, generator=gen)
+    else:
+        t = torch.rand(shape, generator=gen) * 2.0  # U(0, 2) as in the reference test
+    return t.to(dtype)
+
+
+def _run(q, k, v, sm_scale, causal, mask):
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    out = torch.empty_like(qc)
+    attention_forward(qc, kc, vc, out, sm_scale, is_causal=causal, attention_mask=None if mask is None else mask.cuda())
+    torch.cuda.synchronize()
+    return out
+
+
+SHAPES = [
+    (1, 3, 8, 64), (2, 3, 16, 64), (1, 2, 33, 64), (2, 2, 128, 64), (1, 2, 257, 64), (2, 4, 384, 64),
+    (1, 4, 512, 64), (1, 1, 1500, 64), (1, 2, 128, 128), (1, 2, 200, 128), (1, 1, 1024, 128),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("causal", [False, True], ids=["noncausal", "causal"])
+@pytest.mark.parametrize("mask_kind", ["none", "padding", "bias"])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_attention_vs_oracle(shape, mask_kind, causal, dtype, close):
+    B, H, S, D = shape
+    gen = torch.Generator().manual_seed(0)
+    q, k, v = (_mk(shape, dtype, gen) for _ in range(3))
+    sm_scale = 0.3 if D == 64 else 0.125
+    mask = None
+    if mask_kind == "padding":
+        lengths = torch.randint(1, S + 1, (B,), generator=gen)
+        mask = torch.zeros((B, 1, 1, S))
+        for b in range(B):
+            mask[b, :, :, lengths[b]:] = float("-inf")
+    elif mask_kind == "bias":
+        mask = torch.rand((B, H, S, S), generator=gen)
+    print(f"case shape={shape} mask={mask_kind} causal={causal} dtype={dtype}", flush=True)
+    out = _run(q, k, v, sm_scale, causal, mask)
+    ref = attention_oracle(q, k, v, sm_scale, causal, mask)
+    close(out, ref, dtype, what=f"attention {shape} {mask_kind} causal={causal}")
+
+
+def test_attention_u02_inputs_like_reference(close):
+    # reference draws q, k, v from U(0, 2) with sm_scale 0.3 (test/test_attention.py:91-99): large positive logits
+    gen = torch.Generator().manual_seed(1)
+    shape = (2, 4, 256, 64)
+    q, k, v = (_mk(shape, torch.float16, gen, lo=0) for _ in range(3))
+    out = _run(q, k, v, 0.3, False, None)
+    close(out, attention_oracle(q, k, v, 0.3), what="attention U(0,2)")
+
+
+def test_attention_mixed_strides(close):
+    # reference test/test_attention.py:110-129: column-major q, batch-interleaved k, transposed mask
+    gen = torch.Generator().manual_seed(2)
+    B, H, S, D = 2, 3, 96, 64
+    q = torch.randn((B, H, D, S), generator=gen).half().transpose(-1, -2)  # feature stride != 1 -> scalar kernel
+    k = torch.randn((H, B, S, D), generator=gen).half().transpose(0, 1)     # batch/head swapped strides
+    v = torch.randn((B, H, S, D), generator=gen).half()
+    mask = torch.rand((B, H, S, S), generator=gen).transpose(-1, -2)
+    out = _run(q, k, v, 0.3, False, mask)
+    close(out, attention_oracle(q, k, v, 0.3, False, mask), what="attention mixed strides")
+
+
+def test_attention_bert_permuted_views(close):
+    # q/k/v as BERT produces them: [B,S,H,D] linear outputs viewed as [B,H,S,D]
+    gen = torch.Generator().manual_seed(3)
+    B, H, S, D = 2, 12, 160, 64
+    q, k, v = (torch.randn((B, S, H, D), generator=gen).half().permute(0, 2, 1, 3) for _ in range(3))
+    lengths = torch.tensor([160, 97])
+    mask = torch.zeros((B, 1, 1, S))
+    for b in range(B):
+        mask[b, :, :, lengths[b]:] = torch.finfo(torch.float32).min
+    out = _run(q, k, v, 0.125, False, mask)
+    close(out, attention_oracle(q, k, v, 0.125, False, mask), what="attention permuted views")
+
+
+def test_attention_cross_attention_single_query(close):
+    # reference test/test_attention.py:133-145: q_len 1, k_len 24, mask [1, 8, 1, 24]
+    gen = torch.Generator().manual_seed(4)
+    q = torch.randn((5, 8, 1, 64), generator=gen).half()
+    k = torch.randn((5, 8, 24, 64), generator=gen).half()
+    v = torch.randn((5, 8, 24, 64), generator=gen).half()
+    mask = torch.randn((1, 8, 1, 24), generator=gen)
+    out = _run(q, k, v, 1.0, False, mask)
+    close(out, attention_oracle(q, k, v, 1.0, False, mask), what="cross attention")
+
+
+def test_attention_scalar_kernel_matches(close):
+    gen = torch.Generator().manual_seed(5)
+    shape = (1, 2, 130, 64)
+    q, k, v = (_mk(shape, torch.float16, gen) for _ in range(3))
+    mask = torch.rand((1, 2, 130, 130), generator=gen)
+    lib = _lib.load()
+    lib.kernl_attention_force_scalar(1)
+    try:
+        for causal in (False, True):
+            out = _run(q, k, v, 0.2, causal, mask)
+            close(out, attention_oracle(q, k, v, 0.2, causal, mask), what=f"scalar kernel causal={causal}")
+    finally:
+        lib.kernl_attention_force_scalar(0)
+
+
+def test_attention_head_size_not_mfma(close):
+    gen = torch.Generator().manual_seed(6)
+    shape = (1, 2, 70, 80)
+    q, k, v = (_mk(shape, torch.float16, gen) for _ in range(3))
+    out = _run(q, k, v, 0.1, True, None)
+    close(out, attention_oracle(q, k, v, 0.1, True, None), what="head size 80")
+
+
+def test_fully_masked_row_is_finite_uniform_average():
+    # -inf mask entries are clamped to finfo.min (reference attention.py:380): a row whose keys are all masked
+    # returns the plain average of V instead of NaN.
+    gen = torch.Generator().manual_seed(7)
+    shape = (2, 2, 128, 64)
+    q, k, v = (_mk(shape, torch.float16, gen) for _ in range(3))
+    mask = torch.zeros((2, 1, 1, 128))
+    mask[1] = float("-inf")
+    out = _run(q, k, v, 0.125, False, mask).float().cpu()
+    assert torch.isfinite(out).all()
+    expected = v[1].float().mean(dim=-2, keepdim=True).expand(-1, 128, -1)
+    assert (out[1] - expected).abs().max().item() < 5e-3
+
+
+def test_attention_properties_full_size(close):
+    # BASELINE config 1 at full size: [32,12,512,64], padding lengths U[256,512], scale 1/8.
+    gen = torch.Generator().manual_seed(0)
+    shape = (32, 12, 512, 64)
+    q, k, v = (torch.randn(shape, generator=gen).half() for _ in range(3))
+    lengths = torch.randint(256, 513, (32,), generator=gen)
+    mask = torch.zeros((32, 1, 1, 512))
+    for b in range(32):
+        mask[b, :, :, lengths[b]:] = float("-inf")
+    out = _run(q, k, v, 0.125, False, mask)
+    ref = attention_oracle(q, k, v, 0.125, False, mask)
+    close(out, ref, what="config 1")
+    # V = 1 => O = 1 exactly representable
+    ones = torch.ones_like(v)
+    out1 = _run(q, k, ones, 0.125, False, mask).float().cpu()
+    assert (out1 - 1.0).abs().max().item() <= 2e-3
+    # keys beyond the padding length must not influence the output: scramble them
+    k2, v2 = k.clone(), v.clone()
+    for b in range(32):
+        k2[b, :, lengths[b]:] = 7.0
+        v2[b, :, lengths[b]:] = -9.0
+    out2 = _run(q, k2, v2, 0.125, False, mask)
+    assert torch.equal(out2.cpu(), out.cpu())
+
+
+def test_attention_rejects_bad_arguments():
+    q = torch.zeros((1, 2, 16, 64), dtype=torch.float16, device="cuda")
+    out = torch.empty_like(q)
+    with pytest.raises(AssertionError):
+        attention_forward(q.float(), q.float(), q.float(), out.float(), 1.0)  # fp32 not supported
+    with pytest.raises(AssertionError):
+        attention_forward(q, q, q, out, 1.0, False, torch.zeros((3, 1, 1, 16), device="cuda"))  # bad batch broadcast
+    with pytest.raises(AssertionError):
+        attention_forward(q, q, q, out, 1.0, False, torch.zeros((1, 1, 1, 15), device="cuda"))  # bad key count

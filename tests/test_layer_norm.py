@@ -1,0 +1,106 @@
+"""GPU parity of LayerNorm / RMSNorm against the CPU oracle.
+
+Cases follow the reference's test/test_layer_norm.py:47-123 (square shapes 128..4096, large-mean input
+-20 + 0.5·randn, RMSNorm, transposed 250x250 input) plus BASELINE config 2's [16384, 768] at full size.
+"""
+import pytest
+import torch
+
+from kernl_amd.implementations.layer_norm import add_layer_norm, layer_norm
+from oracle import effective_eps, layer_norm_oracle, rms_norm_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32], ids=["fp16", "bf16", "fp32"])
+@pytest.mark.parametrize("shape", [128, 512, 1024, 2048, 4096], ids=lambda s: f"{s}x{s}")
+def test_layer_norm_vs_oracle(shape, dtype, close):
+    gen = torch.Generator().manual_seed(0)
+    M = N = shape
+    x = (-20 + 0.5 * torch.randn((M, N), generator=gen)).to(dtype)
+    w = torch.rand((N,), generator=gen).to(dtype)
+    b = torch.randn((N,), generator=gen).to(dtype)
+    eps = 1e-5
+    print(f"case {M}x{N} {dtype}", flush=True)
+    out = layer_norm(x.cuda(), w.cuda(), b.cuda(), eps)
+    torch.cuda.synchronize()
+    ref = layer_norm_oracle(x, w, b, effective_eps(eps, dtype))
+    close(out, ref, torch.float16 if dtype == torch.float32 else dtype, scale=4.0, what=f"layernorm {shape}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [(64, 128), (100, 768), (33, 1000), (7, 4096), (5, 8192), (3, 10000), (9, 250)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_rms_norm_vs_oracle(shape, dtype, close):
+    gen = torch.Generator().manual_seed(1)
+    x = torch.randn(shape, generator=gen).to(dtype)
+    w = (1 + 0.1 * torch.randn((shape[1],), generator=gen)).to(dtype)
+    out = layer_norm(x.cuda(), w.cuda(), None, 1e-5, use_rms_norm=True)
+    torch.cuda.synchronize()
+    close(out, rms_norm_oracle(x, w, effective_eps(1e-5, dtype)), dtype, scale=4.0, what=f"rmsnorm {shape}")
+
+
+def test_layer_norm_odd_sizes_and_3d(close):
+    gen = torch.Generator().manual_seed(2)
+    for shape in [(3, 7, 768), (2, 5, 100), (4, 1, 8192), (2, 3, 9000), (1, 2, 3, 64)]:
+        x = torch.randn(shape, generator=gen).half()
+        w = (1 + 0.1 * torch.randn((shape[-1],), generator=gen)).half()
+        b = (0.1 * torch.randn((shape[-1],), generator=gen)).half()
+        out = layer_norm(x.cuda(), w.cuda(), b.cuda(), 1e-12)
+        torch.cuda.synchronize()
+        assert out.shape == x.shape
+        close(out, layer_norm_oracle(x, w, b, effective_eps(1e-12, torch.float16)), scale=4.0, what=f"layernorm {shape}")
+
+
+def test_layer_norm_transposed_input(close):
+    # reference test/test_layer_norm.py:110-123
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn((250, 250), generator=gen).half().t()
+    w = torch.rand((250,), generator=gen).half()
+    b = torch.randn((250,), generator=gen).half()
+    assert not x.is_contiguous()
+    xc = x.cuda()
+    assert xc.stride() == x.stride() and not xc.is_contiguous()
+    out = layer_norm(xc, w.cuda(), b.cuda(), 1e-5)
+    torch.cuda.synchronize()
+    close(out, layer_norm_oracle(x, w, b, 1.6e-5), scale=4.0, what="layernorm transposed")
+
+
+def test_layer_norm_config2_full_size(close):
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn((16384, 768), generator=gen).half()
+    w = (1 + 0.1 * torch.randn((768,), generator=gen)).half()
+    b = (0.1 * torch.randn((768,), generator=gen)).half()
+    out = layer_norm(x.cuda(), w.cuda(), b.cuda(), 1e-12)
+    torch.cuda.synchronize()
+    close(out, layer_norm_oracle(x, w, b, effective_eps(1e-12, torch.float16)), scale=4.0, what="config 2 layernorm")
+    # size-independent properties: with w = 1, b = 0 every output row has mean 0 and mean square 1 - eps·rstd²
+    ones, zeros = torch.ones((768,), dtype=torch.float16), torch.zeros((768,), dtype=torch.float16)
+    y = layer_norm(x.cuda(), ones.cuda(), zeros.cuda(), 1e-12).float().cpu()
+    assert y.mean(dim=-1).abs().max().item() < 2e-3
+    assert (y.pow(2).mean(dim=-1) - 1).abs().max().item() < 5e-3
+    # shifting a row by a constant does not change LayerNorm (up to the fp16 rounding of the shifted input)
+    y2 = layer_norm((x.float() + 0.5).half().cuda(), ones.cuda(), zeros.cuda(), 1e-12).float().cpu()
+    assert (y2 - y).abs().max().item() < 1e-2
+
+
+def test_add_layer_norm_matches_separate_add(close):
+    gen = torch.Generator().manual_seed(4)
+    for shape in [(512, 768), (4, 40, 768), (30, 1000)]:
+        x = torch.randn(shape, generator=gen).half()
+        r = torch.randn(shape, generator=gen).half()
+        w = (1 + 0.1 * torch.randn((shape[-1],), generator=gen)).half()
+        b = (0.1 * torch.randn((shape[-1],), generator=gen)).half()
+        out = add_layer_norm(x.cuda(), r.cuda(), w.cuda(), b.cuda(), 1e-12)
+        torch.cuda.synchronize()
+        ref = layer_norm_oracle(x.float() + r.float(), w, b, 1.6e-5)
+        close(out, ref, scale=4.0, what=f"add+layernorm {shape}")
+
+
+def test_layer_norm_rejects_bad_arguments():
+    x = torch.zeros((4, 64), dtype=torch.float16, device="cuda")
+    w = torch.ones((64,), dtype=torch.float16, device="cuda")
+    with pytest.raises(AssertionError):
+        layer_norm(x, w.float(), None, 1e-5)
+    with pytest.raises(AssertionError):
+        layer_norm(x, w, w.float(), 1e-5)

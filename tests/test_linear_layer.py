@@ -1,0 +1,134 @@
+"""GPU parity of the fused linear layer against the CPU oracle.
+
+Cases follow the reference's test/test_linear_layer.py:48-99 (shapes (bs, M, 768, 768), bias on/off, activations
+"", tanh, gelu, relu, contiguous and `.mT` inputs, fp16 and fp32) plus BASELINE config 2 at full size.
+"""
+import pytest
+import torch
+
+from kernl_amd import _lib
+from kernl_amd.implementations.linear_layer import linear_layer
+from oracle import linear_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(M, N, K, dtype, gen, w_std=1.0, bias=True, batch=None):
+    xs = (M, K) if batch is None else (batch, M, K)
+    x = torch.randn(xs, generator=gen).to(dtype)
+    w = (torch.randn((N, K), generator=gen) * w_std).to(dtype)
+    b = (torch.randn((N,), generator=gen) * w_std).to(dtype) if bias else None
+    return x, w, b
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32], ids=["fp16", "bf16", "fp32"])
+@pytest.mark.parametrize("activation", ["", "tanh", "gelu", "fast_gelu", "relu", "silu"])
+@pytest.mark.parametrize("bias", [True, False], ids=["bias", "nobias"])
+@pytest.mark.parametrize("shape", [(1, 8, 8, 8), (1, 8, 768, 768), (16, 16, 768, 768), (1, 128, 768, 768),
+                                   (16, 512, 768, 768), (1, 300, 520, 264)], ids=lambda s: "x".join(map(str, s)))
+def test_linear_vs_oracle(shape, bias, activation, dtype, close):
+    bs, M, N, K = shape
+    if dtype == torch.float32 and bs * M > 2048:
+        pytest.skip("fp32 path is the slow FMA kernel; covered at smaller sizes")
+    gen = torch.Generator().manual_seed(0)
+    # weights ~ N(0, 1/K) keep outputs at unit scale so the absolute tolerance is meaningful
+    x, w, b = _inputs(M, N, K, dtype, gen, w_std=K ** -0.5, bias=bias, batch=bs)
+    print(f"case shape={shape} bias={bias} act={activation!r} dtype={dtype}", flush=True)
+    out = linear_layer(x.cuda(), w.cuda(), None if b is None else b.cuda(), activation=activation)
+    torch.cuda.synchronize()
+    assert out.shape == (bs, M, N) and out.dtype == dtype
+    ref = linear_oracle(x, w, b, activation)
+    close(out, ref, torch.float16 if dtype == torch.float32 else dtype, what=f"linear {shape} {activation!r}")
+
+
+@pytest.mark.parametrize("tile", [1, 2, 3], ids=["256x256", "256x192", "128x128"])
+@pytest.mark.parametrize("shape", [(1000, 600, 776), (256, 256, 64), (513, 385, 1032)], ids=lambda s: "x".join(map(str, s)))
+def test_linear_every_tile_shape(shape, tile, close):
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(1)
+    x, w, b = _inputs(M, N, K, torch.float16, gen, w_std=K ** -0.5)
+    lib = _lib.load()
+    lib.kernl_linear_force_tile(tile)
+    try:
+        out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation="gelu")
+        torch.cuda.synchronize()
+    finally:
+        lib.kernl_linear_force_tile(0)
+    close(out, linear_oracle(x, w, b, "gelu"), what=f"linear tile {tile} {shape}")
+
+
+def test_linear_non_contiguous_input(close):
+    # reference test/test_linear_layer.py:73-78: x.mT of a contiguous [K, M] matrix
+    gen = torch.Generator().manual_seed(2)
+    M, N, K = 256, 768, 768
+    xt = torch.randn((4, K, M), generator=gen).half()
+    w = (torch.randn((N, K), generator=gen) * K ** -0.5).half()
+    b = torch.randn((N,), generator=gen).half()
+    x = xt.mT
+    assert not x.is_contiguous()
+    out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation="tanh")
+    torch.cuda.synchronize()
+    close(out, linear_oracle(x, w, b, "tanh"), what="linear x.mT")
+    # 2-D column-major input goes through the strided kernel without a copy
+    x2 = xt[0].mT
+    x2c = x2.cuda()
+    assert x2c.stride() == x2.stride() and x2c.stride(1) != 1
+    out2 = linear_layer(x2c, w.cuda(), b.cuda())
+    torch.cuda.synchronize()
+    close(out2, linear_oracle(x2, w, b, ""), what="linear 2-D column-major x")
+
+
+def test_linear_saves_activation_inputs(close):
+    gen = torch.Generator().manual_seed(3)
+    M, N, K = 384, 512, 256
+    x, w, b = _inputs(M, N, K, torch.float16, gen, w_std=K ** -0.5)
+    act_in = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation="gelu", act_inputs=act_in)
+    torch.cuda.synchronize()
+    ref, pre = linear_oracle(x, w, b, "gelu", return_act_inputs=True)
+    close(out, ref, what="linear out")
+    close(act_in, pre, what="linear act_inputs")
+
+
+@pytest.mark.parametrize("which", ["up", "down"])
+def test_linear_config2_full_size(which, close):
+    # BASELINE config 2: up-projection [16384,768]x[3072,768]ᵀ + bias + tanh-GELU; down-projection back, no activation
+    gen = torch.Generator().manual_seed(0)
+    if which == "up":
+        M, N, K, act = 16384, 3072, 768, "fast_gelu"
+    else:
+        M, N, K, act = 16384, 768, 3072, ""
+    x = torch.randn((M, K), generator=gen).half()
+    w = (torch.randn((N, K), generator=gen) * 0.02).half()
+    b = (torch.randn((N,), generator=gen) * 0.02).half()
+    out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation=act)
+    torch.cuda.synchronize()
+    ref = linear_oracle(x, w, b, act)
+    close(out, ref, scale=max(1.0, ref.abs().max().item() / 4), what=f"config 2 {which}")
+    # linearity in x (size independent): f(2x) - b = 2 (f(x) - b) holds exactly in fp16 for the no-activation case
+    if act == "":
+        nb = linear_layer(x.cuda(), w.cuda(), None)
+        nb2 = linear_layer((x * 2).cuda(), w.cuda(), None)
+        torch.cuda.synchronize()
+        assert torch.equal(nb2.cpu(), (nb * 2).cpu())
+
+
+def test_linear_rejects_bad_arguments():
+    x = torch.zeros((4, 8), dtype=torch.float16, device="cuda")
+    w = torch.zeros((16, 8), dtype=torch.float16, device="cuda")
+    with pytest.raises(AssertionError):
+        linear_layer(x, w.float(), None)  # dtype mismatch
+    with pytest.raises(AssertionError):
+        linear_layer(x, torch.zeros((16, 9), dtype=torch.float16, device="cuda"), None)  # K mismatch
+    with pytest.raises(AssertionError):
+        linear_layer(x, w.t().contiguous().t(), None)  # weight must be contiguous
+    with pytest.raises(AssertionError):
+        linear_layer(x, w, torch.zeros((15,), dtype=torch.float16, device="cuda"))  # bias size
+
+
+def test_unknown_activation_is_identity(close):
+    gen = torch.Generator().manual_seed(4)
+    x, w, b = _inputs(64, 64, 64, torch.float16, gen, w_std=0.125)
+    out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation="swish-not-a-name")
+    torch.cuda.synchronize()
+    close(out, linear_oracle(x, w, b, ""), what="unknown activation")
