@@ -105,12 +105,13 @@ def test_linear_config2_full_size(which, close):
     torch.cuda.synchronize()
     ref = linear_oracle(x, w, b, act)
     close(out, ref, scale=max(1.0, ref.abs().max().item() / 4), what=f"config 2 {which}")
-    # linearity in x (size independent): f(2x) - b = 2 (f(x) - b) holds exactly in fp16 for the no-activation case
+    # linearity in x (size independent): without bias and activation f(2x) = 2 f(x); scaling by 2 is exact in
+    # fp32 and in fp16, except that a subnormal fp16 result gains one bit when doubled (spacing 2^-24)
     if act == "":
         nb = linear_layer(x.cuda(), w.cuda(), None)
         nb2 = linear_layer((x * 2).cuda(), w.cuda(), None)
         torch.cuda.synchronize()
-        assert torch.equal(nb2.cpu(), (nb * 2).cpu())
+        assert (nb2.float() - nb.float() * 2).abs().max().item() <= 2.0 ** -23
 
 
 def test_linear_rejects_bad_arguments():
