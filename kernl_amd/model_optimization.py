@@ -1,0 +1,46 @@
+"""`optimize_model`: the public entry point (reference: src/kernl/model_optimization.py:27-66).
+
+The model's `forward` is wrapped in TorchDynamo with a backend that (1) rewrites the captured torch.fx graph so that
+attention, linear(+activation) and LayerNorm/RMSNorm sub-graphs call the fused gfx950 kernels and (2) captures the
+rewritten graph in a hipGraph fed from a static input pool.
+"""
+from typing import List
+
+import torch
+import torch._dynamo as torchdynamo
+
+from kernl_amd import _lib
+from kernl_amd.optimizer.cuda_graph import cuda_graphs_wrapper, static_inputs_pool
+from kernl_amd.optimizer.dynamo_backend import dynamo_backend_ofi
+
+
+# Module level so that several forwards of one model (encoder / decoder) share it
+# (reference: model_optimization.py:25-29).
+def _compiler(gm: torch.fx.GraphModule, example_inputs: List[torch.Tensor]):
+    dynamo_backend_ofi(gm)
+    return cuda_graphs_wrapper(gm, example_inputs)
+
+
+def optimize_model(model: torch.nn.Module) -> None:
+    """Replace `model.forward` by the optimized version, in place; the original stays as `model.forward_original`.
+
+        model = AutoModel.from_pretrained(...).eval().cuda()
+        optimize_model(model)
+        model(**inputs)
+
+    Needs a gfx950 (MI355X) device, the model on it, and the built `libkernl_hip.so`; there is no fallback.
+    """
+    assert torch.cuda.is_available(), "A ROCm GPU is required to use kernl_amd"
+    arch = getattr(torch.cuda.get_device_properties(torch.cuda.current_device()), "gcnArchName", "")
+    if not arch.startswith("gfx950"):
+        raise RuntimeError(f"kernl_amd kernels are built for gfx950 (MI355X) only, found '{arch}'")
+    assert next(model.parameters()).device.type == "cuda", "Model must be on GPU"
+    _lib.load()  # fail now, not in the middle of the first forward
+    static_inputs_pool.clear()
+    model.forward_original = model.forward
+
+    @torchdynamo.optimize(_compiler)
+    def run(*args, **kwargs):
+        return model.forward_original(*args, **kwargs)
+
+    model.forward = run

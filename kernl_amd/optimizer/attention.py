@@ -1,0 +1,218 @@
+"""Attention graph patterns (reference: src/kernl/optimizer/attention.py:24-112).
+
+`attention_wrapper` is the fx leaf the rewritten graph calls.  Patterns 1-3 are the reference's (BERT `/ 8.0 + mask`,
+T5 `+ position_bias` with float softmax, Whisper bmm); the wildcard-scale and `scaled_dot_product_attention` patterns
+cover what current transformers versions emit.
+"""
+from typing import Optional
+
+import torch
+
+from kernl_amd.implementations.attention import attention_forward
+from kernl_amd.utils.extended_matcher import replace_pattern
+
+
+def _per_key_view(mask: torch.Tensor) -> torch.Tensor:
+    """A mask that was `expand`ed over the query dimension carries one value per key: look at a single row."""
+    if mask.dim() == 4 and mask.size(2) > 1 and mask.stride(2) == 0:
+        return mask[:, :, :1, :]
+    return mask
+
+
+def attention_wrapper(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    output: torch.Tensor,
+    sm_scale: float,
+    is_causal: bool,
+    attention_mask: Optional[torch.Tensor],
+) -> torch.Tensor:
+    # bmm-shaped tensors use their first dimension for batch and heads together; the kernel wants 4 dimensions
+    extend_head = q.dim() == 3
+    if extend_head:
+        q, k, v, output = q.unsqueeze(1), k.unsqueeze(1), v.unsqueeze(1), output.unsqueeze(1)
+        if attention_mask is not None and attention_mask.dim() == 3:
+            attention_mask = attention_mask.unsqueeze(1)
+    if attention_mask is not None:
+        attention_mask = _per_key_view(attention_mask)
+    # The reference hands single-query attention over long keys to a split-K kernel or to eager PyTorch
+    # (optimizer/attention.py:45-49); the HIP kernel covers that shape itself.
+    attention_forward(q, k, v, output, sm_scale, is_causal=is_causal, attention_mask=attention_mask)
+    if extend_head:
+        output = output.squeeze(1)
+    return output
+
+
+def sdpa_wrapper(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    attn_mask: Optional[torch.Tensor],
+    scale: Optional[float],
+    is_causal: bool,
+    assume_causal: bool,
+) -> torch.Tensor:
+    """`F.scaled_dot_product_attention(q, k, v, attn_mask, 0.0, is_causal, scale)` on the fused kernel.  A boolean
+    mask (True = attend) becomes the additive 0 / -inf mask the kernel takes."""
+    if scale is None:
+        scale = q.size(-1) ** -0.5
+    mask = attn_mask
+    if mask is not None:
+        while mask.dim() < 4:
+            mask = mask.unsqueeze(0)
+        mask = _per_key_view(mask)
+        if mask.dtype == torch.bool:
+            mask = torch.zeros(mask.shape, dtype=torch.float32, device=mask.device).masked_fill_(~mask, float("-inf"))
+    output = torch.empty_like(q)
+    return attention_wrapper(q, k, v, output, float(scale), bool(is_causal) or assume_causal, mask)
+
+
+torch.fx.wrap("attention_wrapper")
+torch.fx.wrap("sdpa_wrapper")
+
+
+def fuse_attention_pattern_1(gm: torch.fx.GraphModule, is_causal: bool):
+    """BERT as the reference saw it: softmax(q·kᵀ / 8.0 + mask)·v."""
+
+    def pattern(q, k, attention_mask, v):
+        transpose_10 = k.transpose(-1, -2)
+        matmul_20 = torch.matmul(q, transpose_10)
+        truediv_10 = matmul_20 / 8.0
+        add_30 = truediv_10 + attention_mask
+        softmax_10 = torch.nn.functional.softmax(add_30, dim=-1)
+        matmul_21 = torch.matmul(softmax_10, v)
+        return matmul_21
+
+    def replace(q, k, attention_mask, v):
+        output = torch.empty_like(q)
+        output = attention_wrapper(q, k, v, output, 1 / 8.0, is_causal, attention_mask)
+        return output
+
+    replace_pattern(gm, pattern, replace)
+
+
+def fuse_attention_pattern_2(gm: torch.fx.GraphModule, is_causal: bool):
+    """T5: scores + position_bias, softmax in float, cast back; no scaling."""
+
+    def pattern(q, k, encoder_decoder_position_bias, v):
+        transpose_3 = k.transpose(3, 2)
+        matmul = torch.matmul(q, transpose_3)
+        add_2 = torch.add(matmul, encoder_decoder_position_bias)
+        float_1 = add_2.float()
+        softmax = torch.nn.functional.softmax(float_1, dim=-1)
+        type_as = softmax.type_as(add_2)
+        matmul_1 = torch.matmul(type_as, v)
+        return matmul_1
+
+    def replace(q, k, encoder_decoder_position_bias, v):
+        output = torch.empty_like(q)
+        output = attention_wrapper(q, k, v, output, 1.0, is_causal, encoder_decoder_position_bias)
+        return output
+
+    replace_pattern(gm, pattern, replace)
+
+
+def fuse_attention_pattern_3(gm: torch.fx.GraphModule, is_causal: bool):
+    """Whisper: bmm-shaped, pre-scaled q, no mask."""
+
+    def pattern(q, k, v):
+        transpose_46 = k.transpose(1, 2)
+        bmm_22 = torch.bmm(q, transpose_46)
+        softmax_11 = torch.nn.functional.softmax(bmm_22, dim=-1)
+        bmm_23 = torch.bmm(softmax_11, v)
+        return bmm_23
+
+    def replace(q, k, v):
+        output = torch.empty_like(q)
+        output = attention_wrapper(q, k, v, output, 1.0, is_causal, None)
+        return output
+
+    replace_pattern(gm, pattern, replace)
+
+
+_TRANSPOSES = ((-1, -2), (-2, -1), (2, 3), (3, 2))
+
+
+def _scaled_patterns(d0: int, d1: int, is_causal: bool):
+    """(pattern, replacement) pairs for one spelling of the key transposition.  `literal_scale` only binds to a python
+    number in the graph (the kernel takes the scale as a host float)."""
+
+    def pattern_mul_mask(q, k, literal_scale, attention_mask, v):
+        scores = torch.matmul(q, k.transpose(d0, d1)) * literal_scale
+        probs = torch.nn.functional.softmax(scores + attention_mask, dim=-1)
+        return torch.matmul(probs, v)
+
+    def replace_mul_mask(q, k, literal_scale, attention_mask, v):
+        output = torch.empty_like(q)
+        return attention_wrapper(q, k, v, output, literal_scale, is_causal, attention_mask)
+
+    def pattern_div_mask(q, k, literal_scale, attention_mask, v):
+        scores = torch.matmul(q, k.transpose(d0, d1)) / literal_scale
+        probs = torch.nn.functional.softmax(scores + attention_mask, dim=-1)
+        return torch.matmul(probs, v)
+
+    def replace_div_mask(q, k, literal_scale, attention_mask, v):
+        output = torch.empty_like(q)
+        return attention_wrapper(q, k, v, output, 1.0 / literal_scale, is_causal, attention_mask)
+
+    def pattern_mul(q, k, literal_scale, v):
+        scores = torch.matmul(q, k.transpose(d0, d1)) * literal_scale
+        probs = torch.nn.functional.softmax(scores, dim=-1)
+        return torch.matmul(probs, v)
+
+    def replace_mul(q, k, literal_scale, v):
+        output = torch.empty_like(q)
+        return attention_wrapper(q, k, v, output, literal_scale, is_causal, None)
+
+    def pattern_div(q, k, literal_scale, v):
+        scores = torch.matmul(q, k.transpose(d0, d1)) / literal_scale
+        probs = torch.nn.functional.softmax(scores, dim=-1)
+        return torch.matmul(probs, v)
+
+    def replace_div(q, k, literal_scale, v):
+        output = torch.empty_like(q)
+        return attention_wrapper(q, k, v, output, 1.0 / literal_scale, is_causal, None)
+
+    return (
+        (pattern_mul_mask, replace_mul_mask),
+        (pattern_div_mask, replace_div_mask),
+        (pattern_mul, replace_mul),
+        (pattern_div, replace_div),
+    )
+
+
+def fuse_attention_scaled(gm: torch.fx.GraphModule, is_causal: bool):
+    """softmax(q·kᵀ {*, /} s (+ mask))·v for ANY literal scale `s`: what eager attention of current transformers models
+    traces to (`matmul(q, k.transpose(2, 3)) * scaling + mask`).  The scale is a wildcard bound to the graph's literal."""
+    for d0, d1 in _TRANSPOSES:
+        for pattern, replacement in _scaled_patterns(d0, d1, is_causal):
+            replace_pattern(gm, pattern, replacement)
+
+
+def fuse_attention_sdpa(gm: torch.fx.GraphModule, is_causal: bool):
+    """`F.scaled_dot_product_attention` without dropout."""
+    sdpa = torch.nn.functional.scaled_dot_product_attention
+    for node in list(gm.graph.nodes):
+        if node.op != "call_function" or node.target is not sdpa:
+            continue
+        pair = node.normalized_arguments(gm, normalize_to_only_use_kwargs=True)
+        kwargs = dict(pair.kwargs) if pair is not None else None
+        if kwargs is None:
+            names = ("query", "key", "value", "attn_mask", "dropout_p", "is_causal", "scale", "enable_gqa")
+            kwargs = dict(zip(names, node.args))
+            kwargs.update(node.kwargs)
+        if kwargs.get("dropout_p", 0.0) != 0.0 or kwargs.get("enable_gqa", False):
+            continue
+        scale, causal = kwargs.get("scale"), kwargs.get("is_causal", False)
+        if isinstance(scale, torch.fx.Node) or isinstance(causal, torch.fx.Node):
+            continue
+        with gm.graph.inserting_before(node):
+            new = gm.graph.call_function(
+                sdpa_wrapper,
+                (kwargs["query"], kwargs["key"], kwargs["value"], kwargs.get("attn_mask"), scale, causal, is_causal),
+            )
+        node.replace_all_uses_with(new)
+        gm.graph.erase_node(node)
+    gm.graph.lint()
+    gm.recompile()

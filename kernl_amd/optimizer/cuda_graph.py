@@ -1,0 +1,143 @@
+"""hipGraph capture of a rewritten graph, fed from a static input pool
+(reference: src/kernl/optimizer/cuda_graph.py:26-138).
+
+The reference delegates capture to torch-inductor's `cudagraphify_impl`; here the capture is done directly with
+`torch.cuda.CUDAGraph` (hipGraph on ROCm): a warm-up call on a side stream, one capture, then every call copies the
+caller's tensors into the pool slots the graph reads and replays.  The kernels behind the fused operators launch on
+torch's current stream and neither allocate outside torch's caching allocator nor synchronise, which is what stream
+capture needs.
+
+Inputs that live at a fixed address for the life of the model — parameters and buffers, which torch.compile passes
+to a backend as graph inputs — are used in place; only real per-call inputs go through the pool.
+"""
+import math
+from typing import Callable, Iterable, List, Optional, Sequence, Union
+
+import torch
+from torch._subclasses import FakeTensor
+
+from kernl_amd.optimizer.pool_cuda_graphs import CudaGraphPool, get_aligned_size
+
+static_inputs_pool: List[CudaGraphPool] = []
+
+
+def get_pool_size(inputs: List[torch.Tensor], existing_pools: List[CudaGraphPool]) -> int:
+    """Bytes for a new pool: the aligned sizes of `inputs`, at least as large as any existing pool, rounded up to a
+    power of two while below 1 GiB so that few, reusable pools get created (reference: cuda_graph.py:29-44)."""
+    size = sum(get_aligned_size(p) for p in inputs)
+    size = max([size] + [p.size for p in existing_pools])
+    if size < 1024 * 1024 * 1024:
+        size = 2 ** math.ceil(math.log2(size))
+    return max(size, 8)
+
+
+def argsort(iterable: Iterable, key: Callable) -> List[int]:
+    """Indices that sort `iterable` by `key`, stable (known answer: test/test_cuda_graph.py:8)."""
+    return [i for i, _ in sorted(enumerate(iterable), key=lambda pair: key(pair[1]))]
+
+
+def prepare_inputs(inputs: Sequence[torch.Tensor], pools: List[CudaGraphPool]) -> List[torch.Tensor]:
+    """Copy `inputs` into pool memory and return the copies, in input order.
+
+    Placement follows the reference (cuda_graph.py:57-100): rewind every pool, visit pools smallest first and inputs
+    in increasing storage size, put each input into the first pool with room; inputs that fit nowhere share ONE new
+    pool sized by `get_pool_size`.  The procedure is deterministic, so the same input signature always lands on the
+    same addresses — the property graph replay relies on.
+    """
+    for p in pools:
+        p.reset()
+    pools.sort(key=lambda p: p.size)
+    order = argsort(inputs, key=lambda t: t.untyped_storage().nbytes())
+    copies: List[Optional[torch.Tensor]] = [None] * len(inputs)
+    homeless: List[int] = []
+    for idx in order:
+        t = inputs[idx]
+        for pool in pools:
+            if pool.can_store(t):
+                copies[idx] = pool.copy_to_pool(t)
+                break
+        else:
+            homeless.append(idx)
+    if homeless:
+        pool = CudaGraphPool(get_pool_size([inputs[i] for i in homeless], pools), device=inputs[homeless[0]].device)
+        pools.append(pool)
+        for idx in homeless:
+            assert pool.can_store(inputs[idx])
+            copies[idx] = pool.copy_to_pool(inputs[idx])
+    return copies
+
+
+def _is_static_address(t) -> bool:
+    """Parameters and buffers handed over by torch.compile keep their address between calls."""
+    if not isinstance(t, torch.Tensor):
+        return True  # python scalars / symbolic ints are baked into the capture
+    if isinstance(t, torch.nn.Parameter):
+        return True
+    return getattr(t, "_dynamo_static_input_type", None) is not None
+
+
+class _CapturedGraph:
+    """One captured hipGraph of `model` for one input signature."""
+
+    def __init__(self, model: Callable, inputs: Sequence, static_idx: Sequence[int]):
+        self.static_idx = set(static_idx)
+        self.dynamic_idx = [i for i in range(len(inputs)) if i not in self.static_idx]
+        self.pools = static_inputs_pool
+        self.graph_inputs = list(inputs)
+        copies = prepare_inputs([inputs[i] for i in self.dynamic_idx], self.pools) if self.dynamic_idx else []
+        for i, c in zip(self.dynamic_idx, copies):
+            self.graph_inputs[i] = c
+        self.static_ptrs = {i: inputs[i].data_ptr() for i in self.static_idx if isinstance(inputs[i], torch.Tensor)}
+        device = next((t.device for t in inputs if isinstance(t, torch.Tensor) and t.is_cuda), torch.device("cuda"))
+        # warm-up outside capture: kernel modules get loaded, one-time parameter casts happen, and kernels that
+        # mutate their inputs do so once before the capture (reference: cuda_graph.py:115)
+        side = torch.cuda.Stream(device=device)
+        side.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(side):
+            model(*self.graph_inputs)
+        torch.cuda.current_stream(device).wait_stream(side)
+        torch.cuda.synchronize(device)
+        # parameters may have been re-allocated by the one-time cast: record their final addresses
+        self.static_ptrs = {i: inputs[i].data_ptr() for i in self.static_idx if isinstance(inputs[i], torch.Tensor)}
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=side):
+            out = model(*self.graph_inputs)
+        self.outputs = out
+        torch.cuda.synchronize(device)
+
+    def matches(self, args: Sequence) -> bool:
+        for i, ptr in self.static_ptrs.items():
+            if args[i].data_ptr() != ptr:
+                return False
+        return True
+
+    def __call__(self, *args):
+        if self.dynamic_idx:
+            copies = prepare_inputs([args[i] for i in self.dynamic_idx], self.pools)
+            for i, c in zip(self.dynamic_idx, copies):
+                # same signature => same placement; anything else would replay on stale addresses
+                assert c.data_ptr() == self.graph_inputs[i].data_ptr(), "static input pool placement changed"
+        self.graph.replay()
+        return self.outputs
+
+
+def cuda_graphs_wrapper(model: Callable, inputs: Union[list, tuple]) -> Callable:
+    """Returns a callable with `model`'s signature that replays a captured hipGraph.
+
+    As in the reference (cuda_graph.py:103-138): with real example inputs the capture happens here; with FakeTensor
+    example inputs (torch.compile's default) it is deferred to the first call with real tensors.  The returned
+    outputs are the graph's STATIC output buffers: they are overwritten by the next call.
+    """
+    assert isinstance(inputs, (list, tuple))
+    static_idx = [i for i, t in enumerate(inputs) if _is_static_address(t)]
+    captured: Optional[_CapturedGraph] = None
+
+    def run(*args):
+        nonlocal captured
+        if captured is None or not captured.matches(args):
+            captured = _CapturedGraph(model, list(args), static_idx)
+        return captured(*args)
+
+    if not any(isinstance(t, FakeTensor) for t in inputs):
+        captured = _CapturedGraph(model, list(inputs), static_idx)
+    return run

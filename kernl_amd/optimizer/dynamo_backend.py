@@ -1,0 +1,32 @@
+"""The ordered rewrite pipeline applied to every graph TorchDynamo captures
+(reference: src/kernl/optimizer/dynamo_backend.py:25-34)."""
+import torch
+
+from kernl_amd.optimizer.attention import (
+    fuse_attention_pattern_1,
+    fuse_attention_pattern_2,
+    fuse_attention_pattern_3,
+    fuse_attention_scaled,
+    fuse_attention_sdpa,
+)
+from kernl_amd.optimizer.dropout import remove_dropout
+from kernl_amd.optimizer.layer_norm import replace_layer_norm, replace_layer_norm_fn, replace_layer_norm_rms
+from kernl_amd.optimizer.linear import replace_all_linear
+from kernl_amd.optimizer.mask import sink_expand_below_where
+from kernl_amd.optimizer.normalizer import normalize_operators
+
+
+def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
+    normalize_operators(gm)
+    remove_dropout(gm)
+    sink_expand_below_where(gm)
+    fuse_attention_pattern_1(gm, assume_causal)
+    fuse_attention_pattern_2(gm, assume_causal)
+    fuse_attention_pattern_3(gm, assume_causal)
+    fuse_attention_scaled(gm, assume_causal)
+    fuse_attention_sdpa(gm, assume_causal)
+    replace_all_linear(gm)
+    replace_layer_norm(gm)
+    replace_layer_norm_fn(gm)
+    replace_layer_norm_rms(gm)
+    return gm

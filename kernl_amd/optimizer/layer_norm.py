@@ -1,0 +1,126 @@
+"""LayerNorm / RMSNorm graph patterns (reference: src/kernl/optimizer/layer_norm.py:22-74).
+
+Module-form patterns are the reference's.  The functional forms are what torch.compile hands to a backend today
+(`F.layer_norm(x, shape, weight, bias, eps)` on lifted parameters); eps and the RMSNorm epsilon are wildcards bound to
+the graph's literal, so a Llama norm with eps 1e-5 matches as well as T5's 1e-6.  A LayerNorm whose input is
+`a + b` with no other consumer is rewritten to the fused add+LayerNorm kernel.
+"""
+import torch
+
+from kernl_amd.implementations.layer_norm import add_layer_norm, layer_norm
+from kernl_amd.utils.extended_matcher import replace_pattern
+
+
+def _half_params_once(v: torch.Tensor, *params) -> None:
+    # one-time in-place down-cast, as the reference does (optimizer/layer_norm.py:24-27)
+    if v.dtype == torch.float16 or torch.is_autocast_enabled("cuda"):
+        for p in params:
+            if p is not None and p.dtype == torch.float32:
+                p.data = p.data.half()
+
+
+def layer_norm_wrapper(v: torch.Tensor, layernorm: torch.nn.LayerNorm):
+    _half_params_once(v, layernorm.weight, layernorm.bias)
+    return layer_norm(v, layernorm.weight, layernorm.bias, layernorm.eps)
+
+
+def layer_norm_wrapper_functional(v: torch.Tensor, normalized_shape, weight, bias, eps: float):
+    if len(normalized_shape) != 1 or weight is None:
+        return torch.nn.functional.layer_norm(v, normalized_shape, weight, bias, eps)
+    _half_params_once(v, weight, bias)
+    return layer_norm(v, weight, bias, eps)
+
+
+def add_layer_norm_wrapper_functional(a: torch.Tensor, b: torch.Tensor, normalized_shape, weight, bias, eps: float):
+    if (
+        len(normalized_shape) != 1
+        or weight is None
+        or not isinstance(a, torch.Tensor)
+        or not isinstance(b, torch.Tensor)
+        or a.shape != b.shape
+        or a.dtype != b.dtype
+    ):
+        return torch.nn.functional.layer_norm(a + b, normalized_shape, weight, bias, eps)
+    _half_params_once(a, weight, bias)
+    return add_layer_norm(a, b, weight, bias, eps)
+
+
+def layer_norm_rms_wrapper(v: torch.Tensor, weight: torch.Tensor, eps: float):
+    if weight.dtype != v.dtype:
+        weight = weight.to(v.dtype)
+    return layer_norm(v, weight, None, eps, None, use_rms_norm=True)
+
+
+torch.fx.wrap("layer_norm_wrapper")
+torch.fx.wrap("layer_norm_wrapper_functional")
+torch.fx.wrap("add_layer_norm_wrapper_functional")
+torch.fx.wrap("layer_norm_rms_wrapper")
+
+
+def replace_layer_norm(gm: torch.fx.GraphModule):
+    class Pattern(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layernorm = torch.nn.LayerNorm((1, 1))
+
+        def forward(self, v):
+            return self.layernorm(v)
+
+    class Replacement(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layernorm = torch.nn.LayerNorm((1, 1))
+
+        def forward(self, v):
+            return layer_norm_wrapper(v, self.layernorm)
+
+    replace_pattern(gm, Pattern(), Replacement())
+
+
+def replace_layer_norm_fn(gm: torch.fx.GraphModule):
+    def pattern_add(a, b, literal_shape, weight, bias, literal_eps):
+        return torch.nn.functional.layer_norm(a + b, literal_shape, weight, bias, literal_eps)
+
+    def replace_add(a, b, literal_shape, weight, bias, literal_eps):
+        return add_layer_norm_wrapper_functional(a, b, literal_shape, weight, bias, literal_eps)
+
+    def pattern(v, literal_shape, weight, bias, literal_eps):
+        return torch.nn.functional.layer_norm(v, literal_shape, weight, bias, literal_eps)
+
+    def replace(v, literal_shape, weight, bias, literal_eps):
+        return layer_norm_wrapper_functional(v, literal_shape, weight, bias, literal_eps)
+
+    replace_pattern(gm, pattern_add, replace_add)
+    replace_pattern(gm, pattern, replace)
+
+
+def replace_layer_norm_rms(gm: torch.fx.GraphModule):
+    # T5 spelling (reference pattern, eps generalised from the literal 1e-06)
+    def pattern(v, weight, literal_eps):
+        to_38 = v.to(torch.float32)
+        pow_32 = to_38.pow(2)
+        mean_31 = pow_32.mean(-1, keepdim=True)
+        add_68 = mean_31 + literal_eps
+        rsqrt_31 = torch.rsqrt(add_68)
+        mul_69 = v * rsqrt_31
+        mul_70 = weight * mul_69
+        return mul_70
+
+    def replace(v, weight, literal_eps):
+        return layer_norm_rms_wrapper(v, weight, literal_eps)
+
+    replace_pattern(gm, pattern, replace)
+
+    # Llama spelling: normalise the fp32 copy, cast back to the input dtype, then scale
+    for dtype in (torch.float16, torch.bfloat16, torch.float32):
+
+        def make(dtype):
+            def pattern_llama(v, weight, literal_eps):
+                h = v.to(torch.float32)
+                variance = h.pow(2).mean(-1, keepdim=True)
+                h2 = h * torch.rsqrt(variance + literal_eps)
+                return weight * h2.to(dtype)
+
+            return pattern_llama
+
+        replace_pattern(gm, make(dtype), replace)

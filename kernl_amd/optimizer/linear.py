@@ -1,0 +1,143 @@
+"""Linear-layer graph patterns (reference: src/kernl/optimizer/linear.py:24-115).
+
+`linear_wrapper` (module form) and `linear_wrapper_functional` are the fx leaves the rewritten graph calls.  Fused
+activation patterns run before the bare ones, as in the reference (:109-115).  torch.compile now hands `nn.Linear`
+to a backend as `F.linear(x, weight, bias)` on lifted parameters, so the functional patterns carry the same set of
+activations as the module ones.
+"""
+from typing import Callable
+
+import torch
+
+from kernl_amd.implementations.linear_layer import linear_layer
+from kernl_amd.utils.extended_matcher import replace_pattern
+
+
+def linear_wrapper(v: torch.Tensor, linear: torch.nn.Linear, activation=""):
+    return linear_wrapper_functional(v, linear.weight, linear.bias, activation=activation)
+
+
+torch.fx.wrap("linear_wrapper")
+
+
+def linear_wrapper_functional(v: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, activation=""):
+    # One-time, in-place down-cast of fp32 parameters so they are not converted on every call
+    # (reference: optimizer/linear.py:33-36).  Only when the activations already are fp16 or autocast will make them so.
+    if weight.dtype == torch.float32 and (v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")):
+        weight.data = weight.data.half()
+    if bias is not None and bias.dtype == torch.float32 and (v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")):
+        bias.data = bias.data.half()
+    if not weight.is_contiguous():
+        weight = weight.contiguous()
+    return linear_layer(v, weight, bias, activation=activation)
+
+
+torch.fx.wrap("linear_wrapper_functional")
+
+
+def replace_linear_activation(gm: torch.fx.GraphModule, activation_module: Callable, activation: str):
+    class Pattern(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.linear = torch.nn.Linear(1, 1)
+            self.activation = activation_module
+
+        def forward(self, v):
+            return self.activation(self.linear(v))
+
+    class Replacement(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.linear = torch.nn.Linear(1, 1)
+            self.activation = activation_module
+
+        def forward(self, v):
+            return linear_wrapper(v, self.linear, activation=activation)
+
+    replace_pattern(gm, Pattern(), Replacement())
+
+
+def replace_linear(gm: torch.fx.GraphModule):
+    class Pattern(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.linear = torch.nn.Linear(1, 1)
+
+        def forward(self, v):
+            return self.linear(v)
+
+    class Replacement(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.linear = torch.nn.Linear(1, 1)
+
+        def forward(self, v):
+            return linear_wrapper(v, self.linear)
+
+    replace_pattern(gm, Pattern(), Replacement())
+
+
+def _functional_activation_patterns():
+    F = torch.nn.functional
+    return (
+        (lambda t: F.gelu(t), "gelu"),
+        (lambda t: F.gelu(t, approximate="tanh"), "fast_gelu"),
+        (lambda t: torch.tanh(t), "tanh"),
+        (lambda t: F.tanh(t), "tanh"),
+        (lambda t: t.tanh(), "tanh"),
+        (lambda t: F.relu(t), "relu"),
+        (lambda t: torch.relu(t), "relu"),
+        (lambda t: F.silu(t), "silu"),
+    )
+
+
+def replace_linear_fn_activation(gm: torch.fx.GraphModule):
+    """activation(F.linear(v, weight, bias)) -> one fused call.  `bias` also binds to the literal None."""
+    for act_fn, name in _functional_activation_patterns():
+
+        def make(act_fn, name):
+            def pattern(v, weight, bias):
+                return act_fn(torch.nn.functional.linear(v, weight, bias))
+
+            def replace(v, weight, bias):
+                return linear_wrapper_functional(v, weight, bias, activation=name)
+
+            return pattern, replace
+
+        pat, rep = make(act_fn, name)
+        replace_pattern(gm, pat, rep)
+
+
+def replace_linear_fn(gm: torch.fx.GraphModule):
+    def pattern(v, weight, bias):
+        return torch.nn.functional.linear(v, weight, bias)
+
+    def replace(v, weight, bias):
+        output = linear_wrapper_functional(v, weight, bias)
+        return output
+
+    replace_pattern(gm, pattern, replace)
+
+
+def replace_linear_fn_constant_match(gm: torch.fx.GraphModule):
+    """F.linear(v, weight, None) spelled with a literal None (reference: optimizer/linear.py:97-106).  The wildcard
+    `bias` of `replace_linear_fn` already binds to None; kept so the reference's pass list maps one to one."""
+
+    def pattern(v, weight):
+        return torch.nn.functional.linear(v, weight, None)
+
+    def replace(v, weight):
+        output = linear_wrapper_functional(v, weight, None)
+        return output
+
+    replace_pattern(gm, pattern, replace)
+
+
+def replace_all_linear(gm: torch.fx.GraphModule):
+    replace_linear_activation(gm, torch.nn.Tanh(), "tanh")
+    replace_linear_activation(gm, torch.nn.ReLU(), "relu")
+    replace_linear_activation(gm, torch.nn.functional.gelu, "gelu")
+    replace_linear_fn_activation(gm)
+    replace_linear(gm)
+    replace_linear_fn(gm)
+    replace_linear_fn_constant_match(gm)
