@@ -39,7 +39,9 @@ def optimize_model(model: torch.nn.Module) -> None:
     static_inputs_pool.clear()
     model.forward_original = model.forward
 
-    @torchdynamo.optimize(_compiler)
+    # Static shapes: a hipGraph is specific to its shapes, so every new input shape is a new (cached) compilation,
+    # exactly as with the reference's default TorchDynamo settings.
+    @torchdynamo.optimize(_compiler, dynamic=False)
     def run(*args, **kwargs):
         return model.forward_original(*args, **kwargs)
 

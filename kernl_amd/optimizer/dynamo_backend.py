@@ -12,13 +12,14 @@ from kernl_amd.optimizer.attention import (
 from kernl_amd.optimizer.dropout import remove_dropout
 from kernl_amd.optimizer.layer_norm import replace_layer_norm, replace_layer_norm_fn, replace_layer_norm_rms
 from kernl_amd.optimizer.linear import replace_all_linear
-from kernl_amd.optimizer.mask import sink_expand_below_where
+from kernl_amd.optimizer.mask import scalar_tensors_to_full, sink_expand_below_where
 from kernl_amd.optimizer.normalizer import normalize_operators
 
 
 def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
     normalize_operators(gm)
     remove_dropout(gm)
+    scalar_tensors_to_full(gm)
     sink_expand_below_where(gm)
     fuse_attention_pattern_1(gm, assume_causal)
     fuse_attention_pattern_2(gm, assume_causal)

@@ -17,7 +17,33 @@ def _is_scalar(value) -> bool:
     if isinstance(value, Node):
         if value.op == "call_function" and value.target is torch.tensor and value.args and isinstance(value.args[0], (int, float)):
             return True
+        if value.op == "call_function" and value.target is torch.full and len(value.args) >= 2 and value.args[0] == ():
+            return True
     return False
+
+
+def scalar_tensors_to_full(gm: torch.fx.GraphModule):
+    """`torch.tensor(<python number>, device=gpu)` is a copy from pageable host memory, which stream capture refuses;
+    `torch.full((), number, ...)` builds the same 0-d tensor with a fill kernel."""
+    changed = False
+    for node in list(gm.graph.nodes):
+        if node.op != "call_function" or node.target is not torch.tensor:
+            continue
+        if len(node.args) != 1 or not isinstance(node.args[0], (int, float)) or isinstance(node.args[0], bool):
+            continue
+        kwargs = {k: v for k, v in node.kwargs.items() if k in ("dtype", "device")}
+        if set(node.kwargs) - {"dtype", "device", "requires_grad"}:
+            continue
+        if "dtype" not in kwargs:
+            kwargs["dtype"] = torch.get_default_dtype() if isinstance(node.args[0], float) else torch.int64
+        with gm.graph.inserting_before(node):
+            full = gm.graph.call_function(torch.full, ((), node.args[0]), kwargs)
+        node.replace_all_uses_with(full)
+        gm.graph.erase_node(node)
+        changed = True
+    if changed:
+        gm.graph.lint()
+        gm.recompile()
 
 
 def sink_expand_below_where(gm: torch.fx.GraphModule):
