@@ -1,0 +1,289 @@
+#!/usr/bin/env python3
+"""Headline benchmark on ONE MI355X:  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one fused-attention forward over BASELINE config 1: q, k, v fp16 [32, 12, 512, 64] ~ N(0, 1),
+scale 1/8, non-causal, additive padding mask from per-sequence lengths U[256, 512] with -inf beyond the length.
+Inputs are generated on the CPU with seed 0, moved to HBM before the timed region, and W warm-up steps are run.
+
+One JSON line is printed:
+  value / ms_per_step   wall clock over exactly K back-to-back steps between two device synchronisations, expressed
+                        with the DENSE flop count 4·B·H·M·N·D (padded keys counted);
+  roofline              the attention kernel against the fp16 dense MFMA peak; `achieved` uses the same dense flop
+                        count over the average launch duration measured with HIP events around every launch of the
+                        timed region (on torch's current stream, which is where the kernels are launched);
+  cpu_baseline          the CPU oracle (fp32 eager PyTorch on the host cores) on a bounded sample of the same workload;
+  extra                 the other numbers the metric names: executed (skip-aware) attention flops, fused linear and
+                        LayerNorm at BASELINE config 2, BERT-base b32 s512 fp16 forward latency through
+                        `optimize_model` (hipGraph replay, median wall clock of 10), and CPU timings beside them.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_MFMA_F16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
+PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E
+
+
+def _event_times(fn, n, flush=None):
+    import torch
+
+    times = []
+    for _ in range(n):
+        if flush is not None:
+            flush.zero_()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        fn()
+        e.record()
+        e.synchronize()
+        times.append(s.elapsed_time(e))
+    return times
+
+
+def config1_inputs():
+    import torch
+
+    gen = torch.Generator().manual_seed(0)
+    shape = (32, 12, 512, 64)
+    q, k, v = (torch.randn(shape, generator=gen).half() for _ in range(3))
+    lengths = torch.randint(256, 513, (32,), generator=gen)
+    mask = torch.zeros((32, 1, 1, 512), dtype=torch.float32)
+    for b in range(32):
+        mask[b, :, :, lengths[b]:] = float("-inf")
+    return q, k, v, mask, lengths
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--skip-e2e", action="store_true", help="skip the BERT-base forward latency")
+    ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline timings")
+    ap.add_argument("--skip-extra", action="store_true", help="only the headline attention numbers")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build targets one GPU per process and ships no multi-GPU path; run with --gpus 1")
+
+    import torch
+
+    from kernl_amd import _lib
+    from kernl_amd.implementations.attention import attention_forward
+    from kernl_amd.implementations.layer_norm import layer_norm
+    from kernl_amd.implementations.linear_layer import linear_layer
+
+    _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ------------------------------------------------------------------ headline: fused attention, config 1
+    q, k, v, mask, lengths = config1_inputs()
+    B, H, S, D = q.shape
+    dense_flop = 4.0 * B * H * S * S * D
+    # key tiles of 128 that are entirely padding are skipped by the kernel: flops actually executed
+    executed_flop = sum(4.0 * H * S * D * (128 * ((int(n) + 127) // 128)) for n in lengths)
+    qd, kd, vd, md = q.to(dev), k.to(dev), v.to(dev), mask.to(dev)
+    out = torch.empty_like(qd)
+
+    def step():
+        attention_forward(qd, kd, vd, out, 0.125, False, md)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    for i in range(args.steps):
+        starts[i].record()
+        step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    launch_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    avg_launch_ms = sum(launch_ms) / len(launch_ms)
+    value = dense_flop / (ms_per_step * 1e-3) / 1e12
+    achieved = dense_flop / (avg_launch_ms * 1e-3) / 1e12
+    attn_bytes = 4 * B * H * S * D * 2 + mask.numel() * 4
+
+    result = {
+        "metric": "fused-attn TFLOP/s + BERT-base b32 s512 fp16 fwd latency (ms), 1 MI355X",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: fused attention forward, q/k/v fp16 [32,12,512,64] N(0,1), scale 1/8, non-causal, "
+            "additive padding mask [32,1,1,512] fp32 (0 / -inf, lengths U[256,512]), seed 0",
+            "flop_count": "dense 4*B*H*M*N*D = 25.77 GFLOP per step (padded keys counted)",
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(achieved, 2),
+            "peak": PEAK_MFMA_F16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_MFMA_F16_TFLOPS, 4),
+            "traffic": None,
+        },
+    }
+    extra = {
+        "attention_avg_launch_us": round(avg_launch_ms * 1e3, 2),
+        "attention_min_launch_us": round(min(launch_ms) * 1e3, 2),
+        "attention_executed_tflops": round(executed_flop / (avg_launch_ms * 1e-3) / 1e12, 2),
+        "attention_executed_fraction_of_dense": round(executed_flop / dense_flop, 4),
+        "attention_algorithmic_gbps": round(attn_bytes / (avg_launch_ms * 1e-3) / 1e9, 1),
+        "attention_hbm_frac": round(attn_bytes / (avg_launch_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+    }
+
+    # ------------------------------------------------------------------ CPU baseline on a bounded sample
+    if not args.skip_cpu:
+        from oracle import attention_oracle
+
+        torch.set_num_threads(os.cpu_count() or 1)
+        nb = 4  # batches 0..3 of the 32: 1/8 of the workload
+        qs, ks, vs, ms = q[:nb], k[:nb], v[:nb], mask[:nb]
+        attention_oracle(qs, ks, vs, 0.125, False, ms)
+        times = []
+        t_begin = time.perf_counter()
+        while len(times) < 5 or (time.perf_counter() - t_begin < 10.0 and len(times) < 50):
+            t = time.perf_counter()
+            attention_oracle(qs, ks, vs, 0.125, False, ms)
+            times.append(time.perf_counter() - t)
+        med = statistics.median(times)
+        result["cpu_baseline"] = {
+            "value": round(dense_flop * nb / B / med / 1e12, 4),
+            "unit": "TFLOP/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"oracle.attention_oracle (fp32 eager PyTorch on the host) on batches 0..{nb - 1} of 32 of the same "
+            f"inputs, median of {len(times)} runs, {med * 1e3:.1f} ms each; dense flop count",
+        }
+    else:
+        result["cpu_baseline"] = None
+
+    # ------------------------------------------------------------------ the other kernels of the metric (config 2)
+    if not args.skip_extra:
+        flush = torch.empty(256 * 1024 * 1024, dtype=torch.int8, device=dev)
+        gen = torch.Generator().manual_seed(0)
+        M, Kd, N = 16384, 768, 3072
+        x_up = torch.randn((M, Kd), generator=gen).half().to(dev)
+        w_up = (torch.randn((N, Kd), generator=gen) * 0.02).half().to(dev)
+        b_up = (torch.randn((N,), generator=gen) * 0.02).half().to(dev)
+        x_dn = torch.randn((M, N), generator=gen).half().to(dev)
+        w_dn = (torch.randn((Kd, N), generator=gen) * 0.02).half().to(dev)
+        b_dn = (torch.randn((Kd,), generator=gen) * 0.02).half().to(dev)
+        x_ln = torch.randn((M, Kd), generator=gen).half().to(dev)
+        g_ln = (1 + 0.1 * torch.randn((Kd,), generator=gen)).half().to(dev)
+        be_ln = (0.1 * torch.randn((Kd,), generator=gen)).half().to(dev)
+        lin_flop = 2.0 * M * N * Kd
+        ln_bytes = 2 * (2 * M * Kd + 2 * Kd)
+
+        def measure(fn, label, work, unit_scale, peak):
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
+            warm = statistics.median(_event_times(fn, 30))
+            cold = statistics.median(_event_times(fn, 30, flush))
+            extra[f"{label}_us_warm"] = round(warm * 1e3, 2)
+            extra[f"{label}_us_cold"] = round(cold * 1e3, 2)
+            rate = work / (warm * 1e-3) / unit_scale
+            extra[f"{label}_rate_warm"] = round(rate, 1)
+            extra[f"{label}_rate_cold"] = round(work / (cold * 1e-3) / unit_scale, 1)
+            extra[f"{label}_frac_of_peak_warm"] = round(rate / peak, 4)
+
+        measure(lambda: linear_layer(x_up, w_up, b_up, "fast_gelu"), "linear_up_tanh_gelu_tflops", lin_flop, 1e12,
+                PEAK_MFMA_F16_TFLOPS)
+        measure(lambda: linear_layer(x_dn, w_dn, b_dn, ""), "linear_down_tflops", lin_flop, 1e12, PEAK_MFMA_F16_TFLOPS)
+
+        # LayerNorm is ~10 us of GPU time: replay a hipGraph of 20 launches so that launch gaps do not count
+        ln_out = [None]
+
+        def ln_once():
+            ln_out[0] = layer_norm(x_ln, g_ln, be_ln, 1e-12)
+
+        ln_once()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        reps = 20
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(reps):
+                ln_once()
+        torch.cuda.synchronize()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t = statistics.median(_event_times(graph.replay, 20)) / reps
+        extra["layernorm_us_graph_replay"] = round(t * 1e3, 2)
+        extra["layernorm_gbps_graph_replay"] = round(ln_bytes / (t * 1e-3) / 1e9, 1)
+        extra["layernorm_frac_of_hbm_peak"] = round(ln_bytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
+        cold = statistics.median(_event_times(ln_once, 30, flush))
+        extra["layernorm_us_cold_single_launch"] = round(cold * 1e3, 2)
+        del flush
+
+    # ------------------------------------------------------------------ BERT-base b32 s512 through optimize_model
+    if not args.skip_e2e and not args.skip_extra:
+        try:
+            from transformers import BertConfig, BertModel
+
+            from kernl_amd.model_optimization import optimize_model
+
+            torch.manual_seed(0)
+            cfg = BertConfig()
+            cfg._attn_implementation = "eager"
+            model = BertModel(cfg).eval().half().to(dev)
+            gen = torch.Generator().manual_seed(0)
+            ids = torch.randint(0, 30522, (32, 512), generator=gen)
+            lens = torch.randint(256, 513, (32,), generator=gen)
+            amask = (torch.arange(512)[None, :] < lens[:, None]).long()
+            ids_d, amask_d = ids.to(dev), amask.to(dev)
+            optimize_model(model)
+            with torch.inference_mode():
+                for _ in range(10):
+                    model(input_ids=ids_d, attention_mask=amask_d)
+                torch.cuda.synchronize()
+                times = []
+                for _ in range(10):
+                    t = time.perf_counter()
+                    model(input_ids=ids_d, attention_mask=amask_d)
+                    torch.cuda.synchronize()
+                    times.append((time.perf_counter() - t) * 1e3)
+            ms = statistics.median(times)
+            extra["bert_base_b32_s512_fp16_fwd_ms"] = round(ms, 3)
+            extra["bert_base_b32_s512_tflops"] = round(3.092e12 / (ms * 1e-3) / 1e12, 1)
+            if not args.skip_cpu:
+                # CPU eager fp32 on 2 of the 32 sequences, scaled by 16 (the model is batch-parallel)
+                torch.manual_seed(0)
+                cpu_model = BertModel(cfg).eval()
+                with torch.inference_mode():
+                    cpu_model(input_ids=ids[:2], attention_mask=amask[:2])
+                    t = time.perf_counter()
+                    cpu_model(input_ids=ids[:2], attention_mask=amask[:2])
+                    dt = time.perf_counter() - t
+                extra["bert_base_b32_s512_cpu_fp32_ms_scaled_from_2_of_32"] = round(dt * 1e3 * 16, 1)
+        except Exception as exc:  # the headline number must still be reported
+            extra["bert_base_b32_s512_error"] = f"{type(exc).__name__}: {exc}"[:300]
+
+    result["extra"] = extra
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -12,7 +12,12 @@ from kernl_amd.optimizer.attention import (
 from kernl_amd.optimizer.dropout import remove_dropout
 from kernl_amd.optimizer.layer_norm import replace_layer_norm, replace_layer_norm_fn, replace_layer_norm_rms
 from kernl_amd.optimizer.linear import replace_all_linear
-from kernl_amd.optimizer.mask import scalar_tensors_to_full, sink_expand_below_where
+from kernl_amd.optimizer.mask import (
+    drop_all_true_conjuncts,
+    merge_nested_expands,
+    scalar_tensors_to_full,
+    sink_expand_below_where,
+)
 from kernl_amd.optimizer.normalizer import normalize_operators
 
 
@@ -20,7 +25,10 @@ def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
     normalize_operators(gm)
     remove_dropout(gm)
     scalar_tensors_to_full(gm)
+    drop_all_true_conjuncts(gm)
+    merge_nested_expands(gm)
     sink_expand_below_where(gm)
+    merge_nested_expands(gm)
     fuse_attention_pattern_1(gm, assume_causal)
     fuse_attention_pattern_2(gm, assume_causal)
     fuse_attention_pattern_3(gm, assume_causal)

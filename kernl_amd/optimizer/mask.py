@@ -7,6 +7,8 @@ although every query row is identical (33 MB at batch 32, sequence 512, re-read 
 `where`; the mask the attention kernel then receives is a stride-0 view of a [B,1,1,S] tensor and is consumed as one
 value per key.  No counterpart in the reference, whose BERT graphs carried a [B,1,1,S] mask already.
 """
+import operator
+
 import torch
 from torch.fx import Node
 
@@ -42,6 +44,108 @@ def scalar_tensors_to_full(gm: torch.fx.GraphModule):
         gm.graph.erase_node(node)
         changed = True
     if changed:
+        gm.graph.lint()
+        gm.recompile()
+
+
+# Pure, shape-static ops that may be evaluated while compiling when every tensor operand is itself a constant.
+_FOLDABLE_FUNCTIONS = {
+    torch.arange, torch.ones, torch.zeros, torch.full, torch.tril, torch.triu,
+    operator.add, operator.sub, operator.mul, operator.and_, operator.or_, operator.getitem,
+    operator.ge, operator.gt, operator.le, operator.lt, operator.eq, operator.ne,
+    torch.add, torch.sub, torch.mul, torch.bitwise_and, torch.bitwise_or,
+}
+_FOLDABLE_METHODS = {"new_ones", "new_zeros", "to", "expand", "view", "reshape", "unsqueeze", "squeeze", "bool", "long", "int"}
+_FOLD_LIMIT = 1 << 22  # elements
+
+
+def _fold_constants(gm: torch.fx.GraphModule):
+    """node -> tensor value, for nodes computable from literals alone (index grids and the like)."""
+    values = {}
+
+    def materialize(arg):
+        return torch.fx.node.map_arg(arg, lambda n: values[n])
+
+    for node in gm.graph.nodes:
+        if node.op == "call_function" and node.target in _FOLDABLE_FUNCTIONS:
+            pass
+        elif node.op == "call_method" and node.target in _FOLDABLE_METHODS:
+            pass
+        else:
+            continue
+        if not all(n in values for n in node.all_input_nodes):
+            continue
+        if node.op == "call_method" and not node.all_input_nodes:
+            continue
+        try:
+            args, kwargs = materialize(node.args), materialize(node.kwargs)
+            out = node.target(*args, **kwargs) if node.op == "call_function" else getattr(args[0], node.target)(*args[1:], **kwargs)
+        except Exception:
+            continue
+        if isinstance(out, torch.Tensor) and out.numel() <= _FOLD_LIMIT:
+            values[node] = out
+    return values
+
+
+def drop_all_true_conjuncts(gm: torch.fx.GraphModule):
+    """`c & x` where `c` folds to an all-True constant is `x` broadcast to the result shape.
+
+    transformers builds attention masks as `mask_function(q_idx, kv_idx) & padding[b, kv_idx]`; for an encoder the
+    first conjunct is the constant grid `q_idx >= 0`, whose only effect is to blow the per-key padding mask up to a
+    [B,1,S,S] matrix.  Removing it leaves an `expand` of the [B,1,1,S] padding mask."""
+    values = _fold_constants(gm)
+    changed = False
+    for node in list(gm.graph.nodes):
+        if node.op != "call_function" or node.target not in (operator.and_, torch.bitwise_and) or len(node.args) != 2:
+            continue
+        a, b = node.args
+        for const, other in ((a, b), (b, a)):
+            if not (isinstance(const, Node) and const in values and isinstance(other, Node) and other not in values):
+                continue
+            cval = values[const]
+            if cval.dtype != torch.bool or not bool(cval.all()):
+                continue
+            other_val = other.meta.get("example_value")
+            if other_val is None or other_val.dtype != torch.bool:
+                continue
+            out_shape = tuple(torch.broadcast_shapes(tuple(cval.shape), tuple(other_val.shape)))
+            if not all(isinstance(d, int) for d in out_shape):
+                continue
+            with gm.graph.inserting_before(node):
+                if len(out_shape) == other_val.dim():
+                    new = gm.graph.call_method("expand", (other,) + out_shape)
+                else:
+                    continue
+            new.meta["example_value"] = other_val.expand(out_shape)
+            node.replace_all_uses_with(new)
+            gm.graph.erase_node(node)
+            changed = True
+            break
+    if changed:
+        gm.graph.eliminate_dead_code()
+        gm.graph.lint()
+        gm.recompile()
+
+
+def merge_nested_expands(gm: torch.fx.GraphModule):
+    """x.expand(s1).expand(s2) -> x.expand(s2) when the ranks agree (keeps stride-0 dims visible to later passes)."""
+    changed = False
+    for node in list(gm.graph.nodes):
+        if not (node.op == "call_method" and node.target == "expand" and not node.kwargs):
+            continue
+        inner = node.args[0]
+        if not (isinstance(inner, Node) and inner.op == "call_method" and inner.target == "expand" and not inner.kwargs):
+            continue
+        if len(inner.args) != len(node.args) or len(inner.users) != 1:
+            continue
+        inner_shape, outer_shape = inner.args[1:], node.args[1:]
+        if not all(isinstance(d, int) for d in inner_shape + outer_shape):
+            continue
+        merged = tuple(i if o == -1 else o for i, o in zip(inner_shape, outer_shape))
+        node.args = (inner.args[0],) + merged
+        changed = True
+    if changed:
+        gm.graph.eliminate_dead_code()
         gm.graph.lint()
         gm.recompile()
 
