@@ -1,0 +1,193 @@
+"""Pins the CPU oracle (no GPU): closed forms against torch library routines, algorithm restatements against the
+closed forms, and the invariants / known answers that a dropped term, wrong sign or transposed operand would break.
+The reference holds no stored numeric vectors for this path (its tests recompute expectations with torch at run
+time); its known-answer material is `closest_power_of_2` (test/test_attention.py:148-157) and the graph-pool answers
+(test/test_cuda_graph.py), covered in test_host_logic.py."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import (
+    activation_oracle,
+    attention_oracle,
+    attention_tiled_oracle,
+    effective_eps,
+    layer_norm_oracle,
+    layer_norm_welford_oracle,
+    linear_oracle,
+    rms_norm_oracle,
+)
+
+
+def _qkv(shape, seed=0, n=None):
+    gen = torch.Generator().manual_seed(seed)
+    q = torch.randn(shape, generator=gen)
+    kshape = shape if n is None else (shape[0], shape[1], n, shape[3])
+    return q, torch.randn(kshape, generator=gen), torch.randn(kshape, generator=gen)
+
+
+def _brute_force_attention(q, k, v, scale, causal, mask):
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    out = torch.zeros((B, H, M, D), dtype=torch.float64)
+    for b in range(B):
+        for h in range(H):
+            for m in range(M):
+                logits = []
+                for n in range(N):
+                    s = sum(float(q[b, h, m, d]) * float(k[b, h, n, d]) for d in range(D)) * scale
+                    if mask is not None:
+                        s += float(mask[b if mask.shape[0] > 1 else 0, h if mask.shape[1] > 1 else 0,
+                                        m if mask.shape[2] > 1 else 0, n])
+                    if causal and n > m:
+                        s = -math.inf
+                    logits.append(s)
+                mx = max(logits)
+                w = [math.exp(x - mx) for x in logits]
+                z = sum(w)
+                for d in range(D):
+                    out[b, h, m, d] = sum(w[n] * float(v[b, h, n, d]) for n in range(N)) / z
+    return out
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("masked", [False, True])
+def test_attention_closed_form_vs_brute_force(causal, masked):
+    q, k, v = _qkv((2, 2, 5, 4), seed=1, n=7 if not causal else 5)
+    mask = torch.randn((2, 1, 5, k.shape[2]), generator=torch.Generator().manual_seed(2)) if masked else None
+    got = attention_oracle(q, k, v, 0.7, causal, mask)
+    want = _brute_force_attention(q, k, v, 0.7, causal, mask)
+    assert torch.allclose(got.double(), want, atol=1e-5)
+
+
+def test_attention_matches_torch_sdpa():
+    q, k, v = _qkv((2, 3, 33, 16), seed=3)
+    got = attention_oracle(q, k, v, 0.25, False, None)
+    want = torch.nn.functional.scaled_dot_product_attention(q, k, v, scale=0.25)
+    assert torch.allclose(got, want, atol=1e-5)
+    got_c = attention_oracle(q, k, v, 0.25, True, None)
+    want_c = torch.nn.functional.scaled_dot_product_attention(q, k, v, scale=0.25, is_causal=True)
+    assert torch.allclose(got_c, want_c, atol=1e-5)
+
+
+def test_attention_invariants():
+    q, k, v = _qkv((1, 2, 40, 8), seed=4)
+    # V = 1 => O = 1
+    assert torch.allclose(attention_oracle(q, k, torch.ones_like(v), 0.3), torch.ones_like(q), atol=1e-6)
+    # causal row 0 attends key 0 only
+    assert torch.allclose(attention_oracle(q, k, v, 0.3, True)[:, :, 0], v[:, :, 0], atol=1e-6)
+    # permuting the keys (and values with them) changes nothing without a causal mask
+    perm = torch.randperm(40, generator=torch.Generator().manual_seed(5))
+    assert torch.allclose(attention_oracle(q, k[:, :, perm], v[:, :, perm], 0.3), attention_oracle(q, k, v, 0.3), atol=1e-5)
+    # keys behind a -inf padding mask are as good as absent
+    mask = torch.zeros((1, 1, 1, 40))
+    mask[..., 25:] = float("-inf")
+    assert torch.allclose(attention_oracle(q, k, v, 0.3, False, mask), attention_oracle(q, k[:, :, :25], v[:, :, :25], 0.3), atol=1e-5)
+    # the mask is ADDED (sign check): a large positive bias on one key makes the output that key's value
+    bias = torch.zeros((1, 1, 1, 40))
+    bias[..., 7] = 200.0
+    assert torch.allclose(attention_oracle(q, k, v, 0.3, False, bias), v[:, :, 7:8].expand_as(q), atol=1e-4)
+
+
+@pytest.mark.parametrize("seq", [8, 16, 33, 128, 257])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("mask_kind", ["none", "vector", "matrix"])
+def test_tiled_restatement_equals_closed_form(seq, causal, mask_kind):
+    q, k, v = _qkv((2, 2, seq, 8), seed=seq)
+    gen = torch.Generator().manual_seed(seq + 1)
+    mask = None
+    if mask_kind == "vector":
+        mask = torch.zeros((2, 1, 1, seq))
+        mask[1, ..., seq // 2 + 1:] = float("-inf")
+    elif mask_kind == "matrix":
+        mask = torch.rand((1, 2, seq, seq), generator=gen)
+    got = attention_tiled_oracle(q.numpy(), k.numpy(), v.numpy(), 0.3, causal, None if mask is None else mask.numpy())
+    want = attention_oracle(q, k, v, 0.3, causal, mask)
+    assert np.allclose(got, want.double().numpy(), atol=1e-5)
+
+
+def test_tiled_restatement_fully_masked_row_is_uniform_average():
+    q, k, v = _qkv((1, 1, 4, 8), seed=9, n=20)
+    mask = np.full((1, 1, 1, 20), -np.inf, dtype=np.float32)
+    got = attention_tiled_oracle(q.numpy(), k.numpy(), v.numpy(), 0.5, False, mask)
+    assert np.isfinite(got).all()
+    assert np.allclose(got, v.double().mean(dim=2, keepdim=True).expand(-1, -1, 4, -1).numpy(), atol=1e-6)
+    # fp16 clamp value: the add does not absorb q·kᵀ, so the result is the ordinary softmax over all keys
+    got16 = attention_tiled_oracle(q.numpy(), k.numpy(), v.numpy(), 0.5, False, mask.astype(np.float16))
+    assert np.allclose(got16, attention_oracle(q, k, v, 0.5).double().numpy(), atol=1e-6)
+
+
+def test_activation_known_points():
+    x = torch.tensor([0.0, -1.0, 1.0, 3.0, -3.0])
+    assert torch.equal(activation_oracle(x, "relu"), torch.tensor([0.0, 0.0, 1.0, 3.0, 0.0]))
+    gelu = activation_oracle(x, "gelu")
+    assert gelu[0] == 0 and abs(gelu[2].item() - 0.8413447) < 1e-6 and abs(gelu[1].item() + 0.1586553) < 1e-6
+    fast = activation_oracle(x, "fast_gelu")
+    assert fast[0] == 0 and abs(fast[2].item() - 0.8411920) < 1e-6
+    assert torch.allclose(activation_oracle(x, "tanh"), torch.tanh(x))
+    assert torch.allclose(activation_oracle(x, "gelu"), torch.nn.functional.gelu(x), atol=1e-6)
+    assert torch.allclose(activation_oracle(x, "fast_gelu"), torch.nn.functional.gelu(x, approximate="tanh"), atol=1e-6)
+    assert torch.allclose(activation_oracle(x, "silu"), torch.nn.functional.silu(x), atol=1e-6)
+    assert torch.equal(activation_oracle(x, "no-such-activation"), x)
+
+
+def test_linear_closed_form():
+    gen = torch.Generator().manual_seed(0)
+    x, w, b = torch.randn((3, 7, 16), generator=gen), torch.randn((5, 16), generator=gen), torch.randn((5,), generator=gen)
+    assert torch.allclose(linear_oracle(x, w, b), torch.nn.functional.linear(x, w, b), atol=1e-5)
+    assert torch.allclose(linear_oracle(x, w, None, "relu"), torch.relu(torch.nn.functional.linear(x, w)), atol=1e-5)
+    # weight is [N, K] (a transposed operand would not even have the right shape here) and strided x works
+    xt = torch.randn((16, 7), generator=gen)
+    assert torch.allclose(linear_oracle(xt.mT, w, b), torch.nn.functional.linear(xt.t(), w, b), atol=1e-5)
+    out, pre = linear_oracle(x, w, b, "gelu", return_act_inputs=True)
+    assert torch.allclose(pre, torch.nn.functional.linear(x, w, b), atol=1e-5)
+    assert torch.allclose(out, torch.nn.functional.gelu(pre), atol=1e-6)
+    # hand-computed 2x2 case: x = [[1, 2]], w = [[3, 4], [5, 6]], b = [1, -1] -> [[12, 16]]
+    assert torch.equal(linear_oracle(torch.tensor([[1.0, 2.0]]), torch.tensor([[3.0, 4.0], [5.0, 6.0]]), torch.tensor([1.0, -1.0])),
+                       torch.tensor([[12.0, 16.0]]))
+
+
+def test_layer_norm_closed_form_and_large_mean():
+    gen = torch.Generator().manual_seed(0)
+    x = -20 + 0.5 * torch.randn((64, 1024), generator=gen)  # reference test/test_layer_norm.py:58
+    w, b = torch.rand((1024,), generator=gen), torch.randn((1024,), generator=gen)
+    assert torch.allclose(layer_norm_oracle(x, w, b, 1e-5), torch.nn.functional.layer_norm(x, (1024,), w, b, 1e-5), atol=2e-5)
+    # known answer: row [1, 2, 3, 4], unit weight, eps 0 -> (x - 2.5) / sqrt(1.25)
+    row = torch.tensor([[1.0, 2.0, 3.0, 4.0]])
+    want = (row - 2.5) / math.sqrt(1.25)
+    assert torch.allclose(layer_norm_oracle(row, torch.ones(4), None, 0.0), want, atol=1e-6)
+
+
+def test_rms_norm_closed_form():
+    gen = torch.Generator().manual_seed(1)
+    x, w = torch.randn((8, 300), generator=gen), torch.rand((300,), generator=gen)
+    want = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+    assert torch.allclose(rms_norm_oracle(x, w, 1e-6), want, atol=1e-6)
+    # constant row c: x / |c| (eps 0)
+    assert torch.allclose(rms_norm_oracle(torch.full((1, 16), -3.0), torch.ones(16), 0.0), torch.full((1, 16), -1.0), atol=1e-6)
+    assert torch.allclose(rms_norm_oracle(x, w, 1e-6), torch.nn.functional.rms_norm(x, (300,), w, 1e-6), atol=1e-5)
+
+
+@pytest.mark.parametrize("n", [128, 512, 1024, 4096, 5000, 9000])
+@pytest.mark.parametrize("rms", [False, True])
+def test_welford_restatement_equals_closed_form(n, rms):
+    gen = torch.Generator().manual_seed(n)
+    x = -20 + 0.5 * torch.randn((6, n), generator=gen)
+    w, b = torch.rand((n,), generator=gen), torch.randn((n,), generator=gen)
+    out, mean, rstd = layer_norm_welford_oracle(x.numpy(), w.numpy(), None if rms else b.numpy(), 1e-5, rms)
+    want = rms_norm_oracle(x, w, 1e-5) if rms else layer_norm_oracle(x, w, b, 1e-5)
+    assert np.allclose(out, want.numpy(), atol=2e-3, rtol=1e-4)
+    if rms:
+        assert np.all(mean == 0)
+    else:
+        assert np.allclose(mean, x.mean(-1).numpy(), atol=1e-4)
+        assert np.allclose(rstd, (1 / torch.sqrt(x.var(-1, unbiased=False) + 1e-5)).numpy(), rtol=2e-3)
+
+
+def test_effective_eps():
+    assert effective_eps(1e-12, torch.float16) == 1.6e-5
+    assert effective_eps(1e-3, torch.float16) == 1e-3
+    assert effective_eps(1e-12, torch.bfloat16) == 1e-12
+    assert effective_eps(1e-12, torch.float32) == 1e-12
