@@ -27,6 +27,7 @@ EXPORTED_SYMBOLS = (
     "kernl_add_layernorm_fwd",
     "kernl_linear_force_tile",
     "kernl_attention_force_scalar",
+    "kernl_attention_set_variant",
 )
 
 _i64 = ctypes.c_int64
@@ -70,6 +71,8 @@ def load() -> ctypes.CDLL:
     lib.kernl_linear_force_tile.argtypes = [ctypes.c_int]
     lib.kernl_attention_force_scalar.restype = None
     lib.kernl_attention_force_scalar.argtypes = [ctypes.c_int]
+    lib.kernl_attention_set_variant.restype = None
+    lib.kernl_attention_set_variant.argtypes = [ctypes.c_int]
     _lib = lib
     return lib
 

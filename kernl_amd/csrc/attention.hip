@@ -55,8 +55,8 @@ __device__ __forceinline__ float scale_mask(float mv, float clamp) {
     return fmaxf(mv * kLog2eA, kClampFloor);
 }
 
-template <typename T, int D, int BN, int SUB, int MASK_MODE, bool CAUSAL>
-__global__ void __launch_bounds__(256, 2) attention_mfma_kernel(const AttnParams p) {
+template <typename T, int D, int BN, int SUB, int WPE, int MASK_MODE, bool CAUSAL>
+__global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnParams p) {
     typedef typename Vec8<T>::type vec8;
     constexpr int BM = 128;
     constexpr int KROW = D * 2, VROW = BN * 2;           // LDS row bytes of the K and Vᵀ tiles
@@ -65,7 +65,9 @@ __global__ void __launch_bounds__(256, 2) attention_mfma_kernel(const AttnParams
     constexpr int NBS = SUB / 32, DB = D / 32, KS = D / 16;
     constexpr int DC = D / 8;                            // 16-byte chunks per K/V row
     constexpr int KI = BN * DC / 256;                    // K chunks per thread per tile
-    static_assert(BN * D == 8192, "each thread transposes exactly one 4x8 block of V per tile");
+    constexpr int VBLK = (BN / 4) * DC;                  // 4-key x 8-feature blocks of V per tile
+    static_assert(VBLK == 256 || VBLK == 128, "a thread transposes at most one 4x8 block of V per tile");
+    static_assert(BN * DC % 256 == 0, "K chunks must split evenly over the threads");
 
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
     __shared__ int tile_list[kMaxTiles];
@@ -142,26 +144,29 @@ __global__ void __launch_bounds__(256, 2) attention_mfma_kernel(const AttnParams
     const int v_dc = tid % DC, v_ng = tid / DC;  // this thread's 4-key x 8-feature block of V
     vec8 kst[KI], vst[4];
     float bias_st = 0.0f;
+    int staged_n0 = 0;  // first key of the tile held in the staging registers
     auto gload = [&](int tile) {
         const int n0 = tile * BN;
+        staged_n0 = n0;
+        // rows past the last key are read from the last key's row (always mapped) and zeroed in lstore
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
             const int qd = tid + 256 * i;
             const int row = qd / DC, c = qd % DC;
-            vec8 z = {};
-            kst[i] = (n0 + row < N) ? *reinterpret_cast<const vec8 *>(kp + (int64_t)(n0 + row) * p.ks[2] + c * 8) : z;
+            kst[i] = *reinterpret_cast<const vec8 *>(kp + (int64_t)min(n0 + row, N - 1) * p.ks[2] + c * 8);
         }
+        if (VBLK == 256 || tid < VBLK) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int n = n0 + v_ng * 4 + r;
-            vec8 z = {};
-            vst[r] = (n < N) ? *reinterpret_cast<const vec8 *>(vp + (int64_t)n * p.vs[2] + v_dc * 8) : z;
+            for (int r = 0; r < 4; ++r) {
+                const int n = min(n0 + v_ng * 4 + r, N - 1);
+                vst[r] = *reinterpret_cast<const vec8 *>(vp + (int64_t)n * p.vs[2] + v_dc * 8);
+            }
         }
         if (tid < BN) {
             const int n = n0 + tid;
             float bv = 0.0f;
-            if (MASK_MODE == MASK_VECTOR && n < N)
-                bv = scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_base + n * p.ms[3]), p.clamp);
+            if (MASK_MODE == MASK_VECTOR)
+                bv = scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_base + min(n, N - 1) * p.ms[3]), p.clamp);
             if (n >= N) bv = -INFINITY;
             bias_st = bv;
         }
@@ -169,6 +174,15 @@ __global__ void __launch_bounds__(256, 2) attention_mfma_kernel(const AttnParams
     auto lstore = [&](int stage) {
         unsigned char *kb = smem + stage * STAGE;
         unsigned char *vb = kb + K_BYTES;
+        if (staged_n0 + BN > N) {  // tail tile (uniform): keys past the end contribute exact zeros
+            const vec8 z = {};
+#pragma unroll
+            for (int i = 0; i < KI; ++i)
+                if (staged_n0 + (tid + 256 * i) / DC >= N) kst[i] = z;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (staged_n0 + v_ng * 4 + r >= N) vst[r] = z;
+        }
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
             const int qd = tid + 256 * i;
@@ -180,14 +194,16 @@ __global__ void __launch_bounds__(256, 2) attention_mfma_kernel(const AttnParams
         const int nloc = v_ng * 4;
         const int pos = (nloc & ~12) | ((nloc & 4) << 1) | ((nloc & 8) >> 1);
         const int chunk = pos >> 3, half = (pos >> 2) & 1;
+        if (VBLK == 256 || tid < VBLK) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int d = v_dc * 8 + e;
-            const int x = d & 31;
-            const int row = (d & ~31) + 8 * ((x >> 2) & 3) + 4 * (x >> 4) + (x & 3);
-            T quad[4] = {vst[0][e], vst[1][e], vst[2][e], vst[3][e]};
-            *reinterpret_cast<uint64_t *>(vb + swz_offset<VROW>(row, chunk) + half * 8) =
-                *reinterpret_cast<const uint64_t *>(quad);
+            for (int e = 0; e < 8; ++e) {
+                const int d = v_dc * 8 + e;
+                const int x = d & 31;
+                const int row = (d & ~31) + 8 * ((x >> 2) & 3) + 4 * (x >> 4) + (x & 3);
+                T quad[4] = {vst[0][e], vst[1][e], vst[2][e], vst[3][e]};
+                *reinterpret_cast<uint64_t *>(vb + swz_offset<VROW>(row, chunk) + half * 8) =
+                    *reinterpret_cast<const uint64_t *>(quad);
+            }
         }
         if (tid < BN) *reinterpret_cast<float *>(kb + K_BYTES + V_BYTES + tid * 4) = bias_st;
     };
@@ -216,6 +232,10 @@ __global__ void __launch_bounds__(256, 2) attention_mfma_kernel(const AttnParams
         gload(use_list ? tile_list[0] : 0);
         lstore(0);
     }
+    // Every load issued so far (Q fragments included) has to have landed before the loop: otherwise the
+    // compiler must assume they may still be in flight at the first MFMA of each iteration and waits there for
+    // the vector-memory counter to drain, which also drains the prefetch of the next tile issued just before.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
 
     for (int it = 0; it < nt; ++it) {
@@ -284,7 +304,7 @@ __global__ void __launch_bounds__(256, 2) attention_mfma_kernel(const AttnParams
                     for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[nb][v]);
                 mx *= c;  // c > 0 on this path (checked by the host)
             }
-            mx = fmaxf(mx, swap32(mx));
+            mx = halves32_max(mx);  // the other 16-key half of every 32-key block lives in lane ^ 32
             const float m_new = fmaxf(m_i, mx);
             const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
             const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
@@ -337,7 +357,7 @@ __global__ void __launch_bounds__(256, 2) attention_mfma_kernel(const AttnParams
     }
 
     // ---- normalise and store: lane holds features 32 d + 16 lh + (0..15) of row my_m
-    const float l_tot = l_i + swap32(l_i);
+    const float l_tot = halves32_sum(l_i);
     const float inv_l = 1.0f / l_tot;
     if (my_m < M) {
         T *orow = op + (int64_t)my_m * p.os[2] + lh * 16;
@@ -422,11 +442,11 @@ __global__ void __launch_bounds__(64) attention_scalar_kernel(const AttnParams p
 // ----------------------------------------------------------------------------------------------------
 // host dispatch
 // ----------------------------------------------------------------------------------------------------
-template <typename T, int D, int BN, int SUB>
+template <typename T, int D, int BN, int SUB, int WPE>
 static void launch_mfma(const AttnParams &p, int mask_mode, bool causal, hipStream_t st) {
     const int bh_padded = ((p.B * p.H + 7) / 8) * 8;
     dim3 grid((unsigned)(bh_padded * p.nq_tiles)), block(256);
-#define KERNL_ATTN_LAUNCH(MM, C) hipLaunchKernelGGL((attention_mfma_kernel<T, D, BN, SUB, MM, C>), grid, block, 0, st, p)
+#define KERNL_ATTN_LAUNCH(MM, C) hipLaunchKernelGGL((attention_mfma_kernel<T, D, BN, SUB, WPE, MM, C>), grid, block, 0, st, p)
     if (mask_mode == MASK_NONE) {
         if (causal) KERNL_ATTN_LAUNCH(MASK_NONE, true);
         else KERNL_ATTN_LAUNCH(MASK_NONE, false);
@@ -441,10 +461,12 @@ static void launch_mfma(const AttnParams &p, int mask_mode, bool causal, hipStre
 }
 
 int g_attention_force_scalar = 0;  // test hook: route everything through the scalar kernel
+int g_attention_variant = 0;       // tuning hook: tile shape of the head-size-64 MFMA kernel
 
 }  // namespace kernl
 
 extern "C" void kernl_attention_force_scalar(int on) { kernl::g_attention_force_scalar = on; }
+extern "C" void kernl_attention_set_variant(int which) { kernl::g_attention_variant = which; }
 
 extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
                                    int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
@@ -510,11 +532,15 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
                          rows_ok(out, o_strides) && (int64_t)((B * H + 7) / 8) * 8 * p.nq_tiles < (1ll << 31);
     if (mfma_ok) {
         if (dtype == KERNL_F16) {
-            if (D == 64) launch_mfma<f16, 64, 128, 64>(p, mask_mode, causal, st);
-            else launch_mfma<f16, 128, 64, 32>(p, mask_mode, causal, st);
+            if (D == 64) {
+                if (g_attention_variant == 1) launch_mfma<f16, 64, 128, 64, 2>(p, mask_mode, causal, st);
+                else if (g_attention_variant == 2) launch_mfma<f16, 64, 64, 64, 2>(p, mask_mode, causal, st);
+                else launch_mfma<f16, 64, 64, 64, 3>(p, mask_mode, causal, st);
+            }
+            else launch_mfma<f16, 128, 64, 32, 2>(p, mask_mode, causal, st);
         } else {
-            if (D == 64) launch_mfma<bf16, 64, 128, 64>(p, mask_mode, causal, st);
-            else launch_mfma<bf16, 128, 64, 32>(p, mask_mode, causal, st);
+            if (D == 64) launch_mfma<bf16, 64, 64, 64, 3>(p, mask_mode, causal, st);
+            else launch_mfma<bf16, 128, 64, 32, 2>(p, mask_mode, causal, st);
         }
         return check_launch("attention (mfma)");
     }

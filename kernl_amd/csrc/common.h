@@ -117,9 +117,25 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
-// Value held by the lane 32 positions away (lane l <-> lane l ^ 32).
-__device__ __forceinline__ float swap32(float v) {
-    return __shfl_xor(v, 32, 64);
+// Both 32-lane halves of the wave exchange a value: afterwards every lane has the value its counterpart in the
+// lower half held (`lo`) and the one its counterpart in the upper half held (`hi`).
+// v_permlane32_swap exchanges the upper 32 lanes of its first operand with the lower 32 lanes of its second; fed
+// the same value twice, the first result is the lower half replicated, the second the upper half replicated.
+__device__ __forceinline__ void halves32(float v, float &lo, float &hi) {
+    const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+    const auto r = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+    lo = __builtin_bit_cast(float, (uint32_t)r[0]);
+    hi = __builtin_bit_cast(float, (uint32_t)r[1]);
+}
+__device__ __forceinline__ float halves32_max(float v) {
+    float lo, hi;
+    halves32(v, lo, hi);
+    return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float halves32_sum(float v) {
+    float lo, hi;
+    halves32(v, lo, hi);
+    return lo + hi;
 }
 
 // ----------------------------------------------------------------------------------------------------

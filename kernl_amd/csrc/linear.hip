@@ -80,7 +80,7 @@ struct LinearTile {
     static constexpr int GROUP_M = 4;  // m-tiles walked together so one XCD's L2 sees a compact block
 };
 
-template <typename T, typename Cfg, int ACT>
+template <typename T, typename Cfg, int ACT, bool K_TAIL>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_BLOCKS)
 linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
                    T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx,
@@ -112,16 +112,19 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     const int wave_m = wave % Cfg::WAVES_M, wave_n = wave / Cfg::WAVES_M;
     const int lr = lane & 31, lh = lane >> 5;
 
-    // ---- global -> register staging: thread owns chunks q = tid + THREADS*i, row q / CPR, chunk q % CPR
-    const T *xg[Cfg::XI];
-    const T *wg[Cfg::WI];
-    int xl[Cfg::XI], wl[Cfg::WI];  // LDS byte offsets inside a stage
+    // ---- global -> register staging: thread owns chunks q = tid + THREADS*i, row q / CPR, chunk q % CPR.
+    // Addresses are a wave-uniform base (tile origin + k, advanced on the scalar unit) plus a per-thread 32-bit
+    // byte offset; rows past M or N are clamped to the last valid row (their results are never stored).
+    const unsigned char *xbase = reinterpret_cast<const unsigned char *>(X + (int64_t)m0 * ldx);
+    const unsigned char *wbase = reinterpret_cast<const unsigned char *>(W + (int64_t)n0 * K);
+    uint32_t xg[Cfg::XI], wg[Cfg::WI];  // byte offsets from xbase / wbase
+    int xl[Cfg::XI], wl[Cfg::WI];       // LDS byte offsets inside a stage
 #pragma unroll
     for (int i = 0; i < Cfg::XI; ++i) {
         const int q = tid + Cfg::THREADS * i;
         const int row = q / CPR, c = q % CPR;
-        const int gm = min(m0 + row, M - 1);
-        xg[i] = X + (int64_t)gm * ldx + c * 8;
+        const int gm = min(m0 + row, M - 1) - m0;
+        xg[i] = (uint32_t)(((int64_t)gm * ldx + c * 8) * 2);
         xl[i] = swz_offset<RB>(row, c);
     }
 #pragma unroll
@@ -129,32 +132,47 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         const int q = tid + Cfg::THREADS * i;
         const int row = q / CPR, c = q % CPR;
         // LDS row `row` feeds MFMA row (row % 32) of its 32-block and carries weight row rowperm16(row % 32).
-        const int gn = min(n0 + (row & ~31) + rowperm16(row & 31), N - 1);
-        wg[i] = W + (int64_t)gn * K + c * 8;
+        const int gn = min(n0 + (row & ~31) + rowperm16(row & 31), N - 1) - n0;
+        wg[i] = (uint32_t)(((int64_t)gn * K + c * 8) * 2);
         wl[i] = Cfg::X_BYTES + swz_offset<RB>(row, c);
     }
     const int kchunk = (tid % CPR) * 8;  // same for every i because THREADS % CPR == 0
 
+    // ---- software pipeline over k-tiles of BK:
+    //   registers hold tile kt+1 (fetched from HBM/L2 during iteration kt-1), LDS stage kt&1 holds tile kt.
+    //   Iteration kt, k-step s:  read the operand fragments of step s+1 from LDS, store a quarter of tile kt+1
+    //   from registers into the other LDS stage, run the MFMAs of step s, and re-issue the global loads of the
+    //   same quarter for tile kt+2.  Global latency gets a whole iteration to hide, LDS stores ride under the
+    //   MFMAs, and there is one barrier per k-tile.  The loop body is branch-free: past the last k-tile the
+    //   loads re-read the last tile and the stores fill a stage nobody reads, which keeps the number of loads in
+    //   flight known at compile time (the memory counters are waited on by count).
+    constexpr int KSTEPS = BK / 16;
     vec8 xs[Cfg::XI], ws[Cfg::WI];
-    auto gload = [&](int k0) {
-        const bool in = (k0 + kchunk) < K;  // K % 8 == 0: a chunk is entirely inside or outside
+    const int nk = (K + BK - 1) / BK;
+    const int k_last = (nk - 1) * BK;
+
+    auto gload_part = [&](int k0, int part) {  // chunks i with i % KSTEPS == part
+        int koff = min(k0, k_last);
+        // K_TAIL: a chunk beyond K re-reads the first chunk of its row (always mapped); it is zeroed in lstore_part
+        if (K_TAIL && koff + kchunk >= K) koff = -kchunk;
+        const unsigned char *xb = xbase + (int64_t)koff * 2, *wb = wbase + (int64_t)koff * 2;
 #pragma unroll
-        for (int i = 0; i < Cfg::XI; ++i) {
-            vec8 z = {};
-            xs[i] = in ? *reinterpret_cast<const vec8 *>(xg[i] + k0) : z;
-        }
+        for (int i = 0; i < Cfg::XI; ++i)
+            if (i % KSTEPS == part) xs[i] = *reinterpret_cast<const vec8 *>(xb + xg[i]);
 #pragma unroll
-        for (int i = 0; i < Cfg::WI; ++i) {
-            vec8 z = {};
-            ws[i] = in ? *reinterpret_cast<const vec8 *>(wg[i] + k0) : z;
-        }
+        for (int i = 0; i < Cfg::WI; ++i)
+            if (i % KSTEPS == part) ws[i] = *reinterpret_cast<const vec8 *>(wb + wg[i]);
     };
-    auto lstore = [&](int stage) {
+    auto lstore_part = [&](int stage, int k0, int part) {
         unsigned char *base = smem + stage * Cfg::STAGE_BYTES;
+        const bool zero = K_TAIL && (min(k0, k_last) + kchunk >= K);
+        const vec8 z = {};
 #pragma unroll
-        for (int i = 0; i < Cfg::XI; ++i) *reinterpret_cast<vec8 *>(base + xl[i]) = xs[i];
+        for (int i = 0; i < Cfg::XI; ++i)
+            if (i % KSTEPS == part) *reinterpret_cast<vec8 *>(base + xl[i]) = (K_TAIL && zero) ? z : xs[i];
 #pragma unroll
-        for (int i = 0; i < Cfg::WI; ++i) *reinterpret_cast<vec8 *>(base + wl[i]) = ws[i];
+        for (int i = 0; i < Cfg::WI; ++i)
+            if (i % KSTEPS == part) *reinterpret_cast<vec8 *>(base + wl[i]) = (K_TAIL && zero) ? z : ws[i];
     };
 
     f32x16 acc[TM][TN];
@@ -165,37 +183,48 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // LDS rows this lane reads for its operand fragments
-    int xrow[TM], wrow[TN];
+    // LDS byte offsets of this lane's operand fragments for k-step 0.  Chunk index 2*step + lh and the XOR swizzle
+    // only touch bits 4..6 of the offset, so step s is the same offset XOR 32*s.
+    static_assert(RB == 128, "fragment addressing below assumes 64-element k-tiles");
+    int xoff[TM], woff[TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) xrow[i] = wave_m * Cfg::WM + i * 32 + lr;
+    for (int i = 0; i < TM; ++i) xoff[i] = swz_offset<RB>(wave_m * Cfg::WM + i * 32 + lr, lh);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) wrow[j] = wave_n * Cfg::WN + j * 32 + lr;
+    for (int j = 0; j < TN; ++j) woff[j] = Cfg::X_BYTES + swz_offset<RB>(wave_n * Cfg::WN + j * 32 + lr, lh);
 
-    const int nk = (K + BK - 1) / BK;
-    gload(0);
-    lstore(0);
+#pragma unroll
+    for (int part = 0; part < KSTEPS; ++part) gload_part(0, part);
+#pragma unroll
+    for (int part = 0; part < KSTEPS; ++part) lstore_part(0, 0, part);
+#pragma unroll
+    for (int part = 0; part < KSTEPS; ++part) gload_part(BK, part);
     __syncthreads();
 
+    vec8 fa[2][TN], fb[2][TM];
     for (int kt = 0; kt < nk; ++kt) {
-        if (kt + 1 < nk) gload((kt + 1) * BK);
-        const unsigned char *sx = smem + (kt & 1) * Cfg::STAGE_BYTES;
-        const unsigned char *sw = sx + Cfg::X_BYTES;
+        const unsigned char *cur = smem + (kt & 1) * Cfg::STAGE_BYTES;
+        const int nxt = (kt + 1) & 1;
 #pragma unroll
-        for (int s = 0; s < BK / 16; ++s) {
-            vec8 a[TN], b[TM];
+        for (int j = 0; j < TN; ++j) fa[0][j] = *reinterpret_cast<const vec8 *>(cur + woff[j]);
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-                a[j] = *reinterpret_cast<const vec8 *>(sw + swz_offset<RB>(wrow[j], 2 * s + lh));
+        for (int i = 0; i < TM; ++i) fb[0][i] = *reinterpret_cast<const vec8 *>(cur + xoff[i]);
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            if (st + 1 < KSTEPS) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    fa[(st + 1) & 1][j] = *reinterpret_cast<const vec8 *>(cur + (woff[j] ^ (32 * (st + 1))));
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    fb[(st + 1) & 1][i] = *reinterpret_cast<const vec8 *>(cur + (xoff[i] ^ (32 * (st + 1))));
+            }
+            lstore_part(nxt, (kt + 1) * BK, st);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                b[i] = *reinterpret_cast<const vec8 *>(sx + swz_offset<RB>(xrow[i], 2 * s + lh));
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = mfma32(a[j], b[i], acc[i][j]);
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma32(fa[st & 1][j], fb[st & 1][i], acc[i][j]);
+            gload_part((kt + 2) * BK, st);
         }
-        if (kt + 1 < nk) lstore((kt + 1) & 1);
         __syncthreads();
     }
 
@@ -325,9 +354,9 @@ struct LinearArgs {
     hipStream_t st;
 };
 
-template <typename T, typename Cfg, int ACT>
+template <typename T, typename Cfg, int ACT, bool K_TAIL>
 static void launch_mfma_act(const LinearArgs &a) {
-    auto kern = linear_mfma_kernel<T, Cfg, ACT>;
+    auto kern = linear_mfma_kernel<T, Cfg, ACT, K_TAIL>;
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -349,15 +378,15 @@ static void launch_mfma_act(const LinearArgs &a) {
                        out_vec_ok, ai_vec_ok, bias_vec_ok);
 }
 
-template <typename T, typename Cfg>
+template <typename T, typename Cfg, bool K_TAIL>
 static void launch_mfma_cfg(const LinearArgs &a) {
     switch (a.act) {
-        case KERNL_ACT_RELU: launch_mfma_act<T, Cfg, KERNL_ACT_RELU>(a); break;
-        case KERNL_ACT_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_TANH>(a); break;
-        case KERNL_ACT_GELU_ERF: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_ERF>(a); break;
-        case KERNL_ACT_GELU_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_TANH>(a); break;
-        case KERNL_ACT_SILU: launch_mfma_act<T, Cfg, KERNL_ACT_SILU>(a); break;
-        default: launch_mfma_act<T, Cfg, KERNL_ACT_NONE>(a); break;
+        case KERNL_ACT_RELU: launch_mfma_act<T, Cfg, KERNL_ACT_RELU, K_TAIL>(a); break;
+        case KERNL_ACT_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_TANH, K_TAIL>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_ERF, K_TAIL>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_TANH, K_TAIL>(a); break;
+        case KERNL_ACT_SILU: launch_mfma_act<T, Cfg, KERNL_ACT_SILU, K_TAIL>(a); break;
+        default: launch_mfma_act<T, Cfg, KERNL_ACT_NONE, K_TAIL>(a); break;
     }
 }
 
@@ -390,9 +419,12 @@ static int linear_mfma_dispatch(const LinearArgs &a) {
         if (c2 < best) { best = c2; pick = 2; }
         if (c3 < best) { best = c3; pick = 3; }
     }
-    if (pick == 1) launch_mfma_cfg<T, Tile256x256>(a);
-    else if (pick == 2) launch_mfma_cfg<T, Tile256x192>(a);
-    else launch_mfma_cfg<T, Tile128x128>(a);
+    // A k-extent that is not a multiple of the 64-element k-tile needs the zero-filling variant of the loop, which
+    // is only built for the 128x128 tile.
+    if (a.K % 64 != 0) launch_mfma_cfg<T, Tile128x128, true>(a);
+    else if (pick == 1) launch_mfma_cfg<T, Tile256x256, false>(a);
+    else if (pick == 2) launch_mfma_cfg<T, Tile256x192, false>(a);
+    else launch_mfma_cfg<T, Tile128x128, false>(a);
     return check_launch("linear (mfma)");
 }
 
@@ -439,7 +471,8 @@ extern "C" int kernl_linear_fwd(const void *x, const void *w, const void *bias, 
     a.st = static_cast<hipStream_t>(stream);
 
     if (dtype == KERNL_F16 || dtype == KERNL_BF16) {
-        const bool mfma_ok = a.x_cs == 1 && K % 8 == 0 && a.x_rs % 8 == 0 && aligned16(x) && aligned16(w);
+        const bool mfma_ok = a.x_cs == 1 && K % 8 == 0 && a.x_rs % 8 == 0 && aligned16(x) && aligned16(w) &&
+                             a.x_rs < (1 << 22) && K < (1 << 22);  // per-thread byte offsets inside a tile fit 32 bits
         if (mfma_ok) return dtype == KERNL_F16 ? linear_mfma_dispatch<f16>(a) : linear_mfma_dispatch<bf16>(a);
         if ((M + 63) / 64 > 65535) return set_error(KERNL_ERR_UNSUPPORTED, "linear: M too large for the strided path");
         return dtype == KERNL_F16 ? linear_fma_dispatch<f16>(a) : linear_fma_dispatch<bf16>(a);
