@@ -80,7 +80,7 @@ struct LinearTile {
     static constexpr int GROUP_M = 4;  // m-tiles walked together so one XCD's L2 sees a compact block
 };
 
-template <typename T, typename Cfg, int ACT, bool K_TAIL>
+template <typename T, typename Cfg, int ACT>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_BLOCKS)
 linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
                    T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx,
@@ -113,18 +113,23 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     const int lr = lane & 31, lh = lane >> 5;
 
     // ---- global -> register staging: thread owns chunks q = tid + THREADS*i, row q / CPR, chunk q % CPR.
-    // Addresses are a wave-uniform base (tile origin + k, advanced on the scalar unit) plus a per-thread 32-bit
-    // byte offset; rows past M or N are clamped to the last valid row (their results are never stored).
-    const unsigned char *xbase = reinterpret_cast<const unsigned char *>(X + (int64_t)m0 * ldx);
-    const unsigned char *wbase = reinterpret_cast<const unsigned char *>(W + (int64_t)n0 * K);
-    uint32_t xg[Cfg::XI], wg[Cfg::WI];  // byte offsets from xbase / wbase
+    // Loads are buffer loads: a wave-uniform resource (tile origin, extent up to the end of the last valid row),
+    // a loop-invariant per-thread 32-bit byte offset and the k position in a scalar register.  Anything past the
+    // extent — rows beyond M or N, k-tiles beyond K — reads as zero without touching memory, so the loop needs
+    // neither clamps nor branches; only a chunk that starts beyond K INSIDE a valid row is redirected by hand.
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    const int rows_x = min(BM, M - m0), rows_w = min(BN, N - n0);
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T *>(X + (int64_t)m0 * ldx), 0, (int)((((int64_t)rows_x - 1) * ldx + K) * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T *>(W + (int64_t)n0 * K), 0, (int)((int64_t)rows_w * K * 2), 0x00020000);
+    uint32_t xg[Cfg::XI], wg[Cfg::WI];  // byte offsets from the tile origins
     int xl[Cfg::XI], wl[Cfg::WI];       // LDS byte offsets inside a stage
 #pragma unroll
     for (int i = 0; i < Cfg::XI; ++i) {
         const int q = tid + Cfg::THREADS * i;
         const int row = q / CPR, c = q % CPR;
-        const int gm = min(m0 + row, M - 1) - m0;
-        xg[i] = (uint32_t)(((int64_t)gm * ldx + c * 8) * 2);
+        xg[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) : kOutOfRange;
         xl[i] = swz_offset<RB>(row, c);
     }
 #pragma unroll
@@ -132,8 +137,8 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         const int q = tid + Cfg::THREADS * i;
         const int row = q / CPR, c = q % CPR;
         // LDS row `row` feeds MFMA row (row % 32) of its 32-block and carries weight row rowperm16(row % 32).
-        const int gn = min(n0 + (row & ~31) + rowperm16(row & 31), N - 1) - n0;
-        wg[i] = (uint32_t)(((int64_t)gn * K + c * 8) * 2);
+        const int wrow = (row & ~31) + rowperm16(row & 31);
+        wg[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) : kOutOfRange;
         wl[i] = Cfg::X_BYTES + swz_offset<RB>(row, c);
     }
     const int kchunk = (tid % CPR) * 8;  // same for every i because THREADS % CPR == 0
@@ -143,36 +148,34 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     //   Iteration kt, k-step s:  read the operand fragments of step s+1 from LDS, store a quarter of tile kt+1
     //   from registers into the other LDS stage, run the MFMAs of step s, and re-issue the global loads of the
     //   same quarter for tile kt+2.  Global latency gets a whole iteration to hide, LDS stores ride under the
-    //   MFMAs, and there is one barrier per k-tile.  The loop body is branch-free: past the last k-tile the
-    //   loads re-read the last tile and the stores fill a stage nobody reads, which keeps the number of loads in
-    //   flight known at compile time (the memory counters are waited on by count).
+    //   MFMAs, and there is one barrier per k-tile.  The loop body is branch-free (past the last k-tile the loads
+    //   return zeros and the stores fill a stage nobody reads), which keeps the number of loads in flight known
+    //   at compile time: the memory counters are waited on by count.
     constexpr int KSTEPS = BK / 16;
     vec8 xs[Cfg::XI], ws[Cfg::WI];
     const int nk = (K + BK - 1) / BK;
-    const int k_last = (nk - 1) * BK;
 
     auto gload_part = [&](int k0, int part) {  // chunks i with i % KSTEPS == part
-        int koff = min(k0, k_last);
-        // K_TAIL: a chunk beyond K re-reads the first chunk of its row (always mapped); it is zeroed in lstore_part
-        if (K_TAIL && koff + kchunk >= K) koff = -kchunk;
-        const unsigned char *xb = xbase + (int64_t)koff * 2, *wb = wbase + (int64_t)koff * 2;
+        const bool inside = k0 + kchunk < K;   // K % 8 == 0: a 16-byte chunk is entirely inside or outside
 #pragma unroll
         for (int i = 0; i < Cfg::XI; ++i)
-            if (i % KSTEPS == part) xs[i] = *reinterpret_cast<const vec8 *>(xb + xg[i]);
+            if (i % KSTEPS == part)
+                xs[i] = __builtin_bit_cast(
+                    vec8, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, inside ? xg[i] : kOutOfRange, k0 * 2, 0));
 #pragma unroll
         for (int i = 0; i < Cfg::WI; ++i)
-            if (i % KSTEPS == part) ws[i] = *reinterpret_cast<const vec8 *>(wb + wg[i]);
+            if (i % KSTEPS == part)
+                ws[i] = __builtin_bit_cast(
+                    vec8, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, inside ? wg[i] : kOutOfRange, k0 * 2, 0));
     };
-    auto lstore_part = [&](int stage, int k0, int part) {
+    auto lstore_part = [&](int stage, int part) {
         unsigned char *base = smem + stage * Cfg::STAGE_BYTES;
-        const bool zero = K_TAIL && (min(k0, k_last) + kchunk >= K);
-        const vec8 z = {};
 #pragma unroll
         for (int i = 0; i < Cfg::XI; ++i)
-            if (i % KSTEPS == part) *reinterpret_cast<vec8 *>(base + xl[i]) = (K_TAIL && zero) ? z : xs[i];
+            if (i % KSTEPS == part) *reinterpret_cast<vec8 *>(base + xl[i]) = xs[i];
 #pragma unroll
         for (int i = 0; i < Cfg::WI; ++i)
-            if (i % KSTEPS == part) *reinterpret_cast<vec8 *>(base + wl[i]) = (K_TAIL && zero) ? z : ws[i];
+            if (i % KSTEPS == part) *reinterpret_cast<vec8 *>(base + wl[i]) = ws[i];
     };
 
     f32x16 acc[TM][TN];
@@ -185,7 +188,7 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 
     // LDS byte offsets of this lane's operand fragments for k-step 0.  Chunk index 2*step + lh and the XOR swizzle
     // only touch bits 4..6 of the offset, so step s is the same offset XOR 32*s.
-    static_assert(RB == 128, "fragment addressing below assumes 64-element k-tiles");
+    static_assert(RB == 128 || RB == 64, "fragment addressing below assumes 64- or 32-element k-tiles");
     int xoff[TM], woff[TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i) xoff[i] = swz_offset<RB>(wave_m * Cfg::WM + i * 32 + lr, lh);
@@ -195,7 +198,7 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 #pragma unroll
     for (int part = 0; part < KSTEPS; ++part) gload_part(0, part);
 #pragma unroll
-    for (int part = 0; part < KSTEPS; ++part) lstore_part(0, 0, part);
+    for (int part = 0; part < KSTEPS; ++part) lstore_part(0, part);
 #pragma unroll
     for (int part = 0; part < KSTEPS; ++part) gload_part(BK, part);
     __syncthreads();
@@ -218,12 +221,15 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
                 for (int i = 0; i < TM; ++i)
                     fb[(st + 1) & 1][i] = *reinterpret_cast<const vec8 *>(cur + (xoff[i] ^ (32 * (st + 1))));
             }
-            lstore_part(nxt, (kt + 1) * BK, st);
+            lstore_part(nxt, st);
+            __builtin_amdgcn_sched_barrier(0);  // keep the order: fragment reads, LDS stores, MFMAs, global loads
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) acc[i][j] = mfma32(fa[st & 1][j], fb[st & 1][i], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
             gload_part((kt + 2) * BK, st);
+            __builtin_amdgcn_sched_barrier(0);
         }
         __syncthreads();
     }
@@ -354,9 +360,9 @@ struct LinearArgs {
     hipStream_t st;
 };
 
-template <typename T, typename Cfg, int ACT, bool K_TAIL>
+template <typename T, typename Cfg, int ACT>
 static void launch_mfma_act(const LinearArgs &a) {
-    auto kern = linear_mfma_kernel<T, Cfg, ACT, K_TAIL>;
+    auto kern = linear_mfma_kernel<T, Cfg, ACT>;
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -378,15 +384,15 @@ static void launch_mfma_act(const LinearArgs &a) {
                        out_vec_ok, ai_vec_ok, bias_vec_ok);
 }
 
-template <typename T, typename Cfg, bool K_TAIL>
+template <typename T, typename Cfg>
 static void launch_mfma_cfg(const LinearArgs &a) {
     switch (a.act) {
-        case KERNL_ACT_RELU: launch_mfma_act<T, Cfg, KERNL_ACT_RELU, K_TAIL>(a); break;
-        case KERNL_ACT_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_TANH, K_TAIL>(a); break;
-        case KERNL_ACT_GELU_ERF: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_ERF, K_TAIL>(a); break;
-        case KERNL_ACT_GELU_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_TANH, K_TAIL>(a); break;
-        case KERNL_ACT_SILU: launch_mfma_act<T, Cfg, KERNL_ACT_SILU, K_TAIL>(a); break;
-        default: launch_mfma_act<T, Cfg, KERNL_ACT_NONE, K_TAIL>(a); break;
+        case KERNL_ACT_RELU: launch_mfma_act<T, Cfg, KERNL_ACT_RELU>(a); break;
+        case KERNL_ACT_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_TANH>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_ERF>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_TANH>(a); break;
+        case KERNL_ACT_SILU: launch_mfma_act<T, Cfg, KERNL_ACT_SILU>(a); break;
+        default: launch_mfma_act<T, Cfg, KERNL_ACT_NONE>(a); break;
     }
 }
 
@@ -394,6 +400,7 @@ static void launch_mfma_cfg(const LinearArgs &a) {
 typedef LinearTile<256, 256, 64, 2, 4, 1> Tile256x256;
 typedef LinearTile<256, 192, 64, 4, 2, 1> Tile256x192;
 typedef LinearTile<128, 128, 64, 2, 2, 2> Tile128x128;
+typedef LinearTile<256, 128, 32, 2, 2, 2> Tile256x128k32;  // 48 KB of LDS: two workgroups per CU
 
 // Number of "rounds" a tile shape needs on 256 CUs times the work of one tile: a proxy for run time.
 static double tile_cost(int M, int N, int bm, int bn, int blocks_per_cu) {
@@ -419,12 +426,10 @@ static int linear_mfma_dispatch(const LinearArgs &a) {
         if (c2 < best) { best = c2; pick = 2; }
         if (c3 < best) { best = c3; pick = 3; }
     }
-    // A k-extent that is not a multiple of the 64-element k-tile needs the zero-filling variant of the loop, which
-    // is only built for the 128x128 tile.
-    if (a.K % 64 != 0) launch_mfma_cfg<T, Tile128x128, true>(a);
-    else if (pick == 1) launch_mfma_cfg<T, Tile256x256, false>(a);
-    else if (pick == 2) launch_mfma_cfg<T, Tile256x192, false>(a);
-    else launch_mfma_cfg<T, Tile128x128, false>(a);
+    if (pick == 1) launch_mfma_cfg<T, Tile256x256>(a);
+    else if (pick == 2) launch_mfma_cfg<T, Tile256x192>(a);
+    else if (pick == 4) launch_mfma_cfg<T, Tile256x128k32>(a);
+    else launch_mfma_cfg<T, Tile128x128>(a);
     return check_launch("linear (mfma)");
 }
 
