@@ -88,8 +88,8 @@ def main():
     q, k, v, mask, lengths = config1_inputs()
     B, H, S, D = q.shape
     dense_flop = 4.0 * B * H * S * S * D
-    # key tiles of 128 that are entirely padding are skipped by the kernel: flops actually executed
-    executed_flop = sum(4.0 * H * S * D * (128 * ((int(n) + 127) // 128)) for n in lengths)
+    # key tiles of 64 that are entirely padding are skipped by the kernel: flops actually executed
+    executed_flop = sum(4.0 * H * S * D * (64 * ((int(n) + 63) // 64)) for n in lengths)
     qd, kd, vd, md = q.to(dev), k.to(dev), v.to(dev), mask.to(dev)
     out = torch.empty_like(qd)
 

@@ -140,72 +140,75 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
         for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const vec8 *>(qrow + s * 16);
     }
 
-    // ---- global -> register staging of one K/V tile
+    // ---- global -> register staging of one K/V tile.  Buffer loads: a uniform resource covering this head's
+    // K (V) rows, a loop-invariant 32-bit thread offset and the tile's first row as a scalar offset.  Rows past
+    // the last key lie beyond the resource's extent and read as zero in hardware.
     const int v_dc = tid % DC, v_ng = tid / DC;  // this thread's 4-key x 8-feature block of V
-    vec8 kst[KI], vst[4];
-    float bias_st = 0.0f;
-    int staged_n0 = 0;  // first key of the tile held in the staging registers
-    auto gload = [&](int tile) {
-        const int n0 = tile * BN;
-        staged_n0 = n0;
-        // rows past the last key are read from the last key's row (always mapped) and zeroed in lstore
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T *>(kp), 0, (int)((((int64_t)N - 1) * p.ks[2] + D) * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T *>(vp), 0, (int)((((int64_t)N - 1) * p.vs[2] + D) * 2), 0x00020000);
+    uint32_t kg[KI], vg[4];  // byte offsets of this thread's chunks inside a tile
+    int kl[KI], vl[8];       // LDS byte offsets inside a stage
 #pragma unroll
-        for (int i = 0; i < KI; ++i) {
-            const int qd = tid + 256 * i;
-            const int row = qd / DC, c = qd % DC;
-            kst[i] = *reinterpret_cast<const vec8 *>(kp + (int64_t)min(n0 + row, N - 1) * p.ks[2] + c * 8);
-        }
-        if (VBLK == 256 || tid < VBLK) {
+    for (int i = 0; i < KI; ++i) {
+        const int qd = tid + 256 * i;
+        const int row = qd / DC, c = qd % DC;
+        kg[i] = (uint32_t)(((int64_t)row * p.ks[2] + c * 8) * 2);
+        kl[i] = swz_offset<KROW>(row, c);
+    }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int n = min(n0 + v_ng * 4 + r, N - 1);
-                vst[r] = *reinterpret_cast<const vec8 *>(vp + (int64_t)n * p.vs[2] + v_dc * 8);
-            }
-        }
-        if (tid < BN) {
-            const int n = n0 + tid;
-            float bv = 0.0f;
-            if (MASK_MODE == MASK_VECTOR)
-                bv = scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_base + min(n, N - 1) * p.ms[3]), p.clamp);
-            if (n >= N) bv = -INFINITY;
-            bias_st = bv;
-        }
-    };
-    auto lstore = [&](int stage) {
-        unsigned char *kb = smem + stage * STAGE;
-        unsigned char *vb = kb + K_BYTES;
-        if (staged_n0 + BN > N) {  // tail tile (uniform): keys past the end contribute exact zeros
-            const vec8 z = {};
-#pragma unroll
-            for (int i = 0; i < KI; ++i)
-                if (staged_n0 + (tid + 256 * i) / DC >= N) kst[i] = z;
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                if (staged_n0 + v_ng * 4 + r >= N) vst[r] = z;
-        }
-#pragma unroll
-        for (int i = 0; i < KI; ++i) {
-            const int qd = tid + 256 * i;
-            const int row = qd / DC, c = qd % DC;
-            *reinterpret_cast<vec8 *>(kb + swz_offset<KROW>(row, c)) = kst[i];
-        }
+    for (int r = 0; r < 4; ++r) vg[r] = (uint32_t)(((int64_t)(v_ng * 4 + r) * p.vs[2] + v_dc * 8) * 2);
+    {
         // Vᵀ: feature d lives in LDS row (d & ~31) + inverse_rowperm16(d & 31); the 4 keys of this thread go to
-        // 8-byte slot pos/4 of that row where pos swaps bits 2 and 3 of the key index (see header comment).
+        // the 8-byte slot pos/4 of that row, where pos swaps bits 2 and 3 of the key index (see header comment).
         const int nloc = v_ng * 4;
         const int pos = (nloc & ~12) | ((nloc & 4) << 1) | ((nloc & 8) >> 1);
         const int chunk = pos >> 3, half = (pos >> 2) & 1;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int d = v_dc * 8 + e;
+            const int x = d & 31;
+            const int row = (d & ~31) + 8 * ((x >> 2) & 3) + 4 * (x >> 4) + (x & 3);
+            vl[e] = K_BYTES + swz_offset<VROW>(row, chunk) + half * 8;
+        }
+    }
+    vec8 kst[KI], vst[4];
+    float bias_st = 0.0f;
+    auto gload = [&](int tile) {
+        const int n0 = tile * BN;
+        const int k_soff = (int)((int64_t)n0 * p.ks[2] * 2), v_soff = (int)((int64_t)n0 * p.vs[2] * 2);
+#pragma unroll
+        for (int i = 0; i < KI; ++i)
+            kst[i] = __builtin_bit_cast(vec8, __builtin_amdgcn_raw_buffer_load_b128(krsrc, kg[i], k_soff, 0));
+        if (VBLK == 256 || tid < VBLK) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                vst[r] = __builtin_bit_cast(vec8, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vg[r], v_soff, 0));
+        }
+        if (MASK_MODE == MASK_VECTOR || n0 + BN > N) {
+            if (tid < BN) {
+                const int n = n0 + tid;
+                float bv = 0.0f;
+                if (MASK_MODE == MASK_VECTOR)
+                    bv = scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_base + min(n, N - 1) * p.ms[3]), p.clamp);
+                if (n >= N) bv = -INFINITY;
+                bias_st = bv;
+            }
+        }
+    };
+    auto lstore = [&](int stage) {
+        unsigned char *sb = smem + stage * STAGE;
+#pragma unroll
+        for (int i = 0; i < KI; ++i) *reinterpret_cast<vec8 *>(sb + kl[i]) = kst[i];
         if (VBLK == 256 || tid < VBLK) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const int d = v_dc * 8 + e;
-                const int x = d & 31;
-                const int row = (d & ~31) + 8 * ((x >> 2) & 3) + 4 * (x >> 4) + (x & 3);
                 T quad[4] = {vst[0][e], vst[1][e], vst[2][e], vst[3][e]};
-                *reinterpret_cast<uint64_t *>(vb + swz_offset<VROW>(row, chunk) + half * 8) =
-                    *reinterpret_cast<const uint64_t *>(quad);
+                *reinterpret_cast<uint64_t *>(sb + vl[e]) = *reinterpret_cast<const uint64_t *>(quad);
             }
         }
-        if (tid < BN) *reinterpret_cast<float *>(kb + K_BYTES + V_BYTES + tid * 4) = bias_st;
+        if (tid < BN) *reinterpret_cast<float *>(sb + K_BYTES + V_BYTES + tid * 4) = bias_st;
     };
 
     // ---- running state of this lane's query row
@@ -308,32 +311,28 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
             const float m_new = fmaxf(m_i, mx);
             const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
             const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
-            float rs = 0.0f;
+            // exponentiate in place; the row sum is taken below from the ROUNDED probabilities (two per
+            // v_dot2c), i.e. from exactly the values that enter P·V
             if (general) {
 #pragma unroll
                 for (int nb = 0; nb < NBS; ++nb)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const float pv = __builtin_amdgcn_exp2f(s_acc[nb][v] - m_use);
-                        s_acc[nb][v] = pv;
-                        rs += pv;
-                    }
+                    for (int v = 0; v < 16; ++v) s_acc[nb][v] = __builtin_amdgcn_exp2f(s_acc[nb][v] - m_use);
             } else {
 #pragma unroll
                 for (int nb = 0; nb < NBS; ++nb)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const float pv = __builtin_amdgcn_exp2f(s_acc[nb][v] * c - m_use);
-                        s_acc[nb][v] = pv;
-                        rs += pv;
-                    }
+                    for (int v = 0; v < 16; ++v) s_acc[nb][v] = __builtin_amdgcn_exp2f(s_acc[nb][v] * c - m_use);
             }
-            l_i = l_i * alpha + rs;
+            // the accumulator only needs rescaling when some row of this wave saw a new maximum
+            if (__builtin_amdgcn_ballot_w64(m_new != m_i) != 0) {
+#pragma unroll
+                for (int d = 0; d < DB; ++d)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
+            }
             m_i = m_new;
-#pragma unroll
-            for (int d = 0; d < DB; ++d)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
+            float rs = 0.0f;
 
             // ---- Oᵀ += Vᵀ · Pᵀ
 #pragma unroll
@@ -341,8 +340,10 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                 const int nb = ps >> 1, half8 = (ps & 1) * 8;
                 u32x4 pk;
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int j = 0; j < 4; ++j) {
                     pk[j] = pack2<T>(s_acc[nb][half8 + 2 * j], s_acc[nb][half8 + 2 * j + 1]);
+                    rs = pair_sum_acc<T>(pk[j], rs);
+                }
                 const vec8 pf = __builtin_bit_cast(vec8, pk);
 #pragma unroll
                 for (int d = 0; d < DB; ++d) {
@@ -350,6 +351,7 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                     o_acc[d] = mfma32(vf, pf, o_acc[d]);
                 }
             }
+            l_i = l_i * alpha + rs;
         }
 
         if (it + 1 < nt) lstore((it + 1) & 1);
@@ -529,17 +531,23 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
     };
     const bool mfma_ok = !g_attention_force_scalar && (D == 64 || D == 128) && sm_scale > 0.0f &&
                          rows_ok(q, q_strides) && rows_ok(k, k_strides) && rows_ok(v, v_strides) &&
-                         rows_ok(out, o_strides) && (int64_t)((B * H + 7) / 8) * 8 * p.nq_tiles < (1ll << 31);
+                         rows_ok(out, o_strides) && (int64_t)((B * H + 7) / 8) * 8 * p.nq_tiles < (1ll << 31) &&
+                         k_strides[2] > 0 && v_strides[2] > 0 &&  // one head's K / V extent must fit 31-bit byte offsets
+                         (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30);
     if (mfma_ok) {
         if (dtype == KERNL_F16) {
             if (D == 64) {
-                if (g_attention_variant == 1) launch_mfma<f16, 64, 128, 64, 2>(p, mask_mode, causal, st);
-                else if (g_attention_variant == 2) launch_mfma<f16, 64, 64, 64, 2>(p, mask_mode, causal, st);
-                else launch_mfma<f16, 64, 64, 64, 3>(p, mask_mode, causal, st);
+                // measured on config 1: 64-key tiles at 3 waves/SIMD win without causal masking (finer skipping of
+                // padded key tiles, more waves to interleave), 128-key tiles at 2 waves/SIMD win with it
+                int variant = g_attention_variant;
+                if (variant == 0) variant = (causal || mask_mode == MASK_MATRIX) ? 3 : 1;
+                if (variant == 1) launch_mfma<f16, 64, 64, 64, 3>(p, mask_mode, causal, st);
+                else if (variant == 2) launch_mfma<f16, 64, 64, 64, 2>(p, mask_mode, causal, st);
+                else launch_mfma<f16, 64, 128, 64, 2>(p, mask_mode, causal, st);
             }
             else launch_mfma<f16, 128, 64, 32, 2>(p, mask_mode, causal, st);
         } else {
-            if (D == 64) launch_mfma<bf16, 64, 64, 64, 3>(p, mask_mode, causal, st);
+            if (D == 64) launch_mfma<bf16, 64, 128, 64, 2>(p, mask_mode, causal, st);
             else launch_mfma<bf16, 128, 64, 32, 2>(p, mask_mode, causal, st);
         }
         return check_launch("attention (mfma)");

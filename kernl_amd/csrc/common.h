@@ -90,6 +90,20 @@ __device__ __forceinline__ uint32_t pack2<bf16>(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, p);
 }
 
+// acc + lo + hi of a packed pair of 16-bit values, accumulated in fp32 (v_dot2c_f32_{f16,bf16} against (1, 1)).
+template <typename T>
+__device__ __forceinline__ float pair_sum_acc(uint32_t packed, float acc);
+template <>
+__device__ __forceinline__ float pair_sum_acc<f16>(uint32_t packed, float acc) {
+    const f16x2 ones = {(f16)1.0f, (f16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, packed), ones, acc, false);
+}
+template <>
+__device__ __forceinline__ float pair_sum_acc<bf16>(uint32_t packed, float acc) {
+    const bf16x2 ones = {(bf16)1.0f, (bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, packed), ones, acc, false);
+}
+
 // ----------------------------------------------------------------------------------------------------
 // wave64 reductions: quad permutes and row mirrors on DPP, the last two steps through scalar lane reads.
 // Every lane receives the full result.
