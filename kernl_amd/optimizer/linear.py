@@ -133,6 +133,84 @@ def replace_linear_fn_constant_match(gm: torch.fx.GraphModule):
     replace_pattern(gm, pattern, replace)
 
 
+# concatenated parameters of fused sibling projections, keyed by the identity of the original tensors
+_fused_params = {}
+
+
+def fused_linear_wrapper(v: torch.Tensor, weights, biases):
+    """Several activation-free linears of the SAME input (BERT's query/key/value projections) as ONE GEMM against
+    the row-concatenated weights; returns the outputs as column slices of the single result.
+
+    The concatenated weight is built on the first call (the warm-up call that precedes graph capture) and cached by
+    the storage addresses and versions of the originals, so replays neither allocate nor copy.  No counterpart in the
+    reference, which launches one Triton GEMM per projection."""
+    key = tuple((w.data_ptr(), w._version, w.dtype) for w in weights) + tuple(
+        (0, 0, None) if b is None else (b.data_ptr(), b._version, b.dtype) for b in biases
+    )
+    cached = _fused_params.get(key)
+    if cached is None:
+        for w, b in zip(weights, biases):
+            # same one-time down-cast as linear_wrapper_functional
+            if w.dtype == torch.float32 and (v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")):
+                w.data = w.data.half()
+            if b is not None and b.dtype == torch.float32 and (v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")):
+                b.data = b.data.half()
+        weight = torch.cat([w.detach() for w in weights], dim=0).contiguous()
+        bias = None
+        if any(b is not None for b in biases):
+            bias = torch.cat(
+                [torch.zeros(w.shape[0], dtype=w.dtype, device=w.device) if b is None else b.detach() for w, b in zip(weights, biases)]
+            ).contiguous()
+        key = tuple((w.data_ptr(), w._version, w.dtype) for w in weights) + tuple(
+            (0, 0, None) if b is None else (b.data_ptr(), b._version, b.dtype) for b in biases
+        )
+        cached = (weight, bias, [w.shape[0] for w in weights])
+        _fused_params[key] = cached
+    weight, bias, sizes = cached
+    out = linear_layer(v, weight, bias, activation="")
+    return tuple(torch.split(out, sizes, dim=-1))
+
+
+torch.fx.wrap("fused_linear_wrapper")
+
+
+def fuse_sibling_linears(gm: torch.fx.GraphModule):
+    """`linear_wrapper_functional(v, w_i, b_i)` calls without activation that share the input `v` and whose weights
+    are graph inputs or attributes (i.e. parameters, not computed tensors) become one `fused_linear_wrapper` call."""
+    import operator
+
+    groups = {}
+    for node in gm.graph.nodes:
+        if node.op != "call_function" or node.target is not linear_wrapper_functional:
+            continue
+        if node.kwargs.get("activation", "") != "" or len(node.args) != 3:
+            continue
+        v, w, b = node.args
+        if not isinstance(v, torch.fx.Node) or not isinstance(w, torch.fx.Node) or w.op not in ("placeholder", "get_attr"):
+            continue
+        if b is not None and not (isinstance(b, torch.fx.Node) and b.op in ("placeholder", "get_attr")):
+            continue
+        shape = getattr(w.meta.get("example_value"), "shape", None)
+        groups.setdefault((v, None if shape is None else tuple(shape[1:])), []).append(node)
+    changed = False
+    for (v, _), nodes in groups.items():
+        if len(nodes) < 2:
+            continue
+        first = nodes[0]
+        with gm.graph.inserting_before(first):
+            fused = gm.graph.call_function(
+                fused_linear_wrapper, (v, [n.args[1] for n in nodes], [n.args[2] for n in nodes])
+            )
+            parts = [gm.graph.call_function(operator.getitem, (fused, i)) for i in range(len(nodes))]
+        for n, part in zip(nodes, parts):
+            n.replace_all_uses_with(part)
+            gm.graph.erase_node(n)
+        changed = True
+    if changed:
+        gm.graph.lint()
+        gm.recompile()
+
+
 def replace_all_linear(gm: torch.fx.GraphModule):
     replace_linear_activation(gm, torch.nn.Tanh(), "tanh")
     replace_linear_activation(gm, torch.nn.ReLU(), "relu")
@@ -141,3 +219,4 @@ def replace_all_linear(gm: torch.fx.GraphModule):
     replace_linear(gm)
     replace_linear_fn(gm)
     replace_linear_fn_constant_match(gm)
+    fuse_sibling_linears(gm)

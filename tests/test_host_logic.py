@@ -265,7 +265,9 @@ def test_backend_rewrites_dynamo_graph_of_bert():
         assert len(graphs) == 1
         t = _targets(graphs[0])
         assert t.count(fused) == 2
-        assert t.count("linear_wrapper_functional") == 2 * 6 + 1
+        # query/key/value projections share their input: one fused GEMM per layer, 3 + pooler stay separate
+        assert t.count("fused_linear_wrapper") == 2
+        assert t.count("linear_wrapper_functional") == 2 * 3 + 1
         assert t.count("add_layer_norm_wrapper_functional") == 5
         assert "softmax" not in t and "dropout" not in t and "gelu" not in t and "layer_norm" not in t and "linear" not in t
         # the padding mask reaches the kernel as a broadcast of a per-key tensor, not as a [B,1,S,S] matrix
