@@ -156,7 +156,9 @@ def main():
             "peak": PEAK_MFMA_F16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_MFMA_F16_TFLOPS, 4),
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy of known
+            # size (profiles/attention_config1_pmc_traffic.txt); algorithmic bytes are 100.7e6
+            "traffic": 99.3e6,
         },
     }
     extra = {
