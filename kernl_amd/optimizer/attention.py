@@ -174,11 +174,33 @@ def _scaled_patterns(d0: int, d1: int, is_causal: bool):
         output = torch.empty_like(q)
         return attention_wrapper(q, k, v, output, 1.0 / literal_scale, is_causal, None)
 
+    # softmax evaluated in fp32 and cast back (Llama-style eager attention); the fused kernel always keeps its
+    # softmax statistics in fp32, so the casts disappear
+    def pattern_mul_mask_f32(q, k, literal_scale, attention_mask, v, literal_dtype):
+        scores = torch.matmul(q, k.transpose(d0, d1)) * literal_scale
+        probs = torch.nn.functional.softmax(scores + attention_mask, dim=-1, dtype=torch.float32).to(literal_dtype)
+        return torch.matmul(probs, v)
+
+    def replace_mul_mask_f32(q, k, literal_scale, attention_mask, v, literal_dtype):
+        output = torch.empty_like(q)
+        return attention_wrapper(q, k, v, output, literal_scale, is_causal, attention_mask)
+
+    def pattern_mul_f32(q, k, literal_scale, v, literal_dtype):
+        scores = torch.matmul(q, k.transpose(d0, d1)) * literal_scale
+        probs = torch.nn.functional.softmax(scores, dim=-1, dtype=torch.float32).to(literal_dtype)
+        return torch.matmul(probs, v)
+
+    def replace_mul_f32(q, k, literal_scale, v, literal_dtype):
+        output = torch.empty_like(q)
+        return attention_wrapper(q, k, v, output, literal_scale, is_causal, None)
+
     return (
         (pattern_mul_mask, replace_mul_mask),
         (pattern_div_mask, replace_div_mask),
+        (pattern_mul_mask_f32, replace_mul_mask_f32),
         (pattern_mul, replace_mul),
         (pattern_div, replace_div),
+        (pattern_mul_f32, replace_mul_f32),
     )
 
 

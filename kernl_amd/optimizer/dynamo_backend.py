@@ -13,6 +13,7 @@ from kernl_amd.optimizer.dropout import remove_dropout
 from kernl_amd.optimizer.layer_norm import replace_layer_norm, replace_layer_norm_fn, replace_layer_norm_rms
 from kernl_amd.optimizer.linear import replace_all_linear
 from kernl_amd.optimizer.mask import (
+    constant_causal_masks_to_flag,
     drop_all_true_conjuncts,
     merge_nested_expands,
     scalar_tensors_to_full,
@@ -34,6 +35,7 @@ def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
     fuse_attention_pattern_3(gm, assume_causal)
     fuse_attention_scaled(gm, assume_causal)
     fuse_attention_sdpa(gm, assume_causal)
+    constant_causal_masks_to_flag(gm)
     replace_all_linear(gm)
     replace_layer_norm(gm)
     replace_layer_norm_fn(gm)

@@ -50,7 +50,7 @@ def scalar_tensors_to_full(gm: torch.fx.GraphModule):
 
 # Pure, shape-static ops that may be evaluated while compiling when every tensor operand is itself a constant.
 _FOLDABLE_FUNCTIONS = {
-    torch.arange, torch.ones, torch.zeros, torch.full, torch.tril, torch.triu,
+    torch.arange, torch.ones, torch.zeros, torch.full, torch.tril, torch.triu, torch.where,
     operator.add, operator.sub, operator.mul, operator.and_, operator.or_, operator.getitem,
     operator.ge, operator.gt, operator.le, operator.lt, operator.eq, operator.ne,
     torch.add, torch.sub, torch.mul, torch.bitwise_and, torch.bitwise_or,
@@ -169,5 +169,48 @@ def sink_expand_below_where(gm: torch.fx.GraphModule):
         gm.graph.erase_node(cond)
         changed = True
     if changed:
+        gm.graph.lint()
+        gm.recompile()
+
+
+def constant_causal_masks_to_flag(gm: torch.fx.GraphModule):
+    """An attention mask that is a compile-time constant and exactly the lower-triangular (causal) pattern is
+    dropped in favour of the kernel's `is_causal` flag: no [1,1,S,S] matrix is built, read or added.
+
+    Applies to the fused calls produced by `kernl_amd.optimizer.attention` (run after them).  A boolean mask must
+    equal tril; an additive mask must be 0 on and below the diagonal and <= -1e4 above it.  Only square masks
+    qualify (the kernel's causal mode is top-left aligned)."""
+    from kernl_amd.optimizer.attention import attention_wrapper, sdpa_wrapper
+
+    values = None
+    changed = False
+    for node in list(gm.graph.nodes):
+        if node.op != "call_function" or node.target not in (attention_wrapper, sdpa_wrapper):
+            continue
+        mask_idx = 6 if node.target is attention_wrapper else 3
+        mask = node.args[mask_idx]
+        if not isinstance(mask, Node):
+            continue
+        if values is None:
+            values = _fold_constants(gm)
+        val = values.get(mask)
+        if val is None or val.dim() < 2 or val.shape[-1] != val.shape[-2] or val.shape[-1] < 2:
+            continue
+        flat = val.reshape(-1, val.shape[-2], val.shape[-1])
+        tril = torch.tril(torch.ones(val.shape[-2:], dtype=torch.bool, device=val.device))
+        if val.dtype == torch.bool:
+            is_causal = bool((flat == tril).all())
+        else:
+            f = flat.float()
+            is_causal = bool(((f == 0) == tril).all()) and bool((f[:, ~tril] <= -1e4).all())
+        if not is_causal:
+            continue
+        args = list(node.args)
+        args[mask_idx] = None
+        args[5] = True  # is_causal, same position in both wrappers
+        node.args = tuple(args)
+        changed = True
+    if changed:
+        gm.graph.eliminate_dead_code()
         gm.graph.lint()
         gm.recompile()

@@ -300,3 +300,38 @@ def test_rms_norm_and_swiglu_patterns():
     assert rms.args[2] == 1e-05
     acts = sorted(n.kwargs.get("activation", "") for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "linear_wrapper_functional")
     assert acts == ["", "silu"]
+
+
+def test_llama_graph_rewrite_and_constant_causal_mask():
+    """HF Llama: Llama-spelled RMSNorm (eps wildcard), SiLU fused into the gate projection, query/key/value fused
+    into one GEMM, and the constant causal mask replaced by the kernel's is_causal flag."""
+    from transformers import LlamaConfig, LlamaModel
+
+    for attn_impl, fused, mask_idx in (("eager", "attention_wrapper", 6), ("sdpa", "sdpa_wrapper", 3)):
+        torch.manual_seed(0)
+        cfg = LlamaConfig(num_hidden_layers=2, hidden_size=128, num_attention_heads=2, num_key_value_heads=2,
+                          intermediate_size=256, vocab_size=100, rms_norm_eps=1e-5)
+        cfg._attn_implementation = attn_impl
+        model = LlamaModel(cfg).eval()
+        graphs = []
+
+        def backend(gm, example_inputs):
+            dynamo_backend_ofi(gm)
+            graphs.append(gm)
+            return lambda *a: None
+
+        torch._dynamo.reset()
+        try:
+            with torch.inference_mode():
+                torch._dynamo.optimize(backend, dynamic=False)(model.forward)(input_ids=torch.randint(0, 100, (1, 16)))
+        except Exception:
+            pass
+        assert len(graphs) == 1
+        t = _targets(graphs[0])
+        assert t.count(fused) == 2
+        assert t.count("layer_norm_rms_wrapper") == 2 * 2 + 1 and "rsqrt" not in t
+        assert t.count("fused_linear_wrapper") == 2 and "silu" not in t and "softmax" not in t
+        for node in graphs[0].graph.nodes:
+            if node.op == "call_function" and node.target.__name__ == fused:
+                assert node.args[mask_idx] is None and node.args[5] is True
+    torch._dynamo.reset()
