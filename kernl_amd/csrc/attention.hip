@@ -130,7 +130,7 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
         __syncthreads();
     }
     const bool use_list = (MASK_MODE == MASK_VECTOR && !CAUSAL && nt_all <= kMaxTiles);
-    const int nt = use_list ? n_listed : nt_all;
+    const int nt = use_list ? __builtin_amdgcn_readfirstlane(n_listed) : nt_all;
 
     // ---- Q fragments (MFMA "B" side: lane holds its query row, 8 consecutive features per k-step)
     vec8 qf[KS];
@@ -232,7 +232,7 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
     const int64_t mask_row = mask_base + (int64_t)min(my_m, M - 1) * (MASK_MODE == MASK_MATRIX ? p.ms[2] : 0);
 
     if (nt > 0) {
-        gload(use_list ? tile_list[0] : 0);
+        gload(use_list ? __builtin_amdgcn_readfirstlane(tile_list[0]) : 0);
         lstore(0);
     }
     // Every load issued so far (Q fragments included) has to have landed before the loop: otherwise the
@@ -242,9 +242,11 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
     __syncthreads();
 
     for (int it = 0; it < nt; ++it) {
-        const int tile = use_list ? tile_list[it] : it;
+        // tile indices come from LDS: tell the compiler they are wave-uniform, otherwise every buffer load that
+        // takes them as a scalar offset is wrapped in a waterfall loop
+        const int tile = use_list ? __builtin_amdgcn_readfirstlane(tile_list[it]) : it;
         const int n0 = tile * BN;
-        if (it + 1 < nt) gload(use_list ? tile_list[it + 1] : it + 1);
+        if (it + 1 < nt) gload(use_list ? __builtin_amdgcn_readfirstlane(tile_list[it + 1]) : it + 1);
 
         const unsigned char *kb = smem + (it & 1) * STAGE;
         const unsigned char *vb = kb + K_BYTES;
@@ -253,7 +255,7 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
         // The tile is consumed in sub-tiles of SUB keys, each a complete online-softmax step, which keeps
         // the live score registers at SUB/2 per lane.
         const bool tile_general = (MASK_MODE == MASK_MATRIX) || (n0 + BN > N) ||
-                                  (MASK_MODE == MASK_VECTOR && (use_list ? (tile_cls[tile] != 0) : true));
+                                  (MASK_MODE == MASK_VECTOR && (use_list ? (__builtin_amdgcn_readfirstlane(tile_cls[tile]) != 0) : true));
 #pragma nounroll
         for (int sub = 0; sub < BN / SUB; ++sub) {
             const int ns0 = n0 + sub * SUB;  // first key of the sub-tile
