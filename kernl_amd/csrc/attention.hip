@@ -27,6 +27,7 @@ static constexpr float kLog2eA = 1.4426950408889634f;
 static constexpr float kNegBig = -1.0e30f;            // anything below: exp2(x - rowmax) is exactly 0
 static constexpr float kClampFloor = -1.7014118e38f;  // scaled mask values are kept finite (-FLT_MAX / 2)
 static constexpr int kMaxTiles = 256;
+static constexpr float kRescaleThreshold = 8.0f;  // log2 units
 
 enum { MASK_NONE = 0, MASK_VECTOR = 1, MASK_MATRIX = 2 };
 
@@ -310,9 +311,21 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                 mx *= c;  // c > 0 on this path (checked by the host)
             }
             mx = halves32_max(mx);  // the other 16-key half of every 32-key block lives in lane ^ 32
-            const float m_new = fmaxf(m_i, mx);
-            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
+            // m_i is the exponent REFERENCE of this row, not necessarily its running maximum: it is only moved (and
+            // the accumulator and row sum rescaled) when the new maximum exceeds it by more than 2^8, so probabilities
+            // stay <= 256 — exact in fp32 and well inside the 16-bit range — and after the first tiles the rescale
+            // almost never runs.  The final O / l is independent of the reference.
+            if (__builtin_amdgcn_ballot_w64(mx > m_i + kRescaleThreshold) != 0) {
+                const float m_new = fmaxf(m_i, mx);
+                const float alpha = __builtin_amdgcn_exp2f(m_i - ((m_new == -INFINITY) ? 0.0f : m_new));
+                l_i *= alpha;
+#pragma unroll
+                for (int d = 0; d < DB; ++d)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
+                m_i = m_new;
+            }
+            const float m_use = (m_i == -INFINITY) ? 0.0f : m_i;
             // exponentiate in place; the row sum is taken below from the ROUNDED probabilities (two per
             // v_dot2c), i.e. from exactly the values that enter P·V
             if (general) {
@@ -326,14 +339,6 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
 #pragma unroll
                     for (int v = 0; v < 16; ++v) s_acc[nb][v] = __builtin_amdgcn_exp2f(s_acc[nb][v] * c - m_use);
             }
-            // the accumulator only needs rescaling when some row of this wave saw a new maximum
-            if (__builtin_amdgcn_ballot_w64(m_new != m_i) != 0) {
-#pragma unroll
-                for (int d = 0; d < DB; ++d)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
-            }
-            m_i = m_new;
             float rs = 0.0f;
 
             // ---- Oᵀ += Vᵀ · Pᵀ
@@ -353,7 +358,7 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                     o_acc[d] = mfma32(vf, pf, o_acc[d]);
                 }
             }
-            l_i = l_i * alpha + rs;
+            l_i += rs;
         }
 
         if (it + 1 < nt) lstore((it + 1) & 1);
