@@ -66,8 +66,8 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
     constexpr int NBS = SUB / 32, DB = D / 32, KS = D / 16;
     constexpr int DC = D / 8;                            // 16-byte chunks per K/V row
     constexpr int KI = BN * DC / 256;                    // K chunks per thread per tile
-    constexpr int VBLK = (BN / 4) * DC;                  // 4-key x 8-feature blocks of V per tile
-    static_assert(VBLK == 256 || VBLK == 128, "a thread transposes at most one 4x8 block of V per tile");
+    constexpr int VKEYS = BN * DC / 256;                 // every thread transposes a VKEYS-key x 8-feature block of V
+    static_assert(VKEYS == 4 || VKEYS == 2, "V blocks of 4 or 2 keys");
     static_assert(BN * DC % 256 == 0, "K chunks must split evenly over the threads");
 
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
@@ -144,12 +144,12 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
     // ---- global -> register staging of one K/V tile.  Buffer loads: a uniform resource covering this head's
     // K (V) rows, a loop-invariant 32-bit thread offset and the tile's first row as a scalar offset.  Rows past
     // the last key lie beyond the resource's extent and read as zero in hardware.
-    const int v_dc = tid % DC, v_ng = tid / DC;  // this thread's 4-key x 8-feature block of V
+    const int v_dc = tid % DC, v_ng = tid / DC;  // this thread's VKEYS-key x 8-feature block of V
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<T *>(kp), 0, (int)((((int64_t)N - 1) * p.ks[2] + D) * 2), 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<T *>(vp), 0, (int)((((int64_t)N - 1) * p.vs[2] + D) * 2), 0x00020000);
-    uint32_t kg[KI], vg[4];  // byte offsets of this thread's chunks inside a tile
+    uint32_t kg[KI], vg[VKEYS];  // byte offsets of this thread's chunks inside a tile
     int kl[KI], vl[8];       // LDS byte offsets inside a stage
 #pragma unroll
     for (int i = 0; i < KI; ++i) {
@@ -159,22 +159,23 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
         kl[i] = swz_offset<KROW>(row, c);
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) vg[r] = (uint32_t)(((int64_t)(v_ng * 4 + r) * p.vs[2] + v_dc * 8) * 2);
+    for (int r = 0; r < VKEYS; ++r) vg[r] = (uint32_t)(((int64_t)(v_ng * VKEYS + r) * p.vs[2] + v_dc * 8) * 2);
     {
-        // Vᵀ: feature d lives in LDS row (d & ~31) + inverse_rowperm16(d & 31); the 4 keys of this thread go to
-        // the 8-byte slot pos/4 of that row, where pos swaps bits 2 and 3 of the key index (see header comment).
-        const int nloc = v_ng * 4;
+        // Vᵀ: feature d lives in LDS row (d & ~31) + inverse_rowperm16(d & 31); the VKEYS consecutive keys of this
+        // thread stay adjacent at position pos of that row, where pos swaps bits 2 and 3 of the key index (see
+        // header comment).
+        const int nloc = v_ng * VKEYS;
         const int pos = (nloc & ~12) | ((nloc & 4) << 1) | ((nloc & 8) >> 1);
-        const int chunk = pos >> 3, half = (pos >> 2) & 1;
+        const int chunk = pos >> 3, within = (pos & 7) * 2;  // 16-byte chunk, byte offset inside it
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const int d = v_dc * 8 + e;
             const int x = d & 31;
             const int row = (d & ~31) + 8 * ((x >> 2) & 3) + 4 * (x >> 4) + (x & 3);
-            vl[e] = K_BYTES + swz_offset<VROW>(row, chunk) + half * 8;
+            vl[e] = K_BYTES + swz_offset<VROW>(row, chunk) + within;
         }
     }
-    vec8 kst[KI], vst[4];
+    vec8 kst[KI], vst[VKEYS];
     float bias_st = 0.0f;
     auto gload = [&](int tile) {
         const int n0 = tile * BN;
@@ -182,11 +183,9 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
 #pragma unroll
         for (int i = 0; i < KI; ++i)
             kst[i] = __builtin_bit_cast(vec8, __builtin_amdgcn_raw_buffer_load_b128(krsrc, kg[i], k_soff, 0));
-        if (VBLK == 256 || tid < VBLK) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                vst[r] = __builtin_bit_cast(vec8, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vg[r], v_soff, 0));
-        }
+        for (int r = 0; r < VKEYS; ++r)
+            vst[r] = __builtin_bit_cast(vec8, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vg[r], v_soff, 0));
         if (MASK_MODE == MASK_VECTOR || n0 + BN > N) {
             if (tid < BN) {
                 const int n = n0 + tid;
@@ -202,11 +201,14 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
         unsigned char *sb = smem + stage * STAGE;
 #pragma unroll
         for (int i = 0; i < KI; ++i) *reinterpret_cast<vec8 *>(sb + kl[i]) = kst[i];
-        if (VBLK == 256 || tid < VBLK) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                T quad[4] = {vst[0][e], vst[1][e], vst[2][e], vst[3][e]};
+        for (int e = 0; e < 8; ++e) {
+            if (VKEYS == 4) {
+                T quad[4] = {vst[0][e], vst[1][e], vst[VKEYS - 2][e], vst[VKEYS - 1][e]};
                 *reinterpret_cast<uint64_t *>(sb + vl[e]) = *reinterpret_cast<const uint64_t *>(quad);
+            } else {
+                T pair[2] = {vst[0][e], vst[1][e]};
+                *reinterpret_cast<uint32_t *>(sb + vl[e]) = *reinterpret_cast<const uint32_t *>(pair);
             }
         }
         if (tid < BN) *reinterpret_cast<float *>(sb + K_BYTES + V_BYTES + tid * 4) = bias_st;
