@@ -269,8 +269,10 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
             // along a Vᵀ row the sub-tile is SUB/8 chunks further; under the XOR swizzle that is an XOR too
             const int vsub_xor = sub * (SUB / 8) * 16;
 
-            // ---- Sᵀ = K · Qᵀ
+            // ---- Sᵀ = K · Qᵀ.  MFMA phases run at raised wave priority: a wave that is ready to feed the matrix
+            // pipe goes first, the other waves of the SIMD fill the gaps with their softmax VALU work.
             f32x16 s_acc[NBS];
+            __builtin_amdgcn_s_setprio(2);
 #pragma unroll
             for (int nb = 0; nb < NBS; ++nb) {
 #pragma unroll
@@ -281,6 +283,8 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                     s_acc[nb] = mfma32(kf, qf[ks], s_acc[nb]);
                 }
             }
+
+            __builtin_amdgcn_s_setprio(0);
 
             // ---- online softmax on this lane's row; key of s_acc[nb][v] is ns0 + 32 nb + 8 (v/4) + 4 lh + (v%4)
             const bool general = tile_general || (CAUSAL && (ns0 + SUB - 1 > m_wave0));
@@ -344,6 +348,7 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
             float rs = 0.0f;
 
             // ---- Oᵀ += Vᵀ · Pᵀ
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int ps = 0; ps < SUB / 16; ++ps) {
                 const int nb = ps >> 1, half8 = (ps & 1) * 8;
@@ -360,6 +365,7 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                     o_acc[d] = mfma32(vf, pf, o_acc[d]);
                 }
             }
+            __builtin_amdgcn_s_setprio(0);
             l_i += rs;
         }
 
