@@ -126,9 +126,8 @@ int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, 
  *   kernl_linear_force_tile      0 = heuristic (default), 1 = 256x256, 2 = 256x192, 3 = 128x128 output tile
  *                                of the MFMA linear kernel.
  *   kernl_attention_force_scalar non-zero routes every attention call through the strided scalar kernel.
- *   kernl_attention_set_variant  key-tile shape / occupancy of the head-size-64 fp16 MFMA attention kernel:
- *                                0 = heuristic, 1 = 64 keys at 3 waves/SIMD, 2 = 64 keys at 2 waves/SIMD,
- *                                3 = 128 keys at 2 waves/SIMD.
+ *   kernl_attention_set_variant  register budget of the head-size-64 MFMA attention kernel: 0 = heuristic,
+ *                                1 = built for 3 waves/SIMD, 2 = built for 2 waves/SIMD.
  */
 void kernl_linear_force_tile(int which);
 void kernl_attention_force_scalar(int on);

@@ -7,15 +7,16 @@
 // renormalisation, attention.py:399-417) — the same value up to fp32 rounding.
 //
 // MFMA path.  A workgroup of 4 waves owns 128 query rows of one (batch, head); each wave owns 32 of them.
-// Key/value tiles are staged HBM -> VGPR -> LDS (double buffered, one barrier per tile):
-//   K tile  [BN keys][D]      row-major, 16-byte chunks XOR-swizzled;
-//   Vᵀ tile [D][BN keys]      transposed in registers on the way in (each thread holds a 4-key x 8-feature
-//                             block), because P·V contracts over keys and an MFMA lane needs 8 consecutive
-//                             values of the contraction index.
+// Key/value tiles of 64 keys go HBM -> LDS directly (buffer loads with the LDS flag, double buffered, one barrier
+// per tile):
+//   K tile [64 keys][D]   row-major, 16-byte chunks XOR-swizzled;
+//   V tile [64 keys][D]   row-major, 64-byte windows XOR-swizzled; P·V contracts over keys and an MFMA lane needs 8
+//                         consecutive values of the contraction index, which the transposing LDS read
+//                         (ds_read_b64_tr_b16) delivers from this layout.
 // Scores are computed TRANSPOSED: Sᵀ = K·Qᵀ with K on the MFMA "A" side, so a lane ends up with the scores of
-// ONE query row (lane % 32) against BN/2 keys.  Row max and row sum are then lane-local loops plus a single
+// ONE query row (lane % 32) against 32 keys.  Row max and row sum are then lane-local loops plus a single
 // exchange with lane ^ 32, and the fp32 score registers, once exponentiated and packed to 16 bit, already are
-// the MFMA "B" operand of Oᵀ = Vᵀ·Pᵀ — P never touches LDS.  Vᵀ rows are stored through rowperm16, so each lane
+// the MFMA "B" operand of Oᵀ = Vᵀ·Pᵀ — P never touches LDS.  Vᵀ rows are fed through rowperm16, so each lane
 // finishes with 16 consecutive output features of its query row and writes them as two 16-byte stores.
 #include <math.h>
 
@@ -56,27 +57,42 @@ __device__ __forceinline__ float scale_mask(float mv, float clamp) {
     return fmaxf(mv * kLog2eA, kClampFloor);
 }
 
-template <typename T, int D, int BN, int SUB, int WPE, int MASK_MODE, bool CAUSAL>
-__global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnParams p) {
+// ----------------------------------------------------------------------------------------------------
+// Streaming MFMA kernel: 64-key tiles staged by buffer loads that write LDS directly (no register staging, no
+// transposition pass): K swizzled as above, V row-major with its 64-byte windows swizzled, read back through the
+// transposing LDS load.  A wave issues one instruction every few cycles whatever its kind, so the loop is kept
+// free of bookkeeping: key tiles that need no masking at all ("clean") run first through a branch-free body that
+// is unrolled over the two LDS stages; the others (ragged last tile, masked, causal diagonal) follow in a general
+// body.  The order of key tiles does not matter to the online softmax.
+// ----------------------------------------------------------------------------------------------------
+template <bool B>
+struct BoolC {
+    static constexpr bool value = B;
+};
+template <int I>
+struct IntC {
+    static constexpr int value = I;
+};
+
+template <typename T, int D, int WPE, int MASK_MODE, bool CAUSAL>
+__global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnParams p) {
     typedef typename Vec8<T>::type vec8;
-    constexpr int BM = 128;
-    constexpr int KROW = D * 2, VROW = BN * 2;           // LDS row bytes of the K and Vᵀ tiles
-    constexpr int K_BYTES = BN * KROW, V_BYTES = D * VROW;
-    constexpr int STAGE = K_BYTES + V_BYTES + BN * 4;    // + per-key additive term (fp32)
-    constexpr int NBS = SUB / 32, DB = D / 32, KS = D / 16;
-    constexpr int DC = D / 8;                            // 16-byte chunks per K/V row
-    constexpr int KI = BN * DC / 256;                    // K chunks per thread per tile
-    constexpr int VKEYS = BN * DC / 256;                 // every thread transposes a VKEYS-key x 8-feature block of V
-    static_assert(VKEYS == 4 || VKEYS == 2, "V blocks of 4 or 2 keys");
-    static_assert(BN * DC % 256 == 0, "K chunks must split evenly over the threads");
+    typedef __attribute__((address_space(3))) void lds_void;
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    constexpr int BM = 128, BN = 64;
+    constexpr int KROW = D * 2, VP = D * 2;               // LDS row bytes of the K tile [key][D] and V tile [key][D]
+    constexpr int K_BYTES = BN * KROW, V_BYTES = BN * VP;
+    constexpr int STAGE = K_BYTES + V_BYTES + BN * 4;     // + per-key additive term (fp32)
+    constexpr int NBS = BN / 32, DB = D / 32, KS = D / 16;
+    constexpr int DC = D / 8;                             // 16-byte chunks per K/V row
+    constexpr int KI = BN * DC / 256;                     // 1 KB loads per wave for each of K and V
 
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
     __shared__ int tile_list[kMaxTiles];
-    __shared__ int tile_cls[kMaxTiles];
-    __shared__ int n_listed;
+    __shared__ int list_counts[2];
 
-    // ---- which (batch, head, query tile): ids are dealt round-robin over 8 XCDs; keep all query tiles of a
-    // head on one XCD and adjacent in time so K/V re-reads hit that XCD's L2.
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int bh = (slot / p.nq_tiles) * 8 + xcd;
     int qt = slot % p.nq_tiles;
@@ -84,9 +100,10 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
     if (CAUSAL) qt = p.nq_tiles - 1 - qt;  // longest rows first
     const int b = bh / p.H, h = bh % p.H;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 31, lh = lane >> 5;
-    const int m_wave0 = qt * BM + wave * 32;
+    const int q0 = qt * BM;
+    const int m_wave0 = q0 + wave * 32;
     const int my_m = m_wave0 + lr;
     const int M = p.M, N = p.N;
 
@@ -96,14 +113,17 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
     T *op = static_cast<T *>(p.o) + b * p.os[0] + h * p.os[1];
     const int64_t mask_base = (MASK_MODE != MASK_NONE) ? b * p.ms[0] + h * p.ms[1] : 0;
 
-    // ---- key range and tile list
-    int n_end = N;
-    if (CAUSAL) n_end = min(N, qt * BM + BM);
+    // ---- key tiles: [0, n_clean) of the processing order need no masking, [n_clean, nt) take the general body
+    const int n_end = CAUSAL ? min(N, q0 + BM) : N;
     const int nt_all = (n_end + BN - 1) / BN;
-
-    if (MASK_MODE == MASK_VECTOR && !CAUSAL && nt_all <= kMaxTiles) {
-        // classify key tiles from the per-key mask: 0 = all zero (no add needed), 1 = general,
-        // 2 = every entry so negative that the tile contributes exactly 0 (skippable if some other tile is not).
+    constexpr bool MAY_LIST = (MASK_MODE == MASK_VECTOR && !CAUSAL);
+    const bool use_list = MAY_LIST && nt_all <= kMaxTiles;
+    int nt = nt_all, n_clean = 0;
+    if (MASK_MODE == MASK_NONE) n_clean = CAUSAL ? min(N / BN, q0 / BN) : N / BN;
+    if (use_list) {
+        // classify from the per-key mask: 0 = all zero and full, 1 = general, 2 = so negative that the tile
+        // contributes exactly 0 (dropped if any other tile is kept)
+        int *cls = reinterpret_cast<int *>(smem);
         for (int t = wave; t < nt_all; t += 4) {
             bool nonzero = false, normal = false;
             for (int n = t * BN + lane; n < min(N, t * BN + BN); n += 64) {
@@ -112,26 +132,30 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                 normal |= (mv > kNegBig);
             }
             const bool any_nonzero = __ballot(nonzero) != 0, any_normal = __ballot(normal) != 0;
-            if (lane == 0) tile_cls[t] = !any_normal ? 2 : (any_nonzero ? 1 : 0);
+            if (lane == 0) cls[t] = !any_normal ? 2 : ((any_nonzero || t * BN + BN > N) ? 1 : 0);
         }
         __syncthreads();
         if (tid == 0) {
             int cnt = 0;
             for (int t = 0; t < nt_all; ++t)
-                if (tile_cls[t] != 2) tile_list[cnt++] = t;
-            if (cnt == 0) {  // every key masked: keep them all, the result is the (finite) uniform average
-                for (int t = 0; t < nt_all; ++t) {
-                    tile_list[t] = t;
-                    tile_cls[t] = 1;
-                }
+                if (cls[t] == 0) tile_list[cnt++] = t;
+            const int nc = cnt;
+            for (int t = 0; t < nt_all; ++t)
+                if (cls[t] == 1) tile_list[cnt++] = t;
+            if (cnt == 0) {  // every key masked: keep all tiles, the result is the (finite) uniform average
+                for (int t = 0; t < nt_all; ++t) tile_list[t] = t;
                 cnt = nt_all;
             }
-            n_listed = cnt;
+            list_counts[0] = nc;
+            list_counts[1] = cnt;
         }
         __syncthreads();
+        n_clean = __builtin_amdgcn_readfirstlane(list_counts[0]);
+        nt = __builtin_amdgcn_readfirstlane(list_counts[1]);
+        __syncthreads();  // the class table shares LDS with the first stage
     }
-    const bool use_list = (MASK_MODE == MASK_VECTOR && !CAUSAL && nt_all <= kMaxTiles);
-    const int nt = use_list ? __builtin_amdgcn_readfirstlane(n_listed) : nt_all;
+    n_clean &= ~1;  // the clean body is unrolled over both stages; an odd leftover goes through the general body
+    auto tile_of = [&](int idx) -> int { return use_list ? __builtin_amdgcn_readfirstlane(tile_list[idx]) : idx; };
 
     // ---- Q fragments (MFMA "B" side: lane holds its query row, 8 consecutive features per k-step)
     vec8 qf[KS];
@@ -141,77 +165,52 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
         for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const vec8 *>(qrow + s * 16);
     }
 
-    // ---- global -> register staging of one K/V tile.  Buffer loads: a uniform resource covering this head's
-    // K (V) rows, a loop-invariant 32-bit thread offset and the tile's first row as a scalar offset.  Rows past
-    // the last key lie beyond the resource's extent and read as zero in hardware.
-    const int v_dc = tid % DC, v_ng = tid / DC;  // this thread's VKEYS-key x 8-feature block of V
-    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<T *>(kp), 0, (int)((((int64_t)N - 1) * p.ks[2] + D) * 2), 0x00020000);
-    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<T *>(vp), 0, (int)((((int64_t)N - 1) * p.vs[2] + D) * 2), 0x00020000);
-    uint32_t kg[KI], vg[VKEYS];  // byte offsets of this thread's chunks inside a tile
-    int kl[KI], vl[8];       // LDS byte offsets inside a stage
+    // ---- staging: the i-th load of a wave fills the 1 KB of 16-byte chunks [256 i + 64 wave, +64) of a tile;
+    // every lane fetches the chunk of global memory that belongs at its LDS position under the tile's swizzle
+    // (V: the 64-byte window of a row is XORed with low key bits so that a transposing read of 4 consecutive keys
+    // x 32 features touches every bank once).  Rows past the last key lie beyond the extent of the buffer
+    // resource and arrive as zeros.
+    uint32_t kdma[KI], vdma[KI];
 #pragma unroll
     for (int i = 0; i < KI; ++i) {
         const int qd = tid + 256 * i;
-        const int row = qd / DC, c = qd % DC;
-        kg[i] = (uint32_t)(((int64_t)row * p.ks[2] + c * 8) * 2);
-        kl[i] = swz_offset<KROW>(row, c);
+        const int row = qd / DC, cs = qd % DC;
+        kdma[i] = (uint32_t)(((int64_t)row * p.ks[2] + swz_chunk<KROW>(row, cs) * 8) * 2);
+        const int vsw = (D == 64) ? ((row >> 1) & 1) : (row & 3);
+        vdma[i] = (uint32_t)(((int64_t)row * p.vs[2] + (cs ^ (vsw << 2)) * 8) * 2);
     }
-#pragma unroll
-    for (int r = 0; r < VKEYS; ++r) vg[r] = (uint32_t)(((int64_t)(v_ng * VKEYS + r) * p.vs[2] + v_dc * 8) * 2);
-    {
-        // Vᵀ: feature d lives in LDS row (d & ~31) + inverse_rowperm16(d & 31); the VKEYS consecutive keys of this
-        // thread stay adjacent at position pos of that row, where pos swaps bits 2 and 3 of the key index (see
-        // header comment).
-        const int nloc = v_ng * VKEYS;
-        const int pos = (nloc & ~12) | ((nloc & 4) << 1) | ((nloc & 8) >> 1);
-        const int chunk = pos >> 3, within = (pos & 7) * 2;  // 16-byte chunk, byte offset inside it
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int d = v_dc * 8 + e;
-            const int x = d & 31;
-            const int row = (d & ~31) + 8 * ((x >> 2) & 3) + 4 * (x >> 4) + (x & 3);
-            vl[e] = K_BYTES + swz_offset<VROW>(row, chunk) + within;
-        }
-    }
-    vec8 kst[KI], vst[VKEYS];
-    float bias_st = 0.0f;
-    auto gload = [&](int tile) {
-        const int n0 = tile * BN;
-        const int k_soff = (int)((int64_t)n0 * p.ks[2] * 2), v_soff = (int)((int64_t)n0 * p.vs[2] * 2);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
+    const uint32_t dma_base = lds_base + wave * 1024;
+    const uint64_t kaddr = (uint64_t)(uintptr_t)kp, vaddr = (uint64_t)(uintptr_t)vp;
+    const u32x4 krsrc = {(uint32_t)kaddr, (uint32_t)(kaddr >> 32) & 0xFFFFu,
+                         (uint32_t)((((int64_t)N - 1) * p.ks[2] + D) * 2), 0x00020000u};
+    const u32x4 vrsrc = {(uint32_t)vaddr, (uint32_t)(vaddr >> 32) & 0xFFFFu,
+                         (uint32_t)((((int64_t)N - 1) * p.vs[2] + D) * 2), 0x00020000u};
+    const int k_tile_bytes = (int)((int64_t)BN * p.ks[2] * 2), v_tile_bytes = (int)((int64_t)BN * p.vs[2] * 2);
+    // Inline assembly on purpose: the compiler, seeing LDS written by a load, would make every later LDS read
+    // wait for the vector-memory counter, i.e. for the prefetch itself.  The explicit wait before the barrier
+    // that publishes the stage is the one that matters.
+    auto dma = [&](int tile, int stage) {
+        const int k_soff = tile * k_tile_bytes, v_soff = tile * v_tile_bytes;
+        const uint32_t sb = dma_base + stage * STAGE;
 #pragma unroll
         for (int i = 0; i < KI; ++i)
-            kst[i] = __builtin_bit_cast(vec8, __builtin_amdgcn_raw_buffer_load_b128(krsrc, kg[i], k_soff, 0));
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :: "s"(sb + i * 4096), "v"(kdma[i]), "s"(krsrc), "s"(k_soff) : "memory", "m0");
 #pragma unroll
-        for (int r = 0; r < VKEYS; ++r)
-            vst[r] = __builtin_bit_cast(vec8, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vg[r], v_soff, 0));
-        if (MASK_MODE == MASK_VECTOR || n0 + BN > N) {
-            if (tid < BN) {
-                const int n = n0 + tid;
-                float bv = 0.0f;
-                if (MASK_MODE == MASK_VECTOR)
-                    bv = scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_base + min(n, N - 1) * p.ms[3]), p.clamp);
-                if (n >= N) bv = -INFINITY;
-                bias_st = bv;
-            }
-        }
+        for (int i = 0; i < KI; ++i)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :: "s"(sb + K_BYTES + i * 4096), "v"(vdma[i]), "s"(vrsrc), "s"(v_soff) : "memory", "m0");
     };
-    auto lstore = [&](int stage) {
-        unsigned char *sb = smem + stage * STAGE;
-#pragma unroll
-        for (int i = 0; i < KI; ++i) *reinterpret_cast<vec8 *>(sb + kl[i]) = kst[i];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            if (VKEYS == 4) {
-                T quad[4] = {vst[0][e], vst[1][e], vst[VKEYS - 2][e], vst[VKEYS - 1][e]};
-                *reinterpret_cast<uint64_t *>(sb + vl[e]) = *reinterpret_cast<const uint64_t *>(quad);
-            } else {
-                T pair[2] = {vst[0][e], vst[1][e]};
-                *reinterpret_cast<uint32_t *>(sb + vl[e]) = *reinterpret_cast<const uint32_t *>(pair);
-            }
-        }
-        if (tid < BN) *reinterpret_cast<float *>(sb + K_BYTES + V_BYTES + tid * 4) = bias_st;
+    // per-key additive term of a general tile (mask value in the log2 domain, -inf past the last key); thread tid
+    // < 64 owns key tid of the tile
+    auto key_bias = [&](int tile) -> float {
+        const int n = tile * BN + tid;
+        float bv = 0.0f;
+        if (MASK_MODE == MASK_VECTOR)
+            bv = scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_base + min(n, N - 1) * p.ms[3]), p.clamp);
+        if (n >= N) bv = -INFINITY;
+        return bv;
     };
 
     // ---- running state of this lane's query row
@@ -221,56 +220,41 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
     for (int d = 0; d < DB; ++d)
 #pragma unroll
         for (int v = 0; v < 16; ++v) o_acc[d][v] = 0.0f;
-
     const float c = p.scale_log2;
 
-    // LDS byte offsets of this lane's operand fragments inside a sub-tile, minus the 32-row block term
-    // (a compile-time constant that folds into the instruction offset).  The swizzle phase of a row depends
-    // only on its low bits, so it is the same in every 32-row block.
-    int k_off[KS], v_off[SUB / 16];
+    // LDS byte offsets of this lane's operand fragments.  K: row lr of a 32-key block, chunk 2 ks + lh.  V: in each
+    // group of 16 lanes, lane i hands the transposing read the address of 4 consecutive features of key (i / 4)
+    // and receives feature column i of the 4-key x 16-feature block, i.e. 4 consecutive keys of one feature; the
+    // 16 lanes of a group are MFMA rows 16 (group % 2) + 0..15, whose features (through rowperm16) are four runs
+    // of 4.
+    int k_off[KS], vt_off[DB];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) k_off[ks] = swz_offset<KROW>(lr, 2 * ks + lh);
+    {
+        const int i16 = lane & 15, g16 = lane >> 4;
+        const int kq = i16 >> 2;
+        const int fs = rowperm16(16 * (g16 & 1) + 4 * (i16 & 3));
+        const int vsw = (D == 64) ? (kq >> 1) : kq;
 #pragma unroll
-    for (int ps = 0; ps < SUB / 16; ++ps) v_off[ps] = swz_offset<VROW>(lr, 2 * ps + lh);
+        for (int d = 0; d < DB; ++d) vt_off[d] = K_BYTES + (4 * lh + kq) * VP + ((d ^ vsw) * 64) + fs * 2;
+    }
     const int64_t mask_row = mask_base + (int64_t)min(my_m, M - 1) * (MASK_MODE == MASK_MATRIX ? p.ms[2] : 0);
 
-    if (nt > 0) {
-        gload(use_list ? __builtin_amdgcn_readfirstlane(tile_list[0]) : 0);
-        lstore(0);
-    }
-    // Every load issued so far (Q fragments included) has to have landed before the loop: otherwise the
-    // compiler must assume they may still be in flight at the first MFMA of each iteration and waits there for
-    // the vector-memory counter to drain, which also drains the prefetch of the next tile issued just before.
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();
-
-    for (int it = 0; it < nt; ++it) {
-        // tile indices come from LDS: tell the compiler they are wave-uniform, otherwise every buffer load that
-        // takes them as a scalar offset is wrapped in a waterfall loop
-        const int tile = use_list ? __builtin_amdgcn_readfirstlane(tile_list[it]) : it;
+    // one key tile: prefetch the next one into the other stage, scores, online softmax, P·V, publish
+    auto tile_step = [&](auto general_c, auto stage_c, int idx) {
+        constexpr bool GENERAL = decltype(general_c)::value;
+        constexpr int ST = decltype(stage_c)::value;
+        const int tile = tile_of(idx);
         const int n0 = tile * BN;
-        if (it + 1 < nt) gload(use_list ? __builtin_amdgcn_readfirstlane(tile_list[it + 1]) : it + 1);
+        const int tile_next = tile_of(min(idx + 1, nt - 1));
+        dma(tile_next, ST ^ 1);
+        float bias_next = 0.0f;
+        if (GENERAL && tid < BN) bias_next = key_bias(tile_next);
 
-        const unsigned char *kb = smem + (it & 1) * STAGE;
-        const unsigned char *vb = kb + K_BYTES;
-        const float *colbias = reinterpret_cast<const float *>(kb + K_BYTES + V_BYTES);
-
-        // The tile is consumed in sub-tiles of SUB keys, each a complete online-softmax step, which keeps
-        // the live score registers at SUB/2 per lane.
-        const bool tile_general = (MASK_MODE == MASK_MATRIX) || (n0 + BN > N) ||
-                                  (MASK_MODE == MASK_VECTOR && (use_list ? (__builtin_amdgcn_readfirstlane(tile_cls[tile]) != 0) : true));
-#pragma nounroll
-        for (int sub = 0; sub < BN / SUB; ++sub) {
-            const int ns0 = n0 + sub * SUB;  // first key of the sub-tile
-            // a wave whose 32 rows all lie above this causal sub-tile has nothing to do in it
-            if (CAUSAL && ns0 > m_wave0 + 31) break;
-            if (ns0 >= N) break;
-            const unsigned char *ksub = kb + sub * SUB * KROW;
-            // along a Vᵀ row the sub-tile is SUB/8 chunks further; under the XOR swizzle that is an XOR too
-            const int vsub_xor = sub * (SUB / 8) * 16;
-
-            // ---- Sᵀ = K · Qᵀ.  MFMA phases run at raised wave priority: a wave that is ready to feed the matrix
-            // pipe goes first, the other waves of the SIMD fill the gaps with their softmax VALU work.
+        const unsigned char *sb = smem + ST * STAGE;
+        // a wave whose 32 rows all lie above a causal tile has nothing to compute in it
+        if (!(GENERAL && CAUSAL && n0 > m_wave0 + 31)) {
+            // ---- Sᵀ = K · Qᵀ
             f32x16 s_acc[NBS];
             __builtin_amdgcn_s_setprio(2);
 #pragma unroll
@@ -279,22 +263,21 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                 for (int v = 0; v < 16; ++v) s_acc[nb][v] = 0.0f;
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    const vec8 kf = *reinterpret_cast<const vec8 *>(ksub + nb * 32 * KROW + k_off[ks]);
+                    const vec8 kf = *reinterpret_cast<const vec8 *>(sb + nb * 32 * KROW + k_off[ks]);
                     s_acc[nb] = mfma32(kf, qf[ks], s_acc[nb]);
                 }
             }
-
             __builtin_amdgcn_s_setprio(0);
 
-            // ---- online softmax on this lane's row; key of s_acc[nb][v] is ns0 + 32 nb + 8 (v/4) + 4 lh + (v%4)
-            const bool general = tile_general || (CAUSAL && (ns0 + SUB - 1 > m_wave0));
+            // ---- online softmax on this lane's row; key of s_acc[nb][v] is n0 + 32 nb + 8 (v/4) + 4 lh + (v%4)
             float mx = -INFINITY;
-            if (general) {
+            if (GENERAL) {
+                const float *colbias = reinterpret_cast<const float *>(sb + K_BYTES + V_BYTES);
 #pragma unroll
                 for (int nb = 0; nb < NBS; ++nb) {
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
-                        const int nl = sub * SUB + nb * 32 + g * 8 + lh * 4;  // key index inside the tile
+                        const int nl = nb * 32 + g * 8 + lh * 4;  // key index inside the tile
                         const f32x4 cb = *reinterpret_cast<const f32x4 *>(colbias + nl);
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
@@ -314,13 +297,13 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                 for (int nb = 0; nb < NBS; ++nb)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[nb][v]);
-                mx *= c;  // c > 0 on this path (checked by the host)
+                mx *= c;  // c > 0 (checked by the host)
             }
             mx = halves32_max(mx);  // the other 16-key half of every 32-key block lives in lane ^ 32
-            // m_i is the exponent REFERENCE of this row, not necessarily its running maximum: it is only moved (and
-            // the accumulator and row sum rescaled) when the new maximum exceeds it by more than 2^8, so probabilities
-            // stay <= 256 — exact in fp32 and well inside the 16-bit range — and after the first tiles the rescale
-            // almost never runs.  The final O / l is independent of the reference.
+            // m_i is the exponent REFERENCE of this row, not necessarily its running maximum: it only moves (and the
+            // accumulator and row sum are rescaled) when the new maximum exceeds it by more than 2^8, so
+            // probabilities stay <= 256 — exact in fp32, well inside the 16-bit range — and after the first tiles
+            // the rescale almost never runs.  The final O / l is independent of the reference.
             if (__builtin_amdgcn_ballot_w64(mx > m_i + kRescaleThreshold) != 0) {
                 const float m_new = fmaxf(m_i, mx);
                 const float alpha = __builtin_amdgcn_exp2f(m_i - ((m_new == -INFINITY) ? 0.0f : m_new));
@@ -332,25 +315,18 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                 m_i = m_new;
             }
             const float m_use = (m_i == -INFINITY) ? 0.0f : m_i;
-            // exponentiate in place; the row sum is taken below from the ROUNDED probabilities (two per
-            // v_dot2c), i.e. from exactly the values that enter P·V
-            if (general) {
 #pragma unroll
-                for (int nb = 0; nb < NBS; ++nb)
+            for (int nb = 0; nb < NBS; ++nb)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s_acc[nb][v] = __builtin_amdgcn_exp2f(s_acc[nb][v] - m_use);
-            } else {
-#pragma unroll
-                for (int nb = 0; nb < NBS; ++nb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) s_acc[nb][v] = __builtin_amdgcn_exp2f(s_acc[nb][v] * c - m_use);
-            }
-            float rs = 0.0f;
+                for (int v = 0; v < 16; ++v)
+                    s_acc[nb][v] = __builtin_amdgcn_exp2f(GENERAL ? s_acc[nb][v] - m_use : s_acc[nb][v] * c - m_use);
 
-            // ---- Oᵀ += Vᵀ · Pᵀ
+            // ---- Oᵀ += Vᵀ · Pᵀ; the row sum is taken from the ROUNDED probabilities (two per v_dot2c), i.e. from
+            // exactly the values that enter the product
+            float rs = 0.0f;
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-            for (int ps = 0; ps < SUB / 16; ++ps) {
+            for (int ps = 0; ps < BN / 16; ++ps) {
                 const int nb = ps >> 1, half8 = (ps & 1) * 8;
                 u32x4 pk;
 #pragma unroll
@@ -361,16 +337,45 @@ __global__ void __launch_bounds__(256, WPE) attention_mfma_kernel(const AttnPara
                 const vec8 pf = __builtin_bit_cast(vec8, pk);
 #pragma unroll
                 for (int d = 0; d < DB; ++d) {
-                    const vec8 vf = *reinterpret_cast<const vec8 *>(vb + d * 32 * VROW + (v_off[ps] ^ vsub_xor));
-                    o_acc[d] = mfma32(vf, pf, o_acc[d]);
+                    const unsigned char *va = sb + 16 * ps * VP + vt_off[d];
+                    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)va);
+                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(va + 8 * VP));
+                    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    o_acc[d] = mfma32(__builtin_bit_cast(vec8, both), pf, o_acc[d]);
                 }
             }
             __builtin_amdgcn_s_setprio(0);
             l_i += rs;
         }
 
-        if (it + 1 < nt) lstore((it + 1) & 1);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the next tile is in LDS
+        if (GENERAL && tid < BN)
+            *reinterpret_cast<float *>(smem + (ST ^ 1) * STAGE + K_BYTES + V_BYTES + tid * 4) = bias_next;
         __syncthreads();
+    };
+
+    if (nt > 0) {
+        const int t0 = tile_of(0);
+        dma(t0, 0);
+        if (n_clean == 0 && tid < BN) *reinterpret_cast<float *>(smem + K_BYTES + V_BYTES + tid * 4) = key_bias(t0);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far (Q fragments included) has landed
+    __syncthreads();
+
+    int idx = 0;
+    for (; idx < n_clean; idx += 2) {
+        tile_step(BoolC<false>(), IntC<0>(), idx);
+        tile_step(BoolC<false>(), IntC<1>(), idx + 1);
+    }
+    if (idx < nt) {
+        if (n_clean > 0) {  // the additive terms of the first general tile (it sits in stage 0: n_clean is even)
+            if (tid < BN) *reinterpret_cast<float *>(smem + K_BYTES + V_BYTES + tid * 4) = key_bias(tile_of(idx));
+            __syncthreads();
+        }
+        for (; idx < nt; idx += 2) {
+            tile_step(BoolC<true>(), IntC<0>(), idx);
+            if (idx + 1 < nt) tile_step(BoolC<true>(), IntC<1>(), idx + 1);
+        }
     }
 
     // ---- normalise and store: lane holds features 32 d + 16 lh + (0..15) of row my_m
@@ -459,11 +464,11 @@ __global__ void __launch_bounds__(64) attention_scalar_kernel(const AttnParams p
 // ----------------------------------------------------------------------------------------------------
 // host dispatch
 // ----------------------------------------------------------------------------------------------------
-template <typename T, int D, int BN, int SUB, int WPE>
-static void launch_mfma(const AttnParams &p, int mask_mode, bool causal, hipStream_t st) {
+template <typename T, int D, int WPE>
+static void launch_stream(const AttnParams &p, int mask_mode, bool causal, hipStream_t st) {
     const int bh_padded = ((p.B * p.H + 7) / 8) * 8;
     dim3 grid((unsigned)(bh_padded * p.nq_tiles)), block(256);
-#define KERNL_ATTN_LAUNCH(MM, C) hipLaunchKernelGGL((attention_mfma_kernel<T, D, BN, SUB, WPE, MM, C>), grid, block, 0, st, p)
+#define KERNL_ATTN_LAUNCH(MM, C) hipLaunchKernelGGL((attention_stream_kernel<T, D, WPE, MM, C>), grid, block, 0, st, p)
     if (mask_mode == MASK_NONE) {
         if (causal) KERNL_ATTN_LAUNCH(MASK_NONE, true);
         else KERNL_ATTN_LAUNCH(MASK_NONE, false);
@@ -478,7 +483,7 @@ static void launch_mfma(const AttnParams &p, int mask_mode, bool causal, hipStre
 }
 
 int g_attention_force_scalar = 0;  // test hook: route everything through the scalar kernel
-int g_attention_variant = 0;       // tuning hook: tile shape of the head-size-64 MFMA kernel
+int g_attention_variant = 0;       // tuning hook: register budget (waves per SIMD) of the head-size-64 MFMA kernel
 
 }  // namespace kernl
 
@@ -550,20 +555,19 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
                          k_strides[2] > 0 && v_strides[2] > 0 &&  // one head's K / V extent must fit 31-bit byte offsets
                          (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30);
     if (mfma_ok) {
+        // head size 64: 115 VGPRs without a matrix mask (up to 4 waves per SIMD); the matrix-mask body needs the
+        // register budget of 2 waves per SIMD.  Head size 128: 2 waves per SIMD.
+        int wpe = (D == 64 && mask_mode != MASK_MATRIX) ? 3 : 2;
+        if (D == 64 && g_attention_variant == 1) wpe = 3;
+        if (D == 64 && g_attention_variant == 2) wpe = 2;
         if (dtype == KERNL_F16) {
-            if (D == 64) {
-                // measured on config 1: 64-key tiles at 3 waves/SIMD win without causal masking (finer skipping of
-                // padded key tiles, more waves to interleave), 128-key tiles at 2 waves/SIMD win with it
-                int variant = g_attention_variant;
-                if (variant == 0) variant = (causal || mask_mode == MASK_MATRIX) ? 3 : 1;
-                if (variant == 1) launch_mfma<f16, 64, 64, 64, 3>(p, mask_mode, causal, st);
-                else if (variant == 2) launch_mfma<f16, 64, 64, 64, 2>(p, mask_mode, causal, st);
-                else launch_mfma<f16, 64, 128, 64, 2>(p, mask_mode, causal, st);
-            }
-            else launch_mfma<f16, 128, 64, 32, 2>(p, mask_mode, causal, st);
+            if (D == 64 && wpe == 3) launch_stream<f16, 64, 3>(p, mask_mode, causal, st);
+            else if (D == 64) launch_stream<f16, 64, 2>(p, mask_mode, causal, st);
+            else launch_stream<f16, 128, 2>(p, mask_mode, causal, st);
         } else {
-            if (D == 64) launch_mfma<bf16, 64, 128, 64, 2>(p, mask_mode, causal, st);
-            else launch_mfma<bf16, 128, 64, 32, 2>(p, mask_mode, causal, st);
+            if (D == 64 && wpe == 3) launch_stream<bf16, 64, 3>(p, mask_mode, causal, st);
+            else if (D == 64) launch_stream<bf16, 64, 2>(p, mask_mode, causal, st);
+            else launch_stream<bf16, 128, 2>(p, mask_mode, causal, st);
         }
         return check_launch("attention (mfma)");
     }
