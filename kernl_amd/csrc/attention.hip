@@ -20,6 +20,8 @@
 // finishes with 16 consecutive output features of its query row and writes them as two 16-byte stores.
 #include <math.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace kernl {
@@ -27,7 +29,6 @@ namespace kernl {
 static constexpr float kLog2eA = 1.4426950408889634f;
 static constexpr float kNegBig = -1.0e30f;            // anything below: exp2(x - rowmax) is exactly 0
 static constexpr float kClampFloor = -1.7014118e38f;  // scaled mask values are kept finite (-FLT_MAX / 2)
-static constexpr int kMaxTiles = 256;
 static constexpr float kRescaleThreshold = 8.0f;  // log2 units
 
 enum { MASK_NONE = 0, MASK_VECTOR = 1, MASK_MATRIX = 2 };
@@ -90,8 +91,6 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     constexpr int KI = BN * DC / 256;                     // 1 KB loads per wave for each of K and V
 
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
-    __shared__ int tile_list[kMaxTiles];
-    __shared__ int list_counts[2];
 
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int bh = (slot / p.nq_tiles) * 8 + xcd;
@@ -112,50 +111,6 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     const T *vp = static_cast<const T *>(p.v) + b * p.vs[0] + h * p.vs[1];
     T *op = static_cast<T *>(p.o) + b * p.os[0] + h * p.os[1];
     const int64_t mask_base = (MASK_MODE != MASK_NONE) ? b * p.ms[0] + h * p.ms[1] : 0;
-
-    // ---- key tiles: [0, n_clean) of the processing order need no masking, [n_clean, nt) take the general body
-    const int n_end = CAUSAL ? min(N, q0 + BM) : N;
-    const int nt_all = (n_end + BN - 1) / BN;
-    constexpr bool MAY_LIST = (MASK_MODE == MASK_VECTOR && !CAUSAL);
-    const bool use_list = MAY_LIST && nt_all <= kMaxTiles;
-    int nt = nt_all, n_clean = 0;
-    if (MASK_MODE == MASK_NONE) n_clean = CAUSAL ? min(N / BN, q0 / BN) : N / BN;
-    if (use_list) {
-        // classify from the per-key mask: 0 = all zero and full, 1 = general, 2 = so negative that the tile
-        // contributes exactly 0 (dropped if any other tile is kept)
-        int *cls = reinterpret_cast<int *>(smem);
-        for (int t = wave; t < nt_all; t += 4) {
-            bool nonzero = false, normal = false;
-            for (int n = t * BN + lane; n < min(N, t * BN + BN); n += 64) {
-                const float mv = scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_base + n * p.ms[3]), p.clamp);
-                nonzero |= (mv != 0.0f);
-                normal |= (mv > kNegBig);
-            }
-            const bool any_nonzero = __ballot(nonzero) != 0, any_normal = __ballot(normal) != 0;
-            if (lane == 0) cls[t] = !any_normal ? 2 : ((any_nonzero || t * BN + BN > N) ? 1 : 0);
-        }
-        __syncthreads();
-        if (tid == 0) {
-            int cnt = 0;
-            for (int t = 0; t < nt_all; ++t)
-                if (cls[t] == 0) tile_list[cnt++] = t;
-            const int nc = cnt;
-            for (int t = 0; t < nt_all; ++t)
-                if (cls[t] == 1) tile_list[cnt++] = t;
-            if (cnt == 0) {  // every key masked: keep all tiles, the result is the (finite) uniform average
-                for (int t = 0; t < nt_all; ++t) tile_list[t] = t;
-                cnt = nt_all;
-            }
-            list_counts[0] = nc;
-            list_counts[1] = cnt;
-        }
-        __syncthreads();
-        n_clean = __builtin_amdgcn_readfirstlane(list_counts[0]);
-        nt = __builtin_amdgcn_readfirstlane(list_counts[1]);
-        __syncthreads();  // the class table shares LDS with the first stage
-    }
-    n_clean &= ~1;  // the clean body is unrolled over both stages; an odd leftover goes through the general body
-    auto tile_of = [&](int idx) -> int { return use_list ? __builtin_amdgcn_readfirstlane(tile_list[idx]) : idx; };
 
     // ---- Q fragments (MFMA "B" side: lane holds its query row, 8 consecutive features per k-step)
     vec8 qf[KS];
@@ -213,6 +168,132 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         return bv;
     };
 
+    // ---- key tiles: [0, n_clean) of the processing order need no masking, [n_clean, nt) take the general body
+    const int n_end = CAUSAL ? min(N, q0 + BM) : N;
+    const int nt_all = (n_end + BN - 1) / BN;
+    constexpr bool MAY_LIST = (MASK_MODE == MASK_VECTOR && !CAUSAL);
+    const bool use_list = MAY_LIST && nt_all <= 64;
+    int nt = nt_all, n_clean = 0;
+    if (MASK_MODE == MASK_NONE) n_clean = CAUSAL ? min(N / BN, q0 / BN) : N / BN;
+    // the first tile is fetched before the mask has been looked at: tile 0 almost always comes first
+    if (nt_all > 0) dma(0, 0);
+    // With a per-key mask every wave classifies all key tiles by itself (the mask row is a few KB, and this way no
+    // barrier or LDS table is needed): bit t of clean_bits = tile t is all zero and full, of gen_bits = it needs
+    // the general body; tiles in neither set are so negative everywhere that they contribute exactly 0 and are
+    // dropped.  Both sets are wave-uniform scalars; tiles are taken from them lowest index first.
+    uint64_t clean_bits = 0, gen_bits = 0;
+    if (use_list) {
+        // lane l looks at key 64 t + l of tile t; 32-bit offsets (the host checks that a mask row fits them)
+        auto classify = [&](auto *mrow) {
+            const int ms3 = (int)p.ms[3];
+            const int lane_off = lane * ms3, tile_step_off = BN * ms3;
+            for (int t0 = 0; t0 < nt_all; t0 += 8) {
+                float mv[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    mv[j] = 0.0f;
+                    if (t0 + j < nt_all && (t0 + j) * BN + lane < N) mv[j] = (float)mrow[lane_off + (t0 + j) * tile_step_off];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int t = t0 + j;
+                    if (t < nt_all) {
+                        const bool valid = t * BN + lane < N;
+                        const float sm = scale_mask(mv[j], p.clamp);
+                        const bool any_nonzero = __ballot(valid && (sm != 0.0f)) != 0;
+                        const bool any_normal = __ballot(valid && (sm > kNegBig)) != 0;
+                        if (any_normal) {
+                            if (any_nonzero || t * BN + BN > N) gen_bits |= 1ull << t;
+                            else clean_bits |= 1ull << t;
+                        }
+                    }
+                }
+            }
+        };
+        // Contiguous, 16-byte aligned mask rows take a shorter route: a lane loads 4 consecutive keys, so 16 lanes
+        // cover a tile and one load covers 4 tiles; lanes 0..3 then each judge one of those tiles from the two
+        // wave-wide ballots.
+        auto classify4 = [&](auto *mrow) {
+            typedef typename std::remove_cv<typename std::remove_pointer<decltype(mrow)>::type>::type MT;
+            const __amdgpu_buffer_rsrc_t mrsrc =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<MT *>(mrow), 0, N * (int)sizeof(MT), 0x00020000);
+            for (int j = 0; j * 256 < N; ++j) {
+                const int e0 = (64 * j + lane) * 4;
+                float mv[4];
+                if constexpr (sizeof(MT) == 4) {
+                    const f32x4 raw = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(mrsrc, e0 * 4, 0, 0));
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) mv[r] = raw[r];
+                } else {
+                    typedef MT mt4 __attribute__((ext_vector_type(4)));
+                    const mt4 raw = __builtin_bit_cast(mt4, __builtin_amdgcn_raw_buffer_load_b64(mrsrc, e0 * 2, 0, 0));
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) mv[r] = (float)raw[r];
+                }
+                bool nz = false, nm = false;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float sm = scale_mask(mv[r], p.clamp);
+                    const bool valid = e0 + r < N;
+                    nz |= valid && (sm != 0.0f);
+                    nm |= valid && (sm > kNegBig);
+                }
+                const uint64_t bz = __ballot(nz), bn = __ballot(nm);
+                const int k = lane & 3, t = 4 * j + k;
+                const bool any_nz = ((bz >> (16 * k)) & 0xFFFFull) != 0, any_nm = ((bn >> (16 * k)) & 0xFFFFull) != 0;
+                const bool mine = lane < 4 && t < nt_all && any_nm;
+                const bool general = any_nz || t * BN + BN > N;
+                clean_bits |= (__ballot(mine && !general) & 0xFull) << (4 * j);
+                gen_bits |= (__ballot(mine && general) & 0xFull) << (4 * j);
+            }
+        };
+        const bool rows_vectorizable = p.ms[3] == 1;
+        if (p.mask_dtype == KERNL_F32) {
+            const float *mrow = static_cast<const float *>(p.mask) + mask_base;
+            if (rows_vectorizable && aligned16(mrow)) classify4(mrow);
+            else classify(mrow);
+        } else if (p.mask_dtype == KERNL_F16) {
+            const f16 *mrow = static_cast<const f16 *>(p.mask) + mask_base;
+            if (rows_vectorizable && aligned16(mrow)) classify4(mrow);
+            else classify(mrow);
+        } else {
+            const bf16 *mrow = static_cast<const bf16 *>(p.mask) + mask_base;
+            if (rows_vectorizable && aligned16(mrow)) classify4(mrow);
+            else classify(mrow);
+        }
+        // every key masked: keep all tiles, the result is the (finite) uniform average
+        if ((clean_bits | gen_bits) == 0) gen_bits = (nt_all >= 64) ? ~0ull : ((1ull << nt_all) - 1ull);
+        // the clean body is unrolled over both stages: an odd leftover goes through the general body
+        if (__popcll(clean_bits) & 1) {
+            const uint64_t top = 1ull << (63 - __clzll((long long)clean_bits));
+            clean_bits &= ~top;
+            gen_bits |= top;
+        }
+        n_clean = __popcll(clean_bits);
+        nt = n_clean + __popcll(gen_bits);
+    }
+    n_clean &= ~1;
+    // next tile of the processing order; past the end it repeats `last` (a harmless extra prefetch)
+    int order_pos = 0;
+    auto next_tile = [&](int last) -> int {
+        int t;
+        if (use_list) {
+            if (clean_bits != 0) {
+                t = __builtin_ctzll(clean_bits);
+                clean_bits &= clean_bits - 1;
+            } else if (gen_bits != 0) {
+                t = __builtin_ctzll(gen_bits);
+                gen_bits &= gen_bits - 1;
+            } else {
+                t = last;
+            }
+        } else {
+            t = min(order_pos, nt - 1);
+        }
+        ++order_pos;
+        return __builtin_amdgcn_readfirstlane(t);
+    };
+
     // ---- running state of this lane's query row
     float m_i = -INFINITY, l_i = 0.0f;
     f32x16 o_acc[DB];
@@ -240,13 +321,17 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     }
     const int64_t mask_row = mask_base + (int64_t)min(my_m, M - 1) * (MASK_MODE == MASK_MATRIX ? p.ms[2] : 0);
 
+    int t_cur = 0, t_nxt = 0;
+    if (nt > 0) {
+        t_cur = next_tile(0);
+        t_nxt = next_tile(t_cur);
+    }
     // one key tile: prefetch the next one into the other stage, scores, online softmax, P·V, publish
     auto tile_step = [&](auto general_c, auto stage_c, int idx) {
         constexpr bool GENERAL = decltype(general_c)::value;
         constexpr int ST = decltype(stage_c)::value;
-        const int tile = tile_of(idx);
+            const int tile = t_cur, tile_next = t_nxt;
         const int n0 = tile * BN;
-        const int tile_next = tile_of(min(idx + 1, nt - 1));
         dma(tile_next, ST ^ 1);
         float bias_next = 0.0f;
         if (GENERAL && tid < BN) bias_next = key_bias(tile_next);
@@ -352,12 +437,13 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         if (GENERAL && tid < BN)
             *reinterpret_cast<float *>(smem + (ST ^ 1) * STAGE + K_BYTES + V_BYTES + tid * 4) = bias_next;
         __syncthreads();
+        t_cur = t_nxt;
+        t_nxt = next_tile(t_nxt);
     };
 
     if (nt > 0) {
-        const int t0 = tile_of(0);
-        dma(t0, 0);
-        if (n_clean == 0 && tid < BN) *reinterpret_cast<float *>(smem + K_BYTES + V_BYTES + tid * 4) = key_bias(t0);
+        if (t_cur != 0) dma(t_cur, 0);
+        if (n_clean == 0 && tid < BN) *reinterpret_cast<float *>(smem + K_BYTES + V_BYTES + tid * 4) = key_bias(t_cur);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far (Q fragments included) has landed
     __syncthreads();
@@ -369,7 +455,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     }
     if (idx < nt) {
         if (n_clean > 0) {  // the additive terms of the first general tile (it sits in stage 0: n_clean is even)
-            if (tid < BN) *reinterpret_cast<float *>(smem + K_BYTES + V_BYTES + tid * 4) = key_bias(tile_of(idx));
+            if (tid < BN) *reinterpret_cast<float *>(smem + K_BYTES + V_BYTES + tid * 4) = key_bias(t_cur);
             __syncthreads();
         }
         for (; idx < nt; idx += 2) {
@@ -553,7 +639,8 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
                          rows_ok(q, q_strides) && rows_ok(k, k_strides) && rows_ok(v, v_strides) &&
                          rows_ok(out, o_strides) && (int64_t)((B * H + 7) / 8) * 8 * p.nq_tiles < (1ll << 31) &&
                          k_strides[2] > 0 && v_strides[2] > 0 &&  // one head's K / V extent must fit 31-bit byte offsets
-                         (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30);
+                         (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30) &&
+                         (mask == nullptr || (mask_strides[3] >= 0 && (N + 128) * mask_strides[3] < (1ll << 30)));
     if (mfma_ok) {
         // head size 64: 115 VGPRs without a matrix mask (up to 4 waves per SIMD); the matrix-mask body needs the
         // register budget of 2 waves per SIMD.  Head size 128: 2 waves per SIMD.

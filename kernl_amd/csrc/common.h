@@ -175,6 +175,6 @@ __device__ __forceinline__ int swz_offset(int row, int chunk) {  // byte offset 
 int set_error(int status, const char *fmt, ...);
 int check_launch(const char *what);
 
-static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+__host__ __device__ static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace kernl
