@@ -44,6 +44,7 @@ struct AttnParams {
     float sm_scale;
     float clamp;  // replacement for -inf mask entries
     int nq_tiles;
+    int mask_fast;  // matrix mask rows can be read as aligned 4-element vectors through 32-bit offsets
 };
 
 __device__ __forceinline__ float load_mask_value(const void *mask, int dtype, int64_t off) {
@@ -320,6 +321,33 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         for (int d = 0; d < DB; ++d) vt_off[d] = K_BYTES + (4 * lh + kq) * VP + ((d ^ vsw) * 64) + fs * 2;
     }
     const int64_t mask_row = mask_base + (int64_t)min(my_m, M - 1) * (MASK_MODE == MASK_MATRIX ? p.ms[2] : 0);
+    // Matrix masks on the fast route: the 8 runs of 4 consecutive keys a lane needs from its mask row are
+    // fetched one tile ahead, right after the previous tile's values have been consumed, into the same registers.
+    constexpr bool MATRIX = (MASK_MODE == MASK_MATRIX);
+    const bool m_fast = MATRIX && p.mask_fast != 0;
+    const bool m_f32 = p.mask_dtype == KERNL_F32;
+    const int m_esize = m_f32 ? 4 : 2;
+    const __amdgpu_buffer_rsrc_t mrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char *>(static_cast<const char *>(p.mask)) + (MATRIX ? mask_base * m_esize : 0), 0,
+        MATRIX ? (int)((((int64_t)M - 1) * p.ms[2] + N) * m_esize) : 0, 0x00020000);
+    const int m_voff = MATRIX ? (int)((int64_t)min(my_m, M - 1) * p.ms[2] + lh * 4) * m_esize : 0;
+    const float clamp_eff = fmaxf(p.clamp, kClampFloor / kLog2eA);  // (-inf -> clamp) * log2(e) stays finite
+    u32x4 mreg[MATRIX ? 2 * NBS * 2 : 1];
+    auto mask_issue = [&](auto route_c, int tile) {
+        constexpr int ROUTE = decltype(route_c)::value;
+        if (ROUTE == 2) {
+#pragma unroll
+            for (int i = 0; i < NBS * 4; ++i)
+                mreg[i] = __builtin_amdgcn_raw_buffer_load_b128(mrsrc, m_voff + ((i >> 2) * 32 + (i & 3) * 8) * 4, tile * BN * 4, 0);
+        } else if (ROUTE == 1) {
+#pragma unroll
+            for (int i = 0; i < NBS * 4; ++i) {
+                const u32x2 two = __builtin_amdgcn_raw_buffer_load_b64(mrsrc, m_voff + ((i >> 2) * 32 + (i & 3) * 8) * 2, tile * BN * 2, 0);
+                mreg[i >> 1][2 * (i & 1)] = two[0];
+                mreg[i >> 1][2 * (i & 1) + 1] = two[1];
+            }
+        }
+    };
 
     int t_cur = 0, t_nxt = 0;
     if (nt > 0) {
@@ -327,12 +355,19 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         t_nxt = next_tile(t_cur);
     }
     // one key tile: prefetch the next one into the other stage, scores, online softmax, P·V, publish
-    auto tile_step = [&](auto general_c, auto stage_c, int idx) {
+    // ROUTE: how a matrix mask is read (0 = element by element, 1 = prefetched 16-bit vectors, 2 = prefetched fp32
+    // vectors); a compile-time choice so that the tile body carries no branches for it
+    auto tile_step = [&](auto general_c, auto stage_c, auto route_c) {
         constexpr bool GENERAL = decltype(general_c)::value;
         constexpr int ST = decltype(stage_c)::value;
+        constexpr int ROUTE = decltype(route_c)::value;
             const int tile = t_cur, tile_next = t_nxt;
         const int n0 = tile * BN;
-        dma(tile_next, ST ^ 1);
+        // With a prefetched matrix mask the compiler waits for ALL vector-memory loads before it touches the last
+        // mask register (it does not know about the loads issued in assembly), so there the next tile is only
+        // requested once the mask values have been consumed.
+        constexpr bool LATE_DMA = GENERAL && (MASK_MODE == MASK_MATRIX);
+        if (!LATE_DMA) dma(tile_next, ST ^ 1);
         float bias_next = 0.0f;
         if (GENERAL && tid < BN) bias_next = key_bias(tile_next);
 
@@ -364,12 +399,29 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                     for (int g = 0; g < 4; ++g) {
                         const int nl = nb * 32 + g * 8 + lh * 4;  // key index inside the tile
                         const f32x4 cb = *reinterpret_cast<const f32x4 *>(colbias + nl);
+                        f32x4 mm = {0.0f, 0.0f, 0.0f, 0.0f};
+                        if (MATRIX && ROUTE != 0) {
+                            const int i = nb * 4 + g;
+                            if (ROUTE == 2) {
+                                mm = __builtin_bit_cast(f32x4, mreg[i]);
+                            } else {
+                                typedef T t4 __attribute__((ext_vector_type(4)));
+                                const u32x2 two = {mreg[i >> 1][2 * (i & 1)], mreg[i >> 1][2 * (i & 1) + 1]};
+                                const t4 h4 = __builtin_bit_cast(t4, two);
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) mm[r] = (float)h4[r];
+                            }
+                        }
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
                             float sv = s_acc[nb][g * 4 + r] * c + cb[r];
-                            if (MASK_MODE == MASK_MATRIX) {
-                                const int n = min(n0 + nl + r, N - 1);
-                                sv += scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_row + n * p.ms[3]), p.clamp);
+                            if (MATRIX) {
+                                if (ROUTE != 0) {
+                                    sv = fmaf(fmaxf(mm[r], clamp_eff), kLog2eA, sv);
+                                } else {
+                                    const int n = min(n0 + nl + r, N - 1);
+                                    sv += scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_row + n * p.ms[3]), p.clamp);
+                                }
                             }
                             if (CAUSAL && (n0 + nl + r > my_m)) sv = -INFINITY;
                             s_acc[nb][g * 4 + r] = sv;
@@ -384,6 +436,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                     for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[nb][v]);
                 mx *= c;  // c > 0 (checked by the host)
             }
+            if (LATE_DMA) dma(tile_next, ST ^ 1);
             mx = halves32_max(mx);  // the other 16-key half of every 32-key block lives in lane ^ 32
             // m_i is the exponent REFERENCE of this row, not necessarily its running maximum: it only moves (and the
             // accumulator and row sum are rescaled) when the new maximum exceeds it by more than 2^8, so
@@ -431,9 +484,12 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
             }
             __builtin_amdgcn_s_setprio(0);
             l_i += rs;
+        } else if (LATE_DMA) {
+            dma(tile_next, ST ^ 1);
         }
 
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the next tile is in LDS
+        if (GENERAL && MATRIX) mask_issue(route_c, tile_next);
         if (GENERAL && tid < BN)
             *reinterpret_cast<float *>(smem + (ST ^ 1) * STAGE + K_BYTES + V_BYTES + tid * 4) = bias_next;
         __syncthreads();
@@ -450,18 +506,24 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 
     int idx = 0;
     for (; idx < n_clean; idx += 2) {
-        tile_step(BoolC<false>(), IntC<0>(), idx);
-        tile_step(BoolC<false>(), IntC<1>(), idx + 1);
+        tile_step(BoolC<false>(), IntC<0>(), IntC<0>());
+        tile_step(BoolC<false>(), IntC<1>(), IntC<0>());
     }
     if (idx < nt) {
         if (n_clean > 0) {  // the additive terms of the first general tile (it sits in stage 0: n_clean is even)
             if (tid < BN) *reinterpret_cast<float *>(smem + K_BYTES + V_BYTES + tid * 4) = key_bias(t_cur);
             __syncthreads();
         }
-        for (; idx < nt; idx += 2) {
-            tile_step(BoolC<true>(), IntC<0>(), idx);
-            if (idx + 1 < nt) tile_step(BoolC<true>(), IntC<1>(), idx + 1);
-        }
+        auto general_tiles = [&](auto route_c) {
+            if (MATRIX) mask_issue(route_c, t_cur);
+            for (; idx < nt; idx += 2) {
+                tile_step(BoolC<true>(), IntC<0>(), route_c);
+                if (idx + 1 < nt) tile_step(BoolC<true>(), IntC<1>(), route_c);
+            }
+        };
+        if (MATRIX && m_fast && m_f32) general_tiles(IntC<2>());
+        else if (MATRIX && m_fast) general_tiles(IntC<1>());
+        else general_tiles(IntC<0>());
     }
 
     // ---- normalise and store: lane holds features 32 d + 16 lh + (0..15) of row my_m
@@ -629,6 +691,12 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
     p.scale_log2 = sm_scale * 1.4426950408889634f;
     p.clamp = mask_min_clamp;
     p.nq_tiles = (int)((M + 127) / 128);
+    p.mask_fast = 0;
+    if (mask_mode == MASK_MATRIX && (mask_dtype == KERNL_F32 || mask_dtype == dtype)) {
+        const int64_t es = mask_dtype == KERNL_F32 ? 4 : 2;
+        p.mask_fast = mask_strides[3] == 1 && p.ms[0] % 4 == 0 && p.ms[1] % 4 == 0 && p.ms[2] % 4 == 0 && p.ms[2] > 0 &&
+                      aligned16(mask) && ((M - 1) * p.ms[2] + N + 128) * es < (1ll << 31);
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool causal = is_causal != 0;
 
@@ -642,8 +710,8 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
                          (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30) &&
                          (mask == nullptr || (mask_strides[3] >= 0 && (N + 128) * mask_strides[3] < (1ll << 30)));
     if (mfma_ok) {
-        // head size 64: 115 VGPRs without a matrix mask (up to 4 waves per SIMD); the matrix-mask body needs the
-        // register budget of 2 waves per SIMD.  Head size 128: 2 waves per SIMD.
+        // head size 64: ~115 VGPRs without a matrix mask (up to 4 waves per SIMD); the matrix-mask body (mask values
+        // prefetched in registers) needs the register budget of 2 waves per SIMD.  Head size 128: 2 waves per SIMD.
         int wpe = (D == 64 && mask_mode != MASK_MATRIX) ? 3 : 2;
         if (D == 64 && g_attention_variant == 1) wpe = 3;
         if (D == 64 && g_attention_variant == 2) wpe = 2;
