@@ -123,8 +123,9 @@ int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, 
 
 /*
  * Test and tuning hooks (process-wide, not thread-safe; no counterpart in the reference).
- *   kernl_linear_force_tile      0 = heuristic (default), 1 = 256x256, 2 = 256x192, 3 = 128x128 output tile
- *                                of the MFMA linear kernel.
+ *   kernl_linear_force_tile      0 = heuristic (default); output tile of the MFMA linear kernel: 1 = 256x256,
+ *                                2 = 256x192, 3 = 128x128, 4 = 256x128 with 32-wide k-tiles, 5 = 256x256 with one
+ *                                wave per SIMD (needs K % 64 == 0, otherwise 128x128 is used).
  *   kernl_attention_force_scalar non-zero routes every attention call through the strided scalar kernel.
  *   kernl_attention_set_variant  register budget of the head-size-64 MFMA attention kernel: 0 = heuristic,
  *                                1 = built for 3 waves/SIMD, 2 = built for 2 waves/SIMD.

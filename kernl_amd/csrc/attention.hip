@@ -67,15 +67,6 @@ __device__ __forceinline__ float scale_mask(float mv, float clamp) {
 // is unrolled over the two LDS stages; the others (ragged last tile, masked, causal diagonal) follow in a general
 // body.  The order of key tiles does not matter to the online softmax.
 // ----------------------------------------------------------------------------------------------------
-template <bool B>
-struct BoolC {
-    static constexpr bool value = B;
-};
-template <int I>
-struct IntC {
-    static constexpr int value = I;
-};
-
 template <typename T, int D, int WPE, int MASK_MODE, bool CAUSAL>
 __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnParams p) {
     typedef typename Vec8<T>::type vec8;

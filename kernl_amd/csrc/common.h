@@ -28,6 +28,16 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 static constexpr int kWave = 64;
 
+// compile-time constants passed as (empty) arguments to generic lambdas
+template <bool B>
+struct BoolC {
+    static constexpr bool value = B;
+};
+template <int I>
+struct IntC {
+    static constexpr int value = I;
+};
+
 // 16-bit storage types map to their 8-wide MFMA operand vector.
 template <typename T>
 struct Vec8;

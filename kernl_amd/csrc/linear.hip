@@ -60,6 +60,82 @@ __device__ __forceinline__ float apply_act(float x, int act) {
 }
 
 // ----------------------------------------------------------------------------------------------------
+// Epilogue shared by the MFMA kernels: lane (lr, lh) holds, for 32x32 block (i, j) of its wave's tile, output row
+// m_wave + 32 i + lr and the 16 consecutive columns starting at n_wave + 32 j + 16 lh.  Bias add, optional store of
+// the pre-activation, activation, one rounding to the output dtype, 16-byte stores where the layout allows.
+// ----------------------------------------------------------------------------------------------------
+template <typename T, int ACT, int TM, int TN>
+__device__ __forceinline__ void linear_epilogue(f32x16 (&acc)[TM][TN], int m_wave, int n_wave, int lr, int lh,
+                                                const T *__restrict__ bias, T *__restrict__ out,
+                                                T *__restrict__ act_in, int M, int N, int64_t out_rs, int64_t out_cs,
+                                                int64_t ai_rs, int64_t ai_cs, int out_vec_ok, int ai_vec_ok,
+                                                int bias_vec_ok) {
+    typedef typename Vec8<T>::type vec8;
+    const bool HAS_BIAS = bias != nullptr, SAVE_ACT_IN = act_in != nullptr;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int n = n_wave + j * 32 + lh * 16;
+        float bv[16];
+        if (HAS_BIAS) {
+            if (bias_vec_ok && n + 16 <= N) {
+                const vec8 b0 = *reinterpret_cast<const vec8 *>(bias + n);
+                const vec8 b1 = *reinterpret_cast<const vec8 *>(bias + n + 8);
+#pragma unroll
+                for (int v = 0; v < 8; ++v) {
+                    bv[v] = to_float(b0[v]);
+                    bv[8 + v] = to_float(b1[v]);
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) bv[v] = (n + v < N) ? to_float(bias[n + v]) : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int m = m_wave + i * 32 + lr;
+            if (m >= M || n >= N) continue;
+            float r[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) r[v] = HAS_BIAS ? acc[i][j][v] + bv[v] : acc[i][j][v];
+            if (SAVE_ACT_IN) {
+                if (ai_vec_ok && n + 16 <= N) {
+                    u32x4 p0, p1;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
+                        p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
+                    }
+                    T *p = act_in + (int64_t)m * ai_rs + n;
+                    *reinterpret_cast<u32x4 *>(p) = p0;
+                    *reinterpret_cast<u32x4 *>(p + 8) = p1;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        if (n + v < N) act_in[(int64_t)m * ai_rs + (int64_t)(n + v) * ai_cs] = from_float<T>(r[v]);
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) r[v] = apply_act(r[v], ACT);
+            if (out_vec_ok && n + 16 <= N) {
+                u32x4 p0, p1;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
+                    p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
+                }
+                T *p = out + (int64_t)m * out_rs + n;
+                *reinterpret_cast<u32x4 *>(p) = p0;
+                *reinterpret_cast<u32x4 *>(p + 8) = p1;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (n + v < N) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
+            }
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------------
 // MFMA kernel
 // ----------------------------------------------------------------------------------------------------
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int MIN_BLOCKS_>
@@ -87,7 +163,6 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
                    int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n,
                    int out_vec_ok, int ai_vec_ok, int bias_vec_ok) {
     typedef typename Vec8<T>::type vec8;
-    const bool HAS_BIAS = bias != nullptr, SAVE_ACT_IN = act_in != nullptr;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, CPR = Cfg::CPR, RB = Cfg::ROW_BYTES;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -234,69 +309,177 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         __syncthreads();
     }
 
-    // ---- epilogue: lane (lr, lh) holds, for block (i, j), output row m0 + WM*wave_m + 32 i + lr and the 16
-    // consecutive columns starting at n0 + WN*wave_n + 32 j + 16 lh.
+    linear_epilogue<T, ACT, TM, TN>(acc, m0 + wave_m * Cfg::WM, n0 + wave_n * Cfg::WN, lr, lh, bias, out, act_in, M, N, out_rs,
+                                    out_cs, ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bias_vec_ok);
+}
+
+// ----------------------------------------------------------------------------------------------------
+// Wide MFMA kernel for K % 64 == 0: 256x256 output tile, 4 waves, ONE wave per SIMD owning a 128x128 sub-tile
+// (16 accumulator blocks = 256 registers, which the compiler keeps in the accumulation half of the register file).
+// Per 16-wide k-step a wave runs 16 MFMAs on 8 operand fragments — half the LDS traffic per MFMA of the 8-wave
+// kernel above.  Operand tiles go HBM -> LDS directly (buffer loads with the LDS flag), two 64 KB stages.  With a
+// single wave per SIMD nothing else can fill a stall, so the instruction stream is laid out by hand: every MFMA
+// is followed by at most one LDS read or one tile load, and the barrier that publishes the next k-tile sits in
+// front of the LAST k-step's MFMAs, whose operands are already in registers — the matrix pipe stays busy while
+// the first fragments of the next tile are fetched.
+// ----------------------------------------------------------------------------------------------------
+template <typename T, int ACT>
+__global__ void __launch_bounds__(256, 1)
+linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
+                   T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
+                   int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok, int ai_vec_ok,
+                   int bias_vec_ok) {
+    typedef typename Vec8<T>::type vec8;
+    constexpr int BM = 256, BN = 256, BK = 64, RB = BK * 2, CPR = BK / 8, TM = 4, TN = 4, KSTEPS = BK / 16;
+    constexpr int X_BYTES = BM * RB, W_BYTES = BN * RB, STAGE = X_BYTES + W_BYTES;
+    constexpr int LOADS = BM * CPR / 256;  // 1 KB loads per wave for each operand tile
+    constexpr int GROUP_M = 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) >> 3;
+    const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || t >= total) return;
+    const int group_span = GROUP_M * tiles_n;
+    const int group = t / group_span;
+    const int first_m = group * GROUP_M;
+    const int gsize = min(tiles_m - first_m, GROUP_M);
+    const int in_group = t - group * group_span;
+    const int tile_m = first_m + in_group % gsize;
+    const int tile_n = in_group / gsize;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave & 1, wave_n = wave >> 1;
+    const int lr = lane & 31, lh = lane >> 5;
+
+    // ---- tile loads: load i of a wave fills the 1 KB of 16-byte chunks [256 i + 64 wave, +64) of an operand tile;
+    // every lane fetches the chunk that belongs at its LDS position under the swizzle.  Rows beyond M / N and
+    // k-tiles beyond K lie outside the buffer resource and arrive as zeros.
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    const int rows_x = min(BM, M - m0), rows_w = min(BN, N - n0);
+    const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx), waddr = (uint64_t)(uintptr_t)(W + (int64_t)n0 * K);
+    const u32x4 xrsrc = {(uint32_t)xaddr, (uint32_t)(xaddr >> 32) & 0xFFFFu,
+                         (uint32_t)((((int64_t)rows_x - 1) * ldx + K) * 2), 0x00020000u};
+    const u32x4 wrsrc = {(uint32_t)waddr, (uint32_t)(waddr >> 32) & 0xFFFFu, (uint32_t)((int64_t)rows_w * K * 2),
+                         0x00020000u};
+    // A wave's loads of one operand tile land in one contiguous 8 KB block (load i at +1 KB i), so that groups of 4
+    // loads share one write of the LDS base register and differ only in the instruction's immediate offset.  That
+    // immediate is added to the memory address too, hence it is subtracted from the per-lane offsets here.
+    uint32_t xd[LOADS], wd[LOADS];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int n = n0 + wave_n * Cfg::WN + j * 32 + lh * 16;
-        float bv[16];
-        if (HAS_BIAS) {
-            if (bias_vec_ok && n + 16 <= N) {
-                const vec8 b0 = *reinterpret_cast<const vec8 *>(bias + n);
-                const vec8 b1 = *reinterpret_cast<const vec8 *>(bias + n + 8);
-#pragma unroll
-                for (int v = 0; v < 8; ++v) {
-                    bv[v] = to_float(b0[v]);
-                    bv[8 + v] = to_float(b1[v]);
-                }
-            } else {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) bv[v] = (n + v < N) ? to_float(bias[n + v]) : 0.0f;
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int m = m0 + wave_m * Cfg::WM + i * 32 + lr;
-            if (m >= M || n >= N) continue;
-            float r[16];
-#pragma unroll
-            for (int v = 0; v < 16; ++v) r[v] = HAS_BIAS ? acc[i][j][v] + bv[v] : acc[i][j][v];
-            if (SAVE_ACT_IN) {
-                if (ai_vec_ok && n + 16 <= N) {
-                    u32x4 p0, p1;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
-                        p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
-                    }
-                    T *p = act_in + (int64_t)m * ai_rs + n;
-                    *reinterpret_cast<u32x4 *>(p) = p0;
-                    *reinterpret_cast<u32x4 *>(p + 8) = p1;
-                } else {
-#pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        if (n + v < N) act_in[(int64_t)m * ai_rs + (int64_t)(n + v) * ai_cs] = from_float<T>(r[v]);
-                }
-            }
-#pragma unroll
-            for (int v = 0; v < 16; ++v) r[v] = apply_act(r[v], ACT);
-            if (out_vec_ok && n + 16 <= N) {
-                u32x4 p0, p1;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
-                    p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
-                }
-                T *p = out + (int64_t)m * out_rs + n;
-                *reinterpret_cast<u32x4 *>(p) = p0;
-                *reinterpret_cast<u32x4 *>(p + 8) = p1;
-            } else {
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    if (n + v < N) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
-            }
-        }
+    for (int i = 0; i < LOADS; ++i) {
+        const int q = (wave * LOADS + i) * 64 + lane;  // 16-byte chunk index inside the tile
+        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        const uint32_t imm = (uint32_t)(i & 3) * 1024u;
+        xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) - imm : kOutOfRange;
+        // LDS row `row` feeds MFMA row (row % 32) of its 32-block and carries weight row rowperm16(row % 32)
+        const int wrow = (row & ~31) + rowperm16(row & 31);
+        wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - imm : kOutOfRange;
     }
+    typedef __attribute__((address_space(3))) void lds_void;
+    const uint32_t dma_base = (uint32_t)(uintptr_t)(lds_void *)smem + wave * (LOADS * 1024);
+    // inline assembly on purpose: the compiler would make every later LDS read wait for loads it sees writing LDS.
+    // `group` (0 or 1) selects loads 4 group .. 4 group + 3; `first` writes the LDS base register for the group.
+    auto load4 = [&](const u32x4 &rsrc, const uint32_t (&off)[LOADS], uint32_t lds, int group, int part, int k0) {
+        const int i = 4 * group + part;
+        if (part == 0)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :: "s"(lds + group * 4096), "v"(off[i]), "s"(rsrc), "s"(k0 * 2) : "memory", "m0");
+        else if (part == 1)
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds" :: "v"(off[i]), "s"(rsrc), "s"(k0 * 2) : "memory");
+        else if (part == 2)
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:2048 lds" :: "v"(off[i]), "s"(rsrc), "s"(k0 * 2) : "memory");
+        else
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off[i]), "s"(rsrc), "s"(k0 * 2) : "memory");
+    };
+    // load l (0..15) of a k-tile: X loads 0..7, then W loads 0..7
+    auto tile_load = [&](int l, int stage, int k0) {
+        if (l < LOADS) load4(xrsrc, xd, dma_base + stage * STAGE, l >> 2, l & 3, k0);
+        else load4(wrsrc, wd, dma_base + stage * STAGE + X_BYTES, (l - LOADS) >> 2, l & 3, k0);
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // LDS byte offsets of this lane's operand fragments, one register per (k-step, block): with a whole register
+    // file per wave there is room to keep them all, and no address arithmetic is left in the loop
+    int xoff[KSTEPS][TM], woff[KSTEPS][TN];
+#pragma unroll
+    for (int st = 0; st < KSTEPS; ++st) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) xoff[st][i] = swz_offset<RB>(wave_m * 128 + i * 32 + lr, 2 * st + lh);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) woff[st][j] = X_BYTES + swz_offset<RB>(wave_n * 128 + j * 32 + lr, 2 * st + lh);
+    }
+
+    const int nk = K / BK;
+#pragma unroll
+    for (int l = 0; l < 2 * LOADS; ++l) tile_load(l, 0, 0);
+#pragma unroll
+    for (int l = 0; l < 2 * LOADS; ++l) tile_load(l, 1, BK);
+    static_assert(2 * LOADS == 16, "the wait below encodes vmcnt(16)");
+    __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): all of tile 0 has landed, tile 1 may still be in flight
+    __syncthreads();
+
+    vec8 fa[2][TN], fb[2][TM];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fa[0][j] = *reinterpret_cast<const vec8 *>(smem + woff[0][j]);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fb[0][i] = *reinterpret_cast<const vec8 *>(smem + xoff[0][i]);
+
+    // one k-tile held in stage CUR (a compile-time constant, so that stage offsets fold into instruction offsets)
+    auto k_tile = [&](auto cur_c, int kt) {
+        constexpr int CUR = decltype(cur_c)::value;
+        const unsigned char *cur = smem + CUR * STAGE;
+        const unsigned char *nxt = smem + (CUR ^ 1) * STAGE;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            const int ob = st & 1, nb = ob ^ 1;
+            // fragments to fetch during this step: those of the next step — for the last step, step 0 of the next
+            // k-tile, which is why the barrier publishing that tile comes first
+            const unsigned char *src = (st + 1 < KSTEPS) ? cur : nxt;
+            const int sn = (st + 1) % KSTEPS;
+            if (st == KSTEPS - 1) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads of the next k-tile have landed
+                __syncthreads();
+            }
+#pragma unroll
+            for (int m = 0; m < TM * TN; ++m) {
+                const int i = m / TN, j = m % TN;
+                acc[i][j] = mfma32(fa[ob][j], fb[ob][i], acc[i][j]);
+                if (m < TN) fa[nb][m] = *reinterpret_cast<const vec8 *>(src + woff[sn][m]);
+                else if (m < TN + TM) fb[nb][m - TN] = *reinterpret_cast<const vec8 *>(src + xoff[sn][m - TN]);
+                // tile kt + 2 goes into the stage every wave has just finished reading, one load behind each MFMA
+                if (st == KSTEPS - 1) tile_load(m, CUR, (kt + 2) * BK);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+        k_tile(IntC<0>(), kt);
+        k_tile(IntC<1>(), kt + 1);
+    }
+    if (kt < nk) k_tile(IntC<0>(), kt);
+
+    // one call per 32-row block: each stays small enough for the compiler to unroll completely, so the accumulators
+    // are only ever indexed by constants and never leave the register file
+#define KERNL_WIDE_EPILOGUE(I)                                                                                          \
+    linear_epilogue<T, ACT, 1, TN>(*reinterpret_cast<f32x16(*)[1][TN]>(&acc[I]), m0 + wave_m * 128 + 32 * (I),          \
+                                   n0 + wave_n * 128, lr, lh, bias, out, act_in, M, N, out_rs, out_cs, ai_rs, ai_cs,    \
+                                   out_vec_ok, ai_vec_ok, bias_vec_ok)
+    KERNL_WIDE_EPILOGUE(0);
+    KERNL_WIDE_EPILOGUE(1);
+    KERNL_WIDE_EPILOGUE(2);
+    KERNL_WIDE_EPILOGUE(3);
+#undef KERNL_WIDE_EPILOGUE
 }
 
 // ----------------------------------------------------------------------------------------------------
@@ -396,6 +579,40 @@ static void launch_mfma_cfg(const LinearArgs &a) {
     }
 }
 
+template <typename T, int ACT>
+static void launch_wide_act(const LinearArgs &a) {
+    auto kern = linear_wide_kernel<T, ACT>;
+    constexpr int LDS_BYTES = 2 * (256 + 256) * 128;
+    static bool attr_done = false;  // benign race: the attribute call is idempotent
+    if (!attr_done) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        attr_done = true;
+    }
+    const int tiles_m = (a.M + 255) / 256, tiles_n = (a.N + 255) / 256;
+    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+    const T *bias = static_cast<const T *>(a.bias);
+    T *out = static_cast<T *>(a.out);
+    T *act_in = static_cast<T *>(a.act_in);
+    const int out_vec_ok = a.out_cs == 1 && a.out_rs % 8 == 0 && aligned16(out);
+    const int ai_vec_ok = act_in != nullptr && a.ai_cs == 1 && a.ai_rs % 8 == 0 && aligned16(act_in);
+    const int bias_vec_ok = bias != nullptr && aligned16(bias);
+    hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
+                       static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
+                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok);
+}
+
+template <typename T>
+static void launch_wide(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_wide_act<T, KERNL_ACT_RELU>(a); break;
+        case KERNL_ACT_TANH: launch_wide_act<T, KERNL_ACT_TANH>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_wide_act<T, KERNL_ACT_GELU_ERF>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_wide_act<T, KERNL_ACT_GELU_TANH>(a); break;
+        case KERNL_ACT_SILU: launch_wide_act<T, KERNL_ACT_SILU>(a); break;
+        default: launch_wide_act<T, KERNL_ACT_NONE>(a); break;
+    }
+}
+
 //                         BM   BN  BK  WAVES_M WAVES_N  MIN_BLOCKS
 typedef LinearTile<256, 256, 64, 2, 4, 1> Tile256x256;
 typedef LinearTile<256, 192, 64, 4, 2, 1> Tile256x192;
@@ -412,7 +629,7 @@ static double tile_cost(int M, int N, int bm, int bn, int blocks_per_cu) {
     return (double)rounds * bm * bn * blocks_per_cu / eff;
 }
 
-int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128
+int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256
 
 template <typename T>
 static int linear_mfma_dispatch(const LinearArgs &a) {
@@ -425,8 +642,13 @@ static int linear_mfma_dispatch(const LinearArgs &a) {
         double best = c1;
         if (c2 < best) { best = c2; pick = 2; }
         if (c3 < best) { best = c3; pick = 3; }
+        // long k-loops over many full tiles with a cheap epilogue: one wave per SIMD with a 128x128 sub-tile
+        const int64_t tiles256 = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
+        if (pick == 1 && a.K % 64 == 0 && a.K >= 4096 && tiles256 >= 512 && (a.act == KERNL_ACT_NONE || a.act == KERNL_ACT_RELU))
+            pick = 5;
     }
-    if (pick == 1) launch_mfma_cfg<T, Tile256x256>(a);
+    if (pick == 5 && a.K % 64 == 0) launch_wide<T>(a);
+    else if (pick == 1) launch_mfma_cfg<T, Tile256x256>(a);
     else if (pick == 2) launch_mfma_cfg<T, Tile256x192>(a);
     else if (pick == 4) launch_mfma_cfg<T, Tile256x128k32>(a);
     else launch_mfma_cfg<T, Tile128x128>(a);
