@@ -68,6 +68,12 @@ def main():
     ap.add_argument("--skip-e2e", action="store_true", help="skip the BERT-base forward latency")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline timings")
     ap.add_argument("--skip-extra", action="store_true", help="only the headline attention numbers")
+    ap.add_argument(
+        "--pmc-probe",
+        action="store_true",
+        help="launch the headline kernel 3 times, then copy a 64 MiB tensor 3 times, and exit: the workload of the "
+        "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (the copy of known size scales the counters)",
+    )
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU per process and ships no multi-GPU path; run with --gpus 1")
@@ -96,15 +102,24 @@ def main():
     def step():
         attention_forward(qd, kd, vd, out, 0.125, False, md)
 
+    if args.pmc_probe:
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        src = torch.empty(32 * 1024 * 1024, dtype=torch.half, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        return
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    # The K timed steps are replayed from ONE hipGraph holding K launches with an event pair around each (this is
-    # how the product path runs the kernels — optimize_model replays a hipGraph — and it keeps the ~50 us of
-    # Python/ctypes work per eager call out of a ~50 us kernel's timing).  Falls back to eager launches if event
-    # nodes cannot be captured.
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    # The K timed steps are replayed from ONE hipGraph holding K launches (this is how the product path runs the
+    # kernels — optimize_model replays a hipGraph — and it keeps the ~40 us of Python/ctypes work per eager call out
+    # of a ~40 us kernel's timing).  The replay is bracketed by a host clock (value) and by a HIP event pair on the
+    # stream the replay is launched on (average launch duration for the roofline).
     graph = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -114,19 +129,24 @@ def main():
     torch.cuda.synchronize()
     graph.replay()  # untimed: first replay uploads the graph
     torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    ev0.record()
     graph.replay()
+    ev1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
-    # per-launch durations with HIP events on the launch stream, same kernel, same inputs, eager launches
+    avg_launch_ms = ev0.elapsed_time(ev1) / args.steps
+    # eager launches with an event pair each, for comparison: these include the gap the host leaves between launches
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
     for i in range(args.steps):
         starts[i].record()
         step()
         ends[i].record()
     torch.cuda.synchronize()
     launch_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
-    avg_launch_ms = sum(launch_ms) / len(launch_ms)
     value = dense_flop / (ms_per_step * 1e-3) / 1e12
     achieved = dense_flop / (avg_launch_ms * 1e-3) / 1e12
     attn_bytes = 4 * B * H * S * D * 2 + mask.numel() * 4
@@ -158,12 +178,13 @@ def main():
             "frac": round(achieved / PEAK_MFMA_F16_TFLOPS, 4),
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy of known
             # size (profiles/attention_config1_pmc_traffic.txt); algorithmic bytes are 100.7e6
-            "traffic": 99.3e6,
+            "traffic": 92.0e6,
         },
     }
     extra = {
         "attention_avg_launch_us": round(avg_launch_ms * 1e3, 2),
-        "attention_min_launch_us": round(min(launch_ms) * 1e3, 2),
+        "attention_eager_avg_launch_us": round(sum(launch_ms) / len(launch_ms) * 1e3, 2),
+        "attention_eager_min_launch_us": round(min(launch_ms) * 1e3, 2),
         "attention_executed_tflops": round(executed_flop / (avg_launch_ms * 1e-3) / 1e12, 2),
         "attention_executed_fraction_of_dense": round(executed_flop / dense_flop, 4),
         "attention_algorithmic_gbps": round(attn_bytes / (avg_launch_ms * 1e-3) / 1e9, 1),
