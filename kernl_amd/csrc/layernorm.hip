@@ -16,59 +16,85 @@ struct Row16 {  // one 16-byte chunk of a row
     T v[kElems];
 };
 
-// One wave per row; lane l owns chunks l, l+64, ... (CHUNKS of them at most).
-template <typename T, int CHUNKS, bool RMS, bool HAS_RES>
+// A group of GROUP_WAVES waves (1 or the 4 of the block) per row; thread t of the group owns chunks t, t + G, ...
+// (G = 64 GROUP_WAVES, CHUNKS of them at most).  A group walks rows with a fixed stride and fetches the next row
+// before it reduces the current one, so that loads of one row overlap the arithmetic and the stores of another.
+template <typename T, int CHUNKS, bool RMS, bool HAS_RES, int GROUP_WAVES>
 __global__ void __launch_bounds__(256)
 layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const T *__restrict__ w,
                       const T *__restrict__ b, T *__restrict__ out, float *__restrict__ mean_out,
                       float *__restrict__ rstd_out, int M, int N, int64_t x_rs, int64_t res_rs,
-                      int64_t out_rs, float eps) {
+                      int64_t out_rs, float eps, int stream_out) {
     constexpr int E = Row16<T>::kElems;
+    constexpr int G = 64 * GROUP_WAVES;
     typedef Row16<T> chunk_t;
+    __shared__ float red[2][4];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int waves_per_block = blockDim.x >> 6;
+    const int t = GROUP_WAVES == 1 ? lane : (int)threadIdx.x;  // index inside the group
+    const int groups_per_block = 4 / GROUP_WAVES;
+    const int group = GROUP_WAVES == 1 ? wave : 0;
     const int nchunks = N / E;
     const float inv_n = 1.0f / (float)N;
 
-    // gamma / beta stay in registers (as 16-bit pairs) for every row this wave visits.
+    // sum over the group: wave reduction, then (4-wave groups) a round trip through LDS
+    auto group_sum = [&](float v, int slot) -> float {
+        v = wave_sum(v);
+        if (GROUP_WAVES == 1) return v;
+        __syncthreads();  // the previous use of this slot has been read by everyone
+        if (lane == 0) red[slot][wave] = v;
+        __syncthreads();
+        return (red[slot][0] + red[slot][1]) + (red[slot][2] + red[slot][3]);
+    };
+
+    // gamma / beta stay in registers (as 16-bit values) for every row this group visits.
     chunk_t wv[CHUNKS], bv[CHUNKS];
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
-        const int ci = lane + c * 64;
+        const int ci = t + c * G;
         if (ci < nchunks) {
             wv[c] = *reinterpret_cast<const chunk_t *>(w + (int64_t)ci * E);
             if (b != nullptr) bv[c] = *reinterpret_cast<const chunk_t *>(b + (int64_t)ci * E);
         }
     }
 
-    for (int row = blockIdx.x * waves_per_block + wave; row < M; row += gridDim.x * waves_per_block) {
-        float v[CHUNKS][E];
-        const T *xr = x + (int64_t)row * x_rs;
+    const int row_step = gridDim.x * groups_per_block;
+    int row = blockIdx.x * groups_per_block + group;
+    chunk_t xn[CHUNKS], rn[HAS_RES ? CHUNKS : 1];
+    auto fetch = [&](int r) {
+        const T *xr = x + (int64_t)r * x_rs;
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
-            const int ci = lane + c * 64;
-            if (ci < nchunks) {
-                chunk_t t = *reinterpret_cast<const chunk_t *>(xr + (int64_t)ci * E);
-#pragma unroll
-                for (int e = 0; e < E; ++e) v[c][e] = to_float(t.v[e]);
-            } else {
-#pragma unroll
-                for (int e = 0; e < E; ++e) v[c][e] = 0.0f;
-            }
+            const int ci = t + c * G;
+            if (ci < nchunks) xn[c] = *reinterpret_cast<const chunk_t *>(xr + (int64_t)ci * E);
         }
         if (HAS_RES) {
-            const T *rr = res + (int64_t)row * res_rs;
+            const T *rr = res + (int64_t)r * res_rs;
 #pragma unroll
             for (int c = 0; c < CHUNKS; ++c) {
-                const int ci = lane + c * 64;
-                if (ci < nchunks) {
-                    chunk_t t = *reinterpret_cast<const chunk_t *>(rr + (int64_t)ci * E);
-#pragma unroll
-                    for (int e = 0; e < E; ++e) v[c][e] += to_float(t.v[e]);
-                }
+                const int ci = t + c * G;
+                if (ci < nchunks) rn[c] = *reinterpret_cast<const chunk_t *>(rr + (int64_t)ci * E);
             }
         }
+    };
+    if (row < M) fetch(row);
+
+    for (; row < M; row += row_step) {
+        float v[CHUNKS][E];
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) {
+            const int ci = t + c * G;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                float a = 0.0f;
+                if (ci < nchunks) {
+                    a = to_float(xn[c].v[e]);
+                    if (HAS_RES) a += to_float(rn[c].v[e]);
+                }
+                v[c][e] = a;
+            }
+        }
+        if (row + row_step < M) fetch(row + row_step);
 
         float mean = 0.0f, var;
         if (RMS) {
@@ -77,18 +103,18 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
             for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
                 for (int e = 0; e < E; ++e) ss += v[c][e] * v[c][e];
-            var = wave_sum(ss) * inv_n;
+            var = group_sum(ss, 0) * inv_n;
         } else {
             float s = 0.0f;
 #pragma unroll
             for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
                 for (int e = 0; e < E; ++e) s += v[c][e];
-            mean = wave_sum(s) * inv_n;
+            mean = group_sum(s, 0) * inv_n;
             float ss = 0.0f;
 #pragma unroll
             for (int c = 0; c < CHUNKS; ++c) {
-                const int ci = lane + c * 64;
+                const int ci = t + c * G;
                 if (ci < nchunks) {
 #pragma unroll
                     for (int e = 0; e < E; ++e) {
@@ -97,10 +123,10 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
                     }
                 }
             }
-            var = wave_sum(ss) * inv_n;
+            var = group_sum(ss, 1) * inv_n;
         }
         const float rstd = 1.0f / sqrtf(var + eps);
-        if (lane == 0) {
+        if (t == 0) {
             if (mean_out != nullptr) mean_out[row] = mean;
             if (rstd_out != nullptr) rstd_out[row] = rstd;
         }
@@ -108,7 +134,7 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
         T *orow = out + (int64_t)row * out_rs;
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
-            const int ci = lane + c * 64;
+            const int ci = t + c * G;
             if (ci < nchunks) {
                 chunk_t o;
 #pragma unroll
@@ -117,7 +143,13 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
                     if (b != nullptr) y += to_float(bv[c].v[e]);
                     o.v[e] = from_float<T>(y);
                 }
-                *reinterpret_cast<chunk_t *>(orow + (int64_t)ci * E) = o;
+                // Outputs too large to stay cached until their consumer runs are written with streaming stores
+                // (measured +15 % bandwidth here); smaller ones with plain stores, because the GEMM that follows
+                // in a model then finds them in L2 / MALL (measured: streaming stores cost BERT-base 1 % end to end).
+                if (stream_out)
+                    __builtin_nontemporal_store(__builtin_bit_cast(u32x4, o), reinterpret_cast<u32x4 *>(orow + (int64_t)ci * E));
+                else
+                    *reinterpret_cast<chunk_t *>(orow + (int64_t)ci * E) = o;
             }
         }
     }
@@ -174,13 +206,14 @@ layernorm_strided_kernel(const T *__restrict__ x, const T *__restrict__ res, con
     }
 }
 
-template <typename T, int CHUNKS>
+template <typename T, int CHUNKS, int GROUP_WAVES>
 static void launch_rows(bool rms, bool has_res, dim3 grid, hipStream_t st, const T *x, const T *res,
                         const T *w, const T *b, T *out, float *mean, float *rstd, int M, int N, int64_t x_rs,
                         int64_t res_rs, int64_t out_rs, float eps) {
-#define KERNL_LN_LAUNCH(R, H)                                                                          \
-    hipLaunchKernelGGL((layernorm_rows_kernel<T, CHUNKS, R, H>), grid, dim3(256), 0, st, x, res, w, b, \
-                       out, mean, rstd, M, N, x_rs, res_rs, out_rs, eps)
+#define KERNL_LN_LAUNCH(R, H)                                                                                       \
+    hipLaunchKernelGGL((layernorm_rows_kernel<T, CHUNKS, R, H, GROUP_WAVES>), grid, dim3(256), 0, st, x, res, w, b, \
+                       out, mean, rstd, M, N, x_rs, res_rs, out_rs, eps, stream_out)
+    const int stream_out = (int64_t)M * N * (int64_t)sizeof(T) > (128ll << 20);
     if (rms) {
         if (has_res) KERNL_LN_LAUNCH(true, true);
         else KERNL_LN_LAUNCH(true, false);
@@ -209,19 +242,27 @@ static int layernorm_dispatch(const void *x_, const void *res_, const void *w_, 
                         aligned16(x) && aligned16(out) && aligned16(w) && (b == nullptr || aligned16(b)) &&
                         (!has_res || aligned16(res)) && row_chunks <= 64 * 16;
     if (vec_ok) {
-        // 4 rows per 256-thread block; enough blocks to cover the rows, capped so that gamma/beta loads
-        // amortise over several rows on large inputs.
-        const int64_t blocks_needed = (M + 3) / 4;
-        const int grid = (int)(blocks_needed < 8192 ? blocks_needed : 8192);
-        const int chunks = (int)((row_chunks + 63) / 64);
-#define KERNL_LN_CASE(C)                                                                                   \
-    launch_rows<T, C>(rms, has_res, dim3(grid), st, x, res, w, b, out, mean, rstd, (int)M, (int)N, x_rs, \
-                      res_rs, out_rs, eps)
-        if (chunks <= 1) KERNL_LN_CASE(1);
-        else if (chunks <= 2) KERNL_LN_CASE(2);
-        else if (chunks <= 4) KERNL_LN_CASE(4);
-        else if (chunks <= 8) KERNL_LN_CASE(8);
-        else KERNL_LN_CASE(16);
+        // Rows of up to 1024 chunks stay in registers.  Long rows on few-row inputs are spread over the 4 waves of a
+        // block (more loads in flight per row); otherwise a wave per row, 4 rows per block.  The grid is capped at
+        // 8 waves per SIMD so that every group walks several rows and gamma/beta loads amortise.
+        const bool block_per_row = row_chunks > 128 && M < 16384;
+        const int64_t blocks_needed = block_per_row ? M : (M + 3) / 4;
+        const int grid = (int)(blocks_needed < 2048 ? blocks_needed : 2048);
+        const int chunks = (int)((row_chunks + (block_per_row ? 255 : 63)) / (block_per_row ? 256 : 64));
+#define KERNL_LN_CASE(C, GW)                                                                                   \
+    launch_rows<T, C, GW>(rms, has_res, dim3(grid), st, x, res, w, b, out, mean, rstd, (int)M, (int)N, x_rs, \
+                          res_rs, out_rs, eps)
+        if (block_per_row) {
+            if (chunks <= 1) KERNL_LN_CASE(1, 4);
+            else if (chunks <= 2) KERNL_LN_CASE(2, 4);
+            else KERNL_LN_CASE(4, 4);
+        } else {
+            if (chunks <= 1) KERNL_LN_CASE(1, 1);
+            else if (chunks <= 2) KERNL_LN_CASE(2, 1);
+            else if (chunks <= 4) KERNL_LN_CASE(4, 1);
+            else if (chunks <= 8) KERNL_LN_CASE(8, 1);
+            else KERNL_LN_CASE(16, 1);
+        }
 #undef KERNL_LN_CASE
     } else {
         const int grid = (int)(M < 65535 ? M : 65535);
