@@ -75,6 +75,28 @@ int kernl_attention_fwd(const void *q, const void *k, const void *v, void *out, 
                         float sm_scale, int is_causal, float mask_min_clamp, int dtype, void *stream);
 
 /*
+ * Split-K attention for very few query rows (decoding: q_len = 1 against a long key sequence).  Same arguments and
+ * semantics as kernl_attention_fwd plus a workspace; the keys of every (batch, head, query row) are split into
+ * ranges that run in parallel and are merged by a second kernel.  Replaces the `_fwd_part_1[grid]` /
+ * `_fwd_part_2[grid_part2]` launches of src/kernl/implementations/attention_skinny.py:458-535 (the reference
+ * allocates its partial maxima / sums / products there, :416-441; here the caller passes them as one workspace).
+ * Unlike the reference's dispatch (src/kernl/optimizer/attention.py:45-49, which falls back to eager PyTorch for
+ * masked or causal single-query attention) masks and is_causal are handled.
+ *
+ *   workspace        device memory of at least kernl_attention_skinny_workspace_bytes(B,H,M,N,D) bytes (fp32
+ *                    partial results); may be NULL / smaller, which only reduces the number of key ranges.
+ *   D                a power of two in 8..256; q, k, v need unit feature stride and 16-byte aligned rows.
+ *   B*H*M            at most 65535.
+ */
+int64_t kernl_attention_skinny_workspace_bytes(int64_t B, int64_t H, int64_t M, int64_t N, int64_t D);
+int kernl_attention_skinny_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
+                               void *workspace, int64_t workspace_bytes, int64_t B, int64_t H, int64_t M, int64_t N,
+                               int64_t D, const int64_t q_strides[4], const int64_t k_strides[4],
+                               const int64_t v_strides[4], const int64_t o_strides[4], const int64_t mask_sizes[4],
+                               const int64_t mask_strides[4], int mask_dtype, float sm_scale, int is_causal,
+                               float mask_min_clamp, int dtype, void *stream);
+
+/*
  * Fused linear layer:  out[M,N] = act(x[M,K] · w[N,K]ᵀ + bias[N]).
  * Replaces the `kernel_fma[grid](...)` launch of src/kernl/implementations/linear_layer.py:254-278
  * (kernel body :92-210).

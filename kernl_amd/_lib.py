@@ -22,6 +22,8 @@ EXPORTED_SYMBOLS = (
     "kernl_version",
     "kernl_last_error_string",
     "kernl_attention_fwd",
+    "kernl_attention_skinny_workspace_bytes",
+    "kernl_attention_skinny_fwd",
     "kernl_linear_fwd",
     "kernl_layernorm_fwd",
     "kernl_add_layernorm_fwd",
@@ -60,6 +62,12 @@ def load() -> ctypes.CDLL:
     lib.kernl_attention_fwd.restype = ctypes.c_int
     lib.kernl_attention_fwd.argtypes = (
         [_vp] * 5 + [_i64] * 5 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, _vp]
+    )
+    lib.kernl_attention_skinny_workspace_bytes.restype = _i64
+    lib.kernl_attention_skinny_workspace_bytes.argtypes = [_i64] * 5
+    lib.kernl_attention_skinny_fwd.restype = ctypes.c_int
+    lib.kernl_attention_skinny_fwd.argtypes = (
+        [_vp] * 6 + [_i64] * 6 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, _vp]
     )
     lib.kernl_linear_fwd.restype = ctypes.c_int
     lib.kernl_linear_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
@@ -115,6 +123,32 @@ def attention_fwd(q, k, v, out, mask, sm_scale: float, is_causal: bool, mask_min
             float(sm_scale), int(bool(is_causal)), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
         )
     _check(st, "kernl_attention_fwd")
+
+
+def attention_skinny_workspace_bytes(B: int, H: int, M: int, N: int, D: int) -> int:
+    return int(load().kernl_attention_skinny_workspace_bytes(B, H, M, N, D))
+
+
+def attention_skinny_fwd(q, k, v, out, mask, workspace, sm_scale: float, is_causal: bool, mask_min_clamp: float) -> None:
+    _require_gpu(q, k, v, out, mask, workspace)
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    lib = load()
+    if mask is not None:
+        msizes, mstrides, mdtype, mptr = _arr(mask.shape), _arr(mask.stride()), DTYPE_CODE[mask.dtype], mask.data_ptr()
+    else:
+        msizes, mstrides, mdtype, mptr = None, None, KERNL_F32, None
+    ws_ptr = None if workspace is None else workspace.data_ptr()
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with torch.cuda.device(q.device):
+        st = lib.kernl_attention_skinny_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), mptr, ws_ptr, ws_bytes,
+            B, H, M, N, D,
+            _arr(q.stride()), _arr(k.stride()), _arr(v.stride()), _arr(out.stride()),
+            msizes, mstrides, mdtype,
+            float(sm_scale), int(bool(is_causal)), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
+        )
+    _check(st, "kernl_attention_skinny_fwd")
 
 
 def linear_fwd(x2d, weight, bias, out2d, act_in2d, activation: int) -> None:

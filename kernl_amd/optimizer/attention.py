@@ -9,6 +9,7 @@ from typing import Optional
 import torch
 
 from kernl_amd.implementations.attention import attention_forward
+from kernl_amd.implementations.attention_skinny import skinny_attention_forward
 from kernl_amd.utils.extended_matcher import replace_pattern
 
 
@@ -17,6 +18,14 @@ def _per_key_view(mask: torch.Tensor) -> torch.Tensor:
     if mask.dim() == 4 and mask.size(2) > 1 and mask.stride(2) == 0:
         return mask[:, :, :1, :]
     return mask
+
+
+def _rows_aligned(*tensors: torch.Tensor) -> bool:
+    """Unit feature stride and 16-byte aligned rows (what the split-K kernel's vector loads need)."""
+    for t in tensors:
+        if t.stride(-1) != 1 or t.data_ptr() % 16 != 0 or any(st % 8 != 0 for st in t.stride()[:-1]):
+            return False
+    return True
 
 
 def attention_wrapper(
@@ -36,9 +45,14 @@ def attention_wrapper(
             attention_mask = attention_mask.unsqueeze(1)
     if attention_mask is not None:
         attention_mask = _per_key_view(attention_mask)
-    # The reference hands single-query attention over long keys to a split-K kernel or to eager PyTorch
-    # (optimizer/attention.py:45-49); the HIP kernel covers that shape itself.
-    attention_forward(q, k, v, output, sm_scale, is_causal=is_causal, attention_mask=attention_mask)
+    # Single-query attention over long keys has no parallelism over rows: like the reference
+    # (optimizer/attention.py:45-49) hand it to the split-K kernel — which here also takes masks and the causal
+    # flag, where the reference falls back to eager PyTorch.  Head sizes it does not cover stay on the tiled kernel.
+    dhead = q.size(-1)
+    if q.size(-2) == 1 and k.size(-2) > 50 and 8 <= dhead <= 256 and (dhead & (dhead - 1)) == 0 and _rows_aligned(q, k, v):
+        skinny_attention_forward(q, k, v, output, sm_scale, is_causal=is_causal, attention_mask=attention_mask)
+    else:
+        attention_forward(q, k, v, output, sm_scale, is_causal=is_causal, attention_mask=attention_mask)
     if extend_head:
         output = output.squeeze(1)
     return output
