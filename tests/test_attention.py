@@ -175,3 +175,24 @@ def test_attention_rejects_bad_arguments():
         attention_forward(q, q, q, out, 1.0, False, torch.zeros((3, 1, 1, 16), device="cuda"))  # bad batch broadcast
     with pytest.raises(AssertionError):
         attention_forward(q, q, q, out, 1.0, False, torch.zeros((1, 1, 1, 15), device="cuda"))  # bad key count
+
+
+@pytest.mark.parametrize("n_keys", [4096, 4100, 6000], ids=lambda n: f"{n}keys")
+@pytest.mark.parametrize("mask_kind", ["padding", "all_masked"])
+def test_attention_long_key_sequences_with_vector_mask(n_keys, mask_kind, close):
+    # up to 64 key tiles the per-key mask is classified tile by tile (clean / general / dropped sets kept in two
+    # 64-bit words); longer sequences take every tile through the general body
+    gen = torch.Generator().manual_seed(11)
+    q = torch.randn((1, 2, 160, 64), generator=gen).half()
+    k = torch.randn((1, 2, n_keys, 64), generator=gen).half()
+    v = torch.randn((1, 2, n_keys, 64), generator=gen).half()
+    mask = torch.zeros((1, 1, 1, n_keys))
+    if mask_kind == "padding":
+        mask[..., n_keys - 1500:] = float("-inf")
+        mask[..., 100:300] = float("-inf")
+        ref = attention_oracle(q, k, v, 0.125, False, mask)
+    else:
+        mask[:] = float("-inf")
+        ref = v.float().mean(dim=-2, keepdim=True).expand(-1, -1, 160, -1)
+    out = _run(q, k, v, 0.125, False, mask)
+    close(out, ref, torch.float16, what=f"attention {n_keys} keys {mask_kind}")
