@@ -137,21 +137,26 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     // Inline assembly on purpose: the compiler, seeing LDS written by a load, would make every later LDS read
     // wait for the vector-memory counter, i.e. for the prefetch itself.  The explicit wait before the barrier
     // that publishes the stage is the one that matters.
-    auto dma = [&](int tile, int stage) {
-        const int k_soff = tile * k_tile_bytes, v_soff = tile * v_tile_bytes;
-        const uint32_t sb = dma_base + stage * STAGE;
+    auto uniform = [](uint32_t x) __attribute__((always_inline)) -> uint32_t { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); };
+    auto dma = [&](int tile, int stage) __attribute__((always_inline)) {
+        // every operand below is wave-uniform; saying so explicitly keeps them in scalar registers whatever the
+        // control flow around the call looks like to the compiler
+        const uint32_t k_soff = uniform((uint32_t)(tile * k_tile_bytes)), v_soff = uniform((uint32_t)(tile * v_tile_bytes));
+        const uint32_t sb = uniform(dma_base + stage * STAGE);
+        const u32x4 kr = {uniform(krsrc[0]), uniform(krsrc[1]), uniform(krsrc[2]), uniform(krsrc[3])};
+        const u32x4 vr = {uniform(vrsrc[0]), uniform(vrsrc[1]), uniform(vrsrc[2]), uniform(vrsrc[3])};
 #pragma unroll
         for (int i = 0; i < KI; ++i)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :: "s"(sb + i * 4096), "v"(kdma[i]), "s"(krsrc), "s"(k_soff) : "memory", "m0");
+                         :: "s"(sb + i * 4096), "v"(kdma[i]), "s"(kr), "s"(k_soff) : "memory", "m0");
 #pragma unroll
         for (int i = 0; i < KI; ++i)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :: "s"(sb + K_BYTES + i * 4096), "v"(vdma[i]), "s"(vrsrc), "s"(v_soff) : "memory", "m0");
+                         :: "s"(sb + K_BYTES + i * 4096), "v"(vdma[i]), "s"(vr), "s"(v_soff) : "memory", "m0");
     };
     // per-key additive term of a general tile (mask value in the log2 domain, -inf past the last key); thread tid
     // < 64 owns key tid of the tile
-    auto key_bias = [&](int tile) -> float {
+    auto key_bias = [&](int tile) __attribute__((always_inline)) -> float {
         const int n = tile * BN + tid;
         float bv = 0.0f;
         if (MASK_MODE == MASK_VECTOR)
@@ -176,7 +181,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     uint64_t clean_bits = 0, gen_bits = 0;
     if (use_list) {
         // lane l looks at key 64 t + l of tile t; 32-bit offsets (the host checks that a mask row fits them)
-        auto classify = [&](auto *mrow) {
+        auto classify = [&](auto *mrow) __attribute__((always_inline)) {
             const int ms3 = (int)p.ms[3];
             const int lane_off = lane * ms3, tile_step_off = BN * ms3;
             for (int t0 = 0; t0 < nt_all; t0 += 8) {
@@ -205,7 +210,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         // Contiguous, 16-byte aligned mask rows take a shorter route: a lane loads 4 consecutive keys, so 16 lanes
         // cover a tile and one load covers 4 tiles; lanes 0..3 then each judge one of those tiles from the two
         // wave-wide ballots.
-        auto classify4 = [&](auto *mrow) {
+        auto classify4 = [&](auto *mrow) __attribute__((always_inline)) {
             typedef typename std::remove_cv<typename std::remove_pointer<decltype(mrow)>::type>::type MT;
             const __amdgpu_buffer_rsrc_t mrsrc =
                 __builtin_amdgcn_make_buffer_rsrc(const_cast<MT *>(mrow), 0, N * (int)sizeof(MT), 0x00020000);
@@ -255,19 +260,12 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         }
         // every key masked: keep all tiles, the result is the (finite) uniform average
         if ((clean_bits | gen_bits) == 0) gen_bits = (nt_all >= 64) ? ~0ull : ((1ull << nt_all) - 1ull);
-        // the clean body is unrolled over both stages: an odd leftover goes through the general body
-        if (__popcll(clean_bits) & 1) {
-            const uint64_t top = 1ull << (63 - __clzll((long long)clean_bits));
-            clean_bits &= ~top;
-            gen_bits |= top;
-        }
         n_clean = __popcll(clean_bits);
         nt = n_clean + __popcll(gen_bits);
     }
-    n_clean &= ~1;
     // next tile of the processing order; past the end it repeats `last` (a harmless extra prefetch)
     int order_pos = 0;
-    auto next_tile = [&](int last) -> int {
+    auto next_tile = [&](int last) __attribute__((always_inline)) -> int {
         int t;
         if (use_list) {
             if (clean_bits != 0) {
@@ -324,7 +322,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     const int m_voff = MATRIX ? (int)((int64_t)min(my_m, M - 1) * p.ms[2] + lh * 4) * m_esize : 0;
     const float clamp_eff = fmaxf(p.clamp, kClampFloor / kLog2eA);  // (-inf -> clamp) * log2(e) stays finite
     u32x4 mreg[MATRIX ? 2 * NBS * 2 : 1];
-    auto mask_issue = [&](auto route_c, int tile) {
+    auto mask_issue = [&](auto route_c, int tile) __attribute__((always_inline)) {
         constexpr int ROUTE = decltype(route_c)::value;
         if (ROUTE == 2) {
 #pragma unroll
@@ -348,7 +346,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     // one key tile: prefetch the next one into the other stage, scores, online softmax, P·V, publish
     // ROUTE: how a matrix mask is read (0 = element by element, 1 = prefetched 16-bit vectors, 2 = prefetched fp32
     // vectors); a compile-time choice so that the tile body carries no branches for it
-    auto tile_step = [&](auto general_c, auto stage_c, auto route_c) {
+    auto tile_step = [&](auto general_c, auto stage_c, auto route_c) __attribute__((always_inline)) {
         constexpr bool GENERAL = decltype(general_c)::value;
         constexpr int ST = decltype(stage_c)::value;
         constexpr int ROUTE = decltype(route_c)::value;
@@ -495,18 +493,29 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far (Q fragments included) has landed
     __syncthreads();
 
+    // clean tiles in pairs over the two stages; an odd one leaves the general tiles starting in stage 1
     int idx = 0;
-    for (; idx < n_clean; idx += 2) {
+    for (; idx + 1 < n_clean; idx += 2) {
         tile_step(BoolC<false>(), IntC<0>(), IntC<0>());
         tile_step(BoolC<false>(), IntC<1>(), IntC<0>());
     }
+    const bool odd_clean = idx < n_clean;
+    if (odd_clean) {
+        tile_step(BoolC<false>(), IntC<0>(), IntC<0>());
+        ++idx;
+    }
     if (idx < nt) {
-        if (n_clean > 0) {  // the additive terms of the first general tile (it sits in stage 0: n_clean is even)
-            if (tid < BN) *reinterpret_cast<float *>(smem + K_BYTES + V_BYTES + tid * 4) = key_bias(t_cur);
+        if (n_clean > 0) {  // the additive terms of the first general tile
+            if (tid < BN)
+                *reinterpret_cast<float *>(smem + (odd_clean ? STAGE : 0) + K_BYTES + V_BYTES + tid * 4) = key_bias(t_cur);
             __syncthreads();
         }
-        auto general_tiles = [&](auto route_c) {
+        auto general_tiles = [&](auto route_c) __attribute__((always_inline)) {
             if (MATRIX) mask_issue(route_c, t_cur);
+            if (odd_clean) {
+                tile_step(BoolC<true>(), IntC<1>(), route_c);
+                ++idx;
+            }
             for (; idx < nt; idx += 2) {
                 tile_step(BoolC<true>(), IntC<0>(), route_c);
                 if (idx + 1 < nt) tile_step(BoolC<true>(), IntC<1>(), route_c);
@@ -701,17 +710,17 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
                          (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30) &&
                          (mask == nullptr || (mask_strides[3] >= 0 && (N + 128) * mask_strides[3] < (1ll << 30)));
     if (mfma_ok) {
-        // head size 64: ~115 VGPRs without a matrix mask (up to 4 waves per SIMD); the matrix-mask body (mask values
-        // prefetched in registers) needs the register budget of 2 waves per SIMD.  Head size 128: 2 waves per SIMD.
-        int wpe = (D == 64 && mask_mode != MASK_MATRIX) ? 3 : 2;
-        if (D == 64 && g_attention_variant == 1) wpe = 3;
+        // head size 64 without a matrix mask fits the register budget of 4 waves per SIMD (128 VGPRs); the
+        // matrix-mask body (mask values prefetched in registers) and head size 128 run at 2 waves per SIMD.
+        int wpe = (D == 64 && mask_mode != MASK_MATRIX) ? 4 : 2;
+        if (D == 64 && g_attention_variant == 1) wpe = 4;
         if (D == 64 && g_attention_variant == 2) wpe = 2;
         if (dtype == KERNL_F16) {
-            if (D == 64 && wpe == 3) launch_stream<f16, 64, 3>(p, mask_mode, causal, st);
+            if (D == 64 && wpe == 4) launch_stream<f16, 64, 4>(p, mask_mode, causal, st);
             else if (D == 64) launch_stream<f16, 64, 2>(p, mask_mode, causal, st);
             else launch_stream<f16, 128, 2>(p, mask_mode, causal, st);
         } else {
-            if (D == 64 && wpe == 3) launch_stream<bf16, 64, 3>(p, mask_mode, causal, st);
+            if (D == 64 && wpe == 4) launch_stream<bf16, 64, 4>(p, mask_mode, causal, st);
             else if (D == 64) launch_stream<bf16, 64, 2>(p, mask_mode, causal, st);
             else launch_stream<bf16, 128, 2>(p, mask_mode, causal, st);
         }
