@@ -97,6 +97,23 @@ int kernl_attention_skinny_fwd(const void *q, const void *k, const void *v, void
                                float mask_min_clamp, int dtype, void *stream);
 
 /*
+ * Rotary position embedding, half-split convention:  out = x·cos + rotate_half(x)·sin, with
+ * rotate_half(x)[d] = -x[d + D/2] (d < D/2), x[d - D/2] (d >= D/2); fp32 arithmetic, one rounding.
+ * The reference applies the same rotation (in Meta's interleaved-pair convention) inside its fused query/key
+ * projection: experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:69-100 (`rbe_triton`), eager form
+ * experimental/llama-v2/llama/model.py:78-88.  Here it is one kernel per tensor, replacing the eight element-wise
+ * kernels a traced Hugging Face decoder runs for it.
+ *
+ *   x, out           [B,H,S,D], f16, bf16 or f32 (dtype), any strides (16-byte vector path for the 16-bit types when
+ *                    the feature stride is 1 and rows are 16-byte aligned); D even.
+ *   cos, sin         tables of table_dtype (f16 / bf16 / f32) with sizes table_sizes = {B|1, H|1, S, D}.
+ */
+int kernl_rope_fwd(const void *x, const void *cos, const void *sin, void *out, int64_t B, int64_t H, int64_t S,
+                   int64_t D, const int64_t x_strides[4], const int64_t out_strides[4], const int64_t table_sizes[4],
+                   const int64_t cos_strides[4], const int64_t sin_strides[4], int table_dtype, int dtype,
+                   void *stream);
+
+/*
  * Fused linear layer:  out[M,N] = act(x[M,K] · w[N,K]ᵀ + bias[N]).
  * Replaces the `kernel_fma[grid](...)` launch of src/kernl/implementations/linear_layer.py:254-278
  * (kernel body :92-210).

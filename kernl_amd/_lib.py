@@ -24,6 +24,7 @@ EXPORTED_SYMBOLS = (
     "kernl_attention_fwd",
     "kernl_attention_skinny_workspace_bytes",
     "kernl_attention_skinny_fwd",
+    "kernl_rope_fwd",
     "kernl_linear_fwd",
     "kernl_layernorm_fwd",
     "kernl_add_layernorm_fwd",
@@ -69,6 +70,8 @@ def load() -> ctypes.CDLL:
     lib.kernl_attention_skinny_fwd.argtypes = (
         [_vp] * 6 + [_i64] * 6 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, _vp]
     )
+    lib.kernl_rope_fwd.restype = ctypes.c_int
+    lib.kernl_rope_fwd.argtypes = [_vp] * 4 + [_i64] * 4 + [_i64p] * 5 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_linear_fwd.restype = ctypes.c_int
     lib.kernl_linear_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_layernorm_fwd.restype = ctypes.c_int
@@ -149,6 +152,20 @@ def attention_skinny_fwd(q, k, v, out, mask, workspace, sm_scale: float, is_caus
             float(sm_scale), int(bool(is_causal)), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
         )
     _check(st, "kernl_attention_skinny_fwd")
+
+
+def rope_fwd(x, cos, sin, out) -> None:
+    """x, out [B,H,S,D]; cos, sin [B|1,H|1,S,D] of the same dtype as each other."""
+    _require_gpu(x, cos, sin, out)
+    B, H, S, D = x.shape
+    lib = load()
+    with torch.cuda.device(x.device):
+        st = lib.kernl_rope_fwd(
+            x.data_ptr(), cos.data_ptr(), sin.data_ptr(), out.data_ptr(), B, H, S, D,
+            _arr(x.stride()), _arr(out.stride()), _arr(cos.shape), _arr(cos.stride()), _arr(sin.stride()),
+            DTYPE_CODE[cos.dtype], DTYPE_CODE[x.dtype], _stream(x),
+        )
+    _check(st, "kernl_rope_fwd")
 
 
 def linear_fwd(x2d, weight, bias, out2d, act_in2d, activation: int) -> None:

@@ -10,6 +10,7 @@ from kernl_amd.optimizer.attention import (
     fuse_attention_sdpa,
 )
 from kernl_amd.optimizer.dropout import remove_dropout
+from kernl_amd.optimizer.kv_cache import drop_empty_cat_operands
 from kernl_amd.optimizer.layer_norm import replace_layer_norm, replace_layer_norm_fn, replace_layer_norm_rms
 from kernl_amd.optimizer.linear import replace_all_linear
 from kernl_amd.optimizer.mask import (
@@ -20,11 +21,14 @@ from kernl_amd.optimizer.mask import (
     sink_expand_below_where,
 )
 from kernl_amd.optimizer.normalizer import normalize_operators
+from kernl_amd.optimizer.rotary import fuse_rotary_embedding
 
 
 def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
     normalize_operators(gm)
     remove_dropout(gm)
+    drop_empty_cat_operands(gm)
+    fuse_rotary_embedding(gm)
     scalar_tensors_to_full(gm)
     drop_all_true_conjuncts(gm)
     merge_nested_expands(gm)

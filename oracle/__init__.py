@@ -13,4 +13,6 @@ from oracle.ops import (  # noqa: F401
     layer_norm_welford_oracle,
     linear_oracle,
     rms_norm_oracle,
+    rotary_complex_oracle,
+    rotary_oracle,
 )

@@ -19,6 +19,9 @@ How each function is pinned (tests/test_oracle.py):
   layer_norm_welford_oracle equals layer_norm_oracle to fp32 rounding for N in {128 .. 4096 .. 5000}
   rms_norm_oracle         x * rsqrt(mean(x^2)+eps) * w closed form; constant-row known answer
   effective_eps           code reading only (layer_norm.py:295-296)
+  rotary_oracle           equals rotary_complex_oracle (the reference's complex product) under the even/odd <-> half
+                          permutation; zero angle = identity; angles add; quarter turn of a unit vector; norms kept
+  rotary_complex_oracle   torch.view_as_complex product as in the reference; pinned by the same known answers
 Nothing here is "parity unpinned".
 """
 import math
@@ -239,3 +242,28 @@ def layer_norm_welford_oracle(
             y = y + bias.astype(np.float32)
         out[row] = y
     return out, means, rstds
+
+
+# ------------------------------------------------------------------------------------------------------------------
+# rotary position embedding
+# ------------------------------------------------------------------------------------------------------------------
+def rotary_oracle(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """Half-split convention: feature d < D/2 pairs with feature d + D/2.  out = x*cos + rotate_half(x)*sin in fp32;
+    cos, sin broadcast against x ([.., S, D], both halves of the last dimension holding the same angles in the
+    usual tables, though nothing here requires it).  Same rotation as experimental/llama-v2/llama/model.py:78-88 with
+    the features permuted."""
+    xf, c, s = x.float(), cos.float(), sin.float()
+    half = x.shape[-1] // 2
+    lo, hi = xf[..., :half], xf[..., half:]
+    out_lo = lo * c[..., :half] - hi * s[..., :half]
+    out_hi = hi * c[..., half:] + lo * s[..., half:]
+    return torch.cat((out_lo, out_hi), dim=-1)
+
+
+def rotary_complex_oracle(x: torch.Tensor, angles: torch.Tensor) -> torch.Tensor:
+    """Interleaved-pair convention exactly as the reference computes it (experimental/llama-v2/llama/model.py:78-88):
+    features (2i, 2i+1) are the real and imaginary parts of a complex number multiplied by exp(i*angle_i).
+    x [.., S, D], angles [S, D/2]."""
+    xc = torch.view_as_complex(x.float().reshape(*x.shape[:-1], -1, 2).contiguous())
+    rot = torch.polar(torch.ones_like(angles, dtype=torch.float32), angles.float())
+    return torch.view_as_real(xc * rot).flatten(-2)

@@ -331,7 +331,69 @@ def test_llama_graph_rewrite_and_constant_causal_mask():
         assert t.count(fused) == 2
         assert t.count("layer_norm_rms_wrapper") == 2 * 2 + 1 and "rsqrt" not in t
         assert t.count("fused_linear_wrapper") == 2 and "silu" not in t and "softmax" not in t
+        # rotary embedding: one fused call each for queries and keys per layer, nothing left of rotate_half
+        assert t.count("rotary_wrapper") == 2 * 2 and "neg" not in t
+        # the fresh key/value cache no longer copies: the only cat left builds the angle table
+        assert t.count("cat") == 1
         for node in graphs[0].graph.nodes:
             if node.op == "call_function" and node.target.__name__ == fused:
                 assert node.args[mask_idx] is None and node.args[5] is True
+                assert node.args[0].target.__name__ == "rotary_wrapper" and node.args[1].target.__name__ == "rotary_wrapper"
     torch._dynamo.reset()
+
+
+def test_empty_cat_operands_are_dropped():
+    from kernl_amd.optimizer.kv_cache import drop_empty_cat_operands
+
+    # TorchDynamo records the literal as a call of torch.tensor (symbolic_trace would fold it into an attribute)
+    g = torch.fx.Graph()
+    a_n, b_n = g.placeholder("a"), g.placeholder("b")
+    empty = g.call_function(torch.tensor, ([],))
+    one = g.call_function(torch.cat, ([empty, a_n],), {"dim": -2})
+    empty2 = g.call_function(torch.tensor, ([],))
+    two = g.call_function(torch.cat, ([empty2, a_n, b_n],), {"dim": -2})
+    keep = g.call_function(torch.cat, ([a_n, b_n],), {"dim": -1})
+    g.output((one, two, keep))
+    gm = torch.fx.GraphModule(torch.nn.Module(), g)
+    a, b = torch.randn(2, 3, 4), torch.randn(2, 3, 4)
+    expect = gm(a, b)
+    drop_empty_cat_operands(gm)
+    cats = [n for n in gm.graph.nodes if n.op == "call_function" and n.target is torch.cat]
+    assert len(cats) == 2 and all(len(n.args[0]) == 2 for n in cats)
+    assert not any(n.op == "call_function" and n.target is torch.tensor for n in gm.graph.nodes)
+    for got, want in zip(gm(a, b), expect):
+        assert torch.equal(got, want)
+
+
+def test_rotary_pass_only_fires_on_a_mid_split():
+    from kernl_amd.optimizer.rotary import fuse_rotary_embedding
+
+    def trace(split):
+        class M(torch.nn.Module):
+            def forward(self, x, cos, sin):
+                x1, x2 = x[..., :split], x[..., split:]
+                return x * cos + torch.cat((-x2, x1), dim=-1) * sin
+
+        gm = torch.fx.symbolic_trace(M())
+        for n in gm.graph.nodes:
+            if n.op == "placeholder" and n.name == "x":
+                n.meta["example_value"] = torch.empty(1, 2, 4, 8)
+        return gm
+
+    gm = trace(4)
+    fuse_rotary_embedding(gm)
+    assert _targets(gm).count("rotary_wrapper") == 1 and "cat" not in _targets(gm)
+    gm = trace(2)  # not a rotation by halves: left alone
+    fuse_rotary_embedding(gm)
+    assert "rotary_wrapper" not in _targets(gm) and "cat" in _targets(gm)
+    # sin and cos swapped between the operands is still the same expression; a different source tensor is not
+    class Other(torch.nn.Module):
+        def forward(self, x, y, cos, sin):
+            return x * cos + torch.cat((-y[..., 4:], y[..., :4]), dim=-1) * sin
+
+    gm = torch.fx.symbolic_trace(Other())
+    for n in gm.graph.nodes:
+        if n.op == "placeholder" and n.name in ("x", "y"):
+            n.meta["example_value"] = torch.empty(1, 2, 4, 8)
+    fuse_rotary_embedding(gm)
+    assert "rotary_wrapper" not in _targets(gm)

@@ -18,6 +18,8 @@ from oracle import (
     layer_norm_welford_oracle,
     linear_oracle,
     rms_norm_oracle,
+    rotary_complex_oracle,
+    rotary_oracle,
 )
 
 
@@ -191,3 +193,60 @@ def test_effective_eps():
     assert effective_eps(1e-3, torch.float16) == 1e-3
     assert effective_eps(1e-12, torch.bfloat16) == 1e-12
     assert effective_eps(1e-12, torch.float32) == 1e-12
+
+
+def _angles(S, D, theta=10000.0):
+    inv_freq = 1.0 / (theta ** (torch.arange(0, D, 2).float() / D))
+    return torch.outer(torch.arange(S).float(), inv_freq)  # [S, D/2]
+
+
+def _tables(angles):
+    emb = torch.cat((angles, angles), dim=-1)
+    return emb.cos(), emb.sin()
+
+
+def test_rotary_half_split_equals_reference_complex_product():
+    """The half-split form on features permuted [even..., odd...] is the reference's complex multiplication."""
+    gen = torch.Generator().manual_seed(0)
+    B, H, S, D = 2, 3, 17, 16
+    x = torch.randn((B, H, S, D), generator=gen)
+    ang = _angles(S, D)
+    ref = rotary_complex_oracle(x, ang)  # interleaved layout
+    to_half = torch.cat((torch.arange(0, D, 2), torch.arange(1, D, 2)))
+    cos, sin = _tables(ang)
+    out = rotary_oracle(x[..., to_half], cos, sin)
+    assert torch.allclose(out, ref[..., to_half], atol=1e-6, rtol=1e-6)
+
+
+def test_rotary_known_answers():
+    gen = torch.Generator().manual_seed(1)
+    S, D = 5, 8
+    x = torch.randn((1, 2, S, D), generator=gen)
+    zero = torch.zeros((S, D // 2))
+    assert torch.equal(rotary_oracle(x, *_tables(zero)), x)
+    assert torch.allclose(rotary_complex_oracle(x, zero), x)
+    # quarter turn: the unit vector on feature 0 moves to its partner, with a plus sign; the partner moves to minus
+    quarter = torch.full((S, D // 2), math.pi / 2)
+    e0 = torch.zeros((1, 1, S, D))
+    e0[..., 0] = 1.0
+    out = rotary_oracle(e0, *_tables(quarter))
+    expect = torch.zeros_like(e0)
+    expect[..., D // 2] = 1.0
+    assert torch.allclose(out, expect, atol=1e-6)
+    eh = torch.zeros((1, 1, S, D))
+    eh[..., D // 2] = 1.0
+    expect = torch.zeros_like(eh)
+    expect[..., 0] = -1.0
+    assert torch.allclose(rotary_oracle(eh, *_tables(quarter)), expect, atol=1e-6)
+    ec = torch.zeros((1, 1, S, D))
+    ec[..., 0] = 1.0  # real part of pair 0 -> imaginary part of pair 0
+    expect = torch.zeros_like(ec)
+    expect[..., 1] = 1.0
+    assert torch.allclose(rotary_complex_oracle(ec, quarter), expect, atol=1e-6)
+    # angles add, norms of each pair are preserved
+    a, b = _angles(S, D), 0.37 * _angles(S, D) + 0.1
+    twice = rotary_oracle(rotary_oracle(x, *_tables(a)), *_tables(b))
+    assert torch.allclose(twice, rotary_oracle(x, *_tables(a + b)), atol=1e-5)
+    out = rotary_oracle(x, *_tables(a))
+    pair_norm = lambda t: t[..., : D // 2] ** 2 + t[..., D // 2:] ** 2
+    assert torch.allclose(pair_norm(out), pair_norm(x), atol=1e-5)
