@@ -132,6 +132,22 @@ int kernl_linear_fwd(const void *x, const void *w, const void *bias, void *out, 
                      const int64_t act_in_strides[2], int activation, int dtype, void *stream);
 
 /*
+ * Gated linear unit:  out[M,N] = act(x·w_gateᵀ + b_gate) * (x·w_valueᵀ + b_value)  as ONE GEMM.
+ * Replaces the `ff_llama` launch of experimental/llama-v2/kernel/fused_kernel_ff.py:10-79 (SwiGLU: act = SiLU; that
+ * kernel's RMSNorm prologue is not part of this entry point) — and the three kernels (two GEMMs, one multiply) a
+ * traced decoder runs for `act_fn(gate_proj(x)) * up_proj(x)`.
+ *
+ *   w     [2N,K] contiguous, the two weights interleaved in blocks of 32 rows: rows [64b, 64b+32) are rows
+ *         [32b, 32b+32) of w_gate, rows [64b+32, 64b+64) the same rows of w_value.  N must be a multiple of 32.
+ *   bias  NULL or [2N], interleaved like w.
+ *   x     [M,K] with unit feature stride, 16-byte aligned rows, K a multiple of 8; f16 or bf16 only.
+ *   activation  KERNL_ACT_* applied to the gate half (SILU for SwiGLU, GELU_TANH / GELU_ERF for GeGLU).
+ */
+int kernl_linear_glu_fwd(const void *x, const void *w, const void *bias, void *out, int64_t M, int64_t N, int64_t K,
+                         const int64_t x_strides[2], const int64_t out_strides[2], int activation, int dtype,
+                         void *stream);
+
+/*
  * LayerNorm / RMSNorm forward over the last dimension of a 2-D view x[M,N].
  * Replaces the `implementation[(M,)](...)` launch of src/kernl/implementations/layer_norm.py:314-331
  * (kernel body :115-205).

@@ -26,6 +26,7 @@ EXPORTED_SYMBOLS = (
     "kernl_attention_skinny_fwd",
     "kernl_rope_fwd",
     "kernl_linear_fwd",
+    "kernl_linear_glu_fwd",
     "kernl_layernorm_fwd",
     "kernl_add_layernorm_fwd",
     "kernl_linear_force_tile",
@@ -74,6 +75,8 @@ def load() -> ctypes.CDLL:
     lib.kernl_rope_fwd.argtypes = [_vp] * 4 + [_i64] * 4 + [_i64p] * 5 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_linear_fwd.restype = ctypes.c_int
     lib.kernl_linear_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
+    lib.kernl_linear_glu_fwd.restype = ctypes.c_int
+    lib.kernl_linear_glu_fwd.argtypes = [_vp] * 4 + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_layernorm_fwd.restype = ctypes.c_int
     lib.kernl_layernorm_fwd.argtypes = [_vp] * 6 + [_i64] * 6 + [ctypes.c_float, ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_add_layernorm_fwd.restype = ctypes.c_int
@@ -182,6 +185,20 @@ def linear_fwd(x2d, weight, bias, out2d, act_in2d, activation: int) -> None:
             int(activation), DTYPE_CODE[x2d.dtype], _stream(x2d),
         )
     _check(st, "kernl_linear_fwd")
+
+
+def linear_glu_fwd(x2d, weight_interleaved, bias_interleaved, out2d, activation: int) -> None:
+    _require_gpu(x2d, weight_interleaved, bias_interleaved, out2d)
+    M, K = x2d.shape
+    N = weight_interleaved.shape[0] // 2
+    lib = load()
+    with torch.cuda.device(x2d.device):
+        st = lib.kernl_linear_glu_fwd(
+            x2d.data_ptr(), weight_interleaved.data_ptr(),
+            None if bias_interleaved is None else bias_interleaved.data_ptr(), out2d.data_ptr(),
+            M, N, K, _arr(x2d.stride()), _arr(out2d.stride()), int(activation), DTYPE_CODE[x2d.dtype], _stream(x2d),
+        )
+    _check(st, "kernl_linear_glu_fwd")
 
 
 def layernorm_fwd(x2d, weight, bias, out2d, mean, rstd, eps: float, is_rms: bool, residual2d=None) -> None:

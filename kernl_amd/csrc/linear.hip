@@ -63,7 +63,15 @@ __device__ __forceinline__ float apply_act(float x, int act) {
 // Epilogue shared by the MFMA kernels: lane (lr, lh) holds, for 32x32 block (i, j) of its wave's tile, output row
 // m_wave + 32 i + lr and the 16 consecutive columns starting at n_wave + 32 j + 16 lh.  Bias add, optional store of
 // the pre-activation, activation, one rounding to the output dtype, 16-byte stores where the layout allows.
+//
+// Gated form (ACT has kGluBit set): the weight rows alternate in blocks of 32 between the gate and the value
+// projection, so blocks (i, 2p) and (i, 2p + 1) of a lane hold the gate and the value of the SAME 16 output elements;
+// out[m, n] = act(gate + bias_gate) * (value + bias_value) with N counting the interleaved rows (twice the output
+// width).  The same product as the reference's fused feed-forward kernel forms from two accumulators
+// (experimental/llama-v2/kernel/fused_kernel_ff.py:36-75).
 // ----------------------------------------------------------------------------------------------------
+static constexpr int kGluBit = 8;
+
 template <typename T, int ACT, int TM, int TN>
 __device__ __forceinline__ void linear_epilogue(f32x16 (&acc)[TM][TN], int m_wave, int n_wave, int lr, int lh,
                                                 const T *__restrict__ bias, T *__restrict__ out,
@@ -71,6 +79,51 @@ __device__ __forceinline__ void linear_epilogue(f32x16 (&acc)[TM][TN], int m_wav
                                                 int64_t ai_rs, int64_t ai_cs, int out_vec_ok, int ai_vec_ok,
                                                 int bias_vec_ok) {
     typedef typename Vec8<T>::type vec8;
+    if constexpr ((ACT & kGluBit) != 0) {
+        static_assert(TN % 2 == 0, "gated epilogue pairs neighbouring 32-column blocks");
+        constexpr int BASE = ACT & (kGluBit - 1);
+        const int n_total = N >> 1;
+#pragma unroll
+        for (int pr = 0; pr < TN / 2; ++pr) {
+            const int n = (n_wave >> 1) + pr * 32 + lh * 16;         // output column
+            const int nb = n_wave + pr * 64 + lh * 16;               // interleaved row of the gate bias
+            float bg[16], bu[16];
+            if (bias != nullptr && n < n_total) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    bg[v] = to_float(bias[nb + v]);
+                    bu[v] = to_float(bias[nb + 32 + v]);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int m = m_wave + i * 32 + lr;
+                if (m >= M || n >= n_total) continue;  // n_total is a multiple of 32: a block is in or out as a whole
+                float r[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const float g = bias != nullptr ? acc[i][2 * pr][v] + bg[v] : acc[i][2 * pr][v];
+                    const float u = bias != nullptr ? acc[i][2 * pr + 1][v] + bu[v] : acc[i][2 * pr + 1][v];
+                    r[v] = apply_act(g, BASE) * u;
+                }
+                if (out_vec_ok) {
+                    u32x4 p0, p1;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
+                        p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
+                    }
+                    T *p = out + (int64_t)m * out_rs + n;
+                    *reinterpret_cast<u32x4 *>(p) = p0;
+                    *reinterpret_cast<u32x4 *>(p + 8) = p1;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
+                }
+            }
+        }
+        return;
+    }
     const bool HAS_BIAS = bias != nullptr, SAVE_ACT_IN = act_in != nullptr;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
@@ -579,6 +632,19 @@ static void launch_mfma_cfg(const LinearArgs &a) {
     }
 }
 
+// gated epilogues: tiles whose waves span an even number of 32-column blocks
+template <typename T, typename Cfg>
+static void launch_mfma_glu(const LinearArgs &a) {
+    switch (a.act & (kGluBit - 1)) {
+        case KERNL_ACT_GELU_ERF: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_GELU_ERF>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_GELU_TANH>(a); break;
+        case KERNL_ACT_RELU: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_RELU>(a); break;
+        case KERNL_ACT_NONE: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_NONE>(a); break;
+        case KERNL_ACT_TANH: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_TANH>(a); break;
+        default: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_SILU>(a); break;
+    }
+}
+
 template <typename T, int ACT>
 static void launch_wide_act(const LinearArgs &a) {
     auto kern = linear_wide_kernel<T, ACT>;
@@ -603,6 +669,17 @@ static void launch_wide_act(const LinearArgs &a) {
 
 template <typename T>
 static void launch_wide(const LinearArgs &a) {
+    if (a.act & kGluBit) {
+        switch (a.act & (kGluBit - 1)) {
+            case KERNL_ACT_GELU_ERF: launch_wide_act<T, kGluBit | KERNL_ACT_GELU_ERF>(a); break;
+            case KERNL_ACT_GELU_TANH: launch_wide_act<T, kGluBit | KERNL_ACT_GELU_TANH>(a); break;
+            case KERNL_ACT_RELU: launch_wide_act<T, kGluBit | KERNL_ACT_RELU>(a); break;
+            case KERNL_ACT_NONE: launch_wide_act<T, kGluBit | KERNL_ACT_NONE>(a); break;
+            case KERNL_ACT_TANH: launch_wide_act<T, kGluBit | KERNL_ACT_TANH>(a); break;
+            default: launch_wide_act<T, kGluBit | KERNL_ACT_SILU>(a); break;
+        }
+        return;
+    }
     switch (a.act) {
         case KERNL_ACT_RELU: launch_wide_act<T, KERNL_ACT_RELU>(a); break;
         case KERNL_ACT_TANH: launch_wide_act<T, KERNL_ACT_TANH>(a); break;
@@ -634,6 +711,18 @@ int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256,
 template <typename T>
 static int linear_mfma_dispatch(const LinearArgs &a) {
     int pick = g_linear_force_tile;
+    if (a.act & kGluBit) {
+        // tiles 256x192 and 256x128 give a wave an odd number of column blocks: not usable for gate/value pairs
+        const int64_t tiles256 = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
+        if (pick == 0) {
+            pick = tile_cost(a.M, a.N, 128, 128, 2) < tile_cost(a.M, a.N, 256, 256, 1) ? 3 : 1;
+            if (pick == 1 && a.K % 64 == 0 && a.K >= 4096 && tiles256 >= 512) pick = 5;
+        }
+        if (pick == 5 && a.K % 64 == 0) launch_wide<T>(a);
+        else if (pick == 3) launch_mfma_glu<T, Tile128x128>(a);
+        else launch_mfma_glu<T, Tile256x256>(a);
+        return check_launch("gated linear (mfma)");
+    }
     if (pick == 0) {
         const double c1 = tile_cost(a.M, a.N, 256, 256, 1);
         const double c2 = tile_cost(a.M, a.N, 256, 192, 1);
@@ -709,4 +798,39 @@ extern "C" int kernl_linear_fwd(const void *x, const void *w, const void *bias, 
         return linear_fma_dispatch<float>(a);
     }
     return set_error(KERNL_ERR_UNSUPPORTED, "linear: unknown dtype %d", dtype);
+}
+
+extern "C" int kernl_linear_glu_fwd(const void *x, const void *w, const void *bias, void *out, int64_t M, int64_t N,
+                                    int64_t K, const int64_t x_strides[2], const int64_t out_strides[2],
+                                    int activation, int dtype, void *stream) {
+    using namespace kernl;
+    if (x == nullptr || w == nullptr || out == nullptr || x_strides == nullptr || out_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "gated linear: x, w, out and their strides must not be NULL");
+    if (M < 0 || N <= 0 || K <= 0)
+        return set_error(KERNL_ERR_INVALID_ARG, "gated linear: bad sizes M=%lld N=%lld K=%lld", (long long)M,
+                         (long long)N, (long long)K);
+    if (N % 32 != 0)
+        return set_error(KERNL_ERR_UNSUPPORTED, "gated linear: output width %lld must be a multiple of 32 (the "
+                         "interleaving block)", (long long)N);
+    if (M > INT32_MAX || 2 * N > INT32_MAX || K > INT32_MAX)
+        return set_error(KERNL_ERR_UNSUPPORTED, "gated linear: sizes must fit in 31 bits");
+    if (activation < KERNL_ACT_NONE || activation > KERNL_ACT_SILU)
+        return set_error(KERNL_ERR_INVALID_ARG, "gated linear: unknown activation %d", activation);
+    if (dtype != KERNL_F16 && dtype != KERNL_BF16)
+        return set_error(KERNL_ERR_UNSUPPORTED, "gated linear: only f16 and bf16 are supported, got dtype %d", dtype);
+    LinearArgs a;
+    a.x = x; a.w = w; a.bias = bias; a.out = out; a.act_in = nullptr;
+    a.M = (int)M; a.N = (int)(2 * N); a.K = (int)K;  // the kernels see the interleaved weight: twice the output width
+    a.x_rs = x_strides[0]; a.x_cs = x_strides[1];
+    a.out_rs = out_strides[0]; a.out_cs = out_strides[1];
+    a.ai_rs = 0; a.ai_cs = 0;
+    a.act = kGluBit | activation;
+    a.st = static_cast<hipStream_t>(stream);
+    const bool mfma_ok = a.x_cs == 1 && K % 8 == 0 && a.x_rs % 8 == 0 && aligned16(x) && aligned16(w) &&
+                         a.x_rs < (1 << 22) && K < (1 << 22);
+    if (!mfma_ok)
+        return set_error(KERNL_ERR_UNSUPPORTED, "gated linear: x must have unit feature stride, 16-byte aligned rows "
+                         "and K a multiple of 8");
+    if (M == 0) return KERNL_OK;
+    return dtype == KERNL_F16 ? linear_mfma_dispatch<f16>(a) : linear_mfma_dispatch<bf16>(a);
 }

@@ -63,3 +63,48 @@ def linear_layer(
 ) -> torch.Tensor:
     """Reference: linear_layer.py:285-292."""
     return LinearLayer.apply(x, weight, bias, activation, act_inputs)
+
+
+GLU_BLOCK = 32  # rows per interleaving block of `kernl_linear_glu_fwd`
+
+
+def interleave_glu_rows(gate: torch.Tensor, value: torch.Tensor) -> torch.Tensor:
+    """[N, ...] gate and value parameters -> [2N, ...] with 32-row blocks alternating gate, value."""
+    assert gate.shape == value.shape and gate.shape[0] % GLU_BLOCK == 0
+    g = gate.reshape(gate.shape[0] // GLU_BLOCK, 1, GLU_BLOCK, *gate.shape[1:])
+    v = value.reshape(value.shape[0] // GLU_BLOCK, 1, GLU_BLOCK, *value.shape[1:])
+    return torch.cat((g, v), dim=1).reshape(2 * gate.shape[0], *gate.shape[1:]).contiguous()
+
+
+def glu_supported(x: torch.Tensor, out_features: int) -> bool:
+    """What the gated kernel needs; callers run the two projections separately otherwise."""
+    return (
+        x.dtype in (torch.float16, torch.bfloat16)
+        and out_features % GLU_BLOCK == 0
+        and x.shape[-1] % 8 == 0
+    )
+
+
+class LinearGLU(torch.autograd.Function):
+    @staticmethod
+    @custom_fwd(device_type="cuda", cast_inputs=torch.float16)
+    def forward(ctx, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], activation: str) -> torch.Tensor:
+        assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
+        assert x.dtype in (torch.float16, torch.bfloat16), f"Unsupported dtype {x.dtype}"
+        assert weight.is_contiguous() and weight.shape[0] % (2 * GLU_BLOCK) == 0
+        assert x.shape[-1] == weight.shape[1], f"Incompatible dimensions: {x.shape} - {weight.shape}"
+        assert bias is None or (bias.is_contiguous() and bias.dtype == x.dtype and bias.shape[0] == weight.shape[0])
+        x_ = x if x.ndim == 2 else x.reshape(-1, x.shape[-1])
+        if x_.stride(-1) != 1 or x_.stride(0) % 8 != 0 or x_.data_ptr() % 16 != 0:
+            x_ = x_.contiguous()
+        M, N = x_.shape[0], weight.shape[0] // 2
+        out = torch.empty((M, N), device=x.device, dtype=x.dtype)
+        _lib.linear_glu_fwd(x_, weight, bias, out, ACTIVATIONS.get(activation, _lib.ACT_NONE))
+        return out if x.ndim == 2 else out.reshape(*x.shape[:-1], N)
+
+
+def linear_glu_layer(x: torch.Tensor, weight_interleaved: torch.Tensor, bias_interleaved: Optional[torch.Tensor], activation="silu") -> torch.Tensor:
+    """activation(x @ w_gateᵀ + b_gate) * (x @ w_valueᵀ + b_value) with the parameters interleaved by
+    `interleave_glu_rows`.  Reference: `kernel_ff` (experimental/llama-v2/kernel/fused_kernel_ff.py:82-117), without
+    its RMSNorm prologue."""
+    return LinearGLU.apply(x, weight_interleaved, bias_interleaved, activation)

@@ -9,7 +9,7 @@ from typing import Callable
 
 import torch
 
-from kernl_amd.implementations.linear_layer import linear_layer
+from kernl_amd.implementations.linear_layer import GLU_BLOCK, interleave_glu_rows, linear_glu_layer, linear_layer
 from kernl_amd.utils.extended_matcher import replace_pattern
 
 
@@ -211,6 +211,92 @@ def fuse_sibling_linears(gm: torch.fx.GraphModule):
         gm.recompile()
 
 
+def glu_linear_wrapper(v: torch.Tensor, w_gate, b_gate, w_value, b_value, activation: str):
+    """activation(linear(v, w_gate, b_gate)) * linear(v, w_value, b_value) as one GEMM with a gated epilogue: the
+    feed-forward entry of SwiGLU / GeGLU decoders (reference: `kernel_ff`,
+    experimental/llama-v2/kernel/fused_kernel_ff.py:82-117).
+
+    The block-interleaved weight the kernel takes is built on the first call (before graph capture) and cached like
+    the fused sibling projections above.  Shapes or dtypes the gated kernel does not cover run as the two fused
+    linears and the multiplication they were in the original graph."""
+    half = v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")
+    dtype = torch.float16 if half else v.dtype
+    usable = (
+        dtype in (torch.float16, torch.bfloat16)
+        and w_gate.shape == w_value.shape
+        and w_gate.shape[0] % GLU_BLOCK == 0
+        and w_gate.shape[1] % 8 == 0
+        and (b_gate is None) == (b_value is None)
+    )
+    if not usable:
+        gate = linear_wrapper_functional(v, w_gate, b_gate, activation=activation)
+        return gate * linear_wrapper_functional(v, w_value, b_value)
+    params = (w_gate, w_value) + (() if b_gate is None else (b_gate, b_value))
+    key = ("glu",) + tuple((p.data_ptr(), p._version, p.dtype) for p in params)
+    cached = _fused_params.get(key)
+    if cached is None:
+        for p in params:
+            if p.dtype == torch.float32 and half:
+                p.data = p.data.half()
+        weight = interleave_glu_rows(w_gate.detach(), w_value.detach())
+        bias = None if b_gate is None else interleave_glu_rows(b_gate.detach(), b_value.detach())
+        key = ("glu",) + tuple((p.data_ptr(), p._version, p.dtype) for p in params)
+        cached = (weight, bias)
+        _fused_params[key] = cached
+    weight, bias = cached
+    return linear_glu_layer(v, weight, bias, activation=activation)
+
+
+torch.fx.wrap("glu_linear_wrapper")
+
+_GLU_ACTIVATIONS = ("silu", "gelu", "fast_gelu", "relu", "tanh")
+
+
+def fuse_gated_linears(gm: torch.fx.GraphModule):
+    """`linear(v, w_gate, activation=act) * linear(v, w_value)` — both products consumed only by the multiplication,
+    the same input, parameters as weights — becomes one `glu_linear_wrapper` call."""
+    import operator
+
+    def is_param(n):
+        return n is None or (isinstance(n, torch.fx.Node) and n.op in ("placeholder", "get_attr"))
+
+    def as_linear(n, want_activation):
+        if not (isinstance(n, torch.fx.Node) and n.op == "call_function" and n.target is linear_wrapper_functional):
+            return None
+        if len(n.args) != 3 or len(n.users) != 1 or set(n.kwargs) - {"activation"}:
+            return None
+        act = n.kwargs.get("activation", "")
+        if (act in _GLU_ACTIVATIONS) != want_activation or (not want_activation and act != ""):
+            return None
+        v, w, b = n.args
+        if not isinstance(v, torch.fx.Node) or w is None or not is_param(w) or not is_param(b):
+            return None
+        return v, w, b, act
+
+    changed = False
+    for node in list(gm.graph.nodes):
+        if not (node.op == "call_function" and node.target in (operator.mul, torch.mul) and len(node.args) == 2 and not node.kwargs):
+            continue
+        for gate_n, value_n in (node.args, node.args[::-1]):
+            gate, value = as_linear(gate_n, True), as_linear(value_n, False)
+            if gate is None or value is None or gate[0] is not value[0] or gate_n is value_n:
+                continue
+            with gm.graph.inserting_before(node):
+                fused = gm.graph.call_function(
+                    glu_linear_wrapper, (gate[0], gate[1], gate[2], value[1], value[2], gate[3])
+                )
+            fused.meta = dict(node.meta)
+            node.replace_all_uses_with(fused)
+            gm.graph.erase_node(node)
+            gm.graph.erase_node(gate_n)
+            gm.graph.erase_node(value_n)
+            changed = True
+            break
+    if changed:
+        gm.graph.lint()
+        gm.recompile()
+
+
 def replace_all_linear(gm: torch.fx.GraphModule):
     replace_linear_activation(gm, torch.nn.Tanh(), "tanh")
     replace_linear_activation(gm, torch.nn.ReLU(), "relu")
@@ -219,4 +305,5 @@ def replace_all_linear(gm: torch.fx.GraphModule):
     replace_linear(gm)
     replace_linear_fn(gm)
     replace_linear_fn_constant_match(gm)
+    fuse_gated_linears(gm)
     fuse_sibling_linears(gm)

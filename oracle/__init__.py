@@ -9,6 +9,7 @@ from oracle.ops import (  # noqa: F401
     attention_oracle,
     attention_tiled_oracle,
     effective_eps,
+    glu_oracle,
     layer_norm_oracle,
     layer_norm_welford_oracle,
     linear_oracle,

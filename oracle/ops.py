@@ -19,6 +19,8 @@ How each function is pinned (tests/test_oracle.py):
   layer_norm_welford_oracle equals layer_norm_oracle to fp32 rounding for N in {128 .. 4096 .. 5000}
   rms_norm_oracle         x * rsqrt(mean(x^2)+eps) * w closed form; constant-row known answer
   effective_eps           code reading only (layer_norm.py:295-296)
+  glu_oracle              (a*sigmoid(a))*b written out as in the reference kernel vs F.silu(F.linear)*F.linear; gate = 0
+                          gives 0, value weights = 0 with unit bias gives act(gate)
   rotary_oracle           equals rotary_complex_oracle (the reference's complex product) under the even/odd <-> half
                           permutation; zero angle = identity; angles add; quarter turn of a unit vector; norms kept
   rotary_complex_oracle   torch.view_as_complex product as in the reference; pinned by the same known answers
@@ -177,6 +179,21 @@ def linear_oracle(
 # ------------------------------------------------------------------------------------------------------------------
 # layer norm
 # ------------------------------------------------------------------------------------------------------------------
+def glu_oracle(
+    x: torch.Tensor,
+    w_gate: torch.Tensor,
+    b_gate: Optional[torch.Tensor],
+    w_value: torch.Tensor,
+    b_value: Optional[torch.Tensor],
+    activation: str = "silu",
+) -> torch.Tensor:
+    """act(x·w_gateᵀ + b_gate) * (x·w_valueᵀ + b_value) in fp32: the product the reference's fused feed-forward
+    forms from its two accumulators, `(acc1 * sigmoid(acc1)) * acc2`
+    (experimental/llama-v2/kernel/fused_kernel_ff.py:36-75, eager form llama/model.py `FeedForward.forward`)."""
+    gate = linear_oracle(x, w_gate, b_gate, activation)
+    return gate * linear_oracle(x, w_value, b_value, "")
+
+
 def effective_eps(eps: float, dtype: torch.dtype) -> float:
     """eps the reference actually uses: clamped to >= 1.6e-5 for fp16 inputs (implementations/layer_norm.py:295-296)."""
     return max(eps, 1.6e-5) if dtype == torch.float16 else eps

@@ -298,8 +298,10 @@ def test_rms_norm_and_swiglu_patterns():
     assert t.count("layer_norm_rms_wrapper") == 1 and "rsqrt" not in t and "pow" not in t
     rms = next(n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "layer_norm_rms_wrapper")
     assert rms.args[2] == 1e-05
-    acts = sorted(n.kwargs.get("activation", "") for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "linear_wrapper_functional")
-    assert acts == ["", "silu"]
+    # silu(linear) * linear on the same input with graph-input weights: one gated GEMM
+    glu = [n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "glu_linear_wrapper"]
+    assert len(glu) == 1 and glu[0].args[5] == "silu" and "linear_wrapper_functional" not in t and "mul" not in t
+    assert glu[0].args[1].name == "gate_w" and glu[0].args[3].name == "up_w"
 
 
 def test_llama_graph_rewrite_and_constant_causal_mask():
@@ -331,6 +333,8 @@ def test_llama_graph_rewrite_and_constant_causal_mask():
         assert t.count(fused) == 2
         assert t.count("layer_norm_rms_wrapper") == 2 * 2 + 1 and "rsqrt" not in t
         assert t.count("fused_linear_wrapper") == 2 and "silu" not in t and "softmax" not in t
+        # SwiGLU: gate and up projections and their product are one gated GEMM per layer
+        assert t.count("glu_linear_wrapper") == 2 and t.count("linear_wrapper_functional") == 2 * 2
         # rotary embedding: one fused call each for queries and keys per layer, nothing left of rotate_half
         assert t.count("rotary_wrapper") == 2 * 2 and "neg" not in t
         # the fresh key/value cache no longer copies: the only cat left builds the angle table
@@ -397,3 +401,48 @@ def test_rotary_pass_only_fires_on_a_mid_split():
             n.meta["example_value"] = torch.empty(1, 2, 4, 8)
     fuse_rotary_embedding(gm)
     assert "rotary_wrapper" not in _targets(gm)
+
+
+def test_glu_row_interleaving_and_pass():
+    from kernl_amd.implementations.linear_layer import interleave_glu_rows
+    from kernl_amd.optimizer.linear import replace_all_linear
+    F = torch.nn.functional
+
+    gate = torch.arange(96 * 3).reshape(96, 3)
+    value = -torch.arange(96 * 3).reshape(96, 3)
+    w = interleave_glu_rows(gate, value)
+    assert w.shape == (192, 3)
+    for b in range(3):
+        assert torch.equal(w[64 * b: 64 * b + 32], gate[32 * b: 32 * b + 32])
+        assert torch.equal(w[64 * b + 32: 64 * b + 64], value[32 * b: 32 * b + 32])
+    assert torch.equal(interleave_glu_rows(gate[:, 0], value[:, 0]), w[:, 0])
+
+    class Mlp(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.g, self.u, self.d = torch.nn.Linear(8, 32, bias=False), torch.nn.Linear(8, 32, bias=False), torch.nn.Linear(32, 8, bias=False)
+
+        def forward(self, x):
+            gate = F.silu(F.linear(x, self.g.weight, None))
+            up = F.linear(x, self.u.weight, None)
+            return F.linear(gate * up, self.d.weight, None)
+
+    gm = torch.fx.symbolic_trace(Mlp())
+    replace_all_linear(gm)
+    t = _targets(gm)
+    assert t.count("glu_linear_wrapper") == 1 and t.count("linear_wrapper_functional") == 1 and "mul" not in t
+    glu = next(n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "glu_linear_wrapper")
+    assert glu.args[1].target == "g.weight" and glu.args[3].target == "u.weight" and glu.args[5] == "silu"
+
+    class Shared(torch.nn.Module):  # the gate is also used elsewhere: must stay
+        def __init__(self):
+            super().__init__()
+            self.g, self.u = torch.nn.Linear(8, 32, bias=False), torch.nn.Linear(8, 32, bias=False)
+
+        def forward(self, x):
+            gate = F.silu(F.linear(x, self.g.weight, None))
+            return gate * F.linear(x, self.u.weight, None), gate
+
+    gm = torch.fx.symbolic_trace(Shared())
+    replace_all_linear(gm)
+    assert "glu_linear_wrapper" not in _targets(gm)

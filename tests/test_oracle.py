@@ -14,6 +14,7 @@ from oracle import (
     attention_oracle,
     attention_tiled_oracle,
     effective_eps,
+    glu_oracle,
     layer_norm_oracle,
     layer_norm_welford_oracle,
     linear_oracle,
@@ -250,3 +251,23 @@ def test_rotary_known_answers():
     out = rotary_oracle(x, *_tables(a))
     pair_norm = lambda t: t[..., : D // 2] ** 2 + t[..., D // 2:] ** 2
     assert torch.allclose(pair_norm(out), pair_norm(x), atol=1e-5)
+
+
+def test_glu_closed_form_and_known_answers():
+    gen = torch.Generator().manual_seed(4)
+    x = torch.randn((9, 24), generator=gen)
+    wg, wv = torch.randn((16, 24), generator=gen), torch.randn((16, 24), generator=gen)
+    bg, bv = torch.randn((16,), generator=gen), torch.randn((16,), generator=gen)
+    F = torch.nn.functional
+    out = glu_oracle(x, wg, bg, wv, bv, "silu")
+    assert torch.allclose(out, F.silu(F.linear(x, wg, bg)) * F.linear(x, wv, bv), atol=1e-5, rtol=1e-5)
+    a, b = x @ wg.T + bg, x @ wv.T + bv  # the two accumulators of the reference kernel
+    assert torch.allclose(out, (a * torch.sigmoid(a)) * b, atol=1e-5, rtol=1e-5)
+    assert torch.allclose(glu_oracle(x, wg, None, wv, None, "fast_gelu"),
+                          F.gelu(F.linear(x, wg), approximate="tanh") * F.linear(x, wv), atol=1e-5, rtol=1e-5)
+    # a zero gate silences the unit; a constant value of one leaves act(gate)
+    assert torch.equal(glu_oracle(x, torch.zeros_like(wg), None, wv, bv, "silu"), torch.zeros((9, 16)))
+    ones = glu_oracle(x, wg, bg, torch.zeros_like(wv), torch.ones_like(bv), "silu")
+    assert torch.allclose(ones, F.silu(F.linear(x, wg, bg)), atol=1e-6)
+    # gate and value are not interchangeable
+    assert not torch.allclose(out, glu_oracle(x, wv, bv, wg, bg, "silu"), atol=1e-3)
