@@ -372,9 +372,9 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 // Per 16-wide k-step a wave runs 16 MFMAs on 8 operand fragments — half the LDS traffic per MFMA of the 8-wave
 // kernel above.  Operand tiles go HBM -> LDS directly (buffer loads with the LDS flag), two 64 KB stages.  With a
 // single wave per SIMD nothing else can fill a stall, so the instruction stream is laid out by hand: every MFMA
-// is followed by at most one LDS read or one tile load, and the barrier that publishes the next k-tile sits in
-// front of the LAST k-step's MFMAs, whose operands are already in registers — the matrix pipe stays busy while
-// the first fragments of the next tile are fetched.
+// is followed by at most one LDS read or one tile load (both issue in the shadow of the MFMA), fragments are read
+// two k-steps ahead, and the one barrier per k-tile sits in front of k-step 2, after which the stage just consumed
+// takes the next-but-one k-tile.
 // ----------------------------------------------------------------------------------------------------
 template <typename T, int ACT>
 __global__ void __launch_bounds__(256, 1)
@@ -481,36 +481,43 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): all of tile 0 has landed, tile 1 may still be in flight
     __syncthreads();
 
-    vec8 fa[2][TN], fb[2][TM];
+    // Fragments are fetched TWO k-steps ahead into four register sets (set = k-step): the last reads of a stage are
+    // then issued during k-step 1 of its tile, the barrier sits in front of k-step 2, and the stage can take the loads
+    // of k-tile kt + 2 during k-steps 2 and 3, one load every other MFMA.  A burst of 16 loads in one k-step followed
+    // by a wait for all of them stalls a lone wave: 64 KB need >= 1024 cycles to pass the CU's 64 B/clk fill path.
+    vec8 fa[4][TN], fb[4][TM];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fa[0][j] = *reinterpret_cast<const vec8 *>(smem + woff[0][j]);
+    for (int st = 0; st < 2; ++st) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) fb[0][i] = *reinterpret_cast<const vec8 *>(smem + xoff[0][i]);
+        for (int j = 0; j < TN; ++j) fa[st][j] = *reinterpret_cast<const vec8 *>(smem + woff[st][j]);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fb[st][i] = *reinterpret_cast<const vec8 *>(smem + xoff[st][i]);
+    }
 
     // one k-tile held in stage CUR (a compile-time constant, so that stage offsets fold into instruction offsets)
-    auto k_tile = [&](auto cur_c, int kt) {
+    auto k_tile = [&](auto cur_c, int kt) __attribute__((always_inline)) {
         constexpr int CUR = decltype(cur_c)::value;
         const unsigned char *cur = smem + CUR * STAGE;
         const unsigned char *nxt = smem + (CUR ^ 1) * STAGE;
 #pragma unroll
         for (int st = 0; st < KSTEPS; ++st) {
-            const int ob = st & 1, nb = ob ^ 1;
-            // fragments to fetch during this step: those of the next step — for the last step, step 0 of the next
-            // k-tile, which is why the barrier publishing that tile comes first
-            const unsigned char *src = (st + 1 < KSTEPS) ? cur : nxt;
-            const int sn = (st + 1) % KSTEPS;
-            if (st == KSTEPS - 1) {
-                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads of the next k-tile have landed
-                __syncthreads();
+            const int sn = (st + 2) % KSTEPS;                       // k-step whose fragments are fetched now
+            const unsigned char *src = (st + 2 < KSTEPS) ? cur : nxt;
+            if (st == 2) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads of k-tile kt + 1 have landed
+                __syncthreads();                     // ... everyone's have, and nobody reads stage CUR any more
             }
 #pragma unroll
             for (int m = 0; m < TM * TN; ++m) {
                 const int i = m / TN, j = m % TN;
-                acc[i][j] = mfma32(fa[ob][j], fb[ob][i], acc[i][j]);
-                if (m < TN) fa[nb][m] = *reinterpret_cast<const vec8 *>(src + woff[sn][m]);
-                else if (m < TN + TM) fb[nb][m - TN] = *reinterpret_cast<const vec8 *>(src + xoff[sn][m - TN]);
-                // tile kt + 2 goes into the stage every wave has just finished reading, one load behind each MFMA
-                if (st == KSTEPS - 1) tile_load(m, CUR, (kt + 2) * BK);
+                acc[i][j] = mfma32(fa[st][j], fb[st][i], acc[i][j]);
+                if ((m & 1) == 0) {
+                    const int r = m >> 1;
+                    if (r < TN) fa[sn][r] = *reinterpret_cast<const vec8 *>(src + woff[sn][r]);
+                    else fb[sn][r - TN] = *reinterpret_cast<const vec8 *>(src + xoff[sn][r - TN]);
+                } else if (st >= 2) {
+                    tile_load((st - 2) * 8 + (m >> 1), CUR, (kt + 2) * BK);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }

@@ -43,7 +43,8 @@ def test_linear_vs_oracle(shape, bias, activation, dtype, close):
 
 @pytest.mark.parametrize("tile", [1, 2, 3, 4, 5], ids=["256x256", "256x192", "128x128", "256x128k32", "wide256x256"])
 @pytest.mark.parametrize(
-    "shape", [(1000, 600, 776), (256, 256, 64), (513, 385, 1032), (700, 520, 1024)], ids=lambda s: "x".join(map(str, s))
+    "shape", [(1000, 600, 776), (256, 256, 64), (513, 385, 1032), (700, 520, 1024), (300, 260, 32), (257, 513, 96), (640, 512, 160)],
+    ids=lambda s: "x".join(map(str, s))
 )
 def test_linear_every_tile_shape(shape, tile, close):
     M, N, K = shape
