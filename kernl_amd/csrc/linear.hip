@@ -72,50 +72,93 @@ __device__ __forceinline__ float apply_act(float x, int act) {
 // ----------------------------------------------------------------------------------------------------
 static constexpr int kGluBit = 8;
 
-template <typename T, int ACT, int TM, int TN>
+// Bias of a wave's TN column blocks as packed 16-bit values: raw[j] holds the 16 consecutive entries starting at
+// n_wave + 32 j + 16 lh.  Fetched ONCE per tile and ahead of time: with one or two waves per SIMD a load issued where
+// its value is needed stalls the whole epilogue for a memory round trip.
+template <typename T, int TN>
+__device__ __forceinline__ void bias_fetch(const T *__restrict__ bias, int n_wave, int lh, int N, int bias_vec_ok,
+                                           u32x4 (&raw)[TN][2]) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int n = n_wave + j * 32 + lh * 16;
+        if (bias == nullptr) {
+            raw[j][0] = u32x4{0, 0, 0, 0};
+            raw[j][1] = u32x4{0, 0, 0, 0};
+        } else if (bias_vec_ok && n + 16 <= N) {
+            raw[j][0] = *reinterpret_cast<const u32x4 *>(bias + n);
+            raw[j][1] = *reinterpret_cast<const u32x4 *>(bias + n + 8);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; v += 2) {
+                const uint32_t lo = n + v < N ? (uint32_t)__builtin_bit_cast(uint16_t, bias[n + v]) : 0u;
+                const uint32_t hi = n + v + 1 < N ? (uint32_t)__builtin_bit_cast(uint16_t, bias[n + v + 1]) : 0u;
+                raw[j][v >> 3][(v & 7) >> 1] = lo | (hi << 16);
+            }
+        }
+    }
+}
+template <typename T>
+__device__ __forceinline__ float bias_elem(const u32x4 (&raw)[2], int v) {
+    const uint32_t word = raw[v >> 3][(v & 7) >> 1];
+    const uint16_t bits = (uint16_t)((v & 1) ? (word >> 16) : (word & 0xFFFFu));
+    return to_float(__builtin_bit_cast(T, bits));
+}
+
+// ROW0 / ROWS select the 32-row blocks handled by one call (the wide kernel calls once per block so that each call
+// unrolls completely).  Waves whose blocks lie inside the matrix and whose output rows take 16-byte stores run a
+// straight-line path; edge tiles, strided outputs and the pre-activation side output run the general one.
+template <typename T, int ACT, int TM, int TN, int ROW0 = 0, int ROWS = TM>
 __device__ __forceinline__ void linear_epilogue(f32x16 (&acc)[TM][TN], int m_wave, int n_wave, int lr, int lh,
                                                 const T *__restrict__ bias, T *__restrict__ out,
                                                 T *__restrict__ act_in, int M, int N, int64_t out_rs, int64_t out_cs,
                                                 int64_t ai_rs, int64_t ai_cs, int out_vec_ok, int ai_vec_ok,
-                                                int bias_vec_ok) {
-    typedef typename Vec8<T>::type vec8;
+                                                int bias_vec_ok, const u32x4 (&braw)[TN][2]) {
+    auto store16 = [&](T *p, const float (&r)[16]) __attribute__((always_inline)) {
+        u32x4 p0, p1;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
+            p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
+        }
+        *reinterpret_cast<u32x4 *>(p) = p0;
+        *reinterpret_cast<u32x4 *>(p + 8) = p1;
+    };
+    const bool rows_inside = m_wave + (ROW0 + ROWS) * 32 <= M;
     if constexpr ((ACT & kGluBit) != 0) {
         static_assert(TN % 2 == 0, "gated epilogue pairs neighbouring 32-column blocks");
         constexpr int BASE = ACT & (kGluBit - 1);
         const int n_total = N >> 1;
+        const bool interior = rows_inside && (n_wave >> 1) + TN * 16 <= n_total && out_vec_ok;
+        if (__builtin_amdgcn_readfirstlane((int)interior)) {
+#pragma unroll
+            for (int pr = 0; pr < TN / 2; ++pr) {
+                T *col = out + (int64_t)(m_wave + lr) * out_rs + (n_wave >> 1) + pr * 32 + lh * 16;
+#pragma unroll
+                for (int i = ROW0; i < ROW0 + ROWS; ++i) {
+                    float r[16];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        r[v] = apply_act(acc[i][2 * pr][v] + bias_elem<T>(braw[2 * pr], v), BASE) *
+                               (acc[i][2 * pr + 1][v] + bias_elem<T>(braw[2 * pr + 1], v));
+                    store16(col + (int64_t)(i * 32) * out_rs, r);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int pr = 0; pr < TN / 2; ++pr) {
             const int n = (n_wave >> 1) + pr * 32 + lh * 16;         // output column
-            const int nb = n_wave + pr * 64 + lh * 16;               // interleaved row of the gate bias
-            float bg[16], bu[16];
-            if (bias != nullptr && n < n_total) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    bg[v] = to_float(bias[nb + v]);
-                    bu[v] = to_float(bias[nb + 32 + v]);
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
+            for (int i = ROW0; i < ROW0 + ROWS; ++i) {
                 const int m = m_wave + i * 32 + lr;
                 if (m >= M || n >= n_total) continue;  // n_total is a multiple of 32: a block is in or out as a whole
                 float r[16];
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const float g = bias != nullptr ? acc[i][2 * pr][v] + bg[v] : acc[i][2 * pr][v];
-                    const float u = bias != nullptr ? acc[i][2 * pr + 1][v] + bu[v] : acc[i][2 * pr + 1][v];
-                    r[v] = apply_act(g, BASE) * u;
-                }
+                for (int v = 0; v < 16; ++v)
+                    r[v] = apply_act(acc[i][2 * pr][v] + bias_elem<T>(braw[2 * pr], v), BASE) *
+                           (acc[i][2 * pr + 1][v] + bias_elem<T>(braw[2 * pr + 1], v));
                 if (out_vec_ok) {
-                    u32x4 p0, p1;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
-                        p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
-                    }
-                    T *p = out + (int64_t)m * out_rs + n;
-                    *reinterpret_cast<u32x4 *>(p) = p0;
-                    *reinterpret_cast<u32x4 *>(p + 8) = p1;
+                    store16(out + (int64_t)m * out_rs + n, r);
                 } else {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
@@ -124,43 +167,35 @@ __device__ __forceinline__ void linear_epilogue(f32x16 (&acc)[TM][TN], int m_wav
         }
         return;
     }
-    const bool HAS_BIAS = bias != nullptr, SAVE_ACT_IN = act_in != nullptr;
+    const bool interior = rows_inside && n_wave + TN * 32 <= N && out_vec_ok && act_in == nullptr;
+    if (__builtin_amdgcn_readfirstlane((int)interior)) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            T *col = out + (int64_t)(m_wave + lr) * out_rs + n_wave + j * 32 + lh * 16;
+#pragma unroll
+            for (int i = ROW0; i < ROW0 + ROWS; ++i) {
+                float r[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) r[v] = apply_act(acc[i][j][v] + bias_elem<T>(braw[j], v), ACT);
+                store16(col + (int64_t)(i * 32) * out_rs, r);
+            }
+        }
+        return;
+    }
+    const bool SAVE_ACT_IN = act_in != nullptr;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int n = n_wave + j * 32 + lh * 16;
-        float bv[16];
-        if (HAS_BIAS) {
-            if (bias_vec_ok && n + 16 <= N) {
-                const vec8 b0 = *reinterpret_cast<const vec8 *>(bias + n);
-                const vec8 b1 = *reinterpret_cast<const vec8 *>(bias + n + 8);
 #pragma unroll
-                for (int v = 0; v < 8; ++v) {
-                    bv[v] = to_float(b0[v]);
-                    bv[8 + v] = to_float(b1[v]);
-                }
-            } else {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) bv[v] = (n + v < N) ? to_float(bias[n + v]) : 0.0f;
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
+        for (int i = ROW0; i < ROW0 + ROWS; ++i) {
             const int m = m_wave + i * 32 + lr;
             if (m >= M || n >= N) continue;
             float r[16];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) r[v] = HAS_BIAS ? acc[i][j][v] + bv[v] : acc[i][j][v];
+            for (int v = 0; v < 16; ++v) r[v] = acc[i][j][v] + bias_elem<T>(braw[j], v);  // zeros without a bias
             if (SAVE_ACT_IN) {
                 if (ai_vec_ok && n + 16 <= N) {
-                    u32x4 p0, p1;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
-                        p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
-                    }
-                    T *p = act_in + (int64_t)m * ai_rs + n;
-                    *reinterpret_cast<u32x4 *>(p) = p0;
-                    *reinterpret_cast<u32x4 *>(p + 8) = p1;
+                    store16(act_in + (int64_t)m * ai_rs + n, r);
                 } else {
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
@@ -170,15 +205,7 @@ __device__ __forceinline__ void linear_epilogue(f32x16 (&acc)[TM][TN], int m_wav
 #pragma unroll
             for (int v = 0; v < 16; ++v) r[v] = apply_act(r[v], ACT);
             if (out_vec_ok && n + 16 <= N) {
-                u32x4 p0, p1;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
-                    p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
-                }
-                T *p = out + (int64_t)m * out_rs + n;
-                *reinterpret_cast<u32x4 *>(p) = p0;
-                *reinterpret_cast<u32x4 *>(p + 8) = p1;
+                store16(out + (int64_t)m * out_rs + n, r);
             } else {
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
@@ -307,6 +334,11 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     };
 
     f32x16 acc[TM][TN];
+    // this wave's bias entries: in flight during the main loop where the tile shape leaves registers for them,
+    // fetched in one go after it otherwise
+    constexpr bool EARLY_BIAS = BM * BN < 256 * 256;
+    u32x4 braw[TN][2];
+    if (EARLY_BIAS) bias_fetch<T, TN>(bias, n0 + wave_n * Cfg::WN, lh, N, bias_vec_ok, braw);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -362,8 +394,9 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         __syncthreads();
     }
 
+    if (!EARLY_BIAS) bias_fetch<T, TN>(bias, n0 + wave_n * Cfg::WN, lh, N, bias_vec_ok, braw);
     linear_epilogue<T, ACT, TM, TN>(acc, m0 + wave_m * Cfg::WM, n0 + wave_n * Cfg::WN, lr, lh, bias, out, act_in, M, N, out_rs,
-                                    out_cs, ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bias_vec_ok);
+                                    out_cs, ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bias_vec_ok, braw);
 }
 
 // ----------------------------------------------------------------------------------------------------
@@ -529,12 +562,14 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     }
     if (kt < nk) k_tile(IntC<0>(), kt);
 
+    // all bias entries of the wave's 128 columns in one go: one memory round trip per tile instead of one per block
+    u32x4 braw[TN][2];
+    bias_fetch<T, TN>(bias, n0 + wave_n * 128, lh, N, bias_vec_ok, braw);
     // one call per 32-row block: each stays small enough for the compiler to unroll completely, so the accumulators
     // are only ever indexed by constants and never leave the register file
 #define KERNL_WIDE_EPILOGUE(I)                                                                                          \
-    linear_epilogue<T, ACT, 1, TN>(*reinterpret_cast<f32x16(*)[1][TN]>(&acc[I]), m0 + wave_m * 128 + 32 * (I),          \
-                                   n0 + wave_n * 128, lr, lh, bias, out, act_in, M, N, out_rs, out_cs, ai_rs, ai_cs,    \
-                                   out_vec_ok, ai_vec_ok, bias_vec_ok)
+    linear_epilogue<T, ACT, TM, TN, I, 1>(acc, m0 + wave_m * 128, n0 + wave_n * 128, lr, lh, bias, out, act_in, M, N,    \
+                                          out_rs, out_cs, ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bias_vec_ok, braw)
     KERNL_WIDE_EPILOGUE(0);
     KERNL_WIDE_EPILOGUE(1);
     KERNL_WIDE_EPILOGUE(2);
@@ -703,14 +738,26 @@ typedef LinearTile<256, 192, 64, 4, 2, 1> Tile256x192;
 typedef LinearTile<128, 128, 64, 2, 2, 2> Tile128x128;
 typedef LinearTile<256, 128, 32, 2, 2, 2> Tile256x128k32;  // 48 KB of LDS: two workgroups per CU
 
-// Number of "rounds" a tile shape needs on 256 CUs times the work of one tile: a proxy for run time.
-static double tile_cost(int M, int N, int bm, int bn, int blocks_per_cu) {
+// Run-time proxy of a tile shape: tiles one CU has to work through, times the tile's area relative to 256x256, times
+// a speed factor of the kernel that runs it (measured on the Llama-7B and BERT-base shapes: the wide kernel's k-loop is
+// the fastest, and the longer K is the more the 8-wave kernels fall behind it).
+static double tile_cost(int M, int N, int K, int bm, int bn, double base, double per_k) {
     const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-    const int64_t slots = 256 * blocks_per_cu;
-    const int64_t rounds = (tiles + slots - 1) / slots;
-    // larger tiles move fewer operand bytes per flop; weigh that in mildly.
-    const double eff = 1.0 / (1.0 + 48.0 / bm + 48.0 / bn);
-    return (double)rounds * bm * bn * blocks_per_cu / eff;
+    const int64_t per_cu = (tiles + 255) / 256;
+    const double kf = (double)K / ((double)K + 1500.0);
+    return (double)per_cu * ((double)bm * bn / 65536.0) * (base + per_k * kf);
+}
+// which: 1 = 256x256, 2 = 256x192, 3 = 128x128 (8-wave kernel), 5 = wide 256x256 (needs K % 64 == 0)
+static int pick_tile(int M, int N, int K, bool gated) {
+    int pick = 1;
+    double best = tile_cost(M, N, K, 256, 256, 1.15, 0.3);
+    if (K % 64 == 0) { best = tile_cost(M, N, K, 256, 256, 1.0, 0.0); pick = 5; }
+    // 256x192 gives a wave an odd number of column blocks: not usable for gate/value pairs
+    const double c2 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.2, 0.3);
+    const double c3 = tile_cost(M, N, K, 128, 128, 1.9, 0.4);
+    if (c2 < best) { best = c2; pick = 2; }
+    if (c3 < best) { best = c3; pick = 3; }
+    return pick;
 }
 
 int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256
@@ -718,30 +765,12 @@ int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256,
 template <typename T>
 static int linear_mfma_dispatch(const LinearArgs &a) {
     int pick = g_linear_force_tile;
+    if (pick == 0) pick = pick_tile(a.M, a.N, a.K, (a.act & kGluBit) != 0);
     if (a.act & kGluBit) {
-        // tiles 256x192 and 256x128 give a wave an odd number of column blocks: not usable for gate/value pairs
-        const int64_t tiles256 = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
-        if (pick == 0) {
-            pick = tile_cost(a.M, a.N, 128, 128, 2) < tile_cost(a.M, a.N, 256, 256, 1) ? 3 : 1;
-            if (pick == 1 && a.K % 64 == 0 && a.K >= 4096 && tiles256 >= 512) pick = 5;
-        }
         if (pick == 5 && a.K % 64 == 0) launch_wide<T>(a);
         else if (pick == 3) launch_mfma_glu<T, Tile128x128>(a);
         else launch_mfma_glu<T, Tile256x256>(a);
         return check_launch("gated linear (mfma)");
-    }
-    if (pick == 0) {
-        const double c1 = tile_cost(a.M, a.N, 256, 256, 1);
-        const double c2 = tile_cost(a.M, a.N, 256, 192, 1);
-        const double c3 = tile_cost(a.M, a.N, 128, 128, 2);
-        pick = 1;
-        double best = c1;
-        if (c2 < best) { best = c2; pick = 2; }
-        if (c3 < best) { best = c3; pick = 3; }
-        // long k-loops over many full tiles with a cheap epilogue: one wave per SIMD with a 128x128 sub-tile
-        const int64_t tiles256 = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
-        if (pick == 1 && a.K % 64 == 0 && a.K >= 4096 && tiles256 >= 512 && (a.act == KERNL_ACT_NONE || a.act == KERNL_ACT_RELU))
-            pick = 5;
     }
     if (pick == 5 && a.K % 64 == 0) launch_wide<T>(a);
     else if (pick == 1) launch_mfma_cfg<T, Tile256x256>(a);
