@@ -60,6 +60,28 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
+// D[16x16] += A[16x32] * B[32x16], fp32 accumulate (v_mfma_f32_16x16x32_{f16,bf16}, 4 passes).  Same flops per cycle
+// as the 32x32x16 form with a quarter of the accumulator traffic per flop: under the board's power limit it sustains
+// a higher clock.  Lane l: A holds row (l % 16), k = 8*(l/16) .. +7; B holds column (l % 16), same k range; D element
+// e (0..3) of lane l is row 4*(l/16) + e, column (l % 16).
+typedef float f32x4_acc __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4_acc mfma16(f16x8 a, f16x8 b, f32x4_acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4_acc mfma16(bf16x8 a, bf16x8 b, f32x4_acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// The same instruction with the accumulator pinned to the accumulation registers and updated in place.  With 64
+// four-register accumulators per wave the register allocator otherwise migrates some of them to ordinary registers and
+// copies them back at the loop head.
+__device__ __forceinline__ void mfma16_inplace(f16x8 a, f16x8 b, f32x4_acc &c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma16_inplace(bf16x8 a, bf16x8 b, f32x4_acc &c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
 // Because of the D layout above, feeding MFMA row i with logical row rowperm16(i) makes every lane end up
 // with 16 CONSECUTIVE logical rows: lane half h holds logical rows 16*h + v for v = 0..15.
 __device__ __forceinline__ int rowperm16(int i) { return 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3); }

@@ -400,15 +400,120 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 }
 
 // ----------------------------------------------------------------------------------------------------
-// Wide MFMA kernel for K % 64 == 0: 256x256 output tile, 4 waves, ONE wave per SIMD owning a 128x128 sub-tile
-// (16 accumulator blocks = 256 registers, which the compiler keeps in the accumulation half of the register file).
-// Per 16-wide k-step a wave runs 16 MFMAs on 8 operand fragments — half the LDS traffic per MFMA of the 8-wave
+// Wide MFMA kernel for K % 64 == 0: 256x256 output tile, 4 waves, ONE wave per SIMD owning a 128x128 sub-tile as
+// 8x8 blocks of v_mfma_f32_16x16x32 (256 accumulator registers, kept in the accumulation half of the register file).
+// Per 32-wide k-step a wave runs 64 MFMAs on 16 operand fragments — half the LDS traffic per flop of the 8-wave
 // kernel above.  Operand tiles go HBM -> LDS directly (buffer loads with the LDS flag), two 64 KB stages.  With a
-// single wave per SIMD nothing else can fill a stall, so the instruction stream is laid out by hand: every MFMA
-// is followed by at most one LDS read or one tile load (both issue in the shadow of the MFMA), fragments are read
-// two k-steps ahead, and the one barrier per k-tile sits in front of k-step 2, after which the stage just consumed
-// takes the next-but-one k-tile.
+// single wave per SIMD nothing else can fill a stall, so the instruction stream is laid out by hand: LDS reads and
+// tile loads issue in the shadow of the MFMAs (at most one every other MFMA), fragments are read one k-step (64
+// MFMAs) ahead, and the one barrier per k-tile sits in front of its second k-step, after which the stage just
+// consumed takes the next-but-one k-tile, one load every fourth MFMA.  (A burst of 16 loads followed by a wait for
+// all of them stalls a lone wave: 64 KB need >= 1024 cycles to pass the CU's 64 B/clk fill path.)
+//
+// Weight rows are placed in LDS so that a lane ends up with consecutive output columns: MFMA row r of block j in a
+// 64-row group carries weight row 16 (r/4) + 4 j + r%4, so lane group g = lane/16 holds the 16 columns 16 g .. 16 g+15
+// of the group across its four blocks.  Gated epilogues use 32 (j/2) + 8 (r/4) + 4 (j%2) + r%4 instead: the lane holds
+// gate AND value of the 8 output columns 8 g .. 8 g + 7.
 // ----------------------------------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ u32x4 fetch8(const T *__restrict__ p, int idx, int limit, int vec_ok) {
+    u32x4 r = {0, 0, 0, 0};
+    if (p == nullptr) return r;
+    if (vec_ok && idx + 8 <= limit) return *reinterpret_cast<const u32x4 *>(p + idx);
+#pragma unroll
+    for (int v = 0; v < 8; v += 2) {
+        const uint32_t lo = idx + v < limit ? (uint32_t)__builtin_bit_cast(uint16_t, p[idx + v]) : 0u;
+        const uint32_t hi = idx + v + 1 < limit ? (uint32_t)__builtin_bit_cast(uint16_t, p[idx + v + 1]) : 0u;
+        r[v >> 1] = lo | (hi << 16);
+    }
+    return r;
+}
+
+// Epilogue of m-block IB (16 rows) of a wave of the wide kernel: lane (l16, g) holds row m_wave + 16 IB + l16.
+template <typename T, int ACT, int IB>
+__device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[8][8], int m_wave, int n_wave, int l16, int g,
+                                              T *__restrict__ out, T *__restrict__ act_in, int M, int N,
+                                              int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs,
+                                              int out_vec_ok, int ai_vec_ok, const u32x4 (&braw)[2][2]) {
+    const int m = m_wave + 16 * IB + l16;
+    const bool rows_inside = m_wave + 16 * IB + 16 <= M;
+    if constexpr ((ACT & kGluBit) != 0) {
+        constexpr int BASE = ACT & (kGluBit - 1);
+        const int n_total = N >> 1;
+        const bool interior = rows_inside && (n_wave >> 1) + 64 <= n_total && out_vec_ok;
+        const bool fast = __builtin_amdgcn_readfirstlane((int)interior) != 0;
+#pragma unroll
+        for (int G = 0; G < 2; ++G) {
+            const int n = (n_wave >> 1) + 32 * G + 8 * g;  // 8 consecutive output columns
+            if (!fast && (m >= M || n >= n_total)) continue;  // n_total is a multiple of 32 and n of 8
+            float r[8];
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const float gate = acc[IB][4 * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v);
+                const float value = acc[IB][4 * G + 2 + (v >> 2)][v & 3] + bias_elem<T>(braw[G], 8 + v);
+                r[v] = apply_act(gate, BASE) * value;
+            }
+            if (fast || out_vec_ok) {
+                u32x4 p;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) p[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
+                *reinterpret_cast<u32x4 *>(out + (int64_t)m * out_rs + n) = p;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 8; ++v) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
+            }
+        }
+        return;
+    }
+    auto store16 = [&](T *p, const float (&r)[16]) __attribute__((always_inline)) {
+        u32x4 p0, p1;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
+            p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
+        }
+        *reinterpret_cast<u32x4 *>(p) = p0;
+        *reinterpret_cast<u32x4 *>(p + 8) = p1;
+    };
+    const bool interior = rows_inside && n_wave + 128 <= N && out_vec_ok && act_in == nullptr;
+    if (__builtin_amdgcn_readfirstlane((int)interior)) {
+#pragma unroll
+        for (int G = 0; G < 2; ++G) {
+            float r[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) r[v] = apply_act(acc[IB][4 * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v), ACT);
+            store16(out + (int64_t)m * out_rs + n_wave + 64 * G + 16 * g, r);
+        }
+        return;
+    }
+#pragma unroll
+    for (int G = 0; G < 2; ++G) {
+        const int n = n_wave + 64 * G + 16 * g;
+        if (m >= M || n >= N) continue;
+        float r[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) r[v] = acc[IB][4 * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v);
+        if (act_in != nullptr) {
+            if (ai_vec_ok && n + 16 <= N) {
+                store16(act_in + (int64_t)m * ai_rs + n, r);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (n + v < N) act_in[(int64_t)m * ai_rs + (int64_t)(n + v) * ai_cs] = from_float<T>(r[v]);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) r[v] = apply_act(r[v], ACT);
+        if (out_vec_ok && n + 16 <= N) {
+            store16(out + (int64_t)m * out_rs + n, r);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                if (n + v < N) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
+        }
+    }
+}
+
 template <typename T, int ACT>
 __global__ void __launch_bounds__(256, 1)
 linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
@@ -416,7 +521,8 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
                    int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok, int ai_vec_ok,
                    int bias_vec_ok) {
     typedef typename Vec8<T>::type vec8;
-    constexpr int BM = 256, BN = 256, BK = 64, RB = BK * 2, CPR = BK / 8, TM = 4, TN = 4, KSTEPS = BK / 16;
+    constexpr bool GATED = (ACT & kGluBit) != 0;
+    constexpr int BM = 256, BN = 256, BK = 64, RB = BK * 2, CPR = BK / 8, NB = 8, KSTEPS = BK / 32;
     constexpr int X_BYTES = BM * RB, W_BYTES = BN * RB, STAGE = X_BYTES + W_BYTES;
     constexpr int LOADS = BM * CPR / 256;  // 1 KB loads per wave for each operand tile
     constexpr int GROUP_M = 4;
@@ -438,7 +544,7 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave & 1, wave_n = wave >> 1;
-    const int lr = lane & 31, lh = lane >> 5;
+    const int l16 = lane & 15, g = lane >> 4;
 
     // ---- tile loads: load i of a wave fills the 1 KB of 16-byte chunks [256 i + 64 wave, +64) of an operand tile;
     // every lane fetches the chunk that belongs at its LDS position under the swizzle.  Rows beyond M / N and
@@ -460,15 +566,17 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
         const uint32_t imm = (uint32_t)(i & 3) * 1024u;
         xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) - imm : kOutOfRange;
-        // LDS row `row` feeds MFMA row (row % 32) of its 32-block and carries weight row rowperm16(row % 32)
-        const int wrow = (row & ~31) + rowperm16(row & 31);
+        // LDS row `row` is MFMA row r = row % 16 of block j = (row % 64) / 16 of its 64-row group
+        const int r = row & 15, j = (row >> 4) & 3;
+        const int in_group64 = GATED ? 32 * (j >> 1) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3) : 16 * (r >> 2) + 4 * j + (r & 3);
+        const int wrow = (row & ~63) + in_group64;
         wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - imm : kOutOfRange;
     }
     typedef __attribute__((address_space(3))) void lds_void;
     const uint32_t dma_base = (uint32_t)(uintptr_t)(lds_void *)smem + wave * (LOADS * 1024);
     // inline assembly on purpose: the compiler would make every later LDS read wait for loads it sees writing LDS.
-    // `group` (0 or 1) selects loads 4 group .. 4 group + 3; `first` writes the LDS base register for the group.
-    auto load4 = [&](const u32x4 &rsrc, const uint32_t (&off)[LOADS], uint32_t lds, int group, int part, int k0) {
+    // `group` (0 or 1) selects loads 4 group .. 4 group + 3; its first load writes the LDS base register.
+    auto load4 = [&](const u32x4 &rsrc, const uint32_t (&off)[LOADS], uint32_t lds, int group, int part, int k0) __attribute__((always_inline)) {
         const int i = 4 * group + part;
         if (part == 0)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
@@ -481,28 +589,27 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
             asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off[i]), "s"(rsrc), "s"(k0 * 2) : "memory");
     };
     // load l (0..15) of a k-tile: X loads 0..7, then W loads 0..7
-    auto tile_load = [&](int l, int stage, int k0) {
+    auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
         if (l < LOADS) load4(xrsrc, xd, dma_base + stage * STAGE, l >> 2, l & 3, k0);
         else load4(wrsrc, wd, dma_base + stage * STAGE + X_BYTES, (l - LOADS) >> 2, l & 3, k0);
     };
 
-    f32x16 acc[TM][TN];
+    f32x4_acc acc[NB][NB];  // [m-block][n-block]
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        for (int j = 0; j < NB; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
 
     // LDS byte offsets of this lane's operand fragments, one register per (k-step, block): with a whole register
     // file per wave there is room to keep them all, and no address arithmetic is left in the loop
-    int xoff[KSTEPS][TM], woff[KSTEPS][TN];
+    int xoff[KSTEPS][NB], woff[KSTEPS][NB];
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) xoff[st][i] = swz_offset<RB>(wave_m * 128 + i * 32 + lr, 2 * st + lh);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) woff[st][j] = X_BYTES + swz_offset<RB>(wave_n * 128 + j * 32 + lr, 2 * st + lh);
+        for (int i = 0; i < NB; ++i) {
+            xoff[st][i] = swz_offset<RB>(wave_m * 128 + i * 16 + l16, 4 * st + g);
+            woff[st][i] = X_BYTES + swz_offset<RB>(wave_n * 128 + i * 16 + l16, 4 * st + g);
+        }
     }
 
     const int nk = K / BK;
@@ -514,18 +621,11 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): all of tile 0 has landed, tile 1 may still be in flight
     __syncthreads();
 
-    // Fragments are fetched TWO k-steps ahead into four register sets (set = k-step): the last reads of a stage are
-    // then issued during k-step 1 of its tile, the barrier sits in front of k-step 2, and the stage can take the loads
-    // of k-tile kt + 2 during k-steps 2 and 3, one load every other MFMA.  A burst of 16 loads in one k-step followed
-    // by a wait for all of them stalls a lone wave: 64 KB need >= 1024 cycles to pass the CU's 64 B/clk fill path.
-    vec8 fa[4][TN], fb[4][TM];
+    vec8 fa[KSTEPS][NB], fb[KSTEPS][NB];  // weight and activation fragments, one register set per k-step
 #pragma unroll
-    for (int st = 0; st < 2; ++st) {
+    for (int j = 0; j < NB; ++j) fa[0][j] = *reinterpret_cast<const vec8 *>(smem + woff[0][j]);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fa[st][j] = *reinterpret_cast<const vec8 *>(smem + woff[st][j]);
-#pragma unroll
-        for (int i = 0; i < TM; ++i) fb[st][i] = *reinterpret_cast<const vec8 *>(smem + xoff[st][i]);
-    }
+    for (int i = 0; i < NB; ++i) fb[0][i] = *reinterpret_cast<const vec8 *>(smem + xoff[0][i]);
 
     // one k-tile held in stage CUR (a compile-time constant, so that stage offsets fold into instruction offsets)
     auto k_tile = [&](auto cur_c, int kt) __attribute__((always_inline)) {
@@ -534,22 +634,22 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         const unsigned char *nxt = smem + (CUR ^ 1) * STAGE;
 #pragma unroll
         for (int st = 0; st < KSTEPS; ++st) {
-            const int sn = (st + 2) % KSTEPS;                       // k-step whose fragments are fetched now
-            const unsigned char *src = (st + 2 < KSTEPS) ? cur : nxt;
-            if (st == 2) {
+            const int sn = st ^ 1;                               // k-step whose fragments are fetched now
+            const unsigned char *src = st == 0 ? cur : nxt;
+            if (st == 1) {
                 __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads of k-tile kt + 1 have landed
                 __syncthreads();                     // ... everyone's have, and nobody reads stage CUR any more
             }
 #pragma unroll
-            for (int m = 0; m < TM * TN; ++m) {
-                const int i = m / TN, j = m % TN;
-                acc[i][j] = mfma32(fa[st][j], fb[st][i], acc[i][j]);
-                if ((m & 1) == 0) {
-                    const int r = m >> 1;
-                    if (r < TN) fa[sn][r] = *reinterpret_cast<const vec8 *>(src + woff[sn][r]);
-                    else fb[sn][r - TN] = *reinterpret_cast<const vec8 *>(src + xoff[sn][r - TN]);
-                } else if (st >= 2) {
-                    tile_load((st - 2) * 8 + (m >> 1), CUR, (kt + 2) * BK);
+            for (int m = 0; m < NB * NB; ++m) {
+                const int i = m / NB, j = m % NB;
+                mfma16_inplace(fa[st][j], fb[st][i], acc[i][j]);
+                if ((m & 3) == 0) {
+                    const int r = m >> 2;  // 0..15: the eight weight fragments first, they are all needed at once
+                    if (r < NB) fa[sn][r] = *reinterpret_cast<const vec8 *>(src + woff[sn][r]);
+                    else fb[sn][r - NB] = *reinterpret_cast<const vec8 *>(src + xoff[sn][r - NB]);
+                } else if ((m & 3) == 2 && st == 1) {
+                    tile_load(m >> 2, CUR, (kt + 2) * BK);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -562,18 +662,27 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     }
     if (kt < nk) k_tile(IntC<0>(), kt);
 
-    // all bias entries of the wave's 128 columns in one go: one memory round trip per tile instead of one per block
-    u32x4 braw[TN][2];
-    bias_fetch<T, TN>(bias, n0 + wave_n * 128, lh, N, bias_vec_ok, braw);
-    // one call per 32-row block: each stays small enough for the compiler to unroll completely, so the accumulators
+    // all bias entries of the lane's columns in one go: one memory round trip per tile
+    const int n_wave = n0 + wave_n * 128;
+    u32x4 braw[2][2];
+#pragma unroll
+    for (int G = 0; G < 2; ++G)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            braw[G][h] = fetch8<T>(bias, n_wave + 64 * G + (GATED ? 32 * h + 8 * g : 16 * g + 8 * h), N, bias_vec_ok);
+    // one call per 16-row block: each stays small enough for the compiler to unroll completely, so the accumulators
     // are only ever indexed by constants and never leave the register file
-#define KERNL_WIDE_EPILOGUE(I)                                                                                          \
-    linear_epilogue<T, ACT, TM, TN, I, 1>(acc, m0 + wave_m * 128, n0 + wave_n * 128, lr, lh, bias, out, act_in, M, N,    \
-                                          out_rs, out_cs, ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bias_vec_ok, braw)
+#define KERNL_WIDE_EPILOGUE(I)                                                                                         \
+    wide_epilogue<T, ACT, I>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs, ai_cs,   \
+                             out_vec_ok, ai_vec_ok, braw)
     KERNL_WIDE_EPILOGUE(0);
     KERNL_WIDE_EPILOGUE(1);
     KERNL_WIDE_EPILOGUE(2);
     KERNL_WIDE_EPILOGUE(3);
+    KERNL_WIDE_EPILOGUE(4);
+    KERNL_WIDE_EPILOGUE(5);
+    KERNL_WIDE_EPILOGUE(6);
+    KERNL_WIDE_EPILOGUE(7);
 #undef KERNL_WIDE_EPILOGUE
 }
 
