@@ -523,23 +523,33 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     typedef typename Vec8<T>::type vec8;
     constexpr bool GATED = (ACT & kGluBit) != 0;
     constexpr int BM = 256, BN = 256, BK = 64, RB = BK * 2, CPR = BK / 8, NB = 8, KSTEPS = BK / 32;
-    constexpr int X_BYTES = BM * RB, W_BYTES = BN * RB, STAGE = X_BYTES + W_BYTES;
+    // LDS: [x stage 0 | x stage 1 | w stage 0 | w stage 1], 32 KB each: every fragment address is one per-lane register
+    // plus an immediate of 0 or 32 KB for the stage (the immediate field of an LDS read ends at 64 KB - 1).
+    constexpr int X_BYTES = BM * RB, W_BYTES = BN * RB, W_BASE = 2 * X_BYTES;
+    static_assert(X_BYTES == 32768 && W_BYTES == 32768, "stage immediates");
     constexpr int LOADS = BM * CPR / 256;  // 1 KB loads per wave for each operand tile
     constexpr int GROUP_M = 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
+    // Persistent workgroups: one per CU (at most), each walking the output tiles  slot, slot + slots, ...  of its
+    // XCD's contiguous run of the grouped tile order.  The k-tile stream runs THROUGH tile boundaries: while the last
+    // k-tiles of one output tile are multiplied, the first two k-tiles of the next are already on their way into LDS,
+    // and the epilogue's stores drain under the next tile's main loop.
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) >> 3;
-    const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-    if ((int)(blockIdx.x >> 3) >= per_xcd || t >= total) return;
-    const int group_span = GROUP_M * tiles_n;
-    const int group = t / group_span;
-    const int first_m = group * GROUP_M;
-    const int gsize = min(tiles_m - first_m, GROUP_M);
-    const int in_group = t - group * group_span;
-    const int tile_m = first_m + in_group % gsize;
-    const int tile_n = in_group / gsize;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int xcd = (int)(blockIdx.x & 7), slots = (int)(gridDim.x >> 3);
+    auto tile_origin = [&](int idx, int &m0, int &n0) __attribute__((always_inline)) -> bool {
+        const int t = xcd * per_xcd + idx;
+        if (idx >= per_xcd || t >= total) return false;
+        const int group_span = GROUP_M * tiles_n;
+        const int group = t / group_span;
+        const int first_m = group * GROUP_M;
+        const int gsize = min(tiles_m - first_m, GROUP_M);
+        const int in_group = t - group * group_span;
+        m0 = (first_m + in_group % gsize) * BM;
+        n0 = (in_group / gsize) * BN;
+        return true;
+    };
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -547,31 +557,39 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     const int l16 = lane & 15, g = lane >> 4;
 
     // ---- tile loads: load i of a wave fills the 1 KB of 16-byte chunks [256 i + 64 wave, +64) of an operand tile;
-    // every lane fetches the chunk that belongs at its LDS position under the swizzle.  Rows beyond M / N and
-    // k-tiles beyond K lie outside the buffer resource and arrive as zeros.
+    // every lane fetches the chunk that belongs at its LDS position under the swizzle.  Rows beyond M / N lie outside
+    // the buffer resource and arrive as zeros.  A wave's loads of one operand tile land in one contiguous 8 KB block
+    // (load i at +1 KB i), so that groups of 4 loads share one write of the LDS base register and differ only in the
+    // instruction's immediate offset.  That immediate is added to the memory address too, hence it is subtracted from
+    // the per-lane offsets here.
     constexpr uint32_t kOutOfRange = 0x80000000u;
-    const int rows_x = min(BM, M - m0), rows_w = min(BN, N - n0);
-    const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx), waddr = (uint64_t)(uintptr_t)(W + (int64_t)n0 * K);
-    const u32x4 xrsrc = {(uint32_t)xaddr, (uint32_t)(xaddr >> 32) & 0xFFFFu,
-                         (uint32_t)((((int64_t)rows_x - 1) * ldx + K) * 2), 0x00020000u};
-    const u32x4 wrsrc = {(uint32_t)waddr, (uint32_t)(waddr >> 32) & 0xFFFFu, (uint32_t)((int64_t)rows_w * K * 2),
-                         0x00020000u};
-    // A wave's loads of one operand tile land in one contiguous 8 KB block (load i at +1 KB i), so that groups of 4
-    // loads share one write of the LDS base register and differ only in the instruction's immediate offset.  That
-    // immediate is added to the memory address too, hence it is subtracted from the per-lane offsets here.
+    u32x4 xrsrc = {0, 0, 0, 0x00020000u}, wrsrc = {0, 0, 0, 0x00020000u};
     uint32_t xd[LOADS], wd[LOADS];
+    // points the tile loads at the output tile with origin (m0, n0); `valid` false switches them off
+    auto set_load_tile = [&](bool valid, int m0, int n0) __attribute__((always_inline)) {
+        const int rows_x = valid ? min(BM, M - m0) : 0, rows_w = valid ? min(BN, N - n0) : 0;
+        if (valid) {
+            const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx), waddr = (uint64_t)(uintptr_t)(W + (int64_t)n0 * K);
+            xrsrc[0] = (uint32_t)xaddr;
+            xrsrc[1] = (uint32_t)(xaddr >> 32) & 0xFFFFu;
+            xrsrc[2] = (uint32_t)((((int64_t)rows_x - 1) * ldx + K) * 2);
+            wrsrc[0] = (uint32_t)waddr;
+            wrsrc[1] = (uint32_t)(waddr >> 32) & 0xFFFFu;
+            wrsrc[2] = (uint32_t)((int64_t)rows_w * K * 2);
+        }
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-        const int q = (wave * LOADS + i) * 64 + lane;  // 16-byte chunk index inside the tile
-        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
-        const uint32_t imm = (uint32_t)(i & 3) * 1024u;
-        xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) - imm : kOutOfRange;
-        // LDS row `row` is MFMA row r = row % 16 of block j = (row % 64) / 16 of its 64-row group
-        const int r = row & 15, j = (row >> 4) & 3;
-        const int in_group64 = GATED ? 32 * (j >> 1) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3) : 16 * (r >> 2) + 4 * j + (r & 3);
-        const int wrow = (row & ~63) + in_group64;
-        wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - imm : kOutOfRange;
-    }
+        for (int i = 0; i < LOADS; ++i) {
+            const int q = (wave * LOADS + i) * 64 + lane;  // 16-byte chunk index inside the tile
+            const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+            const uint32_t imm = (uint32_t)(i & 3) * 1024u;
+            xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) - imm : kOutOfRange;
+            // LDS row `row` is MFMA row r = row % 16 of block j = (row % 64) / 16 of its 64-row group
+            const int r = row & 15, j = (row >> 4) & 3;
+            const int in_group64 = GATED ? 32 * (j >> 1) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3) : 16 * (r >> 2) + 4 * j + (r & 3);
+            const int wrow = (row & ~63) + in_group64;
+            wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - imm : kOutOfRange;
+        }
+    };
     typedef __attribute__((address_space(3))) void lds_void;
     const uint32_t dma_base = (uint32_t)(uintptr_t)(lds_void *)smem + wave * (LOADS * 1024);
     // inline assembly on purpose: the compiler would make every later LDS read wait for loads it sees writing LDS.
@@ -590,55 +608,74 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     };
     // load l (0..15) of a k-tile: X loads 0..7, then W loads 0..7
     auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
-        if (l < LOADS) load4(xrsrc, xd, dma_base + stage * STAGE, l >> 2, l & 3, k0);
-        else load4(wrsrc, wd, dma_base + stage * STAGE + X_BYTES, (l - LOADS) >> 2, l & 3, k0);
+        if (l < LOADS) load4(xrsrc, xd, dma_base + stage * X_BYTES, l >> 2, l & 3, k0);
+        else load4(wrsrc, wd, dma_base + W_BASE + stage * W_BYTES, (l - LOADS) >> 2, l & 3, k0);
     };
 
-    f32x4_acc acc[NB][NB];  // [m-block][n-block]
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < NB; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
-
-    // LDS byte offsets of this lane's operand fragments, one register per (k-step, block): with a whole register
-    // file per wave there is room to keep them all, and no address arithmetic is left in the loop
-    int xoff[KSTEPS][NB], woff[KSTEPS][NB];
+    // LDS addresses of this lane's operand fragments in stage 0, one register per (k-step, block): with a whole
+    // register file per wave there is room to keep them all, and no address arithmetic is left in the loop
+    typedef __attribute__((address_space(3))) const unsigned char *lds_bytes;
+    typedef __attribute__((address_space(3))) const vec8 *lds_frag;
+    const lds_bytes lds0 = (lds_bytes)smem;
+    lds_frag xfrag[KSTEPS][NB], wfrag[KSTEPS][NB];
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st) {
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
-            xoff[st][i] = swz_offset<RB>(wave_m * 128 + i * 16 + l16, 4 * st + g);
-            woff[st][i] = X_BYTES + swz_offset<RB>(wave_n * 128 + i * 16 + l16, 4 * st + g);
+            xfrag[st][i] = (lds_frag)(lds0 + swz_offset<RB>(wave_m * 128 + i * 16 + l16, 4 * st + g));
+            wfrag[st][i] = (lds_frag)(lds0 + W_BASE + swz_offset<RB>(wave_n * 128 + i * 16 + l16, 4 * st + g));
         }
     }
+    constexpr int STAGE_FRAGS = X_BYTES / 16;  // pointer increment that selects stage 1
 
     const int nk = K / BK;
+    int idx = (int)(blockIdx.x >> 3);  // position of the tile being multiplied in this XCD's run
+    int m0 = 0, n0 = 0;
+    if (!tile_origin(idx, m0, n0)) return;
+
+    // the load side runs ahead of the multiply side: (load_idx, load_kt) is the next k-tile to request
+    int load_idx = idx, load_kt = 0;
+    set_load_tile(true, m0, n0);
+    auto advance_load = [&]() __attribute__((always_inline)) {
+        if (++load_kt == nk) {
+            load_kt = 0;
+            load_idx += slots;
+            int lm0 = 0, ln0 = 0;
+            const bool more = tile_origin(load_idx, lm0, ln0);
+            set_load_tile(more, lm0, ln0);
+        }
+    };
 #pragma unroll
-    for (int l = 0; l < 2 * LOADS; ++l) tile_load(l, 0, 0);
+    for (int l = 0; l < 2 * LOADS; ++l) tile_load(l, 0, load_kt * BK);
+    advance_load();
 #pragma unroll
-    for (int l = 0; l < 2 * LOADS; ++l) tile_load(l, 1, BK);
+    for (int l = 0; l < 2 * LOADS; ++l) tile_load(l, 1, load_kt * BK);
+    advance_load();
     static_assert(2 * LOADS == 16, "the wait below encodes vmcnt(16)");
-    __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): all of tile 0 has landed, tile 1 may still be in flight
+    __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): the first k-tile has landed, the second may still be in flight
     __syncthreads();
 
     vec8 fa[KSTEPS][NB], fb[KSTEPS][NB];  // weight and activation fragments, one register set per k-step
 #pragma unroll
-    for (int j = 0; j < NB; ++j) fa[0][j] = *reinterpret_cast<const vec8 *>(smem + woff[0][j]);
+    for (int j = 0; j < NB; ++j) fa[0][j] = *wfrag[0][j];
 #pragma unroll
-    for (int i = 0; i < NB; ++i) fb[0][i] = *reinterpret_cast<const vec8 *>(smem + xoff[0][i]);
+    for (int i = 0; i < NB; ++i) fb[0][i] = *xfrag[0][i];
 
-    // one k-tile held in stage CUR (a compile-time constant, so that stage offsets fold into instruction offsets)
-    auto k_tile = [&](auto cur_c, int kt) __attribute__((always_inline)) {
+    f32x4_acc acc[NB][NB];  // [m-block][n-block]
+
+    // One k-tile held in stage CUR (a compile-time constant, so that stage offsets fold into instruction offsets).
+    // `landed`: the loads of the next k-tile are known to have arrived (a wait for later loads has been passed), and
+    // waiting for "everything outstanding" would only wait for the previous tile's output stores.
+    auto k_tile = [&](auto cur_c, bool landed) __attribute__((always_inline)) {
         constexpr int CUR = decltype(cur_c)::value;
-        const unsigned char *cur = smem + CUR * STAGE;
-        const unsigned char *nxt = smem + (CUR ^ 1) * STAGE;
+        const int k0 = load_kt * BK;
 #pragma unroll
         for (int st = 0; st < KSTEPS; ++st) {
             const int sn = st ^ 1;                               // k-step whose fragments are fetched now
-            const unsigned char *src = st == 0 ? cur : nxt;
+            const int src = (st == 0 ? CUR : CUR ^ 1) * STAGE_FRAGS;  // stage holding those fragments
             if (st == 1) {
-                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads of k-tile kt + 1 have landed
-                __syncthreads();                     // ... everyone's have, and nobody reads stage CUR any more
+                if (!landed) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads of the next k-tile are in
+                __syncthreads();                                  // ... everyone's are, and nobody reads stage CUR any more
             }
 #pragma unroll
             for (int m = 0; m < NB * NB; ++m) {
@@ -646,44 +683,64 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
                 mfma16_inplace(fa[st][j], fb[st][i], acc[i][j]);
                 if ((m & 3) == 0) {
                     const int r = m >> 2;  // 0..15: the eight weight fragments first, they are all needed at once
-                    if (r < NB) fa[sn][r] = *reinterpret_cast<const vec8 *>(src + woff[sn][r]);
-                    else fb[sn][r - NB] = *reinterpret_cast<const vec8 *>(src + xoff[sn][r - NB]);
+                    if (r < NB) fa[sn][r] = *(wfrag[sn][r] + src);
+                    else fb[sn][r - NB] = *(xfrag[sn][r - NB] + src);
                 } else if ((m & 3) == 2 && st == 1) {
-                    tile_load(m >> 2, CUR, (kt + 2) * BK);
+                    tile_load(m >> 2, CUR, k0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
-    int kt = 0;
-    for (; kt + 1 < nk; kt += 2) {
-        k_tile(IntC<0>(), kt);
-        k_tile(IntC<1>(), kt + 1);
-    }
-    if (kt < nk) k_tile(IntC<0>(), kt);
 
-    // all bias entries of the lane's columns in one go: one memory round trip per tile
-    const int n_wave = n0 + wave_n * 128;
-    u32x4 braw[2][2];
+    // Every output tile starts in stage 0: the host launches one workgroup per tile when the number of k-tiles is odd.
+    bool landed = false;
+    while (true) {
 #pragma unroll
-    for (int G = 0; G < 2; ++G)
+        for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-            braw[G][h] = fetch8<T>(bias, n_wave + 64 * G + (GATED ? 32 * h + 8 * g : 16 * g + 8 * h), N, bias_vec_ok);
-    // one call per 16-row block: each stays small enough for the compiler to unroll completely, so the accumulators
-    // are only ever indexed by constants and never leave the register file
+            for (int j = 0; j < NB; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+        int kt = 0;
+        for (; kt + 1 < nk; kt += 2) {
+            k_tile(IntC<0>(), landed);
+            advance_load();
+            landed = false;
+            k_tile(IntC<1>(), false);
+            advance_load();
+        }
+        if (kt < nk) {
+            k_tile(IntC<0>(), landed);
+            advance_load();
+        }
+
+        // all bias entries of the lane's columns in one go: one memory round trip per tile.  Its wait also covers the
+        // loads of the next k-tile, which were issued earlier.
+        const int n_wave = n0 + wave_n * 128;
+        u32x4 braw[2][2];
+#pragma unroll
+        for (int G = 0; G < 2; ++G)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                braw[G][h] = fetch8<T>(bias, n_wave + 64 * G + (GATED ? 32 * h + 8 * g : 16 * g + 8 * h), N, bias_vec_ok);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        landed = true;
+        // one call per 16-row block: each stays small enough for the compiler to unroll completely, so the
+        // accumulators are only ever indexed by constants and never leave the register file
 #define KERNL_WIDE_EPILOGUE(I)                                                                                         \
     wide_epilogue<T, ACT, I>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs, ai_cs,   \
                              out_vec_ok, ai_vec_ok, braw)
-    KERNL_WIDE_EPILOGUE(0);
-    KERNL_WIDE_EPILOGUE(1);
-    KERNL_WIDE_EPILOGUE(2);
-    KERNL_WIDE_EPILOGUE(3);
-    KERNL_WIDE_EPILOGUE(4);
-    KERNL_WIDE_EPILOGUE(5);
-    KERNL_WIDE_EPILOGUE(6);
-    KERNL_WIDE_EPILOGUE(7);
+        KERNL_WIDE_EPILOGUE(0);
+        KERNL_WIDE_EPILOGUE(1);
+        KERNL_WIDE_EPILOGUE(2);
+        KERNL_WIDE_EPILOGUE(3);
+        KERNL_WIDE_EPILOGUE(4);
+        KERNL_WIDE_EPILOGUE(5);
+        KERNL_WIDE_EPILOGUE(6);
+        KERNL_WIDE_EPILOGUE(7);
 #undef KERNL_WIDE_EPILOGUE
+        idx += slots;
+        if (!tile_origin(idx, m0, n0)) break;
+    }
 }
 
 // ----------------------------------------------------------------------------------------------------
@@ -813,7 +870,10 @@ static void launch_wide_act(const LinearArgs &a) {
     const int out_vec_ok = a.out_cs == 1 && a.out_rs % 8 == 0 && aligned16(out);
     const int ai_vec_ok = act_in != nullptr && a.ai_cs == 1 && a.ai_rs % 8 == 0 && aligned16(act_in);
     const int bias_vec_ok = bias != nullptr && aligned16(bias);
-    hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
+    // persistent: at most one workgroup per CU (32 per XCD), each walks its share of the XCD's tiles.  The kernel
+    // needs every tile to start in LDS stage 0: with an odd number of k-tiles each workgroup gets a single tile.
+    const int slots = (per_xcd < 32 || (a.K / 64) % 2 != 0) ? per_xcd : 32;
+    hipLaunchKernelGGL(kern, dim3(slots * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
                        a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok);
 }

@@ -131,3 +131,15 @@ def test_glu_argument_errors():
     out = torch.empty((8, 48), dtype=torch.float16, device="cuda")
     with pytest.raises(RuntimeError):
         _lib.linear_glu_fwd(x, w[:48].repeat(2, 1), None, out, _lib.ACT_SILU)  # N = 48
+
+
+def test_glu_more_tiles_than_compute_units(close):
+    M, N, K = 4352, 2208, 128  # 17 x 18 tiles of the interleaved weight: workgroups walk two tiles each
+    x, wg, bg, wv, bv = _case(M, N, K, torch.float16, True, seed=12)
+    lib = _lib.load()
+    lib.kernl_linear_force_tile(5)
+    try:
+        out = _run(x, wg, bg, wv, bv, "silu")
+    finally:
+        lib.kernl_linear_force_tile(0)
+    close(out, glu_oracle(x, wg, bg, wv, bv, "silu"), scale=4.0, what="glu persistent")

@@ -136,3 +136,21 @@ def test_unknown_activation_is_identity(close):
     out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation="swish-not-a-name")
     torch.cuda.synchronize()
     close(out, linear_oracle(x, w, b, ""), what="unknown activation")
+
+
+@pytest.mark.parametrize("shape", [(4352, 4352, 128), (4352, 4300, 192), (4400, 4352, 64), (8200, 2304, 256)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_linear_more_tiles_than_compute_units(shape, close):
+    """More than 256 output tiles of 256x256: workgroups of the persistent kernel walk several tiles each, with the
+    operand stream running through the tile boundaries (even k-tile counts) or one tile per workgroup (odd counts)."""
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(11)
+    x, w, b = _inputs(M, N, K, torch.float16, gen, w_std=K ** -0.5)
+    lib = _lib.load()
+    lib.kernl_linear_force_tile(5)
+    try:
+        out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation="relu")
+        torch.cuda.synchronize()
+    finally:
+        lib.kernl_linear_force_tile(0)
+    close(out, linear_oracle(x, w, b, "relu"), what=f"linear persistent {shape}")
