@@ -429,15 +429,18 @@ __device__ __forceinline__ u32x4 fetch8(const T *__restrict__ p, int idx, int li
     return r;
 }
 
-// Epilogue of m-block IB (16 rows) of a wave of the wide kernel: lane (l16, g) holds row m_wave + 16 IB + l16.
-template <typename T, int ACT, int IB>
-__device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[8][8], int m_wave, int n_wave, int l16, int g,
+// Epilogue of m-block IB (16 rows) of a wave of the wide kernel: lane (l16, g) holds row m_wave + 16 IB + l16 and, in
+// every group of JB n-blocks, the 4 JB consecutive columns starting at 4 JB g (JB = 4: 64-column groups, 2: 32-column).
+template <typename T, int ACT, int IB, int NBN>
+__device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[8][NBN], int m_wave, int n_wave, int l16, int g,
                                               T *__restrict__ out, T *__restrict__ act_in, int M, int N,
                                               int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs,
-                                              int out_vec_ok, int ai_vec_ok, const u32x4 (&braw)[2][2]) {
+                                              int out_vec_ok, int ai_vec_ok,
+                                              const u32x4 (&braw)[NBN == 8 ? 2 : 3][2]) {
     const int m = m_wave + 16 * IB + l16;
     const bool rows_inside = m_wave + 16 * IB + 16 <= M;
     if constexpr ((ACT & kGluBit) != 0) {
+        static_assert(NBN == 8, "gated epilogues pair blocks inside 64-row groups");
         constexpr int BASE = ACT & (kGluBit - 1);
         const int n_total = N >> 1;
         const bool interior = rows_inside && (n_wave >> 1) + 64 <= n_total && out_vec_ok;
@@ -465,56 +468,56 @@ __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[8][8], int m_wave
         }
         return;
     }
-    auto store16 = [&](T *p, const float (&r)[16]) __attribute__((always_inline)) {
-        u32x4 p0, p1;
+    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB, VPG = 4 * JB;  // blocks per group, groups, values per lane and group
+    auto store_vec = [&](T *p, const float (&r)[VPG]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
-            p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
+        for (int h = 0; h < VPG / 8; ++h) {
+            u32x4 pk;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) pk[v] = pack2<T>(r[8 * h + 2 * v], r[8 * h + 2 * v + 1]);
+            *reinterpret_cast<u32x4 *>(p + 8 * h) = pk;
         }
-        *reinterpret_cast<u32x4 *>(p) = p0;
-        *reinterpret_cast<u32x4 *>(p + 8) = p1;
     };
-    const bool interior = rows_inside && n_wave + 128 <= N && out_vec_ok && act_in == nullptr;
+    const bool interior = rows_inside && n_wave + NBN * 16 <= N && out_vec_ok && act_in == nullptr;
     if (__builtin_amdgcn_readfirstlane((int)interior)) {
 #pragma unroll
-        for (int G = 0; G < 2; ++G) {
-            float r[16];
+        for (int G = 0; G < NG; ++G) {
+            float r[VPG];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) r[v] = apply_act(acc[IB][4 * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v), ACT);
-            store16(out + (int64_t)m * out_rs + n_wave + 64 * G + 16 * g, r);
+            for (int v = 0; v < VPG; ++v) r[v] = apply_act(acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v), ACT);
+            store_vec(out + (int64_t)m * out_rs + n_wave + 16 * JB * G + VPG * g, r);
         }
         return;
     }
 #pragma unroll
-    for (int G = 0; G < 2; ++G) {
-        const int n = n_wave + 64 * G + 16 * g;
+    for (int G = 0; G < NG; ++G) {
+        const int n = n_wave + 16 * JB * G + VPG * g;
         if (m >= M || n >= N) continue;
-        float r[16];
+        float r[VPG];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) r[v] = acc[IB][4 * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v);
+        for (int v = 0; v < VPG; ++v) r[v] = acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v);
         if (act_in != nullptr) {
-            if (ai_vec_ok && n + 16 <= N) {
-                store16(act_in + (int64_t)m * ai_rs + n, r);
+            if (ai_vec_ok && n + VPG <= N) {
+                store_vec(act_in + (int64_t)m * ai_rs + n, r);
             } else {
 #pragma unroll
-                for (int v = 0; v < 16; ++v)
+                for (int v = 0; v < VPG; ++v)
                     if (n + v < N) act_in[(int64_t)m * ai_rs + (int64_t)(n + v) * ai_cs] = from_float<T>(r[v]);
             }
         }
 #pragma unroll
-        for (int v = 0; v < 16; ++v) r[v] = apply_act(r[v], ACT);
-        if (out_vec_ok && n + 16 <= N) {
-            store16(out + (int64_t)m * out_rs + n, r);
+        for (int v = 0; v < VPG; ++v) r[v] = apply_act(r[v], ACT);
+        if (out_vec_ok && n + VPG <= N) {
+            store_vec(out + (int64_t)m * out_rs + n, r);
         } else {
 #pragma unroll
-            for (int v = 0; v < 16; ++v)
+            for (int v = 0; v < VPG; ++v)
                 if (n + v < N) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
         }
     }
 }
 
-template <typename T, int ACT>
+template <typename T, int ACT, int NBN>
 __global__ void __launch_bounds__(256, 1)
 linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
                    T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
@@ -522,12 +525,14 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
                    int bias_vec_ok) {
     typedef typename Vec8<T>::type vec8;
     constexpr bool GATED = (ACT & kGluBit) != 0;
-    constexpr int BM = 256, BN = 256, BK = 64, RB = BK * 2, CPR = BK / 8, NB = 8, KSTEPS = BK / 32;
+    static_assert(NBN == 8 || (NBN == 6 && !GATED), "256 or 192 columns per tile; gated epilogues need 256");
+    constexpr int BM = 256, BN = 32 * NBN, BK = 64, RB = BK * 2, CPR = BK / 8, NB = 8, KSTEPS = BK / 32;
     // LDS: [x stage 0 | x stage 1 | w stage 0 | w stage 1], 32 KB each: every fragment address is one per-lane register
     // plus an immediate of 0 or 32 KB for the stage (the immediate field of an LDS read ends at 64 KB - 1).
-    constexpr int X_BYTES = BM * RB, W_BYTES = BN * RB, W_BASE = 2 * X_BYTES;
-    static_assert(X_BYTES == 32768 && W_BYTES == 32768, "stage immediates");
-    constexpr int LOADS = BM * CPR / 256;  // 1 KB loads per wave for each operand tile
+    constexpr int X_BYTES = BM * RB, W_BYTES = 32768, W_BASE = 2 * X_BYTES;
+    static_assert(X_BYTES == 32768 && BN * RB <= W_BYTES, "stage immediates");
+    constexpr int LOADS = BM * CPR / 256, LOADS_W = BN * CPR / 256;  // 1 KB loads per wave for the x and the w tile
+    constexpr int NL = LOADS + LOADS_W;                             // tile loads per wave and k-tile
     constexpr int GROUP_M = 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -564,7 +569,7 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     // the per-lane offsets here.
     constexpr uint32_t kOutOfRange = 0x80000000u;
     u32x4 xrsrc = {0, 0, 0, 0x00020000u}, wrsrc = {0, 0, 0, 0x00020000u};
-    uint32_t xd[LOADS], wd[LOADS];
+    uint32_t xd[LOADS], wd[LOADS_W];
     // points the tile loads at the output tile with origin (m0, n0); `valid` false switches them off
     auto set_load_tile = [&](bool valid, int m0, int n0) __attribute__((always_inline)) {
         const int rows_x = valid ? min(BM, M - m0) : 0, rows_w = valid ? min(BN, N - n0) : 0;
@@ -581,35 +586,39 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         for (int i = 0; i < LOADS; ++i) {
             const int q = (wave * LOADS + i) * 64 + lane;  // 16-byte chunk index inside the tile
             const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
-            const uint32_t imm = (uint32_t)(i & 3) * 1024u;
-            xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) - imm : kOutOfRange;
-            // LDS row `row` is MFMA row r = row % 16 of block j = (row % 64) / 16 of its 64-row group
+            xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
+        }
+#pragma unroll
+        for (int i = 0; i < LOADS_W; ++i) {
+            const int q = (wave * LOADS_W + i) * 64 + lane;
+            const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+            // LDS row `row` is MFMA row r = row % 16 of n-block row / 16; see the placement rule above the kernel
             const int r = row & 15, j = (row >> 4) & 3;
-            const int in_group64 = GATED ? 32 * (j >> 1) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3) : 16 * (r >> 2) + 4 * j + (r & 3);
-            const int wrow = (row & ~63) + in_group64;
-            wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - imm : kOutOfRange;
+            const int wrow = GATED      ? (row & ~63) + 32 * (j >> 1) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3)
+                             : NBN == 8 ? (row & ~63) + 16 * (r >> 2) + 4 * j + (r & 3)
+                                        : (row & ~31) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3);
+            wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
         }
     };
     typedef __attribute__((address_space(3))) void lds_void;
-    const uint32_t dma_base = (uint32_t)(uintptr_t)(lds_void *)smem + wave * (LOADS * 1024);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
     // inline assembly on purpose: the compiler would make every later LDS read wait for loads it sees writing LDS.
     // `group` (0 or 1) selects loads 4 group .. 4 group + 3; its first load writes the LDS base register.
-    auto load4 = [&](const u32x4 &rsrc, const uint32_t (&off)[LOADS], uint32_t lds, int group, int part, int k0) __attribute__((always_inline)) {
-        const int i = 4 * group + part;
+    auto load4 = [&](const u32x4 &rsrc, uint32_t off, uint32_t lds, int group, int part, int k0) __attribute__((always_inline)) {
         if (part == 0)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :: "s"(lds + group * 4096), "v"(off[i]), "s"(rsrc), "s"(k0 * 2) : "memory", "m0");
+                         :: "s"(lds + group * 4096), "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory", "m0");
         else if (part == 1)
-            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds" :: "v"(off[i]), "s"(rsrc), "s"(k0 * 2) : "memory");
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
         else if (part == 2)
-            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:2048 lds" :: "v"(off[i]), "s"(rsrc), "s"(k0 * 2) : "memory");
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:2048 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
         else
-            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off[i]), "s"(rsrc), "s"(k0 * 2) : "memory");
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
     };
-    // load l (0..15) of a k-tile: X loads 0..7, then W loads 0..7
+    // load l (0 .. NL-1) of a k-tile: the x loads, then the w loads
     auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
-        if (l < LOADS) load4(xrsrc, xd, dma_base + stage * X_BYTES, l >> 2, l & 3, k0);
-        else load4(wrsrc, wd, dma_base + W_BASE + stage * W_BYTES, (l - LOADS) >> 2, l & 3, k0);
+        if (l < LOADS) load4(xrsrc, xd[l], lds_base + stage * X_BYTES + wave * (LOADS * 1024), l >> 2, l & 3, k0);
+        else load4(wrsrc, wd[l - LOADS], lds_base + W_BASE + stage * W_BYTES + wave * (LOADS_W * 1024), (l - LOADS) >> 2, l & 3, k0);
     };
 
     // LDS addresses of this lane's operand fragments in stage 0, one register per (k-step, block): with a whole
@@ -617,14 +626,14 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     typedef __attribute__((address_space(3))) const unsigned char *lds_bytes;
     typedef __attribute__((address_space(3))) const vec8 *lds_frag;
     const lds_bytes lds0 = (lds_bytes)smem;
-    lds_frag xfrag[KSTEPS][NB], wfrag[KSTEPS][NB];
+    lds_frag xfrag[KSTEPS][NB], wfrag[KSTEPS][NBN];
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st) {
 #pragma unroll
-        for (int i = 0; i < NB; ++i) {
-            xfrag[st][i] = (lds_frag)(lds0 + swz_offset<RB>(wave_m * 128 + i * 16 + l16, 4 * st + g));
-            wfrag[st][i] = (lds_frag)(lds0 + W_BASE + swz_offset<RB>(wave_n * 128 + i * 16 + l16, 4 * st + g));
-        }
+        for (int i = 0; i < NB; ++i) xfrag[st][i] = (lds_frag)(lds0 + swz_offset<RB>(wave_m * 128 + i * 16 + l16, 4 * st + g));
+#pragma unroll
+        for (int j = 0; j < NBN; ++j)
+            wfrag[st][j] = (lds_frag)(lds0 + W_BASE + swz_offset<RB>(wave_n * (NBN * 16) + j * 16 + l16, 4 * st + g));
     }
     constexpr int STAGE_FRAGS = X_BYTES / 16;  // pointer increment that selects stage 1
 
@@ -646,22 +655,22 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         }
     };
 #pragma unroll
-    for (int l = 0; l < 2 * LOADS; ++l) tile_load(l, 0, load_kt * BK);
+    for (int l = 0; l < NL; ++l) tile_load(l, 0, load_kt * BK);
     advance_load();
 #pragma unroll
-    for (int l = 0; l < 2 * LOADS; ++l) tile_load(l, 1, load_kt * BK);
+    for (int l = 0; l < NL; ++l) tile_load(l, 1, load_kt * BK);
     advance_load();
-    static_assert(2 * LOADS == 16, "the wait below encodes vmcnt(16)");
-    __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): the first k-tile has landed, the second may still be in flight
+    // vmcnt(NL): the first k-tile has landed, the second may still be in flight
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (NL & 15) | ((NL >> 4) << 14));
     __syncthreads();
 
-    vec8 fa[KSTEPS][NB], fb[KSTEPS][NB];  // weight and activation fragments, one register set per k-step
+    vec8 fa[KSTEPS][NBN], fb[KSTEPS][NB];  // weight and activation fragments, one register set per k-step
 #pragma unroll
-    for (int j = 0; j < NB; ++j) fa[0][j] = *wfrag[0][j];
+    for (int j = 0; j < NBN; ++j) fa[0][j] = *wfrag[0][j];
 #pragma unroll
     for (int i = 0; i < NB; ++i) fb[0][i] = *xfrag[0][i];
 
-    f32x4_acc acc[NB][NB];  // [m-block][n-block]
+    f32x4_acc acc[NB][NBN];  // [m-block][n-block]
 
     // One k-tile held in stage CUR (a compile-time constant, so that stage offsets fold into instruction offsets).
     // `landed`: the loads of the next k-tile are known to have arrived (a wait for later loads has been passed), and
@@ -677,16 +686,18 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
                 if (!landed) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads of the next k-tile are in
                 __syncthreads();                                  // ... everyone's are, and nobody reads stage CUR any more
             }
+            constexpr int PERIOD = NBN == 8 ? 4 : 3;  // MFMAs per LDS read / tile load: 64 / 4 = 48 / 3 = 16 issue slots
 #pragma unroll
-            for (int m = 0; m < NB * NB; ++m) {
-                const int i = m / NB, j = m % NB;
+            for (int m = 0; m < NB * NBN; ++m) {
+                const int i = m / NBN, j = m % NBN;
                 mfma16_inplace(fa[st][j], fb[st][i], acc[i][j]);
-                if ((m & 3) == 0) {
-                    const int r = m >> 2;  // 0..15: the eight weight fragments first, they are all needed at once
-                    if (r < NB) fa[sn][r] = *(wfrag[sn][r] + src);
-                    else fb[sn][r - NB] = *(xfrag[sn][r - NB] + src);
-                } else if ((m & 3) == 2 && st == 1) {
-                    tile_load(m >> 2, CUR, k0);
+                const int slot = m / PERIOD;
+                if (m % PERIOD == 0 && slot < NBN + NB) {
+                    // the weight fragments first: the first MFMAs of the next k-step need all of them
+                    if (slot < NBN) fa[sn][slot] = *(wfrag[sn][slot] + src);
+                    else fb[sn][slot - NBN] = *(xfrag[sn][slot - NBN] + src);
+                } else if (m % PERIOD == PERIOD - 2 && st == 1 && slot < NL) {
+                    tile_load(slot, CUR, k0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -699,7 +710,7 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 #pragma unroll
         for (int i = 0; i < NB; ++i)
 #pragma unroll
-            for (int j = 0; j < NB; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int j = 0; j < NBN; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
         int kt = 0;
         for (; kt + 1 < nk; kt += 2) {
             k_tile(IntC<0>(), landed);
@@ -715,19 +726,21 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 
         // all bias entries of the lane's columns in one go: one memory round trip per tile.  Its wait also covers the
         // loads of the next k-tile, which were issued earlier.
-        const int n_wave = n0 + wave_n * 128;
-        u32x4 braw[2][2];
+        const int n_wave = n0 + wave_n * (NBN * 16);
+        constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB;  // n-blocks per lane-contiguous group, groups per wave
+        u32x4 braw[NG][2];
 #pragma unroll
-        for (int G = 0; G < 2; ++G)
+        for (int G = 0; G < NG; ++G)
 #pragma unroll
             for (int h = 0; h < 2; ++h)
-                braw[G][h] = fetch8<T>(bias, n_wave + 64 * G + (GATED ? 32 * h + 8 * g : 16 * g + 8 * h), N, bias_vec_ok);
+                braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0}
+                             : fetch8<T>(bias, n_wave + 16 * JB * G + (GATED ? 32 * h + 8 * g : 4 * JB * g + 8 * h), N, bias_vec_ok);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         landed = true;
         // one call per 16-row block: each stays small enough for the compiler to unroll completely, so the
         // accumulators are only ever indexed by constants and never leave the register file
 #define KERNL_WIDE_EPILOGUE(I)                                                                                         \
-    wide_epilogue<T, ACT, I>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs, ai_cs,   \
+    wide_epilogue<T, ACT, I, NBN>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs, ai_cs,   \
                              out_vec_ok, ai_vec_ok, braw)
         KERNL_WIDE_EPILOGUE(0);
         KERNL_WIDE_EPILOGUE(1);
@@ -853,16 +866,16 @@ static void launch_mfma_glu(const LinearArgs &a) {
     }
 }
 
-template <typename T, int ACT>
+template <typename T, int ACT, int NBN = 8>
 static void launch_wide_act(const LinearArgs &a) {
-    auto kern = linear_wide_kernel<T, ACT>;
+    auto kern = linear_wide_kernel<T, ACT, NBN>;
     constexpr int LDS_BYTES = 2 * (256 + 256) * 128;
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         attr_done = true;
     }
-    const int tiles_m = (a.M + 255) / 256, tiles_n = (a.N + 255) / 256;
+    const int tiles_m = (a.M + 255) / 256, tiles_n = (a.N + 32 * NBN - 1) / (32 * NBN);
     const int per_xcd = (tiles_m * tiles_n + 7) / 8;
     const T *bias = static_cast<const T *>(a.bias);
     T *out = static_cast<T *>(a.out);
@@ -876,6 +889,18 @@ static void launch_wide_act(const LinearArgs &a) {
     hipLaunchKernelGGL(kern, dim3(slots * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
                        a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok);
+}
+
+template <typename T>
+static void launch_wide192(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_wide_act<T, KERNL_ACT_RELU, 6>(a); break;
+        case KERNL_ACT_TANH: launch_wide_act<T, KERNL_ACT_TANH, 6>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_wide_act<T, KERNL_ACT_GELU_ERF, 6>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_wide_act<T, KERNL_ACT_GELU_TANH, 6>(a); break;
+        case KERNL_ACT_SILU: launch_wide_act<T, KERNL_ACT_SILU, 6>(a); break;
+        default: launch_wide_act<T, KERNL_ACT_NONE, 6>(a); break;
+    }
 }
 
 template <typename T>
@@ -916,11 +941,16 @@ static double tile_cost(int M, int N, int K, int bm, int bn, double base, double
     const double kf = (double)K / ((double)K + 1500.0);
     return (double)per_cu * ((double)bm * bn / 65536.0) * (base + per_k * kf);
 }
-// which: 1 = 256x256, 2 = 256x192, 3 = 128x128 (8-wave kernel), 5 = wide 256x256 (needs K % 64 == 0)
+// which: 1 = 256x256, 2 = 256x192, 3 = 128x128 (8-wave kernel), 5 = wide 256x256, 6 = wide 256x192 (K % 64 == 0)
 static int pick_tile(int M, int N, int K, bool gated) {
     int pick = 1;
     double best = tile_cost(M, N, K, 256, 256, 1.15, 0.3);
-    if (K % 64 == 0) { best = tile_cost(M, N, K, 256, 256, 1.0, 0.0); pick = 5; }
+    if (K % 64 == 0) {
+        best = tile_cost(M, N, K, 256, 256, 1.0, 0.0);
+        pick = 5;
+        const double c6 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.04, 0.0);
+        if (c6 < best) { best = c6; pick = 6; }
+    }
     // 256x192 gives a wave an odd number of column blocks: not usable for gate/value pairs
     const double c2 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.2, 0.3);
     const double c3 = tile_cost(M, N, K, 128, 128, 1.9, 0.4);
@@ -929,7 +959,7 @@ static int pick_tile(int M, int N, int K, bool gated) {
     return pick;
 }
 
-int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256
+int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192
 
 template <typename T>
 static int linear_mfma_dispatch(const LinearArgs &a) {
@@ -942,6 +972,7 @@ static int linear_mfma_dispatch(const LinearArgs &a) {
         return check_launch("gated linear (mfma)");
     }
     if (pick == 5 && a.K % 64 == 0) launch_wide<T>(a);
+    else if (pick == 6 && a.K % 64 == 0) launch_wide192<T>(a);
     else if (pick == 1) launch_mfma_cfg<T, Tile256x256>(a);
     else if (pick == 2) launch_mfma_cfg<T, Tile256x192>(a);
     else if (pick == 4) launch_mfma_cfg<T, Tile256x128k32>(a);

@@ -41,7 +41,7 @@ def test_linear_vs_oracle(shape, bias, activation, dtype, close):
     close(out, ref, torch.float16 if dtype == torch.float32 else dtype, what=f"linear {shape} {activation!r}")
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5], ids=["256x256", "256x192", "128x128", "256x128k32", "wide256x256"])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6], ids=["256x256", "256x192", "128x128", "256x128k32", "wide256x256", "wide256x192"])
 @pytest.mark.parametrize(
     "shape", [(1000, 600, 776), (256, 256, 64), (513, 385, 1032), (700, 520, 1024), (300, 260, 32), (257, 513, 96), (640, 512, 160)],
     ids=lambda s: "x".join(map(str, s))
@@ -140,14 +140,15 @@ def test_unknown_activation_is_identity(close):
 
 @pytest.mark.parametrize("shape", [(4352, 4352, 128), (4352, 4300, 192), (4400, 4352, 64), (8200, 2304, 256)],
                          ids=lambda s: "x".join(map(str, s)))
-def test_linear_more_tiles_than_compute_units(shape, close):
+@pytest.mark.parametrize("tile", [5, 6], ids=["wide256x256", "wide256x192"])
+def test_linear_more_tiles_than_compute_units(shape, tile, close):
     """More than 256 output tiles of 256x256: workgroups of the persistent kernel walk several tiles each, with the
     operand stream running through the tile boundaries (even k-tile counts) or one tile per workgroup (odd counts)."""
     M, N, K = shape
     gen = torch.Generator().manual_seed(11)
     x, w, b = _inputs(M, N, K, torch.float16, gen, w_std=K ** -0.5)
     lib = _lib.load()
-    lib.kernl_linear_force_tile(5)
+    lib.kernl_linear_force_tile(tile)
     try:
         out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation="relu")
         torch.cuda.synchronize()
