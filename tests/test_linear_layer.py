@@ -155,3 +155,23 @@ def test_linear_more_tiles_than_compute_units(shape, tile, close):
     finally:
         lib.kernl_linear_force_tile(0)
     close(out, linear_oracle(x, w, b, "relu"), what=f"linear persistent {shape}")
+
+
+@pytest.mark.parametrize("activation", ["gelu", "fast_gelu", "silu", "tanh"])
+def test_activation_curve_through_identity_weights(activation):
+    """The epilogue's activation sampled on a grid (identity weight, no bias): the fp16 kernels use short
+    sigmoid-form approximations (erf-GELU: |error| <= 2.6e-5 by construction), which must hold over the whole range,
+    saturate cleanly for large |x| and stay within an fp16 rounding of the fp32 closed form."""
+    K = 64
+    grid = torch.cat((torch.linspace(-12, 12, 64 * 255), torch.tensor([0.0, -0.0, 30.0, -30.0, 1000.0, -1000.0, 60000.0, -60000.0] * 8)))
+    x = grid.reshape(-1, K).half()
+    w = torch.eye(K).half()
+    out = linear_layer(x.cuda(), w.cuda(), None, activation=activation)
+    torch.cuda.synchronize()
+    ref = linear_oracle(x, w, None, activation)
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    err = (got - ref).abs()
+    bound = 4e-5 + 1.0e-3 * ref.abs()  # approximation error + one fp16 rounding (2^-11 relative, with slack)
+    worst = (err - bound).max().item()
+    assert worst <= 0, f"{activation}: error exceeds bound by {worst:.3e} at x={x.float().flatten()[(err - bound).argmax()].item()}"
