@@ -281,6 +281,44 @@ def main():
         extra["copy_same_bytes_gbps_graph_replay"] = round(2 * x_ln.numel() * 2 / (t * 1e-3) / 1e9, 1)
         del flush
 
+        # ---- the decoder-side kernels (Llama-7B prefill / decode shapes), graph-replayed
+        try:
+            from kernl_amd.implementations.attention_skinny import skinny_attention_forward
+            from kernl_amd.implementations.linear_layer import interleave_glu_rows, linear_glu_layer
+            from kernl_amd.implementations.rotary import rotary_forward
+
+            x_ll = torch.randn((2048, 4096), generator=gen).half().to(dev)
+            w_gate = (torch.randn((11008, 4096), generator=gen) * 0.02).half()
+            w_val = (torch.randn((11008, 4096), generator=gen) * 0.02).half()
+            w_glu = interleave_glu_rows(w_gate, w_val).to(dev)
+            del w_gate, w_val
+            t = graph_time_ms(lambda: linear_glu_layer(x_ll, w_glu, None, "silu"), reps=5)
+            extra["swiglu_2048x4096_to_11008_us_graph_replay"] = round(t * 1e3, 2)
+            extra["swiglu_tflops_graph_replay"] = round(4.0 * 2048 * 11008 * 4096 / (t * 1e-3) / 1e12, 1)
+            extra["swiglu_frac_of_peak"] = round(4.0 * 2048 * 11008 * 4096 / (t * 1e-3) / 1e12 / PEAK_MFMA_F16_TFLOPS, 4)
+            del w_glu, x_ll
+
+            xr = torch.randn((1, 2048, 32, 128), generator=gen).half().to(dev).transpose(1, 2)  # [1,32,2048,128] view
+            ang = torch.outer(torch.arange(2048).float(), 1.0 / (10000.0 ** (torch.arange(0, 128, 2).float() / 128)))
+            emb = torch.cat((ang, ang), dim=-1)[None, None]
+            cos_t, sin_t = emb.cos().half().to(dev), emb.sin().half().to(dev)
+            t = graph_time_ms(lambda: rotary_forward(xr, cos_t, sin_t), reps=20)
+            extra["rotary_1x32x2048x128_us_graph_replay"] = round(t * 1e3, 2)
+            extra["rotary_gbps_graph_replay"] = round(2 * xr.numel() * 2 / (t * 1e-3) / 1e9, 1)
+
+            qd = torch.randn((32, 32, 1, 128), generator=gen).half().to(dev)
+            kd = torch.randn((32, 32, 4096, 128), generator=gen).half().to(dev)
+            vd = torch.randn((32, 32, 4096, 128), generator=gen).half().to(dev)
+            od = torch.empty_like(qd)
+            t = graph_time_ms(lambda: skinny_attention_forward(qd, kd, vd, od, 128 ** -0.5), reps=5)
+            kv_bytes = 2 * kd.numel() * 2
+            extra["decode_attention_32x32x1x4096x128_us_graph_replay"] = round(t * 1e3, 2)
+            extra["decode_attention_gbps_graph_replay"] = round(kv_bytes / (t * 1e-3) / 1e9, 1)
+            extra["decode_attention_frac_of_hbm_peak"] = round(kv_bytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
+            del qd, kd, vd, od
+        except Exception as exc:  # the headline must still be printed
+            extra["decoder_kernels_error"] = f"{type(exc).__name__}: {exc}"[:300]
+
     # ------------------------------------------------------------------ BERT-base b32 s512 through optimize_model
     if not args.skip_e2e and not args.skip_extra:
         try:
