@@ -169,3 +169,87 @@ def test_llama_7b_shaped_layer_full_width():
     assert torch.isfinite(out).all()
     assert ours_rel <= max(5e-3, 1.1 * eager_rel)
     assert early <= 5e-3
+
+
+def _rel_errors(out, eager16, ref):
+    ours = ((out.float().cpu() - ref).abs().mean() / ref.abs().mean()).item()
+    eager = ((eager16 - ref).abs().mean() / ref.abs().mean()).item()
+    return ours, eager
+
+
+@pytest.mark.parametrize("attn", ["eager", "sdpa"])
+def test_t5_shaped_encoder_decoder_matches_fp32_eager(attn):
+    """T5 (reference: test/test_torchdynamo.py:102-131, t5-small): relative position bias as a matrix mask in encoder
+    and decoder self-attention, cross-attention without a mask, T5-spelled RMSNorm, ReLU feed-forward.  Random-init
+    t5-small-shaped model, two layers, encoder 128 tokens, decoder 48."""
+    from transformers import T5Config, T5Model
+
+    from kernl_amd.model_optimization import optimize_model
+
+    torch._dynamo.reset()
+
+    def make():
+        torch.manual_seed(0)
+        cfg = T5Config(d_model=512, d_kv=64, d_ff=2048, num_layers=2, num_heads=8, vocab_size=1000,
+                       layer_norm_epsilon=1.6e-5)  # the fp16 operator clamps eps to >= 1.6e-5 (layer_norm.py:295-296)
+        cfg._attn_implementation = attn
+        return T5Model(cfg).eval()
+
+    gen = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, 1000, (4, 128), generator=gen)
+    dec = torch.randint(0, 1000, (4, 48), generator=gen)
+    with torch.inference_mode():
+        ref = make()(input_ids=ids, decoder_input_ids=dec, use_cache=False).last_hidden_state
+    model = make().half().cuda()
+    with torch.inference_mode():
+        eager16 = model(input_ids=ids.cuda(), decoder_input_ids=dec.cuda(), use_cache=False).last_hidden_state.float().cpu()
+    optimize_model(model)
+    with torch.inference_mode():
+        out = model(input_ids=ids.cuda(), decoder_input_ids=dec.cuda(), use_cache=False).last_hidden_state
+        out = model(input_ids=ids.cuda(), decoder_input_ids=dec.cuda(), use_cache=False).last_hidden_state
+        torch.cuda.synchronize()
+    ours, eager = _rel_errors(out, eager16, ref)
+    print(f"t5-shaped {attn}: mean_rel ours={ours:.5f} fp16-eager={eager:.5f}", flush=True)
+    assert torch.isfinite(out).all()
+    assert ours <= 5e-3
+    assert (out.float().cpu() - ref).abs().max().item() <= 1e-1 * max(1.0, ref.abs().max().item())
+
+
+@pytest.mark.parametrize("attn", ["eager", "sdpa"])
+def test_whisper_shaped_encoder_decoder_matches_fp32_eager(attn):
+    """Whisper (reference: test/test_torchdynamo.py:134-165, whisper-tiny): 1500 encoder positions (not a multiple of
+    any tile), bmm-shaped attention without a mask in the encoder, causal decoder self-attention, cross-attention,
+    LayerNorm with residual adds, GELU feed-forward.  Random-init whisper-tiny-shaped model with two layers."""
+    from transformers import WhisperConfig, WhisperModel
+
+    from kernl_amd.model_optimization import optimize_model
+
+    torch._dynamo.reset()
+
+    def make():
+        torch.manual_seed(0)
+        cfg = WhisperConfig(d_model=384, encoder_layers=2, decoder_layers=2, encoder_attention_heads=6,
+                            decoder_attention_heads=6, encoder_ffn_dim=1536, decoder_ffn_dim=1536, vocab_size=1000,
+                            pad_token_id=0, bos_token_id=1, eos_token_id=2, decoder_start_token_id=1, num_mel_bins=80,
+                            max_source_positions=1500, max_target_positions=64)
+        cfg._attn_implementation = attn
+        return WhisperModel(cfg).eval()
+
+    gen = torch.Generator().manual_seed(6)
+    feats = torch.randn((2, 80, 3000), generator=gen)
+    dec = torch.randint(3, 1000, (2, 24), generator=gen)
+    with torch.inference_mode():
+        ref = make()(input_features=feats, decoder_input_ids=dec, use_cache=False).last_hidden_state
+    model = make().half().cuda()
+    with torch.inference_mode():
+        eager16 = model(input_features=feats.half().cuda(), decoder_input_ids=dec.cuda(), use_cache=False).last_hidden_state.float().cpu()
+    optimize_model(model)
+    with torch.inference_mode():
+        out = model(input_features=feats.half().cuda(), decoder_input_ids=dec.cuda(), use_cache=False).last_hidden_state
+        out = model(input_features=feats.half().cuda(), decoder_input_ids=dec.cuda(), use_cache=False).last_hidden_state
+        torch.cuda.synchronize()
+    ours, eager = _rel_errors(out, eager16, ref)
+    print(f"whisper-shaped {attn}: mean_rel ours={ours:.5f} fp16-eager={eager:.5f}", flush=True)
+    assert torch.isfinite(out).all()
+    assert ours <= 5e-3
+    assert (out.float().cpu() - ref).abs().max().item() <= 1e-1 * max(1.0, ref.abs().max().item())
