@@ -38,6 +38,15 @@ def optimize_model(model: torch.nn.Module) -> None:
     _lib.load()  # fail now, not in the middle of the first forward
     static_inputs_pool.clear()
     model.forward_original = model.forward
+    # Generation with a growing key/value cache meets a new shape at every step.  TorchDynamo gives up on a function
+    # (and silently runs it unoptimised) after `recompile_limit` compilations, 8 by default: far fewer than the steps
+    # of a generate() call.  The reference's own benchmarks raise the same limit to 512
+    # (experimental/benchmarks/inductor.py sets torchdynamo.config.cache_size_limit = 512).
+    for name in ("recompile_limit", "cache_size_limit"):
+        if hasattr(torchdynamo.config, name) and getattr(torchdynamo.config, name) < 512:
+            setattr(torchdynamo.config, name, 512)
+    if hasattr(torchdynamo.config, "accumulated_recompile_limit") and torchdynamo.config.accumulated_recompile_limit < 4096:
+        torchdynamo.config.accumulated_recompile_limit = 4096
 
     # Static shapes: a hipGraph is specific to its shapes, so every new input shape is a new (cached) compilation,
     # exactly as with the reference's default TorchDynamo settings.

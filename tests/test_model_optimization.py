@@ -253,3 +253,70 @@ def test_whisper_shaped_encoder_decoder_matches_fp32_eager(attn):
     assert torch.isfinite(out).all()
     assert ours <= 5e-3
     assert (out.float().cpu() - ref).abs().max().item() <= 1e-1 * max(1.0, ref.abs().max().item())
+
+
+@pytest.mark.parametrize("family", ["t5", "whisper"])
+def test_generation_with_growing_cache(family):
+    """Greedy generation under autocast with `optimize_model` on encoder and decoder, as the reference tests it
+    (test/test_torchdynamo.py:102-165): every decoding step meets a longer key/value cache, i.e. a new shape, a new
+    compilation and a new captured graph; single-query attention runs on the split-K kernel.  Checks that no step falls
+    back to the unoptimised function (TorchDynamo's recompile limit) and that the per-step scores follow the eager
+    model's for as long as the two greedy paths pick the same tokens."""
+    from torch._dynamo.utils import counters
+
+    from kernl_amd.model_optimization import optimize_model
+
+    torch._dynamo.reset()
+    counters.clear()
+    torch.manual_seed(0)
+    gen = torch.Generator().manual_seed(1)
+    if family == "t5":
+        from transformers import T5Config, T5ForConditionalGeneration
+
+        cfg = T5Config(d_model=512, d_kv=64, d_ff=2048, num_layers=2, num_heads=8, vocab_size=1000,
+                       decoder_start_token_id=0, pad_token_id=0, eos_token_id=1, tie_word_embeddings=False)
+        model = T5ForConditionalGeneration(cfg).eval().cuda()
+        ids = torch.randint(2, 1000, (2, 64), generator=gen).cuda()
+        kwargs = dict(input_ids=ids, attention_mask=torch.ones_like(ids))
+        encoder, decoder = model.encoder, model.decoder
+    else:
+        from transformers import WhisperConfig, WhisperForConditionalGeneration
+
+        cfg = WhisperConfig(d_model=384, encoder_layers=2, decoder_layers=2, encoder_attention_heads=6,
+                            decoder_attention_heads=6, encoder_ffn_dim=1536, decoder_ffn_dim=1536, vocab_size=1000,
+                            pad_token_id=0, bos_token_id=1, eos_token_id=2, decoder_start_token_id=1, num_mel_bins=80,
+                            max_source_positions=1500, max_target_positions=64, suppress_tokens=None,
+                            begin_suppress_tokens=None)
+        model = WhisperForConditionalGeneration(cfg).eval().cuda()
+        model.generation_config.suppress_tokens = None
+        model.generation_config.begin_suppress_tokens = None
+        model.generation_config.forced_decoder_ids = None
+        kwargs = dict(input_features=torch.randn((2, 80, 3000), generator=gen).cuda())
+        encoder, decoder = model.model.encoder, model.model.decoder
+    steps = 20
+    kwargs.update(min_new_tokens=steps, max_new_tokens=steps, do_sample=False, output_scores=True, return_dict_in_generate=True)
+    with torch.inference_mode(), torch.autocast(dtype=torch.float16, device_type="cuda"):
+        ref = model.generate(**kwargs)
+    optimize_model(encoder)
+    optimize_model(decoder)
+    with torch.inference_mode(), torch.autocast(dtype=torch.float16, device_type="cuda"):
+        model.generate(**kwargs)        # compiles and captures one graph per step
+        out = model.generate(**kwargs)  # replays them
+        torch.cuda.synchronize()
+    frames = counters["frames"]
+    assert frames["ok"] == frames["total"], f"some steps were not compiled: {dict(frames)}"
+    assert counters["stats"]["unique_graphs"] >= steps, dict(counters["stats"])
+    assert len(out.scores) == len(ref.scores) == steps
+    prompt = ref.sequences.shape[1] - steps
+    agree = 0
+    for t, (a, b) in enumerate(zip(out.scores, ref.scores)):
+        if not torch.equal(out.sequences[:, : prompt + t], ref.sequences[:, : prompt + t]):
+            break
+        finite = torch.isfinite(b)
+        assert torch.equal(torch.isfinite(a), finite)
+        scale = b[finite].abs().max().item()
+        diff = (a.float() - b.float())[finite].abs().max().item()
+        assert diff <= 4e-3 * max(scale, 1.0), f"{family} step {t}: scores differ by {diff} (scale {scale})"
+        agree += 1
+    print(f"{family}: greedy paths agree for {agree} of {steps} steps", flush=True)
+    assert agree >= 3
