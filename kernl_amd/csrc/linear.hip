@@ -453,8 +453,8 @@ __device__ __forceinline__ u32x4 fetch8(const T *__restrict__ p, int idx, int li
 
 // Epilogue of m-block IB (16 rows) of a wave of the wide kernel: lane (l16, g) holds row m_wave + 16 IB + l16 and, in
 // every group of JB n-blocks, the 4 JB consecutive columns starting at 4 JB g (JB = 4: 64-column groups, 2: 32-column).
-template <typename T, int ACT, int IB, int NBN>
-__device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[8][NBN], int m_wave, int n_wave, int l16, int g,
+template <typename T, int ACT, int IB, int NBN, int NBM = 8>
+__device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_wave, int n_wave, int l16, int g,
                                               T *__restrict__ out, T *__restrict__ act_in, int M, int N,
                                               int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs,
                                               int out_vec_ok, int ai_vec_ok,
@@ -779,6 +779,193 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 }
 
 // ----------------------------------------------------------------------------------------------------
+// Half-height variant of the wide kernel for outputs that leave CUs idle with 256-row tiles (M = 2048 against
+// N = 4096 gives 128 tiles of 256x256 but 256 of 128x256): 128 x (256 | 192) tile, 4 waves as 2 x 2, a 64-row
+// sub-tile per wave (4 x NBN blocks of v_mfma_f32_16x16x32).  A k-tile is only 2 x 32 (24) MFMAs long here, too short
+// to cover the load latency with two stages, and the smaller x tile leaves room for a third: THREE stages of
+// 16 KB (x) + 32 KB (w), k-tile T + 3 requested while k-tile T is multiplied, the wait in front of the second k-step
+// only for k-tile T + 1 (vmcnt(NL): the loads of T + 2 may still be in flight).  One workgroup per output tile.
+// ----------------------------------------------------------------------------------------------------
+template <typename T, int ACT, int NBN>
+__global__ void __launch_bounds__(256, 1)
+linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
+                        T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs,
+                        int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok,
+                        int ai_vec_ok, int bias_vec_ok) {
+    typedef typename Vec8<T>::type vec8;
+    static_assert((ACT & kGluBit) == 0 && (NBN == 8 || NBN == 6), "plain epilogues, 256 or 192 columns");
+    constexpr int NBM = 4, BM = 32 * NBM, BN = 32 * NBN, BK = 64, RB = BK * 2, CPR = BK / 8, KSTEPS = BK / 32;
+    constexpr int X_STAGE = BM * RB, W_STAGE = 32768, W_BASE = 3 * X_STAGE;  // [x0|x1|x2|w0|w1|w2]
+    static_assert(X_STAGE == 16384 && BN * RB <= W_STAGE, "stage immediates");
+    constexpr int LOADS_X = BM * CPR / 256, LOADS_W = BN * CPR / 256, NL = LOADS_X + LOADS_W;
+    static_assert(LOADS_X == 4, "one group of four loads for the x tile");
+    constexpr int GROUP_M = 8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) >> 3;
+    const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || t >= total) return;
+    const int group_span = GROUP_M * tiles_n;
+    const int group = t / group_span;
+    const int first_m = group * GROUP_M;
+    const int gsize = min(tiles_m - first_m, GROUP_M);
+    const int in_group = t - group * group_span;
+    const int m0 = (first_m + in_group % gsize) * BM, n0 = (in_group / gsize) * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave & 1, wave_n = wave >> 1;
+    const int l16 = lane & 15, g = lane >> 4;
+
+    // tile loads, as in the wide kernel: every lane fetches the chunk that belongs at its LDS position
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    const int rows_x = min(BM, M - m0), rows_w = min(BN, N - n0);
+    const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx), waddr = (uint64_t)(uintptr_t)(W + (int64_t)n0 * K);
+    const u32x4 xrsrc = {(uint32_t)xaddr, (uint32_t)(xaddr >> 32) & 0xFFFFu,
+                         (uint32_t)((((int64_t)rows_x - 1) * ldx + K) * 2), 0x00020000u};
+    const u32x4 wrsrc = {(uint32_t)waddr, (uint32_t)(waddr >> 32) & 0xFFFFu, (uint32_t)((int64_t)rows_w * K * 2),
+                         0x00020000u};
+    uint32_t xd[LOADS_X], wd[LOADS_W];
+#pragma unroll
+    for (int i = 0; i < LOADS_X; ++i) {
+        const int q = (wave * LOADS_X + i) * 64 + lane;
+        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
+    }
+#pragma unroll
+    for (int i = 0; i < LOADS_W; ++i) {
+        const int q = (wave * LOADS_W + i) * 64 + lane;
+        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        const int r = row & 15, j = (row >> 4) & 3;
+        const int wrow = NBN == 8 ? (row & ~63) + 16 * (r >> 2) + 4 * j + (r & 3) : (row & ~31) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3);
+        wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
+    }
+    typedef __attribute__((address_space(3))) void lds_void;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
+    auto load4 = [&](const u32x4 &rsrc, uint32_t off, uint32_t lds, int group4, int part, int k0) __attribute__((always_inline)) {
+        if (part == 0)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :: "s"(lds + group4 * 4096), "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory", "m0");
+        else if (part == 1)
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
+        else if (part == 2)
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:2048 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
+        else
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
+    };
+    auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
+        if (l < LOADS_X) load4(xrsrc, xd[l], lds_base + stage * X_STAGE + wave * (LOADS_X * 1024), 0, l, k0);
+        else load4(wrsrc, wd[l - LOADS_X], lds_base + W_BASE + stage * W_STAGE + wave * (LOADS_W * 1024), (l - LOADS_X) >> 2, (l - LOADS_X) & 3, k0);
+    };
+
+    // fragment addresses: x stages are 16 KB apart (immediates 0 / 16 K / 32 K); w stages 32 KB apart, and an LDS
+    // read's immediate ends at 64 KB - 1, so the third w stage has address registers of its own
+    typedef __attribute__((address_space(3))) const unsigned char *lds_bytes;
+    typedef __attribute__((address_space(3))) const vec8 *lds_frag;
+    const lds_bytes lds0 = (lds_bytes)smem;
+    lds_frag xfrag[KSTEPS][NBM], wfrag[KSTEPS][NBN], wfrag2[KSTEPS][NBN];
+#pragma unroll
+    for (int st = 0; st < KSTEPS; ++st) {
+#pragma unroll
+        for (int i = 0; i < NBM; ++i) xfrag[st][i] = (lds_frag)(lds0 + swz_offset<RB>(wave_m * (NBM * 16) + i * 16 + l16, 4 * st + g));
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) {
+            wfrag[st][j] = (lds_frag)(lds0 + W_BASE + swz_offset<RB>(wave_n * (NBN * 16) + j * 16 + l16, 4 * st + g));
+            wfrag2[st][j] = wfrag[st][j] + 2 * (W_STAGE / 16);
+        }
+    }
+
+    // Every k-tile slot issues its NL loads, so that the counter waits stay exact up to the end; requests past the
+    // last k-tile fetch that tile again (into a stage nobody reads any more) instead of running past the row ends.
+    const int nk = K / BK;
+#pragma unroll
+    for (int s3 = 0; s3 < 3; ++s3)
+#pragma unroll
+        for (int l = 0; l < NL; ++l) tile_load(l, s3, min(s3, nk - 1) * BK);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * NL) & 15) | (((2 * NL) >> 4) << 14));  // vmcnt(2 NL): k-tile 0 has landed
+    __syncthreads();
+
+    vec8 fa[KSTEPS][NBN], fb[KSTEPS][NBM];
+#pragma unroll
+    for (int j = 0; j < NBN; ++j) fa[0][j] = *wfrag[0][j];
+#pragma unroll
+    for (int i = 0; i < NBM; ++i) fb[0][i] = *xfrag[0][i];
+
+    f32x4_acc acc[NBM][NBN];
+#pragma unroll
+    for (int i = 0; i < NBM; ++i)
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // fragment reads of stage S3 for k-step st (compile-time stage: immediates, or the second register set)
+    auto read_w = [&](auto s3_c, int st, int j) __attribute__((always_inline)) -> vec8 {
+        constexpr int S3 = decltype(s3_c)::value;
+        return S3 == 2 ? *wfrag2[st][j] : *(wfrag[st][j] + S3 * (W_STAGE / 16));
+    };
+    auto read_x = [&](auto s3_c, int st, int i) __attribute__((always_inline)) -> vec8 {
+        constexpr int S3 = decltype(s3_c)::value;
+        return *(xfrag[st][i] + S3 * (X_STAGE / 16));
+    };
+    auto k_tile = [&](auto cur_c, int kt) __attribute__((always_inline)) {
+        constexpr int CUR = decltype(cur_c)::value, NXT = (CUR + 1) % 3;
+        const int k_next = min(kt + 3, nk - 1) * BK;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            const int sn = st ^ 1;
+            if (st == 1) {
+                __builtin_amdgcn_s_waitcnt(0x0F70 | (NL & 15) | ((NL >> 4) << 14));  // vmcnt(NL): k-tile kt + 1 has landed
+                __syncthreads();
+            }
+#pragma unroll
+            for (int m = 0; m < NBM * NBN; ++m) {
+                const int i = m / NBN, j = m % NBN;
+                mfma16_inplace(fa[st][j], fb[st][i], acc[i][j]);
+                const int slot = m >> 1;
+                if ((m & 1) == 0 && slot < NBN + NBM) {
+                    if (st == 0) {
+                        if (slot < NBN) fa[sn][slot] = read_w(IntC<CUR>(), sn, slot);
+                        else fb[sn][slot - NBN] = read_x(IntC<CUR>(), sn, slot - NBN);
+                    } else {
+                        if (slot < NBN) fa[sn][slot] = read_w(IntC<NXT>(), sn, slot);
+                        else fb[sn][slot - NBN] = read_x(IntC<NXT>(), sn, slot - NBN);
+                    }
+                } else if ((m & 1) == 1 && st == 1 && slot < NL) {
+                    tile_load(slot, CUR, k_next);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    int kt = 0;
+    for (; kt + 2 < nk; kt += 3) {
+        k_tile(IntC<0>(), kt);
+        k_tile(IntC<1>(), kt + 1);
+        k_tile(IntC<2>(), kt + 2);
+    }
+    if (kt < nk) k_tile(IntC<0>(), kt);
+    if (kt + 1 < nk) k_tile(IntC<1>(), kt + 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no load may still be writing LDS when the workgroup ends
+
+    const int n_wave = n0 + wave_n * (NBN * 16);
+    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB;
+    u32x4 braw[NG][2];
+#pragma unroll
+    for (int G = 0; G < NG; ++G)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0} : fetch8<T>(bias, n_wave + 16 * JB * G + 4 * JB * g + 8 * h, N, bias_vec_ok);
+#define KERNL_HALF_EPILOGUE(I)                                                                                         \
+    wide_epilogue<T, ACT, I, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, \
+                                       ai_rs, ai_cs, out_vec_ok, ai_vec_ok, braw)
+    KERNL_HALF_EPILOGUE(0);
+    KERNL_HALF_EPILOGUE(1);
+    KERNL_HALF_EPILOGUE(2);
+    KERNL_HALF_EPILOGUE(3);
+#undef KERNL_HALF_EPILOGUE
+}
+
+// ----------------------------------------------------------------------------------------------------
 // FMA kernel: any dtype, any strides.  64x64 output tile, 16x16 threads, 4x4 outputs per thread, fp32 LDS tiles.
 // ----------------------------------------------------------------------------------------------------
 template <typename T>
@@ -913,6 +1100,40 @@ static void launch_wide_act(const LinearArgs &a) {
                        a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok);
 }
 
+template <typename T, int ACT, int NBN>
+static void launch_wide_half_act(const LinearArgs &a) {
+    auto kern = linear_wide_half_kernel<T, ACT, NBN>;
+    constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768;
+    static bool attr_done = false;  // benign race: the attribute call is idempotent
+    if (!attr_done) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        attr_done = true;
+    }
+    const int tiles_m = (a.M + 127) / 128, tiles_n = (a.N + 32 * NBN - 1) / (32 * NBN);
+    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+    const T *bias = static_cast<const T *>(a.bias);
+    T *out = static_cast<T *>(a.out);
+    T *act_in = static_cast<T *>(a.act_in);
+    const int out_vec_ok = a.out_cs == 1 && a.out_rs % 8 == 0 && aligned16(out);
+    const int ai_vec_ok = act_in != nullptr && a.ai_cs == 1 && a.ai_rs % 8 == 0 && aligned16(act_in);
+    const int bias_vec_ok = bias != nullptr && aligned16(bias);
+    hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
+                       static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
+                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok);
+}
+
+template <typename T, int NBN>
+static void launch_wide_half(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_wide_half_act<T, KERNL_ACT_RELU, NBN>(a); break;
+        case KERNL_ACT_TANH: launch_wide_half_act<T, KERNL_ACT_TANH, NBN>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_wide_half_act<T, KERNL_ACT_GELU_ERF, NBN>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_wide_half_act<T, KERNL_ACT_GELU_TANH, NBN>(a); break;
+        case KERNL_ACT_SILU: launch_wide_half_act<T, KERNL_ACT_SILU, NBN>(a); break;
+        default: launch_wide_half_act<T, KERNL_ACT_NONE, NBN>(a); break;
+    }
+}
+
 template <typename T>
 static void launch_wide192(const LinearArgs &a) {
     switch (a.act) {
@@ -963,7 +1184,7 @@ static double tile_cost(int M, int N, int K, int bm, int bn, double base, double
     const double kf = (double)K / ((double)K + 1500.0);
     return (double)per_cu * ((double)bm * bn / 65536.0) * (base + per_k * kf);
 }
-// which: 1 = 256x256, 2 = 256x192, 3 = 128x128 (8-wave kernel), 5 = wide 256x256, 6 = wide 256x192 (K % 64 == 0)
+// which: 1 = 256x256, 2 = 256x192, 3 = 128x128 (8-wave kernel), 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192 (K % 64 == 0)
 static int pick_tile(int M, int N, int K, bool gated) {
     int pick = 1;
     double best = tile_cost(M, N, K, 256, 256, 1.15, 0.3);
@@ -972,6 +1193,12 @@ static int pick_tile(int M, int N, int K, bool gated) {
         pick = 5;
         const double c6 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.04, 0.0);
         if (c6 < best) { best = c6; pick = 6; }
+        // half-height tiles: a quarter slower per output element at long K (more operand traffic per MFMA), and a
+        // prologue per tile that weighs more the shorter K is; they win where 256-row tiles leave CUs idle
+        const double c7 = gated ? 1e30 : tile_cost(M, N, K, 128, 256, 1.5, -0.35);
+        if (c7 < best) { best = c7; pick = 7; }
+        const double c8 = gated ? 1e30 : tile_cost(M, N, K, 128, 192, 1.65, -0.35);
+        if (c8 < best) { best = c8; pick = 8; }
     }
     // 256x192 gives a wave an odd number of column blocks: not usable for gate/value pairs
     const double c2 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.2, 0.3);
@@ -981,7 +1208,7 @@ static int pick_tile(int M, int N, int K, bool gated) {
     return pick;
 }
 
-int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192
+int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192
 
 template <typename T>
 static int linear_mfma_dispatch(const LinearArgs &a) {
@@ -995,6 +1222,8 @@ static int linear_mfma_dispatch(const LinearArgs &a) {
     }
     if (pick == 5 && a.K % 64 == 0) launch_wide<T>(a);
     else if (pick == 6 && a.K % 64 == 0) launch_wide192<T>(a);
+    else if (pick == 7 && a.K % 64 == 0) launch_wide_half<T, 8>(a);
+    else if (pick == 8 && a.K % 64 == 0) launch_wide_half<T, 6>(a);
     else if (pick == 1) launch_mfma_cfg<T, Tile256x256>(a);
     else if (pick == 2) launch_mfma_cfg<T, Tile256x192>(a);
     else if (pick == 4) launch_mfma_cfg<T, Tile256x128k32>(a);

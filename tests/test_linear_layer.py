@@ -41,9 +41,14 @@ def test_linear_vs_oracle(shape, bias, activation, dtype, close):
     close(out, ref, torch.float16 if dtype == torch.float32 else dtype, what=f"linear {shape} {activation!r}")
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6], ids=["256x256", "256x192", "128x128", "256x128k32", "wide256x256", "wide256x192"])
+TILE_IDS = ["256x256", "256x192", "128x128", "256x128k32", "wide256x256", "wide256x192", "wide128x256", "wide128x192"]
+
+
+@pytest.mark.parametrize("tile", list(range(1, 9)), ids=TILE_IDS)
 @pytest.mark.parametrize(
-    "shape", [(1000, 600, 776), (256, 256, 64), (513, 385, 1032), (700, 520, 1024), (300, 260, 32), (257, 513, 96), (640, 512, 160)],
+    "shape",
+    [(1000, 600, 776), (256, 256, 64), (513, 385, 1032), (700, 520, 1024), (300, 260, 32), (257, 513, 96), (640, 512, 160),
+     (513, 385, 128), (384, 640, 192), (130, 200, 320)],
     ids=lambda s: "x".join(map(str, s))
 )
 def test_linear_every_tile_shape(shape, tile, close):
@@ -93,6 +98,24 @@ def test_linear_saves_activation_inputs(close):
     close(act_in, pre, what="linear act_inputs")
 
 
+@pytest.mark.parametrize("tile", [5, 6, 7, 8], ids=TILE_IDS[4:])
+def test_linear_wide_tiles_save_activation_inputs(tile, close):
+    gen = torch.Generator().manual_seed(13)
+    M, N, K = 300, 520, 448
+    x, w, b = _inputs(M, N, K, torch.bfloat16, gen, w_std=K ** -0.5)
+    act_in = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    lib = _lib.load()
+    lib.kernl_linear_force_tile(tile)
+    try:
+        out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation="relu", act_inputs=act_in)
+        torch.cuda.synchronize()
+    finally:
+        lib.kernl_linear_force_tile(0)
+    ref, pre = linear_oracle(x, w, b, "relu", return_act_inputs=True)
+    close(out, ref, torch.bfloat16, what=f"tile {tile} out")
+    close(act_in, pre, torch.bfloat16, what=f"tile {tile} act_inputs")
+
+
 @pytest.mark.parametrize("which", ["up", "down"])
 def test_linear_config2_full_size(which, close):
     # BASELINE config 2: up-projection [16384,768]x[3072,768]ᵀ + bias + tanh-GELU; down-projection back, no activation
@@ -140,7 +163,7 @@ def test_unknown_activation_is_identity(close):
 
 @pytest.mark.parametrize("shape", [(4352, 4352, 128), (4352, 4300, 192), (4400, 4352, 64), (8200, 2304, 256)],
                          ids=lambda s: "x".join(map(str, s)))
-@pytest.mark.parametrize("tile", [5, 6], ids=["wide256x256", "wide256x192"])
+@pytest.mark.parametrize("tile", [5, 6, 7, 8], ids=TILE_IDS[4:])
 def test_linear_more_tiles_than_compute_units(shape, tile, close):
     """More than 256 output tiles of 256x256: workgroups of the persistent kernel walk several tiles each, with the
     operand stream running through the tile boundaries (even k-tile counts) or one tile per workgroup (odd counts)."""
