@@ -111,6 +111,12 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 #pragma unroll
         for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const vec8 *>(qrow + s * 16);
     }
+    // Q is multiplied by scale * log2(e) once, here (one more rounding of Q to 16 bits), so that the MFMA result is
+    // the score in the base-2 domain and the tile loop spends no instruction on scaling.
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[s][e] = from_float<T>(to_float(qf[s][e]) * p.scale_log2);
 
     // ---- staging: the i-th load of a wave fills the 1 KB of 16-byte chunks [256 i + 64 wave, +64) of a tile;
     // every lane fetches the chunk of global memory that belongs at its LDS position under the tile's swizzle
@@ -285,13 +291,22 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     };
 
     // ---- running state of this lane's query row
-    float m_i = -INFINITY, l_i = 0.0f;
+    // m_i is the exponent REFERENCE of the row (base-2 domain); its negative, replicated over a block of 16
+    // registers, is the C operand of the first score MFMA of every block, so that the MFMA delivers
+    // score - reference and the exponential needs no subtraction either.
+    // (Head size 128 with a matrix mask has no registers left for that block: there the reference is subtracted
+    // from every score by an instruction of its own.)
+    constexpr bool REF_IN_MFMA = !(D == 128 && MASK_MODE == MASK_MATRIX);
+    float m_i = 0.0f, l_i = 0.0f;
+    bool fresh = true;
+    f32x16 neg_m;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) neg_m[v] = 0.0f;
     f32x16 o_acc[DB];
 #pragma unroll
     for (int d = 0; d < DB; ++d)
 #pragma unroll
         for (int v = 0; v < 16; ++v) o_acc[d][v] = 0.0f;
-    const float c = p.scale_log2;
 
     // LDS byte offsets of this lane's operand fragments.  K: row lr of a 32-key block, chunk 2 ks + lh.  V: in each
     // group of 16 lanes, lane i hands the transposing read the address of 4 consecutive features of key (i / 4)
@@ -369,11 +384,9 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 #pragma unroll
             for (int nb = 0; nb < NBS; ++nb) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) s_acc[nb][v] = 0.0f;
-#pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     const vec8 kf = *reinterpret_cast<const vec8 *>(sb + nb * 32 * KROW + k_off[ks]);
-                    s_acc[nb] = mfma32(kf, qf[ks], s_acc[nb]);
+                    s_acc[nb] = mfma32(kf, qf[ks], ks == 0 ? neg_m : s_acc[nb]);  // neg_m stays 0 without REF_IN_MFMA
                 }
             }
             __builtin_amdgcn_s_setprio(0);
@@ -403,7 +416,8 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                         }
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
-                            float sv = s_acc[nb][g * 4 + r] * c + cb[r];
+                            float sv = s_acc[nb][g * 4 + r] + cb[r];
+                            if (!REF_IN_MFMA) sv -= m_i;
                             if (MATRIX) {
                                 if (ROUTE != 0) {
                                     sv = fmaf(fmaxf(mm[r], clamp_eff), kLog2eA, sv);
@@ -422,31 +436,42 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 #pragma unroll
                 for (int nb = 0; nb < NBS; ++nb)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[nb][v]);
-                mx *= c;  // c > 0 (checked by the host)
+                    for (int v = 0; v < 16; ++v) {
+                        if (!REF_IN_MFMA) s_acc[nb][v] -= m_i;
+                        mx = fmaxf(mx, s_acc[nb][v]);
+                    }
             }
             if (LATE_DMA) dma(tile_next, ST ^ 1);
             mx = halves32_max(mx);  // the other 16-key half of every 32-key block lives in lane ^ 32
-            // m_i is the exponent REFERENCE of this row, not necessarily its running maximum: it only moves (and the
-            // accumulator and row sum are rescaled) when the new maximum exceeds it by more than 2^8, so
-            // probabilities stay <= 256 — exact in fp32, well inside the 16-bit range — and after the first tiles
-            // the rescale almost never runs.  The final O / l is independent of the reference.
-            if (__builtin_amdgcn_ballot_w64(mx > m_i + kRescaleThreshold) != 0) {
-                const float m_new = fmaxf(m_i, mx);
-                const float alpha = __builtin_amdgcn_exp2f(m_i - ((m_new == -INFINITY) ? 0.0f : m_new));
+            // The scores are relative to the reference m_i, which is not the running maximum: it only moves (and
+            // the accumulator and row sum are rescaled) when a score exceeds it by more than 2^8, so probabilities
+            // stay <= 256 — exact in fp32, well inside the 16-bit range — and after the first tiles the rescale
+            // almost never runs.  While the row has seen no finite score yet (`fresh`; both lanes of a row agree on
+            // it, as they agree on mx) nothing has been accumulated, and the reference also moves DOWN to the tile's
+            // maximum: that costs nothing then and keeps rows of very negative scores from underflowing.
+            // The final O / l is independent of the reference.
+            const bool finite_max = mx > -INFINITY;
+            if (__builtin_amdgcn_ballot_w64(mx > kRescaleThreshold || (fresh && finite_max && mx < -kRescaleThreshold)) != 0) {
+                const float delta = fresh ? (finite_max ? mx : 0.0f) : fmaxf(mx, 0.0f);
+                const float alpha = fresh ? 1.0f : __builtin_amdgcn_exp2f(-delta);
                 l_i *= alpha;
 #pragma unroll
                 for (int d = 0; d < DB; ++d)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
-                m_i = m_new;
+#pragma unroll
+                for (int nb = 0; nb < NBS; ++nb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s_acc[nb][v] -= delta;
+                m_i += delta;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) neg_m[v] = REF_IN_MFMA ? -m_i : 0.0f;
             }
-            const float m_use = (m_i == -INFINITY) ? 0.0f : m_i;
+            fresh = fresh && !finite_max;
 #pragma unroll
             for (int nb = 0; nb < NBS; ++nb)
 #pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    s_acc[nb][v] = __builtin_amdgcn_exp2f(GENERAL ? s_acc[nb][v] - m_use : s_acc[nb][v] * c - m_use);
+                for (int v = 0; v < 16; ++v) s_acc[nb][v] = __builtin_amdgcn_exp2f(s_acc[nb][v]);
 
             // ---- Oᵀ += Vᵀ · Pᵀ; the row sum is taken from the ROUNDED probabilities (two per v_dot2c), i.e. from
             // exactly the values that enter the product
@@ -716,11 +741,11 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
         if (D == 64 && g_attention_variant == 1) wpe = 4;
         if (D == 64 && g_attention_variant == 2) wpe = 2;
         if (dtype == KERNL_F16) {
-            if (D == 64 && wpe == 4) launch_stream<f16, 64, 4>(p, mask_mode, causal, st);
+            if (D == 64 && wpe == 4) launch_stream<f16, 64, 3>(p, mask_mode, causal, st);
             else if (D == 64) launch_stream<f16, 64, 2>(p, mask_mode, causal, st);
             else launch_stream<f16, 128, 2>(p, mask_mode, causal, st);
         } else {
-            if (D == 64 && wpe == 4) launch_stream<bf16, 64, 4>(p, mask_mode, causal, st);
+            if (D == 64 && wpe == 4) launch_stream<bf16, 64, 3>(p, mask_mode, causal, st);
             else if (D == 64) launch_stream<bf16, 64, 2>(p, mask_mode, causal, st);
             else launch_stream<bf16, 128, 2>(p, mask_mode, causal, st);
         }
