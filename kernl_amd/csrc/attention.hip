@@ -30,6 +30,7 @@ static constexpr float kLog2eA = 1.4426950408889634f;
 static constexpr float kNegBig = -1.0e30f;            // anything below: exp2(x - rowmax) is exactly 0
 static constexpr float kClampFloor = -1.7014118e38f;  // scaled mask values are kept finite (-FLT_MAX / 2)
 static constexpr float kRescaleThreshold = 8.0f;  // log2 units
+static constexpr float kMaskedScore = -32768.0f;  // base-2 scores below this are mask values, not scores
 
 enum { MASK_NONE = 0, MASK_VECTOR = 1, MASK_MATRIX = 2 };
 
@@ -297,7 +298,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     // (Head size 128 with a matrix mask has no registers left for that block: there the reference is subtracted
     // from every score by an instruction of its own.)
     constexpr bool REF_IN_MFMA = !(D == 128 && MASK_MODE == MASK_MATRIX);
-    float m_i = 0.0f, l_i = 0.0f;
+    float m_i = 0.0f, m_masked = -INFINITY, l_i = 0.0f;
     bool fresh = true;
     f32x16 neg_m;
 #pragma unroll
@@ -378,7 +379,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         const unsigned char *sb = smem + ST * STAGE;
         // a wave whose 32 rows all lie above a causal tile has nothing to compute in it
         if (!(GENERAL && CAUSAL && n0 > m_wave0 + 31)) {
-            // ---- Sᵀ = K · Qᵀ
+            // ---- Sᵀ = K · Qᵀ, relative to the row's reference
             f32x16 s_acc[NBS];
             __builtin_amdgcn_s_setprio(2);
 #pragma unroll
@@ -446,14 +447,32 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
             // The scores are relative to the reference m_i, which is not the running maximum: it only moves (and
             // the accumulator and row sum are rescaled) when a score exceeds it by more than 2^8, so probabilities
             // stay <= 256 — exact in fp32, well inside the 16-bit range — and after the first tiles the rescale
-            // almost never runs.  While the row has seen no finite score yet (`fresh`; both lanes of a row agree on
-            // it, as they agree on mx) nothing has been accumulated, and the reference also moves DOWN to the tile's
-            // maximum: that costs nothing then and keeps rows of very negative scores from underflowing.
-            // The final O / l is independent of the reference.
-            const bool finite_max = mx > -INFINITY;
-            if (__builtin_amdgcn_ballot_w64(mx > kRescaleThreshold || (fresh && finite_max && mx < -kRescaleThreshold)) != 0) {
-                const float delta = fresh ? (finite_max ? mx : 0.0f) : fmaxf(mx, 0.0f);
-                const float alpha = fresh ? 1.0f : __builtin_amdgcn_exp2f(-delta);
+            // almost never runs.  The final O / l is independent of the reference.
+            // A row is `fresh` until it has seen a tile with an ordinary score (both lanes of a row agree on that,
+            // as they agree on mx); until then m_i stays 0.  Tiles whose scores all lie below kMaskedScore (mask
+            // entries of -inf arrive as -1.7e38, half-precision "minus infinity" biases as -9e4) are accumulated
+            // against a reference of their own, m_masked, subtracted explicitly here, so that a row without any
+            // ordinary key still gets its softmax over the masked ones (the plain average of V for -inf masks, as in
+            // the reference implementation).  The first ordinary tile discards that, and sets m_i to its maximum
+            // wherever that lies: the reference in the MFMA never goes where fp32 scores relative to it would lose
+            // their resolution.
+            const bool ordinary = mx > kMaskedScore;
+            if (__builtin_amdgcn_ballot_w64(mx > kRescaleThreshold || (fresh && mx > -INFINITY)) != 0) {
+                float alpha, dsub;
+                if (!fresh) {
+                    dsub = fmaxf(mx, 0.0f);
+                    alpha = __builtin_amdgcn_exp2f(-dsub);
+                    m_i += dsub;
+                } else if (ordinary) {
+                    dsub = mx;
+                    alpha = 0.0f;
+                    m_i = mx;
+                } else {
+                    const float m_new = fmaxf(m_masked, mx);
+                    alpha = (m_masked == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_masked - m_new);
+                    dsub = (m_new == -INFINITY) ? 0.0f : m_new;
+                    m_masked = m_new;
+                }
                 l_i *= alpha;
 #pragma unroll
                 for (int d = 0; d < DB; ++d)
@@ -462,12 +481,11 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 #pragma unroll
                 for (int nb = 0; nb < NBS; ++nb)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s_acc[nb][v] -= delta;
-                m_i += delta;
+                    for (int v = 0; v < 16; ++v) s_acc[nb][v] -= dsub;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) neg_m[v] = REF_IN_MFMA ? -m_i : 0.0f;
             }
-            fresh = fresh && !finite_max;
+            fresh = fresh && !ordinary;
 #pragma unroll
             for (int nb = 0; nb < NBS; ++nb)
 #pragma unroll

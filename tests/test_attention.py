@@ -141,6 +141,48 @@ def test_fully_masked_row_is_finite_uniform_average():
     assert (out[1] - expected).abs().max().item() < 5e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("kind", ["all_very_negative", "growing", "shrinking", "first_tiles_masked", "huge_then_small",
+                                  "half_min_bias"])
+def test_softmax_reference_moves_with_the_scores(kind, dtype, close):
+    """The kernel keeps scores relative to a per-row exponent reference that moves lazily: up when a score exceeds it
+    by more than 2^8, down only while the row has accumulated nothing.  Each case drives one of those moves: scores
+    that are all far below zero, that grow or shrink from key tile to key tile, rows whose first key tiles are fully
+    masked, and one dominant key followed by ordinary ones."""
+    gen = torch.Generator().manual_seed(21)
+    B, H, S, D = 2, 2, 320, 64  # 5 key tiles of 64
+    q = torch.randn((B, H, S, D), generator=gen)
+    k = torch.randn((B, H, S, D), generator=gen)
+    v = torch.randn((B, H, S, D), generator=gen)
+    mask = None
+    tile = torch.arange(S) // 64
+    if kind == "all_very_negative":
+        # every score near -60 (natural-log units): exp underflows in 16 bits unless the reference follows
+        q = q * 0.1 + 1.0
+        k = k * 0.1 - 7.5
+    elif kind == "growing":
+        k = k * (1.0 + 1.5 * tile.float())[None, None, :, None]
+    elif kind == "shrinking":
+        k = k * (7.0 - 1.5 * tile.float())[None, None, :, None]
+    elif kind == "first_tiles_masked":
+        mask = torch.rand((B, H, S, S), generator=gen)
+        mask[:, :, ::2, :128] = float("-inf")   # even rows: the first two key tiles are masked out entirely
+        mask[:, :, 1::3, 64:192] = float("-inf")
+    elif kind == "half_min_bias":
+        # additive masks of finfo(float16).min, as half-precision models build them: a masked prefix on some rows,
+        # every key masked on others (those rows are a softmax over the masked keys, in the oracle too)
+        mask = torch.zeros((B, H, S, S))
+        mask[:, :, ::2, :150] = -65504.0
+        mask[:, :, 7::16, :] = -65504.0
+    elif kind == "huge_then_small":
+        k[:, :, 5, :] = q[:, :, 40, :] * 4.0      # one dominant key in the first tile for row 40 (and large for others)
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    out = _run(q, k, v, 0.125, False, mask)
+    ref = attention_oracle(q, k, v, 0.125, False, mask)
+    assert torch.isfinite(out.float()).all()
+    close(out, ref, dtype, what=f"attention reference moves: {kind}")
+
+
 def test_attention_properties_full_size(close):
     # BASELINE config 1 at full size: [32,12,512,64], padding lengths U[256,512], scale 1/8.
     gen = torch.Generator().manual_seed(0)
