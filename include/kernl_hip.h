@@ -187,7 +187,7 @@ int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, 
  *                                is used; gated epilogues take 1, 3 or 5).
  *   kernl_attention_force_scalar non-zero routes every attention call through the strided scalar kernel.
  *   kernl_attention_set_variant  register budget of the head-size-64 MFMA attention kernel: 0 = heuristic,
- *                                1 = built for 4 waves/SIMD, 2 = built for 2 waves/SIMD.
+ *                                1 = built for 3 waves/SIMD, 2 = built for 2 waves/SIMD.
  */
 void kernl_linear_force_tile(int which);
 void kernl_attention_force_scalar(int on);

@@ -753,17 +753,17 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
                          (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30) &&
                          (mask == nullptr || (mask_strides[3] >= 0 && (N + 128) * mask_strides[3] < (1ll << 30)));
     if (mfma_ok) {
-        // head size 64 without a matrix mask fits the register budget of 4 waves per SIMD (128 VGPRs); the
+        // head size 64 without a matrix mask fits the register budget of 3 waves per SIMD (168 VGPRs); the
         // matrix-mask body (mask values prefetched in registers) and head size 128 run at 2 waves per SIMD.
-        int wpe = (D == 64 && mask_mode != MASK_MATRIX) ? 4 : 2;
-        if (D == 64 && g_attention_variant == 1) wpe = 4;
+        int wpe = (D == 64 && mask_mode != MASK_MATRIX) ? 3 : 2;
+        if (D == 64 && g_attention_variant == 1) wpe = 3;
         if (D == 64 && g_attention_variant == 2) wpe = 2;
         if (dtype == KERNL_F16) {
-            if (D == 64 && wpe == 4) launch_stream<f16, 64, 3>(p, mask_mode, causal, st);
+            if (D == 64 && wpe == 3) launch_stream<f16, 64, 3>(p, mask_mode, causal, st);
             else if (D == 64) launch_stream<f16, 64, 2>(p, mask_mode, causal, st);
             else launch_stream<f16, 128, 2>(p, mask_mode, causal, st);
         } else {
-            if (D == 64 && wpe == 4) launch_stream<bf16, 64, 3>(p, mask_mode, causal, st);
+            if (D == 64 && wpe == 3) launch_stream<bf16, 64, 3>(p, mask_mode, causal, st);
             else if (D == 64) launch_stream<bf16, 64, 2>(p, mask_mode, causal, st);
             else launch_stream<bf16, 128, 2>(p, mask_mode, causal, st);
         }
