@@ -316,6 +316,23 @@ def main():
             extra["decode_attention_gbps_graph_replay"] = round(kv_bytes / (t * 1e-3) / 1e9, 1)
             extra["decode_attention_frac_of_hbm_peak"] = round(kv_bytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
             del qd, kd, vd, od
+
+            # one decoding step's linear layers: a single row of x against 12 different [4096, 4096] weights in turn
+            # (384 MB, more than the 256 MB memory-side cache holds), so every launch streams its weight from HBM
+            from kernl_amd.implementations.linear_layer import linear_layer
+            x_dec = torch.randn((1, 4096), generator=gen).half().to(dev)
+            w_dec = [(torch.randn((4096, 4096), generator=gen) * 0.02).half().to(dev) for _ in range(12)]
+
+            def decode_linears():
+                for w_i in w_dec:
+                    linear_layer(x_dec, w_i, None)
+
+            t = graph_time_ms(decode_linears, reps=4) / len(w_dec)
+            w_bytes = w_dec[0].numel() * 2
+            extra["decode_linear_1x4096x4096_us_graph_replay"] = round(t * 1e3, 2)
+            extra["decode_linear_gbps_graph_replay"] = round(w_bytes / (t * 1e-3) / 1e9, 1)
+            extra["decode_linear_frac_of_hbm_peak"] = round(w_bytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
+            del w_dec, x_dec
         except Exception as exc:  # the headline must still be printed
             extra["decoder_kernels_error"] = f"{type(exc).__name__}: {exc}"[:300]
 

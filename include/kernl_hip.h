@@ -184,7 +184,10 @@ int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, 
  *                                2 = 256x192, 3 = 128x128, 4 = 256x128 with 32-wide k-tiles; persistent kernel with one
  *                                wave per SIMD: 5 = 256x256, 6 = 256x192; its one-tile-per-workgroup variant with
  *                                three LDS stages: 7 = 128x256, 8 = 128x192 (5..8 need K % 64 == 0, otherwise 128x128
- *                                is used; gated epilogues take 1, 3 or 5).
+ *                                is used; gated epilogues take 1, 3 or 5).  With the heuristic, inputs of at most
+ *                                64 rows and K % 64 == 0 go to a kernel that streams the weight once (16 output
+ *                                columns per workgroup); 9 = that kernel where it applies, the heuristic elsewhere;
+ *                                1..8 keep such inputs on the tile kernels.
  *   kernl_attention_force_scalar non-zero routes every attention call through the strided scalar kernel.
  *   kernl_attention_set_variant  register budget of the head-size-64 MFMA attention kernel: 0 = heuristic,
  *                                1 = built for 3 waves/SIMD, 2 = built for 2 waves/SIMD.

@@ -966,6 +966,131 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
 }
 
 // ----------------------------------------------------------------------------------------------------
+// Skinny kernel: at most 64 rows of x (decoding steps, pooled outputs).  The weight matrix is the only large operand
+// and the job is to stream it once at HBM speed with every CU: a workgroup owns 16 output columns (gated: their 16
+// gate and 16 value rows of the interleaved weight), its 4, 8 or 16 waves split K in interleaved 64-wide chunks (long
+// rows get many waves: the loop is bound by memory latency, and what counts is how many bytes a CU has in flight), every lane
+// fetches 32 contiguous bytes of its weight row per chunk (4 lanes cover a 128-byte line), and the fragments go from
+// global memory straight into v_mfma_f32_16x16x32 — weights on the A side, the few x rows on the B side.  The lane
+// of MFMA k-group g supplies k = 16 g + 8 s .. + 7 of the chunk in step s (s = 0, 1), on both sides, which is all
+// the instruction needs.  The waves' partial sums meet in LDS.  x is re-read by every workgroup, from L2.
+// ----------------------------------------------------------------------------------------------------
+template <typename T, int MB, bool GATED, int WAVES, int NR>
+__global__ void __launch_bounds__(64 * WAVES)
+linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
+                     T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
+                     int64_t ai_rs, int64_t ai_cs, int act) {
+    typedef typename Vec8<T>::type vec8;
+    constexpr int NA = GATED ? 2 : 1;        // weight fragments per 16 output columns: plain, or gate and value
+    constexpr int NF = NA * NR;              // weight fragments per step (NR blocks of 16 output columns)
+    constexpr int U = (MB <= 2 && NF <= 2) ? 4 : 2;  // chunks requested together
+    static_assert(WAVES * NF * MB <= 64, "partial sums fit 64 KB of LDS");
+    __shared__ __attribute__((aligned(16))) float red[WAVES][NF * MB][64][4];
+
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int n0 = (int)blockIdx.x * (16 * NR);  // first output column of this workgroup (N counts output columns)
+    // first interleaved row of the 16 output columns starting at nb (gated weights: 32 gate rows, 32 value rows, ...)
+    auto gated_row = [](int nb) -> int { return (nb >> 5) * 64 + (nb & 31); };
+    // rows of the weight this lane reads; columns beyond N repeat the last one and are never stored
+    const T *wp[NF];
+#pragma unroll
+    for (int rb = 0; rb < NR; ++rb) {
+        const int nb = n0 + 16 * rb;
+        if (GATED) {
+            const int row = gated_row(min(nb, N - 16)) + r;
+            wp[rb * NA] = W + (int64_t)row * K + 16 * g;
+            wp[rb * NA + NA - 1] = W + (int64_t)(row + 32) * K + 16 * g;
+        } else {
+            wp[rb * NA] = W + (int64_t)min(nb + r, N - 1) * K + 16 * g;
+        }
+    }
+    const T *xp[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) xp[mb] = X + (int64_t)min(16 * mb + r, M - 1) * ldx + 16 * g;
+
+    f32x4_acc acc[NF][MB];
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[f][mb] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const int nchunks = K / 64;
+    const int rot = (int)((blockIdx.x * 13u) % (unsigned)nchunks);
+    for (int c0 = wave; c0 < nchunks; c0 += WAVES * U) {
+        vec8 wf[U][NF][2], xf[U][MB][2];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            // chunks past the end repeat the last one; their products are left out below.  Workgroups walk the
+            // chunks from different starting points, so that they do not all ask L2 for the same lines of x at once.
+            int cc = min(c0 + WAVES * u, nchunks - 1) + rot;
+            cc = cc >= nchunks ? cc - nchunks : cc;
+            const int k0 = cc * 64;
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+                wf[u][f][0] = *reinterpret_cast<const vec8 *>(wp[f] + k0);
+                wf[u][f][1] = *reinterpret_cast<const vec8 *>(wp[f] + k0 + 8);
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                xf[u][mb][0] = *reinterpret_cast<const vec8 *>(xp[mb] + k0);
+                xf[u][mb][1] = *reinterpret_cast<const vec8 *>(xp[mb] + k0 + 8);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (c0 + WAVES * u < nchunks) {
+#pragma unroll
+                for (int f = 0; f < NF; ++f)
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) {
+                        acc[f][mb] = mfma16(wf[u][f][0], xf[u][mb][0], acc[f][mb]);
+                        acc[f][mb] = mfma16(wf[u][f][1], xf[u][mb][1], acc[f][mb]);
+                    }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[wave][f * MB + mb][lane][e] = acc[f][mb][e];
+    __syncthreads();
+
+    // the waves share the NR x MB blocks of 16 columns x 16 rows: element e of a lane is output column nb + 4 g + e
+    // of x row 16 mb + r
+    for (int unit = wave; unit < NR * MB; unit += WAVES) {
+        const int rb = unit / MB, mb = unit % MB;
+        const int nb = n0 + 16 * rb;
+        const int m = 16 * mb + r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int n = nb + 4 * g + e;
+            float v[NA];
+#pragma unroll
+            for (int a = 0; a < NA; ++a) {
+                float t4[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // fixed summation order: the result does not depend on timing
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) t4[w & 3] += red[w][(rb * NA + a) * MB + mb][lane][e];
+                v[a] = (t4[0] + t4[1]) + (t4[2] + t4[3]);
+            }
+            if (m >= M || n >= N) continue;
+            if (bias != nullptr) {
+                const int brow = GATED ? gated_row(nb) + 4 * g + e : n;
+                v[0] += to_float(bias[brow]);
+                if (GATED) v[NA - 1] += to_float(bias[brow + 32]);
+            }
+            if (!GATED && act_in != nullptr) act_in[(int64_t)m * ai_rs + (int64_t)n * ai_cs] = from_float<T>(v[0]);
+            float y = apply_act16(v[0], act);
+            if (GATED) y *= v[NA - 1];
+            out[(int64_t)m * out_rs + (int64_t)n * out_cs] = from_float<T>(y);
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------------
 // FMA kernel: any dtype, any strides.  64x64 output tile, 16x16 threads, 4x4 outputs per thread, fp32 LDS tiles.
 // ----------------------------------------------------------------------------------------------------
 template <typename T>
@@ -1210,10 +1335,58 @@ static int pick_tile(int M, int N, int K, bool gated) {
 
 int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192
 
+template <typename T, bool GATED, int MB, int NR>
+static void launch_skinny_blocks(const LinearArgs &a) {
+    const int n_out = GATED ? a.N / 2 : a.N;
+    const dim3 grid((unsigned)((n_out + 16 * NR - 1) / (16 * NR)));
+    const int act = a.act & (kGluBit - 1);
+    // waves per workgroup: enough to have a whole block of weight rows in flight when K is long, never more than
+    // there are chunks, and no more than the LDS for their partial sums allows
+    const int nchunks = a.K / 64;
+    constexpr int kMaxWaves = (GATED ? 2 : 1) * NR * MB > 8 ? 4 : (GATED ? 2 : 1) * NR * MB > 4 ? 8 : 16;
+    // ... and few enough that the workgroups one CU gets (256 CUs) are resident together: a 1024-thread workgroup
+    // fills half a CU, and 344 of them would leave a third of the chip idle
+    const int per_cu = ((int)grid.x + 255) / 256;
+    int waves = nchunks >= 64 ? 16 : nchunks >= 24 ? 8 : 4;
+    if (per_cu >= 3) waves = 4;
+    else if (per_cu == 2 && waves > 8) waves = 8;
+#define KERNL_SKINNY(WV)                                                                                                \
+    hipLaunchKernelGGL((linear_skinny_kernel<T, MB, GATED, WV, NR>), grid, dim3(64 * WV), 0, a.st,                      \
+                       static_cast<const T *>(a.x), static_cast<const T *>(a.w), static_cast<const T *>(a.bias),       \
+                       static_cast<T *>(a.out), static_cast<T *>(a.act_in), a.M, n_out, a.K, a.x_rs, a.out_rs, a.out_cs, \
+                       a.ai_rs, a.ai_cs, act)
+    if constexpr (kMaxWaves >= 16) {
+        if (waves >= 16) { KERNL_SKINNY(16); return; }
+    }
+    if constexpr (kMaxWaves >= 8) {
+        if (waves >= 8) { KERNL_SKINNY(8); return; }
+    }
+    KERNL_SKINNY(4);
+#undef KERNL_SKINNY
+}
+
+template <typename T, bool GATED>
+static void launch_skinny(const LinearArgs &a) {
+    const int n_out = GATED ? a.N / 2 : a.N;
+    const int mb = (a.M + 15) / 16;
+    // every workgroup reads all of x (from L2): with enough output columns to fill the chip twice over, a workgroup
+    // takes 32 of them and that traffic halves
+    const bool two = n_out >= 8192;
+    if (mb <= 1) { if (two) launch_skinny_blocks<T, GATED, 1, 2>(a); else launch_skinny_blocks<T, GATED, 1, 1>(a); }
+    else if (mb <= 2) { if (two) launch_skinny_blocks<T, GATED, 2, 2>(a); else launch_skinny_blocks<T, GATED, 2, 1>(a); }
+    else { if (two) launch_skinny_blocks<T, GATED, 4, 2>(a); else launch_skinny_blocks<T, GATED, 4, 1>(a); }
+}
+
 template <typename T>
 static int linear_mfma_dispatch(const LinearArgs &a) {
     int pick = g_linear_force_tile;
-    if (pick == 0) pick = pick_tile(a.M, a.N, a.K, (a.act & kGluBit) != 0);
+    // few rows of x: stream the weight once with every CU (9 forces this kernel where it applies)
+    if ((pick == 0 || pick == 9) && a.M <= 64 && a.K % 64 == 0) {
+        if (a.act & kGluBit) launch_skinny<T, true>(a);
+        else launch_skinny<T, false>(a);
+        return check_launch("linear (skinny)");
+    }
+    if (pick == 0 || pick == 9) pick = pick_tile(a.M, a.N, a.K, (a.act & kGluBit) != 0);
     if (a.act & kGluBit) {
         if (pick == 5 && a.K % 64 == 0) launch_wide<T>(a);
         else if (pick == 3) launch_mfma_glu<T, Tile128x128>(a);

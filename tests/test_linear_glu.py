@@ -143,3 +143,17 @@ def test_glu_more_tiles_than_compute_units(close):
     finally:
         lib.kernl_linear_force_tile(0)
     close(out, glu_oracle(x, wg, bg, wv, bv, "silu"), scale=4.0, what="glu persistent")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("bias", [False, True], ids=["nobias", "bias"])
+@pytest.mark.parametrize("shape", [(1, 11008, 4096), (7, 96, 64), (16, 160, 320), (40, 1024, 192), (64, 352, 4096),
+                                   (33, 8224, 256), (64, 8192, 64)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_glu_few_rows_streams_the_weight(shape, bias, dtype, close):
+    """M <= 64 (reference experimental/llama-v2/test/test_ff.py runs M = 1..128): every workgroup takes 16 gate rows
+    and their 16 value rows of the interleaved weight, the four waves split K."""
+    M, N, K = shape
+    x, wg, bg, wv, bv = _case(M, N, K, dtype, bias, seed=5)
+    out = _run(x, wg, bg, wv, bv, "silu")
+    close(out, glu_oracle(x, wg, bg, wv, bv, "silu"), dtype, what=f"gated, few rows {shape}")

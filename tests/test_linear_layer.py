@@ -116,6 +116,43 @@ def test_linear_wide_tiles_save_activation_inputs(tile, close):
     close(act_in, pre, torch.bfloat16, what=f"tile {tile} act_inputs")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("activation", ["", "gelu", "silu"])
+@pytest.mark.parametrize("shape", [(1, 4096, 512), (5, 80, 64), (16, 1000, 192), (17, 768, 3072), (33, 2304, 768),
+                                   (64, 4096, 1024), (3, 24, 4096), (5, 8200, 128), (33, 9000, 192), (64, 8192, 128)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_linear_few_rows_streams_the_weight(shape, activation, dtype, close):
+    """At most 64 rows of x (decoding steps): the kernel that streams the weight once, 16 output columns per workgroup.
+    Shapes cover one to four 16-row blocks of x, output widths that are not a multiple of 16, chunk counts that do
+    not divide by the waves of a workgroup, outputs wide enough for 32 columns per workgroup, and the saved
+    pre-activation."""
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(17)
+    x, w, b = _inputs(M, N, K, dtype, gen, w_std=K ** -0.5)
+    act_in = torch.empty((M, N), dtype=dtype, device="cuda")
+    lib = _lib.load()
+    lib.kernl_linear_force_tile(9)
+    try:
+        out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation=activation, act_inputs=act_in)
+        out_nobias = linear_layer(x.cuda(), w.cuda(), None, activation=activation)
+        torch.cuda.synchronize()
+    finally:
+        lib.kernl_linear_force_tile(0)
+    ref, pre = linear_oracle(x, w, b, activation, return_act_inputs=True)
+    close(out, ref, dtype, what=f"few rows {shape} {activation!r}")
+    close(act_in, pre, dtype, what=f"few rows {shape} pre-activation")
+    close(out_nobias, linear_oracle(x, w, None, activation), dtype, what=f"few rows {shape} no bias")
+
+
+def test_linear_few_rows_strided_output_and_batched_input(close):
+    gen = torch.Generator().manual_seed(18)
+    x, w, b = _inputs(2, 640, 256, torch.float16, gen, w_std=1 / 16, batch=3)  # [3, 2, 256] -> 6 rows
+    out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation="tanh")
+    torch.cuda.synchronize()
+    close(out, linear_oracle(x, w, b, "tanh"), what="few rows, batched")
+    assert out.shape == (3, 2, 640)
+
+
 @pytest.mark.parametrize("which", ["up", "down"])
 def test_linear_config2_full_size(which, close):
     # BASELINE config 2: up-projection [16384,768]x[3072,768]ᵀ + bias + tanh-GELU; down-projection back, no activation
