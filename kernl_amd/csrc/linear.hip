@@ -1369,9 +1369,9 @@ template <typename T, bool GATED>
 static void launch_skinny(const LinearArgs &a) {
     const int n_out = GATED ? a.N / 2 : a.N;
     const int mb = (a.M + 15) / 16;
-    // every workgroup reads all of x (from L2): with enough output columns to fill the chip twice over, a workgroup
-    // takes 32 of them and that traffic halves
-    const bool two = n_out >= 8192;
+    // every workgroup reads all of x (from L2): with more than 16 rows of x and enough output columns to fill the
+    // chip twice over, a workgroup takes 32 columns and that traffic halves
+    const bool two = n_out >= 8192 && mb >= 2;
     if (mb <= 1) { if (two) launch_skinny_blocks<T, GATED, 1, 2>(a); else launch_skinny_blocks<T, GATED, 1, 1>(a); }
     else if (mb <= 2) { if (two) launch_skinny_blocks<T, GATED, 2, 2>(a); else launch_skinny_blocks<T, GATED, 2, 1>(a); }
     else { if (two) launch_skinny_blocks<T, GATED, 4, 2>(a); else launch_skinny_blocks<T, GATED, 4, 1>(a); }
