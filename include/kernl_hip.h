@@ -75,6 +75,23 @@ int kernl_attention_fwd(const void *q, const void *k, const void *v, void *out, 
                         float sm_scale, int is_causal, float mask_min_clamp, int dtype, void *stream);
 
 /*
+ * Causal attention of M new query rows at positions start_position .. start_position + M - 1 over the N keys of a
+ * key/value cache: key n contributes to query row m only if n <= m + start_position (start_position = 0 is
+ * kernl_attention_fwd with is_causal; N is usually start_position + M, later keys are never visible) — the mask
+ * the reference model builds, `triu(full(-inf), diagonal=start_pos + 1)` (experimental/llama-v2/llama/model.py:338-343).
+ * Replaces the `_fwd_kernel[grid](...)` launch of experimental/llama-v2/kernel/fused_kernel_attention.py:127-144
+ * (kernel body :21-117, `start_position` at :59-76; that kernel's own comparison agrees with the model's mask at
+ * start_position 0, the only value its self-test runs).  All other arguments as kernl_attention_fwd.
+ */
+int kernl_attention_cached_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
+                               int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
+                               const int64_t q_strides[4], const int64_t k_strides[4],
+                               const int64_t v_strides[4], const int64_t o_strides[4],
+                               const int64_t mask_sizes[4], const int64_t mask_strides[4], int mask_dtype,
+                               float sm_scale, int64_t start_position, float mask_min_clamp, int dtype,
+                               void *stream);
+
+/*
  * Split-K attention for very few query rows (decoding: q_len = 1 against a long key sequence).  Same arguments and
  * semantics as kernl_attention_fwd plus a workspace; the keys of every (batch, head, query row) are split into
  * ranges that run in parallel and are merged by a second kernel.  Replaces the `_fwd_part_1[grid]` /

@@ -22,6 +22,7 @@ EXPORTED_SYMBOLS = (
     "kernl_version",
     "kernl_last_error_string",
     "kernl_attention_fwd",
+    "kernl_attention_cached_fwd",
     "kernl_attention_skinny_workspace_bytes",
     "kernl_attention_skinny_fwd",
     "kernl_rope_fwd",
@@ -64,6 +65,10 @@ def load() -> ctypes.CDLL:
     lib.kernl_attention_fwd.restype = ctypes.c_int
     lib.kernl_attention_fwd.argtypes = (
         [_vp] * 5 + [_i64] * 5 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, _vp]
+    )
+    lib.kernl_attention_cached_fwd.restype = ctypes.c_int
+    lib.kernl_attention_cached_fwd.argtypes = (
+        [_vp] * 5 + [_i64] * 5 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, _i64, ctypes.c_float, ctypes.c_int, _vp]
     )
     lib.kernl_attention_skinny_workspace_bytes.restype = _i64
     lib.kernl_attention_skinny_workspace_bytes.argtypes = [_i64] * 5
@@ -129,6 +134,27 @@ def attention_fwd(q, k, v, out, mask, sm_scale: float, is_causal: bool, mask_min
             float(sm_scale), int(bool(is_causal)), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
         )
     _check(st, "kernl_attention_fwd")
+
+
+def attention_cached_fwd(q, k, v, out, mask, sm_scale: float, start_position: int, mask_min_clamp: float) -> None:
+    """Causal attention of the rows of q, which sit at positions start_position.. of the sequence held in k / v."""
+    _require_gpu(q, k, v, out, mask)
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    lib = load()
+    if mask is not None:
+        msizes, mstrides, mdtype, mptr = _arr(mask.shape), _arr(mask.stride()), DTYPE_CODE[mask.dtype], mask.data_ptr()
+    else:
+        msizes, mstrides, mdtype, mptr = None, None, KERNL_F32, None
+    with torch.cuda.device(q.device):
+        st = lib.kernl_attention_cached_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), mptr,
+            B, H, M, N, D,
+            _arr(q.stride()), _arr(k.stride()), _arr(v.stride()), _arr(out.stride()),
+            msizes, mstrides, mdtype,
+            float(sm_scale), int(start_position), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
+        )
+    _check(st, "kernl_attention_cached_fwd")
 
 
 def attention_skinny_workspace_bytes(B: int, H: int, M: int, N: int, D: int) -> int:

@@ -46,6 +46,7 @@ struct AttnParams {
     float clamp;  // replacement for -inf mask entries
     int nq_tiles;
     int mask_fast;  // matrix mask rows can be read as aligned 4-element vectors through 32-bit offsets
+    int causal_off;  // causal: query row m sees keys 0 .. m + causal_off (0: top-left aligned)
 };
 
 __device__ __forceinline__ float load_mask_value(const void *mask, int dtype, int64_t off) {
@@ -173,12 +174,12 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     };
 
     // ---- key tiles: [0, n_clean) of the processing order need no masking, [n_clean, nt) take the general body
-    const int n_end = CAUSAL ? min(N, q0 + BM) : N;
+    const int n_end = CAUSAL ? min(N, q0 + BM + p.causal_off) : N;
     const int nt_all = (n_end + BN - 1) / BN;
     constexpr bool MAY_LIST = (MASK_MODE == MASK_VECTOR && !CAUSAL);
     const bool use_list = MAY_LIST && nt_all <= 64;
     int nt = nt_all, n_clean = 0;
-    if (MASK_MODE == MASK_NONE) n_clean = CAUSAL ? min(N / BN, q0 / BN) : N / BN;
+    if (MASK_MODE == MASK_NONE) n_clean = CAUSAL ? min(N / BN, (q0 + p.causal_off + 1) / BN) : N / BN;
     // the first tile is fetched before the mask has been looked at: tile 0 almost always comes first
     if (nt_all > 0) dma(0, 0);
     // With a per-key mask every wave classifies all key tiles by itself (the mask row is a few KB, and this way no
@@ -378,7 +379,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 
         const unsigned char *sb = smem + ST * STAGE;
         // a wave whose 32 rows all lie above a causal tile has nothing to compute in it
-        if (!(GENERAL && CAUSAL && n0 > m_wave0 + 31)) {
+        if (!(GENERAL && CAUSAL && n0 > m_wave0 + 31 + p.causal_off)) {
             // ---- Sᵀ = K · Qᵀ, relative to the row's reference
             f32x16 s_acc[NBS];
             __builtin_amdgcn_s_setprio(2);
@@ -427,7 +428,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                                     sv += scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_row + n * p.ms[3]), p.clamp);
                                 }
                             }
-                            if (CAUSAL && (n0 + nl + r > my_m)) sv = -INFINITY;
+                            if (CAUSAL && (n0 + nl + r > my_m + p.causal_off)) sv = -INFINITY;
                             s_acc[nb][g * 4 + r] = sv;
                             mx = fmaxf(mx, sv);
                         }
@@ -607,7 +608,7 @@ __global__ void __launch_bounds__(64) attention_scalar_kernel(const AttnParams p
     __syncthreads();
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     float m_i = -INFINITY, l_i = 0.0f;
-    const int n_end = causal ? min(p.N, m + 1) : p.N;
+    const int n_end = causal ? min(p.N, m + 1 + p.causal_off) : p.N;
     for (int n0 = 0; n0 < n_end; n0 += 64) {
         const int n = n0 + lane;
         float s = -INFINITY;
@@ -681,13 +682,16 @@ int g_attention_variant = 0;       // tuning hook: register budget (waves per SI
 extern "C" void kernl_attention_force_scalar(int on) { kernl::g_attention_force_scalar = on; }
 extern "C" void kernl_attention_set_variant(int which) { kernl::g_attention_variant = which; }
 
-extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
-                                   int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
-                                   const int64_t q_strides[4], const int64_t k_strides[4],
-                                   const int64_t v_strides[4], const int64_t o_strides[4],
-                                   const int64_t mask_sizes[4], const int64_t mask_strides[4], int mask_dtype,
-                                   float sm_scale, int is_causal, float mask_min_clamp, int dtype, void *stream) {
+static int attention_entry(const void *q, const void *k, const void *v, void *out, const void *mask,
+                           int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
+                           const int64_t q_strides[4], const int64_t k_strides[4],
+                           const int64_t v_strides[4], const int64_t o_strides[4],
+                           const int64_t mask_sizes[4], const int64_t mask_strides[4], int mask_dtype,
+                           float sm_scale, int is_causal, int64_t start_position, float mask_min_clamp, int dtype,
+                           void *stream) {
     using namespace kernl;
+    if (start_position < 0 || start_position > (1 << 24))
+        return set_error(KERNL_ERR_INVALID_ARG, "attention: start_position %lld out of range", (long long)start_position);
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr || q_strides == nullptr ||
         k_strides == nullptr || v_strides == nullptr || o_strides == nullptr)
         return set_error(KERNL_ERR_INVALID_ARG, "attention: q, k, v, out and their strides must not be NULL");
@@ -735,6 +739,7 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
     p.clamp = mask_min_clamp;
     p.nq_tiles = (int)((M + 127) / 128);
     p.mask_fast = 0;
+    p.causal_off = is_causal != 0 ? (int)start_position : 0;
     if (mask_mode == MASK_MATRIX && (mask_dtype == KERNL_F32 || mask_dtype == dtype)) {
         const int64_t es = mask_dtype == KERNL_F32 ? 4 : 2;
         p.mask_fast = mask_strides[3] == 1 && p.ms[0] % 4 == 0 && p.ms[1] % 4 == 0 && p.ms[2] % 4 == 0 && p.ms[2] > 0 &&
@@ -778,4 +783,25 @@ extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, 
     else
         hipLaunchKernelGGL((attention_scalar_kernel<bf16>), grid, dim3(64), 0, st, p, (int)D, mask_mode, (int)causal);
     return check_launch("attention (scalar)");
+}
+
+extern "C" int kernl_attention_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
+                                   int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
+                                   const int64_t q_strides[4], const int64_t k_strides[4],
+                                   const int64_t v_strides[4], const int64_t o_strides[4],
+                                   const int64_t mask_sizes[4], const int64_t mask_strides[4], int mask_dtype,
+                                   float sm_scale, int is_causal, float mask_min_clamp, int dtype, void *stream) {
+    return attention_entry(q, k, v, out, mask, B, H, M, N, D, q_strides, k_strides, v_strides, o_strides, mask_sizes,
+                           mask_strides, mask_dtype, sm_scale, is_causal, 0, mask_min_clamp, dtype, stream);
+}
+
+extern "C" int kernl_attention_cached_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
+                                          int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
+                                          const int64_t q_strides[4], const int64_t k_strides[4],
+                                          const int64_t v_strides[4], const int64_t o_strides[4],
+                                          const int64_t mask_sizes[4], const int64_t mask_strides[4], int mask_dtype,
+                                          float sm_scale, int64_t start_position, float mask_min_clamp, int dtype,
+                                          void *stream) {
+    return attention_entry(q, k, v, out, mask, B, H, M, N, D, q_strides, k_strides, v_strides, o_strides, mask_sizes,
+                           mask_strides, mask_dtype, sm_scale, 1, start_position, mask_min_clamp, dtype, stream);
 }

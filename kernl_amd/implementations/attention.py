@@ -60,8 +60,12 @@ class Attention(torch.autograd.Function):
         sm_scale: float,
         is_causal: bool,
         attention_mask: Optional[torch.Tensor] = None,
+        start_position: int = 0,
     ):
         """out = softmax(q·kᵀ·sm_scale + causal + attention_mask)·v, written into `output` (caller allocated).
+
+        With `is_causal`, query row m sees keys 0 .. m + start_position: `start_position` > 0 is the causal attention
+        of new tokens over a key/value cache (reference: experimental/llama-v2/kernel/fused_kernel_attention.py:59-76).
 
         q [batch, heads, m, d]; k, v [batch, heads, n, d]; attention_mask additive, broadcastable as
         [batch|1, heads|1, m|1, n].  fp32 inputs are not supported (reference: attention.py:455-497); under
@@ -93,7 +97,10 @@ class Attention(torch.autograd.Function):
             assert attention_mask.dtype in _lib.DTYPE_CODE, f"Mask must be a floating tensor, got {attention_mask.dtype}"
             min_clamp = torch.finfo(attention_mask.dtype).min
 
-        _lib.attention_fwd(q, k, v, output, attention_mask, sm_scale, is_causal, min_clamp)
+        if is_causal and start_position:
+            _lib.attention_cached_fwd(q, k, v, output, attention_mask, sm_scale, int(start_position), min_clamp)
+        else:
+            _lib.attention_fwd(q, k, v, output, attention_mask, sm_scale, is_causal, min_clamp)
         return output
 
 
@@ -105,6 +112,8 @@ def attention_forward(
     sm_scale: float,
     is_causal: bool = False,
     attention_mask: Optional[torch.Tensor] = None,
+    start_position: int = 0,
 ):
-    """Reference: attention.py:532-541."""
-    return Attention.apply(q, k, v, output, sm_scale, is_causal, attention_mask)
+    """Reference: attention.py:532-541; `start_position` as in `triton_fa` of
+    experimental/llama-v2/kernel/fused_kernel_attention.py:113-146."""
+    return Attention.apply(q, k, v, output, sm_scale, is_causal, attention_mask, start_position)

@@ -45,12 +45,16 @@ def attention_oracle(
     sm_scale: float,
     is_causal: bool = False,
     attention_mask: Optional[torch.Tensor] = None,
+    start_position: int = 0,
 ) -> torch.Tensor:
     """softmax(q·kᵀ·sm_scale + mask, causal)·v in fp32 on the CPU.
 
     Follows `attention_reference`, implementations/attention.py:29-61: scale, ADD the mask, set keys n > m to -inf
     when causal (`tril` of an [m, n] matrix, i.e. top-left aligned), softmax over keys, times v.  Inputs of any
-    float dtype are upcast to fp32 first; the result is fp32.
+    float dtype are upcast to fp32 first; the result is fp32.  `start_position` shifts the causal diagonal: keys
+    n > m + start_position are masked, the `triu(..., diagonal=start_pos + 1)` mask of
+    experimental/llama-v2/llama/model.py:338-343 (pinned in tests/test_oracle.py by the rows start_position.. of a
+    top-left aligned causal attention over the whole sequence).
     """
     q32, k32, v32 = q.detach().float().cpu(), k.detach().float().cpu(), v.detach().float().cpu()
     p = torch.matmul(q32, k32.transpose(-1, -2)) * sm_scale
@@ -58,7 +62,7 @@ def attention_oracle(
         p = p + attention_mask.detach().float().cpu()
     if is_causal:
         m_size, n_size = q32.size(-2), k32.size(-2)
-        keep = torch.tril(torch.ones((m_size, n_size), dtype=torch.bool))
+        keep = torch.tril(torch.ones((m_size, n_size), dtype=torch.bool), diagonal=start_position)
         p = torch.where(keep, p, torch.tensor(float("-inf")))
     p = torch.softmax(p, dim=-1)
     return torch.matmul(p, v32)

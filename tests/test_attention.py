@@ -183,6 +183,31 @@ def test_softmax_reference_moves_with_the_scores(kind, dtype, close):
     close(out, ref, dtype, what=f"attention reference moves: {kind}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("mask_kind", ["none", "bias"])
+@pytest.mark.parametrize("case", [(1, 4, 1, 300, 64), (2, 3, 17, 64, 64), (1, 2, 130, 333, 64), (1, 2, 128, 128, 128),
+                                  (1, 1, 300, 1000, 128), (2, 2, 64, 0, 64), (1, 2, 40, 700, 80)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_causal_attention_over_a_cache(case, mask_kind, dtype, close):
+    """M new query rows at positions start.. against the start + M (+ a few unused) keys of a cache
+    (reference: experimental/llama-v2/kernel/fused_kernel_attention.py, `start_position`; mask semantics
+    llama/model.py:338-343).  Head size 80 takes the scalar kernel."""
+    B, H, M, start, D = case
+    N = start + M + (5 if start % 2 else 0)   # some cases carry keys beyond every row's horizon
+    gen = torch.Generator().manual_seed(23)
+    q = torch.randn((B, H, M, D), generator=gen).to(dtype)
+    k = torch.randn((B, H, N, D), generator=gen).to(dtype)
+    v = torch.randn((B, H, N, D), generator=gen).to(dtype)
+    mask = torch.rand((B, H, M, N), generator=gen) if mask_kind == "bias" else None
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    out = torch.empty_like(qc)
+    attention_forward(qc, kc, vc, out, 0.2, is_causal=True, attention_mask=None if mask is None else mask.cuda(),
+                      start_position=start)
+    torch.cuda.synchronize()
+    ref = attention_oracle(q, k, v, 0.2, True, mask, start_position=start)
+    close(out, ref, dtype, what=f"cached causal attention {case} {mask_kind}")
+
+
 def test_attention_properties_full_size(close):
     # BASELINE config 1 at full size: [32,12,512,64], padding lengths U[256,512], scale 1/8.
     gen = torch.Generator().manual_seed(0)

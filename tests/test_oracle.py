@@ -271,3 +271,29 @@ def test_glu_closed_form_and_known_answers():
     assert torch.allclose(ones, F.silu(F.linear(x, wg, bg)), atol=1e-6)
     # gate and value are not interchangeable
     assert not torch.allclose(out, glu_oracle(x, wv, bv, wg, bg, "silu"), atol=1e-3)
+
+
+def test_attention_oracle_start_position_is_a_row_window_of_full_causal_attention():
+    """Causal attention of M new rows at positions s.. over N = s + M keys equals rows s.. of the ordinary (top-left
+    aligned) causal attention of the whole sequence; keys beyond the horizon of the last row change nothing; and
+    the element-by-element rule (key n visible to row m iff n <= m + s) holds in a scalar loop."""
+    gen = torch.Generator().manual_seed(31)
+    s_pos, M, D = 37, 21, 8
+    N = s_pos + M
+    q_all = torch.randn((1, 2, N, D), generator=gen)
+    k = torch.randn((1, 2, N, D), generator=gen)
+    v = torch.randn((1, 2, N, D), generator=gen)
+    full = attention_oracle(q_all, k, v, 0.4, True, None)
+    part = attention_oracle(q_all[:, :, s_pos:], k, v, 0.4, True, None, start_position=s_pos)
+    assert torch.allclose(part, full[:, :, s_pos:], atol=1e-6)
+    # extra keys behind the last visible one are ignored
+    k_more = torch.cat((k, torch.randn((1, 2, 9, D), generator=gen)), dim=2)
+    v_more = torch.cat((v, torch.randn((1, 2, 9, D), generator=gen)), dim=2)
+    assert torch.allclose(attention_oracle(q_all[:, :, s_pos:], k_more, v_more, 0.4, True, None, start_position=s_pos), part, atol=1e-6)
+    # scalar restatement of one row
+    m = 5
+    row = q_all[0, 1, s_pos + m]
+    scores = [float(row @ k[0, 1, n]) * 0.4 for n in range(N) if n <= m + s_pos]
+    w = torch.softmax(torch.tensor(scores), dim=0)
+    expect = sum(w[n] * v[0, 1, n] for n in range(len(scores)))
+    assert torch.allclose(part[0, 1, m], expect, atol=1e-5)
