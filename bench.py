@@ -315,7 +315,15 @@ def main():
             extra["decode_attention_32x32x1x4096x128_us_graph_replay"] = round(t * 1e3, 2)
             extra["decode_attention_gbps_graph_replay"] = round(kv_bytes / (t * 1e-3) / 1e9, 1)
             extra["decode_attention_frac_of_hbm_peak"] = round(kv_bytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
-            del qd, kd, vd, od
+            # the same step with the keys and values stored as fp8 e5m2: half the bytes to stream
+            from kernl_amd.implementations.attention_skinny import to_e5m2
+            kd8, vd8 = to_e5m2(kd), to_e5m2(vd)
+            del kd, vd
+            t = graph_time_ms(lambda: skinny_attention_forward(qd, kd8, vd8, od, 128 ** -0.5), reps=5)
+            extra["decode_attention_fp8kv_us_graph_replay"] = round(t * 1e3, 2)
+            extra["decode_attention_fp8kv_gbps_graph_replay"] = round(2 * kd8.numel() / (t * 1e-3) / 1e9, 1)
+            extra["decode_attention_fp8kv_frac_of_hbm_peak"] = round(2 * kd8.numel() / (t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
+            del qd, kd8, vd8, od
 
             # one decoding step's linear layers: a single row of x against 12 different [4096, 4096] weights in turn
             # (384 MB, more than the 256 MB memory-side cache holds), so every launch streams its weight from HBM

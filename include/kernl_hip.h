@@ -114,6 +114,20 @@ int kernl_attention_skinny_fwd(const void *q, const void *k, const void *v, void
                                float mask_min_clamp, int dtype, void *stream);
 
 /*
+ * kernl_attention_skinny_fwd with the keys and values stored as one byte per element: fp8 e5m2, i.e. the upper byte
+ * of the fp16 encoding (what the reference keeps in its int8 key/value caches, experimental/llama-v2/kernel/
+ * fused_kernel_fp8.py:40-56,68-72, and widens inside its kernel, fused_kernel_attention.py:69-71,90-92).  k and v
+ * strides count bytes; rows must be 8-byte aligned.  q, out and `dtype` are 16-bit as before; half the bytes of the
+ * key/value stream, the same arithmetic (fp32) on the decoded values.
+ */
+int kernl_attention_skinny_kv8_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
+                                   void *workspace, int64_t workspace_bytes, int64_t B, int64_t H, int64_t M, int64_t N,
+                                   int64_t D, const int64_t q_strides[4], const int64_t k_strides[4],
+                                   const int64_t v_strides[4], const int64_t o_strides[4], const int64_t mask_sizes[4],
+                                   const int64_t mask_strides[4], int mask_dtype, float sm_scale, int is_causal,
+                                   float mask_min_clamp, int dtype, void *stream);
+
+/*
  * Rotary position embedding, half-split convention:  out = x·cos + rotate_half(x)·sin, with
  * rotate_half(x)[d] = -x[d + D/2] (d < D/2), x[d - D/2] (d >= D/2); fp32 arithmetic, one rounding.
  * The reference applies the same rotation (in Meta's interleaved-pair convention) inside its fused query/key

@@ -25,6 +25,7 @@ EXPORTED_SYMBOLS = (
     "kernl_attention_cached_fwd",
     "kernl_attention_skinny_workspace_bytes",
     "kernl_attention_skinny_fwd",
+    "kernl_attention_skinny_kv8_fwd",
     "kernl_rope_fwd",
     "kernl_linear_fwd",
     "kernl_linear_glu_fwd",
@@ -74,6 +75,10 @@ def load() -> ctypes.CDLL:
     lib.kernl_attention_skinny_workspace_bytes.argtypes = [_i64] * 5
     lib.kernl_attention_skinny_fwd.restype = ctypes.c_int
     lib.kernl_attention_skinny_fwd.argtypes = (
+        [_vp] * 6 + [_i64] * 6 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, _vp]
+    )
+    lib.kernl_attention_skinny_kv8_fwd.restype = ctypes.c_int
+    lib.kernl_attention_skinny_kv8_fwd.argtypes = (
         [_vp] * 6 + [_i64] * 6 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, _vp]
     )
     lib.kernl_rope_fwd.restype = ctypes.c_int
@@ -173,7 +178,9 @@ def attention_skinny_fwd(q, k, v, out, mask, workspace, sm_scale: float, is_caus
     ws_ptr = None if workspace is None else workspace.data_ptr()
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     with torch.cuda.device(q.device):
-        st = lib.kernl_attention_skinny_fwd(
+        one_byte = k.dtype in (torch.int8, torch.uint8, torch.float8_e5m2)
+        entry = lib.kernl_attention_skinny_kv8_fwd if one_byte else lib.kernl_attention_skinny_fwd
+        st = entry(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), mptr, ws_ptr, ws_bytes,
             B, H, M, N, D,
             _arr(q.stride()), _arr(k.stride()), _arr(v.stride()), _arr(out.stride()),

@@ -10,6 +10,8 @@
 // softmax and the groups are merged once at the end (registers -> LDS -> workspace).
 #include <math.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace kernl {
@@ -24,6 +26,7 @@ struct SkinnyParams {
     int B, H, M, N, D, splits;
     int64_t qs[4], ks[4], vs[4], os[4], ms[4];
     int mask_dtype, has_mask, causal;
+    int kv8;  // k and v hold one byte per element: fp8 e5m2, the upper byte of the fp16 encoding
     float scale_log2, clamp;
 };
 
@@ -47,8 +50,46 @@ __device__ __forceinline__ void sk_merge(float &m, float &l, float (&acc)[8], fl
     m = mn;
 }
 
+// 8 features of a key or value row as fp32: from the 16-bit storage type, or from fp8 e5m2 bytes — those are the upper
+// bytes of fp16 values, so decoding is a shift (reference: the int8 caches bit-cast to float8e5 and widened to fp16,
+// experimental/llama-v2/kernel/fused_kernel_attention.py:69-71,90-92).
+template <typename T, bool KV8>
+__device__ __forceinline__ void sk_load8(const void *base, int64_t elem_off, float (&f)[8]) {
+    if constexpr (KV8) {
+        const uint2 raw = *reinterpret_cast<const uint2 *>(static_cast<const unsigned char *>(base) + elem_off);
+        const uint32_t w[2] = {raw.x, raw.y};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const unsigned short h = (unsigned short)(((w[e >> 2] >> (8 * (e & 3))) & 0xFFu) << 8);
+            f[e] = (float)__builtin_bit_cast(_Float16, h);
+        }
+    } else {
+        typedef typename Vec8<T>::type vec8;
+        const vec8 v = *reinterpret_cast<const vec8 *>(static_cast<const T *>(base) + elem_off);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = (float)v[e];
+    }
+}
+
+// The same 8 features as four packed fp16 pairs (fp16 queries only): fp8 e5m2 bytes become fp16 values by moving
+// each byte into the upper half of a 16-bit lane, one byte-permute per pair; fp16 storage is used as it lies.
+template <bool KV8>
+__device__ __forceinline__ void sk_load8_pairs(const void *base, int64_t elem_off, uint32_t (&pk)[4]) {
+    if constexpr (KV8) {
+        const uint2 raw = *reinterpret_cast<const uint2 *>(static_cast<const unsigned char *>(base) + elem_off);
+        pk[0] = __builtin_amdgcn_perm(0u, raw.x, 0x010c000cu);  // bytes {0, b0, 0, b1}
+        pk[1] = __builtin_amdgcn_perm(0u, raw.x, 0x030c020cu);
+        pk[2] = __builtin_amdgcn_perm(0u, raw.y, 0x010c000cu);
+        pk[3] = __builtin_amdgcn_perm(0u, raw.y, 0x030c020cu);
+    } else {
+        const u32x4 raw = *reinterpret_cast<const u32x4 *>(static_cast<const f16 *>(base) + elem_off);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pk[j] = raw[j];
+    }
+}
+
 // DL = D / 8 lanes per key (a power of two, 1..64)
-template <typename T, int DL>
+template <typename T, int DL, bool KV8>
 __global__ void __launch_bounds__(256) attention_skinny_part1(const SkinnyParams p) {
     typedef typename Vec8<T>::type vec8;
     constexpr int KPW = 64 / DL;  // keys per wave and step
@@ -59,8 +100,7 @@ __global__ void __launch_bounds__(256) attention_skinny_part1(const SkinnyParams
     const int dl = lane % DL, kg = lane / DL;
 
     const T *qp = static_cast<const T *>(p.q) + b * p.qs[0] + h * p.qs[1] + (int64_t)m * p.qs[2] + dl * 8;
-    const T *kp = static_cast<const T *>(p.k) + b * p.ks[0] + h * p.ks[1] + dl * 8;
-    const T *vp = static_cast<const T *>(p.v) + b * p.vs[0] + h * p.vs[1] + dl * 8;
+    const int64_t k_base = b * p.ks[0] + h * p.ks[1] + dl * 8, v_base = b * p.vs[0] + h * p.vs[1] + dl * 8;
     const int64_t mask_base = p.has_mask ? b * p.ms[0] + h * p.ms[1] + (int64_t)m * p.ms[2] : 0;
 
     const int n_end = p.causal ? min(p.N, m + 1) : p.N;
@@ -70,23 +110,53 @@ __global__ void __launch_bounds__(256) attention_skinny_part1(const SkinnyParams
     const int c0 = split * per_split, c1 = min(n_end, c0 + per_split);
 
     float qf[8];
+    uint32_t qpk[4];  // the same 8 query features as packed pairs, unscaled (fp16 path)
     {
         const vec8 qv = *reinterpret_cast<const vec8 *>(qp);
 #pragma unroll
         for (int e = 0; e < 8; ++e) qf[e] = (float)qv[e] * p.scale_log2;
+        const u32x4 qraw = __builtin_bit_cast(u32x4, qv);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qpk[j] = qraw[j];
     }
     float mi = -INFINITY, li = 0.0f, acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 2
     for (int n0 = c0 + wave * KPW; n0 < c1; n0 += step) {
         const int n = n0 + kg;
         const bool valid = n < c1;
         const int nn = valid ? n : c1 - 1;  // c1 > c0 here, so c1 - 1 is a valid key
-        const vec8 kv = *reinterpret_cast<const vec8 *>(kp + (int64_t)nn * p.ks[2]);
-        const vec8 vv = *reinterpret_cast<const vec8 *>(vp + (int64_t)nn * p.vs[2]);
+        float vv[8];
         float s = 0.0f;
+        if constexpr (std::is_same<T, f16>::value) {
+            // fp16: the score from four two-element dot products with fp32 accumulation on the packed pairs, the
+            // values widened where they are used
+            typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+            uint32_t kpk[4], vpk[4];
+            sk_load8_pairs<KV8>(p.k, k_base + (int64_t)nn * p.ks[2], kpk);
+            sk_load8_pairs<KV8>(p.v, v_base + (int64_t)nn * p.vs[2], vpk);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) s += qf[e] * (float)kv[e];
+            for (int j = 0; j < 4; ++j)
+                s = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, kpk[j]), __builtin_bit_cast(h2, qpk[j]), s, false);
+            s *= p.scale_log2;
 #pragma unroll
-        for (int off = 1; off < DL; off <<= 1) s += __shfl_xor(s, off, 64);
+            for (int j = 0; j < 4; ++j) {
+                const h2 two = __builtin_bit_cast(h2, vpk[j]);
+                vv[2 * j] = (float)two[0];
+                vv[2 * j + 1] = (float)two[1];
+            }
+        } else {
+            float kv[8];
+            sk_load8<T, KV8>(p.k, k_base + (int64_t)nn * p.ks[2], kv);
+            sk_load8<T, KV8>(p.v, v_base + (int64_t)nn * p.vs[2], vv);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s += qf[e] * kv[e];
+        }
+        // sum over the DL lanes of the key: quad permutes and row mirrors on DPP, no trip through LDS
+        if (DL >= 2) s += dpp_mov<0xB1>(s);
+        if (DL >= 4) s += dpp_mov<0x4E>(s);
+        if (DL >= 8) s += dpp_mov<0x141>(s);
+        if (DL >= 16) s += dpp_mov<0x140>(s);
+        if (DL >= 32) s += __shfl_xor(s, 16, 64);
         if (p.has_mask) s += sk_mask_value(p.mask, p.mask_dtype, mask_base + (int64_t)nn * p.ms[3], p.clamp);
         if (!valid) s = -INFINITY;
         const float mn = fmaxf(mi, s);
@@ -96,7 +166,7 @@ __global__ void __launch_bounds__(256) attention_skinny_part1(const SkinnyParams
         const float pr = (float)from_float<T>(__builtin_amdgcn_exp2f(s - mu));
         li = li * alpha + pr;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] = acc[e] * alpha + pr * (float)vv[e];
+        for (int e = 0; e < 8; ++e) acc[e] = acc[e] * alpha + pr * vv[e];
         mi = mn;
     }
     // merge the KPW lane groups of the wave (same dl, different kg)
@@ -186,25 +256,27 @@ __global__ void __launch_bounds__(256) attention_skinny_part2(const SkinnyParams
     }
 }
 
-static int skinny_splits(int64_t rows, int64_t N, int D) {
+// key ranges per row: about `workgroups` workgroups over the whole grid (1024 = 4 per CU is where 16-bit keys and
+// values reach their bandwidth; one-byte storage has half the bytes per key in flight and wants all 8 per CU)
+static int skinny_splits(int64_t rows, int64_t N, int D, int workgroups) {
     const int step = 4 * (64 / (D / 8));
-    int64_t want = (1024 + rows - 1) / rows;  // about 4 workgroups per CU over the whole grid
+    int64_t want = (workgroups + rows - 1) / rows;
     const int64_t most = (N + step - 1) / step;
     if (want > most) want = most;
     if (want > 64) want = 64;
     return (int)(want < 1 ? 1 : want);
 }
 
-template <typename T>
+template <typename T, bool KV8>
 static void launch_skinny(const SkinnyParams &p, hipStream_t st) {
     dim3 grid((unsigned)p.splits, (unsigned)(p.B * p.H * p.M));
     switch (p.D / 8) {
-        case 1: hipLaunchKernelGGL((attention_skinny_part1<T, 1>), grid, dim3(256), 0, st, p); break;
-        case 2: hipLaunchKernelGGL((attention_skinny_part1<T, 2>), grid, dim3(256), 0, st, p); break;
-        case 4: hipLaunchKernelGGL((attention_skinny_part1<T, 4>), grid, dim3(256), 0, st, p); break;
-        case 8: hipLaunchKernelGGL((attention_skinny_part1<T, 8>), grid, dim3(256), 0, st, p); break;
-        case 16: hipLaunchKernelGGL((attention_skinny_part1<T, 16>), grid, dim3(256), 0, st, p); break;
-        default: hipLaunchKernelGGL((attention_skinny_part1<T, 32>), grid, dim3(256), 0, st, p); break;
+        case 1: hipLaunchKernelGGL((attention_skinny_part1<T, 1, KV8>), grid, dim3(256), 0, st, p); break;
+        case 2: hipLaunchKernelGGL((attention_skinny_part1<T, 2, KV8>), grid, dim3(256), 0, st, p); break;
+        case 4: hipLaunchKernelGGL((attention_skinny_part1<T, 4, KV8>), grid, dim3(256), 0, st, p); break;
+        case 8: hipLaunchKernelGGL((attention_skinny_part1<T, 8, KV8>), grid, dim3(256), 0, st, p); break;
+        case 16: hipLaunchKernelGGL((attention_skinny_part1<T, 16, KV8>), grid, dim3(256), 0, st, p); break;
+        default: hipLaunchKernelGGL((attention_skinny_part1<T, 32, KV8>), grid, dim3(256), 0, st, p); break;
     }
     if (p.splits > 1)
         hipLaunchKernelGGL((attention_skinny_part2<T>), dim3((unsigned)(p.B * p.H * p.M)), dim3(256), 0, st, p);
@@ -216,17 +288,16 @@ extern "C" int64_t kernl_attention_skinny_workspace_bytes(int64_t B, int64_t H, 
     using namespace kernl;
     if (B <= 0 || H <= 0 || M <= 0 || N <= 0 || D < 8 || D % 8 != 0) return 0;
     const int64_t rows = B * H * M;
-    const int splits = skinny_splits(rows, N, (int)D);
+    const int splits = skinny_splits(rows, N, (int)D, 2048);  // enough for either storage of the keys and values
     return splits > 1 ? rows * splits * (D + 2) * (int64_t)sizeof(float) : 0;
 }
 
-extern "C" int kernl_attention_skinny_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
-                                          void *workspace, int64_t workspace_bytes, int64_t B, int64_t H, int64_t M,
-                                          int64_t N, int64_t D, const int64_t q_strides[4],
-                                          const int64_t k_strides[4], const int64_t v_strides[4],
-                                          const int64_t o_strides[4], const int64_t mask_sizes[4],
-                                          const int64_t mask_strides[4], int mask_dtype, float sm_scale, int is_causal,
-                                          float mask_min_clamp, int dtype, void *stream) {
+static int skinny_entry(const void *q, const void *k, const void *v, void *out, const void *mask, void *workspace,
+                        int64_t workspace_bytes, int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
+                        const int64_t q_strides[4], const int64_t k_strides[4], const int64_t v_strides[4],
+                        const int64_t o_strides[4], const int64_t mask_sizes[4], const int64_t mask_strides[4],
+                        int mask_dtype, float sm_scale, int is_causal, float mask_min_clamp, int dtype, bool kv8,
+                        void *stream) {
     using namespace kernl;
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr || q_strides == nullptr ||
         k_strides == nullptr || v_strides == nullptr || o_strides == nullptr)
@@ -243,8 +314,14 @@ extern "C" int kernl_attention_skinny_fwd(const void *q, const void *k, const vo
     auto rows_ok = [](const void *ptr, const int64_t s[4]) {
         return s[3] == 1 && s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0 && aligned16(ptr);
     };
-    if (!rows_ok(q, q_strides) || !rows_ok(k, k_strides) || !rows_ok(v, v_strides))
-        return set_error(KERNL_ERR_UNSUPPORTED, "skinny attention: q, k, v need unit feature stride and 16-byte aligned rows");
+    // one-byte keys and values: 8 of them are an 8-byte load, and their strides count bytes
+    auto rows8_ok = [](const void *ptr, const int64_t s[4]) {
+        return s[3] == 1 && s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0 && (reinterpret_cast<uintptr_t>(ptr) & 7) == 0;
+    };
+    const bool kv_ok = kv8 ? rows8_ok(k, k_strides) && rows8_ok(v, v_strides) : rows_ok(k, k_strides) && rows_ok(v, v_strides);
+    if (!rows_ok(q, q_strides) || !kv_ok)
+        return set_error(KERNL_ERR_UNSUPPORTED, "skinny attention: q, k, v need unit feature stride and 16-byte aligned rows "
+                         "(8-byte aligned rows for one-byte keys and values)");
     if (N > (1 << 24)) return set_error(KERNL_ERR_UNSUPPORTED, "skinny attention: more than 2^24 keys");
     SkinnyParams p;
     p.has_mask = mask != nullptr;
@@ -267,7 +344,7 @@ extern "C" int kernl_attention_skinny_fwd(const void *q, const void *k, const vo
 
     const int64_t rows = B * H * M;
     if (rows > 65535) return set_error(KERNL_ERR_UNSUPPORTED, "skinny attention: more than 65535 (batch, head, query) rows");
-    int splits = skinny_splits(rows, N, (int)D);
+    int splits = skinny_splits(rows, N, (int)D, kv8 ? 2048 : 1024);
     if (splits > 1) {
         const int64_t per_split = rows * (D + 2) * (int64_t)sizeof(float);
         const int64_t fit = workspace != nullptr ? workspace_bytes / per_split : 0;
@@ -281,10 +358,40 @@ extern "C" int kernl_attention_skinny_fwd(const void *q, const void *k, const vo
     }
     p.mask_dtype = mask_dtype;
     p.causal = is_causal != 0;
+    p.kv8 = kv8 ? 1 : 0;
     p.scale_log2 = sm_scale * 1.4426950408889634f;
     p.clamp = mask_min_clamp;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (dtype == KERNL_F16) launch_skinny<f16>(p, st);
-    else launch_skinny<bf16>(p, st);
+    if (kv8) {
+        if (dtype == KERNL_F16) launch_skinny<f16, true>(p, st);
+        else launch_skinny<bf16, true>(p, st);
+    } else {
+        if (dtype == KERNL_F16) launch_skinny<f16, false>(p, st);
+        else launch_skinny<bf16, false>(p, st);
+    }
     return check_launch("attention (skinny)");
+}
+
+extern "C" int kernl_attention_skinny_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
+                                          void *workspace, int64_t workspace_bytes, int64_t B, int64_t H, int64_t M,
+                                          int64_t N, int64_t D, const int64_t q_strides[4],
+                                          const int64_t k_strides[4], const int64_t v_strides[4],
+                                          const int64_t o_strides[4], const int64_t mask_sizes[4],
+                                          const int64_t mask_strides[4], int mask_dtype, float sm_scale, int is_causal,
+                                          float mask_min_clamp, int dtype, void *stream) {
+    return skinny_entry(q, k, v, out, mask, workspace, workspace_bytes, B, H, M, N, D, q_strides, k_strides, v_strides,
+                        o_strides, mask_sizes, mask_strides, mask_dtype, sm_scale, is_causal, mask_min_clamp, dtype,
+                        false, stream);
+}
+
+extern "C" int kernl_attention_skinny_kv8_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
+                                              void *workspace, int64_t workspace_bytes, int64_t B, int64_t H, int64_t M,
+                                              int64_t N, int64_t D, const int64_t q_strides[4],
+                                              const int64_t k_strides[4], const int64_t v_strides[4],
+                                              const int64_t o_strides[4], const int64_t mask_sizes[4],
+                                              const int64_t mask_strides[4], int mask_dtype, float sm_scale,
+                                              int is_causal, float mask_min_clamp, int dtype, void *stream) {
+    return skinny_entry(q, k, v, out, mask, workspace, workspace_bytes, B, H, M, N, D, q_strides, k_strides, v_strides,
+                        o_strides, mask_sizes, mask_strides, mask_dtype, sm_scale, is_causal, mask_min_clamp, dtype,
+                        true, stream);
 }

@@ -13,6 +13,20 @@ from torch.amp import custom_fwd
 from kernl_amd import _lib
 
 
+ONE_BYTE_KV_DTYPES = (torch.int8, torch.uint8, torch.float8_e5m2)
+
+
+def to_e5m2(x: torch.Tensor) -> torch.Tensor:
+    """fp16 / bf16 / fp32 -> fp8 e5m2 (round to nearest even) as an int8 tensor of the same shape: the storage format
+    of the reference's key/value caches (`f16_to_f8`, experimental/llama-v2/kernel/fused_kernel_fp8.py:40-56)."""
+    return x.to(torch.float8_e5m2).view(torch.int8)
+
+
+def from_e5m2(x: torch.Tensor, dtype: torch.dtype = torch.float16) -> torch.Tensor:
+    """int8 / uint8 / float8_e5m2 storage -> `dtype` (reference: `f8_to_f16`, fused_kernel_fp8.py:20-37)."""
+    return x.view(torch.float8_e5m2).to(dtype)
+
+
 class SkinnyAttention(torch.autograd.Function):
     @staticmethod
     @custom_fwd(device_type="cuda", cast_inputs=torch.float16)
@@ -29,12 +43,16 @@ class SkinnyAttention(torch.autograd.Function):
         """out = softmax(q·kᵀ·sm_scale + causal + attention_mask)·v for very few query rows, written into `output`.
 
         q [batch, heads, m, d] with small m (decoding: 1); k, v [batch, heads, n, d]; attention_mask additive,
-        broadcastable as [batch|1, heads|1, m|1, n] (reference asserts: attention_skinny.py:401-454).
+        broadcastable as [batch|1, heads|1, m|1, n] (reference asserts: attention_skinny.py:401-454).  k and v may
+        be fp8 e5m2 storage (see `to_e5m2`): half the bytes to stream, same arithmetic on the decoded values.
         """
         assert q.shape[-1] == k.shape[-1]
-        assert (
-            q.dtype == k.dtype == v.dtype == output.dtype
-        ), f"All tensors must have the same dtype: {q.dtype}, {k.dtype}, {v.dtype}, {output.dtype}"
+        # keys and values either share the dtype of q, or are both stored as fp8 e5m2 (int8 / uint8 / float8_e5m2
+        # tensors; reference: `assert k.dtype == v.dtype and k.dtype in [torch.float16, torch.int8]`,
+        # experimental/llama-v2/kernel/fused_kernel_attention.py:115)
+        assert k.dtype == v.dtype and q.dtype == output.dtype and (
+            k.dtype == q.dtype or k.dtype in ONE_BYTE_KV_DTYPES
+        ), f"Incompatible dtypes: {q.dtype}, {k.dtype}, {v.dtype}, {output.dtype}"
         assert q.dtype in [torch.float16, torch.bfloat16], f"Only float16 and bfloat16 are supported, got {q.dtype}"
         batch, heads, m_size, dhead = q.size()
         n_size = k.size(2)

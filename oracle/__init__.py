@@ -8,6 +8,7 @@ from oracle.ops import (  # noqa: F401
     activation_oracle,
     attention_oracle,
     attention_tiled_oracle,
+    e5m2_decode_oracle,
     effective_eps,
     glu_oracle,
     layer_norm_oracle,

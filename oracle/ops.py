@@ -288,3 +288,21 @@ def rotary_complex_oracle(x: torch.Tensor, angles: torch.Tensor) -> torch.Tensor
     xc = torch.view_as_complex(x.float().reshape(*x.shape[:-1], -1, 2).contiguous())
     rot = torch.polar(torch.ones_like(angles, dtype=torch.float32), angles.float())
     return torch.view_as_real(xc * rot).flatten(-2)
+
+
+def e5m2_decode_oracle(raw: torch.Tensor) -> torch.Tensor:
+    """fp8 e5m2 bytes (int8 / uint8) -> fp32, from the format's definition: 1 sign bit, 5 exponent bits (bias 15),
+    2 mantissa bits; exponent 0 is subnormal (2^-14 · m/4), exponent 31 is inf (m = 0) or nan.  This is the storage of
+    the reference's key/value caches (experimental/llama-v2/kernel/fused_kernel_fp8.py:40-56), which its attention kernel
+    widens to fp16 before use (fused_kernel_attention.py:69-71).  Pinned in tests/test_oracle.py against
+    torch.float8_e5m2 and against the fp16 encoding's upper byte.
+    """
+    b = raw.detach().cpu().view(torch.uint8).to(torch.int32)
+    sign = torch.where((b >> 7) == 1, -1.0, 1.0)
+    exp = (b >> 2) & 0x1F
+    man = (b & 0x3).to(torch.float32)
+    normal = torch.ldexp(1.0 + man / 4.0, exp - 15)
+    subnormal = torch.ldexp(man / 4.0, torch.full_like(exp, -14))
+    val = torch.where(exp == 0, subnormal, normal)
+    val = torch.where(exp == 31, torch.where(man == 0, torch.tensor(float("inf")), torch.tensor(float("nan"))), val)
+    return sign * val

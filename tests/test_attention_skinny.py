@@ -135,3 +135,43 @@ def test_skinny_rejects_unsupported_head_size():
     k = torch.zeros((1, 1, 64, 48), dtype=torch.half, device="cuda")
     with pytest.raises(_lib.KernlLibraryError, match="head size"):
         skinny_attention_forward(q, k, k.clone(), torch.empty_like(q), 1.0)
+
+
+@pytest.mark.parametrize("storage", ["int8", "float8_e5m2"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [(2, 4, 1, 777, 64), (1, 8, 1, 4096, 128), (3, 2, 1, 51, 32), (2, 2, 3, 300, 64),
+                                   (1, 2, 1, 9, 8)], ids=lambda s: "x".join(map(str, s)))
+def test_skinny_fp8_keys_and_values(shape, dtype, storage, close):
+    """Keys and values stored as fp8 e5m2 (reference: the int8 caches of experimental/llama-v2/kernel/
+    fused_kernel_fp8.py:68-72, read by fused_kernel_attention.py:69-71,90-92): the kernel decodes the bytes and
+    computes as before, so it must match the oracle run on the DECODED keys and values — and the storage conversion
+    itself must match the oracle's decoder."""
+    from kernl_amd.implementations.attention_skinny import from_e5m2, to_e5m2
+    from oracle import e5m2_decode_oracle
+
+    B, H, M, N, D = shape
+    gen = torch.Generator().manual_seed(9)
+    q = torch.randn((B, H, M, D), generator=gen).to(dtype)
+    k = torch.randn((B, H, N, D), generator=gen)
+    v = torch.randn((B, H, N, D), generator=gen)
+    k8, v8 = to_e5m2(k), to_e5m2(v)
+    assert k8.dtype == torch.int8 and k8.shape == k.shape
+    k_dec, v_dec = e5m2_decode_oracle(k8), e5m2_decode_oracle(v8)
+    assert torch.equal(from_e5m2(k8, torch.float32), k_dec)
+    assert (k_dec - k).abs().max() <= 0.125 * k.abs().max()  # 2 mantissa bits: relative step 1/8 at most
+    mask = torch.rand((B, 1, 1, N), generator=gen)
+    if storage == "float8_e5m2":
+        k8, v8 = k8.view(torch.float8_e5m2), v8.view(torch.float8_e5m2)
+    qc = q.cuda()
+    out = torch.empty_like(qc)
+    skinny_attention_forward(qc, k8.cuda(), v8.cuda(), out, 0.25, is_causal=False, attention_mask=mask.cuda())
+    torch.cuda.synchronize()
+    close(out, attention_oracle(q, k_dec, v_dec, 0.25, False, mask), dtype, what=f"skinny fp8 kv {shape}")
+
+
+def test_skinny_fp8_rejects_misaligned_rows():
+    q = torch.randn((1, 1, 1, 64), device="cuda", dtype=torch.float16)
+    kv = torch.zeros((1, 1, 16, 68), device="cuda", dtype=torch.int8)[..., 4:]  # rows start 4 bytes off an 8-byte boundary
+    out = torch.empty_like(q)
+    with pytest.raises(RuntimeError, match="8-byte aligned"):
+        skinny_attention_forward(q, kv, kv, out, 1.0)

@@ -297,3 +297,20 @@ def test_attention_oracle_start_position_is_a_row_window_of_full_causal_attentio
     w = torch.softmax(torch.tensor(scores), dim=0)
     expect = sum(w[n] * v[0, 1, n] for n in range(len(scores)))
     assert torch.allclose(part[0, 1, m], expect, atol=1e-5)
+
+
+def test_e5m2_decode_oracle_against_library_and_fp16_upper_byte():
+    """Every one of the 256 codes: equal to torch.float8_e5m2 widened by the library, and equal to the fp16 value whose
+    upper byte is the code and whose lower byte is zero (nan compared as nan)."""
+    from oracle import e5m2_decode_oracle
+    codes = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    got = e5m2_decode_oracle(codes)
+    lib = codes.view(torch.float8_e5m2).to(torch.float32)
+    upper = (codes.to(torch.int32) << 8).to(torch.int16).view(torch.float16).to(torch.float32)
+    for other in (lib, upper):
+        assert torch.equal(torch.isnan(got), torch.isnan(other))
+        ok = ~torch.isnan(got)
+        assert torch.equal(got[ok], other[ok])
+    # known values: 0x3C = 1.0, 0x40 = 2.0, 0xC5 = -5.0, 0x01 = 2^-16 (smallest subnormal), 0x7B = 57344 (largest finite)
+    for code, value in ((0x3C, 1.0), (0x40, 2.0), (0xC5, -5.0), (0x01, 2.0 ** -16), (0x7B, 57344.0)):
+        assert got[code].item() == value
