@@ -133,21 +133,63 @@ def replace_linear_fn_constant_match(gm: torch.fx.GraphModule):
     replace_pattern(gm, pattern, replace)
 
 
-# concatenated parameters of fused sibling projections, keyed by the identity of the original tensors
-_fused_params = {}
+class _DerivedParams:
+    """Tensors derived from a group of parameters (concatenated or interleaved weights), kept for as long as the
+    parameters they were made from are alive and unchanged.
+
+    The key is the originals' storage addresses, versions and dtypes; an address alone is not an identity — once a
+    model is freed the allocator hands the same addresses to the next one — so every entry also holds weak references
+    to the original tensors and is dropped as soon as one of them has died or moved."""
+
+    def __init__(self):
+        self._entries = {}
+
+    @staticmethod
+    def key_of(params):
+        return tuple((0, 0, None) if p is None else (p.data_ptr(), p._version, p.dtype) for p in params)
+
+    def get(self, params):
+        entry = self._entries.get(self.key_of(params))
+        if entry is None:
+            return None
+        refs, value = entry
+        for ref, p in zip(refs, params):
+            if p is None:
+                continue
+            alive = ref()
+            # the tensor passed in may be an alias of the original (same storage); what matters is that the original
+            # still owns that memory
+            if alive is None or alive.data_ptr() != p.data_ptr() or alive._version != p._version:
+                del self._entries[self.key_of(params)]
+                return None
+        return value
+
+    def put(self, params, value):
+        import weakref
+
+        self._entries = {
+            k: (refs, v) for k, (refs, v) in self._entries.items() if all(r is None or r() is not None for r in refs)
+        }
+        refs = [None if p is None else weakref.ref(p) for p in params]
+        self._entries[self.key_of(params)] = (refs, value)
+
+    def __len__(self):
+        return len(self._entries)
+
+
+# concatenated / interleaved parameters of fused projections
+_fused_params = _DerivedParams()
 
 
 def fused_linear_wrapper(v: torch.Tensor, weights, biases):
     """Several activation-free linears of the SAME input (BERT's query/key/value projections) as ONE GEMM against
     the row-concatenated weights; returns the outputs as column slices of the single result.
 
-    The concatenated weight is built on the first call (the warm-up call that precedes graph capture) and cached by
-    the storage addresses and versions of the originals, so replays neither allocate nor copy.  No counterpart in the
+    The concatenated weight is built on the first call (the warm-up call that precedes graph capture) and kept for as
+    long as the original parameters live unchanged, so capture and replays neither allocate nor copy.  No counterpart in the
     reference, which launches one Triton GEMM per projection."""
-    key = tuple((w.data_ptr(), w._version, w.dtype) for w in weights) + tuple(
-        (0, 0, None) if b is None else (b.data_ptr(), b._version, b.dtype) for b in biases
-    )
-    cached = _fused_params.get(key)
+    originals = tuple(weights) + tuple(biases)
+    cached = _fused_params.get(originals)
     if cached is None:
         for w, b in zip(weights, biases):
             # same one-time down-cast as linear_wrapper_functional
@@ -161,11 +203,8 @@ def fused_linear_wrapper(v: torch.Tensor, weights, biases):
             bias = torch.cat(
                 [torch.zeros(w.shape[0], dtype=w.dtype, device=w.device) if b is None else b.detach() for w, b in zip(weights, biases)]
             ).contiguous()
-        key = tuple((w.data_ptr(), w._version, w.dtype) for w in weights) + tuple(
-            (0, 0, None) if b is None else (b.data_ptr(), b._version, b.dtype) for b in biases
-        )
         cached = (weight, bias, [w.shape[0] for w in weights])
-        _fused_params[key] = cached
+        _fused_params.put(originals, cached)  # keyed after the one-time cast: by the addresses the parameters keep
     weight, bias, sizes = cached
     out = linear_layer(v, weight, bias, activation="")
     return tuple(torch.split(out, sizes, dim=-1))
@@ -232,17 +271,15 @@ def glu_linear_wrapper(v: torch.Tensor, w_gate, b_gate, w_value, b_value, activa
         gate = linear_wrapper_functional(v, w_gate, b_gate, activation=activation)
         return gate * linear_wrapper_functional(v, w_value, b_value)
     params = (w_gate, w_value) + (() if b_gate is None else (b_gate, b_value))
-    key = ("glu",) + tuple((p.data_ptr(), p._version, p.dtype) for p in params)
-    cached = _fused_params.get(key)
+    cached = _fused_params.get(params)
     if cached is None:
         for p in params:
             if p.dtype == torch.float32 and half:
                 p.data = p.data.half()
         weight = interleave_glu_rows(w_gate.detach(), w_value.detach())
         bias = None if b_gate is None else interleave_glu_rows(b_gate.detach(), b_value.detach())
-        key = ("glu",) + tuple((p.data_ptr(), p._version, p.dtype) for p in params)
         cached = (weight, bias)
-        _fused_params[key] = cached
+        _fused_params.put(params, cached)
     weight, bias = cached
     return linear_glu_layer(v, weight, bias, activation=activation)
 

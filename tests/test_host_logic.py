@@ -446,3 +446,37 @@ def test_glu_row_interleaving_and_pass():
     gm = torch.fx.symbolic_trace(Shared())
     replace_all_linear(gm)
     assert "glu_linear_wrapper" not in _targets(gm)
+
+
+def test_derived_parameter_cache_follows_the_life_of_its_parameters():
+    """Concatenated / interleaved weights are kept per group of original parameters.  A storage address is not an
+    identity (the allocator hands a freed model's addresses to the next model), so an entry must stop matching as soon
+    as one of its originals has died, moved or been written to — also when another tensor then shows the same address."""
+    import gc
+
+    from kernl_amd.optimizer.linear import _DerivedParams
+
+    cache = _DerivedParams()
+    a, b = torch.zeros(8), torch.ones(4)
+    assert cache.get((a, None, b)) is None
+    cache.put((a, None, b), "derived from a, b")
+    assert cache.get((a, None, b)) == "derived from a, b"
+    alias = torch.empty(0).set_(a.untyped_storage(), 0, (8,))   # same storage and address, no reference to `a`
+    a.add_(1)                                 # written to: the derived tensor is stale
+    assert cache.get((a, None, b)) is None
+    cache.put((a, None, b), "again")
+    assert cache.get((a, None, b)) == "again"
+    assert _DerivedParams.key_of((alias, None, b)) == _DerivedParams.key_of((a, None, b))  # address, version, dtype
+    del a
+    gc.collect()
+    # `alias` keeps the memory alive at the same address, as a new model's parameter would after the allocator
+    # recycled it — but the tensor the entry was made from is gone
+    assert cache.get((alias, None, b)) is None
+    # entries of dead parameters are swept when something new is stored
+    c = torch.zeros(3)
+    cache.put((c,), 1)
+    del c
+    gc.collect()
+    d = torch.zeros(5)
+    cache.put((d,), 2)
+    assert len(cache) == 1 and cache.get((d,)) == 2

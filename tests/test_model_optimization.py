@@ -320,3 +320,36 @@ def test_generation_with_growing_cache(family):
         agree += 1
     print(f"{family}: greedy paths agree for {agree} of {steps} steps", flush=True)
     assert agree >= 3
+
+
+def test_models_built_one_after_the_other_do_not_share_fused_weights():
+    """Two models of the same shapes, different weights, built and optimized one after the other with the first one
+    freed in between: the allocator may give the second model the first one's parameter addresses, and the
+    concatenated query/key/value weight kept for the first must not be served to the second."""
+    import gc
+
+    from kernl_amd.model_optimization import optimize_model
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q, self.k, self.v = (torch.nn.Linear(256, 256) for _ in range(3))
+
+        def forward(self, x):
+            return self.q(x) + 2.0 * self.k(x) - self.v(x)
+
+    x = torch.randn((4, 128, 256), generator=torch.Generator().manual_seed(0)).half().cuda()
+    for seed in (1, 2, 3):
+        torch._dynamo.reset()
+        torch.manual_seed(seed)
+        model = Block().eval().half().cuda()
+        with torch.inference_mode():
+            expected = model(x).float().cpu()
+        optimize_model(model)
+        with torch.inference_mode():
+            model(x)
+            out = model(x).float().cpu()
+        assert (out - expected).abs().max().item() < 2e-2, f"model {seed}: fused projection used stale weights"
+        del model
+        gc.collect()
+        torch.cuda.empty_cache()
