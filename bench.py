@@ -340,7 +340,18 @@ def main():
             extra["decode_linear_1x4096x4096_us_graph_replay"] = round(t * 1e3, 2)
             extra["decode_linear_gbps_graph_replay"] = round(w_bytes / (t * 1e-3) / 1e9, 1)
             extra["decode_linear_frac_of_hbm_peak"] = round(w_bytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
-            del w_dec, x_dec
+            # the same step with the weights stored as fp8 e5m2
+            w_dec8 = [w_i.to(torch.float8_e5m2).view(torch.int8) for w_i in w_dec]
+            del w_dec
+
+            def decode_linears_fp8():
+                for w_i in w_dec8:
+                    linear_layer(x_dec, w_i, None)
+
+            t = graph_time_ms(decode_linears_fp8, reps=4) / len(w_dec8)
+            extra["decode_linear_fp8w_us_graph_replay"] = round(t * 1e3, 2)
+            extra["decode_linear_fp8w_gbps_graph_replay"] = round(w_dec8[0].numel() / (t * 1e-3) / 1e9, 1)
+            del w_dec8, x_dec
         except Exception as exc:  # the headline must still be printed
             extra["decoder_kernels_error"] = f"{type(exc).__name__}: {exc}"[:300]
 

@@ -165,6 +165,19 @@ int kernl_linear_fwd(const void *x, const void *w, const void *bias, void *out, 
                      const int64_t act_in_strides[2], int activation, int dtype, void *stream);
 
 /*
+ * kernl_linear_fwd for a weight stored as one byte per element, fp8 e5m2 — the upper byte of the fp16 encoding
+ * (reference: `get_model_fp8` turns the weights of the projections into int8 tensors holding float8e5,
+ * experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84, and its kernels widen them on load,
+ * fused_kernel_ff.py:43-47).  w8 [N, K] contiguous bytes.  This is the decoding-step kernel only: M <= 64,
+ * K % 64 == 0, dtype KERNL_F16 (x, bias, out, act_in); anything else returns KERNL_ERR_UNSUPPORTED and the caller
+ * widens the weight.  Half the bytes of the weight stream, fp32 accumulation of the decoded values.
+ */
+int kernl_linear_w8_fwd(const void *x, const void *w8, const void *bias, void *out, void *act_in,
+                        int64_t M, int64_t N, int64_t K, const int64_t x_strides[2],
+                        const int64_t out_strides[2], const int64_t act_in_strides[2], int activation,
+                        int dtype, void *stream);
+
+/*
  * Gated linear unit:  out[M,N] = act(x·w_gateᵀ + b_gate) * (x·w_valueᵀ + b_value)  as ONE GEMM.
  * Replaces the `ff_llama` launch of experimental/llama-v2/kernel/fused_kernel_ff.py:10-79 (SwiGLU: act = SiLU; that
  * kernel's RMSNorm prologue is not part of this entry point) — and the three kernels (two GEMMs, one multiply) a

@@ -28,6 +28,7 @@ EXPORTED_SYMBOLS = (
     "kernl_attention_skinny_kv8_fwd",
     "kernl_rope_fwd",
     "kernl_linear_fwd",
+    "kernl_linear_w8_fwd",
     "kernl_linear_glu_fwd",
     "kernl_layernorm_fwd",
     "kernl_add_layernorm_fwd",
@@ -85,6 +86,8 @@ def load() -> ctypes.CDLL:
     lib.kernl_rope_fwd.argtypes = [_vp] * 4 + [_i64] * 4 + [_i64p] * 5 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_linear_fwd.restype = ctypes.c_int
     lib.kernl_linear_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
+    lib.kernl_linear_w8_fwd.restype = ctypes.c_int
+    lib.kernl_linear_w8_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_linear_glu_fwd.restype = ctypes.c_int
     lib.kernl_linear_glu_fwd.argtypes = [_vp] * 4 + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_layernorm_fwd.restype = ctypes.c_int
@@ -218,6 +221,32 @@ def linear_fwd(x2d, weight, bias, out2d, act_in2d, activation: int) -> None:
             int(activation), DTYPE_CODE[x2d.dtype], _stream(x2d),
         )
     _check(st, "kernl_linear_fwd")
+
+
+def linear_w8_supported(x2d, weight8) -> bool:
+    """What `kernl_linear_w8_fwd` takes: fp16 rows, at most 64 of them, K a multiple of 64."""
+    M, K = x2d.shape
+    return (
+        x2d.dtype == torch.float16 and M <= 64 and K % 64 == 0 and x2d.stride(1) == 1 and x2d.stride(0) % 8 == 0
+        and x2d.data_ptr() % 16 == 0 and weight8.is_contiguous() and weight8.data_ptr() % 16 == 0
+    )
+
+
+def linear_w8_fwd(x2d, weight8, bias, out2d, act_in2d, activation: int) -> None:
+    """weight8 [N, K]: fp8 e5m2 bytes (int8 / uint8 / float8_e5m2)."""
+    _require_gpu(x2d, weight8, bias, out2d, act_in2d)
+    M, K = x2d.shape
+    N = weight8.shape[0]
+    lib = load()
+    with torch.cuda.device(x2d.device):
+        st = lib.kernl_linear_w8_fwd(
+            x2d.data_ptr(), weight8.data_ptr(), None if bias is None else bias.data_ptr(), out2d.data_ptr(),
+            None if act_in2d is None else act_in2d.data_ptr(),
+            M, N, K,
+            _arr(x2d.stride()), _arr(out2d.stride()), None if act_in2d is None else _arr(act_in2d.stride()),
+            int(activation), DTYPE_CODE[x2d.dtype], _stream(x2d),
+        )
+    _check(st, "kernl_linear_w8_fwd")
 
 
 def linear_glu_fwd(x2d, weight_interleaved, bias_interleaved, out2d, activation: int) -> None:

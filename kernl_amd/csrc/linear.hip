@@ -10,6 +10,8 @@
 // "B" side, i.e. the instruction produces a 32(n) x 32(m) block of outᵀ; together with the row permutation
 // rowperm16 on the weight tile this leaves every lane holding 16 consecutive output columns of one output
 // row, so bias loads and output stores are 16-byte vectors without any shuffle through LDS.
+#include <type_traits>
+
 #include "common.h"
 
 namespace kernl {
@@ -975,7 +977,11 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
 // of MFMA k-group g supplies k = 16 g + 8 s .. + 7 of the chunk in step s (s = 0, 1), on both sides, which is all
 // the instruction needs.  The waves' partial sums meet in LDS.  x is re-read by every workgroup, from L2.
 // ----------------------------------------------------------------------------------------------------
-template <typename T, int MB, bool GATED, int WAVES, int NR>
+// W8: the weight is stored as one byte per element, fp8 e5m2 — the upper byte of the fp16 encoding (reference:
+// `get_model_fp8`, experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84, read back with `.to(tl.float8e5,
+// bitcast=True).to(tl.float16)`, fused_kernel_ff.py:43-47).  A lane then fetches its 16 weights of a chunk as ONE
+// 16-byte load and byte-permutes them into the two fp16 fragments; fp16 activations only.
+template <typename T, int MB, bool GATED, int WAVES, int NR, bool W8 = false>
 __global__ void __launch_bounds__(64 * WAVES)
 linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
                      T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
@@ -993,16 +999,19 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
     // first interleaved row of the 16 output columns starting at nb (gated weights: 32 gate rows, 32 value rows, ...)
     auto gated_row = [](int nb) -> int { return (nb >> 5) * 64 + (nb & 31); };
     // rows of the weight this lane reads; columns beyond N repeat the last one and are never stored
-    const T *wp[NF];
+    static_assert(!W8 || std::is_same<T, f16>::value, "one-byte weights are decoded to fp16");
+    typedef typename std::conditional<W8, unsigned char, T>::type WT;  // what a weight element is stored as
+    const WT *wbase = reinterpret_cast<const WT *>(W);
+    const WT *wp[NF];
 #pragma unroll
     for (int rb = 0; rb < NR; ++rb) {
         const int nb = n0 + 16 * rb;
         if (GATED) {
             const int row = gated_row(min(nb, N - 16)) + r;
-            wp[rb * NA] = W + (int64_t)row * K + 16 * g;
-            wp[rb * NA + NA - 1] = W + (int64_t)(row + 32) * K + 16 * g;
+            wp[rb * NA] = wbase + (int64_t)row * K + 16 * g;
+            wp[rb * NA + NA - 1] = wbase + (int64_t)(row + 32) * K + 16 * g;
         } else {
-            wp[rb * NA] = W + (int64_t)min(nb + r, N - 1) * K + 16 * g;
+            wp[rb * NA] = wbase + (int64_t)min(nb + r, N - 1) * K + 16 * g;
         }
     }
     const T *xp[MB];
@@ -1028,8 +1037,22 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
             const int k0 = cc * 64;
 #pragma unroll
             for (int f = 0; f < NF; ++f) {
-                wf[u][f][0] = *reinterpret_cast<const vec8 *>(wp[f] + k0);
-                wf[u][f][1] = *reinterpret_cast<const vec8 *>(wp[f] + k0 + 8);
+                if constexpr (W8) {
+                    const u32x4 raw = *reinterpret_cast<const u32x4 *>(wp[f] + k0);
+                    u32x4 lo, hi;  // bytes {0, b0, 0, b1} / {0, b2, 0, b3} of every word: fp16 pairs
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        lo[2 * j] = __builtin_amdgcn_perm(0u, raw[j], 0x010c000cu);
+                        lo[2 * j + 1] = __builtin_amdgcn_perm(0u, raw[j], 0x030c020cu);
+                        hi[2 * j] = __builtin_amdgcn_perm(0u, raw[2 + j], 0x010c000cu);
+                        hi[2 * j + 1] = __builtin_amdgcn_perm(0u, raw[2 + j], 0x030c020cu);
+                    }
+                    wf[u][f][0] = __builtin_bit_cast(vec8, lo);
+                    wf[u][f][1] = __builtin_bit_cast(vec8, hi);
+                } else {
+                    wf[u][f][0] = *reinterpret_cast<const vec8 *>(wp[f] + k0);
+                    wf[u][f][1] = *reinterpret_cast<const vec8 *>(wp[f] + k0 + 8);
+                }
             }
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
@@ -1335,7 +1358,7 @@ static int pick_tile(int M, int N, int K, bool gated) {
 
 int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192
 
-template <typename T, bool GATED, int MB, int NR>
+template <typename T, bool GATED, int MB, int NR, bool W8>
 static void launch_skinny_blocks(const LinearArgs &a) {
     const int n_out = GATED ? a.N / 2 : a.N;
     const dim3 grid((unsigned)((n_out + 16 * NR - 1) / (16 * NR)));
@@ -1351,7 +1374,7 @@ static void launch_skinny_blocks(const LinearArgs &a) {
     if (per_cu >= 3) waves = 4;
     else if (per_cu == 2 && waves > 8) waves = 8;
 #define KERNL_SKINNY(WV)                                                                                                \
-    hipLaunchKernelGGL((linear_skinny_kernel<T, MB, GATED, WV, NR>), grid, dim3(64 * WV), 0, a.st,                      \
+    hipLaunchKernelGGL((linear_skinny_kernel<T, MB, GATED, WV, NR, W8>), grid, dim3(64 * WV), 0, a.st,                      \
                        static_cast<const T *>(a.x), static_cast<const T *>(a.w), static_cast<const T *>(a.bias),       \
                        static_cast<T *>(a.out), static_cast<T *>(a.act_in), a.M, n_out, a.K, a.x_rs, a.out_rs, a.out_cs, \
                        a.ai_rs, a.ai_cs, act)
@@ -1365,16 +1388,16 @@ static void launch_skinny_blocks(const LinearArgs &a) {
 #undef KERNL_SKINNY
 }
 
-template <typename T, bool GATED>
+template <typename T, bool GATED, bool W8 = false>
 static void launch_skinny(const LinearArgs &a) {
     const int n_out = GATED ? a.N / 2 : a.N;
     const int mb = (a.M + 15) / 16;
     // every workgroup reads all of x (from L2): with more than 16 rows of x and enough output columns to fill the
     // chip twice over, a workgroup takes 32 columns and that traffic halves
     const bool two = n_out >= 8192 && mb >= 2;
-    if (mb <= 1) { if (two) launch_skinny_blocks<T, GATED, 1, 2>(a); else launch_skinny_blocks<T, GATED, 1, 1>(a); }
-    else if (mb <= 2) { if (two) launch_skinny_blocks<T, GATED, 2, 2>(a); else launch_skinny_blocks<T, GATED, 2, 1>(a); }
-    else { if (two) launch_skinny_blocks<T, GATED, 4, 2>(a); else launch_skinny_blocks<T, GATED, 4, 1>(a); }
+    if (mb <= 1) { if (two) launch_skinny_blocks<T, GATED, 1, 2, W8>(a); else launch_skinny_blocks<T, GATED, 1, 1, W8>(a); }
+    else if (mb <= 2) { if (two) launch_skinny_blocks<T, GATED, 2, 2, W8>(a); else launch_skinny_blocks<T, GATED, 2, 1, W8>(a); }
+    else { if (two) launch_skinny_blocks<T, GATED, 4, 2, W8>(a); else launch_skinny_blocks<T, GATED, 4, 1, W8>(a); }
 }
 
 template <typename T>
@@ -1493,4 +1516,38 @@ extern "C" int kernl_linear_glu_fwd(const void *x, const void *w, const void *bi
                          "and K a multiple of 8");
     if (M == 0) return KERNL_OK;
     return dtype == KERNL_F16 ? linear_mfma_dispatch<f16>(a) : linear_mfma_dispatch<bf16>(a);
+}
+
+extern "C" int kernl_linear_w8_fwd(const void *x, const void *w8, const void *bias, void *out, void *act_in, int64_t M,
+                                   int64_t N, int64_t K, const int64_t x_strides[2], const int64_t out_strides[2],
+                                   const int64_t act_in_strides[2], int activation, int dtype, void *stream) {
+    using namespace kernl;
+    if (x == nullptr || w8 == nullptr || out == nullptr || x_strides == nullptr || out_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear (fp8 weight): x, w, out and their strides must not be NULL");
+    if (act_in != nullptr && act_in_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear (fp8 weight): act_in given without strides");
+    if (M < 0 || N <= 0 || K <= 0)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear (fp8 weight): bad sizes M=%lld N=%lld K=%lld", (long long)M,
+                         (long long)N, (long long)K);
+    if (activation < KERNL_ACT_NONE || activation > KERNL_ACT_SILU)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear (fp8 weight): unknown activation %d", activation);
+    if (dtype != KERNL_F16)
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear (fp8 weight): activations must be f16, got dtype %d", dtype);
+    if (M > 64 || K % 64 != 0 || N > INT32_MAX || K > INT32_MAX)
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear (fp8 weight): at most 64 rows of x and K a multiple of 64 "
+                         "(M=%lld K=%lld); widen the weight for larger inputs", (long long)M, (long long)K);
+    if (x_strides[1] != 1 || x_strides[0] % 8 != 0 || !aligned16(x) || !aligned16(w8))
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear (fp8 weight): x needs unit feature stride and 16-byte aligned "
+                         "rows, the weight a 16-byte aligned base");
+    if (M == 0) return KERNL_OK;
+    LinearArgs a;
+    a.x = x; a.w = w8; a.bias = bias; a.out = out; a.act_in = act_in;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.x_rs = x_strides[0]; a.x_cs = x_strides[1];
+    a.out_rs = out_strides[0]; a.out_cs = out_strides[1];
+    a.ai_rs = act_in ? act_in_strides[0] : 0; a.ai_cs = act_in ? act_in_strides[1] : 0;
+    a.act = activation;
+    a.st = static_cast<hipStream_t>(stream);
+    launch_skinny<f16, false, true>(a);
+    return check_launch("linear (skinny, fp8 weight)");
 }

@@ -22,6 +22,9 @@ ACTIVATIONS = {
 }
 
 
+ONE_BYTE_WEIGHT_DTYPES = (torch.int8, torch.uint8, torch.float8_e5m2)
+
+
 class LinearLayer(torch.autograd.Function):
     @staticmethod
     @custom_fwd(device_type="cuda", cast_inputs=torch.float16)
@@ -35,6 +38,20 @@ class LinearLayer(torch.autograd.Function):
     ) -> torch.Tensor:
         """e = activation(x @ weightᵀ + bias); `act_inputs` (optional, [M, N]) receives the pre-activation."""
         x_ = x if x.ndim == 2 else x.reshape(-1, x.shape[-1])
+
+        if weight.dtype in ONE_BYTE_WEIGHT_DTYPES:
+            # fp8 e5m2 weight storage (reference: experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84): decoding
+            # steps stream the bytes; larger inputs widen the weight first and take the ordinary kernels
+            assert x.dtype == torch.float16, f"fp8 weights go with float16 activations, got {x.dtype}"
+            assert weight.is_contiguous() and x_.shape[1] == weight.shape[1]
+            if x_.stride(-1) != 1 or x_.stride(0) % 8 != 0 or x_.data_ptr() % 16 != 0:
+                x_ = x_.contiguous()
+            if _lib.linear_w8_supported(x_, weight):
+                M, N = x_.shape[0], weight.shape[0]
+                outputs = torch.empty((M, N), device=x.device, dtype=x.dtype)
+                _lib.linear_w8_fwd(x_, weight, bias, outputs, act_inputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
+                return outputs if x.ndim == 2 else outputs.reshape(*x.shape[:-1], N)
+            weight = weight.view(torch.float8_e5m2).to(torch.float16)
 
         assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
         if bias is not None:

@@ -144,6 +144,28 @@ def test_linear_few_rows_streams_the_weight(shape, activation, dtype, close):
     close(out_nobias, linear_oracle(x, w, None, activation), dtype, what=f"few rows {shape} no bias")
 
 
+@pytest.mark.parametrize("activation", ["", "silu"])
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (5, 80, 64), (16, 1000, 192), (33, 9000, 192), (64, 512, 1024),
+                                   (100, 256, 128), (4, 96, 72)], ids=lambda s: "x".join(map(str, s)))
+def test_linear_fp8_weight_storage(shape, activation, close):
+    """Weight stored as fp8 e5m2 (reference: `get_model_fp8`, experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84):
+    the result must be the oracle's on the DECODED weight.  Up to 64 rows and K % 64 == 0 stream the bytes; 100 rows
+    and K = 72 go through the widened weight."""
+    from oracle import e5m2_decode_oracle
+
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(29)
+    x, w, b = _inputs(M, N, K, torch.float16, gen, w_std=K ** -0.5)
+    w8 = w.to(torch.float8_e5m2).view(torch.int8)
+    w_dec = e5m2_decode_oracle(w8)
+    act_in = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    out = linear_layer(x.cuda(), w8.cuda(), b.cuda(), activation=activation, act_inputs=act_in)
+    torch.cuda.synchronize()
+    ref, pre = linear_oracle(x, w_dec, b, activation, return_act_inputs=True)
+    close(out, ref, what=f"fp8 weight {shape} {activation!r}")
+    close(act_in, pre, what=f"fp8 weight {shape} pre-activation")
+
+
 def test_linear_few_rows_strided_output_and_batched_input(close):
     gen = torch.Generator().manual_seed(18)
     x, w, b = _inputs(2, 640, 256, torch.float16, gen, w_std=1 / 16, batch=3)  # [3, 2, 256] -> 6 rows
