@@ -178,6 +178,21 @@ int kernl_linear_w8_fwd(const void *x, const void *w8, const void *bias, void *o
                         int dtype, void *stream);
 
 /*
+ * RMSNorm fused into the linear layer that consumes it:
+ *     out = activation( rsqrt(mean(x^2) + eps) * ((x * rms_weight) @ w^T) + bias )        (gated = 0)
+ *     out = activation(gate) * value, both computed like that from the interleaved weight    (gated != 0)
+ * Replaces the `rms_matmul_rbe[grid](...)` launch without its rotary epilogue (experimental/llama-v2/kernel/
+ * fused_kernel_proj_qkv.py:116-183, 186-213) and the RMSNorm prologue of `ff_llama` (fused_kernel_ff.py:10-79): as
+ * there, x * rms_weight is rounded to the 16-bit type before the product and the inverse root mean square, one
+ * scalar per row, multiplies the finished sums.  This is the decoding-step kernel: M <= 64, K % 64 == 0, f16 / bf16;
+ * anything else returns KERNL_ERR_UNSUPPORTED and the caller normalises and multiplies in two calls.  w [N, K], or
+ * [2N, K] interleaved as for kernl_linear_glu_fwd; bias likewise or NULL.
+ */
+int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float eps, const void *w, const void *bias, void *out,
+                         int64_t M, int64_t N, int64_t K, const int64_t x_strides[2], const int64_t out_strides[2],
+                         int activation, int gated, int dtype, void *stream);
+
+/*
  * Gated linear unit:  out[M,N] = act(x·w_gateᵀ + b_gate) * (x·w_valueᵀ + b_value)  as ONE GEMM.
  * Replaces the `ff_llama` launch of experimental/llama-v2/kernel/fused_kernel_ff.py:10-79 (SwiGLU: act = SiLU; that
  * kernel's RMSNorm prologue is not part of this entry point) — and the three kernels (two GEMMs, one multiply) a

@@ -29,6 +29,7 @@ EXPORTED_SYMBOLS = (
     "kernl_rope_fwd",
     "kernl_linear_fwd",
     "kernl_linear_w8_fwd",
+    "kernl_linear_rms_fwd",
     "kernl_linear_glu_fwd",
     "kernl_layernorm_fwd",
     "kernl_add_layernorm_fwd",
@@ -88,6 +89,10 @@ def load() -> ctypes.CDLL:
     lib.kernl_linear_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_linear_w8_fwd.restype = ctypes.c_int
     lib.kernl_linear_w8_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
+    lib.kernl_linear_rms_fwd.restype = ctypes.c_int
+    lib.kernl_linear_rms_fwd.argtypes = (
+        [_vp, _vp, ctypes.c_float, _vp, _vp, _vp] + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int] * 3 + [_vp]
+    )
     lib.kernl_linear_glu_fwd.restype = ctypes.c_int
     lib.kernl_linear_glu_fwd.argtypes = [_vp] * 4 + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_layernorm_fwd.restype = ctypes.c_int
@@ -247,6 +252,30 @@ def linear_w8_fwd(x2d, weight8, bias, out2d, act_in2d, activation: int) -> None:
             int(activation), DTYPE_CODE[x2d.dtype], _stream(x2d),
         )
     _check(st, "kernl_linear_w8_fwd")
+
+
+def linear_rms_supported(x2d) -> bool:
+    """What `kernl_linear_rms_fwd` takes: 16-bit rows, at most 64 of them, K a multiple of 64."""
+    M, K = x2d.shape
+    return (
+        x2d.dtype in (torch.float16, torch.bfloat16) and M <= 64 and K % 64 == 0 and x2d.stride(1) == 1
+        and x2d.stride(0) % 8 == 0 and x2d.data_ptr() % 16 == 0
+    )
+
+
+def linear_rms_fwd(x2d, rms_weight, eps: float, weight, bias, out2d, activation: int, gated: bool) -> None:
+    _require_gpu(x2d, rms_weight, weight, bias, out2d)
+    M, K = x2d.shape
+    N = out2d.shape[1]
+    lib = load()
+    with torch.cuda.device(x2d.device):
+        st = lib.kernl_linear_rms_fwd(
+            x2d.data_ptr(), rms_weight.data_ptr(), float(eps), weight.data_ptr(),
+            None if bias is None else bias.data_ptr(), out2d.data_ptr(), M, N, K,
+            _arr(x2d.stride()), _arr(out2d.stride()), int(activation), int(bool(gated)), DTYPE_CODE[x2d.dtype],
+            _stream(x2d),
+        )
+    _check(st, "kernl_linear_rms_fwd")
 
 
 def linear_glu_fwd(x2d, weight_interleaved, bias_interleaved, out2d, activation: int) -> None:

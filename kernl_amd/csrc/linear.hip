@@ -981,17 +981,22 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
 // `get_model_fp8`, experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84, read back with `.to(tl.float8e5,
 // bitcast=True).to(tl.float16)`, fused_kernel_ff.py:43-47).  A lane then fetches its 16 weights of a chunk as ONE
 // 16-byte load and byte-permutes them into the two fp16 fragments; fp16 activations only.
-template <typename T, int MB, bool GATED, int WAVES, int NR, bool W8 = false>
+// RMS: x is RMS-normalised on the way in (reference: `rms_matmul_rbe`, experimental/llama-v2/kernel/
+// fused_kernel_proj_qkv.py:116-183): the x fragments are multiplied by the norm's weight (rounded to 16 bit, as there),
+// every lane sums the squares of the x values that pass through it, and because the inverse root mean square is one
+// scalar per row it is applied to the finished sums: out = rsqrt(mean(x^2) + eps) * ((x * g) @ w^T) + bias.
+template <typename T, int MB, bool GATED, int WAVES, int NR, bool W8 = false, bool RMS = false>
 __global__ void __launch_bounds__(64 * WAVES)
 linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
                      T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
-                     int64_t ai_rs, int64_t ai_cs, int act) {
+                     int64_t ai_rs, int64_t ai_cs, int act, const T *__restrict__ rms_w, float eps) {
     typedef typename Vec8<T>::type vec8;
     constexpr int NA = GATED ? 2 : 1;        // weight fragments per 16 output columns: plain, or gate and value
     constexpr int NF = NA * NR;              // weight fragments per step (NR blocks of 16 output columns)
-    constexpr int U = (MB <= 2 && NF <= 2) ? 4 : 2;  // chunks requested together
+    constexpr int U = (MB <= 2 && NF <= 2 && !RMS) ? 4 : 2;  // chunks requested together
     static_assert(WAVES * NF * MB <= 64, "partial sums fit 64 KB of LDS");
     __shared__ __attribute__((aligned(16))) float red[WAVES][NF * MB][64][4];
+    __shared__ float red_sq[RMS ? WAVES : 1][MB][16];
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
     const int r = lane & 15, g = lane >> 4;
@@ -1024,10 +1029,13 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) acc[f][mb] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
 
+    float sq[MB];  // sum of squares of the x values this lane has seen, per 16-row block (RMS)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) sq[mb] = 0.0f;
     const int nchunks = K / 64;
     const int rot = (int)((blockIdx.x * 13u) % (unsigned)nchunks);
     for (int c0 = wave; c0 < nchunks; c0 += WAVES * U) {
-        vec8 wf[U][NF][2], xf[U][MB][2];
+        vec8 wf[U][NF][2], xf[U][MB][2], gf[RMS ? U : 1][2];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             // chunks past the end repeat the last one; their products are left out below.  Workgroups walk the
@@ -1059,10 +1067,27 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
                 xf[u][mb][0] = *reinterpret_cast<const vec8 *>(xp[mb] + k0);
                 xf[u][mb][1] = *reinterpret_cast<const vec8 *>(xp[mb] + k0 + 8);
             }
+            if constexpr (RMS) {
+                gf[u][0] = *reinterpret_cast<const vec8 *>(rms_w + k0 + 16 * g);
+                gf[u][1] = *reinterpret_cast<const vec8 *>(rms_w + k0 + 16 * g + 8);
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (c0 + WAVES * u < nchunks) {
+                if constexpr (RMS) {
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                const float xv = to_float(xf[u][mb][h][e]);
+                                sq[mb] = fmaf(xv, xv, sq[mb]);
+                            }
+                            xf[u][mb][h] = xf[u][mb][h] * gf[u][h];
+                        }
+                }
 #pragma unroll
                 for (int f = 0; f < NF; ++f)
 #pragma unroll
@@ -1080,6 +1105,16 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
             for (int e = 0; e < 4; ++e) red[wave][f * MB + mb][lane][e] = acc[f][mb][e];
+    if constexpr (RMS) {
+        // a row's squares are spread over the 4 lanes r, r + 16, r + 32, r + 48 of every wave
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            float t = sq[mb];
+            t += __shfl_xor(t, 16, 64);
+            t += __shfl_xor(t, 32, 64);
+            if (g == 0) red_sq[wave][mb][r] = t;
+        }
+    }
     __syncthreads();
 
     // the waves share the NR x MB blocks of 16 columns x 16 rows: element e of a lane is output column nb + 4 g + e
@@ -1088,6 +1123,13 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
         const int rb = unit / MB, mb = unit % MB;
         const int nb = n0 + 16 * rb;
         const int m = 16 * mb + r;
+        float rstd = 1.0f;
+        if constexpr (RMS) {
+            float t = 0.0f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) t += red_sq[w][mb][r];
+            rstd = 1.0f / sqrtf(t / (float)K + eps);
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int n = nb + 4 * g + e;
@@ -1097,7 +1139,7 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
                 float t4[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // fixed summation order: the result does not depend on timing
 #pragma unroll
                 for (int w = 0; w < WAVES; ++w) t4[w & 3] += red[w][(rb * NA + a) * MB + mb][lane][e];
-                v[a] = (t4[0] + t4[1]) + (t4[2] + t4[3]);
+                v[a] = ((t4[0] + t4[1]) + (t4[2] + t4[3])) * rstd;
             }
             if (m >= M || n >= N) continue;
             if (bias != nullptr) {
@@ -1358,15 +1400,17 @@ static int pick_tile(int M, int N, int K, bool gated) {
 
 int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192
 
-template <typename T, bool GATED, int MB, int NR, bool W8>
-static void launch_skinny_blocks(const LinearArgs &a) {
+template <typename T, bool GATED, int MB, int NR, bool W8, bool RMS = false>
+static void launch_skinny_blocks(const LinearArgs &a, const void *rms_w = nullptr, float eps = 0.0f) {
     const int n_out = GATED ? a.N / 2 : a.N;
     const dim3 grid((unsigned)((n_out + 16 * NR - 1) / (16 * NR)));
     const int act = a.act & (kGluBit - 1);
     // waves per workgroup: enough to have a whole block of weight rows in flight when K is long, never more than
     // there are chunks, and no more than the LDS for their partial sums allows
     const int nchunks = a.K / 64;
-    constexpr int kMaxWaves = (GATED ? 2 : 1) * NR * MB > 8 ? 4 : (GATED ? 2 : 1) * NR * MB > 4 ? 8 : 16;
+    // (the normalising form also keeps a few more loads per chunk in flight: half the waves for it)
+    constexpr int kUnits = (GATED ? 2 : 1) * NR * MB * (RMS ? 2 : 1);
+    constexpr int kMaxWaves = kUnits > 8 ? 4 : kUnits > 4 ? 8 : 16;
     // ... and few enough that the workgroups one CU gets (256 CUs) are resident together: a 1024-thread workgroup
     // fills half a CU, and 344 of them would leave a third of the chip idle
     const int per_cu = ((int)grid.x + 255) / 256;
@@ -1374,10 +1418,10 @@ static void launch_skinny_blocks(const LinearArgs &a) {
     if (per_cu >= 3) waves = 4;
     else if (per_cu == 2 && waves > 8) waves = 8;
 #define KERNL_SKINNY(WV)                                                                                                \
-    hipLaunchKernelGGL((linear_skinny_kernel<T, MB, GATED, WV, NR, W8>), grid, dim3(64 * WV), 0, a.st,                      \
+    hipLaunchKernelGGL((linear_skinny_kernel<T, MB, GATED, WV, NR, W8, RMS>), grid, dim3(64 * WV), 0, a.st,                      \
                        static_cast<const T *>(a.x), static_cast<const T *>(a.w), static_cast<const T *>(a.bias),       \
                        static_cast<T *>(a.out), static_cast<T *>(a.act_in), a.M, n_out, a.K, a.x_rs, a.out_rs, a.out_cs, \
-                       a.ai_rs, a.ai_cs, act)
+                       a.ai_rs, a.ai_cs, act, static_cast<const T *>(rms_w), eps)
     if constexpr (kMaxWaves >= 16) {
         if (waves >= 16) { KERNL_SKINNY(16); return; }
     }
@@ -1398,6 +1442,15 @@ static void launch_skinny(const LinearArgs &a) {
     if (mb <= 1) { if (two) launch_skinny_blocks<T, GATED, 1, 2, W8>(a); else launch_skinny_blocks<T, GATED, 1, 1, W8>(a); }
     else if (mb <= 2) { if (two) launch_skinny_blocks<T, GATED, 2, 2, W8>(a); else launch_skinny_blocks<T, GATED, 2, 1, W8>(a); }
     else { if (two) launch_skinny_blocks<T, GATED, 4, 2, W8>(a); else launch_skinny_blocks<T, GATED, 4, 1, W8>(a); }
+}
+
+// RMS-normalised input: 16 output columns per workgroup, 16-bit weights
+template <typename T, bool GATED>
+static void launch_skinny_rms(const LinearArgs &a, const void *rms_w, float eps) {
+    const int mb = (a.M + 15) / 16;
+    if (mb <= 1) launch_skinny_blocks<T, GATED, 1, 1, false, true>(a, rms_w, eps);
+    else if (mb <= 2) launch_skinny_blocks<T, GATED, 2, 1, false, true>(a, rms_w, eps);
+    else launch_skinny_blocks<T, GATED, 4, 1, false, true>(a, rms_w, eps);
 }
 
 template <typename T>
@@ -1550,4 +1603,45 @@ extern "C" int kernl_linear_w8_fwd(const void *x, const void *w8, const void *bi
     a.st = static_cast<hipStream_t>(stream);
     launch_skinny<f16, false, true>(a);
     return check_launch("linear (skinny, fp8 weight)");
+}
+
+extern "C" int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float eps, const void *w, const void *bias,
+                                    void *out, int64_t M, int64_t N, int64_t K, const int64_t x_strides[2],
+                                    const int64_t out_strides[2], int activation, int gated, int dtype, void *stream) {
+    using namespace kernl;
+    if (x == nullptr || rms_weight == nullptr || w == nullptr || out == nullptr || x_strides == nullptr ||
+        out_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "rms linear: x, rms_weight, w, out and their strides must not be NULL");
+    if (M < 0 || N <= 0 || K <= 0)
+        return set_error(KERNL_ERR_INVALID_ARG, "rms linear: bad sizes M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+                         (long long)K);
+    if (activation < KERNL_ACT_NONE || activation > KERNL_ACT_SILU)
+        return set_error(KERNL_ERR_INVALID_ARG, "rms linear: unknown activation %d", activation);
+    if (dtype != KERNL_F16 && dtype != KERNL_BF16)
+        return set_error(KERNL_ERR_UNSUPPORTED, "rms linear: only f16 and bf16 are supported, got dtype %d", dtype);
+    if (gated && N % 32 != 0)
+        return set_error(KERNL_ERR_UNSUPPORTED, "rms linear: gated output width %lld must be a multiple of 32", (long long)N);
+    if (M > 64 || K % 64 != 0 || 2 * N > INT32_MAX || K > INT32_MAX)
+        return set_error(KERNL_ERR_UNSUPPORTED, "rms linear: at most 64 rows of x and K a multiple of 64 (M=%lld K=%lld); "
+                         "normalise and multiply separately for larger inputs", (long long)M, (long long)K);
+    if (x_strides[1] != 1 || x_strides[0] % 8 != 0 || !aligned16(x) || !aligned16(w) || !aligned16(rms_weight))
+        return set_error(KERNL_ERR_UNSUPPORTED, "rms linear: x needs unit feature stride and 16-byte aligned rows, the "
+                         "weights 16-byte aligned bases");
+    if (M == 0) return KERNL_OK;
+    LinearArgs a;
+    a.x = x; a.w = w; a.bias = bias; a.out = out; a.act_in = nullptr;
+    a.M = (int)M; a.N = (int)(gated ? 2 * N : N); a.K = (int)K;
+    a.x_rs = x_strides[0]; a.x_cs = x_strides[1];
+    a.out_rs = out_strides[0]; a.out_cs = out_strides[1];
+    a.ai_rs = 0; a.ai_cs = 0;
+    a.act = activation;
+    a.st = static_cast<hipStream_t>(stream);
+    if (dtype == KERNL_F16) {
+        if (gated) launch_skinny_rms<f16, true>(a, rms_weight, eps);
+        else launch_skinny_rms<f16, false>(a, rms_weight, eps);
+    } else {
+        if (gated) launch_skinny_rms<bf16, true>(a, rms_weight, eps);
+        else launch_skinny_rms<bf16, false>(a, rms_weight, eps);
+    }
+    return check_launch("rms linear (skinny)");
 }

@@ -125,3 +125,39 @@ def linear_glu_layer(x: torch.Tensor, weight_interleaved: torch.Tensor, bias_int
     `interleave_glu_rows`.  Reference: `kernel_ff` (experimental/llama-v2/kernel/fused_kernel_ff.py:82-117), without
     its RMSNorm prologue."""
     return LinearGLU.apply(x, weight_interleaved, bias_interleaved, activation)
+
+
+def rms_linear_layer(
+    x: torch.Tensor,
+    rms_weight: torch.Tensor,
+    eps: float,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    activation: str = "",
+    gated: bool = False,
+) -> torch.Tensor:
+    """activation(linear(rms_norm(x, rms_weight, eps), weight, bias)) — or, with `gated`, the gated linear unit of the
+    normalised input (weight and bias interleaved by `interleave_glu_rows`) — in one launch for decoding steps.
+
+    Reference: `rms_matmul_rbe_wrapper` without the rotary epilogue (experimental/llama-v2/kernel/
+    fused_kernel_proj_qkv.py:186-213) and `kernel_ff` (fused_kernel_ff.py:82-117), whose kernels normalise inside the
+    product.  Inputs the fused kernel does not take (more than 64 rows, K not a multiple of 64) are normalised by the
+    RMSNorm kernel and multiplied by the linear kernels."""
+    from kernl_amd.implementations.layer_norm import layer_norm
+
+    assert x.dtype == weight.dtype == rms_weight.dtype and x.dtype in (torch.float16, torch.bfloat16)
+    assert weight.is_contiguous() and rms_weight.is_contiguous() and rms_weight.shape[0] == x.shape[-1]
+    x_ = x if x.ndim == 2 else x.reshape(-1, x.shape[-1])
+    if x_.stride(-1) != 1 or x_.stride(0) % 8 != 0 or x_.data_ptr() % 16 != 0:
+        x_ = x_.contiguous()
+    n_out = weight.shape[0] // 2 if gated else weight.shape[0]
+    if x.dtype == torch.float16:
+        eps = max(eps, 1.6e-5)  # the fp16 policy of the RMSNorm operator (reference: layer_norm.py:295-296)
+    if _lib.linear_rms_supported(x_) and (not gated or n_out % GLU_BLOCK == 0):
+        out = torch.empty((x_.shape[0], n_out), device=x.device, dtype=x.dtype)
+        _lib.linear_rms_fwd(x_, rms_weight, eps, weight, bias, out, ACTIVATIONS.get(activation, _lib.ACT_NONE), gated)
+        return out if x.ndim == 2 else out.reshape(*x.shape[:-1], n_out)
+    normed = layer_norm(x, rms_weight, None, eps, use_rms_norm=True)
+    if gated:
+        return linear_glu_layer(normed, weight, bias, activation)
+    return linear_layer(normed, weight, bias, activation)

@@ -188,6 +188,13 @@ def fused_linear_wrapper(v: torch.Tensor, weights, biases):
     The concatenated weight is built on the first call (the warm-up call that precedes graph capture) and kept for as
     long as the original parameters live unchanged, so capture and replays neither allocate nor copy.  No counterpart in the
     reference, which launches one Triton GEMM per projection."""
+    weight, bias, sizes = _concatenated_params(v, weights, biases)
+    out = linear_layer(v, weight, bias, activation="")
+    return tuple(torch.split(out, sizes, dim=-1))
+
+
+def _concatenated_params(v: torch.Tensor, weights, biases):
+    """Row-concatenated weight (and bias) of sibling projections, built once per group of parameters."""
     originals = tuple(weights) + tuple(biases)
     cached = _fused_params.get(originals)
     if cached is None:
@@ -205,9 +212,7 @@ def fused_linear_wrapper(v: torch.Tensor, weights, biases):
             ).contiguous()
         cached = (weight, bias, [w.shape[0] for w in weights])
         _fused_params.put(originals, cached)  # keyed after the one-time cast: by the addresses the parameters keep
-    weight, bias, sizes = cached
-    out = linear_layer(v, weight, bias, activation="")
-    return tuple(torch.split(out, sizes, dim=-1))
+    return cached
 
 
 torch.fx.wrap("fused_linear_wrapper")
@@ -258,6 +263,15 @@ def glu_linear_wrapper(v: torch.Tensor, w_gate, b_gate, w_value, b_value, activa
     The block-interleaved weight the kernel takes is built on the first call (before graph capture) and cached like
     the fused sibling projections above.  Shapes or dtypes the gated kernel does not cover run as the two fused
     linears and the multiplication they were in the original graph."""
+    usable, half = _glu_usable(v, w_gate, b_gate, w_value, b_value)
+    if not usable:
+        gate = linear_wrapper_functional(v, w_gate, b_gate, activation=activation)
+        return gate * linear_wrapper_functional(v, w_value, b_value)
+    weight, bias = _interleaved_params(half, w_gate, b_gate, w_value, b_value)
+    return linear_glu_layer(v, weight, bias, activation=activation)
+
+
+def _glu_usable(v: torch.Tensor, w_gate, b_gate, w_value, b_value):
     half = v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")
     dtype = torch.float16 if half else v.dtype
     usable = (
@@ -267,9 +281,11 @@ def glu_linear_wrapper(v: torch.Tensor, w_gate, b_gate, w_value, b_value, activa
         and w_gate.shape[1] % 8 == 0
         and (b_gate is None) == (b_value is None)
     )
-    if not usable:
-        gate = linear_wrapper_functional(v, w_gate, b_gate, activation=activation)
-        return gate * linear_wrapper_functional(v, w_value, b_value)
+    return usable, half
+
+
+def _interleaved_params(half: bool, w_gate, b_gate, w_value, b_value):
+    """Block-interleaved weight (and bias) of a gated linear unit, built once per group of parameters."""
     params = (w_gate, w_value) + (() if b_gate is None else (b_gate, b_value))
     cached = _fused_params.get(params)
     if cached is None:
@@ -280,8 +296,7 @@ def glu_linear_wrapper(v: torch.Tensor, w_gate, b_gate, w_value, b_value, activa
         bias = None if b_gate is None else interleave_glu_rows(b_gate.detach(), b_value.detach())
         cached = (weight, bias)
         _fused_params.put(params, cached)
-    weight, bias = cached
-    return linear_glu_layer(v, weight, bias, activation=activation)
+    return cached
 
 
 torch.fx.wrap("glu_linear_wrapper")
@@ -329,6 +344,119 @@ def fuse_gated_linears(gm: torch.fx.GraphModule):
             gm.graph.erase_node(value_n)
             changed = True
             break
+    if changed:
+        gm.graph.lint()
+        gm.recompile()
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# RMSNorm fused into the projections that consume it (decoding steps)
+# ---------------------------------------------------------------------------------------------------------------------
+def _rms_fusable(x: torch.Tensor, rms_weight: torch.Tensor) -> bool:
+    """The fused kernel takes at most 64 rows of 16-bit x with K a multiple of 64; more rows are normalised once by
+    the RMSNorm kernel instead of once per workgroup."""
+    rows = x.numel() // x.shape[-1] if x.numel() else 0
+    return (
+        x.is_cuda
+        and x.dtype in (torch.float16, torch.bfloat16)
+        and 0 < rows <= 64
+        and x.shape[-1] % 64 == 0
+        and rms_weight.shape == (x.shape[-1],)
+    )
+
+
+def _rms_weight_like(x: torch.Tensor, rms_weight: torch.Tensor) -> torch.Tensor:
+    if rms_weight.dtype == torch.float32 and x.dtype == torch.float16:
+        rms_weight.data = rms_weight.data.half()  # one-time, as for the other parameters
+    return rms_weight if rms_weight.dtype == x.dtype else rms_weight.to(x.dtype)
+
+
+def rms_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, weight, bias, activation=""):
+    """linear_wrapper_functional(layer_norm_rms_wrapper(x, rms_weight, eps), weight, bias, activation) — one launch
+    for decoding steps (reference: `rms_matmul_rbe_wrapper`, experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:186-213)."""
+    from kernl_amd.implementations.linear_layer import rms_linear_layer
+    from kernl_amd.optimizer.layer_norm import layer_norm_rms_wrapper
+
+    if not _rms_fusable(x, rms_weight) or weight.dtype not in (x.dtype, torch.float32):
+        return linear_wrapper_functional(layer_norm_rms_wrapper(x, rms_weight, eps), weight, bias, activation=activation)
+    if weight.dtype == torch.float32:
+        weight.data = weight.data.half()
+    if bias is not None and bias.dtype == torch.float32:
+        bias.data = bias.data.half()
+    if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        return linear_wrapper_functional(layer_norm_rms_wrapper(x, rms_weight, eps), weight, bias, activation=activation)
+    w = weight if weight.is_contiguous() else weight.contiguous()
+    return rms_linear_layer(x, _rms_weight_like(x, rms_weight), eps, w, bias, activation)
+
+
+def rms_fused_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, weights, biases):
+    """fused_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), weights, biases): the query / key / value
+    projections of a decoder layer with the RMSNorm in front of them (reference: `rms_matmul_rbe_qkv_wrapper`,
+    experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:289-344, without its rotary epilogue)."""
+    from kernl_amd.implementations.linear_layer import rms_linear_layer
+    from kernl_amd.optimizer.layer_norm import layer_norm_rms_wrapper
+
+    if not _rms_fusable(x, rms_weight):
+        return fused_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), weights, biases)
+    weight, bias, sizes = _concatenated_params(x, weights, biases)
+    if weight.dtype != x.dtype:
+        return fused_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), weights, biases)
+    out = rms_linear_layer(x, _rms_weight_like(x, rms_weight), eps, weight, bias, "")
+    return tuple(torch.split(out, sizes, dim=-1))
+
+
+def rms_glu_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, w_gate, b_gate, w_value, b_value, activation: str):
+    """glu_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), ...): the feed-forward entry of a SwiGLU decoder
+    with its RMSNorm (reference: `kernel_ff`, experimental/llama-v2/kernel/fused_kernel_ff.py:82-117, whose kernel
+    normalises inside the product, :10-79)."""
+    from kernl_amd.implementations.linear_layer import rms_linear_layer
+    from kernl_amd.optimizer.layer_norm import layer_norm_rms_wrapper
+
+    usable, half = _glu_usable(x, w_gate, b_gate, w_value, b_value)
+    if not usable or not _rms_fusable(x, rms_weight):
+        return glu_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), w_gate, b_gate, w_value, b_value, activation)
+    weight, bias = _interleaved_params(half, w_gate, b_gate, w_value, b_value)
+    if weight.dtype != x.dtype:
+        return glu_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), w_gate, b_gate, w_value, b_value, activation)
+    return rms_linear_layer(x, _rms_weight_like(x, rms_weight), eps, weight, bias, activation, gated=True)
+
+
+torch.fx.wrap("rms_linear_wrapper")
+torch.fx.wrap("rms_fused_linear_wrapper")
+torch.fx.wrap("rms_glu_linear_wrapper")
+
+
+def fuse_rms_norm_into_linears(gm: torch.fx.GraphModule):
+    """An RMSNorm whose only consumers are linear layers taking it as their input is folded into them: every such
+    consumer becomes its `rms_*` form on the un-normalised tensor and the norm node goes away.  Whether the one-launch
+    kernel runs is decided per call from the number of rows (decoding steps: yes; prefill: the RMSNorm kernel once,
+    then the ordinary linear kernels).  Runs after the linear and layer-norm passes."""
+    from kernl_amd.optimizer.layer_norm import layer_norm_rms_wrapper
+
+    fused_form = {
+        linear_wrapper_functional: rms_linear_wrapper,
+        fused_linear_wrapper: rms_fused_linear_wrapper,
+        glu_linear_wrapper: rms_glu_linear_wrapper,
+    }
+    changed = False
+    for node in list(gm.graph.nodes):
+        if node.op != "call_function" or node.target is not layer_norm_rms_wrapper or len(node.args) != 3 or node.kwargs:
+            continue
+        users = list(node.users)
+        if not users or not all(
+            u.op == "call_function" and u.target in fused_form and len(u.args) >= 1 and u.args[0] is node
+            and sum(1 for inp in u.all_input_nodes if inp is node) == 1
+            for u in users
+        ):
+            continue
+        x, rms_weight, eps = node.args
+        for u in users:
+            with gm.graph.inserting_before(u):
+                new = gm.graph.call_function(fused_form[u.target], (x, rms_weight, eps) + tuple(u.args[1:]), dict(u.kwargs))
+            u.replace_all_uses_with(new)
+            gm.graph.erase_node(u)
+        gm.graph.erase_node(node)
+        changed = True
     if changed:
         gm.graph.lint()
         gm.recompile()

@@ -295,13 +295,35 @@ def test_rms_norm_and_swiglu_patterns():
     gm = torch.fx.symbolic_trace(LlamaNorm())
     dynamo_backend_ofi(gm)
     t = _targets(gm)
-    assert t.count("layer_norm_rms_wrapper") == 1 and "rsqrt" not in t and "pow" not in t
-    rms = next(n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "layer_norm_rms_wrapper")
-    assert rms.args[2] == 1e-05
-    # silu(linear) * linear on the same input with graph-input weights: one gated GEMM
-    glu = [n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "glu_linear_wrapper"]
-    assert len(glu) == 1 and glu[0].args[5] == "silu" and "linear_wrapper_functional" not in t and "mul" not in t
-    assert glu[0].args[1].name == "gate_w" and glu[0].args[3].name == "up_w"
+    assert "rsqrt" not in t and "pow" not in t
+    # silu(linear) * linear on the same input with graph-input weights: one gated GEMM — and the RMSNorm, whose only
+    # consumer that GEMM is, folded into it: (x, norm weight, eps, gate weight, gate bias, up weight, up bias, act)
+    assert "layer_norm_rms_wrapper" not in t and "glu_linear_wrapper" not in t
+    glu = [n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "rms_glu_linear_wrapper"]
+    assert len(glu) == 1 and glu[0].args[7] == "silu" and "linear_wrapper_functional" not in t and "mul" not in t
+    assert glu[0].args[0].name == "hidden_states" and glu[0].args[1].target == "weight" and glu[0].args[2] == 1e-05
+    assert glu[0].args[3].name == "gate_w" and glu[0].args[5].name == "up_w"
+
+
+def test_rms_norm_with_another_consumer_is_not_folded():
+    """The norm's output also feeds something that is not a linear layer (here it is returned): it has to exist."""
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.ones(32))
+            self.proj = torch.nn.Linear(32, 16, bias=False)
+
+        def forward(self, hidden_states):
+            h = hidden_states.to(torch.float32)
+            variance = h.pow(2).mean(-1, keepdim=True)
+            h = h * torch.rsqrt(variance + 1e-05)
+            normed = self.weight * h.to(torch.float16)
+            return self.proj(normed), normed
+
+    gm = torch.fx.symbolic_trace(Block())
+    dynamo_backend_ofi(gm)
+    t = _targets(gm)
+    assert t.count("layer_norm_rms_wrapper") == 1 and "rms_linear_wrapper" not in t
 
 
 def test_llama_graph_rewrite_and_constant_causal_mask():
@@ -331,10 +353,12 @@ def test_llama_graph_rewrite_and_constant_causal_mask():
         assert len(graphs) == 1
         t = _targets(graphs[0])
         assert t.count(fused) == 2
-        assert t.count("layer_norm_rms_wrapper") == 2 * 2 + 1 and "rsqrt" not in t
-        assert t.count("fused_linear_wrapper") == 2 and "silu" not in t and "softmax" not in t
+        # the two norms of every layer are folded into the projections they feed; the final norm stays
+        assert t.count("layer_norm_rms_wrapper") == 1 and "rsqrt" not in t
+        assert t.count("rms_fused_linear_wrapper") == 2 and "silu" not in t and "softmax" not in t
         # SwiGLU: gate and up projections and their product are one gated GEMM per layer
-        assert t.count("glu_linear_wrapper") == 2 and t.count("linear_wrapper_functional") == 2 * 2
+        assert t.count("rms_glu_linear_wrapper") == 2 and t.count("linear_wrapper_functional") == 2 * 2
+        assert "fused_linear_wrapper" not in t and "glu_linear_wrapper" not in t
         # rotary embedding: one fused call each for queries and keys per layer, nothing left of rotate_half
         assert t.count("rotary_wrapper") == 2 * 2 and "neg" not in t
         # the fresh key/value cache no longer copies: the only cat left builds the angle table

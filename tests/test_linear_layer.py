@@ -166,6 +166,39 @@ def test_linear_fp8_weight_storage(shape, activation, close):
     close(act_in, pre, what=f"fp8 weight {shape} pre-activation")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("kind", ["plain", "plain_bias_silu", "gated"])
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (5, 96, 64), (16, 1024, 192), (33, 2304, 768), (64, 512, 1024),
+                                   (100, 256, 128), (4, 96, 72)], ids=lambda s: "x".join(map(str, s)))
+def test_rms_norm_fused_into_the_linear_layer(shape, kind, dtype, close):
+    """out = act(rms_norm(x) @ wᵀ + b) in one launch for decoding steps (reference: `rms_matmul_rbe` without the rotary
+    epilogue, experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:116-183; gated: `ff_llama`, fused_kernel_ff.py:10-79),
+    against the composition of the RMSNorm and linear oracles.  100 rows and K = 72 take the two-kernel route."""
+    from kernl_amd.implementations.linear_layer import interleave_glu_rows, rms_linear_layer
+    from oracle import glu_oracle, rms_norm_oracle
+
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(41)
+    x = (torch.randn((M, K), generator=gen) * 3.0 + 0.5).to(dtype)       # rows far from unit RMS
+    g = (1.0 + 0.2 * torch.randn((K,), generator=gen)).to(dtype)
+    eps = 1e-5 if dtype == torch.bfloat16 else 1.6e-5
+    normed = rms_norm_oracle(x, g, eps)
+    if kind == "gated":
+        wg = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+        wv = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+        out = rms_linear_layer(x.cuda(), g.cuda(), eps, interleave_glu_rows(wg, wv).cuda(), None, "silu", gated=True)
+        ref = glu_oracle(normed, wg, None, wv, None, "silu")
+    else:
+        w = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+        b = (0.5 * torch.randn((N,), generator=gen)).to(dtype) if kind == "plain_bias_silu" else None
+        act = "silu" if kind == "plain_bias_silu" else ""
+        out = rms_linear_layer(x.cuda(), g.cuda(), eps, w.cuda(), None if b is None else b.cuda(), act)
+        ref = linear_oracle(normed, w, b, act)
+    torch.cuda.synchronize()
+    assert out.shape == (M, N) and out.dtype == dtype
+    close(out, ref, dtype, what=f"rms + linear {shape} {kind}")
+
+
 def test_linear_few_rows_strided_output_and_batched_input(close):
     gen = torch.Generator().manual_seed(18)
     x, w, b = _inputs(2, 640, 256, torch.float16, gen, w_std=1 / 16, batch=3)  # [3, 2, 256] -> 6 rows

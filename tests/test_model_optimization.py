@@ -141,6 +141,41 @@ def test_llama_shaped_decoder_matches_fp32_eager(attn):
     assert (out.float().cpu() - ref).abs().max().item() <= 1e-1
 
 
+def test_llama_shaped_short_input_runs_the_one_launch_norm_projections(monkeypatch):
+    """24 tokens (at most 64 rows): both RMSNorms of every layer run inside the projections they feed
+    (`kernl_linear_rms_fwd`: fused query/key/value and the gated feed-forward entry), the result still matches the
+    fp32 model."""
+    from kernl_amd import _lib
+    from kernl_amd.model_optimization import optimize_model
+
+    torch._dynamo.reset()
+    calls = {"rms": 0, "gated": 0}
+    real = _lib.linear_rms_fwd
+
+    def counting(x2d, rms_weight, eps, weight, bias, out2d, activation, gated):
+        calls["rms"] += 1
+        calls["gated"] += int(bool(gated))
+        return real(x2d, rms_weight, eps, weight, bias, out2d, activation, gated)
+
+    monkeypatch.setattr(_lib, "linear_rms_fwd", counting)
+    gen = torch.Generator().manual_seed(6)
+    ids = torch.randint(0, 1000, (2, 12), generator=gen)
+    ref_model = _llama(2, 512, 4, 1408, "sdpa", eps=1.6e-5)
+    with torch.inference_mode():
+        ref = ref_model(input_ids=ids, use_cache=False).last_hidden_state
+    model = _llama(2, 512, 4, 1408, "sdpa").half().cuda()
+    optimize_model(model)
+    with torch.inference_mode():
+        out = model(input_ids=ids.cuda(), use_cache=False).last_hidden_state
+        out = model(input_ids=ids.cuda(), use_cache=False).last_hidden_state
+        torch.cuda.synchronize()
+    # warm-up and capture each run the two layers once: 2 x 2 x (one fused q/k/v + one gated feed-forward entry)
+    assert calls["rms"] == 8 and calls["gated"] == 4, calls
+    ours_rel = ((out.float().cpu() - ref).abs().mean() / ref.abs().mean()).item()
+    print(f"llama-shaped, 24 rows: mean_rel ours={ours_rel:.5f}", flush=True)
+    assert torch.isfinite(out).all() and ours_rel <= 5e-3
+
+
 def test_llama_7b_shaped_layer_full_width():
     # one decoder layer at Llama-2-7B width (4096, 32 heads of 128, SwiGLU 11008), batch 1, 2048 tokens, causal.
     # With N(0, 0.02) random weights attention is close to uniform over up to 2048 keys and fp16 itself is several
