@@ -30,9 +30,10 @@ __device__ __forceinline__ float act_sigmoid(float x) {
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-kLog2e * x));
 }
 __device__ __forceinline__ float act_gelu_tanh(float x) {
-    // 0.5 x (1 + tanh(u)) = x * sigmoid(2u),  u = sqrt(2/pi) (x + 0.044715 x^3)
-    const float u2 = x * (1.5957691216057308f + 0.07135481627f * x * x);
-    return x * act_sigmoid(u2);
+    // 0.5 x (1 + tanh(u)) = x * sigmoid(2u) = x / (1 + 2^(-log2(e) 2u)),  u = sqrt(2/pi) (x + 0.044715 x^3);
+    // the factor -log2(e) is folded into the two coefficients of 2u
+    const float t = x * (-1.5957691216057308f * kLog2e + (-0.07135481627f * kLog2e) * x * x);
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
 }
 __device__ __forceinline__ float act_gelu_erf(float x) {
     // 0.5 x (1 + erf(x / sqrt 2)) with erf from Abramowitz & Stegun 7.1.26 (|error| <= 1.5e-7):
@@ -52,12 +53,13 @@ __device__ __forceinline__ float act_gelu_erf(float x) {
 
 // erf-GELU for 16-bit outputs: x * sigmoid(x (a + b s + c s^2)), s = min(x^2, 49) — the form of the tanh variant with
 // one more term, fitted to x Phi(x): |error| <= 2.6e-5 everywhere (a tenth of an fp16 ulp at 1), for two
-// transcendental and six plain instructions instead of two and fourteen.  The clamp keeps the polynomial on its fitted
+// transcendental and five plain instructions instead of two and fourteen.  The clamp keeps the polynomial on its fitted
 // range (it changes sign beyond |x| = 11); at |x| = 7 the sigmoid has long saturated.
 __device__ __forceinline__ float act_gelu_erf_fast(float x) {
     const float s = fminf(x * x, 49.0f);
-    const float p = (-0.0007030433895f * s + 0.07401135561f) * s + 1.595015695f;
-    return x * act_sigmoid(x * p);
+    // the polynomial carries the factor -log2(e) of the base-2 exponential: x * sigmoid(x p) = x / (1 + 2^(x q))
+    const float q = ((0.0007030433895f * kLog2e) * s - 0.07401135561f * kLog2e) * s - 1.595015695f * kLog2e;
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * q));
 }
 
 // activation of the MFMA kernels, whose outputs are fp16 / bf16
