@@ -50,13 +50,25 @@ __device__ __forceinline__ void sk_merge(float &m, float &l, float (&acc)[8], fl
     m = mn;
 }
 
-// 8 features of a key or value row as fp32: from the 16-bit storage type, or from fp8 e5m2 bytes — those are the upper
-// bytes of fp16 values, so decoding is a shift (reference: the int8 caches bit-cast to float8e5 and widened to fp16,
+// 8 features of a key or value row as they lie in memory: 8 bytes of fp8 e5m2 storage, or 16 bytes of the 16-bit type
+template <bool KV8>
+struct SkRaw {
+    typedef typename std::conditional<KV8, uint2, u32x4>::type type;
+};
+
+template <typename T, bool KV8>
+__device__ __forceinline__ typename SkRaw<KV8>::type sk_load_raw(const void *base, int64_t elem_off) {
+    typedef typename SkRaw<KV8>::type raw_t;
+    if constexpr (KV8) return *reinterpret_cast<const raw_t *>(static_cast<const unsigned char *>(base) + elem_off);
+    else return *reinterpret_cast<const raw_t *>(static_cast<const T *>(base) + elem_off);
+}
+
+// ... as fp32: from the 16-bit storage type, or from fp8 e5m2 bytes — those are the upper bytes of fp16 values, so
+// decoding is a shift (reference: the int8 caches bit-cast to float8e5 and widened to fp16,
 // experimental/llama-v2/kernel/fused_kernel_attention.py:69-71,90-92).
 template <typename T, bool KV8>
-__device__ __forceinline__ void sk_load8(const void *base, int64_t elem_off, float (&f)[8]) {
+__device__ __forceinline__ void sk_widen8(const typename SkRaw<KV8>::type &raw, float (&f)[8]) {
     if constexpr (KV8) {
-        const uint2 raw = *reinterpret_cast<const uint2 *>(static_cast<const unsigned char *>(base) + elem_off);
         const uint32_t w[2] = {raw.x, raw.y};
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -65,33 +77,32 @@ __device__ __forceinline__ void sk_load8(const void *base, int64_t elem_off, flo
         }
     } else {
         typedef typename Vec8<T>::type vec8;
-        const vec8 v = *reinterpret_cast<const vec8 *>(static_cast<const T *>(base) + elem_off);
+        const vec8 v = __builtin_bit_cast(vec8, raw);
 #pragma unroll
         for (int e = 0; e < 8; ++e) f[e] = (float)v[e];
     }
 }
 
-// The same 8 features as four packed fp16 pairs (fp16 queries only): fp8 e5m2 bytes become fp16 values by moving
-// each byte into the upper half of a 16-bit lane, one byte-permute per pair; fp16 storage is used as it lies.
+// ... as four packed fp16 pairs (fp16 queries only): fp8 e5m2 bytes become fp16 values by moving each byte into the
+// upper half of a 16-bit lane, one byte-permute per pair; fp16 storage is used as it lies.
 template <bool KV8>
-__device__ __forceinline__ void sk_load8_pairs(const void *base, int64_t elem_off, uint32_t (&pk)[4]) {
+__device__ __forceinline__ void sk_pairs8(const typename SkRaw<KV8>::type &raw, uint32_t (&pk)[4]) {
     if constexpr (KV8) {
-        const uint2 raw = *reinterpret_cast<const uint2 *>(static_cast<const unsigned char *>(base) + elem_off);
         pk[0] = __builtin_amdgcn_perm(0u, raw.x, 0x010c000cu);  // bytes {0, b0, 0, b1}
         pk[1] = __builtin_amdgcn_perm(0u, raw.x, 0x030c020cu);
         pk[2] = __builtin_amdgcn_perm(0u, raw.y, 0x010c000cu);
         pk[3] = __builtin_amdgcn_perm(0u, raw.y, 0x030c020cu);
     } else {
-        const u32x4 raw = *reinterpret_cast<const u32x4 *>(static_cast<const f16 *>(base) + elem_off);
 #pragma unroll
         for (int j = 0; j < 4; ++j) pk[j] = raw[j];
     }
 }
 
-// DL = D / 8 lanes per key (a power of two, 1..64)
-template <typename T, int DL, bool KV8>
+// DL = D / 8 lanes per key (a power of two, 1..64); KPI keys per lane and trip of the loop
+template <typename T, int DL, bool KV8, int KPI>
 __global__ void __launch_bounds__(256) attention_skinny_part1(const SkinnyParams p) {
     typedef typename Vec8<T>::type vec8;
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
     constexpr int KPW = 64 / DL;  // keys per wave and step
     __shared__ float red[4][DL][10];
     const int row = blockIdx.y, split = blockIdx.x;
@@ -120,53 +131,76 @@ __global__ void __launch_bounds__(256) attention_skinny_part1(const SkinnyParams
         for (int j = 0; j < 4; ++j) qpk[j] = qraw[j];
     }
     float mi = -INFINITY, li = 0.0f, acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll 2
-    for (int n0 = c0 + wave * KPW; n0 < c1; n0 += step) {
-        const int n = n0 + kg;
-        const bool valid = n < c1;
-        const int nn = valid ? n : c1 - 1;  // c1 > c0 here, so c1 - 1 is a valid key
-        float vv[8];
-        float s = 0.0f;
-        if constexpr (std::is_same<T, f16>::value) {
-            // fp16: the score from four two-element dot products with fp32 accumulation on the packed pairs, the
-            // values widened where they are used
-            typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-            uint32_t kpk[4], vpk[4];
-            sk_load8_pairs<KV8>(p.k, k_base + (int64_t)nn * p.ks[2], kpk);
-            sk_load8_pairs<KV8>(p.v, v_base + (int64_t)nn * p.vs[2], vpk);
+    // KPI keys per lane and trip: all their loads are issued before the first is used (the cross-lane sums keep the
+    // compiler from unrolling this loop by itself), and they share one move of the softmax reference
+    for (int n0 = c0 + wave * KPW; n0 < c1; n0 += step * KPI) {
+        typename SkRaw<KV8>::type kr[KPI], vr[KPI];
+        bool valid[KPI];
+        int nn[KPI];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                s = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, kpk[j]), __builtin_bit_cast(h2, qpk[j]), s, false);
-            s *= p.scale_log2;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const h2 two = __builtin_bit_cast(h2, vpk[j]);
-                vv[2 * j] = (float)two[0];
-                vv[2 * j + 1] = (float)two[1];
-            }
-        } else {
-            float kv[8];
-            sk_load8<T, KV8>(p.k, k_base + (int64_t)nn * p.ks[2], kv);
-            sk_load8<T, KV8>(p.v, v_base + (int64_t)nn * p.vs[2], vv);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) s += qf[e] * kv[e];
+        for (int u = 0; u < KPI; ++u) {
+            const int n = n0 + u * step + kg;
+            valid[u] = n < c1;
+            nn[u] = valid[u] ? n : c1 - 1;  // c1 > c0 here, so c1 - 1 is a valid key
+            kr[u] = sk_load_raw<T, KV8>(p.k, k_base + (int64_t)nn[u] * p.ks[2]);
+            vr[u] = sk_load_raw<T, KV8>(p.v, v_base + (int64_t)nn[u] * p.vs[2]);
         }
-        // sum over the DL lanes of the key: quad permutes and row mirrors on DPP, no trip through LDS
-        if (DL >= 2) s += dpp_mov<0xB1>(s);
-        if (DL >= 4) s += dpp_mov<0x4E>(s);
-        if (DL >= 8) s += dpp_mov<0x141>(s);
-        if (DL >= 16) s += dpp_mov<0x140>(s);
-        if (DL >= 32) s += __shfl_xor(s, 16, 64);
-        if (p.has_mask) s += sk_mask_value(p.mask, p.mask_dtype, mask_base + (int64_t)nn * p.ms[3], p.clamp);
-        if (!valid) s = -INFINITY;
-        const float mn = fmaxf(mi, s);
+        float s[KPI];
+        float mn = mi;
+#pragma unroll
+        for (int u = 0; u < KPI; ++u) {
+            float su = 0.0f;
+            if constexpr (std::is_same<T, f16>::value) {
+                // fp16: four two-element dot products with fp32 accumulation on the packed pairs
+                uint32_t kpk[4];
+                sk_pairs8<KV8>(kr[u], kpk);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    su = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, kpk[j]), __builtin_bit_cast(h2, qpk[j]), su, false);
+                su *= p.scale_log2;
+            } else {
+                float kv[8];
+                sk_widen8<T, KV8>(kr[u], kv);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) su += qf[e] * kv[e];
+            }
+            // sum over the DL lanes of the key: quad permutes and row mirrors on DPP, no trip through LDS
+            if (DL >= 2) su += dpp_mov<0xB1>(su);
+            if (DL >= 4) su += dpp_mov<0x4E>(su);
+            if (DL >= 8) su += dpp_mov<0x141>(su);
+            if (DL >= 16) su += dpp_mov<0x140>(su);
+            if (DL >= 32) su += __shfl_xor(su, 16, 64);
+            if (p.has_mask) su += sk_mask_value(p.mask, p.mask_dtype, mask_base + (int64_t)nn[u] * p.ms[3], p.clamp);
+            if (!valid[u]) su = -INFINITY;
+            s[u] = su;
+            mn = fmaxf(mn, su);
+        }
         const float mu = (mn == -INFINITY) ? 0.0f : mn;
         const float alpha = __builtin_amdgcn_exp2f(mi - mu);
-        // P is rounded to the storage dtype before P·V, as in the tiled kernel and the reference (attention.py:424)
-        const float pr = (float)from_float<T>(__builtin_amdgcn_exp2f(s - mu));
-        li = li * alpha + pr;
+        li *= alpha;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] = acc[e] * alpha + pr * vv[e];
+        for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+#pragma unroll
+        for (int u = 0; u < KPI; ++u) {
+            // P is rounded to the storage dtype before P·V, as in the tiled kernel and the reference (attention.py:424)
+            const float pr = (float)from_float<T>(__builtin_amdgcn_exp2f(s[u] - mu));
+            li += pr;
+            float vv[8];
+            if constexpr (std::is_same<T, f16>::value) {
+                uint32_t vpk[4];
+                sk_pairs8<KV8>(vr[u], vpk);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const h2 two = __builtin_bit_cast(h2, vpk[j]);
+                    vv[2 * j] = (float)two[0];
+                    vv[2 * j + 1] = (float)two[1];
+                }
+            } else {
+                sk_widen8<T, KV8>(vr[u], vv);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += pr * vv[e];
+        }
         mi = mn;
     }
     // merge the KPW lane groups of the wave (same dl, different kg)
@@ -256,8 +290,10 @@ __global__ void __launch_bounds__(256) attention_skinny_part2(const SkinnyParams
     }
 }
 
-// key ranges per row: about `workgroups` workgroups over the whole grid (1024 = 4 per CU is where 16-bit keys and
-// values reach their bandwidth; one-byte storage has half the bytes per key in flight and wants all 8 per CU)
+// key ranges per row: about `workgroups` workgroups over the whole grid.  With 64 bytes of keys and of values in flight
+// per lane, one workgroup per CU reaches the bandwidth for 16-bit storage and two for one-byte storage; more ranges
+// only add to the merge.
+constexpr int kSkWorkgroups16 = 256, kSkWorkgroups8 = 512;
 static int skinny_splits(int64_t rows, int64_t N, int D, int workgroups) {
     const int step = 4 * (64 / (D / 8));
     int64_t want = (workgroups + rows - 1) / rows;
@@ -267,17 +303,23 @@ static int skinny_splits(int64_t rows, int64_t N, int D, int workgroups) {
     return (int)(want < 1 ? 1 : want);
 }
 
-template <typename T, bool KV8>
-static void launch_skinny(const SkinnyParams &p, hipStream_t st) {
+template <typename T, bool KV8, int KPI>
+static void launch_skinny_part1(const SkinnyParams &p, hipStream_t st) {
     dim3 grid((unsigned)p.splits, (unsigned)(p.B * p.H * p.M));
     switch (p.D / 8) {
-        case 1: hipLaunchKernelGGL((attention_skinny_part1<T, 1, KV8>), grid, dim3(256), 0, st, p); break;
-        case 2: hipLaunchKernelGGL((attention_skinny_part1<T, 2, KV8>), grid, dim3(256), 0, st, p); break;
-        case 4: hipLaunchKernelGGL((attention_skinny_part1<T, 4, KV8>), grid, dim3(256), 0, st, p); break;
-        case 8: hipLaunchKernelGGL((attention_skinny_part1<T, 8, KV8>), grid, dim3(256), 0, st, p); break;
-        case 16: hipLaunchKernelGGL((attention_skinny_part1<T, 16, KV8>), grid, dim3(256), 0, st, p); break;
-        default: hipLaunchKernelGGL((attention_skinny_part1<T, 32, KV8>), grid, dim3(256), 0, st, p); break;
+        case 1: hipLaunchKernelGGL((attention_skinny_part1<T, 1, KV8, KPI>), grid, dim3(256), 0, st, p); break;
+        case 2: hipLaunchKernelGGL((attention_skinny_part1<T, 2, KV8, KPI>), grid, dim3(256), 0, st, p); break;
+        case 4: hipLaunchKernelGGL((attention_skinny_part1<T, 4, KV8, KPI>), grid, dim3(256), 0, st, p); break;
+        case 8: hipLaunchKernelGGL((attention_skinny_part1<T, 8, KV8, KPI>), grid, dim3(256), 0, st, p); break;
+        case 16: hipLaunchKernelGGL((attention_skinny_part1<T, 16, KV8, KPI>), grid, dim3(256), 0, st, p); break;
+        default: hipLaunchKernelGGL((attention_skinny_part1<T, 32, KV8, KPI>), grid, dim3(256), 0, st, p); break;
     }
+}
+
+template <typename T, bool KV8>
+static void launch_skinny(const SkinnyParams &p, hipStream_t st) {
+    // keys per lane and trip: 64 bytes of keys and as many of values in flight per lane with either storage
+    launch_skinny_part1<T, KV8, KV8 ? 8 : 4>(p, st);
     if (p.splits > 1)
         hipLaunchKernelGGL((attention_skinny_part2<T>), dim3((unsigned)(p.B * p.H * p.M)), dim3(256), 0, st, p);
 }
@@ -288,7 +330,7 @@ extern "C" int64_t kernl_attention_skinny_workspace_bytes(int64_t B, int64_t H, 
     using namespace kernl;
     if (B <= 0 || H <= 0 || M <= 0 || N <= 0 || D < 8 || D % 8 != 0) return 0;
     const int64_t rows = B * H * M;
-    const int splits = skinny_splits(rows, N, (int)D, 2048);  // enough for either storage of the keys and values
+    const int splits = skinny_splits(rows, N, (int)D, kSkWorkgroups8);  // enough for either storage of the keys and values
     return splits > 1 ? rows * splits * (D + 2) * (int64_t)sizeof(float) : 0;
 }
 
@@ -344,7 +386,7 @@ static int skinny_entry(const void *q, const void *k, const void *v, void *out, 
 
     const int64_t rows = B * H * M;
     if (rows > 65535) return set_error(KERNL_ERR_UNSUPPORTED, "skinny attention: more than 65535 (batch, head, query) rows");
-    int splits = skinny_splits(rows, N, (int)D, kv8 ? 2048 : 1024);
+    int splits = skinny_splits(rows, N, (int)D, kv8 ? kSkWorkgroups8 : kSkWorkgroups16);
     if (splits > 1) {
         const int64_t per_split = rows * (D + 2) * (int64_t)sizeof(float);
         const int64_t fit = workspace != nullptr ? workspace_bytes / per_split : 0;
