@@ -163,6 +163,17 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// sums over the lower and over the upper 32 lanes of the wave, both to every lane
+__device__ __forceinline__ void half_wave_sums(float v, float &lo, float &hi) {
+    v = row16_sum(v);
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    lo = r0 + r1;
+    hi = r2 + r3;
+}
+
 // Both 32-lane halves of the wave exchange a value: afterwards every lane has the value its counterpart in the
 // lower half held (`lo`) and the one its counterpart in the upper half held (`hi`).
 // v_permlane32_swap exchanges the upper 32 lanes of its first operand with the lower 32 lanes of its second; fed

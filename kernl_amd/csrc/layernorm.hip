@@ -19,26 +19,34 @@ struct Row16 {  // one 16-byte chunk of a row
 // A group of GROUP_WAVES waves (1 or the 4 of the block) per row; thread t of the group owns chunks t, t + G, ...
 // (G = 64 GROUP_WAVES, CHUNKS of them at most).  A group walks rows with a fixed stride and fetches the next row
 // before it reduces the current one, so that loads of one row overlap the arithmetic and the stores of another.
-template <typename T, int CHUNKS, bool RMS, bool HAS_RES, int GROUP_WAVES>
+// HALF (single-wave groups only): a group is half a wave, so that a wave works on two rows at once — rows of 32·k
+// chunks with odd k (768 fp16 values are 96 chunks) then keep every lane busy.
+template <typename T, int CHUNKS, bool RMS, bool HAS_RES, int GROUP_WAVES, bool HALF = false>
 __global__ void __launch_bounds__(256)
 layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const T *__restrict__ w,
                       const T *__restrict__ b, T *__restrict__ out, float *__restrict__ mean_out,
                       float *__restrict__ rstd_out, int M, int N, int64_t x_rs, int64_t res_rs,
                       int64_t out_rs, float eps, int stream_out) {
     constexpr int E = Row16<T>::kElems;
-    constexpr int G = 64 * GROUP_WAVES;
+    static_assert(!HALF || GROUP_WAVES == 1, "half-wave groups are single-wave groups split in two");
+    constexpr int G = HALF ? 32 : 64 * GROUP_WAVES;
     typedef Row16<T> chunk_t;
     __shared__ float red[2][4];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int t = GROUP_WAVES == 1 ? lane : (int)threadIdx.x;  // index inside the group
-    const int groups_per_block = 4 / GROUP_WAVES;
-    const int group = GROUP_WAVES == 1 ? wave : 0;
+    const int t = HALF ? (lane & 31) : GROUP_WAVES == 1 ? lane : (int)threadIdx.x;  // index inside the group
+    const int groups_per_block = HALF ? 8 : 4 / GROUP_WAVES;
+    const int group = HALF ? 2 * wave + (lane >> 5) : GROUP_WAVES == 1 ? wave : 0;
     const int nchunks = N / E;
     const float inv_n = 1.0f / (float)N;
 
     // sum over the group: wave reduction, then (4-wave groups) a round trip through LDS
     auto group_sum = [&](float v, int slot) -> float {
+        if (HALF) {
+            float lo, hi;
+            half_wave_sums(v, lo, hi);
+            return lane < 32 ? lo : hi;
+        }
         v = wave_sum(v);
         if (GROUP_WAVES == 1) return v;
         __syncthreads();  // the previous use of this slot has been read by everyone
@@ -79,7 +87,10 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
     };
     if (row < M) fetch(row);
 
-    for (; row < M; row += row_step) {
+    // with half-wave groups the wave stays together while its lower half has a row; the upper half's last row may
+    // lie beyond M, then it computes on zeros and stores nothing
+    for (int lead = row - (HALF ? lane >> 5 : 0); lead < M; lead += row_step, row += row_step) {
+        const bool live = !HALF || row < M;
         float v[CHUNKS][E];
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
@@ -87,7 +98,7 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 float a = 0.0f;
-                if (ci < nchunks) {
+                if (ci < nchunks && live) {
                     a = to_float(xn[c].v[e]);
                     if (HAS_RES) a += to_float(rn[c].v[e]);
                 }
@@ -126,7 +137,7 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
             var = group_sum(ss, 1) * inv_n;
         }
         const float rstd = 1.0f / sqrtf(var + eps);
-        if (t == 0) {
+        if (t == 0 && live) {
             if (mean_out != nullptr) mean_out[row] = mean;
             if (rstd_out != nullptr) rstd_out[row] = rstd;
         }
@@ -135,7 +146,7 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
             const int ci = t + c * G;
-            if (ci < nchunks) {
+            if (ci < nchunks && live) {
                 chunk_t o;
 #pragma unroll
                 for (int e = 0; e < E; ++e) {
@@ -206,12 +217,12 @@ layernorm_strided_kernel(const T *__restrict__ x, const T *__restrict__ res, con
     }
 }
 
-template <typename T, int CHUNKS, int GROUP_WAVES>
+template <typename T, int CHUNKS, int GROUP_WAVES, bool HALF = false>
 static void launch_rows(bool rms, bool has_res, dim3 grid, hipStream_t st, const T *x, const T *res,
                         const T *w, const T *b, T *out, float *mean, float *rstd, int M, int N, int64_t x_rs,
                         int64_t res_rs, int64_t out_rs, float eps) {
 #define KERNL_LN_LAUNCH(R, H)                                                                                       \
-    hipLaunchKernelGGL((layernorm_rows_kernel<T, CHUNKS, R, H, GROUP_WAVES>), grid, dim3(256), 0, st, x, res, w, b, \
+    hipLaunchKernelGGL((layernorm_rows_kernel<T, CHUNKS, R, H, GROUP_WAVES, HALF>), grid, dim3(256), 0, st, x, res, w, b, \
                        out, mean, rstd, M, N, x_rs, res_rs, out_rs, eps, stream_out)
     const int stream_out = (int64_t)M * N * (int64_t)sizeof(T) > (128ll << 20);
     if (rms) {
@@ -244,15 +255,27 @@ static int layernorm_dispatch(const void *x_, const void *res_, const void *w_, 
     if (vec_ok) {
         // Rows of up to 1024 chunks stay in registers.  Long rows on few-row inputs are spread over the 4 waves of a
         // block (more loads in flight per row); otherwise a wave per row, 4 rows per block.  The grid is capped at
-        // 8 waves per SIMD so that every group walks several rows and gamma/beta loads amortise.
+        // 8 waves per SIMD (4 where a wave takes two rows) so that every group walks several rows and gamma/beta loads
+        // amortise.
         const bool block_per_row = row_chunks > 128 && M < 16384;
-        const int64_t blocks_needed = block_per_row ? M : (M + 3) / 4;
-        const int grid = (int)(blocks_needed < 2048 ? blocks_needed : 2048);
+        // Two rows per wave, 32 lanes each, where that leaves fewer lanes idle than a wave per row (rows of up to 32
+        // or of 65..96 chunks).
+        const bool half_wave = !block_per_row && (row_chunks <= 32 || (row_chunks > 64 && row_chunks <= 96));
+        const int64_t grid_cap = half_wave ? 1024 : 2048;
+        const int64_t blocks_needed = block_per_row ? M : half_wave ? (M + 7) / 8 : (M + 3) / 4;
+        const int grid = (int)(blocks_needed < grid_cap ? blocks_needed : grid_cap);
         const int chunks = (int)((row_chunks + (block_per_row ? 255 : 63)) / (block_per_row ? 256 : 64));
 #define KERNL_LN_CASE(C, GW)                                                                                   \
     launch_rows<T, C, GW>(rms, has_res, dim3(grid), st, x, res, w, b, out, mean, rstd, (int)M, (int)N, x_rs, \
                           res_rs, out_rs, eps)
-        if (block_per_row) {
+        if (half_wave) {
+            if (row_chunks <= 32)
+                launch_rows<T, 1, 1, true>(rms, has_res, dim3(grid), st, x, res, w, b, out, mean, rstd, (int)M, (int)N,
+                                           x_rs, res_rs, out_rs, eps);
+            else
+                launch_rows<T, 3, 1, true>(rms, has_res, dim3(grid), st, x, res, w, b, out, mean, rstd, (int)M, (int)N,
+                                           x_rs, res_rs, out_rs, eps);
+        } else if (block_per_row) {
             if (chunks <= 1) KERNL_LN_CASE(1, 4);
             else if (chunks <= 2) KERNL_LN_CASE(2, 4);
             else KERNL_LN_CASE(4, 4);

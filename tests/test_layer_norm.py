@@ -84,6 +84,41 @@ def test_layer_norm_config2_full_size(close):
     assert (y2 - y).abs().max().item() < 1e-2
 
 
+@pytest.mark.parametrize("dtype,n", [(torch.float16, 768), (torch.bfloat16, 256), (torch.float32, 384),
+                                     (torch.float16, 136), (torch.float32, 128), (torch.float16, 520)],
+                         ids=["fp16-768", "bf16-256", "fp32-384", "fp16-136", "fp32-128", "fp16-520"])
+def test_rows_that_share_a_wave(dtype, n, close):
+    # rows of up to 32 or of 65..96 sixteen-byte chunks are taken two to a wave: odd row counts leave the last wave
+    # with one row, and more rows than the grid holds make every wave walk several pairs
+    from kernl_amd import _lib
+
+    gen = torch.Generator().manual_seed(7)
+    for rows in (1, 2, 7, 8, 9, 8201):
+        x = (3 + 2 * torch.randn((rows, n), generator=gen)).to(dtype)
+        r = torch.randn((rows, n), generator=gen).to(dtype)
+        w = (1 + 0.1 * torch.randn((n,), generator=gen)).to(dtype)
+        b = (0.1 * torch.randn((n,), generator=gen)).to(dtype)
+        eps = effective_eps(1e-5, dtype)
+        tol = torch.float16 if dtype == torch.float32 else dtype
+        print(f"case rows={rows} n={n} {dtype}", flush=True)
+        out = layer_norm(x.cuda(), w.cuda(), b.cuda(), 1e-5)
+        close(out, layer_norm_oracle(x, w, b, eps), tol, scale=4.0, what=f"layernorm {rows}x{n}")
+        out = layer_norm(x.cuda(), w.cuda(), None, 1e-5, use_rms_norm=True)
+        close(out, rms_norm_oracle(x, w, eps), tol, scale=4.0, what=f"rmsnorm {rows}x{n}")
+        out = add_layer_norm(x.cuda(), r.cuda(), w.cuda(), b.cuda(), 1e-5)
+        close(out, layer_norm_oracle(x.float() + r.float(), w, b, eps), tol, scale=4.0, what=f"add+layernorm {rows}x{n}")
+        # the saved statistics of every row, those of a lone last row included
+        xg, o = x.cuda(), torch.empty((rows, n), dtype=dtype, device="cuda")
+        mean = torch.full((rows,), float("nan"), device="cuda")
+        rstd = torch.full((rows,), float("nan"), device="cuda")
+        _lib.layernorm_fwd(xg, w.cuda(), b.cuda(), o, mean, rstd, eps, False, None)
+        torch.cuda.synchronize()
+        xd = x.double()
+        assert (mean.cpu().double() - xd.mean(dim=-1)).abs().max().item() < 1e-4
+        want = (xd.var(dim=-1, unbiased=False) + eps).rsqrt()
+        assert ((rstd.cpu().double() - want).abs() / want).max().item() < 1e-4
+
+
 def test_add_layer_norm_matches_separate_add(close):
     gen = torch.Generator().manual_seed(4)
     for shape in [(512, 768), (4, 40, 768), (30, 1000)]:
