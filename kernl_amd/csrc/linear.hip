@@ -1438,9 +1438,33 @@ template <typename T, bool GATED, bool W8 = false>
 static void launch_skinny(const LinearArgs &a) {
     const int n_out = GATED ? a.N / 2 : a.N;
     const int mb = (a.M + 15) / 16;
-    // every workgroup reads all of x (from L2): with more than 16 rows of x and enough output columns to fill the
-    // chip twice over, a workgroup takes 32 columns and that traffic halves
+    // every workgroup reads all of x (from L2), so more output columns per workgroup mean less of that traffic.
+    // Gated and one-byte weights: with more than 16 rows of x and enough output columns to fill the chip twice over,
+    // a workgroup takes 32 columns
     const bool two = n_out >= 8192 && mb >= 2;
+    if constexpr (!W8 && !GATED) {
+        // 16-bit plain weights, 8 rows of x or more (measured at 8..64 rows, 4096..32000 columns): as few 16-column
+        // blocks per workgroup as put the whole grid on the chip at once, one workgroup per CU — 11008 columns in
+        // blocks of 48 are 230 workgroups, where blocks of 32 leave 88 CUs with two workgroups and the rest with one;
+        // grids that do not fit either way take 32 columns, 64 with more than 48 rows
+        int nr = 1;
+        if (a.M >= 8) {
+            nr = (n_out + 16 * 256 - 1) / (16 * 256);
+            if (nr > 4) nr = mb >= 4 ? 4 : 2;
+        }
+#define KERNL_SKINNY_NR(NRV)                                            \
+    do {                                                                \
+        if (mb <= 1) launch_skinny_blocks<T, GATED, 1, NRV, W8>(a);      \
+        else if (mb <= 2) launch_skinny_blocks<T, GATED, 2, NRV, W8>(a); \
+        else launch_skinny_blocks<T, GATED, 4, NRV, W8>(a);              \
+    } while (0)
+        if (nr == 1) KERNL_SKINNY_NR(1);
+        else if (nr == 2) KERNL_SKINNY_NR(2);
+        else if (nr == 3) KERNL_SKINNY_NR(3);
+        else KERNL_SKINNY_NR(4);
+#undef KERNL_SKINNY_NR
+        return;
+    }
     if (mb <= 1) { if (two) launch_skinny_blocks<T, GATED, 1, 2, W8>(a); else launch_skinny_blocks<T, GATED, 1, 1, W8>(a); }
     else if (mb <= 2) { if (two) launch_skinny_blocks<T, GATED, 2, 2, W8>(a); else launch_skinny_blocks<T, GATED, 2, 1, W8>(a); }
     else { if (two) launch_skinny_blocks<T, GATED, 4, 2, W8>(a); else launch_skinny_blocks<T, GATED, 4, 1, W8>(a); }
