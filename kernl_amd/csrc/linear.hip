@@ -1040,8 +1040,12 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
         vec8 wf[U][NF][2], xf[U][MB][2], gf[RMS ? U : 1][2];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            // chunks past the end repeat the last one; their products are left out below.  Workgroups walk the
-            // chunks from different starting points, so that they do not all ask L2 for the same lines of x at once.
+            // chunks past the end are neither fetched nor multiplied (the test is uniform over the wave); only the
+            // 16-wave form with 128 fragment registers in flight, which has none to spare for the branches, fetches
+            // the last chunk again instead.  Workgroups walk the chunks from different starting points, so that they
+            // do not all ask L2 for the same lines of x at once.
+            constexpr bool kSkipTail = !(WAVES == 16 && U * (NF + MB) >= 16);
+            if (kSkipTail && c0 + WAVES * u >= nchunks) continue;
             int cc = min(c0 + WAVES * u, nchunks - 1) + rot;
             cc = cc >= nchunks ? cc - nchunks : cc;
             const int k0 = cc * 64;
