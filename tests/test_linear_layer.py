@@ -119,13 +119,14 @@ def test_linear_wide_tiles_save_activation_inputs(tile, close):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
 @pytest.mark.parametrize("activation", ["", "gelu", "silu"])
 @pytest.mark.parametrize("shape", [(1, 4096, 512), (5, 80, 64), (16, 1000, 192), (17, 768, 3072), (33, 2304, 768),
-                                   (64, 4096, 1024), (3, 24, 4096), (5, 8200, 128), (33, 9000, 192), (64, 8192, 128)],
+                                   (64, 4096, 1024), (3, 24, 4096), (5, 8200, 128), (33, 9000, 192), (64, 8192, 128),
+                                   (9, 12300, 64), (20, 16400, 64), (64, 16400, 128), (40, 11008, 320)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_linear_few_rows_streams_the_weight(shape, activation, dtype, close):
     """At most 64 rows of x (decoding steps): the kernel that streams the weight once, 16 output columns per workgroup.
     Shapes cover one to four 16-row blocks of x, output widths that are not a multiple of 16, chunk counts that do
-    not divide by the waves of a workgroup, outputs wide enough for 32 columns per workgroup, and the saved
-    pre-activation."""
+    not divide by the waves of a workgroup, outputs wide enough for 32, 48 and 64 columns per workgroup (with widths
+    that leave the last workgroup partly empty), and the saved pre-activation."""
     M, N, K = shape
     gen = torch.Generator().manual_seed(17)
     x, w, b = _inputs(M, N, K, dtype, gen, w_std=K ** -0.5)
