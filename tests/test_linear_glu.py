@@ -148,11 +148,13 @@ def test_glu_more_tiles_than_compute_units(close):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
 @pytest.mark.parametrize("bias", [False, True], ids=["nobias", "bias"])
 @pytest.mark.parametrize("shape", [(1, 11008, 4096), (7, 96, 64), (16, 160, 320), (40, 1024, 192), (64, 352, 4096),
-                                   (33, 8224, 256), (64, 8192, 64)],
+                                   (33, 8224, 256), (64, 8192, 64), (16, 11008, 128), (32, 8992, 192), (24, 13824, 64),
+                                   (9, 12320, 64)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_glu_few_rows_streams_the_weight(shape, bias, dtype, close):
     """M <= 64 (reference experimental/llama-v2/test/test_ff.py runs M = 1..128): every workgroup takes 16 gate rows
-    and their 16 value rows of the interleaved weight, the four waves split K."""
+    and their 16 value rows of the interleaved weight (48 or 64 of each where 8..32 rows of x meet more than 8192
+    output columns), the waves split K."""
     M, N, K = shape
     x, wg, bg, wv, bv = _case(M, N, K, dtype, bias, seed=5)
     out = _run(x, wg, bg, wv, bv, "silu")
