@@ -128,6 +128,31 @@ int kernl_attention_skinny_kv8_fwd(const void *q, const void *k, const void *v, 
                                    float mask_min_clamp, int dtype, void *stream);
 
 /*
+ * kernl_attention_skinny_fwd for callers that cannot allocate device memory (code under hipGraph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose operator allocates its
+ * partial maxima / sums / products with torch on every call (src/kernl/implementations/attention_skinny.py:416-441).
+ * The partial results of the key ranges live in a device array of kernl_attention_skinny_static_max_bytes() bytes
+ * (512 KiB) that is part of the library image: every GPU the library runs on holds it until the process ends.  The call
+ * itself performs no hipMalloc / hipFree; the first call on a device looks the array's address up once.
+ *
+ *   - 16-bit keys and values only; arguments as kernl_attention_skinny_fwd without the workspace pair.
+ *   - Problems with kernl_attention_skinny_workspace_bytes(B,H,M,N,D) above the array's size (the largest workspace
+ *     any problem asks for is about 1 MiB: 256..511 rows of head size 256) are refused with KERNL_ERR_UNSUPPORTED
+ *     (nothing is launched); results are bit-identical to kernl_attention_skinny_fwd given a
+ *     workspace of the reported size.
+ *   - Nothing in the array has to start at zero: every slot the merge kernel reads was written by the same call.
+ *   - All calls on one GPU share the array: calls that may overlap in time on one GPU (different streams, different
+ *     threads) race.  Calls on one stream are ordered and safe.
+ */
+int64_t kernl_attention_skinny_static_max_bytes(void);
+int kernl_attention_skinny_static_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
+                                      int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
+                                      const int64_t q_strides[4], const int64_t k_strides[4],
+                                      const int64_t v_strides[4], const int64_t o_strides[4],
+                                      const int64_t mask_sizes[4], const int64_t mask_strides[4], int mask_dtype,
+                                      float sm_scale, int is_causal, float mask_min_clamp, int dtype, void *stream);
+
+/*
  * Rotary position embedding, half-split convention:  out = x·cos + rotate_half(x)·sin, with
  * rotate_half(x)[d] = -x[d + D/2] (d < D/2), x[d - D/2] (d >= D/2); fp32 arithmetic, one rounding.
  * The reference applies the same rotation (in Meta's interleaved-pair convention) inside its fused query/key

@@ -26,6 +26,8 @@ EXPORTED_SYMBOLS = (
     "kernl_attention_skinny_workspace_bytes",
     "kernl_attention_skinny_fwd",
     "kernl_attention_skinny_kv8_fwd",
+    "kernl_attention_skinny_static_max_bytes",
+    "kernl_attention_skinny_static_fwd",
     "kernl_rope_fwd",
     "kernl_linear_fwd",
     "kernl_linear_w8_fwd",
@@ -82,6 +84,12 @@ def load() -> ctypes.CDLL:
     lib.kernl_attention_skinny_kv8_fwd.restype = ctypes.c_int
     lib.kernl_attention_skinny_kv8_fwd.argtypes = (
         [_vp] * 6 + [_i64] * 6 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, _vp]
+    )
+    lib.kernl_attention_skinny_static_max_bytes.restype = _i64
+    lib.kernl_attention_skinny_static_max_bytes.argtypes = []
+    lib.kernl_attention_skinny_static_fwd.restype = ctypes.c_int
+    lib.kernl_attention_skinny_static_fwd.argtypes = (
+        [_vp] * 5 + [_i64] * 5 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, _vp]
     )
     lib.kernl_rope_fwd.restype = ctypes.c_int
     lib.kernl_rope_fwd.argtypes = [_vp] * 4 + [_i64] * 4 + [_i64p] * 5 + [ctypes.c_int, ctypes.c_int, _vp]
@@ -196,6 +204,27 @@ def attention_skinny_fwd(q, k, v, out, mask, workspace, sm_scale: float, is_caus
             float(sm_scale), int(bool(is_causal)), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
         )
     _check(st, "kernl_attention_skinny_fwd")
+
+
+def attention_skinny_static_fwd(q, k, v, out, mask, sm_scale: float, is_causal: bool, mask_min_clamp: float) -> None:
+    """`attention_skinny_fwd` on the library's own static partial-result buffer: no workspace, no allocation."""
+    _require_gpu(q, k, v, out, mask)
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    lib = load()
+    if mask is not None:
+        msizes, mstrides, mdtype, mptr = _arr(mask.shape), _arr(mask.stride()), DTYPE_CODE[mask.dtype], mask.data_ptr()
+    else:
+        msizes, mstrides, mdtype, mptr = None, None, KERNL_F32, None
+    with torch.cuda.device(q.device):
+        st = lib.kernl_attention_skinny_static_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), mptr,
+            B, H, M, N, D,
+            _arr(q.stride()), _arr(k.stride()), _arr(v.stride()), _arr(out.stride()),
+            msizes, mstrides, mdtype,
+            float(sm_scale), int(bool(is_causal)), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
+        )
+    _check(st, "kernl_attention_skinny_static_fwd")
 
 
 def rope_fwd(x, cos, sin, out) -> None:

@@ -414,6 +414,73 @@ static int skinny_entry(const void *q, const void *k, const void *v, void *out, 
     return check_launch("attention (skinny)");
 }
 
+// ----------------------------------------------------------------------------------------------------
+// Entry point that allocates nothing: the partial results live in a file-scope device array instead of a
+// caller-provided workspace.  Every GPU holds its own copy of the array at its own address; the address is
+// looked up once per device (with that device current) and kept.
+// ----------------------------------------------------------------------------------------------------
+namespace kernl {
+
+static constexpr int64_t kSkScratchBytes = 512ll << 10;
+static constexpr int kSkMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kSkScratchBytes];
+
+// per-device address of `scratch`; written once per device under the lock, read through an acquire load
+static void *g_scratch_ptr[kSkMaxDevices] = {nullptr};
+static int g_scratch_lock = 0;
+
+static int skinny_scratch(void **ptr_out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return set_error(KERNL_ERR_LAUNCH, "skinny attention (static): hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kSkMaxDevices)
+        return set_error(KERNL_ERR_UNSUPPORTED, "skinny attention (static): device index %d outside 0..%d", dev, kSkMaxDevices - 1);
+    void *ptr = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (ptr == nullptr) {
+        while (__atomic_exchange_n(&g_scratch_lock, 1, __ATOMIC_ACQUIRE) != 0) {
+        }
+        ptr = g_scratch_ptr[dev];
+        if (ptr == nullptr) {
+            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e == hipSuccess && ptr != nullptr) __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
+        }
+        __atomic_store_n(&g_scratch_lock, 0, __ATOMIC_RELEASE);
+        if (e != hipSuccess || ptr == nullptr)
+            return set_error(KERNL_ERR_LAUNCH, "skinny attention (static): hipGetSymbolAddress: %s", hipGetErrorString(e));
+    }
+    *ptr_out = ptr;
+    return KERNL_OK;
+}
+
+}  // namespace kernl
+
+extern "C" int64_t kernl_attention_skinny_static_max_bytes(void) { return kernl::kSkScratchBytes; }
+
+extern "C" int kernl_attention_skinny_static_fwd(const void *q, const void *k, const void *v, void *out,
+                                                 const void *mask, int64_t B, int64_t H, int64_t M, int64_t N,
+                                                 int64_t D, const int64_t q_strides[4], const int64_t k_strides[4],
+                                                 const int64_t v_strides[4], const int64_t o_strides[4],
+                                                 const int64_t mask_sizes[4], const int64_t mask_strides[4],
+                                                 int mask_dtype, float sm_scale, int is_causal, float mask_min_clamp,
+                                                 int dtype, void *stream) {
+    using namespace kernl;
+    // the same number of key ranges as kernl_attention_skinny_fwd takes with a workspace of the reported size, so
+    // both entry points add the ranges in the same order; problems whose partial results do not fit are refused
+    const int64_t need = kernl_attention_skinny_workspace_bytes(B, H, M, N, D);
+    if (need > kSkScratchBytes)
+        return set_error(KERNL_ERR_UNSUPPORTED,
+                         "skinny attention (static): partial results need %lld bytes, the static buffer holds %lld; "
+                         "use kernl_attention_skinny_fwd with a workspace",
+                         (long long)need, (long long)kSkScratchBytes);
+    void *ws = nullptr;
+    if (need > 0) {
+        const int st = skinny_scratch(&ws);
+        if (st != KERNL_OK) return st;
+    }
+    return skinny_entry(q, k, v, out, mask, ws, need, B, H, M, N, D, q_strides, k_strides, v_strides, o_strides,
+                        mask_sizes, mask_strides, mask_dtype, sm_scale, is_causal, mask_min_clamp, dtype, false, stream);
+}
+
 extern "C" int kernl_attention_skinny_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
                                           void *workspace, int64_t workspace_bytes, int64_t B, int64_t H, int64_t M,
                                           int64_t N, int64_t D, const int64_t q_strides[4],
