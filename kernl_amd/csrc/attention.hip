@@ -18,48 +18,9 @@
 // exchange with lane ^ 32, and the fp32 score registers, once exponentiated and packed to 16 bit, already are
 // the MFMA "B" operand of Oᵀ = Vᵀ·Pᵀ — P never touches LDS.  Vᵀ rows are fed through rowperm16, so each lane
 // finishes with 16 consecutive output features of its query row and writes them as two 16-byte stores.
-#include <math.h>
-
-#include <type_traits>
-
-#include "common.h"
+#include "attention_common.h"
 
 namespace kernl {
-
-static constexpr float kLog2eA = 1.4426950408889634f;
-static constexpr float kNegBig = -1.0e30f;            // anything below: exp2(x - rowmax) is exactly 0
-static constexpr float kClampFloor = -1.7014118e38f;  // scaled mask values are kept finite (-FLT_MAX / 2)
-static constexpr float kRescaleThreshold = 8.0f;  // log2 units
-static constexpr float kMaskedScore = -32768.0f;  // base-2 scores below this are mask values, not scores
-
-enum { MASK_NONE = 0, MASK_VECTOR = 1, MASK_MATRIX = 2 };
-
-struct AttnParams {
-    const void *q, *k, *v, *mask;
-    void *o;
-    int B, H, M, N;
-    int64_t qs[4], ks[4], vs[4], os[4];  // element strides {batch, head, row, col}
-    int64_t ms[4];                       // mask strides, 0 on broadcast dims
-    int mask_dtype;
-    float scale_log2;  // sm_scale * log2(e)
-    float sm_scale;
-    float clamp;  // replacement for -inf mask entries
-    int nq_tiles;
-    int mask_fast;  // matrix mask rows can be read as aligned 4-element vectors through 32-bit offsets
-    int causal_off;  // causal: query row m sees keys 0 .. m + causal_off (0: top-left aligned)
-};
-
-__device__ __forceinline__ float load_mask_value(const void *mask, int dtype, int64_t off) {
-    if (dtype == KERNL_F32) return static_cast<const float *>(mask)[off];
-    if (dtype == KERNL_F16) return (float)static_cast<const f16 *>(mask)[off];
-    return (float)static_cast<const bf16 *>(mask)[off];
-}
-
-// mask value -> additive term in the log2 domain, finite.
-__device__ __forceinline__ float scale_mask(float mv, float clamp) {
-    if (mv == -INFINITY) mv = clamp;
-    return fmaxf(mv * kLog2eA, kClampFloor);
-}
 
 // ----------------------------------------------------------------------------------------------------
 // Streaming MFMA kernel: 64-key tiles staged by buffer loads that write LDS directly (no register staging, no
@@ -757,6 +718,9 @@ static int attention_entry(const void *q, const void *k, const void *v, void *ou
                          k_strides[2] > 0 && v_strides[2] > 0 &&  // one head's K / V extent must fit 31-bit byte offsets
                          (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30) &&
                          (mask == nullptr || (mask_strides[3] >= 0 && (N + 128) * mask_strides[3] < (1ll << 30)));
+    // the software-pipelined kernel takes what it covers (tuning hook: variant 3 keeps everything on the streaming kernel)
+    if (mfma_ok && g_attention_variant != 3 && launch_attention_pipe(p, (int)D, dtype, mask_mode, causal, st))
+        return check_launch("attention (pipelined mfma)");
     if (mfma_ok) {
         // head size 64 without a matrix mask fits the register budget of 3 waves per SIMD (168 VGPRs); the
         // matrix-mask body (mask values prefetched in registers) and head size 128 run at 2 waves per SIMD.
