@@ -273,8 +273,10 @@ int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, 
  *                                columns per workgroup); 9 = that kernel where it applies, the heuristic elsewhere;
  *                                1..8 keep such inputs on the tile kernels.
  *   kernl_attention_force_scalar non-zero routes every attention call through the strided scalar kernel.
- *   kernl_attention_set_variant  register budget of the head-size-64 MFMA attention kernel: 0 = heuristic,
- *                                1 = built for 3 waves/SIMD, 2 = built for 2 waves/SIMD.
+ *   kernl_attention_set_variant  0 = heuristic; register budget of the head-size-64 streaming attention kernel: 1 = built
+ *                                for 3 waves/SIMD, 2 = built for 2 waves/SIMD; 3 = streaming kernel for every shape,
+ *                                4 = software-pipelined kernel wherever it applies (head size 64; no mask, a per-key
+ *                                mask of at most 2048 keys, or causal), also below 1024 keys.
  */
 void kernl_linear_force_tile(int which);
 void kernl_attention_force_scalar(int on);

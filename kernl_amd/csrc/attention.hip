@@ -453,9 +453,10 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 #pragma unroll
                 for (int v = 0; v < 16; ++v) s_acc[nb][v] = __builtin_amdgcn_exp2f(s_acc[nb][v]);
 
-            // ---- Oᵀ += Vᵀ · Pᵀ; the row sum is taken from the ROUNDED probabilities (two per v_dot2c), i.e. from
-            // exactly the values that enter the product
-            float rs = 0.0f;
+            // ---- Oᵀ += Vᵀ · Pᵀ; the row sum is taken from the unrounded probabilities with plain additions (the
+            // reference does the same, attention.py:399-417): v_dot2c_f32_f16 on the packed pairs, one instruction
+            // less per pair, measured 16 cycles of the matrix pipe each when MFMAs are in flight
+            float rs = 0.0f, rs2 = 0.0f;
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int ps = 0; ps < BN / 16; ++ps) {
@@ -464,7 +465,8 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     pk[j] = pack2<T>(s_acc[nb][half8 + 2 * j], s_acc[nb][half8 + 2 * j + 1]);
-                    rs = pair_sum_acc<T>(pk[j], rs);
+                    rs += s_acc[nb][half8 + 2 * j];
+                    rs2 += s_acc[nb][half8 + 2 * j + 1];
                 }
                 const vec8 pf = __builtin_bit_cast(vec8, pk);
 #pragma unroll
@@ -477,7 +479,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                 }
             }
             __builtin_amdgcn_s_setprio(0);
-            l_i += rs;
+            l_i += rs + rs2;
         } else if (LATE_DMA) {
             dma(tile_next, ST ^ 1);
         }
@@ -718,8 +720,10 @@ static int attention_entry(const void *q, const void *k, const void *v, void *ou
                          k_strides[2] > 0 && v_strides[2] > 0 &&  // one head's K / V extent must fit 31-bit byte offsets
                          (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30) &&
                          (mask == nullptr || (mask_strides[3] >= 0 && (N + 128) * mask_strides[3] < (1ll << 30)));
-    // the software-pipelined kernel takes what it covers (tuning hook: variant 3 keeps everything on the streaming kernel)
-    if (mfma_ok && g_attention_variant != 3 && launch_attention_pipe(p, (int)D, dtype, mask_mode, causal, st))
+    // the software-pipelined kernel takes long key sequences of what it covers (hook: variant 3 keeps everything on the
+    // streaming kernel, variant 4 sends everything the pipelined kernel covers to it)
+    if (mfma_ok && g_attention_variant != 3 &&
+        launch_attention_pipe(p, (int)D, dtype, mask_mode, causal, g_attention_variant == 4, st))
         return check_launch("attention (pipelined mfma)");
     if (mfma_ok) {
         // head size 64 without a matrix mask fits the register budget of 3 waves per SIMD (168 VGPRs); the

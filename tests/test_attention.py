@@ -14,6 +14,17 @@ from oracle import attention_oracle
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["auto", "streaming", "pipelined"])
+def attention_kernel(request):
+    """Every case runs three times: with the library's own choice between its two MFMA kernels, with the streaming
+    kernel forced, and with the software-pipelined kernel forced wherever it applies (head size 64; no mask, per-key
+    mask or causal) — by default that kernel only takes 1024 keys or more, which few of the shapes here have."""
+    lib = _lib.load()
+    lib.kernl_attention_set_variant({"auto": 0, "streaming": 3, "pipelined": 4}[request.param])
+    yield request.param
+    lib.kernl_attention_set_variant(0)
+
+
 def _mk(shape, dtype, gen, lo=None):
     if lo is None:
         t = torch.randn(shape, generator=gen)
