@@ -63,6 +63,32 @@ def test_bert_base_matches_fp32_eager(attn):
         _compare(out2, ref2, mask2, f"bert-base {attn} replay")
 
 
+def test_bert_base_config3_full_size():
+    """BASELINE config 3 at its stated size: BERT-base (seed 0) in fp16 through `optimize_model`, forward captured in a
+    hipGraph, batch 32 x 512 tokens, lengths U[256, 512] — final hidden states against the fp32 eager model on the
+    CPU (counterpart of the reference's test/test_torchdynamo.py:60-83, which stops at 1e-1).  The full-size shapes
+    take kernel paths the smaller cases do not: more GEMM tiles than CUs in the persistent kernel, the 256x192 tile
+    choice, fused add + LayerNorm over 16384 rows, 1536 attention workgroups."""
+    from kernl_amd.model_optimization import optimize_model
+
+    torch._dynamo.reset()
+    gen = torch.Generator().manual_seed(0)
+    ids, mask = _inputs(32, 512, gen, min_len=256)
+    ref_model = _bert()
+    with torch.inference_mode():
+        ref = ref_model(input_ids=ids, attention_mask=mask).last_hidden_state
+    model = _bert().half().cuda()
+    optimize_model(model)
+    with torch.inference_mode():
+        out = model(input_ids=ids.cuda(), attention_mask=mask.cuda()).last_hidden_state  # warm-up + capture
+        out = model(input_ids=ids.cuda(), attention_mask=mask.cuda()).last_hidden_state  # replay
+        torch.cuda.synchronize()
+    _compare(out, ref, mask, "bert-base config 3 (32,512)")
+    # padded query rows are deterministic too (they attend to the valid keys): the whole tensor is finite and close
+    diff_all = (out.float().cpu() - ref).abs()
+    assert diff_all.max().item() <= 1e-1, diff_all.max().item()
+
+
 def test_bert_shape_change_without_rebuild():
     # reference test/test_torchdynamo.py:86-100
     from kernl_amd.model_optimization import optimize_model
@@ -118,12 +144,15 @@ def test_llama_shaped_decoder_matches_fp32_eager(attn):
     torch._dynamo.reset()
     gen = torch.Generator().manual_seed(3)
     ids = torch.randint(0, 1000, (2, 320), generator=gen)
-    # The fp16 operator clamps eps to >= 1.6e-5 (reference layer_norm.py:295-296, applied to RMSNorm as well).  With
-    # N(0, 0.02) weights the hidden states have variance ~4e-4, where 1e-5 vs 1.6e-5 moves rstd by 0.7 %, so the
-    # fp32 reference is built with the eps the operator actually uses.
-    ref_model = _llama(2, 512, 4, 1408, attn, eps=1.6e-5)
+    # The fp32 reference keeps the config's eps (1e-5).  The fp16 operator clamps eps to >= 1.6e-5 (reference
+    # layer_norm.py:295-296, applied to RMSNorm as well); with N(0, 0.02) weights the hidden states have variance
+    # ~4e-4, where that moves rstd by 0.7 %.  What the clamp alone does to the output is measured on the fp32 model
+    # (same weights, eps 1.6e-5) and added to the bound.
+    ref_model = _llama(2, 512, 4, 1408, attn)
     with torch.inference_mode():
         ref = ref_model(input_ids=ids, use_cache=False).last_hidden_state
+        ref_clamped = _llama(2, 512, 4, 1408, attn, eps=1.6e-5)(input_ids=ids, use_cache=False).last_hidden_state
+    clamp_rel = ((ref_clamped - ref).abs().mean() / ref.abs().mean()).item()
     model = _llama(2, 512, 4, 1408, attn).half().cuda()
     with torch.inference_mode():
         eager16 = model(input_ids=ids.cuda(), use_cache=False).last_hidden_state.float().cpu()
@@ -135,9 +164,9 @@ def test_llama_shaped_decoder_matches_fp32_eager(attn):
     # plain fp16 eager (eps 1e-5, unclamped) is printed beside ours for orientation
     eager_rel = ((eager16 - ref).abs().mean() / ref.abs().mean()).item()
     ours_rel = ((out.float().cpu() - ref).abs().mean() / ref.abs().mean()).item()
-    print(f"llama-shaped {attn}: mean_rel ours={ours_rel:.5f} fp16-eager={eager_rel:.5f}", flush=True)
+    print(f"llama-shaped {attn}: mean_rel ours={ours_rel:.5f} fp16-eager={eager_rel:.5f} eps-clamp alone={clamp_rel:.5f}", flush=True)
     assert torch.isfinite(out).all()
-    assert ours_rel <= 5e-3
+    assert ours_rel <= 5e-3 + clamp_rel
     assert (out.float().cpu() - ref).abs().max().item() <= 1e-1
 
 
@@ -160,9 +189,11 @@ def test_llama_shaped_short_input_runs_the_one_launch_norm_projections(monkeypat
     monkeypatch.setattr(_lib, "linear_rms_fwd", counting)
     gen = torch.Generator().manual_seed(6)
     ids = torch.randint(0, 1000, (2, 12), generator=gen)
-    ref_model = _llama(2, 512, 4, 1408, "sdpa", eps=1.6e-5)
+    ref_model = _llama(2, 512, 4, 1408, "sdpa")
     with torch.inference_mode():
         ref = ref_model(input_ids=ids, use_cache=False).last_hidden_state
+        ref_clamped = _llama(2, 512, 4, 1408, "sdpa", eps=1.6e-5)(input_ids=ids, use_cache=False).last_hidden_state
+    clamp_rel = ((ref_clamped - ref).abs().mean() / ref.abs().mean()).item()  # what the operator's fp16 eps clamp alone does
     model = _llama(2, 512, 4, 1408, "sdpa").half().cuda()
     optimize_model(model)
     with torch.inference_mode():
@@ -173,7 +204,7 @@ def test_llama_shaped_short_input_runs_the_one_launch_norm_projections(monkeypat
     assert calls["rms"] == 8 and calls["gated"] == 4, calls
     ours_rel = ((out.float().cpu() - ref).abs().mean() / ref.abs().mean()).item()
     print(f"llama-shaped, 24 rows: mean_rel ours={ours_rel:.5f}", flush=True)
-    assert torch.isfinite(out).all() and ours_rel <= 5e-3
+    assert torch.isfinite(out).all() and ours_rel <= 5e-3 + clamp_rel
 
 
 def test_llama_7b_shaped_layer_full_width():
@@ -187,10 +218,13 @@ def test_llama_7b_shaped_layer_full_width():
     torch._dynamo.reset()
     gen = torch.Generator().manual_seed(4)
     ids = torch.randint(0, 1000, (1, 2048), generator=gen)
-    ref_model = _llama(1, 4096, 32, 11008, eps=1.6e-5)  # see the eps note above
+    ref_model = _llama(1, 4096, 32, 11008)  # the config's own eps (1e-5)
     with torch.inference_mode():
         ref = ref_model(input_ids=ids, use_cache=False).last_hidden_state
-    model = _llama(1, 4096, 32, 11008, eps=1.6e-5).half().cuda()
+        # what the operator's fp16 eps clamp (>= 1.6e-5, reference layer_norm.py:295-296) alone does, on the fp32 model
+        ref_clamped = _llama(1, 4096, 32, 11008, eps=1.6e-5)(input_ids=ids, use_cache=False).last_hidden_state
+    clamp_rel = ((ref_clamped - ref).abs().mean() / ref.abs().mean()).item()
+    model = _llama(1, 4096, 32, 11008).half().cuda()
     with torch.inference_mode():
         eager16 = model(input_ids=ids.cuda(), use_cache=False).last_hidden_state.float().cpu()
     optimize_model(model)
@@ -200,16 +234,52 @@ def test_llama_7b_shaped_layer_full_width():
     eager_rel = ((eager16 - ref).abs().mean() / ref.abs().mean()).item()
     ours_rel = ((out.float().cpu() - ref).abs().mean() / ref.abs().mean()).item()
     early = ((out.float().cpu() - ref)[:, :64].abs().mean() / ref[:, :64].abs().mean()).item()
-    print(f"llama-7b-shaped layer: mean_rel ours={ours_rel:.5f} fp16-eager={eager_rel:.5f} ours(first 64 positions)={early:.5f}", flush=True)
+    print(f"llama-7b-shaped layer: mean_rel ours={ours_rel:.5f} fp16-eager={eager_rel:.5f} eps-clamp alone={clamp_rel:.5f} "
+          f"ours(first 64 positions)={early:.5f}", flush=True)
     assert torch.isfinite(out).all()
-    assert ours_rel <= max(5e-3, 1.1 * eager_rel)
-    assert early <= 5e-3
+    assert ours_rel <= max(5e-3, 1.1 * eager_rel) + clamp_rel
+    assert early <= 5e-3 + clamp_rel
 
 
 def _rel_errors(out, eager16, ref):
     ours = ((out.float().cpu() - ref).abs().mean() / ref.abs().mean()).item()
     eager = ((eager16 - ref).abs().mean() / ref.abs().mean()).item()
     return ours, eager
+
+
+def test_llama_7b_shaped_four_layers_full_width():
+    """BASELINE config 4 at full width and length, four of its 32 layers: hidden 4096, 32 heads of 128, SwiGLU 11008,
+    RoPE base 10000, RMSNorm eps 1e-5, weights N(0, 0.02), batch 1 x 2048 tokens, causal prefill through
+    `optimize_model` — against the fp32 eager model on the CPU, which keeps the config's eps.  The fp16 operator clamps
+    eps to >= 1.6e-5 (reference layer_norm.py:295-296); what that alone does is measured on the fp32 model and added to
+    the bound, and plain fp16 eager PyTorch is printed beside ours.  With random weights attention is close to
+    uniform over up to 2048 keys and fp16 accumulates error with depth and position, so the bound is "no further from
+    fp32 than fp16 eager PyTorch" with 10 % slack, and 5e-3 on the first 64 positions."""
+    from kernl_amd.model_optimization import optimize_model
+
+    torch._dynamo.reset()
+    gen = torch.Generator().manual_seed(7)
+    ids = torch.randint(0, 1000, (1, 2048), generator=gen)
+    with torch.inference_mode():
+        ref = _llama(4, 4096, 32, 11008)(input_ids=ids, use_cache=False).last_hidden_state
+        ref_clamped = _llama(4, 4096, 32, 11008, eps=1.6e-5)(input_ids=ids, use_cache=False).last_hidden_state
+    clamp_rel = ((ref_clamped - ref).abs().mean() / ref.abs().mean()).item()
+    del ref_clamped
+    model = _llama(4, 4096, 32, 11008).half().cuda()
+    with torch.inference_mode():
+        eager16 = model(input_ids=ids.cuda(), use_cache=False).last_hidden_state.float().cpu()
+    optimize_model(model)
+    with torch.inference_mode():
+        out = model(input_ids=ids.cuda(), use_cache=False).last_hidden_state
+        out = model(input_ids=ids.cuda(), use_cache=False).last_hidden_state
+        torch.cuda.synchronize()
+    ours, eager = _rel_errors(out, eager16, ref)
+    early = ((out.float().cpu() - ref)[:, :64].abs().mean() / ref[:, :64].abs().mean()).item()
+    print(f"llama-7b-shaped, 4 layers: mean_rel ours={ours:.5f} fp16-eager={eager:.5f} eps-clamp alone={clamp_rel:.5f} "
+          f"ours(first 64 positions)={early:.5f}", flush=True)
+    assert torch.isfinite(out).all()
+    assert ours <= max(5e-3, 1.1 * eager) + clamp_rel
+    assert early <= 5e-3 + clamp_rel
 
 
 @pytest.mark.parametrize("attn", ["eager", "sdpa"])
