@@ -13,8 +13,10 @@ One JSON line is printed:
                         timed region (on torch's current stream, which is where the kernels are launched);
   cpu_baseline          the CPU oracle (fp32 eager PyTorch on the host cores) on a bounded sample of the same workload;
   extra                 the other numbers the metric names: executed (skip-aware) attention flops, fused linear and
-                        LayerNorm at BASELINE config 2, BERT-base b32 s512 fp16 forward latency through
-                        `optimize_model` (hipGraph replay, median wall clock of 10), and CPU timings beside them.
+                        LayerNorm at BASELINE config 2 — graph-replayed ("warm") and `*_cold_us`: single launches after a
+                        256 MB cache flush, the LayerNorm fraction of the HBM peak on the cold figure —, BERT-base b32
+                        s512 fp16 forward latency through `optimize_model` (hipGraph replay, median wall clock of 10) with
+                        its hidden states checked against the fp32 CPU model, and CPU timings beside them.
 """
 import argparse
 import json
@@ -47,6 +49,20 @@ def _event_times(fn, n, flush=None):
     return times
 
 
+def traffic_from_profile():
+    """HBM bytes per launch of the headline kernel as measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE runs,
+    each scaled by the same counter's reading for a copy of known size): the line `traffic_bytes_per_launch: <number>`
+    of profiles/attention_config1_pmc_traffic.txt, or None when the file is not there."""
+    path = os.path.join(ROOT, "profiles", "attention_config1_pmc_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return float(line.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
 def config1_inputs():
     import torch
 
@@ -58,6 +74,25 @@ def config1_inputs():
     for b in range(32):
         mask[b, :, :, lengths[b]:] = float("-inf")
     return q, k, v, mask, lengths
+
+
+def config2_tensors(dev):
+    import torch
+
+    gen = torch.Generator().manual_seed(0)
+    M, Kd, N = 16384, 768, 3072
+    t = {"M": M, "K": Kd, "N": N}
+    t["x_up"] = torch.randn((M, Kd), generator=gen).half().to(dev)
+    t["w_up"] = (torch.randn((N, Kd), generator=gen) * 0.02).half().to(dev)
+    t["b_up"] = (torch.randn((N,), generator=gen) * 0.02).half().to(dev)
+    t["x_dn"] = torch.randn((M, N), generator=gen).half().to(dev)
+    t["w_dn"] = (torch.randn((Kd, N), generator=gen) * 0.02).half().to(dev)
+    t["b_dn"] = (torch.randn((Kd,), generator=gen) * 0.02).half().to(dev)
+    t["x_ln"] = torch.randn((M, Kd), generator=gen).half().to(dev)
+    t["g_ln"] = (1 + 0.1 * torch.randn((Kd,), generator=gen)).half().to(dev)
+    t["be_ln"] = (0.1 * torch.randn((Kd,), generator=gen)).half().to(dev)
+    t["gen"] = gen
+    return t
 
 
 def main():
@@ -73,6 +108,13 @@ def main():
         action="store_true",
         help="launch the headline kernel 3 times, then copy a 64 MiB tensor 3 times, and exit: the workload of the "
         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (the copy of known size scales the counters)",
+    )
+    ap.add_argument(
+        "--cold-probe",
+        action="store_true",
+        help="launch attention (config 1), both config-2 linears, LayerNorm and a copy of the LayerNorm bytes 20 times "
+        "each, every launch after a 256 MB cache flush, and exit: the workload of the rocprofv3 --kernel-trace run "
+        "behind the *_cold_us figures (profiles/bench_cold_kernel_trace.txt)",
     )
     args = ap.parse_args()
     if args.gpus != 1:
@@ -110,6 +152,24 @@ def main():
         dst = torch.empty_like(src)
         for _ in range(3):
             dst.copy_(src)
+        torch.cuda.synchronize()
+        return
+
+    if args.cold_probe:
+        c2 = config2_tensors(dev)
+        flush = torch.empty(256 * 1024 * 1024, dtype=torch.int8, device=dev)
+        cp_dst = torch.empty_like(c2["x_ln"])
+        probes = [
+            step,
+            lambda: linear_layer(c2["x_up"], c2["w_up"], c2["b_up"], "fast_gelu"),
+            lambda: linear_layer(c2["x_dn"], c2["w_dn"], c2["b_dn"], ""),
+            lambda: layer_norm(c2["x_ln"], c2["g_ln"], c2["be_ln"], 1e-12),
+            lambda: cp_dst.copy_(c2["x_ln"]),
+        ]
+        for fn in probes:
+            for _ in range(20):
+                flush.zero_()
+                fn()
         torch.cuda.synchronize()
         return
 
@@ -177,8 +237,8 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_MFMA_F16_TFLOPS, 4),
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy of known
-            # size (profiles/attention_config1_pmc_traffic.txt); algorithmic bytes are 100.7e6
-            "traffic": 92.0e6,
+            # size, read from profiles/attention_config1_pmc_traffic.txt; algorithmic bytes are 100.7e6
+            "traffic": traffic_from_profile(),
         },
     }
     extra = {
@@ -220,17 +280,11 @@ def main():
     # ------------------------------------------------------------------ the other kernels of the metric (config 2)
     if not args.skip_extra:
         flush = torch.empty(256 * 1024 * 1024, dtype=torch.int8, device=dev)
-        gen = torch.Generator().manual_seed(0)
-        M, Kd, N = 16384, 768, 3072
-        x_up = torch.randn((M, Kd), generator=gen).half().to(dev)
-        w_up = (torch.randn((N, Kd), generator=gen) * 0.02).half().to(dev)
-        b_up = (torch.randn((N,), generator=gen) * 0.02).half().to(dev)
-        x_dn = torch.randn((M, N), generator=gen).half().to(dev)
-        w_dn = (torch.randn((Kd, N), generator=gen) * 0.02).half().to(dev)
-        b_dn = (torch.randn((Kd,), generator=gen) * 0.02).half().to(dev)
-        x_ln = torch.randn((M, Kd), generator=gen).half().to(dev)
-        g_ln = (1 + 0.1 * torch.randn((Kd,), generator=gen)).half().to(dev)
-        be_ln = (0.1 * torch.randn((Kd,), generator=gen)).half().to(dev)
+        c2 = config2_tensors(dev)
+        gen = c2["gen"]
+        M, Kd, N = c2["M"], c2["K"], c2["N"]
+        x_up, w_up, b_up, x_dn, w_dn, b_dn = c2["x_up"], c2["w_up"], c2["b_up"], c2["x_dn"], c2["w_dn"], c2["b_dn"]
+        x_ln, g_ln, be_ln = c2["x_ln"], c2["g_ln"], c2["be_ln"]
         lin_flop = 2.0 * M * N * Kd
         ln_bytes = 2 * (2 * M * Kd + 2 * Kd)
 
@@ -250,35 +304,54 @@ def main():
             torch.cuda.synchronize()
             return statistics.median(_event_times(g.replay, 20)) / reps
 
+        def cold_us(fn):
+            """Median of 30 single launches, each after the 256 MB flush buffer has been rewritten (memory-side cache
+            and L2 hold none of the operands), timed with an event pair around the launch."""
+            return statistics.median(_event_times(fn, 30, flush)) * 1e3
+
         def measure(fn, label, work, unit_scale, peak):
             warm = graph_time_ms(fn)
-            cold = statistics.median(_event_times(fn, 30, flush))  # one eager launch after a 256 MB cache flush
+            cold = cold_us(fn)
             extra[f"{label}_us_graph_replay"] = round(warm * 1e3, 2)
-            extra[f"{label}_us_cold_single_launch"] = round(cold * 1e3, 2)
+            extra[f"{label}_cold_us"] = round(cold, 2)
             rate = work / (warm * 1e-3) / unit_scale
             extra[f"{label}_tflops_graph_replay"] = round(rate, 1)
             extra[f"{label}_frac_of_peak"] = round(rate / peak, 4)
+            extra[f"{label}_cold_frac_of_peak"] = round(work / (cold * 1e-6) / unit_scale / peak, 4)
 
+        extra["attention_cold_us"] = round(cold_us(step), 2)
         measure(lambda: linear_layer(x_up, w_up, b_up, "fast_gelu"), "linear_up_tanh_gelu", lin_flop, 1e12,
                 PEAK_MFMA_F16_TFLOPS)
         measure(lambda: linear_layer(x_dn, w_dn, b_dn, ""), "linear_down", lin_flop, 1e12, PEAK_MFMA_F16_TFLOPS)
 
-        # LayerNorm is ~10 us of GPU time: only the graph-replayed figure is meaningful
+        # LayerNorm: the fraction of the HBM peak is put on the COLD figure (a graph replay of 20 launches over the same
+        # 50 MB runs out of the 256 MB memory-side cache); the warm figure and a copy of the same bytes stand beside it
         ln_out = [None]
 
         def ln_once():
             ln_out[0] = layer_norm(x_ln, g_ln, be_ln, 1e-12)
 
         t = graph_time_ms(ln_once, reps=20)
+        cold = cold_us(ln_once)
         extra["layernorm_us_graph_replay"] = round(t * 1e3, 2)
         extra["layernorm_gbps_graph_replay"] = round(ln_bytes / (t * 1e-3) / 1e9, 1)
-        extra["layernorm_frac_of_hbm_peak"] = round(ln_bytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
-        cold = statistics.median(_event_times(ln_once, 30, flush))
-        extra["layernorm_us_cold_single_launch"] = round(cold * 1e3, 2)
+        extra["layernorm_cold_us"] = round(cold, 2)
+        extra["layernorm_cold_gbps"] = round(ln_bytes / (cold * 1e-6) / 1e9, 1)
+        extra["layernorm_frac_of_hbm_peak"] = round(ln_bytes / (cold * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4)
+        extra["layernorm_warm_frac_of_hbm_peak"] = round(ln_bytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
+        # four times the rows: ramp and drain weigh less
+        x_ln4 = torch.randn((4 * M, Kd), generator=gen).half().to(dev)
+        cold4 = cold_us(lambda: layer_norm(x_ln4, g_ln, be_ln, 1e-12))
+        extra["layernorm_65536x768_cold_us"] = round(cold4, 2)
+        extra["layernorm_65536x768_cold_gbps"] = round(4 * ln_bytes / (cold4 * 1e-6) / 1e9, 1)
+        del x_ln4
         # what a plain device-to-device copy of the same 2 x 25 MB reaches on this box (the practical HBM ceiling)
         cp_src, cp_dst = x_ln, torch.empty_like(x_ln)
         t = graph_time_ms(lambda: cp_dst.copy_(cp_src), reps=20)
+        cold = cold_us(lambda: cp_dst.copy_(cp_src))
         extra["copy_same_bytes_gbps_graph_replay"] = round(2 * x_ln.numel() * 2 / (t * 1e-3) / 1e9, 1)
+        extra["copy_same_bytes_cold_us"] = round(cold, 2)
+        extra["copy_same_bytes_cold_gbps"] = round(2 * x_ln.numel() * 2 / (cold * 1e-6) / 1e9, 1)
         del flush
 
         # ---- the decoder-side kernels (Llama-7B prefill / decode shapes), graph-replayed
@@ -385,16 +458,28 @@ def main():
             ms = statistics.median(times)
             extra["bert_base_b32_s512_fp16_fwd_ms"] = round(ms, 3)
             extra["bert_base_b32_s512_tflops"] = round(3.092e12 / (ms * 1e-3) / 1e12, 1)
+            with torch.inference_mode():
+                hidden = model(input_ids=ids_d, attention_mask=amask_d).last_hidden_state
+                torch.cuda.synchronize()
+            assert torch.isfinite(hidden).all(), "BERT-base b32 s512: non-finite hidden states"
             if not args.skip_cpu:
-                # CPU eager fp32 on 2 of the 32 sequences, scaled by 16 (the model is batch-parallel)
+                # CPU eager fp32 on 2 of the 32 sequences: timed (scaled by 16, the model is batch-parallel) and used to
+                # check the hidden states the timed graph produces for those sequences
                 torch.manual_seed(0)
                 cpu_model = BertModel(cfg).eval()
                 with torch.inference_mode():
                     cpu_model(input_ids=ids[:2], attention_mask=amask[:2])
                     t = time.perf_counter()
-                    cpu_model(input_ids=ids[:2], attention_mask=amask[:2])
+                    ref = cpu_model(input_ids=ids[:2], attention_mask=amask[:2]).last_hidden_state
                     dt = time.perf_counter() - t
                 extra["bert_base_b32_s512_cpu_fp32_ms_scaled_from_2_of_32"] = round(dt * 1e3 * 16, 1)
+                valid = amask[:2].bool()
+                diff = (hidden[:2].float().cpu() - ref).abs()
+                max_abs = diff[valid].max().item()
+                mean_rel = (diff[valid].mean() / ref[valid].abs().mean()).item()
+                extra["bert_base_b32_s512_max_abs_err_vs_fp32_cpu_2_seqs"] = round(max_abs, 5)
+                extra["bert_base_b32_s512_mean_rel_err_vs_fp32_cpu_2_seqs"] = round(mean_rel, 6)
+                assert max_abs <= 5e-2 and mean_rel <= 5e-3, f"BERT-base b32 s512 hidden states off: {max_abs} {mean_rel}"
         except Exception as exc:  # the headline number must still be reported
             extra["bert_base_b32_s512_error"] = f"{type(exc).__name__}: {exc}"[:300]
 
