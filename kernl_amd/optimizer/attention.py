@@ -28,6 +28,25 @@ def _rows_aligned(*tensors: torch.Tensor) -> bool:
     return True
 
 
+SPLIT_K_MAX_ROWS = 65535  # batch x heads x queries the split-K kernel's launch grid can hold
+
+
+def takes_split_k_kernel(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> bool:
+    """Whether a [batch, heads, queries, dhead] problem goes to the split-K (single-query) kernel: one query per
+    row over more than 50 keys (reference: optimizer/attention.py:45), a head size that kernel is built for, rows it
+    can load 16 bytes at a time, and no more rows than its grid holds — larger decode batches stay on the tiled
+    kernel, which takes one-query tiles too."""
+    dhead = q.size(-1)
+    return (
+        q.size(-2) == 1
+        and k.size(-2) > 50
+        and 8 <= dhead <= 256
+        and (dhead & (dhead - 1)) == 0
+        and q.size(0) * q.size(1) * q.size(2) <= SPLIT_K_MAX_ROWS
+        and _rows_aligned(q, k, v)
+    )
+
+
 def attention_wrapper(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -48,8 +67,7 @@ def attention_wrapper(
     # Single-query attention over long keys has no parallelism over rows: like the reference
     # (optimizer/attention.py:45-49) hand it to the split-K kernel — which here also takes masks and the causal
     # flag, where the reference falls back to eager PyTorch.  Head sizes it does not cover stay on the tiled kernel.
-    dhead = q.size(-1)
-    if q.size(-2) == 1 and k.size(-2) > 50 and 8 <= dhead <= 256 and (dhead & (dhead - 1)) == 0 and _rows_aligned(q, k, v):
+    if takes_split_k_kernel(q, k, v):
         skinny_attention_forward(q, k, v, output, sm_scale, is_causal=is_causal, attention_mask=attention_mask)
     else:
         attention_forward(q, k, v, output, sm_scale, is_causal=is_causal, attention_mask=attention_mask)
@@ -90,18 +108,12 @@ def fuse_attention_pattern_1(gm: torch.fx.GraphModule, is_causal: bool):
     """BERT as the reference saw it: softmax(q·kᵀ / 8.0 + mask)·v."""
 
     def pattern(q, k, attention_mask, v):
-        transpose_10 = k.transpose(-1, -2)
-        matmul_20 = torch.matmul(q, transpose_10)
-        truediv_10 = matmul_20 / 8.0
-        add_30 = truediv_10 + attention_mask
-        softmax_10 = torch.nn.functional.softmax(add_30, dim=-1)
-        matmul_21 = torch.matmul(softmax_10, v)
-        return matmul_21
+        scores = torch.matmul(q, k.transpose(-1, -2)) / 8.0
+        probs = torch.nn.functional.softmax(scores + attention_mask, dim=-1)
+        return torch.matmul(probs, v)
 
     def replace(q, k, attention_mask, v):
-        output = torch.empty_like(q)
-        output = attention_wrapper(q, k, v, output, 1 / 8.0, is_causal, attention_mask)
-        return output
+        return attention_wrapper(q, k, v, torch.empty_like(q), 1 / 8.0, is_causal, attention_mask)
 
     replace_pattern(gm, pattern, replace)
 
@@ -109,20 +121,13 @@ def fuse_attention_pattern_1(gm: torch.fx.GraphModule, is_causal: bool):
 def fuse_attention_pattern_2(gm: torch.fx.GraphModule, is_causal: bool):
     """T5: scores + position_bias, softmax in float, cast back; no scaling."""
 
-    def pattern(q, k, encoder_decoder_position_bias, v):
-        transpose_3 = k.transpose(3, 2)
-        matmul = torch.matmul(q, transpose_3)
-        add_2 = torch.add(matmul, encoder_decoder_position_bias)
-        float_1 = add_2.float()
-        softmax = torch.nn.functional.softmax(float_1, dim=-1)
-        type_as = softmax.type_as(add_2)
-        matmul_1 = torch.matmul(type_as, v)
-        return matmul_1
+    def pattern(q, k, position_bias, v):
+        biased = torch.add(torch.matmul(q, k.transpose(3, 2)), position_bias)
+        probs = torch.nn.functional.softmax(biased.float(), dim=-1).type_as(biased)
+        return torch.matmul(probs, v)
 
-    def replace(q, k, encoder_decoder_position_bias, v):
-        output = torch.empty_like(q)
-        output = attention_wrapper(q, k, v, output, 1.0, is_causal, encoder_decoder_position_bias)
-        return output
+    def replace(q, k, position_bias, v):
+        return attention_wrapper(q, k, v, torch.empty_like(q), 1.0, is_causal, position_bias)
 
     replace_pattern(gm, pattern, replace)
 
@@ -131,16 +136,11 @@ def fuse_attention_pattern_3(gm: torch.fx.GraphModule, is_causal: bool):
     """Whisper: bmm-shaped, pre-scaled q, no mask."""
 
     def pattern(q, k, v):
-        transpose_46 = k.transpose(1, 2)
-        bmm_22 = torch.bmm(q, transpose_46)
-        softmax_11 = torch.nn.functional.softmax(bmm_22, dim=-1)
-        bmm_23 = torch.bmm(softmax_11, v)
-        return bmm_23
+        probs = torch.nn.functional.softmax(torch.bmm(q, k.transpose(1, 2)), dim=-1)
+        return torch.bmm(probs, v)
 
     def replace(q, k, v):
-        output = torch.empty_like(q)
-        output = attention_wrapper(q, k, v, output, 1.0, is_causal, None)
-        return output
+        return attention_wrapper(q, k, v, torch.empty_like(q), 1.0, is_causal, None)
 
     replace_pattern(gm, pattern, replace)
 

@@ -16,6 +16,7 @@ from typing import Callable, Iterable, List, Optional, Sequence, Union
 import torch
 from torch._subclasses import FakeTensor
 
+from kernl_amd.optimizer.linear import refresh_fused_parameters
 from kernl_amd.optimizer.pool_cuda_graphs import CudaGraphPool, get_aligned_size
 
 static_inputs_pool: List[CudaGraphPool] = []
@@ -117,6 +118,9 @@ class _CapturedGraph:
             for i, c in zip(self.dynamic_idx, copies):
                 # same signature => same placement; anything else would replay on stale addresses
                 assert c.data_ptr() == self.graph_inputs[i].data_ptr(), "static input pool placement changed"
+        # fused weights that are re-arranged copies of parameters follow their parameters: rewritten in place, at the
+        # address the graph reads, when a parameter's version counter has moved since the last call
+        refresh_fused_parameters(only_changed=True)
         self.graph.replay()
         return self.outputs
 

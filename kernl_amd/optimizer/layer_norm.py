@@ -97,14 +97,8 @@ def replace_layer_norm_fn(gm: torch.fx.GraphModule):
 def replace_layer_norm_rms(gm: torch.fx.GraphModule):
     # T5 spelling (reference pattern, eps generalised from the literal 1e-06)
     def pattern(v, weight, literal_eps):
-        to_38 = v.to(torch.float32)
-        pow_32 = to_38.pow(2)
-        mean_31 = pow_32.mean(-1, keepdim=True)
-        add_68 = mean_31 + literal_eps
-        rsqrt_31 = torch.rsqrt(add_68)
-        mul_69 = v * rsqrt_31
-        mul_70 = weight * mul_69
-        return mul_70
+        mean_square = v.to(torch.float32).pow(2).mean(-1, keepdim=True)
+        return weight * (v * torch.rsqrt(mean_square + literal_eps))
 
     def replace(v, weight, literal_eps):
         return layer_norm_rms_wrapper(v, weight, literal_eps)

@@ -135,43 +135,91 @@ def replace_linear_fn_constant_match(gm: torch.fx.GraphModule):
 
 class _DerivedParams:
     """Tensors derived from a group of parameters (concatenated or interleaved weights), kept for as long as the
-    parameters they were made from are alive and unchanged.
+    parameters they were made from are alive and stay where they are.
 
-    The key is the originals' storage addresses, versions and dtypes; an address alone is not an identity — once a
-    model is freed the allocator hands the same addresses to the next one — so every entry also holds weak references
-    to the original tensors and is dropped as soon as one of them has died or moved."""
+    Two kinds of entry:
+
+    * aliased — the derived tensor IS the parameters' memory: after the concatenation every original is re-pointed at
+      its slice of the fused buffer, so any in-place update of a parameter (optimizer step, `load_state_dict`,
+      `w.data.copy_(...)`) lands in the fused buffer, in eager calls and under hipGraph replays alike;
+    * copied — the derived tensor is a separate arrangement of the values (block-interleaved gate / value rows, which
+      no strided view of the originals can express).  Its entry remembers the originals' version counters; a lookup
+      that finds them changed rebuilds the derived tensor IN PLACE, so graphs captured on its address stay valid.
+      Writes that bypass the version counter (`w.data.copy_(...)`) need `refresh_fused_parameters()`.
+
+    The key is the originals' storage addresses and dtypes; an address alone is not an identity — once a model is
+    freed the allocator hands the same addresses to the next one — so every entry also holds weak references to the
+    original tensors and is dropped as soon as one of them has died or moved."""
+
+    class _Entry:
+        __slots__ = ("refs", "value", "versions", "rebuild")
+
+        def __init__(self, refs, value, versions, rebuild):
+            self.refs, self.value, self.versions, self.rebuild = refs, value, versions, rebuild
 
     def __init__(self):
         self._entries = {}
 
     @staticmethod
     def key_of(params):
-        return tuple((0, 0, None) if p is None else (p.data_ptr(), p._version, p.dtype) for p in params)
+        return tuple((0, None) if p is None else (p.data_ptr(), p.dtype) for p in params)
+
+    @staticmethod
+    def _versions(params):
+        return tuple(-1 if p is None else p._version for p in params)
 
     def get(self, params):
-        entry = self._entries.get(self.key_of(params))
+        key = self.key_of(params)
+        entry = self._entries.get(key)
         if entry is None:
             return None
-        refs, value = entry
-        for ref, p in zip(refs, params):
+        originals = []
+        for ref, p in zip(entry.refs, params):
             if p is None:
+                originals.append(None)
                 continue
             alive = ref()
             # the tensor passed in may be an alias of the original (same storage); what matters is that the original
             # still owns that memory
-            if alive is None or alive.data_ptr() != p.data_ptr() or alive._version != p._version:
-                del self._entries[self.key_of(params)]
+            if alive is None or alive.data_ptr() != p.data_ptr():
+                del self._entries[key]
                 return None
-        return value
+            originals.append(alive)
+        if entry.rebuild is not None:
+            versions = self._versions(originals)
+            if versions != entry.versions:
+                entry.rebuild(entry.value, originals)
+                entry.versions = versions
+        return entry.value
 
-    def put(self, params, value):
+    def put(self, params, value, rebuild=None):
+        """`rebuild(value, originals)` rewrites `value` in place from the originals; None for aliased entries."""
         import weakref
 
-        self._entries = {
-            k: (refs, v) for k, (refs, v) in self._entries.items() if all(r is None or r() is not None for r in refs)
-        }
+        self._drop_dead()
         refs = [None if p is None else weakref.ref(p) for p in params]
-        self._entries[self.key_of(params)] = (refs, value)
+        self._entries[self.key_of(params)] = self._Entry(refs, value, self._versions(params), rebuild)
+
+    def _drop_dead(self):
+        self._entries = {
+            k: e for k, e in self._entries.items() if all(r is None or r() is not None for r in e.refs)
+        }
+
+    def refresh(self, only_changed: bool) -> int:
+        """Rebuild copied entries in place from their live originals; returns how many were rebuilt."""
+        self._drop_dead()
+        n = 0
+        for entry in self._entries.values():
+            if entry.rebuild is None:
+                continue
+            originals = [None if r is None else r() for r in entry.refs]
+            versions = self._versions(originals)
+            if only_changed and versions == entry.versions:
+                continue
+            entry.rebuild(entry.value, originals)
+            entry.versions = versions
+            n += 1
+        return n
 
     def __len__(self):
         return len(self._entries)
@@ -179,6 +227,18 @@ class _DerivedParams:
 
 # concatenated / interleaved parameters of fused projections
 _fused_params = _DerivedParams()
+
+
+def refresh_fused_parameters(only_changed: bool = False) -> int:
+    """Re-derive, in place, every fused weight that is a re-arranged COPY of model parameters (the block-interleaved
+    gate / value weights of gated feed-forward layers) and return how many were rewritten.
+
+    Concatenated query / key / value weights need no refresh: the parameters alias the fused buffer.  Copied ones are
+    refreshed by themselves whenever a parameter's version counter has moved (optimizer steps, `load_state_dict`,
+    `param.copy_()`), in eager calls and before every hipGraph replay; call this after writes the counter does not
+    see (`param.data.copy_(...)`, `param.data.mul_(...)`).  Re-assigning `param.data` to new memory is not supported
+    under a captured graph, as for any other parameter: the graph keeps reading the old address."""
+    return _fused_params.refresh(only_changed)
 
 
 def fused_linear_wrapper(v: torch.Tensor, weights, biases):
@@ -194,7 +254,9 @@ def fused_linear_wrapper(v: torch.Tensor, weights, biases):
 
 
 def _concatenated_params(v: torch.Tensor, weights, biases):
-    """Row-concatenated weight (and bias) of sibling projections, built once per group of parameters."""
+    """Row-concatenated weight (and bias) of sibling projections, built once per group of parameters.  The originals
+    are re-pointed at their slices of the fused buffers, so there is ONE copy of the values and updates of a
+    parameter are updates of the fused weight."""
     originals = tuple(weights) + tuple(biases)
     cached = _fused_params.get(originals)
     if cached is None:
@@ -204,14 +266,21 @@ def _concatenated_params(v: torch.Tensor, weights, biases):
                 w.data = w.data.half()
             if b is not None and b.dtype == torch.float32 and (v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")):
                 b.data = b.data.half()
+        sizes = [w.shape[0] for w in weights]
         weight = torch.cat([w.detach() for w in weights], dim=0).contiguous()
         bias = None
         if any(b is not None for b in biases):
             bias = torch.cat(
                 [torch.zeros(w.shape[0], dtype=w.dtype, device=w.device) if b is None else b.detach() for w, b in zip(weights, biases)]
             ).contiguous()
-        cached = (weight, bias, [w.shape[0] for w in weights])
-        _fused_params.put(originals, cached)  # keyed after the one-time cast: by the addresses the parameters keep
+        row = 0
+        for w, b, n in zip(weights, biases, sizes):
+            w.data = weight[row : row + n]
+            if b is not None:
+                b.data = bias[row : row + n]
+            row += n
+        cached = (weight, bias, sizes)
+        _fused_params.put(originals, cached)  # keyed by the addresses the parameters now have inside the fused buffers
     return cached
 
 
@@ -285,7 +354,8 @@ def _glu_usable(v: torch.Tensor, w_gate, b_gate, w_value, b_value):
 
 
 def _interleaved_params(half: bool, w_gate, b_gate, w_value, b_value):
-    """Block-interleaved weight (and bias) of a gated linear unit, built once per group of parameters."""
+    """Block-interleaved weight (and bias) of a gated linear unit, built once per group of parameters and rewritten in
+    place when the parameters' version counters move."""
     params = (w_gate, w_value) + (() if b_gate is None else (b_gate, b_value))
     cached = _fused_params.get(params)
     if cached is None:
@@ -295,7 +365,13 @@ def _interleaved_params(half: bool, w_gate, b_gate, w_value, b_value):
         weight = interleave_glu_rows(w_gate.detach(), w_value.detach())
         bias = None if b_gate is None else interleave_glu_rows(b_gate.detach(), b_value.detach())
         cached = (weight, bias)
-        _fused_params.put(params, cached)
+
+        def rebuild(value, originals):
+            value[0].copy_(interleave_glu_rows(originals[0].detach(), originals[1].detach()))
+            if value[1] is not None:
+                value[1].copy_(interleave_glu_rows(originals[2].detach(), originals[3].detach()))
+
+        _fused_params.put(params, cached, rebuild)
     return cached
 
 

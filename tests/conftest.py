@@ -21,13 +21,17 @@ def set_seed():
 
 # Tolerance of the fp16/bf16 kernels against the fp32 oracle on the same (already rounded) inputs:
 # max-abs-error <= 1e-2 and mean relative error <= 1e-3 for fp16 outputs of unit scale.  bf16 has 3 fewer mantissa
-# bits than fp16, so its bounds are 8x wider.  Outputs of larger magnitude scale the absolute bound.
-def check_close(actual: torch.Tensor, expected: torch.Tensor, dtype=torch.float16, scale: float = 1.0, what: str = ""):
+# bits than fp16, so its bounds are 8x wider.  Outputs of larger magnitude scale the absolute bound: a number, or
+# "magnitude" for max|expected| / 4 (never below 1) — the spacing of fp16 values doubles with every power of two,
+# and at |y| = 4 the unit bound of 1e-2 is 2.5 spacings.
+def check_close(actual: torch.Tensor, expected: torch.Tensor, dtype=torch.float16, scale=1.0, what: str = ""):
     a = actual.detach().float().cpu()
     e = expected.detach().float().cpu()
     assert a.shape == e.shape, f"{what}: shape {tuple(a.shape)} != {tuple(e.shape)}"
     assert torch.isfinite(a).all(), f"{what}: non-finite values in the kernel output"
     widen = 8.0 if dtype == torch.bfloat16 else 1.0
+    if scale == "magnitude":
+        scale = max(1.0, e.abs().max().item() / 4)
     max_abs = (a - e).abs().max().item()
     mean_rel = ((a - e).abs().mean() / e.abs().mean().clamp_min(1e-12)).item()
     assert max_abs <= 1e-2 * widen * scale, f"{what}: max abs error {max_abs:.3e} > {1e-2 * widen * scale:.1e}"

@@ -130,6 +130,28 @@ def test_attention_wrapper_dispatches_single_query(monkeypatch, close):
         assert len(calls) == expected_calls
 
 
+def test_attention_wrapper_keeps_very_large_decode_batches_on_the_tiled_kernel(monkeypatch, close):
+    # more rows (batch x heads) than the split-K kernel's grid holds: the wrapper must not hand them over
+    import kernl_amd.optimizer.attention as opt
+
+    calls = []
+    real = opt.skinny_attention_forward
+    monkeypatch.setattr(opt, "skinny_attention_forward", lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
+    B, H, N, D = 2200, 32, 64, 64                       # 70400 rows
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    q = torch.randn((B, H, 1, D), generator=gen, device="cuda", dtype=torch.half)
+    k = torch.randn((B, H, N, D), generator=gen, device="cuda", dtype=torch.half)
+    v = torch.randn((B, H, N, D), generator=gen, device="cuda", dtype=torch.half)
+    out = torch.empty_like(q)
+    attention_wrapper(q, k, v, out, 0.125, False, None)
+    torch.cuda.synchronize()
+    assert not calls
+    for b in (0, 1099, B - 1):                          # the oracle on three batch entries, first to last
+        sl = slice(b, b + 1)
+        close(out[sl], attention_oracle(q[sl].cpu(), k[sl].cpu(), v[sl].cpu(), 0.125, False, None), torch.float16,
+              what=f"70400-row decode, batch entry {b}")
+
+
 def test_skinny_rejects_unsupported_head_size():
     q = torch.zeros((1, 1, 1, 48), dtype=torch.half, device="cuda")
     k = torch.zeros((1, 1, 64, 48), dtype=torch.half, device="cuda")

@@ -475,7 +475,8 @@ def test_glu_row_interleaving_and_pass():
 def test_derived_parameter_cache_follows_the_life_of_its_parameters():
     """Concatenated / interleaved weights are kept per group of original parameters.  A storage address is not an
     identity (the allocator hands a freed model's addresses to the next model), so an entry must stop matching as soon
-    as one of its originals has died, moved or been written to — also when another tensor then shows the same address."""
+    as one of its originals has died or moved — also when another tensor then shows the same address — and an entry
+    that is a re-arranged copy is rewritten in place when an original has been written to."""
     import gc
 
     from kernl_amd.optimizer.linear import _DerivedParams
@@ -483,14 +484,22 @@ def test_derived_parameter_cache_follows_the_life_of_its_parameters():
     cache = _DerivedParams()
     a, b = torch.zeros(8), torch.ones(4)
     assert cache.get((a, None, b)) is None
-    cache.put((a, None, b), "derived from a, b")
-    assert cache.get((a, None, b)) == "derived from a, b"
+    derived = torch.zeros(12)
+
+    def rebuild(value, originals):
+        value.copy_(torch.cat([originals[0], originals[2]]))
+
+    cache.put((a, None, b), derived, rebuild)
+    assert cache.get((a, None, b)) is derived
     alias = torch.empty(0).set_(a.untyped_storage(), 0, (8,))   # same storage and address, no reference to `a`
-    a.add_(1)                                 # written to: the derived tensor is stale
-    assert cache.get((a, None, b)) is None
-    cache.put((a, None, b), "again")
-    assert cache.get((a, None, b)) == "again"
-    assert _DerivedParams.key_of((alias, None, b)) == _DerivedParams.key_of((a, None, b))  # address, version, dtype
+    a.add_(1)                                 # written to: the same tensor comes back, rewritten in place
+    again = cache.get((a, None, b))
+    assert again is derived and again.tolist() == [1.0] * 12
+    a.data.add_(1)                            # a write the version counter does not see
+    assert cache.get((a, None, b)).tolist() == [1.0] * 12
+    assert cache.refresh(only_changed=True) == 0 and cache.refresh(only_changed=False) == 1
+    assert cache.get((a, None, b)).tolist() == [2.0] * 8 + [1.0] * 4
+    assert _DerivedParams.key_of((alias, None, b)) == _DerivedParams.key_of((a, None, b))  # address and dtype
     del a
     gc.collect()
     # `alias` keeps the memory alive at the same address, as a new model's parameter would after the allocator
@@ -504,3 +513,85 @@ def test_derived_parameter_cache_follows_the_life_of_its_parameters():
     d = torch.zeros(5)
     cache.put((d,), 2)
     assert len(cache) == 1 and cache.get((d,)) == 2
+
+
+def test_concatenated_projection_weights_alias_their_parameters():
+    """After the first fused call the query / key / value parameters ARE slices of the fused weight: a write through
+    any route, `param.data.copy_()` included, reaches the fused buffer without a rebuild, and the buffer's address (the
+    one a captured graph replays on) never changes."""
+    from kernl_amd.optimizer.linear import _concatenated_params
+
+    torch.manual_seed(0)
+    lins = [torch.nn.Linear(16, n) for n in (8, 8, 24)]
+    before = [(l.weight.detach().clone(), l.bias.detach().clone()) for l in lins]
+    x = torch.zeros(2, 16)
+    weights, biases = [l.weight for l in lins], [l.bias for l in lins]
+    weight, bias, sizes = _concatenated_params(x, weights, biases)
+    assert sizes == [8, 8, 24] and weight.shape == (40, 16) and bias.shape == (40,)
+    row = 0
+    for l, (w0, b0) in zip(lins, before):
+        assert isinstance(l.weight, torch.nn.Parameter) and l.weight.is_contiguous()
+        assert l.weight.data_ptr() == weight[row].data_ptr() and l.bias.data_ptr() == bias[row:].data_ptr()
+        assert torch.equal(l.weight, w0) and torch.equal(l.bias, b0)   # values survive the move
+        row += l.weight.shape[0]
+    lins[1].weight.data.copy_(torch.full((8, 16), 3.0))                  # not seen by the version counter
+    with torch.no_grad():
+        lins[2].bias.mul_(0.0)
+    again = _concatenated_params(x, weights, biases)
+    assert again[0] is weight and again[1] is bias
+    assert torch.equal(weight[8:16], torch.full((8, 16), 3.0)) and torch.equal(bias[16:], torch.zeros(24))
+    # a state dict loaded into the modules lands in the fused buffers too
+    lins[0].load_state_dict({"weight": torch.ones(8, 16), "bias": torch.ones(8)})
+    assert torch.equal(weight[:8], torch.ones(8, 16)) and torch.equal(bias[:8], torch.ones(8))
+    # no bias on one projection: zeros in its place, the others still alias
+    lin_nb = torch.nn.Linear(16, 8, bias=False)
+    lin_b = torch.nn.Linear(16, 8)
+    w2, b2, _ = _concatenated_params(x, [lin_nb.weight, lin_b.weight], [None, lin_b.bias])
+    assert torch.equal(b2[:8], torch.zeros(8)) and lin_b.bias.data_ptr() == b2[8:].data_ptr()
+
+
+def test_interleaved_gate_weights_are_refreshed_in_place():
+    """The block-interleaved weight of a gated linear unit is a copy: version-counted writes refresh it on the next
+    lookup, other writes through `refresh_fused_parameters()`, always at the same address."""
+    from kernl_amd.implementations.linear_layer import interleave_glu_rows
+    from kernl_amd.optimizer.linear import _interleaved_params, refresh_fused_parameters
+
+    torch.manual_seed(0)
+    gate, value = torch.nn.Linear(16, 64, bias=False), torch.nn.Linear(16, 64, bias=False)
+    weight, bias = _interleaved_params(False, gate.weight, None, value.weight, None)
+    assert bias is None and torch.equal(weight, interleave_glu_rows(gate.weight.detach(), value.weight.detach()))
+    ptr = weight.data_ptr()
+    with torch.no_grad():
+        gate.weight.mul_(2.0)
+    again, _ = _interleaved_params(False, gate.weight, None, value.weight, None)
+    assert again is weight and again.data_ptr() == ptr
+    assert torch.equal(weight, interleave_glu_rows(gate.weight.detach(), value.weight.detach()))
+    value.weight.data.add_(1.0)               # bypasses the version counter
+    stale, _ = _interleaved_params(False, gate.weight, None, value.weight, None)
+    assert not torch.equal(stale, interleave_glu_rows(gate.weight.detach(), value.weight.detach()))
+    assert refresh_fused_parameters() >= 1
+    assert weight.data_ptr() == ptr
+    assert torch.equal(weight, interleave_glu_rows(gate.weight.detach(), value.weight.detach()))
+
+
+def test_split_k_dispatch_rule():
+    """Single-query attention goes to the split-K kernel only for what that kernel takes: more than 50 keys
+    (reference: optimizer/attention.py:45), a power-of-two head size from 8 to 256, 16-byte aligned rows and at most
+    65535 rows; everything else stays on the tiled kernel."""
+    from kernl_amd.optimizer.attention import SPLIT_K_MAX_ROWS, takes_split_k_kernel
+
+    def qkv(b, h, m, n, d, dtype=torch.float16):
+        # one batch entry of memory, expanded over the batch: the real shapes without the gigabytes
+        q = torch.zeros((1, h, m, d), dtype=dtype).expand(b, h, m, d)
+        k = torch.zeros((1, h, n, d), dtype=dtype).expand(b, h, n, d)
+        return q, k, k
+
+    assert takes_split_k_kernel(*qkv(2, 4, 1, 51, 64))
+    assert not takes_split_k_kernel(*qkv(2, 4, 1, 50, 64))          # few keys
+    assert not takes_split_k_kernel(*qkv(2, 4, 2, 4096, 64))        # more than one query per row
+    assert not takes_split_k_kernel(*qkv(2, 4, 1, 4096, 80))        # head size not a power of two
+    assert not takes_split_k_kernel(*qkv(2, 4, 1, 4096, 512))       # head size too large
+    assert takes_split_k_kernel(*qkv(2047, 32, 1, 128, 128)) and 2047 * 32 <= SPLIT_K_MAX_ROWS
+    assert not takes_split_k_kernel(*qkv(2048, 32, 1, 128, 128))    # 65536 rows: beyond the kernel's grid
+    q, k, v = qkv(2, 4, 1, 128, 64)
+    assert not takes_split_k_kernel(q[..., 1:], k[..., 1:], v[..., 1:])   # rows no longer 16-byte aligned

@@ -25,7 +25,7 @@ def test_layer_norm_vs_oracle(shape, dtype, close):
     out = layer_norm(x.cuda(), w.cuda(), b.cuda(), eps)
     torch.cuda.synchronize()
     ref = layer_norm_oracle(x, w, b, effective_eps(eps, dtype))
-    close(out, ref, torch.float16 if dtype == torch.float32 else dtype, scale=4.0, what=f"layernorm {shape}")
+    close(out, ref, torch.float16 if dtype == torch.float32 else dtype, scale="magnitude", what=f"layernorm {shape}")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
@@ -37,7 +37,7 @@ def test_rms_norm_vs_oracle(shape, dtype, close):
     w = (1 + 0.1 * torch.randn((shape[1],), generator=gen)).to(dtype)
     out = layer_norm(x.cuda(), w.cuda(), None, 1e-5, use_rms_norm=True)
     torch.cuda.synchronize()
-    close(out, rms_norm_oracle(x, w, effective_eps(1e-5, dtype)), dtype, scale=4.0, what=f"rmsnorm {shape}")
+    close(out, rms_norm_oracle(x, w, effective_eps(1e-5, dtype)), dtype, scale="magnitude", what=f"rmsnorm {shape}")
 
 
 def test_layer_norm_odd_sizes_and_3d(close):
@@ -49,7 +49,7 @@ def test_layer_norm_odd_sizes_and_3d(close):
         out = layer_norm(x.cuda(), w.cuda(), b.cuda(), 1e-12)
         torch.cuda.synchronize()
         assert out.shape == x.shape
-        close(out, layer_norm_oracle(x, w, b, effective_eps(1e-12, torch.float16)), scale=4.0, what=f"layernorm {shape}")
+        close(out, layer_norm_oracle(x, w, b, effective_eps(1e-12, torch.float16)), scale="magnitude", what=f"layernorm {shape}")
 
 
 def test_layer_norm_transposed_input(close):
@@ -63,7 +63,7 @@ def test_layer_norm_transposed_input(close):
     assert xc.stride() == x.stride() and not xc.is_contiguous()
     out = layer_norm(xc, w.cuda(), b.cuda(), 1e-5)
     torch.cuda.synchronize()
-    close(out, layer_norm_oracle(x, w, b, 1.6e-5), scale=4.0, what="layernorm transposed")
+    close(out, layer_norm_oracle(x, w, b, 1.6e-5), scale="magnitude", what="layernorm transposed")
 
 
 def test_layer_norm_config2_full_size(close):
@@ -73,7 +73,7 @@ def test_layer_norm_config2_full_size(close):
     b = (0.1 * torch.randn((768,), generator=gen)).half()
     out = layer_norm(x.cuda(), w.cuda(), b.cuda(), 1e-12)
     torch.cuda.synchronize()
-    close(out, layer_norm_oracle(x, w, b, effective_eps(1e-12, torch.float16)), scale=4.0, what="config 2 layernorm")
+    close(out, layer_norm_oracle(x, w, b, effective_eps(1e-12, torch.float16)), scale="magnitude", what="config 2 layernorm")
     # size-independent properties: with w = 1, b = 0 every output row has mean 0 and mean square 1 - eps·rstd²
     ones, zeros = torch.ones((768,), dtype=torch.float16), torch.zeros((768,), dtype=torch.float16)
     y = layer_norm(x.cuda(), ones.cuda(), zeros.cuda(), 1e-12).float().cpu()
@@ -102,11 +102,11 @@ def test_rows_that_share_a_wave(dtype, n, close):
         tol = torch.float16 if dtype == torch.float32 else dtype
         print(f"case rows={rows} n={n} {dtype}", flush=True)
         out = layer_norm(x.cuda(), w.cuda(), b.cuda(), 1e-5)
-        close(out, layer_norm_oracle(x, w, b, eps), tol, scale=4.0, what=f"layernorm {rows}x{n}")
+        close(out, layer_norm_oracle(x, w, b, eps), tol, scale="magnitude", what=f"layernorm {rows}x{n}")
         out = layer_norm(x.cuda(), w.cuda(), None, 1e-5, use_rms_norm=True)
-        close(out, rms_norm_oracle(x, w, eps), tol, scale=4.0, what=f"rmsnorm {rows}x{n}")
+        close(out, rms_norm_oracle(x, w, eps), tol, scale="magnitude", what=f"rmsnorm {rows}x{n}")
         out = add_layer_norm(x.cuda(), r.cuda(), w.cuda(), b.cuda(), 1e-5)
-        close(out, layer_norm_oracle(x.float() + r.float(), w, b, eps), tol, scale=4.0, what=f"add+layernorm {rows}x{n}")
+        close(out, layer_norm_oracle(x.float() + r.float(), w, b, eps), tol, scale="magnitude", what=f"add+layernorm {rows}x{n}")
         # the saved statistics of every row, those of a lone last row included
         xg, o = x.cuda(), torch.empty((rows, n), dtype=dtype, device="cuda")
         mean = torch.full((rows,), float("nan"), device="cuda")
@@ -129,7 +129,7 @@ def test_add_layer_norm_matches_separate_add(close):
         out = add_layer_norm(x.cuda(), r.cuda(), w.cuda(), b.cuda(), 1e-12)
         torch.cuda.synchronize()
         ref = layer_norm_oracle(x.float() + r.float(), w, b, 1.6e-5)
-        close(out, ref, scale=4.0, what=f"add+layernorm {shape}")
+        close(out, ref, scale="magnitude", what=f"add+layernorm {shape}")
 
 
 def test_layer_norm_rejects_bad_arguments():

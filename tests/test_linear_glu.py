@@ -48,7 +48,7 @@ def test_glu_vs_oracle(shape, activation, bias, dtype, close):
     print(f"case {shape} {activation!r} bias={bias} {dtype}", flush=True)
     out = _run(x, wg, bg, wv, bv, activation)
     assert out.shape == (M, N) and out.dtype == dtype
-    close(out, glu_oracle(x, wg, bg, wv, bv, activation), dtype, scale=4.0, what=f"glu {shape} {activation}")
+    close(out, glu_oracle(x, wg, bg, wv, bv, activation), dtype, scale="magnitude", what=f"glu {shape} {activation}")
 
 
 @pytest.mark.parametrize("tile", [1, 3, 5])
@@ -62,7 +62,7 @@ def test_glu_every_tile_shape(shape, tile, close):
         out = _run(x, wg, bg, wv, bv, "silu")
     finally:
         lib.kernl_linear_force_tile(0)
-    close(out, glu_oracle(x, wg, bg, wv, bv, "silu"), scale=4.0, what=f"glu tile {tile} {shape}")
+    close(out, glu_oracle(x, wg, bg, wv, bv, "silu"), scale="magnitude", what=f"glu tile {tile} {shape}")
 
 
 def test_glu_3d_and_strided_input(close):
@@ -73,11 +73,11 @@ def test_glu_3d_and_strided_input(close):
     out = linear_glu_layer(wide.cuda()[:, :128].view(2, 50, 128), w, None, "silu")  # row stride 256, 3-D
     torch.cuda.synchronize()
     assert out.shape == (2, 50, 64)
-    close(out.view(100, 64), glu_oracle(x, wg, None, wv, None, "silu"), scale=4.0, what="glu strided")
+    close(out.view(100, 64), glu_oracle(x, wg, None, wv, None, "silu"), scale="magnitude", what="glu strided")
     xt = torch.randn((128, 40), generator=torch.Generator().manual_seed(6)).half()
     out = linear_glu_layer(xt.cuda().t(), w, None, "silu")  # feature stride 40: copied to a dense layout first
     torch.cuda.synchronize()
-    close(out, glu_oracle(xt.t(), wg, None, wv, None, "silu"), scale=4.0, what="glu transposed")
+    close(out, glu_oracle(xt.t(), wg, None, wv, None, "silu"), scale="magnitude", what="glu transposed")
 
 
 def test_glu_wrapper_caches_and_falls_back(close):
@@ -87,19 +87,19 @@ def test_glu_wrapper_caches_and_falls_back(close):
     out2 = glu_linear_wrapper(xg, *params, "silu")
     torch.cuda.synchronize()
     assert torch.equal(out1, out2)
-    close(out1, glu_oracle(x, wg, bg, wv, bv, "silu"), scale=4.0, what="glu wrapper")
+    close(out1, glu_oracle(x, wg, bg, wv, bv, "silu"), scale="magnitude", what="glu wrapper")
     # an output width that is no multiple of 32 runs as two linears and a product, with the same result
     x, wg, bg, wv, bv = _case(64, 40, 64, torch.float16, True, seed=8)
     out = glu_linear_wrapper(x.cuda(), wg.cuda(), bg.cuda(), wv.cuda(), bv.cuda(), "silu")
     torch.cuda.synchronize()
-    close(out, glu_oracle(x, wg, bg, wv, bv, "silu"), scale=4.0, what="glu fallback width")
+    close(out, glu_oracle(x, wg, bg, wv, bv, "silu"), scale="magnitude", what="glu fallback width")
     # fp32 parameters with fp16 activations are cast once, as for the plain linear wrapper
     x, wg, _, wv, _ = _case(32, 64, 64, torch.float32, False, seed=9)
     wg_g, wv_g = wg.cuda(), wv.cuda()
     out = glu_linear_wrapper(x.half().cuda(), wg_g, None, wv_g, None, "silu")
     torch.cuda.synchronize()
     assert wg_g.dtype == torch.float16 and out.dtype == torch.float16
-    close(out, glu_oracle(x.half(), wg.half(), None, wv.half(), None, "silu"), scale=4.0, what="glu cast")
+    close(out, glu_oracle(x.half(), wg.half(), None, wv.half(), None, "silu"), scale="magnitude", what="glu cast")
 
 
 def test_glu_llama_7b_prefill_shape(close):
@@ -110,7 +110,7 @@ def test_glu_llama_7b_prefill_shape(close):
     x, wg, _, wv, _ = _case(M, N, K, torch.float16, False, seed=10)
     out = _run(x, wg, None, wv, None, "silu")
     rows = torch.arange(0, M, 41)
-    close(out[rows.cuda()], glu_oracle(x[rows], wg, None, wv, None, "silu"), scale=4.0, what="glu 7b sample")
+    close(out[rows.cuda()], glu_oracle(x[rows], wg, None, wv, None, "silu"), scale="magnitude", what="glu 7b sample")
     doubled = _run(x, wg, None, wv * 2, None, "silu")
     normal = out.abs() >= 2.0 ** -13  # below that fp16 is subnormal and rounding no longer commutes with doubling
     assert torch.equal(doubled[normal], (out * 2)[normal])
@@ -142,7 +142,7 @@ def test_glu_more_tiles_than_compute_units(close):
         out = _run(x, wg, bg, wv, bv, "silu")
     finally:
         lib.kernl_linear_force_tile(0)
-    close(out, glu_oracle(x, wg, bg, wv, bv, "silu"), scale=4.0, what="glu persistent")
+    close(out, glu_oracle(x, wg, bg, wv, bv, "silu"), scale="magnitude", what="glu persistent")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])

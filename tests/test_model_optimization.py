@@ -458,3 +458,60 @@ def test_models_built_one_after_the_other_do_not_share_fused_weights():
         del model
         gc.collect()
         torch.cuda.empty_cache()
+
+
+def test_weight_updates_after_capture_reach_the_fused_weights():
+    """Weights written AFTER the model has been optimized and its hipGraph captured: the fused query/key/value weight
+    aliases its parameters (any write, `param.data.copy_()` included, is seen by the next replay), the interleaved
+    gate/value weight of a gated unit is rewritten in place before a replay when a version-counted write happened,
+    and by `refresh_fused_parameters()` after a write the version counter does not see."""
+    from kernl_amd.model_optimization import optimize_model
+    from kernl_amd.optimizer.linear import refresh_fused_parameters
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q, self.k, self.v = (torch.nn.Linear(256, 256) for _ in range(3))
+            self.gate, self.up = (torch.nn.Linear(256, 512, bias=False) for _ in range(2))
+            self.down = torch.nn.Linear(512, 256, bias=False)
+
+        def forward(self, x):
+            h = self.q(x) + 2.0 * self.k(x) - self.v(x)
+            return self.down(torch.nn.functional.silu(self.gate(h)) * self.up(h))
+
+    torch._dynamo.reset()
+    torch.manual_seed(0)
+    model = Block().eval().half().cuda()
+    twin = Block().eval().half().cuda()          # never optimized: says what the updated weights should give
+    twin.load_state_dict(model.state_dict())
+    x = torch.randn((4, 128, 256), generator=torch.Generator().manual_seed(0)).half().cuda()
+    optimize_model(model)
+
+    def check(what):
+        with torch.inference_mode():
+            out = model(x).float().cpu()
+            expected = twin(x).float().cpu()
+        err = (out - expected).abs().max().item()
+        assert err < 2e-2 * max(1.0, expected.abs().max().item()), f"{what}: replay used stale weights (max abs err {err})"
+
+    with torch.inference_mode():
+        model(x)
+    check("as captured")
+    gen = torch.Generator().manual_seed(1)
+    new_k = (torch.randn((256, 256), generator=gen) * 0.05).half().cuda()
+    for m in (model, twin):
+        m.k.weight.data.copy_(new_k)             # aliased: no version bump needed
+    check("k.weight.data.copy_")
+    new_gate = (torch.randn((512, 256), generator=gen) * 0.05).half().cuda()
+    with torch.no_grad():
+        for m in (model, twin):
+            m.gate.weight.copy_(new_gate)        # version-counted write
+    check("gate.weight.copy_")
+    state = {k: (torch.randn(v.shape, generator=gen) * 0.05).half() for k, v in twin.state_dict().items()}
+    twin.load_state_dict(state)
+    model.load_state_dict(state)
+    check("load_state_dict")
+    for m in (model, twin):
+        m.up.weight.data.mul_(0.5)               # invisible to the version counter
+    assert refresh_fused_parameters() >= 1
+    check("up.weight.data.mul_ + refresh_fused_parameters")

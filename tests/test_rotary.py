@@ -36,7 +36,7 @@ def test_rotary_vs_oracle(shape, dtype, close):
     out = rotary_forward(x.cuda(), cos.cuda(), sin.cuda())
     torch.cuda.synchronize()
     assert out.dtype == dtype and out.stride() == x.stride()
-    close(out, rotary_oracle(x, cos, sin), torch.float16 if dtype == torch.float32 else dtype, scale=2.0, what=f"rotary {shape}")
+    close(out, rotary_oracle(x, cos, sin), torch.float16 if dtype == torch.float32 else dtype, scale="magnitude", what=f"rotary {shape}")
 
 
 @pytest.mark.parametrize("table_dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["t-fp32", "t-fp16", "t-bf16"])
@@ -51,7 +51,7 @@ def test_rotary_table_dtypes_and_per_batch_positions(dtype, table_dtype, close):
     torch.cuda.synchronize()
     out_dtype = torch.result_type(x, cos)
     assert out.dtype == out_dtype
-    close(out, rotary_oracle(x, cos, sin), torch.float16 if out_dtype == torch.float32 else out_dtype, scale=2.0, what="rotary tables")
+    close(out, rotary_oracle(x, cos, sin), torch.float16 if out_dtype == torch.float32 else out_dtype, scale="magnitude", what="rotary tables")
 
 
 def test_rotary_general_tables_and_strides(close):
@@ -67,10 +67,10 @@ def test_rotary_general_tables_and_strides(close):
     sin_b = sin[:1]
     out = rotary_forward(x.cuda(), cos_b.cuda(), sin_b.cuda())
     torch.cuda.synchronize()
-    close(out, rotary_oracle(x, cos_b, sin_b), scale=4.0, what="rotary general")
+    close(out, rotary_oracle(x, cos_b, sin_b), scale="magnitude", what="rotary general")
     out = rotary_forward(x.cuda(), cos.cuda(), sin.cuda().contiguous())
     torch.cuda.synchronize()
-    close(out, rotary_oracle(x, cos, sin), scale=4.0, what="rotary per-batch per-head")
+    close(out, rotary_oracle(x, cos, sin), scale="magnitude", what="rotary per-batch per-head")
 
 
 def test_rotary_round_trip_at_full_size():
