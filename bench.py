@@ -320,6 +320,15 @@ def main():
             extra[f"{label}_cold_frac_of_peak"] = round(work / (cold * 1e-6) / unit_scale / peak, 4)
 
         extra["attention_cold_us"] = round(cold_us(step), 2)
+        # the same problem with one additive value per (query, key): a mask broadcast over heads (fp32), and a
+        # position bias broadcast over the batch, in the model's dtype
+        for label, mshape, mdt in (("attention_mask_b1ss_fp32", (B, 1, S, S), torch.float32),
+                                   ("attention_bias_1hss_fp16", (1, H, S, S), torch.float16)):
+            mm = torch.randn(mshape, generator=gen).to(mdt).to(dev)
+            t = graph_time_ms(lambda: attention_forward(qd, kd, vd, out, 0.125, False, mm))
+            extra[f"{label}_us_graph_replay"] = round(t * 1e3, 2)
+            extra[f"{label}_tflops_graph_replay"] = round(dense_flop / (t * 1e-3) / 1e12, 1)
+            del mm
         measure(lambda: linear_layer(x_up, w_up, b_up, "fast_gelu"), "linear_up_tanh_gelu", lin_flop, 1e12,
                 PEAK_MFMA_F16_TFLOPS)
         measure(lambda: linear_layer(x_dn, w_dn, b_dn, ""), "linear_down", lin_flop, 1e12, PEAK_MFMA_F16_TFLOPS)

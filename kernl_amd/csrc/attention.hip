@@ -45,14 +45,33 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     constexpr int DC = D / 8;                             // 16-byte chunks per K/V row
     constexpr int KI = BN * DC / 256;                     // 1 KB loads per wave for each of K and V
 
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
+    // head size 64 stages matrix masks through LDS: every wave keeps the 32 rows x 64 keys it needs of the current
+    // key tile (8 KB as fp32) in a region of its own
+    constexpr bool MASK_VIA_LDS = (MASK_MODE == MASK_MATRIX && D == 64);
+    constexpr int MASK_WAVE_BYTES = 32 * BN * 4;
+    constexpr int MASK_LDS = MASK_VIA_LDS ? 4 * MASK_WAVE_BYTES : 0;
 
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE + MASK_LDS];
+
+    // Workgroup ids are dealt round-robin to the 8 XCDs.  Normally the query tiles of one (batch, head) share an XCD
+    // and with it the L2 that holds their keys and values; with a matrix mask that is broadcast over heads the
+    // workgroups of one batch entry — all heads — share it, so that the mask, the larger operand, is fetched once.
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int bh = (slot / p.nq_tiles) * 8 + xcd;
-    int qt = slot % p.nq_tiles;
-    if (bh >= p.B * p.H) return;
+    int b, h, qt;
+    if (MASK_MODE == MASK_MATRIX && p.xcd_by_batch) {
+        const int per_batch = p.H * p.nq_tiles;
+        b = (slot / per_batch) * 8 + xcd;
+        h = (slot % per_batch) / p.nq_tiles;
+        qt = slot % p.nq_tiles;
+        if (b >= p.B) return;
+    } else {
+        const int bh = (slot / p.nq_tiles) * 8 + xcd;
+        qt = slot % p.nq_tiles;
+        if (bh >= p.B * p.H) return;
+        b = bh / p.H;
+        h = bh % p.H;
+    }
     if (CAUSAL) qt = p.nq_tiles - 1 - qt;  // longest rows first
-    const int b = bh / p.H, h = bh % p.H;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 31, lh = lane >> 5;
@@ -300,6 +319,70 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     const int m_voff = MATRIX ? (int)((int64_t)min(my_m, M - 1) * p.ms[2] + lh * 4) * m_esize : 0;
     const float clamp_eff = fmaxf(p.clamp, kClampFloor / kLog2eA);  // (-inf -> clamp) * log2(e) stays finite
     u32x4 mreg[MATRIX ? 2 * NBS * 2 : 1];
+    // Routes 3 (fp32) and 4 (16-bit): the wave's 32 mask rows of a key tile travel HBM -> LDS by loads that write LDS
+    // directly, 1 KB per instruction and fully coalesced (a row's 64 keys are 256 or 128 contiguous bytes), and from
+    // there into the lane's registers.  LDS holds row r as 16-byte chunks at r * row_bytes + 16 * (c ^ f(r)), with
+    // f(r) = r % 16 for fp32 rows (16 chunks) and (r / 2) % 8 for 16-bit rows (8 chunks): a lane reads its own row, so
+    // the lanes of a read hit different banks.  Only the wave itself touches its region: program order and the
+    // memory counters are all the synchronisation there is.
+    const uint32_t mlds_base = lds_base + 2 * STAGE + wave * MASK_WAVE_BYTES;
+    const uint64_t maddr = (uint64_t)(uintptr_t)(static_cast<const char *>(p.mask) + (MATRIX ? mask_base * m_esize : 0));
+    const u32x4 mrsrc4 = {(uint32_t)maddr, (uint32_t)(maddr >> 32) & 0xFFFFu,
+                          MATRIX ? (uint32_t)((((int64_t)M - 1) * p.ms[2] + N) * m_esize) : 0u, 0x00020000u};
+    uint32_t mdma[MASK_VIA_LDS ? 8 : 1];
+    if (MASK_VIA_LDS && p.mask_fast == 2) {
+        const int row0 = q0 + wave * 32;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int r, c;
+            if (m_f32) {
+                r = i * 4 + (lane >> 4);
+                c = (lane & 15) ^ (r & 15);
+            } else {
+                r = (i & 3) * 8 + (lane >> 3);
+                c = (lane & 7) ^ ((r >> 1) & 7);
+            }
+            // rows past the last query read the last row again (their results are never stored)
+            mdma[i] = (uint32_t)(((int64_t)min(row0 + r, M - 1) * p.ms[2]) * m_esize + c * 16);
+        }
+    }
+    auto mask_dma = [&](int tile) __attribute__((always_inline)) {
+        const u32x4 mru = {uniform(mrsrc4[0]), uniform(mrsrc4[1]), uniform(mrsrc4[2]), uniform(mrsrc4[3])};
+        const uint32_t soff = uniform((uint32_t)(tile * BN * m_esize));
+        const uint32_t mb = uniform(mlds_base);
+        if (m_f32) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                             :: "s"(mb + i * 1024), "v"(mdma[i]), "s"(mru), "s"(soff) : "memory", "m0");
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                             :: "s"(mb + i * 1024), "v"(mdma[i]), "s"(mru), "s"(soff) : "memory", "m0");
+        }
+    };
+    // LDS -> registers, then (the region being free again) the request for the tile after
+    auto mask_take = [&](auto route_c, int tile_after) __attribute__((always_inline)) {
+        constexpr int ROUTE = decltype(route_c)::value;
+        const unsigned char *mb = smem + 2 * STAGE + wave * MASK_WAVE_BYTES;
+        if (ROUTE == 3) {
+#pragma unroll
+            for (int i = 0; i < NBS * 4; ++i) {
+                const int c = (i >> 2) * 8 + (i & 3) * 2 + lh;
+                mreg[i] = *reinterpret_cast<const u32x4 *>(mb + lr * 256 + ((c ^ (lr & 15)) << 4));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NBS * 4; ++i) {
+                const u32x2 two = *reinterpret_cast<const u32x2 *>(mb + lr * 128 + ((i ^ ((lr >> 1) & 7)) << 4) + lh * 8);
+                mreg[i >> 1][2 * (i & 1)] = two[0];
+                mreg[i >> 1][2 * (i & 1) + 1] = two[1];
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        mask_dma(tile_after);
+    };
     auto mask_issue = [&](auto route_c, int tile) __attribute__((always_inline)) {
         constexpr int ROUTE = decltype(route_c)::value;
         if (ROUTE == 2) {
@@ -324,16 +407,18 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     // one key tile: prefetch the next one into the other stage, scores, online softmax, P·V, publish
     // ROUTE: how a matrix mask is read (0 = element by element, 1 = prefetched 16-bit vectors, 2 = prefetched fp32
     // vectors); a compile-time choice so that the tile body carries no branches for it
-    auto tile_step = [&](auto general_c, auto stage_c, auto route_c) __attribute__((always_inline)) {
+    // EDGE: the tile may hold keys past the last one or beyond the causal diagonal of some row of the workgroup
+    auto tile_step = [&](auto general_c, auto stage_c, auto route_c, auto edge_c) __attribute__((always_inline)) {
         constexpr bool GENERAL = decltype(general_c)::value;
         constexpr int ST = decltype(stage_c)::value;
         constexpr int ROUTE = decltype(route_c)::value;
+        constexpr bool EDGE = decltype(edge_c)::value;
             const int tile = t_cur, tile_next = t_nxt;
         const int n0 = tile * BN;
         // With a prefetched matrix mask the compiler waits for ALL vector-memory loads before it touches the last
         // mask register (it does not know about the loads issued in assembly), so there the next tile is only
         // requested once the mask values have been consumed.
-        constexpr bool LATE_DMA = GENERAL && (MASK_MODE == MASK_MATRIX);
+        constexpr bool LATE_DMA = GENERAL && (MASK_MODE == MASK_MATRIX) && ROUTE < 3;
         if (!LATE_DMA) dma(tile_next, ST ^ 1);
         float bias_next = 0.0f;
         if (GENERAL && tid < BN) bias_next = key_bias(tile_next);
@@ -343,57 +428,81 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         if (!(GENERAL && CAUSAL && n0 > m_wave0 + 31 + p.causal_off)) {
             // ---- Sᵀ = K · Qᵀ, relative to the row's reference
             f32x16 s_acc[NBS];
-            __builtin_amdgcn_s_setprio(2);
+            auto scores = [&]() __attribute__((always_inline)) {
+                __builtin_amdgcn_s_setprio(2);
 #pragma unroll
-            for (int nb = 0; nb < NBS; ++nb) {
+                for (int nb = 0; nb < NBS; ++nb) {
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const vec8 kf = *reinterpret_cast<const vec8 *>(sb + nb * 32 * KROW + k_off[ks]);
-                    s_acc[nb] = mfma32(kf, qf[ks], ks == 0 ? neg_m : s_acc[nb]);  // neg_m stays 0 without REF_IN_MFMA
+                    for (int ks = 0; ks < KS; ++ks) {
+                        const vec8 kf = *reinterpret_cast<const vec8 *>(sb + nb * 32 * KROW + k_off[ks]);
+                        s_acc[nb] = mfma32(kf, qf[ks], ks == 0 ? neg_m : s_acc[nb]);  // neg_m stays 0 without REF_IN_MFMA
+                    }
                 }
-            }
-            __builtin_amdgcn_s_setprio(0);
+                __builtin_amdgcn_s_setprio(0);
+            };
+            scores();
 
             // ---- online softmax on this lane's row; key of s_acc[nb][v] is n0 + 32 nb + 8 (v/4) + 4 lh + (v%4)
             float mx = -INFINITY;
             if (GENERAL) {
                 const float *colbias = reinterpret_cast<const float *>(sb + K_BYTES + V_BYTES);
+                // EXACT: per-key term (-inf past the last key), -inf mask entries replaced by the clamp value, causal
+                // cut.  The short form — prefetched matrix masks on tiles that are no edge — adds the mask value as it
+                // is: an entry of -inf leaves a score of -inf and a probability of exactly 0, which is what the clamped
+                // value gives too unless EVERY key of the row is masked; a row that ends the tile without a finite score
+                // sends the wave through the exact form once more (the key tile is still in LDS).
+                auto masked_scores = [&](auto exact_c) __attribute__((always_inline)) {
+                    constexpr bool EXACT = decltype(exact_c)::value;
 #pragma unroll
-                for (int nb = 0; nb < NBS; ++nb) {
+                    for (int nb = 0; nb < NBS; ++nb) {
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int nl = nb * 32 + g * 8 + lh * 4;  // key index inside the tile
-                        const f32x4 cb = *reinterpret_cast<const f32x4 *>(colbias + nl);
-                        f32x4 mm = {0.0f, 0.0f, 0.0f, 0.0f};
-                        if (MATRIX && ROUTE != 0) {
-                            const int i = nb * 4 + g;
-                            if (ROUTE == 2) {
-                                mm = __builtin_bit_cast(f32x4, mreg[i]);
-                            } else {
-                                typedef T t4 __attribute__((ext_vector_type(4)));
-                                const u32x2 two = {mreg[i >> 1][2 * (i & 1)], mreg[i >> 1][2 * (i & 1) + 1]};
-                                const t4 h4 = __builtin_bit_cast(t4, two);
-#pragma unroll
-                                for (int r = 0; r < 4; ++r) mm[r] = (float)h4[r];
-                            }
-                        }
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            float sv = s_acc[nb][g * 4 + r] + cb[r];
-                            if (!REF_IN_MFMA) sv -= m_i;
-                            if (MATRIX) {
-                                if (ROUTE != 0) {
-                                    sv = fmaf(fmaxf(mm[r], clamp_eff), kLog2eA, sv);
+                        for (int g = 0; g < 4; ++g) {
+                            const int nl = nb * 32 + g * 8 + lh * 4;  // key index inside the tile
+                            f32x4 cb = {0.0f, 0.0f, 0.0f, 0.0f};
+                            if (EXACT) cb = *reinterpret_cast<const f32x4 *>(colbias + nl);
+                            f32x4 mm = {0.0f, 0.0f, 0.0f, 0.0f};
+                            if (MATRIX && ROUTE != 0) {
+                                const int i = nb * 4 + g;
+                                if (ROUTE == 2 || ROUTE == 3) {
+                                    mm = __builtin_bit_cast(f32x4, mreg[i]);
                                 } else {
-                                    const int n = min(n0 + nl + r, N - 1);
-                                    sv += scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_row + n * p.ms[3]), p.clamp);
+                                    typedef T t4 __attribute__((ext_vector_type(4)));
+                                    const u32x2 two = {mreg[i >> 1][2 * (i & 1)], mreg[i >> 1][2 * (i & 1) + 1]};
+                                    const t4 h4 = __builtin_bit_cast(t4, two);
+#pragma unroll
+                                    for (int r = 0; r < 4; ++r) mm[r] = (float)h4[r];
                                 }
                             }
-                            if (CAUSAL && (n0 + nl + r > my_m + p.causal_off)) sv = -INFINITY;
-                            s_acc[nb][g * 4 + r] = sv;
-                            mx = fmaxf(mx, sv);
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                float sv = s_acc[nb][g * 4 + r];
+                                if (EXACT) sv += cb[r];
+                                if (!REF_IN_MFMA) sv -= m_i;
+                                if (MATRIX) {
+                                    if (ROUTE != 0) {
+                                        sv = fmaf(EXACT ? fmaxf(mm[r], clamp_eff) : mm[r], kLog2eA, sv);
+                                    } else {
+                                        const int n = min(n0 + nl + r, N - 1);
+                                        sv += scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_row + n * p.ms[3]), p.clamp);
+                                    }
+                                }
+                                if (EXACT && CAUSAL && (n0 + nl + r > my_m + p.causal_off)) sv = -INFINITY;
+                                s_acc[nb][g * 4 + r] = sv;
+                                mx = fmaxf(mx, sv);
+                            }
                         }
                     }
+                };
+                if (MATRIX && ROUTE != 0 && !EDGE) {
+                    masked_scores(BoolC<false>());
+                    // (written so that a NaN score takes the exact form too)
+                    if (__builtin_amdgcn_ballot_w64(!(halves32_max(mx) > -INFINITY)) != 0) {
+                        scores();
+                        mx = -INFINITY;
+                        masked_scores(BoolC<true>());
+                    }
+                } else {
+                    masked_scores(BoolC<true>());
                 }
             } else {
 #pragma unroll
@@ -485,7 +594,10 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         }
 
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the next tile is in LDS
-        if (GENERAL && MATRIX) mask_issue(route_c, tile_next);
+        if (GENERAL && MATRIX) {
+            if (ROUTE >= 3) mask_take(route_c, min(tile_next + 1, nt - 1));  // matrix masks walk the tiles in order
+            else mask_issue(route_c, tile_next);
+        }
         if (GENERAL && tid < BN)
             *reinterpret_cast<float *>(smem + (ST ^ 1) * STAGE + K_BYTES + V_BYTES + tid * 4) = bias_next;
         __syncthreads();
@@ -503,12 +615,12 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     // clean tiles in pairs over the two stages; an odd one leaves the general tiles starting in stage 1
     int idx = 0;
     for (; idx + 1 < n_clean; idx += 2) {
-        tile_step(BoolC<false>(), IntC<0>(), IntC<0>());
-        tile_step(BoolC<false>(), IntC<1>(), IntC<0>());
+        tile_step(BoolC<false>(), IntC<0>(), IntC<0>(), BoolC<true>());
+        tile_step(BoolC<false>(), IntC<1>(), IntC<0>(), BoolC<true>());
     }
     const bool odd_clean = idx < n_clean;
     if (odd_clean) {
-        tile_step(BoolC<false>(), IntC<0>(), IntC<0>());
+        tile_step(BoolC<false>(), IntC<0>(), IntC<0>(), BoolC<true>());
         ++idx;
     }
     if (idx < nt) {
@@ -518,17 +630,44 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
             __syncthreads();
         }
         auto general_tiles = [&](auto route_c) __attribute__((always_inline)) {
-            if (MATRIX) mask_issue(route_c, t_cur);
-            if (odd_clean) {
-                tile_step(BoolC<true>(), IntC<1>(), route_c);
+            constexpr int ROUTE = decltype(route_c)::value;
+            if (MATRIX && ROUTE >= 3) {
+                mask_dma(t_cur);
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+                mask_take(route_c, t_nxt);
+            } else if (MATRIX) {
+                mask_issue(route_c, t_cur);
+            }
+            // Prefetched matrix masks: the leading tiles that lie entirely before the last key and before the causal
+            // diagonal of the workgroup's first row take the short form of the masking code, in pairs over the two
+            // stages like the clean tiles of the other mask modes (there are no clean tiles with a matrix mask).
+            bool odd = odd_clean;
+            if (MATRIX && ROUTE != 0 && (D == 64 || !CAUSAL)) {  // head size 128, causal: no registers to spare for a second tile body
+                const int n_fast = min(nt, CAUSAL ? min(N / BN, (q0 + p.causal_off + 1) / BN) : N / BN);
+                for (; idx + 1 < n_fast; idx += 2) {
+                    tile_step(BoolC<true>(), IntC<0>(), route_c, BoolC<false>());
+                    tile_step(BoolC<true>(), IntC<1>(), route_c, BoolC<false>());
+                }
+                if (idx < n_fast) {
+                    tile_step(BoolC<true>(), IntC<0>(), route_c, BoolC<false>());
+                    ++idx;
+                    odd = true;
+                }
+            }
+            if (odd && idx < nt) {
+                tile_step(BoolC<true>(), IntC<1>(), route_c, BoolC<true>());
                 ++idx;
             }
             for (; idx < nt; idx += 2) {
-                tile_step(BoolC<true>(), IntC<0>(), route_c);
-                if (idx + 1 < nt) tile_step(BoolC<true>(), IntC<1>(), route_c);
+                tile_step(BoolC<true>(), IntC<0>(), route_c, BoolC<true>());
+                if (idx + 1 < nt) tile_step(BoolC<true>(), IntC<1>(), route_c, BoolC<true>());
             }
+            // the last step's request for another mask tile must have landed before the wave ends
+            if (MATRIX && ROUTE >= 3) __builtin_amdgcn_s_waitcnt(0x0F70);
         };
-        if (MATRIX && m_fast && m_f32) general_tiles(IntC<2>());
+        if (MASK_VIA_LDS && p.mask_fast == 2 && m_f32) general_tiles(IntC<3>());
+        else if (MASK_VIA_LDS && p.mask_fast == 2) general_tiles(IntC<4>());
+        else if (MATRIX && m_fast && m_f32) general_tiles(IntC<2>());
         else if (MATRIX && m_fast) general_tiles(IntC<1>());
         else general_tiles(IntC<0>());
     }
@@ -621,7 +760,7 @@ __global__ void __launch_bounds__(64) attention_scalar_kernel(const AttnParams p
 // ----------------------------------------------------------------------------------------------------
 template <typename T, int D, int WPE>
 static void launch_stream(const AttnParams &p, int mask_mode, bool causal, hipStream_t st) {
-    const int bh_padded = ((p.B * p.H + 7) / 8) * 8;
+    const int bh_padded = (mask_mode == MASK_MATRIX && p.xcd_by_batch) ? ((p.B + 7) / 8) * 8 * p.H : ((p.B * p.H + 7) / 8) * 8;
     dim3 grid((unsigned)(bh_padded * p.nq_tiles)), block(256);
 #define KERNL_ATTN_LAUNCH(MM, C) hipLaunchKernelGGL((attention_stream_kernel<T, D, WPE, MM, C>), grid, block, 0, st, p)
     if (mask_mode == MASK_NONE) {
@@ -702,11 +841,16 @@ static int attention_entry(const void *q, const void *k, const void *v, void *ou
     p.clamp = mask_min_clamp;
     p.nq_tiles = (int)((M + 127) / 128);
     p.mask_fast = 0;
+    p.xcd_by_batch = 0;
     p.causal_off = is_causal != 0 ? (int)start_position : 0;
     if (mask_mode == MASK_MATRIX && (mask_dtype == KERNL_F32 || mask_dtype == dtype)) {
         const int64_t es = mask_dtype == KERNL_F32 ? 4 : 2;
         p.mask_fast = mask_strides[3] == 1 && p.ms[0] % 4 == 0 && p.ms[1] % 4 == 0 && p.ms[2] % 4 == 0 && p.ms[2] > 0 &&
                       aligned16(mask) && ((M - 1) * p.ms[2] + N + 128) * es < (1ll << 31);
+        const int64_t chunk = 16 / es;  // elements per 16 bytes
+        if (p.mask_fast && p.ms[0] % chunk == 0 && p.ms[1] % chunk == 0 && p.ms[2] % chunk == 0) p.mask_fast = 2;
+        // broadcast over heads but not over the batch: the mask outweighs K and V, map workgroups by batch entry
+        p.xcd_by_batch = p.ms[1] == 0 && p.ms[0] != 0 && H > 1;
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool causal = is_causal != 0;
@@ -716,7 +860,7 @@ static int attention_entry(const void *q, const void *k, const void *v, void *ou
     };
     const bool mfma_ok = !g_attention_force_scalar && (D == 64 || D == 128) && sm_scale > 0.0f &&
                          rows_ok(q, q_strides) && rows_ok(k, k_strides) && rows_ok(v, v_strides) &&
-                         rows_ok(out, o_strides) && (int64_t)((B * H + 7) / 8) * 8 * p.nq_tiles < (1ll << 31) &&
+                         rows_ok(out, o_strides) && (int64_t)((B + 7) / 8) * 8 * H * p.nq_tiles < (1ll << 31) &&
                          k_strides[2] > 0 && v_strides[2] > 0 &&  // one head's K / V extent must fit 31-bit byte offsets
                          (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30) &&
                          (mask == nullptr || (mask_strides[3] >= 0 && (N + 128) * mask_strides[3] < (1ll << 30)));

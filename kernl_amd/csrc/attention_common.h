@@ -28,7 +28,9 @@ struct AttnParams {
     float sm_scale;
     float clamp;  // replacement for -inf mask entries
     int nq_tiles;
-    int mask_fast;  // matrix mask rows can be read as aligned 4-element vectors through 32-bit offsets
+    int mask_fast;  // matrix mask rows: 1 = readable as aligned 4-element vectors through 32-bit offsets,
+                    // 2 = 16-byte chunks of a row are aligned too (they can be staged through LDS)
+    int xcd_by_batch;  // workgroups of one batch entry (all heads) share an XCD instead of those of one head
     int causal_off;  // causal: query row m sees keys 0 .. m + causal_off (0: top-left aligned)
 };
 

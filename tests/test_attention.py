@@ -274,3 +274,65 @@ def test_attention_long_key_sequences_with_vector_mask(n_keys, mask_kind, close)
         ref = v.float().mean(dim=-2, keepdim=True).expand(-1, -1, 160, -1)
     out = _run(q, k, v, 0.125, False, mask)
     close(out, ref, torch.float16, what=f"attention {n_keys} keys {mask_kind}")
+
+
+@pytest.mark.parametrize("mask_dtype", ["fp32", "same"], ids=["mask-fp32", "mask-16bit"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize(
+    "layout", ["per_batch", "per_head", "shared", "full", "rows_padded", "with_minus_inf", "cross", "ragged_keys"]
+)
+def test_matrix_masks_of_every_layout(layout, dtype, mask_dtype, close):
+    """One additive value per (query, key): broadcast over heads (a BERT-style extended mask, [B,1,M,N]), over the
+    batch (a T5 position bias, [1,H,M,N]), over both, over neither; rows with padding between them; -inf entries;
+    more keys than queries; key counts that are no multiple of the 64-key tile.  Head size 64 stages these masks
+    through LDS, 16 bytes at a time, so fp32 and 16-bit masks take different routes."""
+    B, H, M, N, D = 3, 5, 200, 200, 64
+    if layout == "cross":
+        M, N = 130, 328
+    if layout == "ragged_keys":
+        M, N = 128, 456          # 456 = 7 * 64 + 8: the last tile has one 16-byte chunk of 16-bit values
+    gen = torch.Generator().manual_seed(17)
+    q = _mk((B, H, M, D), dtype, gen)
+    k, v = _mk((B, H, N, D), dtype, gen), _mk((B, H, N, D), dtype, gen)
+    mdt = torch.float32 if mask_dtype == "fp32" else dtype
+    mshape = {"per_batch": (B, 1, M, N), "per_head": (1, H, M, N), "shared": (1, 1, M, N)}.get(layout, (B, H, M, N))
+    mask = (torch.randn(mshape, generator=gen) * 2.0).to(mdt)
+    if layout == "with_minus_inf":
+        mask = mask.float().masked_fill(torch.rand(mshape, generator=gen) < 0.3, float("-inf")).to(mdt)
+        mask[..., 0] = 0.0       # no fully masked row
+    mask_gpu = mask.cuda()
+    if layout == "rows_padded":  # rows 16-byte aligned but not back to back
+        wide = torch.zeros(mshape[:3] + (N + 24,), dtype=mdt, device="cuda")
+        wide[..., :N] = mask_gpu
+        mask_gpu = wide[..., :N]
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    out = torch.empty_like(qc)
+    print(f"case layout={layout} dtype={dtype} mask={mdt} mask shape={tuple(mask_gpu.shape)} strides={mask_gpu.stride()}", flush=True)
+    attention_forward(qc, kc, vc, out, 0.2, is_causal=False, attention_mask=mask_gpu)
+    torch.cuda.synchronize()
+    close(out, attention_oracle(q, k, v, 0.2, False, mask.float()), dtype, what=f"matrix mask {layout}")
+
+
+def test_matrix_mask_config1_size_properties(close):
+    """[32,12,512,64] with a [32,1,512,512] fp32 mask (workgroups mapped to XCDs by batch entry) and with a
+    [1,12,512,512] bias: a sample of rows against the oracle, and — size independent — a mask that is constant along
+    the keys of every row changes nothing."""
+    B, H, S, D = 32, 12, 512, 64
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    q, k, v = (torch.randn((B, H, S, D), generator=gen, device="cuda", dtype=torch.half) for _ in range(3))
+    plain = torch.empty_like(q)
+    attention_forward(q, k, v, plain, 0.125, is_causal=False, attention_mask=None)
+    for mshape in ((B, 1, S, S), (1, H, S, S)):
+        mask = torch.randn(mshape, generator=gen, device="cuda")
+        out = torch.empty_like(q)
+        attention_forward(q, k, v, out, 0.125, is_causal=False, attention_mask=mask)
+        row_constant = mask[..., :1].expand(mshape).contiguous()
+        same = torch.empty_like(q)
+        attention_forward(q, k, v, same, 0.125, is_causal=False, attention_mask=row_constant)
+        torch.cuda.synchronize()
+        assert (same.float() - plain.float()).abs().max().item() <= 2e-3, f"row-constant mask {mshape} changed the result"
+        for b, h in ((0, 0), (B - 1, H - 1), (13, 7)):
+            mb, mh = (b if mshape[0] > 1 else 0), (h if mshape[1] > 1 else 0)
+            ref = attention_oracle(q[b:b + 1, h:h + 1].cpu(), k[b:b + 1, h:h + 1].cpu(), v[b:b + 1, h:h + 1].cpu(), 0.125, False,
+                                   mask[mb:mb + 1, mh:mh + 1].cpu())
+            close(out[b:b + 1, h:h + 1], ref, torch.float16, what=f"matrix mask {mshape} at batch {b} head {h}")
