@@ -193,9 +193,10 @@ int kernl_linear_fwd(const void *x, const void *w, const void *bias, void *out, 
  * kernl_linear_fwd for a weight stored as one byte per element, fp8 e5m2 — the upper byte of the fp16 encoding
  * (reference: `get_model_fp8` turns the weights of the projections into int8 tensors holding float8e5,
  * experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84, and its kernels widen them on load,
- * fused_kernel_ff.py:43-47).  w8 [N, K] contiguous bytes.  This is the decoding-step kernel only: M <= 64,
- * K % 64 == 0, dtype KERNL_F16 (x, bias, out, act_in); anything else returns KERNL_ERR_UNSUPPORTED and the caller
- * widens the weight.  Half the bytes of the weight stream, fp32 accumulation of the decoded values.
+ * fused_kernel_ff.py:43-47).  w8 [N, K] contiguous bytes, K % 8 == 0, dtype KERNL_F16 (x, bias, out, act_in);
+ * anything else returns KERNL_ERR_UNSUPPORTED.  Up to 64 rows of x (with K % 64 == 0) the weight is streamed once by
+ * every CU; larger inputs take a tiled MFMA kernel that fetches the bytes and widens them on their way into LDS.
+ * Half the bytes of the weight either way, fp32 accumulation of the decoded values.
  */
 int kernl_linear_w8_fwd(const void *x, const void *w8, const void *bias, void *out, void *act_in,
                         int64_t M, int64_t N, int64_t K, const int64_t x_strides[2],

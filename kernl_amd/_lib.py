@@ -258,10 +258,11 @@ def linear_fwd(x2d, weight, bias, out2d, act_in2d, activation: int) -> None:
 
 
 def linear_w8_supported(x2d, weight8) -> bool:
-    """What `kernl_linear_w8_fwd` takes: fp16 rows, at most 64 of them, K a multiple of 64."""
+    """What `kernl_linear_w8_fwd` takes: fp16 rows with unit feature stride, 16-byte aligned, K a multiple of 8."""
     M, K = x2d.shape
     return (
-        x2d.dtype == torch.float16 and M <= 64 and K % 64 == 0 and x2d.stride(1) == 1 and x2d.stride(0) % 8 == 0
+        x2d.dtype == torch.float16 and K % 8 == 0 and K < (1 << 22) and x2d.stride(1) == 1 and x2d.stride(0) % 8 == 0
+        and x2d.stride(0) < (1 << 22)
         and x2d.data_ptr() % 16 == 0 and weight8.is_contiguous() and weight8.data_ptr() % 16 == 0
     )
 

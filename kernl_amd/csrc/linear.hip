@@ -262,7 +262,10 @@ struct LinearTile {
     static constexpr int GROUP_M = 4;  // m-tiles walked together so one XCD's L2 sees a compact block
 };
 
-template <typename T, typename Cfg, int ACT>
+// W8: the weight is stored as one byte per element (fp8 e5m2, the upper byte of the fp16 encoding); a thread fetches
+// 8 bytes where it would fetch a 16-byte chunk and widens them on the way into LDS, so everything after the LDS
+// store is the 16-bit kernel.
+template <typename T, typename Cfg, int ACT, bool W8 = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_BLOCKS)
 linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
                    T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx,
@@ -302,8 +305,10 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     const int rows_x = min(BM, M - m0), rows_w = min(BN, N - n0);
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<T *>(X + (int64_t)m0 * ldx), 0, (int)((((int64_t)rows_x - 1) * ldx + K) * 2), 0x00020000);
+    constexpr int WB = W8 ? 1 : 2;  // bytes per weight element in memory
     const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<T *>(W + (int64_t)n0 * K), 0, (int)((int64_t)rows_w * K * 2), 0x00020000);
+        const_cast<char *>(reinterpret_cast<const char *>(W) + (int64_t)n0 * K * WB), 0, (int)((int64_t)rows_w * K * WB),
+        0x00020000);
     uint32_t xg[Cfg::XI], wg[Cfg::WI];  // byte offsets from the tile origins
     int xl[Cfg::XI], wl[Cfg::WI];       // LDS byte offsets inside a stage
 #pragma unroll
@@ -319,7 +324,7 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         const int row = q / CPR, c = q % CPR;
         // LDS row `row` feeds MFMA row (row % 32) of its 32-block and carries weight row rowperm16(row % 32).
         const int wrow = (row & ~31) + rowperm16(row & 31);
-        wg[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) : kOutOfRange;
+        wg[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * WB) : kOutOfRange;
         wl[i] = Cfg::X_BYTES + swz_offset<RB>(row, c);
     }
     const int kchunk = (tid % CPR) * 8;  // same for every i because THREADS % CPR == 0
@@ -345,9 +350,17 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
                     vec8, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, inside ? xg[i] : kOutOfRange, k0 * 2, 0));
 #pragma unroll
         for (int i = 0; i < Cfg::WI; ++i)
-            if (i % KSTEPS == part)
-                ws[i] = __builtin_bit_cast(
-                    vec8, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, inside ? wg[i] : kOutOfRange, k0 * 2, 0));
+            if (i % KSTEPS == part) {
+                if constexpr (W8) {
+                    const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(wrsrc, inside ? wg[i] : kOutOfRange, k0, 0);
+                    const u32x4 wide = {__builtin_amdgcn_perm(0u, raw[0], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[0], 0x030c020cu),
+                                        __builtin_amdgcn_perm(0u, raw[1], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[1], 0x030c020cu)};
+                    ws[i] = __builtin_bit_cast(vec8, wide);
+                } else {
+                    ws[i] = __builtin_bit_cast(
+                        vec8, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, inside ? wg[i] : kOutOfRange, k0 * 2, 0));
+                }
+            }
     };
     auto lstore_part = [&](int stage, int part) {
         unsigned char *base = smem + stage * Cfg::STAGE_BYTES;
@@ -1222,9 +1235,9 @@ struct LinearArgs {
     hipStream_t st;
 };
 
-template <typename T, typename Cfg, int ACT>
+template <typename T, typename Cfg, int ACT, bool W8 = false>
 static void launch_mfma_act(const LinearArgs &a) {
-    auto kern = linear_mfma_kernel<T, Cfg, ACT>;
+    auto kern = linear_mfma_kernel<T, Cfg, ACT, W8>;
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -1255,6 +1268,19 @@ static void launch_mfma_cfg(const LinearArgs &a) {
         case KERNL_ACT_GELU_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_TANH>(a); break;
         case KERNL_ACT_SILU: launch_mfma_act<T, Cfg, KERNL_ACT_SILU>(a); break;
         default: launch_mfma_act<T, Cfg, KERNL_ACT_NONE>(a); break;
+    }
+}
+
+// one-byte weights (fp16 activations)
+template <typename Cfg>
+static void launch_mfma_w8(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_mfma_act<f16, Cfg, KERNL_ACT_RELU, true>(a); break;
+        case KERNL_ACT_TANH: launch_mfma_act<f16, Cfg, KERNL_ACT_TANH, true>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_mfma_act<f16, Cfg, KERNL_ACT_GELU_ERF, true>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_mfma_act<f16, Cfg, KERNL_ACT_GELU_TANH, true>(a); break;
+        case KERNL_ACT_SILU: launch_mfma_act<f16, Cfg, KERNL_ACT_SILU, true>(a); break;
+        default: launch_mfma_act<f16, Cfg, KERNL_ACT_NONE, true>(a); break;
     }
 }
 
@@ -1626,9 +1652,10 @@ extern "C" int kernl_linear_w8_fwd(const void *x, const void *w8, const void *bi
         return set_error(KERNL_ERR_INVALID_ARG, "linear (fp8 weight): unknown activation %d", activation);
     if (dtype != KERNL_F16)
         return set_error(KERNL_ERR_UNSUPPORTED, "linear (fp8 weight): activations must be f16, got dtype %d", dtype);
-    if (M > 64 || K % 64 != 0 || N > INT32_MAX || K > INT32_MAX)
-        return set_error(KERNL_ERR_UNSUPPORTED, "linear (fp8 weight): at most 64 rows of x and K a multiple of 64 "
-                         "(M=%lld K=%lld); widen the weight for larger inputs", (long long)M, (long long)K);
+    if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || K >= (1 << 22) || x_strides[0] >= (1 << 22))
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear (fp8 weight): sizes too large");
+    if (K % 8 != 0)
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear (fp8 weight): K must be a multiple of 8 (K=%lld)", (long long)K);
     if (x_strides[1] != 1 || x_strides[0] % 8 != 0 || !aligned16(x) || !aligned16(w8))
         return set_error(KERNL_ERR_UNSUPPORTED, "linear (fp8 weight): x needs unit feature stride and 16-byte aligned "
                          "rows, the weight a 16-byte aligned base");
@@ -1641,8 +1668,16 @@ extern "C" int kernl_linear_w8_fwd(const void *x, const void *w8, const void *bi
     a.ai_rs = act_in ? act_in_strides[0] : 0; a.ai_cs = act_in ? act_in_strides[1] : 0;
     a.act = activation;
     a.st = static_cast<hipStream_t>(stream);
-    launch_skinny<f16, false, true>(a);
-    return check_launch("linear (skinny, fp8 weight)");
+    // few rows of x: the kernel that streams the weight once with every CU; otherwise the tiled MFMA kernel, which
+    // widens the bytes on their way into LDS
+    if (M <= 64 && K % 64 == 0) {
+        launch_skinny<f16, false, true>(a);
+        return check_launch("linear (skinny, fp8 weight)");
+    }
+    const int ctas_big = (int)(((M + 255) / 256) * ((N + 255) / 256));
+    if (ctas_big >= 192) launch_mfma_w8<Tile256x256>(a);
+    else launch_mfma_w8<Tile128x128>(a);
+    return check_launch("linear (mfma, fp8 weight)");
 }
 
 extern "C" int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float eps, const void *w, const void *bias,

@@ -41,7 +41,8 @@ class LinearLayer(torch.autograd.Function):
 
         if weight.dtype in ONE_BYTE_WEIGHT_DTYPES:
             # fp8 e5m2 weight storage (reference: experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84): decoding
-            # steps stream the bytes; larger inputs widen the weight first and take the ordinary kernels
+            # steps stream the bytes, larger inputs take a tiled kernel that widens them on their way into LDS; only
+            # a K that is no multiple of 8 widens the whole weight first
             assert x.dtype == torch.float16, f"fp8 weights go with float16 activations, got {x.dtype}"
             assert weight.is_contiguous() and x_.shape[1] == weight.shape[1]
             if x_.stride(-1) != 1 or x_.stride(0) % 8 != 0 or x_.data_ptr() % 16 != 0:

@@ -147,11 +147,13 @@ def test_linear_few_rows_streams_the_weight(shape, activation, dtype, close):
 
 @pytest.mark.parametrize("activation", ["", "silu"])
 @pytest.mark.parametrize("shape", [(1, 4096, 4096), (5, 80, 64), (16, 1000, 192), (33, 9000, 192), (64, 512, 1024),
-                                   (100, 256, 128), (4, 96, 72)], ids=lambda s: "x".join(map(str, s)))
+                                   (100, 256, 128), (4, 96, 72), (65, 200, 136), (300, 1000, 328), (2048, 2304, 768),
+                                   (1024, 4096, 1024), (7, 64, 100)], ids=lambda s: "x".join(map(str, s)))
 def test_linear_fp8_weight_storage(shape, activation, close):
     """Weight stored as fp8 e5m2 (reference: `get_model_fp8`, experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84):
-    the result must be the oracle's on the DECODED weight.  Up to 64 rows and K % 64 == 0 stream the bytes; 100 rows
-    and K = 72 go through the widened weight."""
+    the result must be the oracle's on the DECODED weight.  Up to 64 rows with K % 64 == 0 stream the bytes; more rows,
+    or another K that is a multiple of 8, take the tiled kernel that widens the bytes into LDS (both of its tile
+    shapes are in the list, with ragged edges in every dimension); K = 100 goes through a widened copy."""
     from oracle import e5m2_decode_oracle
 
     M, N, K = shape
