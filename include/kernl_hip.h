@@ -92,6 +92,24 @@ int kernl_attention_cached_fwd(const void *q, const void *k, const void *v, void
                                void *stream);
 
 /*
+ * kernl_attention_fwd / kernl_attention_cached_fwd over keys and values stored as one byte per element, fp8 e5m2 — the
+ * upper byte of the fp16 encoding (reference: `get_model_fp8` turns `cache_k` / `cache_v` into int8 tensors holding
+ * float8e5, experimental/llama-v2/kernel/fused_kernel_fp8.py:68-74, and the attention kernel widens them on load,
+ * fused_kernel_attention.py:66-70, :90-94).  k8, v8: bytes, strides in elements (= bytes); q, out, dtype: KERNL_F16
+ * only; head size 64 or 128, unit feature strides, the other strides multiples of 8, 16-byte aligned bases; no mask or
+ * a per-key mask ([B|1, H|1, 1, N]); with is_causal, query row m sees keys 0 .. m + start_position (ignored
+ * otherwise).  Anything else returns KERNL_ERR_UNSUPPORTED.  Scores, softmax and accumulation as kernl_attention_fwd on
+ * the decoded values.
+ */
+int kernl_attention_kv8_fwd(const void *q, const void *k8, const void *v8, void *out, const void *mask,
+                            int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
+                            const int64_t q_strides[4], const int64_t k_strides[4],
+                            const int64_t v_strides[4], const int64_t o_strides[4],
+                            const int64_t mask_sizes[4], const int64_t mask_strides[4], int mask_dtype,
+                            float sm_scale, int is_causal, int64_t start_position, float mask_min_clamp,
+                            int dtype, void *stream);
+
+/*
  * Split-K attention for very few query rows (decoding: q_len = 1 against a long key sequence).  Same arguments and
  * semantics as kernl_attention_fwd plus a workspace; the keys of every (batch, head, query row) are split into
  * ranges that run in parallel and are merged by a second kernel.  Replaces the `_fwd_part_1[grid]` /

@@ -26,6 +26,7 @@ EXPORTED_SYMBOLS = (
     "kernl_attention_skinny_workspace_bytes",
     "kernl_attention_skinny_fwd",
     "kernl_attention_skinny_kv8_fwd",
+    "kernl_attention_kv8_fwd",
     "kernl_attention_skinny_static_max_bytes",
     "kernl_attention_skinny_static_fwd",
     "kernl_rope_fwd",
@@ -74,6 +75,11 @@ def load() -> ctypes.CDLL:
     lib.kernl_attention_cached_fwd.restype = ctypes.c_int
     lib.kernl_attention_cached_fwd.argtypes = (
         [_vp] * 5 + [_i64] * 5 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, _i64, ctypes.c_float, ctypes.c_int, _vp]
+    )
+    lib.kernl_attention_kv8_fwd.restype = ctypes.c_int
+    lib.kernl_attention_kv8_fwd.argtypes = (
+        [_vp] * 5 + [_i64] * 5 + [_i64p] * 6
+        + [ctypes.c_int, ctypes.c_float, ctypes.c_int, _i64, ctypes.c_float, ctypes.c_int, _vp]
     )
     lib.kernl_attention_skinny_workspace_bytes.restype = _i64
     lib.kernl_attention_skinny_workspace_bytes.argtypes = [_i64] * 5
@@ -176,6 +182,27 @@ def attention_cached_fwd(q, k, v, out, mask, sm_scale: float, start_position: in
             float(sm_scale), int(start_position), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
         )
     _check(st, "kernl_attention_cached_fwd")
+
+
+def attention_kv8_fwd(q, k8, v8, out, mask, sm_scale: float, is_causal: bool, start_position: int, mask_min_clamp: float) -> None:
+    """k8, v8 [B, H, N, D]: fp8 e5m2 bytes (int8 / uint8 / float8_e5m2); q and out fp16."""
+    _require_gpu(q, k8, v8, out, mask)
+    B, H, M, D = q.shape
+    N = k8.shape[2]
+    lib = load()
+    if mask is not None:
+        msizes, mstrides, mdtype, mptr = _arr(mask.shape), _arr(mask.stride()), DTYPE_CODE[mask.dtype], mask.data_ptr()
+    else:
+        msizes, mstrides, mdtype, mptr = None, None, KERNL_F32, None
+    with torch.cuda.device(q.device):
+        st = lib.kernl_attention_kv8_fwd(
+            q.data_ptr(), k8.data_ptr(), v8.data_ptr(), out.data_ptr(), mptr,
+            B, H, M, N, D,
+            _arr(q.stride()), _arr(k8.stride()), _arr(v8.stride()), _arr(out.stride()),
+            msizes, mstrides, mdtype,
+            float(sm_scale), int(bool(is_causal)), int(start_position), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
+        )
+    _check(st, "kernl_attention_kv8_fwd")
 
 
 def attention_skinny_workspace_bytes(B: int, H: int, M: int, N: int, D: int) -> int:

@@ -30,7 +30,11 @@ namespace kernl {
 // is unrolled over the two LDS stages; the others (ragged last tile, masked, causal diagonal) follow in a general
 // body.  The order of key tiles does not matter to the online softmax.
 // ----------------------------------------------------------------------------------------------------
-template <typename T, int D, int WPE, int MASK_MODE, bool CAUSAL>
+// KV8: keys and values are stored as one byte per element (fp8 e5m2, the upper byte of the fp16 encoding).  Their
+// tiles cannot be written to LDS by the load itself then: a thread fetches the 8 bytes of each of its 16-byte LDS
+// chunks into registers while the current tile is processed, widens them and stores them before the barrier that
+// publishes the stage.  Everything that reads LDS is the 16-bit kernel.
+template <typename T, int D, int WPE, int MASK_MODE, bool CAUSAL, bool KV8 = false>
 __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnParams p) {
     typedef typename Vec8<T>::type vec8;
     typedef __attribute__((address_space(3))) void lds_void;
@@ -81,8 +85,9 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     const int M = p.M, N = p.N;
 
     const T *qp = static_cast<const T *>(p.q) + b * p.qs[0] + h * p.qs[1];
-    const T *kp = static_cast<const T *>(p.k) + b * p.ks[0] + h * p.ks[1];
-    const T *vp = static_cast<const T *>(p.v) + b * p.vs[0] + h * p.vs[1];
+    constexpr int KVB = KV8 ? 1 : 2;  // bytes per key / value element in memory
+    const char *kp = static_cast<const char *>(p.k) + (b * p.ks[0] + h * p.ks[1]) * KVB;
+    const char *vp = static_cast<const char *>(p.v) + (b * p.vs[0] + h * p.vs[1]) * KVB;
     T *op = static_cast<T *>(p.o) + b * p.os[0] + h * p.os[1];
     const int64_t mask_base = (MASK_MODE != MASK_NONE) ? b * p.ms[0] + h * p.ms[1] : 0;
 
@@ -110,23 +115,37 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     for (int i = 0; i < KI; ++i) {
         const int qd = tid + 256 * i;
         const int row = qd / DC, cs = qd % DC;
-        kdma[i] = (uint32_t)(((int64_t)row * p.ks[2] + swz_chunk<KROW>(row, cs) * 8) * 2);
+        kdma[i] = (uint32_t)(((int64_t)row * p.ks[2] + swz_chunk<KROW>(row, cs) * 8) * KVB);
         const int vsw = (D == 64) ? ((row >> 1) & 1) : (row & 3);
-        vdma[i] = (uint32_t)(((int64_t)row * p.vs[2] + (cs ^ (vsw << 2)) * 8) * 2);
+        vdma[i] = (uint32_t)(((int64_t)row * p.vs[2] + (cs ^ (vsw << 2)) * 8) * KVB);
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
     const uint32_t dma_base = lds_base + wave * 1024;
     const uint64_t kaddr = (uint64_t)(uintptr_t)kp, vaddr = (uint64_t)(uintptr_t)vp;
     const u32x4 krsrc = {(uint32_t)kaddr, (uint32_t)(kaddr >> 32) & 0xFFFFu,
-                         (uint32_t)((((int64_t)N - 1) * p.ks[2] + D) * 2), 0x00020000u};
+                         (uint32_t)((((int64_t)N - 1) * p.ks[2] + D) * KVB), 0x00020000u};
     const u32x4 vrsrc = {(uint32_t)vaddr, (uint32_t)(vaddr >> 32) & 0xFFFFu,
-                         (uint32_t)((((int64_t)N - 1) * p.vs[2] + D) * 2), 0x00020000u};
-    const int k_tile_bytes = (int)((int64_t)BN * p.ks[2] * 2), v_tile_bytes = (int)((int64_t)BN * p.vs[2] * 2);
+                         (uint32_t)((((int64_t)N - 1) * p.vs[2] + D) * KVB), 0x00020000u};
+    const int k_tile_bytes = (int)((int64_t)BN * p.ks[2] * KVB), v_tile_bytes = (int)((int64_t)BN * p.vs[2] * KVB);
+    // one-byte keys and values: ordinary buffer loads into registers (the compiler tracks them), committed to LDS later
+    const __amdgpu_buffer_rsrc_t krsrc8 = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char *>(kp), 0, KV8 ? (int)((((int64_t)N - 1) * p.ks[2] + D) * KVB) : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc8 = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char *>(vp), 0, KV8 ? (int)((((int64_t)N - 1) * p.vs[2] + D) * KVB) : 0, 0x00020000);
+    u32x2 kraw[KV8 ? KI : 1], vraw[KV8 ? KI : 1];
     // Inline assembly on purpose: the compiler, seeing LDS written by a load, would make every later LDS read
     // wait for the vector-memory counter, i.e. for the prefetch itself.  The explicit wait before the barrier
     // that publishes the stage is the one that matters.
     auto uniform = [](uint32_t x) __attribute__((always_inline)) -> uint32_t { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); };
     auto dma = [&](int tile, int stage) __attribute__((always_inline)) {
+        if constexpr (KV8) {
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+                kraw[i] = __builtin_amdgcn_raw_buffer_load_b64(krsrc8, kdma[i], tile * k_tile_bytes, 0);
+                vraw[i] = __builtin_amdgcn_raw_buffer_load_b64(vrsrc8, vdma[i], tile * v_tile_bytes, 0);
+            }
+            return;
+        }
         // every operand below is wave-uniform; saying so explicitly keeps them in scalar registers whatever the
         // control flow around the call looks like to the compiler
         const uint32_t k_soff = uniform((uint32_t)(tile * k_tile_bytes)), v_soff = uniform((uint32_t)(tile * v_tile_bytes));
@@ -141,6 +160,22 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         for (int i = 0; i < KI; ++i)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                          :: "s"(sb + K_BYTES + i * 4096), "v"(vdma[i]), "s"(vr), "s"(v_soff) : "memory", "m0");
+    };
+    // one-byte keys and values: the fetched bytes, widened (byte b of a dword becomes the 16-bit value b << 8), go to
+    // the LDS positions the direct loads of the 16-bit kernel would have written
+    auto kv8_commit = [&](int stage) __attribute__((always_inline)) {
+        if constexpr (KV8) {
+            unsigned char *sbase = smem + stage * STAGE + tid * 16;
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+                const u32x4 kw = {__builtin_amdgcn_perm(0u, kraw[i][0], 0x010c000cu), __builtin_amdgcn_perm(0u, kraw[i][0], 0x030c020cu),
+                                  __builtin_amdgcn_perm(0u, kraw[i][1], 0x010c000cu), __builtin_amdgcn_perm(0u, kraw[i][1], 0x030c020cu)};
+                const u32x4 vw = {__builtin_amdgcn_perm(0u, vraw[i][0], 0x010c000cu), __builtin_amdgcn_perm(0u, vraw[i][0], 0x030c020cu),
+                                  __builtin_amdgcn_perm(0u, vraw[i][1], 0x010c000cu), __builtin_amdgcn_perm(0u, vraw[i][1], 0x030c020cu)};
+                *reinterpret_cast<u32x4 *>(sbase + i * 4096) = kw;
+                *reinterpret_cast<u32x4 *>(sbase + K_BYTES + i * 4096) = vw;
+            }
+        }
     };
     // per-key additive term of a general tile (mask value in the log2 domain, -inf past the last key); thread tid
     // < 64 owns key tid of the tile
@@ -594,6 +629,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         }
 
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the next tile is in LDS
+        kv8_commit(ST ^ 1);
         if (GENERAL && MATRIX) {
             if (ROUTE >= 3) mask_take(route_c, min(tile_next + 1, nt - 1));  // matrix masks walk the tiles in order
             else mask_issue(route_c, tile_next);
@@ -608,6 +644,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     if (nt > 0) {
         if (t_cur != 0) dma(t_cur, 0);
         if (n_clean == 0 && tid < BN) *reinterpret_cast<float *>(smem + K_BYTES + V_BYTES + tid * 4) = key_bias(t_cur);
+        kv8_commit(0);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far (Q fragments included) has landed
     __syncthreads();
@@ -776,6 +813,22 @@ static void launch_stream(const AttnParams &p, int mask_mode, bool causal, hipSt
 #undef KERNL_ATTN_LAUNCH
 }
 
+// one-byte keys and values: fp16 queries, no mask or a per-key mask
+template <int D>
+static void launch_stream_kv8(const AttnParams &p, int mask_mode, bool causal, hipStream_t st) {
+    const int bh_padded = ((p.B * p.H + 7) / 8) * 8;
+    dim3 grid((unsigned)(bh_padded * p.nq_tiles)), block(256);
+#define KERNL_ATTN_LAUNCH8(MM, C) hipLaunchKernelGGL((attention_stream_kernel<f16, D, 2, MM, C, true>), grid, block, 0, st, p)
+    if (mask_mode == MASK_NONE) {
+        if (causal) KERNL_ATTN_LAUNCH8(MASK_NONE, true);
+        else KERNL_ATTN_LAUNCH8(MASK_NONE, false);
+    } else {
+        if (causal) KERNL_ATTN_LAUNCH8(MASK_VECTOR, true);
+        else KERNL_ATTN_LAUNCH8(MASK_VECTOR, false);
+    }
+#undef KERNL_ATTN_LAUNCH8
+}
+
 int g_attention_force_scalar = 0;  // test hook: route everything through the scalar kernel
 int g_attention_variant = 0;       // tuning hook: register budget (waves per SIMD) of the head-size-64 MFMA kernel
 
@@ -790,7 +843,7 @@ static int attention_entry(const void *q, const void *k, const void *v, void *ou
                            const int64_t v_strides[4], const int64_t o_strides[4],
                            const int64_t mask_sizes[4], const int64_t mask_strides[4], int mask_dtype,
                            float sm_scale, int is_causal, int64_t start_position, float mask_min_clamp, int dtype,
-                           void *stream) {
+                           void *stream, bool kv8 = false) {
     using namespace kernl;
     if (start_position < 0 || start_position > (1 << 24))
         return set_error(KERNL_ERR_INVALID_ARG, "attention: start_position %lld out of range", (long long)start_position);
@@ -864,6 +917,19 @@ static int attention_entry(const void *q, const void *k, const void *v, void *ou
                          k_strides[2] > 0 && v_strides[2] > 0 &&  // one head's K / V extent must fit 31-bit byte offsets
                          (N + 128) * k_strides[2] < (1ll << 30) && (N + 128) * v_strides[2] < (1ll << 30) &&
                          (mask == nullptr || (mask_strides[3] >= 0 && (N + 128) * mask_strides[3] < (1ll << 30)));
+    if (kv8) {
+        // one-byte keys and values only exist on the MFMA kernel: no scalar route, no matrix masks
+        if (dtype != KERNL_F16)
+            return set_error(KERNL_ERR_UNSUPPORTED, "attention (fp8 keys/values): queries and output must be f16, got dtype %d", dtype);
+        if (mask_mode == MASK_MATRIX)
+            return set_error(KERNL_ERR_UNSUPPORTED, "attention (fp8 keys/values): only per-key masks are supported");
+        if (!mfma_ok)
+            return set_error(KERNL_ERR_UNSUPPORTED, "attention (fp8 keys/values): head size 64 or 128, unit feature strides, "
+                             "strides that are multiples of 8 and 16-byte aligned bases are required");
+        if (D == 64) launch_stream_kv8<64>(p, mask_mode, causal, st);
+        else launch_stream_kv8<128>(p, mask_mode, causal, st);
+        return check_launch("attention (mfma, fp8 keys/values)");
+    }
     // the software-pipelined kernel takes long key sequences of what it covers (hook: variant 3 keeps everything on the
     // streaming kernel, variant 4 sends everything the pipelined kernel covers to it)
     if (mfma_ok && g_attention_variant != 3 &&
@@ -916,4 +982,16 @@ extern "C" int kernl_attention_cached_fwd(const void *q, const void *k, const vo
                                           void *stream) {
     return attention_entry(q, k, v, out, mask, B, H, M, N, D, q_strides, k_strides, v_strides, o_strides, mask_sizes,
                            mask_strides, mask_dtype, sm_scale, 1, start_position, mask_min_clamp, dtype, stream);
+}
+
+extern "C" int kernl_attention_kv8_fwd(const void *q, const void *k8, const void *v8, void *out, const void *mask,
+                                       int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
+                                       const int64_t q_strides[4], const int64_t k_strides[4],
+                                       const int64_t v_strides[4], const int64_t o_strides[4],
+                                       const int64_t mask_sizes[4], const int64_t mask_strides[4], int mask_dtype,
+                                       float sm_scale, int is_causal, int64_t start_position, float mask_min_clamp,
+                                       int dtype, void *stream) {
+    return attention_entry(q, k8, v8, out, mask, B, H, M, N, D, q_strides, k_strides, v_strides, o_strides, mask_sizes,
+                           mask_strides, mask_dtype, sm_scale, is_causal, is_causal ? start_position : 0, mask_min_clamp,
+                           dtype, stream, true);
 }

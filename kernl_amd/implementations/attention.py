@@ -12,6 +12,8 @@ from torch.amp import custom_fwd
 
 from kernl_amd import _lib
 
+ONE_BYTE_KV_DTYPES = (torch.int8, torch.uint8, torch.float8_e5m2)  # fp8 e5m2 storage of keys and values
+
 
 def attention_reference(
     q: torch.Tensor,
@@ -72,9 +74,15 @@ class Attention(torch.autograd.Function):
         autocast every floating argument, mask included, is cast to fp16 first, as `custom_fwd` does there.
         """
         assert q.shape[-1] == k.shape[-1]
-        assert (
-            q.dtype == k.dtype == v.dtype == output.dtype
-        ), f"All tensors must have the same dtype: {q.dtype}, {k.dtype}, {v.dtype}, {output.dtype}"
+        # keys and values stored as fp8 e5m2 bytes (reference: `get_model_fp8` on `cache_k` / `cache_v`,
+        # experimental/llama-v2/kernel/fused_kernel_fp8.py:68-74): the kernel widens them on their way into LDS
+        one_byte_kv = k.dtype in ONE_BYTE_KV_DTYPES and v.dtype in ONE_BYTE_KV_DTYPES
+        if one_byte_kv:
+            assert q.dtype == output.dtype == torch.float16, f"fp8 keys/values go with float16 queries, got {q.dtype}"
+        else:
+            assert (
+                q.dtype == k.dtype == v.dtype == output.dtype
+            ), f"All tensors must have the same dtype: {q.dtype}, {k.dtype}, {v.dtype}, {output.dtype}"
         assert q.dtype in [torch.float16, torch.bfloat16], f"Only float16 and bfloat16 are supported, got {q.dtype}"
         batch, head_size, m_size, dhead = q.size()
         n_size = k.size(2)
@@ -97,7 +105,9 @@ class Attention(torch.autograd.Function):
             assert attention_mask.dtype in _lib.DTYPE_CODE, f"Mask must be a floating tensor, got {attention_mask.dtype}"
             min_clamp = torch.finfo(attention_mask.dtype).min
 
-        if is_causal and start_position:
+        if one_byte_kv:
+            _lib.attention_kv8_fwd(q, k, v, output, attention_mask, sm_scale, is_causal, int(start_position), min_clamp)
+        elif is_causal and start_position:
             _lib.attention_cached_fwd(q, k, v, output, attention_mask, sm_scale, int(start_position), min_clamp)
         else:
             _lib.attention_fwd(q, k, v, output, attention_mask, sm_scale, is_causal, min_clamp)

@@ -336,3 +336,55 @@ def test_matrix_mask_config1_size_properties(close):
             ref = attention_oracle(q[b:b + 1, h:h + 1].cpu(), k[b:b + 1, h:h + 1].cpu(), v[b:b + 1, h:h + 1].cpu(), 0.125, False,
                                    mask[mb:mb + 1, mh:mh + 1].cpu())
             close(out[b:b + 1, h:h + 1], ref, torch.float16, what=f"matrix mask {mshape} at batch {b} head {h}")
+
+
+@pytest.mark.parametrize("storage", ["int8", "float8_e5m2"])
+@pytest.mark.parametrize("mask_kind", ["none", "padding"])
+@pytest.mark.parametrize(
+    "case",
+    [(2, 3, 200, 200, 64, False, 0), (1, 4, 130, 333, 64, True, 203), (2, 2, 128, 128, 128, True, 0),
+     (1, 2, 96, 1100, 128, True, 1004), (1, 2, 17, 64, 64, False, 0), (2, 2, 512, 512, 64, True, 0)],
+    ids=lambda c: "x".join(map(str, c)),
+)
+def test_attention_over_fp8_keys_and_values(case, mask_kind, storage, close):
+    """Keys and values stored as fp8 e5m2 bytes (reference: the int8 key/value caches of experimental/llama-v2/kernel/
+    fused_kernel_fp8.py:68-74, widened on load by fused_kernel_attention.py:66-70, :90-94): the tiled kernel must give
+    what the oracle gives on the DECODED keys and values — prefill over such a cache, with and without the causal
+    diagonal shifted by `start_position`, ragged tiles, both head sizes."""
+    from kernl_amd.implementations.attention_skinny import to_e5m2
+    from oracle import e5m2_decode_oracle
+
+    B, H, M, N, D, causal, start = case
+    gen = torch.Generator().manual_seed(23)
+    q = torch.randn((B, H, M, D), generator=gen).half()
+    k8, v8 = to_e5m2(torch.randn((B, H, N, D), generator=gen)), to_e5m2(torch.randn((B, H, N, D), generator=gen))
+    k_dec, v_dec = e5m2_decode_oracle(k8), e5m2_decode_oracle(v8)
+    mask = None
+    if mask_kind == "padding":
+        lengths = torch.randint(max(1, N // 2), N + 1, (B,), generator=gen)
+        mask = torch.zeros((B, 1, 1, N))
+        for b in range(B):
+            mask[b, :, :, lengths[b]:] = float("-inf")
+    if storage == "float8_e5m2":
+        k8, v8 = k8.view(torch.float8_e5m2), v8.view(torch.float8_e5m2)
+    qc = q.cuda()
+    out = torch.empty_like(qc)
+    print(f"case {case} mask={mask_kind} storage={storage}", flush=True)
+    attention_forward(qc, k8.cuda(), v8.cuda(), out, 0.2, is_causal=causal, attention_mask=None if mask is None else mask.cuda(),
+                      start_position=start)
+    torch.cuda.synchronize()
+    ref = attention_oracle(q, k_dec, v_dec, 0.2, causal, mask, start)
+    close(out, ref, torch.float16, what=f"fp8 keys/values {case} {mask_kind}")
+
+
+def test_attention_fp8_keys_and_values_rejections():
+    q = torch.zeros((1, 1, 64, 64), dtype=torch.bfloat16, device="cuda")
+    kv = torch.zeros((1, 1, 64, 64), dtype=torch.int8, device="cuda")
+    with pytest.raises(AssertionError, match="float16"):
+        attention_forward(q, kv, kv, torch.empty_like(q), 1.0)
+    q = q.half()
+    with pytest.raises(_lib.KernlLibraryError, match="per-key"):
+        attention_forward(q, kv, kv, torch.empty_like(q), 1.0, attention_mask=torch.zeros((1, 1, 64, 64), device="cuda"))
+    q48, kv48 = torch.zeros((1, 1, 64, 48), dtype=torch.half, device="cuda"), torch.zeros((1, 1, 64, 48), dtype=torch.int8, device="cuda")
+    with pytest.raises(_lib.KernlLibraryError, match="head size"):
+        attention_forward(q48, kv48, kv48, torch.empty_like(q48), 1.0)
