@@ -41,6 +41,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef short s16x8 __attribute__((ext_vector_type(8)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    typedef AttnTileMap<D> TileMap;                       // staging and fragment addresses of a K / V stage
     constexpr int BM = 128, BN = 64;
     constexpr int KROW = D * 2, VP = D * 2;               // LDS row bytes of the K tile [key][D] and V tile [key][D]
     constexpr int K_BYTES = BN * KROW, V_BYTES = BN * VP;
@@ -114,10 +115,9 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 #pragma unroll
     for (int i = 0; i < KI; ++i) {
         const int qd = tid + 256 * i;
-        const int row = qd / DC, cs = qd % DC;
-        kdma[i] = (uint32_t)(((int64_t)row * p.ks[2] + swz_chunk<KROW>(row, cs) * 8) * KVB);
-        const int vsw = (D == 64) ? ((row >> 1) & 1) : (row & 3);
-        vdma[i] = (uint32_t)(((int64_t)row * p.vs[2] + (cs ^ (vsw << 2)) * 8) * KVB);
+        const int row = TileMap::stage_row(qd);
+        kdma[i] = (uint32_t)(((int64_t)row * p.ks[2] + TileMap::k_stage_chunk(qd) * 8) * KVB);
+        vdma[i] = (uint32_t)(((int64_t)row * p.vs[2] + TileMap::v_stage_chunk(qd) * 8) * KVB);
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
     const uint32_t dma_base = lds_base + wave * 1024;
@@ -332,15 +332,9 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     // of 4.
     int k_off[KS], vt_off[DB];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) k_off[ks] = swz_offset<KROW>(lr, 2 * ks + lh);
-    {
-        const int i16 = lane & 15, g16 = lane >> 4;
-        const int kq = i16 >> 2;
-        const int fs = rowperm16(16 * (g16 & 1) + 4 * (i16 & 3));
-        const int vsw = (D == 64) ? (kq >> 1) : kq;
+    for (int ks = 0; ks < KS; ++ks) k_off[ks] = TileMap::k_frag_offset(lr, lh, ks);
 #pragma unroll
-        for (int d = 0; d < DB; ++d) vt_off[d] = K_BYTES + (4 * lh + kq) * VP + ((d ^ vsw) * 64) + fs * 2;
-    }
+    for (int d = 0; d < DB; ++d) vt_off[d] = K_BYTES + TileMap::v_frag_offset(lane, d);
     const int64_t mask_row = mask_base + (int64_t)min(my_m, M - 1) * (MASK_MODE == MASK_MATRIX ? p.ms[2] : 0);
     // Matrix masks on the fast route: the 8 runs of 4 consecutive keys a lane needs from its mask row are
     // fetched one tile ahead, right after the previous tile's values have been consumed, into the same registers.
@@ -369,14 +363,8 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         const int row0 = q0 + wave * 32;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            int r, c;
-            if (m_f32) {
-                r = i * 4 + (lane >> 4);
-                c = (lane & 15) ^ (r & 15);
-            } else {
-                r = (i & 3) * 8 + (lane >> 3);
-                c = (lane & 7) ^ ((r >> 1) & 7);
-            }
+            const int r = m_f32 ? MaskTileMap<4>::stage_row(i, lane) : MaskTileMap<2>::stage_row(i & 3, lane);
+            const int c = m_f32 ? MaskTileMap<4>::stage_chunk(i, lane) : MaskTileMap<2>::stage_chunk(i & 3, lane);
             // rows past the last query read the last row again (their results are never stored)
             mdma[i] = (uint32_t)(((int64_t)min(row0 + r, M - 1) * p.ms[2]) * m_esize + c * 16);
         }
@@ -403,14 +391,12 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         const unsigned char *mb = smem + 2 * STAGE + wave * MASK_WAVE_BYTES;
         if (ROUTE == 3) {
 #pragma unroll
-            for (int i = 0; i < NBS * 4; ++i) {
-                const int c = (i >> 2) * 8 + (i & 3) * 2 + lh;
-                mreg[i] = *reinterpret_cast<const u32x4 *>(mb + lr * 256 + ((c ^ (lr & 15)) << 4));
-            }
+            for (int i = 0; i < NBS * 4; ++i)
+                mreg[i] = *reinterpret_cast<const u32x4 *>(mb + MaskTileMap<4>::read_offset(lr, lh, i));
         } else {
 #pragma unroll
             for (int i = 0; i < NBS * 4; ++i) {
-                const u32x2 two = *reinterpret_cast<const u32x2 *>(mb + lr * 128 + ((i ^ ((lr >> 1) & 7)) << 4) + lh * 8);
+                const u32x2 two = *reinterpret_cast<const u32x2 *>(mb + MaskTileMap<2>::read_offset(lr, lh, i));
                 mreg[i >> 1][2 * (i & 1)] = two[0];
                 mreg[i >> 1][2 * (i & 1) + 1] = two[1];
             }

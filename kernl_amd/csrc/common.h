@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "../../include/kernl_hip.h"
+#include "index_math.h"
 
 namespace kernl {
 
@@ -81,10 +82,6 @@ __device__ __forceinline__ void mfma16_inplace(f16x8 a, f16x8 b, f32x4_acc &c) {
 __device__ __forceinline__ void mfma16_inplace(bf16x8 a, bf16x8 b, f32x4_acc &c) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
-
-// Because of the D layout above, feeding MFMA row i with logical row rowperm16(i) makes every lane end up
-// with 16 CONSECUTIVE logical rows: lane half h holds logical rows 16*h + v for v = 0..15.
-__device__ __forceinline__ int rowperm16(int i) { return 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3); }
 
 // ----------------------------------------------------------------------------------------------------
 // conversions
@@ -205,23 +202,6 @@ __device__ __forceinline__ float halves32_sum(float v) {
     float lo, hi;
     halves32(v, lo, hi);
     return lo + hi;
-}
-
-// ----------------------------------------------------------------------------------------------------
-// LDS swizzle for tiles whose rows are ROW_BYTES long (64, 128 or 256) and are read as 16-byte chunks by the
-// 32 rows x 2 k-halves pattern of an MFMA operand fetch: 16 consecutive rows reading the same logical chunk
-// land in 16 different 16-byte bank groups.
-// ----------------------------------------------------------------------------------------------------
-template <int ROW_BYTES>
-__device__ __forceinline__ int swz_chunk(int row, int chunk) {
-    static_assert(ROW_BYTES == 64 || ROW_BYTES == 128 || ROW_BYTES == 256, "row must span 4, 8 or 16 chunks");
-    if (ROW_BYTES == 64) return chunk ^ ((row >> 2) & 3);
-    if (ROW_BYTES == 128) return chunk ^ ((row >> 1) & 7);
-    return chunk ^ (row & 15);
-}
-template <int ROW_BYTES>
-__device__ __forceinline__ int swz_offset(int row, int chunk) {  // byte offset inside the tile
-    return row * ROW_BYTES + swz_chunk<ROW_BYTES>(row, chunk) * 16;
 }
 
 // ----------------------------------------------------------------------------------------------------

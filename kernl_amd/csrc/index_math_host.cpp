@@ -1,0 +1,71 @@
+// C entry points over index_math.h for the host-side replay tool (kernl_amd/debugger): the SAME functions the kernels
+// are compiled from, built here with the host compiler only (g++ -shared -fPIC), no HIP involved.
+#include "index_math.h"
+
+using namespace kernl;
+
+extern "C" {
+
+int kernl_idx_rowperm16(int i) { return rowperm16(i); }
+
+int kernl_idx_swz_offset(int row_bytes, int row, int chunk) {
+    if (row_bytes == 64) return swz_offset<64>(row, chunk);
+    if (row_bytes == 128) return swz_offset<128>(row, chunk);
+    if (row_bytes == 256) return swz_offset<256>(row, chunk);
+    return -1;
+}
+
+// which: 0 stage_row(qd), 1 k_stage_chunk(qd), 2 v_stage_chunk(qd), 3 k_frag_offset(lr=a, lh=b, ks=c),
+//        4 v_frag_offset(lane=a, d=b); head size 64 or 128
+int kernl_idx_attention(int head_size, int which, int a, int b, int c) {
+    if (head_size == 64) {
+        typedef AttnTileMap<64> M;
+        switch (which) {
+            case 0: return M::stage_row(a);
+            case 1: return M::k_stage_chunk(a);
+            case 2: return M::v_stage_chunk(a);
+            case 3: return M::k_frag_offset(a, b, c);
+            case 4: return M::v_frag_offset(a, b);
+        }
+    } else if (head_size == 128) {
+        typedef AttnTileMap<128> M;
+        switch (which) {
+            case 0: return M::stage_row(a);
+            case 1: return M::k_stage_chunk(a);
+            case 2: return M::v_stage_chunk(a);
+            case 3: return M::k_frag_offset(a, b, c);
+            case 4: return M::v_frag_offset(a, b);
+        }
+    }
+    return -1;
+}
+
+// which: 0 stage_row(i=a, lane=b), 1 stage_chunk(i=a, lane=b), 2 read_offset(lr=a, lh=b, j=c); element size 4 or 2
+int kernl_idx_mask(int element_size, int which, int a, int b, int c) {
+    if (element_size == 4) {
+        typedef MaskTileMap<4> M;
+        switch (which) {
+            case 0: return M::stage_row(a, b);
+            case 1: return M::stage_chunk(a, b);
+            case 2: return M::read_offset(a, b, c);
+        }
+    } else if (element_size == 2) {
+        typedef MaskTileMap<2> M;
+        switch (which) {
+            case 0: return M::stage_row(a, b);
+            case 1: return M::stage_chunk(a, b);
+            case 2: return M::read_offset(a, b, c);
+        }
+    }
+    return -1;
+}
+
+// layout: 0 = 256 columns, 1 = 192 columns, 2 = gated (256 columns)
+int kernl_idx_wide_weight_row(int layout, int row) {
+    if (layout == 0) return wide_weight_row<false, 8>(row);
+    if (layout == 1) return wide_weight_row<false, 6>(row);
+    if (layout == 2) return wide_weight_row<true, 8>(row);
+    return -1;
+}
+
+}  // extern "C"

@@ -632,10 +632,7 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
             const int q = (wave * LOADS_W + i) * 64 + lane;
             const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
             // LDS row `row` is MFMA row r = row % 16 of n-block row / 16; see the placement rule above the kernel
-            const int r = row & 15, j = (row >> 4) & 3;
-            const int wrow = GATED      ? (row & ~63) + 32 * (j >> 1) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3)
-                             : NBN == 8 ? (row & ~63) + 16 * (r >> 2) + 4 * j + (r & 3)
-                                        : (row & ~31) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3);
+            const int wrow = wide_weight_row<GATED, NBN>(row);
             wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
         }
     };
@@ -854,8 +851,7 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     for (int i = 0; i < LOADS_W; ++i) {
         const int q = (wave * LOADS_W + i) * 64 + lane;
         const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
-        const int r = row & 15, j = (row >> 4) & 3;
-        const int wrow = NBN == 8 ? (row & ~63) + 16 * (r >> 2) + 4 * j + (r & 3) : (row & ~31) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3);
+        const int wrow = wide_weight_row<false, NBN>(row);
         wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
     }
     typedef __attribute__((address_space(3))) void lds_void;
