@@ -237,6 +237,29 @@ int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float eps, const
                          int activation, int gated, int dtype, void *stream);
 
 /*
+ * A decoding step's projection with everything around it in ONE launch (at most 64 rows of x, K % 64 == 0, f16 / bf16,
+ * plain 16-bit weight w [N, K]):
+ *     y   = (rms_weight ? rsqrt(mean(x^2) + eps) * ((x * rms_weight) @ w^T) : x @ w^T) + bias
+ *     y   = rotate(y)           on the columns below rope_cols, when cos / sin are given
+ *     out = y + residual        when residual is given
+ * Replaces the `rms_matmul_rbe_qkv[grid](...)` launch WITH its rotary epilogue (experimental/llama-v2/kernel/
+ * fused_kernel_proj_qkv.py:250-347: RMSNorm prologue, the three projections as one product, rotation of the query and
+ * key columns, :69-100).  Differences: the rotation uses the half-split convention of Hugging Face decoders (inside a
+ * head of head_dim columns, column d pairs with d + head_dim / 2) and reads the cos / sin tables the model computed —
+ * element (b, s, d) at b * table_strides[0] + s * table_strides[1] + d, where row m of x is position m % rows_per_batch
+ * of batch entry m / rows_per_batch — instead of computing angles from a base; and the residual add, which the
+ * reference model leaves to eager PyTorch (experimental/llama-v2/llama/model.py:262-264), has no counterpart there.
+ * cos / sin NULL: no rotation (then rms_weight may be NULL too); with rotation rms_weight is required, head_dim a
+ * multiple of 32 dividing N and rope_cols.  Anything else returns KERNL_ERR_UNSUPPORTED.
+ */
+int kernl_linear_decode_fwd(const void *x, const void *rms_weight, float eps, const void *w, const void *bias,
+                            const void *residual, void *out, int64_t M, int64_t N, int64_t K,
+                            const int64_t x_strides[2], const int64_t out_strides[2],
+                            const int64_t residual_strides[2], const void *cos, const void *sin,
+                            int64_t head_dim, int64_t rope_cols, int64_t rows_per_batch,
+                            const int64_t table_strides[3], int table_dtype, int dtype, void *stream);
+
+/*
  * Gated linear unit:  out[M,N] = act(x·w_gateᵀ + b_gate) * (x·w_valueᵀ + b_value)  as ONE GEMM.
  * Replaces the `ff_llama` launch of experimental/llama-v2/kernel/fused_kernel_ff.py:10-79 (SwiGLU: act = SiLU; that
  * kernel's RMSNorm prologue is not part of this entry point) — and the three kernels (two GEMMs, one multiply) a

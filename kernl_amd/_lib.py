@@ -33,6 +33,7 @@ EXPORTED_SYMBOLS = (
     "kernl_linear_fwd",
     "kernl_linear_w8_fwd",
     "kernl_linear_rms_fwd",
+    "kernl_linear_decode_fwd",
     "kernl_linear_glu_fwd",
     "kernl_layernorm_fwd",
     "kernl_add_layernorm_fwd",
@@ -103,6 +104,11 @@ def load() -> ctypes.CDLL:
     lib.kernl_linear_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_linear_w8_fwd.restype = ctypes.c_int
     lib.kernl_linear_w8_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
+    lib.kernl_linear_decode_fwd.restype = ctypes.c_int
+    lib.kernl_linear_decode_fwd.argtypes = (
+        [_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp] + [_i64] * 3 + [_i64p] * 3 + [_vp, _vp] + [_i64] * 3
+        + [_i64p, ctypes.c_int, ctypes.c_int, _vp]
+    )
     lib.kernl_linear_rms_fwd.restype = ctypes.c_int
     lib.kernl_linear_rms_fwd.argtypes = (
         [_vp, _vp, ctypes.c_float, _vp, _vp, _vp] + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int] * 3 + [_vp]
@@ -333,6 +339,40 @@ def linear_rms_fwd(x2d, rms_weight, eps: float, weight, bias, out2d, activation:
             _stream(x2d),
         )
     _check(st, "kernl_linear_rms_fwd")
+
+
+def linear_decode_supported(x2d, weight) -> bool:
+    """What `kernl_linear_decode_fwd` takes: 16-bit rows, at most 64 of them, K a multiple of 64, a 16-bit weight."""
+    M, K = x2d.shape
+    return (
+        x2d.dtype in (torch.float16, torch.bfloat16) and weight.dtype == x2d.dtype and M <= 64 and K % 64 == 0
+        and x2d.stride(1) == 1 and x2d.stride(0) % 8 == 0 and x2d.data_ptr() % 16 == 0
+        and weight.is_contiguous() and weight.data_ptr() % 16 == 0
+    )
+
+
+def linear_decode_fwd(x2d, rms_weight, eps: float, weight, bias, residual2d, out2d, cos=None, sin=None, head_dim: int = 0,
+                      rope_cols: int = 0, rows_per_batch: int = 1) -> None:
+    """cos / sin: [batch | 1, positions, head_dim] tables (unit feature stride) or None; row m of x2d is position
+    m % rows_per_batch of batch entry m / rows_per_batch."""
+    _require_gpu(x2d, rms_weight, weight, bias, residual2d, out2d, cos, sin)
+    M, K = x2d.shape
+    N = out2d.shape[1]
+    lib = load()
+    if cos is not None:
+        tstrides = _arr((0 if cos.shape[0] == 1 else cos.stride(0), cos.stride(1), cos.stride(2)))
+        tdtype, cptr, sptr = DTYPE_CODE[cos.dtype], cos.data_ptr(), sin.data_ptr()
+    else:
+        tstrides, tdtype, cptr, sptr = None, KERNL_F32, None, None
+    with torch.cuda.device(x2d.device):
+        st = lib.kernl_linear_decode_fwd(
+            x2d.data_ptr(), None if rms_weight is None else rms_weight.data_ptr(), float(eps), weight.data_ptr(),
+            None if bias is None else bias.data_ptr(), None if residual2d is None else residual2d.data_ptr(),
+            out2d.data_ptr(), M, N, K, _arr(x2d.stride()), _arr(out2d.stride()),
+            None if residual2d is None else _arr(residual2d.stride()), cptr, sptr, int(head_dim), int(rope_cols),
+            int(rows_per_batch), tstrides, tdtype, DTYPE_CODE[x2d.dtype], _stream(x2d),
+        )
+    _check(st, "kernl_linear_decode_fwd")
 
 
 def linear_glu_fwd(x2d, weight_interleaved, bias_interleaved, out2d, activation: int) -> None:

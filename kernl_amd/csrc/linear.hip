@@ -996,11 +996,38 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
 // fused_kernel_proj_qkv.py:116-183): the x fragments are multiplied by the norm's weight (rounded to 16 bit, as there),
 // every lane sums the squares of the x values that pass through it, and because the inverse root mean square is one
 // scalar per row it is applied to the finished sums: out = rsqrt(mean(x^2) + eps) * ((x * g) @ w^T) + bias.
-template <typename T, int MB, bool GATED, int WAVES, int NR, bool W8 = false, bool RMS = false>
+// Residual: out = act(...) + residual[m, n] when a residual pointer is given (the `hidden + projection(...)` of a
+// decoder layer; no counterpart in the reference, whose model adds in eager PyTorch).
+// ROPE: rotary position embedding applied to the output columns below `rope_cols`, in the half-split convention —
+// inside every head of `2 * half` columns, column d pairs with d + half:
+//     out[d] = y[d] cos[d] - y[d + half] sin[d],   out[d + half] = y[d + half] cos[d + half] + y[d] sin[d + half]
+// (reference: the rotation inside `rms_matmul_rbe_qkv`, experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:69-100
+// and :186-247, there on interleaved pairs with angles computed in the kernel; here from the cos / sin tables the
+// model computed, indexed by the row's batch entry and position).  A workgroup then owns the 16 columns d0 .. d0 + 15
+// of a head AND their partners (NR = 2 blocks, `half` columns apart), so both members of a pair meet in one lane.
+struct SkinnyExtra {
+    const void *residual;   // [M, N] of T, or null
+    int64_t res_rs, res_cs;
+    const void *cos, *sin;  // rotation tables, element (b, s, d) at b * t_bs + s * t_ss + d
+    int64_t t_bs, t_ss;
+    int table_dtype;        // KERNL_F16 / KERNL_BF16 / KERNL_F32
+    int half;               // half the head size
+    int rope_cols;          // columns [0, rope_cols) are rotated
+    int rows_per_batch;     // row m of x is position m % rows_per_batch of batch entry m / rows_per_batch
+};
+
+__device__ __forceinline__ float table_value(const void *t, int dtype, int64_t off) {
+    if (dtype == KERNL_F32) return static_cast<const float *>(t)[off];
+    if (dtype == KERNL_F16) return (float)static_cast<const f16 *>(t)[off];
+    return (float)static_cast<const bf16 *>(t)[off];
+}
+
+template <typename T, int MB, bool GATED, int WAVES, int NR, bool W8 = false, bool RMS = false, bool ROPE = false>
 __global__ void __launch_bounds__(64 * WAVES)
 linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
                      T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
-                     int64_t ai_rs, int64_t ai_cs, int act, const T *__restrict__ rms_w, float eps) {
+                     int64_t ai_rs, int64_t ai_cs, int act, const T *__restrict__ rms_w, float eps, const SkinnyExtra ex) {
+    static_assert(!ROPE || (NR == 2 && !GATED && !W8), "the rotating form pairs two plain 16-column blocks");
     typedef typename Vec8<T>::type vec8;
     constexpr int NA = GATED ? 2 : 1;        // weight fragments per 16 output columns: plain, or gate and value
     constexpr int NF = NA * NR;              // weight fragments per step (NR blocks of 16 output columns)
@@ -1011,7 +1038,11 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = (int)blockIdx.x * (16 * NR);  // first output column of this workgroup (N counts output columns)
+    // first output column of this workgroup (N counts output columns) and the distance between its column blocks
+    const int blocks_per_half = ROPE ? ex.half / 16 : 1;
+    const int n0 = ROPE ? ((int)blockIdx.x / blocks_per_half) * (2 * ex.half) + ((int)blockIdx.x % blocks_per_half) * 16
+                        : (int)blockIdx.x * (16 * NR);
+    const int rb_stride = ROPE ? ex.half : 16;
     // first interleaved row of the 16 output columns starting at nb (gated weights: 32 gate rows, 32 value rows, ...)
     auto gated_row = [](int nb) -> int { return (nb >> 5) * 64 + (nb & 31); };
     // rows of the weight this lane reads; columns beyond N repeat the last one and are never stored
@@ -1021,7 +1052,7 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
     const WT *wp[NF];
 #pragma unroll
     for (int rb = 0; rb < NR; ++rb) {
-        const int nb = n0 + 16 * rb;
+        const int nb = n0 + rb_stride * rb;
         if (GATED) {
             const int row = gated_row(min(nb, N - 16)) + r;
             wp[rb * NA] = wbase + (int64_t)row * K + 16 * g;
@@ -1134,6 +1165,54 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
 
     // the waves share the NR x MB blocks of 16 columns x 16 rows: element e of a lane is output column nb + 4 g + e
     // of x row 16 mb + r
+    if constexpr (ROPE) {
+        // a wave takes both column blocks of a 16-row block: element e of a lane is column n0 + 4 g + e and its partner
+        for (int mb = wave; mb < MB; mb += WAVES) {
+            const int m = 16 * mb + r;
+            float rstd = 1.0f;
+            if constexpr (RMS) {
+                float t = 0.0f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) t += red_sq[w][mb][r];
+                rstd = 1.0f / sqrtf(t / (float)K + eps);
+            }
+            const int64_t trow = (int64_t)(min(m, M - 1) / ex.rows_per_batch) * ex.t_bs + (int64_t)(min(m, M - 1) % ex.rows_per_batch) * ex.t_ss;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = n0 + 4 * g + e;   // lower member of the pair; the upper one is `half` columns further
+                float v[2];
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    float t4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int w = 0; w < WAVES; ++w) t4[w & 3] += red[w][a * MB + mb][lane][e];
+                    v[a] = ((t4[0] + t4[1]) + (t4[2] + t4[3])) * rstd;
+                }
+                if (m >= M || n >= N) continue;
+                if (bias != nullptr) {
+                    v[0] += to_float(bias[n]);
+                    v[1] += to_float(bias[n + ex.half]);
+                }
+                float y0 = v[0], y1 = v[1];
+                if (n < ex.rope_cols) {
+                    const int d = n % (2 * ex.half);
+                    const float c0 = table_value(ex.cos, ex.table_dtype, trow + d), s0 = table_value(ex.sin, ex.table_dtype, trow + d);
+                    const float c1 = table_value(ex.cos, ex.table_dtype, trow + d + ex.half);
+                    const float s1 = table_value(ex.sin, ex.table_dtype, trow + d + ex.half);
+                    y0 = v[0] * c0 - v[1] * s0;
+                    y1 = v[1] * c1 + v[0] * s1;
+                }
+                if (ex.residual != nullptr) {
+                    const T *res = static_cast<const T *>(ex.residual) + (int64_t)m * ex.res_rs;
+                    y0 += to_float(res[(int64_t)n * ex.res_cs]);
+                    y1 += to_float(res[(int64_t)(n + ex.half) * ex.res_cs]);
+                }
+                out[(int64_t)m * out_rs + (int64_t)n * out_cs] = from_float<T>(y0);
+                out[(int64_t)m * out_rs + (int64_t)(n + ex.half) * out_cs] = from_float<T>(y1);
+            }
+        }
+        return;
+    }
     for (int unit = wave; unit < NR * MB; unit += WAVES) {
         const int rb = unit / MB, mb = unit % MB;
         const int nb = n0 + 16 * rb;
@@ -1165,6 +1244,8 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
             if (!GATED && act_in != nullptr) act_in[(int64_t)m * ai_rs + (int64_t)n * ai_cs] = from_float<T>(v[0]);
             float y = apply_act16(v[0], act);
             if (GATED) y *= v[NA - 1];
+            if (ex.residual != nullptr)
+                y += to_float(static_cast<const T *>(ex.residual)[(int64_t)m * ex.res_rs + (int64_t)n * ex.res_cs]);
             out[(int64_t)m * out_rs + (int64_t)n * out_cs] = from_float<T>(y);
         }
     }
@@ -1229,6 +1310,7 @@ struct LinearArgs {
     int64_t x_rs, x_cs, out_rs, out_cs, ai_rs, ai_cs;
     int act;
     hipStream_t st;
+    const SkinnyExtra *extra = nullptr;  // residual / rotation of the few-row kernel (decoding steps)
 };
 
 template <typename T, typename Cfg, int ACT, bool W8 = false>
@@ -1428,10 +1510,14 @@ static int pick_tile(int M, int N, int K, bool gated) {
 
 int g_linear_force_tile = 0;  // test / tuning hook: 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192
 
-template <typename T, bool GATED, int MB, int NR, bool W8, bool RMS = false>
-static void launch_skinny_blocks(const LinearArgs &a, const void *rms_w = nullptr, float eps = 0.0f) {
+template <typename T, bool GATED, int MB, int NR, bool W8, bool RMS = false, bool ROPE = false>
+static void launch_skinny_blocks(const LinearArgs &a, const void *rms_w = nullptr, float eps = 0.0f,
+                                 const SkinnyExtra *extra = nullptr) {
     const int n_out = GATED ? a.N / 2 : a.N;
-    const dim3 grid((unsigned)((n_out + 16 * NR - 1) / (16 * NR)));
+    const dim3 grid((unsigned)((n_out + 16 * NR - 1) / (16 * NR)));  // the rotating form: N is a multiple of the head size
+    SkinnyExtra ex = {};
+    if (extra != nullptr) ex = *extra;
+    else if (a.extra != nullptr) ex = *a.extra;
     const int act = a.act & (kGluBit - 1);
     // waves per workgroup: enough to have a whole block of weight rows in flight when K is long, never more than
     // there are chunks, and no more than the LDS for their partial sums allows
@@ -1446,10 +1532,10 @@ static void launch_skinny_blocks(const LinearArgs &a, const void *rms_w = nullpt
     if (per_cu >= 3) waves = 4;
     else if (per_cu == 2 && waves > 8) waves = 8;
 #define KERNL_SKINNY(WV)                                                                                                \
-    hipLaunchKernelGGL((linear_skinny_kernel<T, MB, GATED, WV, NR, W8, RMS>), grid, dim3(64 * WV), 0, a.st,                      \
+    hipLaunchKernelGGL((linear_skinny_kernel<T, MB, GATED, WV, NR, W8, RMS, ROPE>), grid, dim3(64 * WV), 0, a.st,                \
                        static_cast<const T *>(a.x), static_cast<const T *>(a.w), static_cast<const T *>(a.bias),       \
                        static_cast<T *>(a.out), static_cast<T *>(a.act_in), a.M, n_out, a.K, a.x_rs, a.out_rs, a.out_cs, \
-                       a.ai_rs, a.ai_cs, act, static_cast<const T *>(rms_w), eps)
+                       a.ai_rs, a.ai_cs, act, static_cast<const T *>(rms_w), eps, ex)
     if constexpr (kMaxWaves >= 16) {
         if (waves >= 16) { KERNL_SKINNY(16); return; }
     }
@@ -1513,6 +1599,25 @@ static void launch_skinny_rms(const LinearArgs &a, const void *rms_w, float eps)
     if (mb <= 1) launch_skinny_blocks<T, GATED, 1, 1, false, true>(a, rms_w, eps);
     else if (mb <= 2) launch_skinny_blocks<T, GATED, 2, 1, false, true>(a, rms_w, eps);
     else launch_skinny_blocks<T, GATED, 4, 1, false, true>(a, rms_w, eps);
+}
+
+// decoding-step projection with optional RMSNorm prologue, rotary epilogue and residual (plain 16-bit weights)
+template <typename T>
+static void launch_skinny_decode(const LinearArgs &a, const void *rms_w, float eps, const SkinnyExtra &ex) {
+    const int mb = (a.M + 15) / 16;
+    if (ex.half > 0) {  // rotating form: two column blocks per workgroup, always with the normalising prologue
+        if (mb <= 1) launch_skinny_blocks<T, false, 1, 2, false, true, true>(a, rms_w, eps, &ex);
+        else if (mb <= 2) launch_skinny_blocks<T, false, 2, 2, false, true, true>(a, rms_w, eps, &ex);
+        else launch_skinny_blocks<T, false, 4, 2, false, true, true>(a, rms_w, eps, &ex);
+    } else if (rms_w != nullptr) {
+        if (mb <= 1) launch_skinny_blocks<T, false, 1, 1, false, true>(a, rms_w, eps, &ex);
+        else if (mb <= 2) launch_skinny_blocks<T, false, 2, 1, false, true>(a, rms_w, eps, &ex);
+        else launch_skinny_blocks<T, false, 4, 1, false, true>(a, rms_w, eps, &ex);
+    } else {
+        LinearArgs b = a;  // the plain kernel with its own grid rule; the residual travels in the arguments
+        b.extra = &ex;
+        launch_skinny<T, false>(b);
+    }
 }
 
 template <typename T>
@@ -1715,4 +1820,68 @@ extern "C" int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float
         else launch_skinny_rms<bf16, false>(a, rms_weight, eps);
     }
     return check_launch("rms linear (skinny)");
+}
+
+extern "C" int kernl_linear_decode_fwd(const void *x, const void *rms_weight, float eps, const void *w, const void *bias,
+                                       const void *residual, void *out, int64_t M, int64_t N, int64_t K,
+                                       const int64_t x_strides[2], const int64_t out_strides[2],
+                                       const int64_t residual_strides[2], const void *cos, const void *sin,
+                                       int64_t head_dim, int64_t rope_cols, int64_t rows_per_batch,
+                                       const int64_t table_strides[3], int table_dtype, int dtype, void *stream) {
+    using namespace kernl;
+    if (x == nullptr || w == nullptr || out == nullptr || x_strides == nullptr || out_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "decode linear: x, w, out and their strides must not be NULL");
+    if (residual != nullptr && residual_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "decode linear: residual given without strides");
+    if (M < 0 || N <= 0 || K <= 0)
+        return set_error(KERNL_ERR_INVALID_ARG, "decode linear: bad sizes M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+                         (long long)K);
+    if (dtype != KERNL_F16 && dtype != KERNL_BF16)
+        return set_error(KERNL_ERR_UNSUPPORTED, "decode linear: only f16 and bf16 are supported, got dtype %d", dtype);
+    if (M > 64 || K % 64 != 0 || N > INT32_MAX || K > INT32_MAX)
+        return set_error(KERNL_ERR_UNSUPPORTED, "decode linear: at most 64 rows of x and K a multiple of 64 (M=%lld K=%lld)",
+                         (long long)M, (long long)K);
+    if (x_strides[1] != 1 || x_strides[0] % 8 != 0 || !aligned16(x) || !aligned16(w) ||
+        (rms_weight != nullptr && !aligned16(rms_weight)))
+        return set_error(KERNL_ERR_UNSUPPORTED, "decode linear: x needs unit feature stride and 16-byte aligned rows, the "
+                         "weights 16-byte aligned bases");
+    const bool rope = cos != nullptr || sin != nullptr;
+    SkinnyExtra ex = {};
+    if (rope) {
+        if (cos == nullptr || sin == nullptr || table_strides == nullptr)
+            return set_error(KERNL_ERR_INVALID_ARG, "decode linear: rotation needs cos, sin and their strides");
+        if (table_dtype != KERNL_F16 && table_dtype != KERNL_BF16 && table_dtype != KERNL_F32)
+            return set_error(KERNL_ERR_UNSUPPORTED, "decode linear: unknown table dtype %d", table_dtype);
+        if (head_dim < 32 || head_dim % 32 != 0 || N % head_dim != 0 || rope_cols < 0 || rope_cols > N ||
+            rope_cols % head_dim != 0 || rows_per_batch <= 0 || table_strides[2] != 1)
+            return set_error(KERNL_ERR_UNSUPPORTED, "decode linear: rotation needs a head size that is a multiple of 32 "
+                             "and divides N and rope_cols, tables with unit feature stride and rows_per_batch > 0");
+        if (rms_weight == nullptr)
+            return set_error(KERNL_ERR_UNSUPPORTED, "decode linear: the rotating form is built with the RMSNorm prologue only");
+        ex.cos = cos; ex.sin = sin;
+        ex.t_bs = table_strides[0]; ex.t_ss = table_strides[1];
+        ex.table_dtype = table_dtype;
+        ex.half = (int)(head_dim / 2);
+        ex.rope_cols = (int)rope_cols;
+        ex.rows_per_batch = (int)rows_per_batch;
+    } else {
+        ex.rows_per_batch = 1;
+    }
+    if (residual != nullptr) {
+        ex.residual = residual;
+        ex.res_rs = residual_strides[0];
+        ex.res_cs = residual_strides[1];
+    }
+    if (M == 0) return KERNL_OK;
+    LinearArgs a;
+    a.x = x; a.w = w; a.bias = bias; a.out = out; a.act_in = nullptr;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.x_rs = x_strides[0]; a.x_cs = x_strides[1];
+    a.out_rs = out_strides[0]; a.out_cs = out_strides[1];
+    a.ai_rs = 0; a.ai_cs = 0;
+    a.act = KERNL_ACT_NONE;
+    a.st = static_cast<hipStream_t>(stream);
+    if (dtype == KERNL_F16) launch_skinny_decode<f16>(a, rms_weight, eps, ex);
+    else launch_skinny_decode<bf16>(a, rms_weight, eps, ex);
+    return check_launch("decode linear (skinny)");
 }

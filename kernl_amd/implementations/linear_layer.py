@@ -162,3 +162,59 @@ def rms_linear_layer(
     if gated:
         return linear_glu_layer(normed, weight, bias, activation)
     return linear_layer(normed, weight, bias, activation)
+
+
+def decode_linear_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether `decode_linear_layer` takes this input: at most 64 rows in all, 16-bit, K a multiple of 64."""
+    if x.dtype not in (torch.float16, torch.bfloat16) or weight.dtype != x.dtype or x.shape[-1] % 64 != 0:
+        return False
+    rows = x.numel() // x.shape[-1]
+    return 0 < rows <= 64 and weight.is_contiguous() and weight.data_ptr() % 16 == 0
+
+
+def decode_linear_layer(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    rms_weight: Optional[torch.Tensor] = None,
+    eps: float = 0.0,
+    residual: Optional[torch.Tensor] = None,
+    cos: Optional[torch.Tensor] = None,
+    sin: Optional[torch.Tensor] = None,
+    head_dim: int = 0,
+    rope_cols: int = 0,
+) -> torch.Tensor:
+    """One launch for a decoding step's projection and what surrounds it:
+
+        y = linear(rms_norm(x, rms_weight, eps) if rms_weight is given else x, weight, bias)
+        y[..., :rope_cols] rotated head by head (half-split rotary embedding) when cos / sin are given
+        out = y + residual when a residual is given
+
+    x [batch, positions, K] or [rows, K], at most 64 rows in all; cos / sin [batch | 1, positions, head_dim] (a 2-D x
+    counts as one batch entry); residual of the output's shape.  Reference: `rms_matmul_rbe_qkv_wrapper`,
+    experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:289-344 (RMSNorm prologue + query/key/value projection +
+    rotation of the query and key columns in one kernel)."""
+    assert decode_linear_supported(x, weight), "decode_linear_layer: at most 64 rows of 16-bit x, K a multiple of 64"
+    assert (cos is None) == (sin is None)
+    K, N = x.shape[-1], weight.shape[0]
+    x_ = x if x.ndim == 2 else x.reshape(-1, K)
+    if x_.stride(-1) != 1 or x_.stride(0) % 8 != 0 or x_.data_ptr() % 16 != 0:
+        x_ = x_.contiguous()
+    rows_per_batch = x.shape[-2] if x.ndim == 3 else x_.shape[0]
+    if rms_weight is not None:
+        assert rms_weight.dtype == x.dtype and rms_weight.is_contiguous() and rms_weight.shape[0] == K
+        if x.dtype == torch.float16:
+            eps = max(eps, 1.6e-5)  # the fp16 policy of the RMSNorm operator (reference: layer_norm.py:295-296)
+    if cos is not None:
+        assert rms_weight is not None, "the rotating form comes with the RMSNorm prologue"
+        assert cos.shape == sin.shape and cos.dtype == sin.dtype and cos.dim() == 3 and cos.shape[-1] == head_dim
+        assert cos.shape[1] == rows_per_batch and cos.shape[0] in (1, x_.shape[0] // rows_per_batch)
+        assert cos.stride(-1) == 1 and sin.stride() == cos.stride(), "tables need unit feature stride and equal layouts"
+        assert head_dim % 32 == 0 and N % head_dim == 0 and rope_cols % head_dim == 0 and 0 <= rope_cols <= N
+    res_ = None
+    if residual is not None:
+        assert residual.dtype == x.dtype and residual.numel() == x_.shape[0] * N
+        res_ = residual.reshape(-1, N)
+    out = torch.empty((x_.shape[0], N), device=x.device, dtype=x.dtype)
+    _lib.linear_decode_fwd(x_, rms_weight, eps, weight, bias, res_, out, cos, sin, head_dim, rope_cols, rows_per_batch)
+    return out if x.ndim == 2 else out.reshape(*x.shape[:-1], N)

@@ -12,7 +12,12 @@ from kernl_amd.optimizer.attention import (
 from kernl_amd.optimizer.dropout import remove_dropout
 from kernl_amd.optimizer.kv_cache import drop_empty_cat_operands
 from kernl_amd.optimizer.layer_norm import replace_layer_norm, replace_layer_norm_fn, replace_layer_norm_rms
-from kernl_amd.optimizer.linear import fuse_rms_norm_into_linears, replace_all_linear
+from kernl_amd.optimizer.linear import (
+    fuse_residual_into_linears,
+    fuse_rms_norm_into_linears,
+    fuse_rotary_into_projections,
+    replace_all_linear,
+)
 from kernl_amd.optimizer.mask import (
     constant_causal_masks_to_flag,
     drop_all_true_conjuncts,
@@ -45,4 +50,6 @@ def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
     replace_layer_norm_fn(gm)
     replace_layer_norm_rms(gm)
     fuse_rms_norm_into_linears(gm)
+    fuse_rotary_into_projections(gm)
+    fuse_residual_into_linears(gm)
     return gm

@@ -497,9 +497,175 @@ def rms_glu_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, w_gate, b_ga
     return rms_linear_layer(x, _rms_weight_like(x, rms_weight), eps, weight, bias, activation, gated=True)
 
 
+def linear_residual_wrapper(v: torch.Tensor, weight: torch.Tensor, bias, residual: torch.Tensor):
+    """residual + linear(v, weight, bias): the attention-output and feed-forward-down projections of a decoder layer with
+    the addition that follows them.  Decoding steps (at most 64 rows) run it as one launch; larger inputs as the linear
+    kernel and the addition they were.  No counterpart in the reference, whose model adds in eager PyTorch
+    (experimental/llama-v2/llama/model.py:262-264)."""
+    from kernl_amd.implementations.linear_layer import decode_linear_layer, decode_linear_supported
+
+    if weight.dtype == torch.float32 and (v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")):
+        weight.data = weight.data.half()
+    if bias is not None and bias.dtype == torch.float32 and (v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")):
+        bias.data = bias.data.half()
+    if (
+        decode_linear_supported(v, weight)
+        and residual.dtype == v.dtype
+        and residual.shape[:-1] == v.shape[:-1]
+        and residual.shape[-1] == weight.shape[0]
+        and (bias is None or bias.dtype == v.dtype)
+        and not torch.is_autocast_enabled("cuda")
+    ):
+        return decode_linear_layer(v, weight, bias, residual=residual)
+    return residual + linear_wrapper_functional(v, weight, bias)
+
+
+def rms_fused_linear_rope_wrapper(x: torch.Tensor, rms_weight, eps: float, weights, biases, cos, sin, n_rotated: int, head_dim: int):
+    """rms_fused_linear_wrapper(x, ...) with the rotary embedding of its first `n_rotated` outputs (query and key) applied
+    head by head: outputs [.., heads_i * head_dim] as before, the rotated ones already rotated.  A decoding step runs
+    norm, product and rotation as ONE launch (reference: `rms_matmul_rbe_qkv_wrapper`,
+    experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:289-344); larger inputs run the kernels they ran before.
+    cos, sin: [batch | 1, 1, positions, head_dim] as Hugging Face decoders hand them to `apply_rotary_pos_emb`."""
+    from kernl_amd.implementations.linear_layer import decode_linear_layer, decode_linear_supported
+    from kernl_amd.implementations.rotary import rotary_forward
+
+    weight, bias, sizes = _concatenated_params(x, weights, biases)
+    fast = (
+        x.dim() == 3
+        and _rms_fusable(x, rms_weight)
+        and decode_linear_supported(x, weight)
+        and (bias is None or bias.dtype == x.dtype)
+        and cos.dim() == 4 and cos.shape == sin.shape and cos.dtype == sin.dtype and cos.shape[1] == 1
+        and cos.shape[2] == x.shape[1] and cos.shape[3] == head_dim and cos.shape[0] in (1, x.shape[0])
+        and cos.stride(-1) == 1 and sin.stride() == cos.stride()
+        and cos.dtype in (torch.float16, torch.bfloat16, torch.float32)
+        and head_dim % 32 == 0 and all(n % head_dim == 0 for n in sizes)
+    )
+    if fast:
+        out = decode_linear_layer(x, weight, bias, _rms_weight_like(x, rms_weight), eps, None, cos.squeeze(1), sin.squeeze(1),
+                                  head_dim=head_dim, rope_cols=sum(sizes[:n_rotated]))
+        return tuple(torch.split(out, sizes, dim=-1))
+    outs = list(rms_fused_linear_wrapper(x, rms_weight, eps, weights, biases))
+    for i in range(n_rotated):
+        o = outs[i]
+        heads = o.reshape(*o.shape[:-1], -1, head_dim).transpose(-3, -2)        # [.., heads, positions, head_dim], a view
+        outs[i] = rotary_forward(heads, cos, sin).transpose(-3, -2).reshape(o.shape)
+    return tuple(outs)
+
+
 torch.fx.wrap("rms_linear_wrapper")
 torch.fx.wrap("rms_fused_linear_wrapper")
 torch.fx.wrap("rms_glu_linear_wrapper")
+torch.fx.wrap("linear_residual_wrapper")
+torch.fx.wrap("rms_fused_linear_rope_wrapper")
+
+
+def fuse_residual_into_linears(gm: torch.fx.GraphModule):
+    """`residual + linear_wrapper_functional(v, w, b)` (either operand order, no activation, the product consumed by the
+    addition only) becomes one `linear_residual_wrapper` call.  Runs after the linear passes."""
+    import operator
+
+    changed = False
+    for node in list(gm.graph.nodes):
+        if not (node.op == "call_function" and node.target in (operator.add, torch.add) and len(node.args) == 2 and not node.kwargs):
+            continue
+        for lin, res in (node.args, node.args[::-1]):
+            if not (isinstance(lin, torch.fx.Node) and isinstance(res, torch.fx.Node)):
+                continue
+            if not (lin.op == "call_function" and lin.target is linear_wrapper_functional and len(lin.users) == 1):
+                continue
+            if len(lin.args) != 3 or lin.kwargs.get("activation", "") != "" or set(lin.kwargs) - {"activation"}:
+                continue
+            if res is lin:
+                continue
+            with gm.graph.inserting_before(node):
+                fused = gm.graph.call_function(linear_residual_wrapper, tuple(lin.args) + (res,))
+            fused.meta = dict(node.meta)
+            node.replace_all_uses_with(fused)
+            gm.graph.erase_node(node)
+            gm.graph.erase_node(lin)
+            changed = True
+            break
+    if changed:
+        gm.graph.lint()
+        gm.recompile()
+
+
+def fuse_rotary_into_projections(gm: torch.fx.GraphModule):
+    """The rotary embedding of the query and key projections moves into the fused projection that produces them:
+
+        f = rms_fused_linear_wrapper(x, g, eps, [wq, wk, wv], biases);  q = f[0].view(B, S, -1, D).transpose(1, 2)
+        rotary_wrapper(q, cos, sin), rotary_wrapper(k, cos, sin)
+
+    becomes `rms_fused_linear_rope_wrapper(x, g, eps, weights, biases, cos, sin, 2, D)` with the views reading its
+    outputs directly.  The rotated outputs must be a leading run of the projection's outputs, each consumed only
+    through that view / transpose chain, all with the same tables.  Runs after `fuse_rms_norm_into_linears`."""
+    import operator
+
+    from kernl_amd.optimizer.rotary import rotary_wrapper
+
+    def chain_of(part: torch.fx.Node):
+        """part = f[i] -> view(.., D) -> transpose(1, 2) -> rotary_wrapper: returns (rotary node, cos, sin, D) or None."""
+        if len(part.users) != 1:
+            return None
+        view = next(iter(part.users))
+        if not (view.op == "call_method" and view.target in ("view", "reshape") and view.args[0] is part and len(view.users) == 1):
+            return None
+        shape = view.args[1] if len(view.args) == 2 and isinstance(view.args[1], (tuple, list)) else view.args[1:]
+        if len(shape) != 4 or not isinstance(shape[-1], int) or shape[-1] <= 0:
+            return None
+        tr = next(iter(view.users))
+        if not (tr.op == "call_method" and tr.target == "transpose" and tuple(tr.args[1:]) in ((1, 2), (2, 1)) and len(tr.users) == 1):
+            return None
+        rot = next(iter(tr.users))
+        if not (rot.op == "call_function" and rot.target is rotary_wrapper and rot.args[0] is tr and len(rot.args) == 3):
+            return None
+        return rot, rot.args[1], rot.args[2], shape[-1]
+
+    changed = False
+    for node in list(gm.graph.nodes):
+        if not (node.op == "call_function" and node.target is rms_fused_linear_wrapper and len(node.args) == 5):
+            continue
+        parts = {}
+        for user in node.users:
+            if user.op == "call_function" and user.target is operator.getitem and isinstance(user.args[1], int):
+                parts[user.args[1]] = user
+        if len(parts) != len(node.users):
+            continue
+        chains = []
+        for i in range(len(parts)):
+            c = chain_of(parts[i]) if i in parts else None
+            if c is None:
+                break
+            if chains and (c[1] is not chains[0][1] or c[2] is not chains[0][2] or c[3] != chains[0][3]):
+                break
+            chains.append(c)
+        if not chains:
+            continue
+        _, cos, sin, head_dim = chains[0]
+        # the tables must be computed before the projection for the fused call to take them: a table node that follows
+        # the projection (Hugging Face unsqueezes them after it) moves up when its own inputs allow that
+        order = {n: i for i, n in enumerate(gm.graph.nodes)}
+        movable = all(
+            order[t] < order[node] or all(order[inp] < order[node] for inp in t.all_input_nodes) for t in (cos, sin)
+        )
+        if not movable:
+            continue
+        for t in dict.fromkeys((cos, sin)):
+            if order[t] > order[node]:
+                node.prepend(t)
+        with gm.graph.inserting_before(node):
+            fused = gm.graph.call_function(rms_fused_linear_rope_wrapper, tuple(node.args) + (cos, sin, len(chains), head_dim))
+        fused.meta = dict(node.meta)
+        node.replace_all_uses_with(fused)
+        gm.graph.erase_node(node)
+        for rot, _, _, _ in chains:
+            rot.replace_all_uses_with(rot.args[0])
+            gm.graph.erase_node(rot)
+        changed = True
+    if changed:
+        gm.graph.lint()
+        gm.recompile()
 
 
 def fuse_rms_norm_into_linears(gm: torch.fx.GraphModule):

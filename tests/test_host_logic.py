@@ -355,18 +355,25 @@ def test_llama_graph_rewrite_and_constant_causal_mask():
         assert t.count(fused) == 2
         # the two norms of every layer are folded into the projections they feed; the final norm stays
         assert t.count("layer_norm_rms_wrapper") == 1 and "rsqrt" not in t
-        assert t.count("rms_fused_linear_wrapper") == 2 and "silu" not in t and "softmax" not in t
+        assert "silu" not in t and "softmax" not in t
         # SwiGLU: gate and up projections and their product are one gated GEMM per layer
-        assert t.count("rms_glu_linear_wrapper") == 2 and t.count("linear_wrapper_functional") == 2 * 2
+        assert t.count("rms_glu_linear_wrapper") == 2
         assert "fused_linear_wrapper" not in t and "glu_linear_wrapper" not in t
-        # rotary embedding: one fused call each for queries and keys per layer, nothing left of rotate_half
-        assert t.count("rotary_wrapper") == 2 * 2 and "neg" not in t
+        # rotary embedding: rotated inside the query/key/value projection (two of its three outputs, head size 64),
+        # nothing left of rotate_half nor of a rotation kernel of its own
+        assert t.count("rms_fused_linear_rope_wrapper") == 2 and "rms_fused_linear_wrapper" not in t
+        assert "rotary_wrapper" not in t and "neg" not in t
+        # the additions after the attention-output and feed-forward-down projections ride in those projections
+        assert t.count("linear_residual_wrapper") == 2 * 2 and "linear_wrapper_functional" not in t
+        assert t.count("add") == 1                      # position ids; no residual addition is left
         # the fresh key/value cache no longer copies: the only cat left builds the angle table
         assert t.count("cat") == 1
         for node in graphs[0].graph.nodes:
+            if node.op == "call_function" and node.target.__name__ == "rms_fused_linear_rope_wrapper":
+                assert node.args[7:] == (2, 64) and node.args[5].target == "unsqueeze" and node.args[6].target == "unsqueeze"
             if node.op == "call_function" and node.target.__name__ == fused:
                 assert node.args[mask_idx] is None and node.args[5] is True
-                assert node.args[0].target.__name__ == "rotary_wrapper" and node.args[1].target.__name__ == "rotary_wrapper"
+                assert node.args[0].target == "transpose" and node.args[1].target == "transpose"
     torch._dynamo.reset()
 
 

@@ -293,3 +293,89 @@ def test_activation_curve_through_identity_weights(activation):
     bound = 4e-5 + 1.0e-3 * ref.abs()  # approximation error + one fp16 rounding (2^-11 relative, with slack)
     worst = (err - bound).max().item()
     assert worst <= 0, f"{activation}: error exceeds bound by {worst:.3e} at x={x.float().flatten()[(err - bound).argmax()].item()}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("table_dtype", ["same", "fp32"])
+@pytest.mark.parametrize(
+    "case",
+    # batch, positions, K, heads (query + key + value), head size, rotated heads, bias, residual
+    [(1, 1, 4096, 96, 128, 64, False, False), (4, 1, 512, 12, 64, 8, True, False), (2, 3, 256, 6, 128, 4, False, True),
+     (33, 1, 320, 9, 32, 9, True, True), (1, 64, 128, 3, 64, 2, False, False), (5, 2, 192, 4, 96, 0, True, True)],
+    ids=lambda c: "x".join(str(int(v)) for v in c),
+)
+def test_decode_projection_with_norm_rotation_and_residual(case, table_dtype, dtype, close):
+    """A decoding step's query/key/value projection in one launch: RMSNorm prologue, the product, rotation of the query
+    and key heads, residual (reference: `rms_matmul_rbe_qkv`, experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:250-347)
+    against the composition of the RMSNorm, linear and rotary oracles."""
+    from kernl_amd.implementations.linear_layer import decode_linear_layer
+    from oracle import rms_norm_oracle, rotary_oracle
+
+    B, S, K, heads, D, rot_heads, with_bias, with_residual = case
+    N = heads * D
+    gen = torch.Generator().manual_seed(43)
+    x = (torch.randn((B, S, K), generator=gen) * 2.0 + 0.3).to(dtype)
+    g = (1.0 + 0.2 * torch.randn((K,), generator=gen)).to(dtype)
+    w = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+    b = (0.5 * torch.randn((N,), generator=gen)).to(dtype) if with_bias else None
+    res = torch.randn((B, S, N), generator=gen).to(dtype) if with_residual else None
+    tdt = dtype if table_dtype == "same" else torch.float32
+    angles = torch.rand((B, S, D), generator=gen) * 6.28          # per batch entry AND position, both halves independent
+    cos, sin = angles.cos().to(tdt), angles.sin().to(tdt)
+    eps = 1e-5 if dtype == torch.bfloat16 else 1.6e-5
+    out = decode_linear_layer(x.cuda(), w.cuda(), None if b is None else b.cuda(), g.cuda(), eps,
+                              None if res is None else res.cuda(), cos.cuda(), sin.cuda(), head_dim=D, rope_cols=rot_heads * D)
+    torch.cuda.synchronize()
+    y = linear_oracle(rms_norm_oracle(x, g, eps), w, b, "")                        # [B, S, N] fp32
+    heads_view = y.reshape(B, S, heads, D)
+    rotated = rotary_oracle(heads_view[:, :, :rot_heads], cos[:, :, None, :], sin[:, :, None, :])
+    ref = torch.cat((rotated, heads_view[:, :, rot_heads:]), dim=2).reshape(B, S, N)
+    if res is not None:
+        ref = ref + res.float()
+    assert out.shape == (B, S, N) and out.dtype == dtype
+    close(out, ref, dtype, scale="magnitude", what=f"decode projection {case}")
+    # tables shared by the batch ([1, S, D]) are read with a zero batch stride
+    out1 = decode_linear_layer(x.cuda(), w.cuda(), None if b is None else b.cuda(), g.cuda(), eps,
+                               None if res is None else res.cuda(), cos[:1].cuda(), sin[:1].cuda(), head_dim=D, rope_cols=rot_heads * D)
+    torch.cuda.synchronize()
+    rotated1 = rotary_oracle(heads_view[:, :, :rot_heads], cos[:1, :, None, :], sin[:1, :, None, :])
+    ref1 = torch.cat((rotated1, heads_view[:, :, rot_heads:]), dim=2).reshape(B, S, N)
+    close(out1, ref1 if res is None else ref1 + res.float(), dtype, scale="magnitude", what=f"decode projection, shared tables {case}")
+
+
+@pytest.mark.parametrize("with_norm", [False, True], ids=["plain", "rms"])
+@pytest.mark.parametrize("shape", [(1, 4096, 11008), (7, 768, 3072), (40, 8192, 512), (64, 96, 64)], ids=lambda s: "x".join(map(str, s)))
+def test_decode_projection_with_residual_only(shape, with_norm, close):
+    """out = residual + linear(x) (the attention-output and feed-forward-down projections of a decoding step), with and
+    without the RMSNorm prologue; every grid rule of the few-row kernel is in the list."""
+    from kernl_amd.implementations.linear_layer import decode_linear_layer
+    from oracle import rms_norm_oracle
+
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(47)
+    x, w, b = _inputs(M, N, K, torch.float16, gen, w_std=K ** -0.5)
+    res = torch.randn((M, N), generator=gen).half()
+    g = (1.0 + 0.2 * torch.randn((K,), generator=gen)).half() if with_norm else None
+    out = decode_linear_layer(x.cuda(), w.cuda(), b.cuda(), None if g is None else g.cuda(), 1.6e-5, res.cuda())
+    torch.cuda.synchronize()
+    xin = rms_norm_oracle(x, g, 1.6e-5) if with_norm else x
+    close(out, linear_oracle(xin, w, b, "") + res.float(), scale="magnitude", what=f"residual projection {shape}")
+
+
+def test_decode_projection_rejections():
+    from kernl_amd import _lib
+    from kernl_amd.implementations.linear_layer import decode_linear_layer, decode_linear_supported
+
+    x = torch.zeros((65, 128), dtype=torch.half, device="cuda")
+    w = torch.zeros((128, 128), dtype=torch.half, device="cuda")
+    assert not decode_linear_supported(x, w) and decode_linear_supported(x[:64], w) and not decode_linear_supported(x[:4, :96], w[:, :96])
+    with pytest.raises(AssertionError):
+        decode_linear_layer(x, w)
+    g = torch.ones((128,), dtype=torch.half, device="cuda")
+    t = torch.zeros((1, 4, 48), dtype=torch.half, device="cuda")
+    with pytest.raises(AssertionError):   # head size 48 is no multiple of 32
+        decode_linear_layer(x[:4], w, None, g, 1e-5, None, t, t, head_dim=48, rope_cols=96)
+    out = torch.empty((4, 128), dtype=torch.half, device="cuda")
+    t64 = torch.zeros((1, 4, 64), dtype=torch.half, device="cuda")
+    with pytest.raises(_lib.KernlLibraryError, match="RMSNorm prologue"):
+        _lib.linear_decode_fwd(x[:4], None, 0.0, w, None, None, out, t64, t64, 64, 64, 4)

@@ -171,21 +171,29 @@ def test_llama_shaped_decoder_matches_fp32_eager(attn):
 
 
 def test_llama_shaped_short_input_runs_the_one_launch_norm_projections(monkeypatch):
-    """24 tokens (at most 64 rows): both RMSNorms of every layer run inside the projections they feed
-    (`kernl_linear_rms_fwd`: fused query/key/value and the gated feed-forward entry), the result still matches the
-    fp32 model."""
+    """24 tokens (at most 64 rows): both RMSNorms of every layer run inside the projections they feed — the fused
+    query/key/value projection together with the rotation of queries and keys (`kernl_linear_decode_fwd`), the gated
+    feed-forward entry (`kernl_linear_rms_fwd`) — the two residual additions of every layer ride in the projections
+    before them, and the result still matches the fp32 model."""
     from kernl_amd import _lib
     from kernl_amd.model_optimization import optimize_model
 
     torch._dynamo.reset()
-    calls = {"rms": 0, "gated": 0}
+    calls = {"rms": 0, "gated": 0, "rotating": 0, "residual": 0}
     real = _lib.linear_rms_fwd
+    real_decode = _lib.linear_decode_fwd
 
     def counting(x2d, rms_weight, eps, weight, bias, out2d, activation, gated):
         calls["rms"] += 1
         calls["gated"] += int(bool(gated))
         return real(x2d, rms_weight, eps, weight, bias, out2d, activation, gated)
 
+    def counting_decode(x2d, rms_weight, eps, weight, bias, residual2d, out2d, cos=None, sin=None, *args, **kwargs):
+        calls["rotating"] += int(cos is not None and rms_weight is not None)
+        calls["residual"] += int(residual2d is not None)
+        return real_decode(x2d, rms_weight, eps, weight, bias, residual2d, out2d, cos, sin, *args, **kwargs)
+
+    monkeypatch.setattr(_lib, "linear_decode_fwd", counting_decode)
     monkeypatch.setattr(_lib, "linear_rms_fwd", counting)
     gen = torch.Generator().manual_seed(6)
     ids = torch.randint(0, 1000, (2, 12), generator=gen)
@@ -200,8 +208,9 @@ def test_llama_shaped_short_input_runs_the_one_launch_norm_projections(monkeypat
         out = model(input_ids=ids.cuda(), use_cache=False).last_hidden_state
         out = model(input_ids=ids.cuda(), use_cache=False).last_hidden_state
         torch.cuda.synchronize()
-    # warm-up and capture each run the two layers once: 2 x 2 x (one fused q/k/v + one gated feed-forward entry)
-    assert calls["rms"] == 8 and calls["gated"] == 4, calls
+    # warm-up and capture each run the two layers once: 2 x 2 x (one rotating q/k/v projection, one gated feed-forward
+    # entry, two projections with a residual)
+    assert calls == {"rms": 4, "gated": 4, "rotating": 4, "residual": 8}, calls
     ours_rel = ((out.float().cpu() - ref).abs().mean() / ref.abs().mean()).item()
     print(f"llama-shaped, 24 rows: mean_rel ours={ours_rel:.5f}", flush=True)
     assert torch.isfinite(out).all() and ours_rel <= 5e-3 + clamp_rel
