@@ -556,7 +556,10 @@ __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_
     }
 }
 
-template <typename T, int ACT, int NBN>
+// W8: the weight is stored as one byte per element (fp8 e5m2, the upper byte of the fp16 encoding).  Its tile travels
+// HBM -> LDS as bytes (half the loads, 64-byte rows, chunks swizzled for 8-byte reads), a fragment is read as 8 bytes
+// and widened by four byte-permutes two read slots later, all in the shadow of the MFMAs; everything else is unchanged.
+template <typename T, int ACT, int NBN, bool W8 = false>
 __global__ void __launch_bounds__(256, 1)
 linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
                    T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
@@ -570,7 +573,10 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     // plus an immediate of 0 or 32 KB for the stage (the immediate field of an LDS read ends at 64 KB - 1).
     constexpr int X_BYTES = BM * RB, W_BYTES = 32768, W_BASE = 2 * X_BYTES;
     static_assert(X_BYTES == 32768 && BN * RB <= W_BYTES, "stage immediates");
-    constexpr int LOADS = BM * CPR / 256, LOADS_W = BN * CPR / 256;  // 1 KB loads per wave for the x and the w tile
+    static_assert(!W8 || (std::is_same<T, f16>::value && NBN == 8 && !GATED), "one-byte weights: fp16, 256 columns, plain");
+    constexpr int WB = W8 ? 1 : 2;                                   // bytes per weight element in memory and in LDS
+    constexpr int RBW = BK * WB, CPRW = RBW / 16;                    // weight tile: row bytes, 16-byte chunks per row
+    constexpr int LOADS = BM * CPR / 256, LOADS_W = BN * CPRW / 256;  // 1 KB loads per wave for the x and the w tile
     constexpr int NL = LOADS + LOADS_W;                             // tile loads per wave and k-tile
     constexpr int GROUP_M = 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -613,13 +619,14 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     auto set_load_tile = [&](bool valid, int m0, int n0) __attribute__((always_inline)) {
         const int rows_x = valid ? min(BM, M - m0) : 0, rows_w = valid ? min(BN, N - n0) : 0;
         if (valid) {
-            const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx), waddr = (uint64_t)(uintptr_t)(W + (int64_t)n0 * K);
+            const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx);
+            const uint64_t waddr = (uint64_t)(uintptr_t)(reinterpret_cast<const char *>(W) + (int64_t)n0 * K * WB);
             xrsrc[0] = (uint32_t)xaddr;
             xrsrc[1] = (uint32_t)(xaddr >> 32) & 0xFFFFu;
             xrsrc[2] = (uint32_t)((((int64_t)rows_x - 1) * ldx + K) * 2);
             wrsrc[0] = (uint32_t)waddr;
             wrsrc[1] = (uint32_t)(waddr >> 32) & 0xFFFFu;
-            wrsrc[2] = (uint32_t)((int64_t)rows_w * K * 2);
+            wrsrc[2] = (uint32_t)((int64_t)rows_w * K * WB);
         }
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
@@ -630,31 +637,31 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 #pragma unroll
         for (int i = 0; i < LOADS_W; ++i) {
             const int q = (wave * LOADS_W + i) * 64 + lane;
-            const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+            const int row = q / CPRW, c = swz_chunk<RBW>(row, q % CPRW);
             // LDS row `row` is MFMA row r = row % 16 of n-block row / 16; see the placement rule above the kernel
             const int wrow = wide_weight_row<GATED, NBN>(row);
-            wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
+            wd[i] = wrow < rows_w ? (uint32_t)((int64_t)wrow * K * WB + c * 16) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
         }
     };
     typedef __attribute__((address_space(3))) void lds_void;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
     // inline assembly on purpose: the compiler would make every later LDS read wait for loads it sees writing LDS.
     // `group` (0 or 1) selects loads 4 group .. 4 group + 3; its first load writes the LDS base register.
-    auto load4 = [&](const u32x4 &rsrc, uint32_t off, uint32_t lds, int group, int part, int k0) __attribute__((always_inline)) {
+    auto load4 = [&](const u32x4 &rsrc, uint32_t off, uint32_t lds, int group, int part, int kbytes) __attribute__((always_inline)) {
         if (part == 0)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :: "s"(lds + group * 4096), "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory", "m0");
+                         :: "s"(lds + group * 4096), "v"(off), "s"(rsrc), "s"(kbytes) : "memory", "m0");
         else if (part == 1)
-            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
         else if (part == 2)
-            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:2048 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:2048 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
         else
-            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
     };
     // load l (0 .. NL-1) of a k-tile: the x loads, then the w loads
     auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
-        if (l < LOADS) load4(xrsrc, xd[l], lds_base + stage * X_BYTES + wave * (LOADS * 1024), l >> 2, l & 3, k0);
-        else load4(wrsrc, wd[l - LOADS], lds_base + W_BASE + stage * W_BYTES + wave * (LOADS_W * 1024), (l - LOADS) >> 2, l & 3, k0);
+        if (l < LOADS) load4(xrsrc, xd[l], lds_base + stage * X_BYTES + wave * (LOADS * 1024), l >> 2, l & 3, k0 * 2);
+        else load4(wrsrc, wd[l - LOADS], lds_base + W_BASE + stage * W_BYTES + wave * (LOADS_W * 1024), (l - LOADS) >> 2, (l - LOADS) & 3, k0 * WB);
     };
 
     // LDS addresses of this lane's operand fragments in stage 0, one register per (k-step, block): with a whole
@@ -668,10 +675,22 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 #pragma unroll
         for (int i = 0; i < NB; ++i) xfrag[st][i] = (lds_frag)(lds0 + swz_offset<RB>(wave_m * 128 + i * 16 + l16, 4 * st + g));
 #pragma unroll
-        for (int j = 0; j < NBN; ++j)
-            wfrag[st][j] = (lds_frag)(lds0 + W_BASE + swz_offset<RB>(wave_n * (NBN * 16) + j * 16 + l16, 4 * st + g));
+        for (int j = 0; j < NBN; ++j) {
+            const int row = wave_n * (NBN * 16) + j * 16 + l16, unit = 4 * st + g;   // 8 k-values per unit
+            wfrag[st][j] = W8 ? (lds_frag)(lds0 + W_BASE + swz_offset<RBW>(row, unit >> 1) + (unit & 1) * 8)
+                              : (lds_frag)(lds0 + W_BASE + swz_offset<RBW>(row, unit));
+        }
     }
     constexpr int STAGE_FRAGS = X_BYTES / 16;  // pointer increment that selects stage 1
+    // one-byte weights: 8 bytes per fragment, widened (byte b of a dword becomes the 16-bit value b << 8)
+    typedef __attribute__((address_space(3))) const u32x2 *lds_frag8;
+    auto read8 = [&](lds_frag ptr) __attribute__((always_inline)) -> u32x2 { return *(lds_frag8)ptr; };
+    auto widen8 = [&](u32x2 raw) __attribute__((always_inline)) -> vec8 {
+        const u32x4 wide = {__builtin_amdgcn_perm(0u, raw[0], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[0], 0x030c020cu),
+                            __builtin_amdgcn_perm(0u, raw[1], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[1], 0x030c020cu)};
+        return __builtin_bit_cast(vec8, wide);
+    };
+    u32x2 wraw[W8 ? NBN : 1];
 
     const int nk = K / BK;
     int idx = (int)(blockIdx.x >> 3);  // position of the tile being multiplied in this XCD's run
@@ -702,7 +721,10 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 
     vec8 fa[KSTEPS][NBN], fb[KSTEPS][NB];  // weight and activation fragments, one register set per k-step
 #pragma unroll
-    for (int j = 0; j < NBN; ++j) fa[0][j] = *wfrag[0][j];
+    for (int j = 0; j < NBN; ++j) {
+        if constexpr (W8) fa[0][j] = widen8(read8(wfrag[0][j]));
+        else fa[0][j] = *wfrag[0][j];
+    }
 #pragma unroll
     for (int i = 0; i < NB; ++i) fb[0][i] = *xfrag[0][i];
 
@@ -730,8 +752,15 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
                 const int slot = m / PERIOD;
                 if (m % PERIOD == 0 && slot < NBN + NB) {
                     // the weight fragments first: the first MFMAs of the next k-step need all of them
-                    if (slot < NBN) fa[sn][slot] = *(wfrag[sn][slot] + src);
-                    else fb[sn][slot - NBN] = *(xfrag[sn][slot - NBN] + src);
+                    if (slot < NBN) {
+                        // (stage offsets are in 16-byte units of the 16-bit layout: a byte-weight stage is W_BYTES further all the same)
+                        if constexpr (W8) wraw[slot] = read8(wfrag[sn][slot] + src);
+                        else fa[sn][slot] = *(wfrag[sn][slot] + src);
+                    } else {
+                        fb[sn][slot - NBN] = *(xfrag[sn][slot - NBN] + src);
+                    }
+                } else if (W8 && m % PERIOD == 1 && slot >= 2 && slot - 2 < NBN) {
+                    fa[sn][slot - 2] = widen8(wraw[slot - 2]);  // two read slots later: the bytes have arrived
                 } else if (m % PERIOD == PERIOD - 2 && st == 1 && slot < NL) {
                     tile_load(slot, CUR, k0);
                 }
@@ -800,7 +829,7 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 // 16 KB (x) + 32 KB (w), k-tile T + 3 requested while k-tile T is multiplied, the wait in front of the second k-step
 // only for k-tile T + 1 (vmcnt(NL): the loads of T + 2 may still be in flight).  One workgroup per output tile.
 // ----------------------------------------------------------------------------------------------------
-template <typename T, int ACT, int NBN>
+template <typename T, int ACT, int NBN, bool W8 = false>
 __global__ void __launch_bounds__(256, 1)
 linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
                         T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs,
@@ -811,7 +840,9 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     constexpr int NBM = 4, BM = 32 * NBM, BN = 32 * NBN, BK = 64, RB = BK * 2, CPR = BK / 8, KSTEPS = BK / 32;
     constexpr int X_STAGE = BM * RB, W_STAGE = 32768, W_BASE = 3 * X_STAGE;  // [x0|x1|x2|w0|w1|w2]
     static_assert(X_STAGE == 16384 && BN * RB <= W_STAGE, "stage immediates");
-    constexpr int LOADS_X = BM * CPR / 256, LOADS_W = BN * CPR / 256, NL = LOADS_X + LOADS_W;
+    static_assert(!W8 || (std::is_same<T, f16>::value && NBN == 8), "one-byte weights: fp16, 256 columns");
+    constexpr int WB = W8 ? 1 : 2, RBW = BK * WB, CPRW = RBW / 16;  // weight tile: bytes per element, row bytes, chunks per row
+    constexpr int LOADS_X = BM * CPR / 256, LOADS_W = BN * CPRW / 256, NL = LOADS_X + LOADS_W;
     static_assert(LOADS_X == 4, "one group of four loads for the x tile");
     constexpr int GROUP_M = 8;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -835,10 +866,11 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     // tile loads, as in the wide kernel: every lane fetches the chunk that belongs at its LDS position
     constexpr uint32_t kOutOfRange = 0x80000000u;
     const int rows_x = min(BM, M - m0), rows_w = min(BN, N - n0);
-    const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx), waddr = (uint64_t)(uintptr_t)(W + (int64_t)n0 * K);
+    const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx);
+    const uint64_t waddr = (uint64_t)(uintptr_t)(reinterpret_cast<const char *>(W) + (int64_t)n0 * K * WB);
     const u32x4 xrsrc = {(uint32_t)xaddr, (uint32_t)(xaddr >> 32) & 0xFFFFu,
                          (uint32_t)((((int64_t)rows_x - 1) * ldx + K) * 2), 0x00020000u};
-    const u32x4 wrsrc = {(uint32_t)waddr, (uint32_t)(waddr >> 32) & 0xFFFFu, (uint32_t)((int64_t)rows_w * K * 2),
+    const u32x4 wrsrc = {(uint32_t)waddr, (uint32_t)(waddr >> 32) & 0xFFFFu, (uint32_t)((int64_t)rows_w * K * WB),
                          0x00020000u};
     uint32_t xd[LOADS_X], wd[LOADS_W];
 #pragma unroll
@@ -850,26 +882,26 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
 #pragma unroll
     for (int i = 0; i < LOADS_W; ++i) {
         const int q = (wave * LOADS_W + i) * 64 + lane;
-        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        const int row = q / CPRW, c = swz_chunk<RBW>(row, q % CPRW);
         const int wrow = wide_weight_row<false, NBN>(row);
-        wd[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * 2) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
+        wd[i] = wrow < rows_w ? (uint32_t)((int64_t)wrow * K * WB + c * 16) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
     }
     typedef __attribute__((address_space(3))) void lds_void;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
-    auto load4 = [&](const u32x4 &rsrc, uint32_t off, uint32_t lds, int group4, int part, int k0) __attribute__((always_inline)) {
+    auto load4 = [&](const u32x4 &rsrc, uint32_t off, uint32_t lds, int group4, int part, int kbytes) __attribute__((always_inline)) {
         if (part == 0)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :: "s"(lds + group4 * 4096), "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory", "m0");
+                         :: "s"(lds + group4 * 4096), "v"(off), "s"(rsrc), "s"(kbytes) : "memory", "m0");
         else if (part == 1)
-            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
         else if (part == 2)
-            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:2048 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:2048 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
         else
-            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off), "s"(rsrc), "s"(k0 * 2) : "memory");
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
     };
     auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
-        if (l < LOADS_X) load4(xrsrc, xd[l], lds_base + stage * X_STAGE + wave * (LOADS_X * 1024), 0, l, k0);
-        else load4(wrsrc, wd[l - LOADS_X], lds_base + W_BASE + stage * W_STAGE + wave * (LOADS_W * 1024), (l - LOADS_X) >> 2, (l - LOADS_X) & 3, k0);
+        if (l < LOADS_X) load4(xrsrc, xd[l], lds_base + stage * X_STAGE + wave * (LOADS_X * 1024), 0, l, k0 * 2);
+        else load4(wrsrc, wd[l - LOADS_X], lds_base + W_BASE + stage * W_STAGE + wave * (LOADS_W * 1024), (l - LOADS_X) >> 2, (l - LOADS_X) & 3, k0 * WB);
     };
 
     // fragment addresses: x stages are 16 KB apart (immediates 0 / 16 K / 32 K); w stages 32 KB apart, and an LDS
@@ -884,7 +916,9 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
         for (int i = 0; i < NBM; ++i) xfrag[st][i] = (lds_frag)(lds0 + swz_offset<RB>(wave_m * (NBM * 16) + i * 16 + l16, 4 * st + g));
 #pragma unroll
         for (int j = 0; j < NBN; ++j) {
-            wfrag[st][j] = (lds_frag)(lds0 + W_BASE + swz_offset<RB>(wave_n * (NBN * 16) + j * 16 + l16, 4 * st + g));
+            const int row = wave_n * (NBN * 16) + j * 16 + l16, unit = 4 * st + g;   // 8 k-values per unit
+            wfrag[st][j] = W8 ? (lds_frag)(lds0 + W_BASE + swz_offset<RBW>(row, unit >> 1) + (unit & 1) * 8)
+                              : (lds_frag)(lds0 + W_BASE + swz_offset<RBW>(row, unit));
             wfrag2[st][j] = wfrag[st][j] + 2 * (W_STAGE / 16);
         }
     }
@@ -899,9 +933,20 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * NL) & 15) | (((2 * NL) >> 4) << 14));  // vmcnt(2 NL): k-tile 0 has landed
     __syncthreads();
 
+    // one-byte weights: 8 bytes per fragment, widened (byte b of a dword becomes the 16-bit value b << 8)
+    typedef __attribute__((address_space(3))) const u32x2 *lds_frag8;
+    auto widen8 = [&](u32x2 raw) __attribute__((always_inline)) -> vec8 {
+        const u32x4 wide = {__builtin_amdgcn_perm(0u, raw[0], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[0], 0x030c020cu),
+                            __builtin_amdgcn_perm(0u, raw[1], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[1], 0x030c020cu)};
+        return __builtin_bit_cast(vec8, wide);
+    };
+    u32x2 wraw[W8 ? NBN : 1];
     vec8 fa[KSTEPS][NBN], fb[KSTEPS][NBM];
 #pragma unroll
-    for (int j = 0; j < NBN; ++j) fa[0][j] = *wfrag[0][j];
+    for (int j = 0; j < NBN; ++j) {
+        if constexpr (W8) fa[0][j] = widen8(*(lds_frag8)wfrag[0][j]);
+        else fa[0][j] = *wfrag[0][j];
+    }
 #pragma unroll
     for (int i = 0; i < NBM; ++i) fb[0][i] = *xfrag[0][i];
 
@@ -915,6 +960,10 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     auto read_w = [&](auto s3_c, int st, int j) __attribute__((always_inline)) -> vec8 {
         constexpr int S3 = decltype(s3_c)::value;
         return S3 == 2 ? *wfrag2[st][j] : *(wfrag[st][j] + S3 * (W_STAGE / 16));
+    };
+    auto read_w8 = [&](auto s3_c, int st, int j) __attribute__((always_inline)) -> u32x2 {
+        constexpr int S3 = decltype(s3_c)::value;
+        return S3 == 2 ? *(lds_frag8)wfrag2[st][j] : *(lds_frag8)(wfrag[st][j] + S3 * (W_STAGE / 16));
     };
     auto read_x = [&](auto s3_c, int st, int i) __attribute__((always_inline)) -> vec8 {
         constexpr int S3 = decltype(s3_c)::value;
@@ -937,14 +986,24 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
                 const int slot = m >> 1;
                 if ((m & 1) == 0 && slot < NBN + NBM) {
                     if (st == 0) {
-                        if (slot < NBN) fa[sn][slot] = read_w(IntC<CUR>(), sn, slot);
-                        else fb[sn][slot - NBN] = read_x(IntC<CUR>(), sn, slot - NBN);
+                        if (slot < NBN) {
+                            if constexpr (W8) wraw[slot] = read_w8(IntC<CUR>(), sn, slot);
+                            else fa[sn][slot] = read_w(IntC<CUR>(), sn, slot);
+                        } else {
+                            fb[sn][slot - NBN] = read_x(IntC<CUR>(), sn, slot - NBN);
+                        }
                     } else {
-                        if (slot < NBN) fa[sn][slot] = read_w(IntC<NXT>(), sn, slot);
-                        else fb[sn][slot - NBN] = read_x(IntC<NXT>(), sn, slot - NBN);
+                        if (slot < NBN) {
+                            if constexpr (W8) wraw[slot] = read_w8(IntC<NXT>(), sn, slot);
+                            else fa[sn][slot] = read_w(IntC<NXT>(), sn, slot);
+                        } else {
+                            fb[sn][slot - NBN] = read_x(IntC<NXT>(), sn, slot - NBN);
+                        }
                     }
-                } else if ((m & 1) == 1 && st == 1 && slot < NL) {
-                    tile_load(slot, CUR, k_next);
+                } else if ((m & 1) == 1) {
+                    if (st == 1 && slot < NL) tile_load(slot, CUR, k_next);
+                    // one-byte weights: widened two read slots after the read, when the bytes have arrived
+                    if (W8 && slot >= 2 && slot - 2 < NBN) fa[sn][slot - 2] = widen8(wraw[slot - 2]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -1362,6 +1421,9 @@ static void launch_mfma_w8(const LinearArgs &a) {
     }
 }
 
+// one-byte weights on the wide kernel (K % 64 == 0)
+static void launch_wide_w8(const LinearArgs &a);
+
 // gated epilogues: tiles whose waves span an even number of 32-column blocks
 template <typename T, typename Cfg>
 static void launch_mfma_glu(const LinearArgs &a) {
@@ -1375,9 +1437,9 @@ static void launch_mfma_glu(const LinearArgs &a) {
     }
 }
 
-template <typename T, int ACT, int NBN = 8>
+template <typename T, int ACT, int NBN = 8, bool W8 = false>
 static void launch_wide_act(const LinearArgs &a) {
-    auto kern = linear_wide_kernel<T, ACT, NBN>;
+    auto kern = linear_wide_kernel<T, ACT, NBN, W8>;
     constexpr int LDS_BYTES = 2 * (256 + 256) * 128;
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
@@ -1400,9 +1462,32 @@ static void launch_wide_act(const LinearArgs &a) {
                        a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok);
 }
 
-template <typename T, int ACT, int NBN>
+template <typename T, int ACT, int NBN, bool W8>
+static void launch_wide_half_act(const LinearArgs &a);
+static void launch_wide_half_w8(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_wide_half_act<f16, KERNL_ACT_RELU, 8, true>(a); break;
+        case KERNL_ACT_TANH: launch_wide_half_act<f16, KERNL_ACT_TANH, 8, true>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_wide_half_act<f16, KERNL_ACT_GELU_ERF, 8, true>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_wide_half_act<f16, KERNL_ACT_GELU_TANH, 8, true>(a); break;
+        case KERNL_ACT_SILU: launch_wide_half_act<f16, KERNL_ACT_SILU, 8, true>(a); break;
+        default: launch_wide_half_act<f16, KERNL_ACT_NONE, 8, true>(a); break;
+    }
+}
+static void launch_wide_w8(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_wide_act<f16, KERNL_ACT_RELU, 8, true>(a); break;
+        case KERNL_ACT_TANH: launch_wide_act<f16, KERNL_ACT_TANH, 8, true>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_wide_act<f16, KERNL_ACT_GELU_ERF, 8, true>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_wide_act<f16, KERNL_ACT_GELU_TANH, 8, true>(a); break;
+        case KERNL_ACT_SILU: launch_wide_act<f16, KERNL_ACT_SILU, 8, true>(a); break;
+        default: launch_wide_act<f16, KERNL_ACT_NONE, 8, true>(a); break;
+    }
+}
+
+template <typename T, int ACT, int NBN, bool W8 = false>
 static void launch_wide_half_act(const LinearArgs &a) {
-    auto kern = linear_wide_half_kernel<T, ACT, NBN>;
+    auto kern = linear_wide_half_kernel<T, ACT, NBN, W8>;
     constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768;
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
@@ -1775,9 +1860,17 @@ extern "C" int kernl_linear_w8_fwd(const void *x, const void *w8, const void *bi
         launch_skinny<f16, false, true>(a);
         return check_launch("linear (skinny, fp8 weight)");
     }
-    const int ctas_big = (int)(((M + 255) / 256) * ((N + 255) / 256));
-    if (ctas_big >= 192) launch_mfma_w8<Tile256x256>(a);
-    else launch_mfma_w8<Tile128x128>(a);
+    // the tile rule of the 16-bit path: its wide family maps to the wide kernel's 256x256 form, the rest to the 8-wave
+    // kernel (hook values 1 / 3 / 5 of kernl_linear_force_tile choose by hand)
+    int pick = g_linear_force_tile != 0 ? g_linear_force_tile : pick_tile((int)M, (int)N, (int)K, false);
+    if (pick >= 5 && pick <= 8 && K % 64 == 0) {
+        // 128-row tiles where 256-row tiles leave CUs idle, and always for at most 128 rows
+        if (pick >= 7 || (M <= 128 && g_linear_force_tile == 0)) launch_wide_half_w8(a);
+        else launch_wide_w8(a);
+        return check_launch("linear (wide, fp8 weight)");
+    }
+    if (pick == 3 || pick >= 5) launch_mfma_w8<Tile128x128>(a);
+    else launch_mfma_w8<Tile256x256>(a);
     return check_launch("linear (mfma, fp8 weight)");
 }
 

@@ -148,12 +148,14 @@ def test_linear_few_rows_streams_the_weight(shape, activation, dtype, close):
 @pytest.mark.parametrize("activation", ["", "silu"])
 @pytest.mark.parametrize("shape", [(1, 4096, 4096), (5, 80, 64), (16, 1000, 192), (33, 9000, 192), (64, 512, 1024),
                                    (100, 256, 128), (4, 96, 72), (65, 200, 136), (300, 1000, 328), (2048, 2304, 768),
-                                   (1024, 4096, 1024), (7, 64, 100)], ids=lambda s: "x".join(map(str, s)))
+                                   (1024, 4096, 1024), (7, 64, 100), (520, 4096, 1024), (2050, 1100, 512), (300, 700, 192)],
+                         ids=lambda s: "x".join(map(str, s)))
 def test_linear_fp8_weight_storage(shape, activation, close):
     """Weight stored as fp8 e5m2 (reference: `get_model_fp8`, experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84):
     the result must be the oracle's on the DECODED weight.  Up to 64 rows with K % 64 == 0 stream the bytes; more rows,
-    or another K that is a multiple of 8, take the tiled kernel that widens the bytes into LDS (both of its tile
-    shapes are in the list, with ragged edges in every dimension); K = 100 goes through a widened copy."""
+    with K % 64 == 0, take the wide kernels (bytes staged into LDS by the loads themselves, widened at the fragment
+    reads: 256-row and 128-row tiles, ragged edges in both dimensions); another K that is a multiple of 8 takes the
+    8-wave kernel that widens the bytes on their way into LDS; K = 100 goes through a widened copy."""
     from oracle import e5m2_decode_oracle
 
     M, N, K = shape
@@ -379,3 +381,22 @@ def test_decode_projection_rejections():
     t64 = torch.zeros((1, 4, 64), dtype=torch.half, device="cuda")
     with pytest.raises(_lib.KernlLibraryError, match="RMSNorm prologue"):
         _lib.linear_decode_fwd(x[:4], None, 0.0, w, None, None, out, t64, t64, 64, 64, 4)
+
+
+@pytest.mark.parametrize("tile", [1, 3, 5, 7], ids=["8wave-256", "8wave-128", "wide-256", "wide-128"])
+def test_linear_fp8_weight_every_kernel(tile, close):
+    """Each of the four kernels that take one-byte weights beyond 64 rows, forced in turn on a shape with ragged edges."""
+    from oracle import e5m2_decode_oracle
+
+    M, N, K = 700, 1300, 384
+    gen = torch.Generator().manual_seed(31)
+    x, w, b = _inputs(M, N, K, torch.float16, gen, w_std=K ** -0.5)
+    w8 = w.to(torch.float8_e5m2).view(torch.int8)
+    lib = _lib.load()
+    lib.kernl_linear_force_tile(tile)
+    try:
+        out = linear_layer(x.cuda(), w8.cuda(), b.cuda(), activation="fast_gelu")
+        torch.cuda.synchronize()
+    finally:
+        lib.kernl_linear_force_tile(0)
+    close(out, linear_oracle(x, e5m2_decode_oracle(w8), b, "fast_gelu"), what=f"fp8 weight, kernel choice {tile}")
