@@ -52,6 +52,7 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
     constexpr int D = 64, BM = 128, BN = 64, NS = 4;
+    typedef AttnTileMap<D> TileMap;                      // staging and fragment addresses of a K / V tile (index_math.h)
     constexpr int KROW = D * 2, VP = D * 2;              // LDS row bytes of the K tile [key][D] and V tile [key][D]
     constexpr int K_BYTES = BN * KROW, V_BYTES = BN * VP;
     constexpr int DB = D / 32, KS = D / 16;
@@ -102,10 +103,9 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
 #pragma unroll
     for (int i = 0; i < KI; ++i) {
         const int qd = tid + 256 * i;
-        const int row = qd / DC, cs = qd % DC;
-        kdma[i] = (uint32_t)(((int64_t)row * p.ks[2] + swz_chunk<KROW>(row, cs) * 8) * 2);
-        const int vsw = (row >> 1) & 1;
-        vdma[i] = (uint32_t)(((int64_t)row * p.vs[2] + (cs ^ (vsw << 2)) * 8) * 2);
+        const int row = TileMap::stage_row(qd);
+        kdma[i] = (uint32_t)(((int64_t)row * p.ks[2] + TileMap::k_stage_chunk(qd) * 8) * 2);
+        vdma[i] = (uint32_t)(((int64_t)row * p.vs[2] + TileMap::v_stage_chunk(qd) * 8) * 2);
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
     const uint32_t dma_base = lds_base + wave * 1024;
@@ -126,15 +126,9 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
     // LDS byte offsets of this lane's operand fragments (see attention.hip)
     int k_off[KS], vt_off[DB];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) k_off[ks] = swz_offset<KROW>(lr, 2 * ks + lh);
-    {
-        const int i16 = lane & 15, g16 = lane >> 4;
-        const int kq = i16 >> 2;
-        const int fs = rowperm16(16 * (g16 & 1) + 4 * (i16 & 3));
-        const int vsw = kq >> 1;
+    for (int ks = 0; ks < KS; ++ks) k_off[ks] = TileMap::k_frag_offset(lr, lh, ks);
 #pragma unroll
-        for (int d = 0; d < DB; ++d) vt_off[d] = V_RING + (4 * lh + kq) * VP + ((d ^ vsw) * 64) + fs * 2;
-    }
+    for (int d = 0; d < DB; ++d) vt_off[d] = V_RING + TileMap::v_frag_offset(lane, d);
     auto k_frag = [&](int ring_slot, int half, int ks) __attribute__((always_inline)) -> vec8 {
         return *reinterpret_cast<const vec8 *>(smem + ring_slot * K_BYTES + half * 32 * KROW + k_off[ks]);
     };
