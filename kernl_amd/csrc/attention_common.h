@@ -47,9 +47,10 @@ __device__ __forceinline__ float scale_mask(float mv, float clamp) {
 }
 
 
-// Software-pipelined MFMA kernel (attention_pipe.hip).  Handles head size 64 with no mask or with a per-key mask of at
-// most kPipeMaxMaskKeys keys (non-causal), and causal attention without a mask; taken from kPipeMinKeys keys on (or
-// whenever it applies, with `force`).  Returns false when it does not take the problem.
+// Software-pipelined MFMA kernel (attention_pipe.hip).  Handles head sizes 64 and 128 with no mask or with a per-key
+// mask of at most kPipeMaxMaskKeys keys (non-causal), and causal attention without a mask; taken from kPipeMinKeys keys
+// on — head size 128 only for causal problems with few (batch, head) pairs — or whenever it applies, with `force`.
+// Returns false when it does not take the problem.
 static constexpr int kPipeMaxMaskKeys = 2048;
 static constexpr int kPipeMinKeys = 1024;
 bool launch_attention_pipe(const AttnParams &p, int D, int dtype, int mask_mode, bool causal, bool force, hipStream_t st);

@@ -45,13 +45,14 @@
 
 namespace kernl {
 
-template <typename T, int MASK_MODE, bool CAUSAL>
-__global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams p) {
+template <typename T, int D, int MASK_MODE, bool CAUSAL>
+__global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(const AttnParams p) {
     typedef typename Vec8<T>::type vec8;
     typedef __attribute__((address_space(3))) void lds_void;
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    constexpr int D = 64, BM = 128, BN = 64, NS = 4;
+    static_assert(D == 64 || D == 128, "head size 64 (two workgroups per CU) or 128 (one: the rings take 128 KB of LDS)");
+    constexpr int BM = 128, BN = 64, NS = 4;
     typedef AttnTileMap<D> TileMap;                      // staging and fragment addresses of a K / V tile (index_math.h)
     constexpr int KROW = D * 2, VP = D * 2;              // LDS row bytes of the K tile [key][D] and V tile [key][D]
     constexpr int K_BYTES = BN * KROW, V_BYTES = BN * VP;
@@ -69,7 +70,11 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
     typedef BoolC<true> Yes;
     typedef BoolC<false> No;
 
-    __shared__ __attribute__((aligned(16))) unsigned char smem[BIAS_OFF + BIAS_KEYS * 4 + 96];
+    // head size 64 fits the 64 KB a kernel may declare; head size 128 takes its 128 KB of rings as dynamic LDS
+    constexpr int LDS_BYTES = BIAS_OFF + BIAS_KEYS * 4 + 96;
+    __shared__ __attribute__((aligned(16))) unsigned char smem_fixed[D == 64 ? LDS_BYTES : 16];
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_dynamic[];
+    unsigned char *const smem = D == 64 ? smem_fixed : smem_dynamic;
     float *bias_lds = reinterpret_cast<float *>(smem + BIAS_OFF);
     float *red_lds = bias_lds + BIAS_KEYS;                                   // 4 floats: per-wave maxima of a mask row
     int *vote_lds = reinterpret_cast<int *>(smem + BIAS_OFF + BIAS_KEYS * 4 + 16);  // 4 ints: per-wave overflow votes
@@ -181,6 +186,10 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
         asm volatile("global_load_dwordx4 %0, %4, off\n\tglobal_load_dwordx4 %1, %4, off offset:32\n\t"
                      "global_load_dwordx4 %2, %4, off offset:64\n\tglobal_load_dwordx4 %3, %4, off offset:96"
                      : "=&v"(q_raw[0]), "=&v"(q_raw[1]), "=&v"(q_raw[2]), "=&v"(q_raw[3]) : "v"(qrow) : "memory");
+        if constexpr (KS == 8)
+            asm volatile("global_load_dwordx4 %0, %4, off offset:128\n\tglobal_load_dwordx4 %1, %4, off offset:160\n\t"
+                         "global_load_dwordx4 %2, %4, off offset:192\n\tglobal_load_dwordx4 %3, %4, off offset:224"
+                         : "=&v"(q_raw[KS - 4]), "=&v"(q_raw[KS - 3]), "=&v"(q_raw[KS - 2]), "=&v"(q_raw[KS - 1]) : "v"(qrow) : "memory");
         const int last = req_nt_all - 1;
         request_first_tiles(0, min(1, last), min(2, last));
         if (VEC) {
@@ -209,6 +218,9 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
         } else {
             asm volatile("s_waitcnt vmcnt(0)" : "+v"(q_raw[0]), "+v"(q_raw[1]), "+v"(q_raw[2]), "+v"(q_raw[3]) :: "memory");
         }
+        // (the wait above is for everything outstanding; this one only ties the other four query registers to it)
+        if constexpr (KS == 8)
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(q_raw[KS - 4]), "+v"(q_raw[KS - 3]), "+v"(q_raw[KS - 2]), "+v"(q_raw[KS - 1]) :: "memory");
     };
     request_item(item);
     auto lds_barrier = []() __attribute__((always_inline)) {  // LDS writes of this wave are done, then the workgroup barrier
@@ -302,10 +314,12 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
     // boundaries: F[m % LA] holds the fragment of slot m.
     // Slot m of a unit: even -> K fragment (ks = m / 2) of the unit's score half; odd -> V fragment (ps, d) of its P·V half.
     constexpr int LA = KERNL_ATTN_PIPE_LOOKAHEAD;
+    constexpr int NSLOT = 2 * KS;     // MFMAs of a unit: KS for the scores of 32 keys, KS = 2 DB for P·V of 32 keys
+    constexpr int SPP = NSLOT / 8;    // slots per pair of probabilities (a unit has 8 pairs)
     vec8 F[LA];
     auto slot_frag = [&](int m, int qk_slot, int qk_half, int pv_slot, int pv_half) __attribute__((always_inline)) -> vec8 {
         if ((m & 1) == 0) return k_frag(qk_slot, qk_half, m >> 1);
-        return v_frag(pv_slot, 2 * pv_half + (m >> 2), (m >> 1) & 1);
+        return v_frag(pv_slot, 2 * pv_half + (m >> 1) / DB, (m >> 1) % DB);
     };
 
     // One unit of the pipeline: 8 slots, each with at most one MFMA, one pair of probabilities and the fragment read
@@ -324,33 +338,36 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
                     int n0, int cur_half) __attribute__((always_inline)) {
         constexpr bool DO_QK = decltype(doqk_c)::value, GENERAL = decltype(general_c)::value, HAS_CARRY = decltype(carry_c)::value;
 #pragma unroll
-        for (int m = 0; m < 8; ++m) {
+        for (int m = 0; m < NSLOT; ++m) {
             if ((m & 1) == 0) {
                 if (DO_QK) Snext = mfma32(F[m % LA], qf[m >> 1], m == 0 ? neg_m : Snext);
             } else {
-                o_acc[(m >> 1) & 1] = mfma32(F[m % LA], __builtin_bit_cast(vec8, Pprev[m >> 2]), o_acc[(m >> 1) & 1]);
+                o_acc[(m >> 1) % DB] = mfma32(F[m % LA], __builtin_bit_cast(vec8, Pprev[(m >> 1) / DB]), o_acc[(m >> 1) % DB]);
             }
             KERNL_SB;
-            if (m + LA < 8) F[m % LA] = slot_frag(m + LA, qk_slot, qk_half, pv_slot, pv_half);
-            else F[m % LA] = slot_frag(m + LA - 8, nqk_slot, nqk_half, npv_slot, npv_half);
+            if (m + LA < NSLOT) F[m % LA] = slot_frag(m + LA, qk_slot, qk_half, pv_slot, pv_half);
+            else F[m % LA] = slot_frag(m + LA - NSLOT, nqk_slot, nqk_half, npv_slot, npv_half);
             KERNL_SB;
-            if (GENERAL) mask_pair(Scur, m, cur_half, n0);
-            const float e0 = __builtin_amdgcn_exp2f(Scur[2 * m]);
-            KERNL_SB;
-            if (m > 0 || HAS_CARRY) la += ce0;
-            KERNL_SB;
-            const float e1 = __builtin_amdgcn_exp2f(Scur[2 * m + 1]);
-            KERNL_SB;
-            if (m > 0 || HAS_CARRY) {
-                lb += ce1;
+            if (m % SPP == 0) {
+                const int e = m / SPP;  // pair of probabilities handled in this slot
+                if (GENERAL) mask_pair(Scur, e, cur_half, n0);
+                const float e0 = __builtin_amdgcn_exp2f(Scur[2 * e]);
                 KERNL_SB;
-                const uint32_t pk = pack2<T>(ce0, ce1);
-                if (m == 0) Pprev[1][3] = pk;
-                else Pcur[(m - 1) / 4][(m - 1) % 4] = pk;
+                if (e > 0 || HAS_CARRY) la += ce0;
+                KERNL_SB;
+                const float e1 = __builtin_amdgcn_exp2f(Scur[2 * e + 1]);
+                KERNL_SB;
+                if (e > 0 || HAS_CARRY) {
+                    lb += ce1;
+                    KERNL_SB;
+                    const uint32_t pk = pack2<T>(ce0, ce1);
+                    if (e == 0) Pprev[1][3] = pk;
+                    else Pcur[(e - 1) / 4][(e - 1) % 4] = pk;
+                }
+                ce0 = e0;
+                ce1 = e1;
+                KERNL_SB;
             }
-            ce0 = e0;
-            ce1 = e1;
-            KERNL_SB;
         }
     };
 
@@ -372,7 +389,7 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
         else unit(Sb, Pb, Sa, Pa, Yes(), general_c, Yes(), k1, 0, ts, 0, k1, 1, ts, 1, n0, 1);
         // this wave's part of K(t+2) and V(t+1) has landed (only this step's requests may still be in flight); after
         // the barrier everybody's has, and nobody reads the ring slots any more that the next step's requests overwrite
-        if (!LAST) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+        if (!LAST) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * KI));  // vmcnt(2 KI): all but the requests of this step
         else __builtin_amdgcn_s_waitcnt(0x0F70);
         __builtin_amdgcn_s_barrier();
 #pragma unroll
@@ -533,12 +550,12 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
             // K(1) and V(0) have landed too: every wave waited for all of the item's first requests before the barrier above
             // the first unit: scores of (1, lower half) if there is a position 1, probabilities of (0, upper), P·V of (0, lower)
 #pragma unroll
-            for (int m = 0; m < LA && m < 8; ++m) F[m] = slot_frag(m, 1, 0, 0, 0);
+            for (int m = 0; m < LA && m < NSLOT; ++m) F[m] = slot_frag(m, 1, 0, 0, 0);
             if (nt > 1) {
                 dma_k(tq[3], 3);
                 dma_v(tq[2], 2);
                 unit(Sb, Pb, Sa, Pa, Yes(), No(), No(), 1, 0, 0, 0, 1, 1, 0, 1, n0, 1);
-                __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+                __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * KI));  // vmcnt(2 KI): all but the requests of this step
             } else {
                 unit(Sb, Pb, Sa, Pa, No(), No(), No(), 1, 0, 0, 0, 1, 1, 0, 1, n0, 1);
                 __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -573,9 +590,9 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
         {
             const int ls = (nt - 1) & 3;
 #pragma unroll
-            for (int m = 1; m < 8; m += 2) {
+            for (int m = 1; m < NSLOT; m += 2) {
                 const vec8 vf = (m < LA) ? F[m % LA] : slot_frag(m, ls, 1, ls, 1);
-                o_acc[(m >> 1) & 1] = mfma32(vf, __builtin_bit_cast(vec8, Pb[m >> 2]), o_acc[(m >> 1) & 1]);
+                o_acc[(m >> 1) % DB] = mfma32(vf, __builtin_bit_cast(vec8, Pb[(m >> 1) / DB]), o_acc[(m >> 1) % DB]);
             }
         }
         // ================= the ring is free: the next item's queries, first tiles and mask row are requested now
@@ -663,9 +680,9 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
 #pragma unroll
                         for (int v = 0; v < 16; ++v) o_acc[d][v] *= alpha;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        o_acc[i & 1] = mfma32(v_frag(3, i >> 1, i & 1), __builtin_bit_cast(vec8, Pa[i >> 1]), o_acc[i & 1]);
-                        o_acc[i & 1] = mfma32(v_frag(3, 2 + (i >> 1), i & 1), __builtin_bit_cast(vec8, Pb[i >> 1]), o_acc[i & 1]);
+                    for (int i = 0; i < 2 * DB; ++i) {
+                        o_acc[i % DB] = mfma32(v_frag(3, i / DB, i % DB), __builtin_bit_cast(vec8, Pa[i / DB]), o_acc[i % DB]);
+                        o_acc[i % DB] = mfma32(v_frag(3, 2 + i / DB, i % DB), __builtin_bit_cast(vec8, Pb[i / DB]), o_acc[i % DB]);
                     }
                     tile = next_tile(tile);
                 }
@@ -696,27 +713,52 @@ __global__ void __launch_bounds__(256, 2) attention_pipe_kernel(const AttnParams
     __builtin_amdgcn_s_waitcnt(0x0F70);  // no load may still be writing LDS when the workgroup ends
 }
 
-template <typename T>
+template <typename T, int D>
 static void launch_pipe_t(const AttnParams &p, int mask_mode, bool causal, hipStream_t st) {
-    // persistent grid: two workgroups per CU (what the LDS rings allow), 64 per XCD, fewer when the busiest XCD has
-    // fewer items
+    // persistent grid: as many workgroups per CU as the LDS rings allow (two at head size 64, one at 128), 32 CUs per
+    // XCD, fewer when the busiest XCD has fewer items
+    constexpr int kPerCu = D == 64 ? 2 : 1;
+    constexpr int kRingBytes = 4 * 2 * 64 * D * 2;
     const int heads_per_xcd = (p.B * p.H + 7) / 8;
     const int64_t items_per_xcd = (int64_t)heads_per_xcd * p.nq_tiles;
-    const int per_xcd = (int)(items_per_xcd < 64 ? items_per_xcd : 64);
+    const int per_xcd = (int)(items_per_xcd < 32 * kPerCu ? items_per_xcd : 32 * kPerCu);
     dim3 grid((unsigned)(8 * per_xcd)), block(256);
-    if (mask_mode == MASK_VECTOR) hipLaunchKernelGGL((attention_pipe_kernel<T, MASK_VECTOR, false>), grid, block, 0, st, p);
-    else if (causal) hipLaunchKernelGGL((attention_pipe_kernel<T, MASK_NONE, true>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((attention_pipe_kernel<T, MASK_NONE, false>), grid, block, 0, st, p);
+    const int lds_bytes = D == 64 ? 0 : kRingBytes + (mask_mode == MASK_VECTOR ? kPipeMaxMaskKeys * 4 : 0) + 96;
+#define KERNL_PIPE_LAUNCH(MM, C)                                                                                        \
+    do {                                                                                                               \
+        auto kern = attention_pipe_kernel<T, D, MM, C>;                                                                \
+        static bool attr_done = false; /* benign race: the attribute call is idempotent */                             \
+        if (!attr_done) {                                                                                              \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                      kRingBytes + kPipeMaxMaskKeys * 4 + 96);                                         \
+            attr_done = true;                                                                                          \
+        }                                                                                                              \
+        hipLaunchKernelGGL(kern, grid, block, lds_bytes, st, p);                                                        \
+    } while (0)
+    if (mask_mode == MASK_VECTOR) KERNL_PIPE_LAUNCH(MASK_VECTOR, false);
+    else if (causal) KERNL_PIPE_LAUNCH(MASK_NONE, true);
+    else KERNL_PIPE_LAUNCH(MASK_NONE, false);
+#undef KERNL_PIPE_LAUNCH
 }
 
 // true if the problem was launched here; false: not covered, the caller takes the streaming kernel
 bool launch_attention_pipe(const AttnParams &p, int D, int dtype, int mask_mode, bool causal, bool force, hipStream_t st) {
-    if (D != 64) return false;
+    if (D != 64 && D != 128) return false;
     if (mask_mode == MASK_MATRIX) return false;
     if (mask_mode == MASK_VECTOR && (causal || p.N > kPipeMaxMaskKeys)) return false;
     if (!force && p.N < kPipeMinKeys) return false;
-    if (dtype == KERNL_F16) launch_pipe_t<f16>(p, mask_mode, causal, st);
-    else launch_pipe_t<bf16>(p, mask_mode, causal, st);
+    // Head size 128 runs one workgroup per CU here and is no faster per tile than the streaming kernel (both sit at the
+    // chip's power limit); what it wins is BALANCE when a causal problem has few (batch, head) pairs: a persistent
+    // workgroup pairs long and short query tiles, where the streaming kernel's grid is one round of unequal workgroups
+    // (measured, [1,32,2048,128] causal: 50 against 60 us; 64 pairs: +3..6 %; 128 pairs or 40: slower).
+    if (!force && D == 128 && !(causal && mask_mode == MASK_NONE && p.B * p.H <= 64 && (p.B * p.H) % 8 == 0)) return false;
+    if (D == 64) {
+        if (dtype == KERNL_F16) launch_pipe_t<f16, 64>(p, mask_mode, causal, st);
+        else launch_pipe_t<bf16, 64>(p, mask_mode, causal, st);
+    } else {
+        if (dtype == KERNL_F16) launch_pipe_t<f16, 128>(p, mask_mode, causal, st);
+        else launch_pipe_t<bf16, 128>(p, mask_mode, causal, st);
+    }
     return true;
 }
 
