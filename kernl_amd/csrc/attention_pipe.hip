@@ -172,7 +172,11 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
     };
     // The loads of the query rows and of the mask row are issued from inline assembly as well: the compiler makes every
     // barrier wait for the vector-memory loads it knows of, and these are meant to stay in flight across the barriers
-    // of the previous item's epilogue.  `item_loads_landed` is the wait that ties their registers.
+    // of the previous item's epilogue.  `item_loads_landed` is the wait that ties their registers.  Between the two the
+    // compiler believes the registers hold their values: were it to SPILL one of them there, it would store what the
+    // load has not delivered yet.  The registers are therefore only ever named by those two statements, and the
+    // build is checked for it: the per-key-mask form of head size 64 has 5-6 spilled registers, none of them these (a
+    // build that moved the LDS rings of that form to dynamic LDS spilled 26 and read garbage mask values).
     auto request_item = [&](int idx) __attribute__((always_inline)) {
         const int bh = 8 * (idx / p.nq_tiles) + xcd, qt = idx % p.nq_tiles;
         req_b = bh / p.H;
