@@ -492,6 +492,50 @@ def main():
         except Exception as exc:  # the headline number must still be reported
             extra["bert_base_b32_s512_error"] = f"{type(exc).__name__}: {exc}"[:300]
 
+        # configs[4] in miniature: TWO decoder layers at Llama-2-7B width (hidden 4096, 32 heads of 128, SwiGLU 11008,
+        # RMSNorm eps 1e-5), batch 1, 2048 tokens, causal, through optimize_model + hipGraph; 32 layers are 16 times
+        # this minus the embedding.  Its attention shape is timed on its own as well.
+        try:
+            import torch._dynamo
+            from transformers import LlamaConfig, LlamaModel
+
+            from kernl_amd.model_optimization import optimize_model
+
+            gen = torch.Generator().manual_seed(0)
+            ql, kl, vl = (torch.randn((1, 32, 2048, 128), generator=gen).half().to(dev) for _ in range(3))
+            ol = torch.empty_like(ql)
+            t = graph_time_ms(lambda: attention_forward(ql, kl, vl, ol, 128 ** -0.5, True, None), reps=5)
+            extra["attention_1x32x2048x128_causal_us_graph_replay"] = round(t * 1e3, 2)
+            extra["attention_1x32x2048x128_causal_tflops"] = round(2.0 * 32 * 2048 * 2048 * 128 / (t * 1e-3) / 1e12, 1)
+            del ql, kl, vl, ol
+            torch._dynamo.reset()
+            torch.manual_seed(0)
+            lcfg = LlamaConfig(num_hidden_layers=2, hidden_size=4096, num_attention_heads=32, num_key_value_heads=32,
+                               intermediate_size=11008, vocab_size=32000, rms_norm_eps=1e-5, max_position_embeddings=4096)
+            lcfg._attn_implementation = "sdpa"
+            llama = LlamaModel(lcfg).eval().half().to(dev)
+            lids = torch.randint(0, 32000, (1, 2048), generator=gen).to(dev)
+            with torch.inference_mode():
+                eager = llama(input_ids=lids, use_cache=False).last_hidden_state.float()
+                optimize_model(llama)
+                for _ in range(4):
+                    got = llama(input_ids=lids, use_cache=False).last_hidden_state
+                torch.cuda.synchronize()
+                times = []
+                for _ in range(10):
+                    t0 = time.perf_counter()
+                    llama(input_ids=lids, use_cache=False)
+                    torch.cuda.synchronize()
+                    times.append((time.perf_counter() - t0) * 1e3)
+            assert torch.isfinite(got).all(), "Llama-shaped prefill: non-finite hidden states"
+            extra["llama7b_width_2_layers_b1_s2048_fp16_fwd_ms"] = round(statistics.median(times), 3)
+            # against eager fp16 PyTorch on the same weights (the fp32 comparison is in tests/test_model_optimization.py)
+            extra["llama7b_width_2_layers_mean_rel_diff_vs_fp16_eager"] = round(
+                ((got.float() - eager).abs().mean() / eager.abs().mean()).item(), 5)
+            del llama
+        except Exception as exc:
+            extra["llama7b_width_error"] = f"{type(exc).__name__}: {exc}"[:300]
+
     result["extra"] = extra
     print(json.dumps(result), flush=True)
 
