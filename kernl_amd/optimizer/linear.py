@@ -206,13 +206,18 @@ class _DerivedParams:
         }
 
     def refresh(self, only_changed: bool) -> int:
-        """Rebuild copied entries in place from their live originals; returns how many were rebuilt."""
-        self._drop_dead()
+        """Rebuild copied entries in place from their live originals; returns how many were rebuilt.  With
+        `only_changed` this is the check in front of every graph replay: a walk over the copied entries that compares
+        version counters and touches nothing else."""
+        if not only_changed:
+            self._drop_dead()
         n = 0
         for entry in self._entries.values():
             if entry.rebuild is None:
                 continue
             originals = [None if r is None else r() for r in entry.refs]
+            if any(o is None and r is not None for o, r in zip(originals, entry.refs)):
+                continue  # an original has died: the entry goes with the next sweep
             versions = self._versions(originals)
             if only_changed and versions == entry.versions:
                 continue

@@ -602,3 +602,36 @@ def test_split_k_dispatch_rule():
     assert not takes_split_k_kernel(*qkv(2048, 32, 1, 128, 128))    # 65536 rows: beyond the kernel's grid
     q, k, v = qkv(2, 4, 1, 128, 64)
     assert not takes_split_k_kernel(q[..., 1:], k[..., 1:], v[..., 1:])   # rows no longer 16-byte aligned
+
+
+def test_residual_additions_fold_into_the_projection_before_them():
+    """`res + linear(...)` in either operand order becomes one call; a projection with an activation, or one whose
+    result is used elsewhere too, keeps its addition."""
+    from kernl_amd.optimizer.linear import fuse_residual_into_linears, replace_all_linear
+
+    F = torch.nn.functional
+
+    class Block(torch.nn.Module):
+        """Parameters used through F.linear, the form torch.compile hands to a backend."""
+
+        def __init__(self):
+            super().__init__()
+            self.wa, self.wb, self.wc, self.wd = (torch.nn.Parameter(torch.randn(8, 8)) for _ in range(4))
+            self.ba = torch.nn.Parameter(torch.randn(8))
+
+        def forward(self, x, r):
+            y = r + F.linear(x, self.wa, self.ba)              # fused
+            y = F.linear(y, self.wb, None) + y                 # fused, projection on the left
+            y = y + F.relu(F.linear(y, self.wc, None))         # activation in between: stays
+            z = F.linear(y, self.wd, None)
+            return z + y, z                                    # the projection has a second user: stays
+
+    torch.manual_seed(0)
+    m = Block().eval()
+    gm = torch.fx.symbolic_trace(m)
+    replace_all_linear(gm)
+    fuse_residual_into_linears(gm)
+    t = _targets(gm)
+    assert t.count("linear_residual_wrapper") == 2 and t.count("add") == 2
+    nodes = [n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "linear_residual_wrapper"]
+    assert [n.args[3].name for n in nodes] == ["r", nodes[0].name]       # the residual operand of each
