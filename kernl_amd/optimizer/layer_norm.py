@@ -24,25 +24,41 @@ def layer_norm_wrapper(v: torch.Tensor, layernorm: torch.nn.LayerNorm):
     return layer_norm(v, layernorm.weight, layernorm.bias, layernorm.eps)
 
 
+_unit_weights = {}
+
+
+def _flat_affine(v: torch.Tensor, normalized_shape, weight, bias):
+    """F.layer_norm over the last len(normalized_shape) dimensions is a LayerNorm over their flattening; a missing
+    weight is a weight of ones (kept per size, dtype and device: built once, before graph capture)."""
+    n = 1
+    for d in normalized_shape:
+        n *= int(d)
+    if weight is None:
+        key = (n, v.dtype, v.device)
+        if key not in _unit_weights:
+            _unit_weights[key] = torch.ones(n, dtype=v.dtype, device=v.device)
+        weight = _unit_weights[key]
+    lead = v.shape[: v.dim() - len(normalized_shape)]
+    return lead, n, weight.reshape(n), None if bias is None else bias.reshape(n)
+
+
 def layer_norm_wrapper_functional(v: torch.Tensor, normalized_shape, weight, bias, eps: float):
-    if len(normalized_shape) != 1 or weight is None:
-        return torch.nn.functional.layer_norm(v, normalized_shape, weight, bias, eps)
     _half_params_once(v, weight, bias)
-    return layer_norm(v, weight, bias, eps)
+    if len(normalized_shape) == 1 and weight is not None:
+        return layer_norm(v, weight, bias, eps)
+    lead, n, w, b = _flat_affine(v, normalized_shape, weight, bias)
+    return layer_norm(v.reshape(*lead, n), w, b, eps).reshape(v.shape)
 
 
 def add_layer_norm_wrapper_functional(a: torch.Tensor, b: torch.Tensor, normalized_shape, weight, bias, eps: float):
-    if (
-        len(normalized_shape) != 1
-        or weight is None
-        or not isinstance(a, torch.Tensor)
-        or not isinstance(b, torch.Tensor)
-        or a.shape != b.shape
-        or a.dtype != b.dtype
-    ):
-        return torch.nn.functional.layer_norm(a + b, normalized_shape, weight, bias, eps)
     _half_params_once(a, weight, bias)
-    return add_layer_norm(a, b, weight, bias, eps)
+    if not isinstance(a, torch.Tensor) or not isinstance(b, torch.Tensor) or a.shape != b.shape or a.dtype != b.dtype:
+        # a python scalar or a broadcast operand: add first (one element-wise kernel), then the LayerNorm kernel
+        return layer_norm_wrapper_functional(a + b, normalized_shape, weight, bias, eps)
+    if len(normalized_shape) == 1 and weight is not None:
+        return add_layer_norm(a, b, weight, bias, eps)
+    lead, n, w, bb = _flat_affine(a, normalized_shape, weight, bias)
+    return add_layer_norm(a.reshape(*lead, n), b.reshape(*lead, n), w, bb, eps).reshape(a.shape)
 
 
 def layer_norm_rms_wrapper(v: torch.Tensor, weight: torch.Tensor, eps: float):

@@ -551,6 +551,21 @@ def rms_fused_linear_rope_wrapper(x: torch.Tensor, rms_weight, eps: float, weigh
                                   head_dim=head_dim, rope_cols=sum(sizes[:n_rotated]))
         return tuple(torch.split(out, sizes, dim=-1))
     outs = list(rms_fused_linear_wrapper(x, rms_weight, eps, weights, biases))
+    first = outs[0]
+    rot_cols = sum(sizes[:n_rotated])
+    adjacent = (
+        n_rotated > 1 and first.dim() == 3 and first.stride(-1) == 1
+        and all(sizes[i] % head_dim == 0 for i in range(n_rotated))
+        and all(outs[i].stride() == first.stride() for i in range(n_rotated))
+        and all(outs[i].data_ptr() == first.data_ptr() + sum(sizes[:i]) * first.element_size() for i in range(n_rotated))
+    )
+    if adjacent:
+        # the rotated outputs are neighbouring column ranges of one buffer: one launch over all their heads
+        both = first.as_strided((first.shape[0], first.shape[1], rot_cols), first.stride())
+        heads = both.reshape(first.shape[0], first.shape[1], -1, head_dim).transpose(1, 2)
+        rotated = rotary_forward(heads, cos, sin).transpose(1, 2).reshape(first.shape[0], first.shape[1], rot_cols)
+        outs[:n_rotated] = torch.split(rotated, sizes[:n_rotated], dim=-1)
+        return tuple(outs)
     for i in range(n_rotated):
         o = outs[i]
         heads = o.reshape(*o.shape[:-1], -1, head_dim).transpose(-3, -2)        # [.., heads, positions, head_dim], a view

@@ -139,3 +139,48 @@ def test_layer_norm_rejects_bad_arguments():
         layer_norm(x, w.float(), None, 1e-5)
     with pytest.raises(AssertionError):
         layer_norm(x, w, w.float(), 1e-5)
+
+
+@pytest.mark.parametrize("form", ["two_dims", "no_affine", "two_dims_add", "no_affine_add", "broadcast_add"])
+def test_functional_layer_norm_forms_all_reach_the_kernel(form, close, monkeypatch):
+    """`F.layer_norm` over two trailing dimensions (= LayerNorm over their flattening), without weight and bias, and with
+    an addition in front: every form runs on the LayerNorm kernel, none on PyTorch's."""
+    import kernl_amd.optimizer.layer_norm as opt
+    from oracle import layer_norm_oracle
+
+    def forbidden(*a, **k):
+        raise AssertionError("F.layer_norm was called")
+
+    monkeypatch.setattr(torch.nn.functional, "layer_norm", forbidden)
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn((6, 10, 4, 64), generator=gen).half()
+    y = torch.randn((6, 10, 4, 64), generator=gen).half()
+    eps = 1.6e-5
+    if form.startswith("two_dims"):
+        w, b = (1 + 0.1 * torch.randn((4, 64), generator=gen)).half(), (0.1 * torch.randn((4, 64), generator=gen)).half()
+        shape = (4, 64)
+    else:
+        w = b = None
+        shape = (64,)
+    wc, bc = (None if w is None else w.cuda()), (None if b is None else b.cuda())
+    if form == "broadcast_add":
+        out = opt.add_layer_norm_wrapper_functional(x.cuda(), y[:1].cuda(), shape, wc, bc, eps)
+        src = x.float() + y[:1].float()
+    elif form.endswith("_add"):
+        out = opt.add_layer_norm_wrapper_functional(x.cuda(), y.cuda(), shape, wc, bc, eps)
+        src = x.float() + y.float()
+    else:
+        out = opt.layer_norm_wrapper_functional(x.cuda(), shape, wc, bc, eps)
+        src = x.float()
+    torch.cuda.synchronize()
+    n = 1
+    for d in shape:
+        n *= d
+    flat = src.reshape(-1, n)
+    if form == "broadcast_add":
+        flat = (x + y[:1]).float().reshape(-1, n)   # the addition of two fp16 tensors rounds to fp16 first
+    wf = torch.ones(n) if w is None else w.float().reshape(n)
+    bf = None if b is None else b.float().reshape(n)
+    ref = layer_norm_oracle(flat, wf, bf, eps).reshape(x.shape)
+    assert out.shape == x.shape and out.dtype == torch.half
+    close(out, ref, scale="magnitude", what=f"functional layer norm, {form}")
