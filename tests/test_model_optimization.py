@@ -436,6 +436,69 @@ def test_generation_with_growing_cache(family):
     assert agree >= 3
 
 
+def test_llama_generation_runs_the_decode_projection_kernel(monkeypatch):
+    """Greedy generation with a growing key/value cache on a Llama-shaped fp16 model under `optimize_model`: each
+    decoding step is a new cache length, hence a new compilation and graph.  In the steps after the prompt every layer's
+    query/key/value projection must run as one call of the few-row projection kernel with the RMS prologue and the
+    rotation, and the output and down projections as calls with the residual; the scores follow the eager fp16
+    model's while the two greedy paths pick the same tokens."""
+    from torch._dynamo.utils import counters
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from kernl_amd import _lib
+    from kernl_amd.model_optimization import optimize_model
+
+    torch._dynamo.reset()
+    counters.clear()
+    torch.manual_seed(0)
+    layers, steps = 2, 12
+    cfg = LlamaConfig(num_hidden_layers=layers, hidden_size=512, num_attention_heads=4, num_key_value_heads=4,
+                      intermediate_size=1408, vocab_size=1000, rms_norm_eps=1e-5, max_position_embeddings=512,
+                      pad_token_id=0, bos_token_id=1, eos_token_id=2)
+    cfg._attn_implementation = "sdpa"
+    model = LlamaForCausalLM(cfg).eval().half().cuda()
+    gen = torch.Generator().manual_seed(1)
+    ids = torch.randint(3, 1000, (2, 20), generator=gen).cuda()
+    kwargs = dict(input_ids=ids, attention_mask=torch.ones_like(ids), min_new_tokens=steps, max_new_tokens=steps,
+                  do_sample=False, output_scores=True, return_dict_in_generate=True)
+    with torch.inference_mode():
+        ref = model.generate(**kwargs)
+
+    calls = {"rotated": 0, "residual": 0}
+    real = _lib.linear_decode_fwd
+
+    def counting(x2d, rms_weight, eps, weight, bias, residual2d, out2d, cos=None, sin=None, *args, **kw):
+        calls["rotated"] += int(cos is not None and rms_weight is not None)
+        calls["residual"] += int(residual2d is not None)
+        return real(x2d, rms_weight, eps, weight, bias, residual2d, out2d, cos, sin, *args, **kw)
+
+    monkeypatch.setattr(_lib, "linear_decode_fwd", counting)
+    optimize_model(model.model)
+    with torch.inference_mode():
+        model.generate(**kwargs)        # compiles and captures one graph per step
+        out = model.generate(**kwargs)  # replays them
+        torch.cuda.synchronize()
+    frames = counters["frames"]
+    assert frames["ok"] == frames["total"], f"some steps were not compiled: {dict(frames)}"
+    assert counters["stats"]["unique_graphs"] >= steps, dict(counters["stats"])
+    # warm-up run and capture run of each of the steps after the prompt
+    assert calls["rotated"] >= 2 * (steps - 1) * layers, calls
+    assert calls["residual"] >= 2 * (steps - 1) * layers * 2, calls
+    prompt = ref.sequences.shape[1] - steps
+    agree = 0
+    for t, (a, b) in enumerate(zip(out.scores, ref.scores)):
+        if not torch.equal(out.sequences[:, : prompt + t], ref.sequences[:, : prompt + t]):
+            break
+        finite = torch.isfinite(b)
+        assert torch.equal(torch.isfinite(a), finite)
+        scale = b[finite].abs().max().item()
+        diff = (a.float() - b.float())[finite].abs().max().item()
+        assert diff <= 1e-2 * max(scale, 1.0), f"step {t}: scores differ by {diff} (scale {scale})"
+        agree += 1
+    print(f"llama: greedy paths agree for {agree} of {steps} steps; decode kernel calls {calls}", flush=True)
+    assert agree >= 3
+
+
 def test_models_built_one_after_the_other_do_not_share_fused_weights():
     """Two models of the same shapes, different weights, built and optimized one after the other with the first one
     freed in between: the allocator may give the second model the first one's parameter addresses, and the
