@@ -34,6 +34,8 @@ EXPORTED_SYMBOLS = (
     "kernl_linear_w8_fwd",
     "kernl_linear_rms_fwd",
     "kernl_linear_decode_fwd",
+    "kernl_linear_fewrow_workspace_bytes",
+    "kernl_linear_fewrow_fwd",
     "kernl_linear_glu_fwd",
     "kernl_layernorm_fwd",
     "kernl_add_layernorm_fwd",
@@ -109,6 +111,10 @@ def load() -> ctypes.CDLL:
         [_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp] + [_i64] * 3 + [_i64p] * 3 + [_vp, _vp] + [_i64] * 3
         + [_i64p, ctypes.c_int, ctypes.c_int, _vp]
     )
+    lib.kernl_linear_fewrow_workspace_bytes.restype = _i64
+    lib.kernl_linear_fewrow_workspace_bytes.argtypes = [_i64] * 3
+    lib.kernl_linear_fewrow_fwd.restype = ctypes.c_int
+    lib.kernl_linear_fewrow_fwd.argtypes = [_vp] * 6 + [_i64] * 4 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_linear_rms_fwd.restype = ctypes.c_int
     lib.kernl_linear_rms_fwd.argtypes = (
         [_vp, _vp, ctypes.c_float, _vp, _vp, _vp] + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int] * 3 + [_vp]
@@ -373,6 +379,43 @@ def linear_decode_fwd(x2d, rms_weight, eps: float, weight, bias, residual2d, out
             int(rows_per_batch), tstrides, tdtype, DTYPE_CODE[x2d.dtype], _stream(x2d),
         )
     _check(st, "kernl_linear_decode_fwd")
+
+
+def linear_fewrow_supported(x2d, weight) -> bool:
+    """What `kernl_linear_fewrow_fwd` takes: 16-bit rows, at most 64 of them, K a multiple of 64 from 256 on."""
+    M, K = x2d.shape
+    return (
+        x2d.dtype in (torch.float16, torch.bfloat16) and weight.dtype == x2d.dtype and 0 < M <= 64
+        and K % 64 == 0 and K >= 256 and x2d.stride(1) == 1 and x2d.stride(0) % 8 == 0 and x2d.data_ptr() % 16 == 0
+        and weight.is_contiguous() and weight.data_ptr() % 16 == 0
+    )
+
+
+def linear_fewrow_workspace_bytes(M: int, N: int, K: int) -> int:
+    return int(load().kernl_linear_fewrow_workspace_bytes(M, N, K))
+
+
+def linear_fewrow_fwd(x2d, weight, bias, residual2d, out2d, activation: int, workspace=None) -> None:
+    """`workspace`: device tensor of at least `linear_fewrow_workspace_bytes` bytes; allocated here when None (a fresh
+    allocation per call: stream-ordered, so calls on different streams never share one)."""
+    _require_gpu(x2d, weight, bias, residual2d, out2d, workspace)
+    M, K = x2d.shape
+    N = out2d.shape[1]
+    lib = load()
+    if workspace is None:
+        need = linear_fewrow_workspace_bytes(M, N, K)
+        if need:
+            workspace = torch.empty(need, dtype=torch.uint8, device=x2d.device)
+    ws_ptr = None if workspace is None else workspace.data_ptr()
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with torch.cuda.device(x2d.device):
+        st = lib.kernl_linear_fewrow_fwd(
+            x2d.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(),
+            None if residual2d is None else residual2d.data_ptr(), out2d.data_ptr(), ws_ptr, ws_bytes, M, N, K,
+            _arr(x2d.stride()), _arr(out2d.stride()), None if residual2d is None else _arr(residual2d.stride()),
+            int(activation), DTYPE_CODE[x2d.dtype], _stream(x2d),
+        )
+    _check(st, "kernl_linear_fewrow_fwd")
 
 
 def linear_glu_fwd(x2d, weight_interleaved, bias_interleaved, out2d, activation: int) -> None:

@@ -25,6 +25,21 @@ ACTIVATIONS = {
 ONE_BYTE_WEIGHT_DTYPES = (torch.int8, torch.uint8, torch.float8_e5m2)
 
 
+FEW_ROW_MIN_ROWS = 17          # up to 16 rows the kernel that gives a workgroup 16 columns and all of K is as fast or faster
+FEW_ROW_MIN_WEIGHT = 1 << 22   # elements: below that (2048 x 2048) launch latency decides and one launch beats two
+
+
+def takes_few_row_kernel(x2d: torch.Tensor, weight: torch.Tensor) -> bool:
+    """17 to 64 rows against a large 16-bit weight run the stream-K kernel (`kernl_linear_fewrow_fwd`): measured against
+    the weight-streaming kernel of `kernl_linear_fwd` at 32 / 64 rows, 5120 x 5120: 18 / 21 us against 34 / 35;
+    4096 x 11008: 25 / 30 against 35 / 53; 12288 x 4096: 27 / 32 against 28 / 37."""
+    return (
+        FEW_ROW_MIN_ROWS <= x2d.shape[0] <= 64
+        and weight.shape[0] * weight.shape[1] >= FEW_ROW_MIN_WEIGHT
+        and _lib.linear_fewrow_supported(x2d, weight)
+    )
+
+
 class LinearLayer(torch.autograd.Function):
     @staticmethod
     @custom_fwd(device_type="cuda", cast_inputs=torch.float16)
@@ -68,7 +83,10 @@ class LinearLayer(torch.autograd.Function):
         outputs = torch.empty((M, N), device=x.device, dtype=x.dtype)
         if act_inputs is not None:
             assert act_inputs.shape == (M, N) and act_inputs.dtype == x.dtype
-        _lib.linear_fwd(x_, weight, bias, outputs, act_inputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
+        if act_inputs is None and takes_few_row_kernel(x_, weight):
+            _lib.linear_fewrow_fwd(x_, weight, bias, None, outputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
+        else:
+            _lib.linear_fwd(x_, weight, bias, outputs, act_inputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
         return outputs if x.ndim == 2 else outputs.reshape(*x.shape[:-1], N)
 
 
@@ -216,5 +234,8 @@ def decode_linear_layer(
         assert residual.dtype == x.dtype and residual.numel() == x_.shape[0] * N
         res_ = residual.reshape(-1, N)
     out = torch.empty((x_.shape[0], N), device=x.device, dtype=x.dtype)
-    _lib.linear_decode_fwd(x_, rms_weight, eps, weight, bias, res_, out, cos, sin, head_dim, rope_cols, rows_per_batch)
+    if rms_weight is None and cos is None and takes_few_row_kernel(x_, weight):
+        _lib.linear_fewrow_fwd(x_, weight, bias, res_, out, _lib.ACT_NONE)
+    else:
+        _lib.linear_decode_fwd(x_, rms_weight, eps, weight, bias, res_, out, cos, sin, head_dim, rope_cols, rows_per_batch)
     return out if x.ndim == 2 else out.reshape(*x.shape[:-1], N)

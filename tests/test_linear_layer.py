@@ -383,6 +383,77 @@ def test_decode_projection_rejections():
         _lib.linear_decode_fwd(x[:4], None, 0.0, w, None, None, out, t64, t64, 64, 64, 4)
 
 
+FEW_ROW_SHAPES = [
+    (33, 200, 256),      # two tiles, the second ragged; a run is exactly one tile: no partial sums
+    (17, 1000, 320),     # five chunks per tile, runs of four: every run crosses into the next tile
+    (64, 777, 704),      # width that is no multiple of 4 (element stores), eleven chunks per tile
+    (20, 384, 1024),     # runs that divide a tile evenly
+    (5, 1000, 320),      # one 16-row block of x
+    (48, 5120, 5120),    # 247 workgroups with runs of 13 units against 80 chunks per tile
+    (64, 4096, 11008),   # long K
+    (33, 11008, 4096),   # 86 tiles
+    (30, 26300, 256),    # 206 tiles: whole tiles per workgroup, the last one ragged
+    (64, 40000, 256),    # more tiles than workgroups: runs of 5 units against 4 chunks per tile
+    (18, 80000, 256),    # runs of 10 units: a workgroup finishes a tile, covers one whole and starts a third
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("shape", FEW_ROW_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_linear_few_rows_stream_k(shape, dtype, close):
+    """`kernl_linear_fewrow_fwd` (units of one tile and one k chunk dealt in equal runs to the workgroups, partial tiles
+    added by a second launch) against the oracle: plain, with bias + activation, and with bias + residual; the
+    workspace is filled with NaNs first, so a partial tile that is read without having been written shows."""
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(53)
+    x, w, b = _inputs(M, N, K, dtype, gen, w_std=K ** -0.5)
+    res = torch.randn((M, N), generator=gen).to(dtype)
+    xd, wd, bd, rd = x.cuda(), w.cuda(), b.cuda(), res.cuda()
+    assert _lib.linear_fewrow_supported(xd, wd)
+    need = _lib.linear_fewrow_workspace_bytes(M, N, K)
+    ws = torch.full((max(need, 16) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    outs = [torch.empty((M, N), dtype=dtype, device="cuda") for _ in range(3)]
+    _lib.linear_fewrow_fwd(xd, wd, None, None, outs[0], _lib.ACT_NONE, ws)
+    _lib.linear_fewrow_fwd(xd, wd, bd, None, outs[1], _lib.ACT_GELU_TANH, ws)
+    _lib.linear_fewrow_fwd(xd, wd, bd, rd, outs[2], _lib.ACT_NONE)   # workspace allocated by the binding
+    torch.cuda.synchronize()
+    close(outs[0], linear_oracle(x, w, None, ""), dtype, what=f"stream-K {shape} plain")
+    close(outs[1], linear_oracle(x, w, b, "fast_gelu"), dtype, what=f"stream-K {shape} bias + gelu")
+    close(outs[2], linear_oracle(x, w, b, "") + res.float(), dtype, scale="magnitude", what=f"stream-K {shape} residual")
+
+
+def test_linear_few_rows_stream_k_is_what_the_operators_run(close, monkeypatch):
+    """17 to 64 rows against a large weight: `linear_layer` and the residual form of `decode_linear_layer` take the
+    stream-K kernel; fewer rows, small weights and a saved pre-activation keep the other kernels.  Strided rows of x
+    and a 3-D input go through unchanged."""
+    from kernl_amd.implementations.linear_layer import decode_linear_layer
+
+    calls = []
+    real = _lib.linear_fewrow_fwd
+    monkeypatch.setattr(_lib, "linear_fewrow_fwd", lambda *a, **k: (calls.append(a[0].shape[0]), real(*a, **k))[1])
+    gen = torch.Generator().manual_seed(59)
+    N, K = 2304, 2048
+    w = (torch.randn((N, K), generator=gen) * K ** -0.5).half()
+    b = torch.randn((N,), generator=gen).half()
+    for rows, expected in ((16, 0), (17, 1), (64, 1), (65, 0)):
+        calls.clear()
+        x = torch.randn((rows, K), generator=gen).half()
+        out = linear_layer(x.cuda(), w.cuda(), b.cuda(), "relu")
+        assert len(calls) == expected, (rows, calls)
+        close(out, linear_oracle(x, w, b, "relu"), torch.float16, what=f"{rows} rows")
+    calls.clear()
+    x = torch.randn((40, K), generator=gen).half()
+    linear_layer(x.cuda(), w.cuda(), b.cuda(), "", act_inputs=torch.empty((40, N), dtype=torch.float16, device="cuda"))
+    linear_layer(x[:, :256].contiguous().cuda(), w[:, :256].contiguous().cuda(), b.cuda(), "")   # a small weight
+    assert calls == []
+    wide = torch.randn((2, 20, 2 * K), generator=gen).half()
+    xs = wide[:, :, :K]                                    # rows 2 K apart, batch of 2 x 20
+    res = torch.randn((2, 20, N), generator=gen).half()
+    out = decode_linear_layer(xs.cuda(), w.cuda(), b.cuda(), residual=res.cuda())
+    assert calls == [40] and out.shape == (2, 20, N)
+    close(out, linear_oracle(xs, w, b, "") + res.float(), torch.float16, scale="magnitude", what="residual form, strided x")
+
+
 @pytest.mark.parametrize("tile", [1, 3, 5, 7], ids=["8wave-256", "8wave-128", "wide-256", "wide-128"])
 def test_linear_fp8_weight_every_kernel(tile, close):
     """Each of the four kernels that take one-byte weights beyond 64 rows, forced in turn on a shape with ragged edges."""
