@@ -239,24 +239,34 @@ int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float eps, const
 /*
  * The linear layer for a FEW rows of x with many columns and a long K (batched decoding steps: 17 to 64 rows, where
  * kernl_linear_fwd's weight-streaming kernel re-reads x once per 16 to 64 output columns and its tile kernels leave
- * most of their rows empty):
- *     out = activation(x @ w^T + bias) (+ residual)
- * Same semantics as kernl_linear_fwd (reference: src/kernl/implementations/linear_layer.py:92-210); the decomposition
- * is the reference's stream-K experiment (experimental/streamk/kernel_streamk.py): the (128-column tile, 64-wide k
- * chunk) units are dealt in equal contiguous runs to at most 256 workgroups, tiles cut by a run boundary are completed
- * from fp32 partial tiles by a second small launch that adds them in a fixed order (results do not depend on timing).
- *   M <= 64, K % 64 == 0, K >= 256, f16 / bf16, x with unit feature stride and 16-byte aligned rows, w [N, K] contiguous.
- *   workspace  device memory of at least kernl_linear_fewrow_workspace_bytes(M, N, K) bytes, 16-byte aligned, contents
- *              irrelevant before and after the call (0 bytes / NULL when that function returns 0); calls that overlap
- *              in time need workspaces of their own.
+ * most of their rows empty), with everything a decoder layer puts around its projections:
+ *     y   = (rms_weight ? rsqrt(mean(x^2) + eps) * ((x * rms_weight) @ w^T) : x @ w^T) + bias
+ *     y   = activation(y)                                  plain form, w [N, K]
+ *     y   = activation(y_gate) * y_value                   gated != 0: w [2N, K], bias [2N], interleaved as for
+ *                                                          kernl_linear_glu_fwd
+ *     y   = rotate(y) on the columns below rope_cols       cos / sin given (no activation, not gated)
+ *     out = y + residual                                   residual given
+ * Semantics of kernl_linear_fwd (reference: src/kernl/implementations/linear_layer.py:92-210), kernl_linear_glu_fwd,
+ * kernl_linear_rms_fwd and kernl_linear_decode_fwd, whose comments name the reference kernels of the fused forms; the
+ * decomposition is the reference's stream-K experiment (experimental/streamk/kernel_streamk.py): the (128-row tile of
+ * the weight, 64-wide k chunk) units are dealt in equal contiguous runs to at most 256 workgroups, tiles cut by a run
+ * boundary are completed from fp32 partial tiles by a second small launch that adds them in a fixed order (results do
+ * not depend on timing) and runs the epilogue.
+ *   M <= 64, K % 64 == 0, K >= 256, f16 / bf16, x with unit feature stride and 16-byte aligned rows, w contiguous.
+ *   workspace  device memory of at least kernl_linear_fewrow_workspace_bytes(M, N, K, gated, rotated) bytes, 16-byte
+ *              aligned, contents irrelevant before and after the call (NULL when that function returns 0); calls that
+ *              overlap in time need workspaces of their own.
  *   residual   [M, N] of the same dtype with its strides, or NULL.
+ *   rotation   arguments as for kernl_linear_decode_fwd; head_dim 32, 64 or 128.
  * Anything else returns KERNL_ERR_UNSUPPORTED; a workspace that is too small KERNL_ERR_INVALID_ARG.
  */
-int64_t kernl_linear_fewrow_workspace_bytes(int64_t M, int64_t N, int64_t K);
-int kernl_linear_fewrow_fwd(const void *x, const void *w, const void *bias, const void *residual, void *out,
-                            void *workspace, int64_t workspace_bytes, int64_t M, int64_t N, int64_t K,
-                            const int64_t x_strides[2], const int64_t out_strides[2],
-                            const int64_t residual_strides[2], int activation, int dtype, void *stream);
+int64_t kernl_linear_fewrow_workspace_bytes(int64_t M, int64_t N, int64_t K, int gated, int rotated);
+int kernl_linear_fewrow_fwd(const void *x, const void *rms_weight, float eps, const void *w, const void *bias,
+                            const void *residual, void *out, void *workspace, int64_t workspace_bytes, int64_t M,
+                            int64_t N, int64_t K, const int64_t x_strides[2], const int64_t out_strides[2],
+                            const int64_t residual_strides[2], const void *cos, const void *sin, int64_t head_dim,
+                            int64_t rope_cols, int64_t rows_per_batch, const int64_t table_strides[3], int table_dtype,
+                            int activation, int gated, int dtype, void *stream);
 
 /*
  * A decoding step's projection with everything around it in ONE launch (at most 64 rows of x, K % 64 == 0, f16 / bf16,

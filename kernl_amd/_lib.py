@@ -112,9 +112,12 @@ def load() -> ctypes.CDLL:
         + [_i64p, ctypes.c_int, ctypes.c_int, _vp]
     )
     lib.kernl_linear_fewrow_workspace_bytes.restype = _i64
-    lib.kernl_linear_fewrow_workspace_bytes.argtypes = [_i64] * 3
+    lib.kernl_linear_fewrow_workspace_bytes.argtypes = [_i64] * 3 + [ctypes.c_int] * 2
     lib.kernl_linear_fewrow_fwd.restype = ctypes.c_int
-    lib.kernl_linear_fewrow_fwd.argtypes = [_vp] * 6 + [_i64] * 4 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
+    lib.kernl_linear_fewrow_fwd.argtypes = (
+        [_vp, _vp, ctypes.c_float] + [_vp] * 5 + [_i64] * 4 + [_i64p] * 3 + [_vp, _vp] + [_i64] * 3
+        + [_i64p] + [ctypes.c_int] * 4 + [_vp]
+    )
     lib.kernl_linear_rms_fwd.restype = ctypes.c_int
     lib.kernl_linear_rms_fwd.argtypes = (
         [_vp, _vp, ctypes.c_float, _vp, _vp, _vp] + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int] * 3 + [_vp]
@@ -391,29 +394,39 @@ def linear_fewrow_supported(x2d, weight) -> bool:
     )
 
 
-def linear_fewrow_workspace_bytes(M: int, N: int, K: int) -> int:
-    return int(load().kernl_linear_fewrow_workspace_bytes(M, N, K))
+def linear_fewrow_workspace_bytes(M: int, N: int, K: int, gated: bool = False, rotated: bool = False) -> int:
+    """N: output width (the gated form's weight has twice as many rows)."""
+    return int(load().kernl_linear_fewrow_workspace_bytes(M, N, K, int(bool(gated)), int(bool(rotated))))
 
 
-def linear_fewrow_fwd(x2d, weight, bias, residual2d, out2d, activation: int, workspace=None) -> None:
+def linear_fewrow_fwd(x2d, weight, bias, residual2d, out2d, activation: int, workspace=None, rms_weight=None,
+                      eps: float = 0.0, gated: bool = False, cos=None, sin=None, head_dim: int = 0, rope_cols: int = 0,
+                      rows_per_batch: int = 1) -> None:
     """`workspace`: device tensor of at least `linear_fewrow_workspace_bytes` bytes; allocated here when None (a fresh
-    allocation per call: stream-ordered, so calls on different streams never share one)."""
-    _require_gpu(x2d, weight, bias, residual2d, out2d, workspace)
+    allocation per call: stream-ordered, so calls on different streams never share one).  cos / sin as for
+    `linear_decode_fwd`; `gated`: weight and bias interleaved as for `linear_glu_fwd`, out2d half as wide."""
+    _require_gpu(x2d, weight, bias, residual2d, out2d, workspace, rms_weight, cos, sin)
     M, K = x2d.shape
     N = out2d.shape[1]
     lib = load()
     if workspace is None:
-        need = linear_fewrow_workspace_bytes(M, N, K)
+        need = linear_fewrow_workspace_bytes(M, N, K, gated, cos is not None)
         if need:
             workspace = torch.empty(need, dtype=torch.uint8, device=x2d.device)
     ws_ptr = None if workspace is None else workspace.data_ptr()
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    if cos is not None:
+        tstrides = _arr((0 if cos.shape[0] == 1 else cos.stride(0), cos.stride(1), cos.stride(2)))
+        tdtype, cptr, sptr = DTYPE_CODE[cos.dtype], cos.data_ptr(), sin.data_ptr()
+    else:
+        tstrides, tdtype, cptr, sptr = None, KERNL_F32, None, None
     with torch.cuda.device(x2d.device):
         st = lib.kernl_linear_fewrow_fwd(
-            x2d.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(),
-            None if residual2d is None else residual2d.data_ptr(), out2d.data_ptr(), ws_ptr, ws_bytes, M, N, K,
-            _arr(x2d.stride()), _arr(out2d.stride()), None if residual2d is None else _arr(residual2d.stride()),
-            int(activation), DTYPE_CODE[x2d.dtype], _stream(x2d),
+            x2d.data_ptr(), None if rms_weight is None else rms_weight.data_ptr(), float(eps), weight.data_ptr(),
+            None if bias is None else bias.data_ptr(), None if residual2d is None else residual2d.data_ptr(),
+            out2d.data_ptr(), ws_ptr, ws_bytes, M, N, K, _arr(x2d.stride()), _arr(out2d.stride()),
+            None if residual2d is None else _arr(residual2d.stride()), cptr, sptr, int(head_dim), int(rope_cols),
+            int(rows_per_batch), tstrides, tdtype, int(activation), int(bool(gated)), DTYPE_CODE[x2d.dtype], _stream(x2d),
         )
     _check(st, "kernl_linear_fewrow_fwd")
 

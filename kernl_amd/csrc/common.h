@@ -90,6 +90,13 @@ __device__ __forceinline__ float to_float(f16 x) { return (float)x; }
 __device__ __forceinline__ float to_float(bf16 x) { return (float)x; }
 __device__ __forceinline__ float to_float(float x) { return x; }
 
+// element `off` of a table of fp32, fp16 or bf16 values (the rotation tables of the decoding kernels)
+__device__ __forceinline__ float table_value(const void *t, int dtype, int64_t off) {
+    if (dtype == KERNL_F32) return static_cast<const float *>(t)[off];
+    if (dtype == KERNL_F16) return (float)static_cast<const f16 *>(t)[off];
+    return (float)static_cast<const bf16 *>(t)[off];
+}
+
 template <typename T>
 __device__ __forceinline__ T from_float(float x);
 template <>

@@ -1007,12 +1007,6 @@ struct SkinnyExtra {
     int rows_per_batch;     // row m of x is position m % rows_per_batch of batch entry m / rows_per_batch
 };
 
-__device__ __forceinline__ float table_value(const void *t, int dtype, int64_t off) {
-    if (dtype == KERNL_F32) return static_cast<const float *>(t)[off];
-    if (dtype == KERNL_F16) return (float)static_cast<const f16 *>(t)[off];
-    return (float)static_cast<const bf16 *>(t)[off];
-}
-
 template <typename T, int MB, bool GATED, int WAVES, int NR, bool W8 = false, bool RMS = false, bool ROPE = false>
 __global__ void __launch_bounds__(64 * WAVES)
 linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,

@@ -1,6 +1,9 @@
 // Linear layer for a FEW rows of x (at most 64: batched decoding steps, pooled outputs), as a stream-K product.
 //
 //     out[M,N] = act(x[M,K] · w[N,K]ᵀ + bias[N]) (+ residual[M,N])
+// and the forms a batched decoding step of a Llama-style layer needs around it, as the one-to-64-row kernel of
+// linear.hip has them (`linear_skinny_kernel`): RMSNorm of x on the way in, the gated linear unit on interleaved
+// weights, rotary embedding of the leading columns, residual — all but the norm's scaling of x in the epilogue.
 //
 // Same semantics as the fused linear kernels (reference: src/kernl/implementations/linear_layer.py:92-210: fp32
 // accumulation, bias added in fp32, activation on the fp32 value, one rounding).  The decomposition is the one of the
@@ -37,8 +40,22 @@
 namespace kernl {
 
 static constexpr int kFewRowWaves = 8;                      // waves per workgroup
-static constexpr int kFewRowTile = 16 * kFewRowWaves;      // output columns per tile
+static constexpr int kFewRowTile = 16 * kFewRowWaves;      // weight rows (output columns) per tile
 static constexpr int kFewRowMaxGrid = 256;                 // one workgroup per CU
+
+enum FewRowMode { kFewRowPlain = 0, kFewRowGated = 1, kFewRowRope = 2 };
+
+struct FewRowArgs {
+    const void *x, *w, *bias, *residual, *rms_w, *cos, *sin;
+    void *out;
+    float *part;      // partial tiles: slot s at s * tile elements
+    float *sqpart;    // sums of squares of the x rows, per workgroup that touched tile 0: [grid][64]
+    int M, N, K;      // N: rows of the weight (gated: twice the output width)
+    int64_t ldx, out_rs, out_cs, res_rs, res_cs, t_bs, t_ss;
+    int act, tiles, nch, run, direct;
+    float eps;
+    int table_dtype, half, rope_cols, rows_per_batch;
+};
 
 struct FewRowPlan {
     int tiles;        // column tiles
@@ -46,12 +63,14 @@ struct FewRowPlan {
     int run;          // units per workgroup
     int grid;         // workgroups
     bool direct;      // every run is exactly one tile: no partial sums
-    int64_t partial_bytes;
+    int64_t partial_bytes, sq_bytes;
 };
 
 static inline int fewrow_row_blocks(int64_t M) { return M <= 16 ? 1 : M <= 32 ? 2 : 4; }
 
-static FewRowPlan fewrow_plan(int64_t M, int64_t N, int64_t K) {
+// N: rows of the weight.  `paired`: the epilogue combines two columns of a tile (gate and value, or the two members of
+// a rotation pair), which only the second kernel does.
+static FewRowPlan fewrow_plan(int64_t M, int64_t N, int64_t K, bool paired) {
     FewRowPlan p;
     p.nch = (int)(K / 64);
     p.tiles = (int)((N + kFewRowTile - 1) / kFewRowTile);
@@ -59,44 +78,56 @@ static FewRowPlan fewrow_plan(int64_t M, int64_t N, int64_t K) {
     int64_t run = (total + kFewRowMaxGrid - 1) / kFewRowMaxGrid;
     if (run < 4) run = 4;
     // whole tiles per workgroup where that costs at most a fifth of the CUs: no partial sums, one launch
-    if (p.tiles <= kFewRowMaxGrid && p.tiles * 5 >= kFewRowMaxGrid * 4) run = p.nch;
+    if (!paired && p.tiles <= kFewRowMaxGrid && p.tiles * 5 >= kFewRowMaxGrid * 4) run = p.nch;
     p.run = (int)run;
     p.grid = (int)((total + run - 1) / run);
-    p.direct = p.run == p.nch;
+    p.direct = !paired && p.run == p.nch;
     p.partial_bytes = p.direct ? 0 : (int64_t)(p.grid + p.tiles) * kFewRowTile * 16 * fewrow_row_blocks(M) * 4;
+    p.sq_bytes = p.direct ? 0 : (int64_t)p.grid * 64 * 4;
     return p;
 }
 
-// Epilogue of one 16 x 16 block of one lane: elements e = 0..3 of `acc` are output columns n .. n + 3 of x row m.
+// Bias, activation, residual and store for elements e = 0..3 of `v`: output columns n .. n + 3 of x row m.
 template <typename T>
-__device__ __forceinline__ void fewrow_epilogue(const f32x4_acc &acc, int m, int n, const T *__restrict__ bias,
-                                                T *__restrict__ out, int M, int N, int64_t out_rs, int64_t out_cs, int act,
-                                                const T *__restrict__ residual, int64_t res_rs, int64_t res_cs) {
-    if (n >= N || m >= M) return;
+__device__ __forceinline__ void fewrow_store(const float (&v)[4], int m, int n, T *__restrict__ out, int n_out,
+                                             int64_t out_rs, int64_t out_cs, const T *__restrict__ residual,
+                                             int64_t res_rs, int64_t res_cs) {
     float y[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        const float b = bias != nullptr ? to_float(bias[min(n + e, N - 1)]) : 0.0f;
-        y[e] = apply_act16(acc[e] + b, act);
-        if (residual != nullptr && n + e < N) y[e] += to_float(residual[(int64_t)m * res_rs + (int64_t)(n + e) * res_cs]);
+        y[e] = v[e];
+        if (residual != nullptr && n + e < n_out) y[e] += to_float(residual[(int64_t)m * res_rs + (int64_t)(n + e) * res_cs]);
     }
-    if (out_cs == 1 && (out_rs & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0 && n + 3 < N) {
-        uint2 v;
-        v.x = pack2<T>(y[0], y[1]);
-        v.y = pack2<T>(y[2], y[3]);
-        *reinterpret_cast<uint2 *>(out + (int64_t)m * out_rs + n) = v;
+    if (out_cs == 1 && (out_rs & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0 && n + 3 < n_out) {
+        uint2 p;
+        p.x = pack2<T>(y[0], y[1]);
+        p.y = pack2<T>(y[2], y[3]);
+        *reinterpret_cast<uint2 *>(out + (int64_t)m * out_rs + n) = p;
     } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            if (n + e < N) out[(int64_t)m * out_rs + (int64_t)(n + e) * out_cs] = from_float<T>(y[e]);
+            if (n + e < n_out) out[(int64_t)m * out_rs + (int64_t)(n + e) * out_cs] = from_float<T>(y[e]);
     }
 }
 
-template <typename T, int MB, int WAVES, int GC, int RING>
-__global__ void __launch_bounds__(64 * WAVES)
-linear_fewrow_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
-                     float *__restrict__ part, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs, int act,
-                     int tiles, int run, int direct, const T *__restrict__ residual, int64_t res_rs, int64_t res_cs) {
+// Plain epilogue of one 16 x 16 block of one lane: elements e = 0..3 of `acc` are output columns n .. n + 3 of x row m;
+// rstd is the row's inverse root mean square (1 without the norm).
+template <typename T>
+__device__ __forceinline__ void fewrow_epilogue(const f32x4_acc &acc, float rstd, int m, int n, const FewRowArgs &a) {
+    if (n >= a.N || m >= a.M) return;
+    const T *bias = static_cast<const T *>(a.bias);
+    float y[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float b = bias != nullptr ? to_float(bias[min(n + e, a.N - 1)]) : 0.0f;
+        y[e] = apply_act16(acc[e] * rstd + b, a.act);
+    }
+    fewrow_store<T>(y, m, n, static_cast<T *>(a.out), a.N, a.out_rs, a.out_cs, static_cast<const T *>(a.residual), a.res_rs,
+                    a.res_cs);
+}
+
+template <typename T, int MB, int WAVES, int GC, int RING, bool RMS>
+__global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowArgs a) {
     typedef typename Vec8<T>::type vec8;
     static_assert(RING % (2 * GC) == 0, "a round of RING units is a whole number of stage pairs");
     constexpr int THREADS = 64 * WAVES;
@@ -104,8 +135,12 @@ linear_fewrow_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
     constexpr int CHUNK_BYTES = MP * 128;       // one staged chunk of x
     constexpr int XP = GC * MP * 8 / THREADS;   // 16-byte pieces of a group of x per thread
     static_assert(GC * MP * 8 % THREADS == 0 && XP >= 1, "every thread stages the same number of pieces");
+    static_assert(2 * GC * CHUNK_BYTES >= THREADS * 4, "the stages double as the buffer of the row sums");
     __shared__ __attribute__((aligned(16))) unsigned char xs[2][GC * CHUNK_BYTES];
+    __shared__ float rstd_s[MP];
 
+    const T *X = static_cast<const T *>(a.x), *W = static_cast<const T *>(a.w);
+    const int M = a.M, N = a.N, K = a.K, tiles = a.tiles, run = a.run, direct = a.direct;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
     const int nch = K / 64;
@@ -138,17 +173,23 @@ linear_fewrow_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
     };
 
     // ---- x: piece i of a thread is 16-byte piece (q & 7) of row (q >> 3) % MP of the group's unit q / (8 MP),
-    // q = tid + THREADS i.  Rows beyond M repeat the last row; units past the end of the run repeat its last unit.
-    vec8 xr[XP];
+    // q = tid + THREADS i — the same row for every i.  Rows beyond M repeat the last row; units past the end of the
+    // run repeat its last unit.  RMS: the norm's weight travels with x, a piece is multiplied by it (one rounding to
+    // 16 bits, as in the reference) on its way into LDS, and the thread adds up the squares of the unscaled values of
+    // the units that count: those of tile 0, whose runs cover every chunk of K exactly once (with whole tiles per
+    // workgroup: all of its own).
+    vec8 xr[XP], gr[RMS ? XP : 1];
     const T *xrow[XP];
     int xunit[XP], xdst[XP];
+    float sq = 0.0f;
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
         const int q = tid + THREADS * i, j = q / (MP * 8), row = (q >> 3) % MP, piece = q & 7;
-        xrow[i] = X + (int64_t)min(row, M - 1) * ldx + piece * 8;
+        xrow[i] = X + (int64_t)min(row, M - 1) * a.ldx + piece * 8;
         xunit[i] = __builtin_amdgcn_readfirstlane(j);   // a wave's 64 pieces belong to one unit
         xdst[i] = j * CHUNK_BYTES + swz_offset<128>(row, piece);
     }
+    const T *grow = static_cast<const T *>(a.rms_w) + (tid & 7) * 8;
     // (the chunk of a group's first unit is kept as a running value: no division in the loop)
     const int last_chunk = (first_chunk + n_units - 1) % nch;
     int xg_unit = 0, xg_chunk = first_chunk;    // first unit of the group the next request is for, and its chunk
@@ -159,14 +200,29 @@ linear_fewrow_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
             c = c >= nch ? c - nch : c;
             c = xg_unit + xunit[i] < n_units ? c : last_chunk;
             xr[i] = *reinterpret_cast<const vec8 *>(xrow[i] + (int64_t)c * 64);
+            if constexpr (RMS) gr[i] = *reinterpret_cast<const vec8 *>(grow + (int64_t)c * 64);
         }
         xg_unit += GC;
         xg_chunk += GC;
         xg_chunk = xg_chunk >= nch ? xg_chunk - nch : xg_chunk;
     };
+    // stages the group requested last (its first unit is xg_unit - GC)
     auto stage_x = [&](int stage) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < XP; ++i) *reinterpret_cast<vec8 *>(xs[stage] + xdst[i]) = xr[i];
+        for (int i = 0; i < XP; ++i) {
+            if constexpr (RMS) {
+                const int u = xg_unit - GC + xunit[i];
+                if (u < n_units && (direct || u_begin + u < nch)) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float xv = to_float(xr[i][e]);
+                        sq = fmaf(xv, xv, sq);
+                    }
+                }
+                xr[i] = xr[i] * gr[i];
+            }
+            *reinterpret_cast<vec8 *>(xs[stage] + xdst[i]) = xr[i];
+        }
     };
     int xoff[MB][2];   // this lane's operand fragments inside a staged chunk
 #pragma unroll
@@ -184,7 +240,7 @@ linear_fewrow_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
     // store the compiler knows of, inside a branch of the loop, makes it wait for EVERY outstanding load at the next
     // use of a fragment (loads and stores share one counter that it then treats as unordered).
     auto flush_partial = [&](int tile) __attribute__((always_inline)) {
-        float4 *dst = reinterpret_cast<float4 *>(part) + (((int64_t)blockIdx.x + tile) * (WAVES * MB) + wave * MB) * 64 + lane;
+        float4 *dst = reinterpret_cast<float4 *>(a.part) + (((int64_t)blockIdx.x + tile) * (WAVES * MB) + wave * MB) * 64 + lane;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
             asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" ::"v"(dst + mb * 64), "v"(acc[mb]) : "memory");
@@ -232,7 +288,7 @@ linear_fewrow_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
             }
         }
     }
-    // ... and the last round, which requests nothing
+    // ... and the last round, which requests no weights
 #pragma unroll
     for (int slot = 0; slot < RING; ++slot) {
         unit_step(i0 + slot, slot);
@@ -244,93 +300,180 @@ linear_fewrow_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
             if (more) __syncthreads();
         }
     }
+
+    if constexpr (RMS) {
+        // a row's squares are spread over the threads (row + MP k) * 8 + p, p = 0..7
+        __syncthreads();                        // every wave is done with the stages
+        float *sqbuf = reinterpret_cast<float *>(&xs[0][0]);
+        sqbuf[tid] = sq;
+        __syncthreads();
+        if (tid < MP) {
+            float t = 0.0f;
+#pragma unroll
+            for (int k = 0; k < THREADS / (8 * MP); ++k)
+#pragma unroll
+                for (int pp = 0; pp < 8; ++pp) t += sqbuf[(tid + MP * k) * 8 + pp];
+            if (direct) rstd_s[tid] = 1.0f / sqrtf(t / (float)K + a.eps);
+            else if (u_begin < nch) a.sqpart[(int64_t)blockIdx.x * 64 + tid] = t;
+        }
+        if (direct) __syncthreads();
+    }
     if (!direct) return;
     // a run of exactly one tile: element e of a lane is output column n + e of x row 16 mb + r
     const int n = first_tile * (16 * WAVES) + 16 * wave + 4 * g;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-        fewrow_epilogue<T>(acc[mb], 16 * mb + r, n, bias, out, M, N, out_rs, out_cs, act, residual, res_rs, res_cs);
+    for (int mb = 0; mb < MB; ++mb) fewrow_epilogue<T>(acc[mb], RMS ? rstd_s[16 * mb + r] : 1.0f, 16 * mb + r, n, a);
 }
 
 // Adds the partial tiles of every tile in workgroup order and runs the epilogue.  One thread per 16-byte element of a
 // tile (the same lane-to-element map as above).  Tile t holds units [t nch, (t + 1) nch), i.e. it was touched by
 // workgroups (t nch) / run .. ((t + 1) nch - 1) / run, and workgroup w left its share in slot w + t.
-template <typename T, int MB, int WAVES>
-__global__ void __launch_bounds__(256)
-linear_fewrow_reduce_kernel(const float *__restrict__ part, const T *__restrict__ bias, T *__restrict__ out, int M, int N,
-                            int64_t out_rs, int64_t out_cs, int act, int tiles, int nch, int run,
-                            const T *__restrict__ residual, int64_t res_rs, int64_t res_cs) {
+//   gated   the weight's rows alternate in blocks of 32 between gate and value (waves 0, 1, 4, 5 hold gates, the waves
+//           two further on the values of the same outputs): out = act(gate + bias) * (value + bias), half as wide
+//   rope    inside a head of 2 * half columns, column d pairs with d + half (`half / 16` waves further on); the pair is
+//           rotated by the row's table entries when it lies below rope_cols; the tile width is a multiple of the head size
+template <typename T, int MB, int WAVES, int MODE>
+__global__ void __launch_bounds__(256) linear_fewrow_reduce_kernel(const FewRowArgs a) {
     constexpr int TILE_ELEMS = WAVES * MB * 64;                      // 16-byte elements of one partial tile
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (int64_t)tiles * TILE_ELEMS) return;
-    const int tile = (int)(idx / TILE_ELEMS), e = (int)(idx - (int64_t)tile * TILE_ELEMS);
-    const int lane = e & 63, mb = (e >> 6) % MB, wave = (e >> 6) / MB;
+    if (idx >= (int64_t)a.tiles * TILE_ELEMS) return;
+    const int tile = (int)(idx / TILE_ELEMS), e0 = (int)(idx - (int64_t)tile * TILE_ELEMS);
+    const int lane = e0 & 63, mb = (e0 >> 6) % MB, wave = (e0 >> 6) / MB;
+    const int pair_waves = MODE == kFewRowGated ? 2 : MODE == kFewRowRope ? a.half / 16 : 0;
+    if (MODE == kFewRowGated && (wave & 2)) return;                  // value blocks: their gate's thread takes them
+    if (MODE == kFewRowRope && ((16 * wave) % (2 * a.half)) >= a.half) return;
+    const int m = 16 * mb + (lane & 15);
+    const int n = tile * (16 * WAVES) + 16 * wave + 4 * (lane >> 4);  // row of the weight (first of four)
+    if (m >= a.M || n >= a.N) return;
+    const int nch = a.nch, run = a.run;
     const int w_first = (tile * nch) / run, w_last = ((tile + 1) * nch - 1) / run;   // units fit 31 bits
-    const float4 *theirs = reinterpret_cast<const float4 *>(part) + ((int64_t)w_first + tile) * TILE_ELEMS + e;
-    f32x4_acc acc = {0.0f, 0.0f, 0.0f, 0.0f};
     const int n_slots = w_last - w_first + 1;
-    int s = 0;
-    for (; s + 4 <= n_slots; s += 4) {   // four loads in flight, added in workgroup order
-        float4 v[4];
+    const float4 *theirs = reinterpret_cast<const float4 *>(a.part) + ((int64_t)w_first + tile) * TILE_ELEMS + e0;
+    auto slot_sum = [&](const float4 *src) __attribute__((always_inline)) -> f32x4_acc {
+        f32x4_acc acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        int s = 0;
+        for (; s + 4 <= n_slots; s += 4) {   // four loads in flight, added in workgroup order
+            float4 v[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = theirs[(int64_t)(s + u) * TILE_ELEMS];
+            for (int u = 0; u < 4; ++u) v[u] = src[(int64_t)(s + u) * TILE_ELEMS];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            acc[0] += v[u].x;
-            acc[1] += v[u].y;
-            acc[2] += v[u].z;
-            acc[3] += v[u].w;
+            for (int u = 0; u < 4; ++u) {
+                acc[0] += v[u].x;
+                acc[1] += v[u].y;
+                acc[2] += v[u].z;
+                acc[3] += v[u].w;
+            }
+        }
+        for (; s < n_slots; ++s) {
+            const float4 v = src[(int64_t)s * TILE_ELEMS];
+            acc[0] += v.x;
+            acc[1] += v.y;
+            acc[2] += v.z;
+            acc[3] += v.w;
+        }
+        return acc;
+    };
+    f32x4_acc acc = slot_sum(theirs);
+    float rstd = 1.0f;
+    if (a.rms_w != nullptr) {
+        float t = 0.0f;
+        const int w_sq_last = (nch - 1) / run;
+        for (int w = 0; w <= w_sq_last; ++w) t += a.sqpart[(int64_t)w * 64 + m];
+        rstd = 1.0f / sqrtf(t / (float)a.K + a.eps);
+    }
+    if (MODE == kFewRowPlain) {
+        fewrow_epilogue<T>(acc, rstd, m, n, a);
+        return;
+    }
+    const f32x4_acc other = slot_sum(theirs + pair_waves * MB * 64);
+    const T *bias = static_cast<const T *>(a.bias);
+    T *out = static_cast<T *>(a.out);
+    const T *residual = static_cast<const T *>(a.residual);
+    if (MODE == kFewRowGated) {
+        // weight rows n .. n + 3 are gates of output columns (n / 64) * 32 + n % 32 ..; their values sit 32 rows on
+        const int n_out = (n >> 6) * 32 + (n & 31);
+        float y[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float bg = bias != nullptr ? to_float(bias[min(n + e, a.N - 1)]) : 0.0f;
+            const float bv = bias != nullptr ? to_float(bias[min(n + e + 32, a.N - 1)]) : 0.0f;
+            y[e] = apply_act16(acc[e] * rstd + bg, a.act) * (other[e] * rstd + bv);
+        }
+        fewrow_store<T>(y, m, n_out, out, a.N / 2, a.out_rs, a.out_cs, residual, a.res_rs, a.res_cs);
+        return;
+    }
+    // rope: columns n .. n + 3 and their partners `half` further on
+    float lo[4], hi[4];
+    const int d = n % (2 * a.half);
+    const int64_t trow = (int64_t)(m / a.rows_per_batch) * a.t_bs + (int64_t)(m % a.rows_per_batch) * a.t_ss;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float v0 = acc[e] * rstd, v1 = other[e] * rstd;
+        if (bias != nullptr) {
+            v0 += to_float(bias[min(n + e, a.N - 1)]);
+            v1 += to_float(bias[min(n + e + a.half, a.N - 1)]);
+        }
+        lo[e] = v0;
+        hi[e] = v1;
+        if (n + e < a.rope_cols) {
+            const float c0 = table_value(a.cos, a.table_dtype, trow + d + e), s0 = table_value(a.sin, a.table_dtype, trow + d + e);
+            const float c1 = table_value(a.cos, a.table_dtype, trow + d + e + a.half);
+            const float s1 = table_value(a.sin, a.table_dtype, trow + d + e + a.half);
+            lo[e] = v0 * c0 - v1 * s0;
+            hi[e] = v1 * c1 + v0 * s1;
         }
     }
-    for (; s < n_slots; ++s) {
-        const float4 v = theirs[(int64_t)s * TILE_ELEMS];
-        acc[0] += v.x;
-        acc[1] += v.y;
-        acc[2] += v.z;
-        acc[3] += v.w;
-    }
-    fewrow_epilogue<T>(acc, 16 * mb + (lane & 15), tile * (16 * WAVES) + 16 * wave + 4 * (lane >> 4), bias, out, M, N, out_rs,
-                       out_cs, act, residual, res_rs, res_cs);
+    fewrow_store<T>(lo, m, n, out, a.N, a.out_rs, a.out_cs, residual, a.res_rs, a.res_cs);
+    fewrow_store<T>(hi, m, n + a.half, out, a.N, a.out_rs, a.out_cs, residual, a.res_rs, a.res_cs);
 }
 
 template <typename T>
-static void launch_fewrow(const void *x, const void *w, const void *bias, const void *residual, void *out, void *workspace,
-                          const FewRowPlan &p, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
-                          int64_t res_rs, int64_t res_cs, int act, hipStream_t st) {
-    float *part = static_cast<float *>(workspace);
+static void launch_fewrow(FewRowArgs a, const FewRowPlan &p, int mode, hipStream_t st) {
+    const int mb = fewrow_row_blocks(a.M);
+    const dim3 grid((unsigned)p.grid), block(64 * kFewRowWaves);
+    const dim3 rgrid((unsigned)(((int64_t)p.tiles * kFewRowWaves * mb * 64 + 255) / 256));
+    const bool rms = a.rms_w != nullptr;
     // x groups of 2 units and a ring of 4 measured best (by 0.5 to 1.4 us against 4 and 8); 16 rows of x are too few
     // pieces for 512 threads to stage 2 units at a time
-#define KERNL_FEWROW(MBV)                                                                                               \
-    do {                                                                                                                \
-        hipLaunchKernelGGL((linear_fewrow_kernel<T, MBV, kFewRowWaves, (MBV == 1 ? 4 : 2), (MBV == 1 ? 8 : 4)>),        \
-                           dim3((unsigned)p.grid),                                                                      \
-                           dim3(64 * kFewRowWaves), 0, st, static_cast<const T *>(x), static_cast<const T *>(w),        \
-                           static_cast<const T *>(bias), static_cast<T *>(out), part, M, N, K, ldx, out_rs, out_cs,    \
-                           act, p.tiles, p.run, p.direct ? 1 : 0, static_cast<const T *>(residual), res_rs, res_cs);   \
-        if (!p.direct)                                                                                                  \
-            hipLaunchKernelGGL((linear_fewrow_reduce_kernel<T, MBV, kFewRowWaves>),                                     \
-                               dim3((unsigned)(((int64_t)p.tiles * kFewRowWaves * MBV * 64 + 255) / 256)), dim3(256), 0, \
-                               st, part, static_cast<const T *>(bias), static_cast<T *>(out), M, N, out_rs, out_cs,     \
-                               act, p.tiles, p.nch, p.run, static_cast<const T *>(residual), res_rs, res_cs);           \
+#define KERNL_FEWROW_MAIN(MBV, RMSV)                                                                                   \
+    hipLaunchKernelGGL((linear_fewrow_kernel<T, MBV, kFewRowWaves, (MBV == 1 ? 4 : 2), (MBV == 1 ? 8 : 4), RMSV>), grid, \
+                       block, 0, st, a)
+#define KERNL_FEWROW_REDUCE(MBV, MODEV)                                                                                \
+    hipLaunchKernelGGL((linear_fewrow_reduce_kernel<T, MBV, kFewRowWaves, MODEV>), rgrid, dim3(256), 0, st, a)
+#define KERNL_FEWROW(MBV)                                                                                              \
+    do {                                                                                                               \
+        if (rms) KERNL_FEWROW_MAIN(MBV, true);                                                                         \
+        else KERNL_FEWROW_MAIN(MBV, false);                                                                            \
+        if (!p.direct) {                                                                                               \
+            if (mode == kFewRowGated) KERNL_FEWROW_REDUCE(MBV, kFewRowGated);                                          \
+            else if (mode == kFewRowRope) KERNL_FEWROW_REDUCE(MBV, kFewRowRope);                                       \
+            else KERNL_FEWROW_REDUCE(MBV, kFewRowPlain);                                                               \
+        }                                                                                                              \
     } while (0)
-    if (M <= 16) KERNL_FEWROW(1);
-    else if (M <= 32) KERNL_FEWROW(2);
+    if (mb == 1) KERNL_FEWROW(1);
+    else if (mb == 2) KERNL_FEWROW(2);
     else KERNL_FEWROW(4);
 #undef KERNL_FEWROW
+#undef KERNL_FEWROW_REDUCE
+#undef KERNL_FEWROW_MAIN
 }
 
 }  // namespace kernl
 
-extern "C" int64_t kernl_linear_fewrow_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+extern "C" int64_t kernl_linear_fewrow_workspace_bytes(int64_t M, int64_t N, int64_t K, int gated, int rotated) {
     using namespace kernl;
     if (M <= 0 || M > 64 || N <= 0 || K < 256 || K % 64 != 0) return 0;
-    return fewrow_plan(M, N, K).partial_bytes;
+    const FewRowPlan p = fewrow_plan(M, gated ? 2 * N : N, K, gated || rotated);
+    return p.partial_bytes + p.sq_bytes;
 }
 
-extern "C" int kernl_linear_fewrow_fwd(const void *x, const void *w, const void *bias, const void *residual, void *out,
-                                       void *workspace, int64_t workspace_bytes, int64_t M, int64_t N, int64_t K,
-                                       const int64_t x_strides[2], const int64_t out_strides[2],
-                                       const int64_t residual_strides[2], int activation, int dtype, void *stream) {
+extern "C" int kernl_linear_fewrow_fwd(const void *x, const void *rms_weight, float eps, const void *w, const void *bias,
+                                       const void *residual, void *out, void *workspace, int64_t workspace_bytes,
+                                       int64_t M, int64_t N, int64_t K, const int64_t x_strides[2],
+                                       const int64_t out_strides[2], const int64_t residual_strides[2], const void *cos,
+                                       const void *sin, int64_t head_dim, int64_t rope_cols, int64_t rows_per_batch,
+                                       const int64_t table_strides[3], int table_dtype, int activation, int gated,
+                                       int dtype, void *stream) {
     using namespace kernl;
     if (x == nullptr || w == nullptr || out == nullptr || x_strides == nullptr || out_strides == nullptr)
         return set_error(KERNL_ERR_INVALID_ARG, "few-row linear: x, w, out and their strides must not be NULL");
@@ -343,29 +486,57 @@ extern "C" int kernl_linear_fewrow_fwd(const void *x, const void *w, const void 
         return set_error(KERNL_ERR_INVALID_ARG, "few-row linear: unknown activation %d", activation);
     if (dtype != KERNL_F16 && dtype != KERNL_BF16)
         return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: only f16 and bf16 are supported, got dtype %d", dtype);
-    if (M > 64 || K % 64 != 0 || K < 256 || N > (1 << 30) || K > INT32_MAX)
+    if (M > 64 || K % 64 != 0 || K < 256 || N > (1 << 29) || K > INT32_MAX)
         return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: at most 64 rows of x and K a multiple of 64, at least 256 "
                          "(M=%lld K=%lld)", (long long)M, (long long)K);
-    if (x_strides[1] != 1 || x_strides[0] % 8 != 0 || !aligned16(x) || !aligned16(w))
+    if (x_strides[1] != 1 || x_strides[0] % 8 != 0 || !aligned16(x) || !aligned16(w) ||
+        (rms_weight != nullptr && !aligned16(rms_weight)))
         return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: x needs unit feature stride and 16-byte aligned rows, the "
-                         "weight a 16-byte aligned base");
+                         "weights 16-byte aligned bases");
     if (workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
         return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: the workspace must be 16-byte aligned");
+    const bool rope = cos != nullptr || sin != nullptr;
+    if (gated && (rope || N % 32 != 0))
+        return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: the gated form takes no rotation and needs an output width "
+                         "that is a multiple of 32 (the interleaving block), got %lld", (long long)N);
+    FewRowArgs a = {};
+    if (rope) {
+        if (cos == nullptr || sin == nullptr || table_strides == nullptr)
+            return set_error(KERNL_ERR_INVALID_ARG, "few-row linear: rotation needs cos, sin and their strides");
+        if (table_dtype != KERNL_F16 && table_dtype != KERNL_BF16 && table_dtype != KERNL_F32)
+            return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: unknown table dtype %d", table_dtype);
+        if ((head_dim != 32 && head_dim != 64 && head_dim != 128) || N % head_dim != 0 || rope_cols < 0 || rope_cols > N ||
+            rope_cols % head_dim != 0 || rows_per_batch <= 0 || table_strides[2] != 1 || activation != KERNL_ACT_NONE)
+            return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: rotation needs a head size of 32, 64 or 128 that divides "
+                             "N and rope_cols, tables with unit feature stride, rows_per_batch > 0 and no activation");
+        a.cos = cos; a.sin = sin;
+        a.t_bs = table_strides[0]; a.t_ss = table_strides[1];
+        a.table_dtype = table_dtype;
+        a.half = (int)(head_dim / 2);
+        a.rope_cols = (int)rope_cols;
+        a.rows_per_batch = (int)rows_per_batch;
+    }
     if (M == 0) return KERNL_OK;
-    if (((N + kFewRowTile - 1) / kFewRowTile) * (K / 64) >= (int64_t)1 << 30)
+    const int64_t n_rows = gated ? 2 * N : N;   // rows of the weight
+    if (((n_rows + kFewRowTile - 1) / kFewRowTile) * (K / 64) >= (int64_t)1 << 30)
         return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: N * K too large");
-    const FewRowPlan p = fewrow_plan(M, N, K);
-    if (!p.direct && (workspace == nullptr || workspace_bytes < p.partial_bytes))
+    const FewRowPlan p = fewrow_plan(M, n_rows, K, gated || rope);
+    const int64_t need = p.partial_bytes + p.sq_bytes;
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need))
         return set_error(KERNL_ERR_INVALID_ARG, "few-row linear: the workspace must hold %lld bytes "
-                         "(kernl_linear_fewrow_workspace_bytes), got %lld", (long long)p.partial_bytes,
+                         "(kernl_linear_fewrow_workspace_bytes), got %lld", (long long)need,
                          (long long)(workspace == nullptr ? 0 : workspace_bytes));
+    a.x = x; a.w = w; a.bias = bias; a.residual = residual; a.rms_w = rms_weight; a.out = out;
+    a.part = static_cast<float *>(workspace);
+    a.sqpart = workspace != nullptr ? reinterpret_cast<float *>(static_cast<char *>(workspace) + p.partial_bytes) : nullptr;
+    a.M = (int)M; a.N = (int)n_rows; a.K = (int)K;
+    a.ldx = x_strides[0]; a.out_rs = out_strides[0]; a.out_cs = out_strides[1];
+    a.res_rs = residual ? residual_strides[0] : 0; a.res_cs = residual ? residual_strides[1] : 0;
+    a.act = activation; a.tiles = p.tiles; a.nch = p.nch; a.run = p.run; a.direct = p.direct ? 1 : 0;
+    a.eps = eps;
+    const int mode = gated ? kFewRowGated : rope ? kFewRowRope : kFewRowPlain;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int64_t res_rs = residual ? residual_strides[0] : 0, res_cs = residual ? residual_strides[1] : 0;
-    if (dtype == KERNL_F16)
-        launch_fewrow<f16>(x, w, bias, residual, out, workspace, p, (int)M, (int)N, (int)K, x_strides[0], out_strides[0],
-                           out_strides[1], res_rs, res_cs, activation, st);
-    else
-        launch_fewrow<bf16>(x, w, bias, residual, out, workspace, p, (int)M, (int)N, (int)K, x_strides[0], out_strides[0],
-                            out_strides[1], res_rs, res_cs, activation, st);
-    return check_launch("linear (few rows, split K)");
+    if (dtype == KERNL_F16) launch_fewrow<f16>(a, p, mode, st);
+    else launch_fewrow<bf16>(a, p, mode, st);
+    return check_launch("linear (few rows, stream-K)");
 }

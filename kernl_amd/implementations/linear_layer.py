@@ -135,7 +135,10 @@ class LinearGLU(torch.autograd.Function):
             x_ = x_.contiguous()
         M, N = x_.shape[0], weight.shape[0] // 2
         out = torch.empty((M, N), device=x.device, dtype=x.dtype)
-        _lib.linear_glu_fwd(x_, weight, bias, out, ACTIVATIONS.get(activation, _lib.ACT_NONE))
+        if takes_few_row_kernel(x_, weight):
+            _lib.linear_fewrow_fwd(x_, weight, bias, None, out, ACTIVATIONS.get(activation, _lib.ACT_NONE), gated=True)
+        else:
+            _lib.linear_glu_fwd(x_, weight, bias, out, ACTIVATIONS.get(activation, _lib.ACT_NONE))
         return out if x.ndim == 2 else out.reshape(*x.shape[:-1], N)
 
 
@@ -174,7 +177,11 @@ def rms_linear_layer(
         eps = max(eps, 1.6e-5)  # the fp16 policy of the RMSNorm operator (reference: layer_norm.py:295-296)
     if _lib.linear_rms_supported(x_) and (not gated or n_out % GLU_BLOCK == 0):
         out = torch.empty((x_.shape[0], n_out), device=x.device, dtype=x.dtype)
-        _lib.linear_rms_fwd(x_, rms_weight, eps, weight, bias, out, ACTIVATIONS.get(activation, _lib.ACT_NONE), gated)
+        if takes_few_row_kernel(x_, weight):
+            _lib.linear_fewrow_fwd(x_, weight, bias, None, out, ACTIVATIONS.get(activation, _lib.ACT_NONE),
+                                   rms_weight=rms_weight, eps=eps, gated=gated)
+        else:
+            _lib.linear_rms_fwd(x_, rms_weight, eps, weight, bias, out, ACTIVATIONS.get(activation, _lib.ACT_NONE), gated)
         return out if x.ndim == 2 else out.reshape(*x.shape[:-1], n_out)
     normed = layer_norm(x, rms_weight, None, eps, use_rms_norm=True)
     if gated:
@@ -234,8 +241,9 @@ def decode_linear_layer(
         assert residual.dtype == x.dtype and residual.numel() == x_.shape[0] * N
         res_ = residual.reshape(-1, N)
     out = torch.empty((x_.shape[0], N), device=x.device, dtype=x.dtype)
-    if rms_weight is None and cos is None and takes_few_row_kernel(x_, weight):
-        _lib.linear_fewrow_fwd(x_, weight, bias, res_, out, _lib.ACT_NONE)
+    if takes_few_row_kernel(x_, weight) and (cos is None or head_dim in (32, 64, 128)):
+        _lib.linear_fewrow_fwd(x_, weight, bias, res_, out, _lib.ACT_NONE, rms_weight=rms_weight, eps=eps, cos=cos, sin=sin,
+                               head_dim=head_dim, rope_cols=rope_cols, rows_per_batch=rows_per_batch)
     else:
         _lib.linear_decode_fwd(x_, rms_weight, eps, weight, bias, res_, out, cos, sin, head_dim, rope_cols, rows_per_batch)
     return out if x.ndim == 2 else out.reshape(*x.shape[:-1], N)

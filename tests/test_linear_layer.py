@@ -422,6 +422,82 @@ def test_linear_few_rows_stream_k(shape, dtype, close):
     close(outs[2], linear_oracle(x, w, b, "") + res.float(), dtype, scale="magnitude", what=f"stream-K {shape} residual")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize(
+    "case",
+    # batch, positions, K, heads (query + key + value), head size, rotated heads, bias, residual
+    [(5, 4, 320, 6, 128, 4, True, True), (33, 1, 256, 10, 64, 10, False, False), (2, 32, 704, 12, 32, 8, True, True),
+     (40, 1, 4096, 96, 128, 64, False, False), (16, 1, 512, 4, 128, 2, False, True), (3, 7, 1024, 7, 64, 0, True, False)],
+    ids=lambda c: "x".join(str(int(v)) for v in c),
+)
+def test_few_rows_stream_k_with_norm_rotation_and_residual(case, dtype, close):
+    """The batched decoding step's query/key/value projection on the stream-K kernel: RMSNorm on the way in (the row sums
+    of squares travel with the partial tiles of tile 0), rotation of the query and key heads and residual in the second
+    launch's epilogue; against the composition of the RMSNorm, linear and rotary oracles, as for the 64-row kernel."""
+    from oracle import rms_norm_oracle, rotary_oracle
+
+    B, S, K, heads, D, rot_heads, with_bias, with_residual = case
+    N, M = heads * D, B * S
+    gen = torch.Generator().manual_seed(61)
+    x = (torch.randn((B, S, K), generator=gen) * 2.0 + 0.3).to(dtype)
+    g = (1.0 + 0.2 * torch.randn((K,), generator=gen)).to(dtype)
+    w = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+    b = (0.5 * torch.randn((N,), generator=gen)).to(dtype) if with_bias else None
+    res = torch.randn((M, N), generator=gen).to(dtype) if with_residual else None
+    angles = torch.rand((B, S, D), generator=gen) * 6.28
+    cos, sin = angles.cos(), angles.sin()                       # fp32 tables
+    eps = 1e-5 if dtype == torch.bfloat16 else 1.6e-5
+    out = torch.empty((M, N), dtype=dtype, device="cuda")
+    need = _lib.linear_fewrow_workspace_bytes(M, N, K, False, True)
+    ws = torch.full((max(need, 16) // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    _lib.linear_fewrow_fwd(x.reshape(M, K).cuda(), w.cuda(), None if b is None else b.cuda(), None if res is None else res.cuda(),
+                           out, _lib.ACT_NONE, ws, rms_weight=g.cuda(), eps=eps, cos=cos.cuda(), sin=sin.cuda(), head_dim=D,
+                           rope_cols=rot_heads * D, rows_per_batch=S)
+    torch.cuda.synchronize()
+    y = linear_oracle(rms_norm_oracle(x, g, eps), w, b, "")
+    heads_view = y.reshape(B, S, heads, D)
+    rotated = rotary_oracle(heads_view[:, :, :rot_heads], cos[:, :, None, :], sin[:, :, None, :])
+    ref = torch.cat((rotated, heads_view[:, :, rot_heads:]), dim=2).reshape(M, N)
+    if res is not None:
+        ref = ref + res.float()
+    close(out, ref, dtype, scale="magnitude", what=f"stream-K decode projection {case}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("with_norm", [False, True], ids=["plain", "rms"])
+@pytest.mark.parametrize("shape", [(20, 352, 320), (33, 96, 256), (64, 11008, 4096), (10, 14336, 256), (48, 1000, 512)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_few_rows_stream_k_gated_and_normalised(shape, with_norm, dtype, close):
+    """The gated linear unit on interleaved weights (the second launch multiplies act(gate) by the value two waves
+    further on) and the plain form with bias + activation, each with and without the RMSNorm prologue; 14336 outputs
+    against K = 256 are 224 tiles (whole tiles per workgroup for the plain form, which then computes the norm's row
+    sums itself)."""
+    from kernl_amd.implementations.linear_layer import interleave_glu_rows
+    from oracle import glu_oracle, rms_norm_oracle
+
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(67)
+    x = (torch.randn((M, K), generator=gen) * 3.0 + 0.5).to(dtype)
+    g = (1.0 + 0.2 * torch.randn((K,), generator=gen)).to(dtype)
+    eps = 1e-5 if dtype == torch.bfloat16 else 1.6e-5
+    xin = rms_norm_oracle(x, g, eps) if with_norm else x
+    kw = dict(rms_weight=g.cuda(), eps=eps) if with_norm else {}
+    w = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+    b = (0.5 * torch.randn((N,), generator=gen)).to(dtype)
+    out = torch.empty((M, N), dtype=dtype, device="cuda")
+    _lib.linear_fewrow_fwd(x.cuda(), w.cuda(), b.cuda(), None, out, _lib.ACT_SILU, **kw)
+    torch.cuda.synchronize()
+    close(out, linear_oracle(xin, w, b, "silu"), dtype, scale="magnitude", what=f"stream-K {shape} bias + silu, norm {with_norm}")
+    if N % 32 == 0:
+        wv = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+        bv = (0.5 * torch.randn((N,), generator=gen)).to(dtype)
+        out = torch.empty((M, N), dtype=dtype, device="cuda")
+        _lib.linear_fewrow_fwd(x.cuda(), interleave_glu_rows(w, wv).cuda(), interleave_glu_rows(b, bv).cuda(), None, out,
+                               _lib.ACT_SILU, gated=True, **kw)
+        torch.cuda.synchronize()
+        close(out, glu_oracle(xin, w, b, wv, bv, "silu"), dtype, scale="magnitude", what=f"stream-K gated {shape}, norm {with_norm}")
+
+
 def test_linear_few_rows_stream_k_is_what_the_operators_run(close, monkeypatch):
     """17 to 64 rows against a large weight: `linear_layer` and the residual form of `decode_linear_layer` take the
     stream-K kernel; fewer rows, small weights and a saved pre-activation keep the other kernels.  Strided rows of x
