@@ -434,6 +434,33 @@ def main():
             extra["decode_linear_fp8w_us_graph_replay"] = round(t * 1e3, 2)
             extra["decode_linear_fp8w_gbps_graph_replay"] = round(w_dec8[0].numel() / (t * 1e-3) / 1e9, 1)
             del w_dec8, x_dec
+
+            # a BATCHED decoding step (32 sequences, one new token each): 32 rows against the same kind of weights,
+            # and against the 4096 x 11008 down projection with the residual — the stream-K few-row kernel
+            from kernl_amd.implementations.linear_layer import decode_linear_layer
+            x32 = torch.randn((32, 4096), generator=gen).half().to(dev)
+            w_sq = [(torch.randn((4096, 4096), generator=gen) * 0.02).half().to(dev) for _ in range(12)]
+
+            def batched_linears():
+                for w_i in w_sq:
+                    linear_layer(x32, w_i, None)
+
+            t = graph_time_ms(batched_linears, reps=4) / len(w_sq)
+            extra["decode_linear_32x4096x4096_us_graph_replay"] = round(t * 1e3, 2)
+            extra["decode_linear_32x4096x4096_gbps"] = round(w_sq[0].numel() * 2 / (t * 1e-3) / 1e9, 1)
+            del w_sq
+            x32f = torch.randn((32, 11008), generator=gen).half().to(dev)
+            res32 = torch.randn((32, 4096), generator=gen).half().to(dev)
+            w_dn = [(torch.randn((4096, 11008), generator=gen) * 0.01).half().to(dev) for _ in range(5)]
+
+            def batched_down():
+                for w_i in w_dn:
+                    decode_linear_layer(x32f, w_i, None, residual=res32)
+
+            t = graph_time_ms(batched_down, reps=4) / len(w_dn)
+            extra["decode_down_residual_32x4096x11008_us_graph_replay"] = round(t * 1e3, 2)
+            extra["decode_down_residual_32x4096x11008_gbps"] = round(w_dn[0].numel() * 2 / (t * 1e-3) / 1e9, 1)
+            del w_dn, x32, x32f, res32
         except Exception as exc:  # the headline must still be printed
             extra["decoder_kernels_error"] = f"{type(exc).__name__}: {exc}"[:300]
 

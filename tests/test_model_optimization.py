@@ -436,12 +436,14 @@ def test_generation_with_growing_cache(family):
     assert agree >= 3
 
 
-def test_llama_generation_runs_the_decode_projection_kernel(monkeypatch):
+@pytest.mark.parametrize("batch, hidden, heads, inter", [(2, 512, 4, 1408), (24, 2048, 16, 5632)], ids=["b2-h512", "b24-h2048"])
+def test_llama_generation_runs_the_decode_projection_kernel(batch, hidden, heads, inter, monkeypatch):
     """Greedy generation with a growing key/value cache on a Llama-shaped fp16 model under `optimize_model`: each
     decoding step is a new cache length, hence a new compilation and graph.  In the steps after the prompt every layer's
     query/key/value projection must run as one call of the few-row projection kernel with the RMS prologue and the
     rotation, and the output and down projections as calls with the residual; the scores follow the eager fp16
-    model's while the two greedy paths pick the same tokens."""
+    model's while the two greedy paths pick the same tokens.  With 24 sequences and 2048-wide layers the decoding steps
+    have enough rows and weights for the stream-K form of those kernels (and of the gated feed-forward entry)."""
     from torch._dynamo.utils import counters
     from transformers import LlamaConfig, LlamaForCausalLM
 
@@ -452,27 +454,38 @@ def test_llama_generation_runs_the_decode_projection_kernel(monkeypatch):
     counters.clear()
     torch.manual_seed(0)
     layers, steps = 2, 12
-    cfg = LlamaConfig(num_hidden_layers=layers, hidden_size=512, num_attention_heads=4, num_key_value_heads=4,
-                      intermediate_size=1408, vocab_size=1000, rms_norm_eps=1e-5, max_position_embeddings=512,
+    cfg = LlamaConfig(num_hidden_layers=layers, hidden_size=hidden, num_attention_heads=heads, num_key_value_heads=heads,
+                      intermediate_size=inter, vocab_size=1000, rms_norm_eps=1.6e-5, max_position_embeddings=512,
                       pad_token_id=0, bos_token_id=1, eos_token_id=2)
+    # (eps 1.6e-5: the value the fp16 RMSNorm operator clamps smaller ones to — reference layer_norm.py:295-296 — so that
+    # the eager model and the operators normalise alike; what the clamp does is measured in the Llama-shaped tests above)
     cfg._attn_implementation = "sdpa"
     model = LlamaForCausalLM(cfg).eval().half().cuda()
     gen = torch.Generator().manual_seed(1)
-    ids = torch.randint(3, 1000, (2, 20), generator=gen).cuda()
+    ids = torch.randint(3, 1000, (batch, 20), generator=gen).cuda()
     kwargs = dict(input_ids=ids, attention_mask=torch.ones_like(ids), min_new_tokens=steps, max_new_tokens=steps,
                   do_sample=False, output_scores=True, return_dict_in_generate=True)
     with torch.inference_mode():
         ref = model.generate(**kwargs)
 
-    calls = {"rotated": 0, "residual": 0}
-    real = _lib.linear_decode_fwd
+    calls = {"rotated": 0, "residual": 0, "gated": 0}
+    real, real_few = _lib.linear_decode_fwd, _lib.linear_fewrow_fwd
 
     def counting(x2d, rms_weight, eps, weight, bias, residual2d, out2d, cos=None, sin=None, *args, **kw):
+        assert batch == 2, "24 rows belong on the stream-K kernel"
         calls["rotated"] += int(cos is not None and rms_weight is not None)
         calls["residual"] += int(residual2d is not None)
         return real(x2d, rms_weight, eps, weight, bias, residual2d, out2d, cos, sin, *args, **kw)
 
+    def counting_few(x2d, weight, bias, residual2d, out2d, activation, workspace=None, **kw):
+        assert batch == 24 and x2d.shape[0] == batch
+        calls["rotated"] += int(kw.get("cos") is not None and kw.get("rms_weight") is not None)
+        calls["residual"] += int(residual2d is not None)
+        calls["gated"] += int(bool(kw.get("gated")) and kw.get("rms_weight") is not None)
+        return real_few(x2d, weight, bias, residual2d, out2d, activation, workspace, **kw)
+
     monkeypatch.setattr(_lib, "linear_decode_fwd", counting)
+    monkeypatch.setattr(_lib, "linear_fewrow_fwd", counting_few)
     optimize_model(model.model)
     with torch.inference_mode():
         model.generate(**kwargs)        # compiles and captures one graph per step
@@ -484,6 +497,7 @@ def test_llama_generation_runs_the_decode_projection_kernel(monkeypatch):
     # warm-up run and capture run of each of the steps after the prompt
     assert calls["rotated"] >= 2 * (steps - 1) * layers, calls
     assert calls["residual"] >= 2 * (steps - 1) * layers * 2, calls
+    assert batch == 2 or calls["gated"] >= 2 * (steps - 1) * layers, calls
     prompt = ref.sequences.shape[1] - steps
     agree = 0
     for t, (a, b) in enumerate(zip(out.scores, ref.scores)):
