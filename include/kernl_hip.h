@@ -237,7 +237,7 @@ int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float eps, const
                          int activation, int gated, int dtype, void *stream);
 
 /*
- * The linear layer for a FEW rows of x with many columns and a long K (batched decoding steps: 17 to 64 rows, where
+ * The linear layer for a FEW rows of x with many columns and a long K (batched decoding steps: 17 to 128 rows, where
  * kernl_linear_fwd's weight-streaming kernel re-reads x once per 16 to 64 output columns and its tile kernels leave
  * most of their rows empty), with everything a decoder layer puts around its projections:
  *     y   = (rms_weight ? rsqrt(mean(x^2) + eps) * ((x * rms_weight) @ w^T) : x @ w^T) + bias
@@ -252,7 +252,7 @@ int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float eps, const
  * the weight, 64-wide k chunk) units are dealt in equal contiguous runs to at most 256 workgroups, tiles cut by a run
  * boundary are completed from fp32 partial tiles by a second small launch that adds them in a fixed order (results do
  * not depend on timing) and runs the epilogue.
- *   M <= 64, K % 64 == 0, K >= 256, f16 / bf16, x with unit feature stride and 16-byte aligned rows, w contiguous.
+ *   M <= 128, K % 64 == 0, K >= 256, f16 / bf16, x with unit feature stride and 16-byte aligned rows, w contiguous.
  *   workspace  device memory of at least kernl_linear_fewrow_workspace_bytes(M, N, K, gated, rotated) bytes, 16-byte
  *              aligned, contents irrelevant before and after the call (NULL when that function returns 0); calls that
  *              overlap in time need workspaces of their own.

@@ -388,7 +388,7 @@ def linear_fewrow_supported(x2d, weight) -> bool:
     """What `kernl_linear_fewrow_fwd` takes: 16-bit rows, at most 64 of them, K a multiple of 64 from 256 on."""
     M, K = x2d.shape
     return (
-        x2d.dtype in (torch.float16, torch.bfloat16) and weight.dtype == x2d.dtype and 0 < M <= 64
+        x2d.dtype in (torch.float16, torch.bfloat16) and weight.dtype == x2d.dtype and 0 < M <= 128
         and K % 64 == 0 and K >= 256 and x2d.stride(1) == 1 and x2d.stride(0) % 8 == 0 and x2d.data_ptr() % 16 == 0
         and weight.is_contiguous() and weight.data_ptr() % 16 == 0
     )

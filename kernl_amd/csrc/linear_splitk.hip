@@ -1,4 +1,4 @@
-// Linear layer for a FEW rows of x (at most 64: batched decoding steps, pooled outputs), as a stream-K product.
+// Linear layer for a FEW rows of x (at most 128: batched decoding steps, pooled outputs), as a stream-K product.
 //
 //     out[M,N] = act(x[M,K] · w[N,K]ᵀ + bias[N]) (+ residual[M,N])
 // and the forms a batched decoding step of a Llama-style layer needs around it, as the one-to-64-row kernel of
@@ -49,7 +49,7 @@ struct FewRowArgs {
     const void *x, *w, *bias, *residual, *rms_w, *cos, *sin;
     void *out;
     float *part;      // partial tiles: slot s at s * tile elements
-    float *sqpart;    // sums of squares of the x rows, per workgroup that touched tile 0: [grid][64]
+    float *sqpart;    // sums of squares of the x rows, per workgroup that touched tile 0: [grid][128]
     int M, N, K;      // N: rows of the weight (gated: twice the output width)
     int64_t ldx, out_rs, out_cs, res_rs, res_cs, t_bs, t_ss;
     int act, tiles, nch, run, direct;
@@ -66,7 +66,8 @@ struct FewRowPlan {
     int64_t partial_bytes, sq_bytes;
 };
 
-static inline int fewrow_row_blocks(int64_t M) { return M <= 16 ? 1 : M <= 32 ? 2 : 4; }
+static constexpr int kFewRowMaxRows = 128;
+static inline int fewrow_row_blocks(int64_t M) { return M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8; }
 
 // N: rows of the weight.  `paired`: the epilogue combines two columns of a tile (gate and value, or the two members of
 // a rotation pair), which only the second kernel does.
@@ -83,7 +84,7 @@ static FewRowPlan fewrow_plan(int64_t M, int64_t N, int64_t K, bool paired) {
     p.grid = (int)((total + run - 1) / run);
     p.direct = !paired && p.run == p.nch;
     p.partial_bytes = p.direct ? 0 : (int64_t)(p.grid + p.tiles) * kFewRowTile * 16 * fewrow_row_blocks(M) * 4;
-    p.sq_bytes = p.direct ? 0 : (int64_t)p.grid * 64 * 4;
+    p.sq_bytes = p.direct ? 0 : (int64_t)p.grid * kFewRowMaxRows * 4;
     return p;
 }
 
@@ -135,7 +136,8 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
     constexpr int CHUNK_BYTES = MP * 128;       // one staged chunk of x
     constexpr int XP = GC * MP * 8 / THREADS;   // 16-byte pieces of a group of x per thread
     static_assert(GC * MP * 8 % THREADS == 0 && XP >= 1, "every thread stages the same number of pieces");
-    static_assert(2 * GC * CHUNK_BYTES >= THREADS * 4, "the stages double as the buffer of the row sums");
+    constexpr int RPT = MP * 8 > THREADS ? MP * 8 / THREADS : 1;   // rows of x a thread stages pieces of
+    static_assert(2 * GC * CHUNK_BYTES >= RPT * THREADS * 4, "the stages double as the buffer of the row sums");
     __shared__ __attribute__((aligned(16))) unsigned char xs[2][GC * CHUNK_BYTES];
     __shared__ float rstd_s[MP];
 
@@ -173,7 +175,8 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
     };
 
     // ---- x: piece i of a thread is 16-byte piece (q & 7) of row (q >> 3) % MP of the group's unit q / (8 MP),
-    // q = tid + THREADS i — the same row for every i.  Rows beyond M repeat the last row; units past the end of the
+    // q = tid + THREADS i — row slot i % RPT of the thread (one row, or two with 128 rows of x).  Rows beyond M repeat
+    // the last row; units past the end of the
     // run repeat its last unit.  RMS: the norm's weight travels with x, a piece is multiplied by it (one rounding to
     // 16 bits, as in the reference) on its way into LDS, and the thread adds up the squares of the unscaled values of
     // the units that count: those of tile 0, whose runs cover every chunk of K exactly once (with whole tiles per
@@ -181,7 +184,9 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
     vec8 xr[XP], gr[RMS ? XP : 1];
     const T *xrow[XP];
     int xunit[XP], xdst[XP];
-    float sq = 0.0f;
+    float sq[RPT];
+#pragma unroll
+    for (int t = 0; t < RPT; ++t) sq[t] = 0.0f;
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
         const int q = tid + THREADS * i, j = q / (MP * 8), row = (q >> 3) % MP, piece = q & 7;
@@ -216,7 +221,7 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         const float xv = to_float(xr[i][e]);
-                        sq = fmaf(xv, xv, sq);
+                        sq[i % RPT] = fmaf(xv, xv, sq[i % RPT]);
                     }
                 }
                 xr[i] = xr[i] * gr[i];
@@ -302,19 +307,20 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
     }
 
     if constexpr (RMS) {
-        // a row's squares are spread over the threads (row + MP k) * 8 + p, p = 0..7
+        // a row's squares are spread over the pieces q = (row + MP k) * 8 + p, p = 0..7 (q = tid + THREADS slot)
         __syncthreads();                        // every wave is done with the stages
         float *sqbuf = reinterpret_cast<float *>(&xs[0][0]);
-        sqbuf[tid] = sq;
+#pragma unroll
+        for (int t = 0; t < RPT; ++t) sqbuf[t * THREADS + tid] = sq[t];
         __syncthreads();
         if (tid < MP) {
             float t = 0.0f;
 #pragma unroll
-            for (int k = 0; k < THREADS / (8 * MP); ++k)
+            for (int k = 0; k < RPT * THREADS / (8 * MP); ++k)
 #pragma unroll
                 for (int pp = 0; pp < 8; ++pp) t += sqbuf[(tid + MP * k) * 8 + pp];
             if (direct) rstd_s[tid] = 1.0f / sqrtf(t / (float)K + a.eps);
-            else if (u_begin < nch) a.sqpart[(int64_t)blockIdx.x * 64 + tid] = t;
+            else if (u_begin < nch) a.sqpart[(int64_t)blockIdx.x * kFewRowMaxRows + tid] = t;
         }
         if (direct) __syncthreads();
     }
@@ -378,7 +384,7 @@ __global__ void __launch_bounds__(256) linear_fewrow_reduce_kernel(const FewRowA
     if (a.rms_w != nullptr) {
         float t = 0.0f;
         const int w_sq_last = (nch - 1) / run;
-        for (int w = 0; w <= w_sq_last; ++w) t += a.sqpart[(int64_t)w * 64 + m];
+        for (int w = 0; w <= w_sq_last; ++w) t += a.sqpart[(int64_t)w * kFewRowMaxRows + m];
         rstd = 1.0f / sqrtf(t / (float)a.K + a.eps);
     }
     if (MODE == kFewRowPlain) {
@@ -452,7 +458,8 @@ static void launch_fewrow(FewRowArgs a, const FewRowPlan &p, int mode, hipStream
     } while (0)
     if (mb == 1) KERNL_FEWROW(1);
     else if (mb == 2) KERNL_FEWROW(2);
-    else KERNL_FEWROW(4);
+    else if (mb == 4) KERNL_FEWROW(4);
+    else KERNL_FEWROW(8);
 #undef KERNL_FEWROW
 #undef KERNL_FEWROW_REDUCE
 #undef KERNL_FEWROW_MAIN
@@ -462,7 +469,7 @@ static void launch_fewrow(FewRowArgs a, const FewRowPlan &p, int mode, hipStream
 
 extern "C" int64_t kernl_linear_fewrow_workspace_bytes(int64_t M, int64_t N, int64_t K, int gated, int rotated) {
     using namespace kernl;
-    if (M <= 0 || M > 64 || N <= 0 || K < 256 || K % 64 != 0) return 0;
+    if (M <= 0 || M > kFewRowMaxRows || N <= 0 || K < 256 || K % 64 != 0) return 0;
     const FewRowPlan p = fewrow_plan(M, gated ? 2 * N : N, K, gated || rotated);
     return p.partial_bytes + p.sq_bytes;
 }
@@ -486,8 +493,8 @@ extern "C" int kernl_linear_fewrow_fwd(const void *x, const void *rms_weight, fl
         return set_error(KERNL_ERR_INVALID_ARG, "few-row linear: unknown activation %d", activation);
     if (dtype != KERNL_F16 && dtype != KERNL_BF16)
         return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: only f16 and bf16 are supported, got dtype %d", dtype);
-    if (M > 64 || K % 64 != 0 || K < 256 || N > (1 << 29) || K > INT32_MAX)
-        return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: at most 64 rows of x and K a multiple of 64, at least 256 "
+    if (M > kFewRowMaxRows || K % 64 != 0 || K < 256 || N > (1 << 29) || K > INT32_MAX)
+        return set_error(KERNL_ERR_UNSUPPORTED, "few-row linear: at most 128 rows of x and K a multiple of 64, at least 256 "
                          "(M=%lld K=%lld)", (long long)M, (long long)K);
     if (x_strides[1] != 1 || x_strides[0] % 8 != 0 || !aligned16(x) || !aligned16(w) ||
         (rms_weight != nullptr && !aligned16(rms_weight)))

@@ -26,15 +26,17 @@ ONE_BYTE_WEIGHT_DTYPES = (torch.int8, torch.uint8, torch.float8_e5m2)
 
 
 FEW_ROW_MIN_ROWS = 17          # up to 16 rows the kernel that gives a workgroup 16 columns and all of K is as fast or faster
+FEW_ROW_MAX_ROWS = 128         # what `kernl_linear_fewrow_fwd` takes
 FEW_ROW_MIN_WEIGHT = 1 << 22   # elements: below that (2048 x 2048) launch latency decides and one launch beats two
 
 
 def takes_few_row_kernel(x2d: torch.Tensor, weight: torch.Tensor) -> bool:
-    """17 to 64 rows against a large 16-bit weight run the stream-K kernel (`kernl_linear_fewrow_fwd`): measured against
+    """17 to 128 rows against a large 16-bit weight run the stream-K kernel (`kernl_linear_fewrow_fwd`): measured against
     the weight-streaming kernel of `kernl_linear_fwd` at 32 / 64 rows, 5120 x 5120: 18 / 21 us against 34 / 35;
-    4096 x 11008: 25 / 30 against 35 / 53; 12288 x 4096: 27 / 32 against 28 / 37."""
+    4096 x 11008: 25 / 30 against 35 / 53; 12288 x 4096: 27 / 32 against 28 / 37 — and against its tile kernels at 128
+    rows: 28 against 63, 38 against 130, 39 against 52."""
     return (
-        FEW_ROW_MIN_ROWS <= x2d.shape[0] <= 64
+        FEW_ROW_MIN_ROWS <= x2d.shape[0] <= FEW_ROW_MAX_ROWS
         and weight.shape[0] * weight.shape[1] >= FEW_ROW_MIN_WEIGHT
         and _lib.linear_fewrow_supported(x2d, weight)
     )
@@ -175,13 +177,14 @@ def rms_linear_layer(
     n_out = weight.shape[0] // 2 if gated else weight.shape[0]
     if x.dtype == torch.float16:
         eps = max(eps, 1.6e-5)  # the fp16 policy of the RMSNorm operator (reference: layer_norm.py:295-296)
+    if takes_few_row_kernel(x_, weight) and (not gated or n_out % GLU_BLOCK == 0):
+        out = torch.empty((x_.shape[0], n_out), device=x.device, dtype=x.dtype)
+        _lib.linear_fewrow_fwd(x_, weight, bias, None, out, ACTIVATIONS.get(activation, _lib.ACT_NONE),
+                               rms_weight=rms_weight, eps=eps, gated=gated)
+        return out if x.ndim == 2 else out.reshape(*x.shape[:-1], n_out)
     if _lib.linear_rms_supported(x_) and (not gated or n_out % GLU_BLOCK == 0):
         out = torch.empty((x_.shape[0], n_out), device=x.device, dtype=x.dtype)
-        if takes_few_row_kernel(x_, weight):
-            _lib.linear_fewrow_fwd(x_, weight, bias, None, out, ACTIVATIONS.get(activation, _lib.ACT_NONE),
-                                   rms_weight=rms_weight, eps=eps, gated=gated)
-        else:
-            _lib.linear_rms_fwd(x_, rms_weight, eps, weight, bias, out, ACTIVATIONS.get(activation, _lib.ACT_NONE), gated)
+        _lib.linear_rms_fwd(x_, rms_weight, eps, weight, bias, out, ACTIVATIONS.get(activation, _lib.ACT_NONE), gated)
         return out if x.ndim == 2 else out.reshape(*x.shape[:-1], n_out)
     normed = layer_norm(x, rms_weight, None, eps, use_rms_norm=True)
     if gated:
@@ -189,12 +192,20 @@ def rms_linear_layer(
     return linear_layer(normed, weight, bias, activation)
 
 
-def decode_linear_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether `decode_linear_layer` takes this input: at most 64 rows in all, 16-bit, K a multiple of 64."""
+def decode_linear_supported(x: torch.Tensor, weight: torch.Tensor, head_dim: Optional[int] = None) -> bool:
+    """Whether `decode_linear_layer` takes this input: 16-bit, K a multiple of 64, at most 64 rows in all — or up to 128
+    against a weight large enough for the stream-K kernel (whose rotation wants a head size of 32, 64 or 128)."""
     if x.dtype not in (torch.float16, torch.bfloat16) or weight.dtype != x.dtype or x.shape[-1] % 64 != 0:
         return False
     rows = x.numel() // x.shape[-1]
-    return 0 < rows <= 64 and weight.is_contiguous() and weight.data_ptr() % 16 == 0
+    if not (weight.is_contiguous() and weight.data_ptr() % 16 == 0):
+        return False
+    if 0 < rows <= 64:
+        return True
+    return (
+        rows <= FEW_ROW_MAX_ROWS and weight.shape[0] * weight.shape[1] >= FEW_ROW_MIN_WEIGHT and x.shape[-1] >= 256
+        and (head_dim is None or head_dim in (32, 64, 128))
+    )
 
 
 def decode_linear_layer(
@@ -215,11 +226,12 @@ def decode_linear_layer(
         y[..., :rope_cols] rotated head by head (half-split rotary embedding) when cos / sin are given
         out = y + residual when a residual is given
 
-    x [batch, positions, K] or [rows, K], at most 64 rows in all; cos / sin [batch | 1, positions, head_dim] (a 2-D x
+    x [batch, positions, K] or [rows, K], at most 64 rows in all (128 against large weights); cos / sin [batch | 1, positions, head_dim] (a 2-D x
     counts as one batch entry); residual of the output's shape.  Reference: `rms_matmul_rbe_qkv_wrapper`,
     experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:289-344 (RMSNorm prologue + query/key/value projection +
     rotation of the query and key columns in one kernel)."""
-    assert decode_linear_supported(x, weight), "decode_linear_layer: at most 64 rows of 16-bit x, K a multiple of 64"
+    assert decode_linear_supported(x, weight, head_dim if cos is not None else None), \
+        "decode_linear_layer: at most 64 rows of 16-bit x (128 against a large weight), K a multiple of 64"
     assert (cos is None) == (sin is None)
     K, N = x.shape[-1], weight.shape[0]
     x_ = x if x.ndim == 2 else x.reshape(-1, K)

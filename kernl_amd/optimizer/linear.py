@@ -538,7 +538,7 @@ def rms_fused_linear_rope_wrapper(x: torch.Tensor, rms_weight, eps: float, weigh
     fast = (
         x.dim() == 3
         and _rms_fusable(x, rms_weight)
-        and decode_linear_supported(x, weight)
+        and decode_linear_supported(x, weight, head_dim)
         and (bias is None or bias.dtype == x.dtype)
         and cos.dim() == 4 and cos.shape == sin.shape and cos.dtype == sin.dtype and cos.shape[1] == 1
         and cos.shape[2] == x.shape[1] and cos.shape[3] == head_dim and cos.shape[0] in (1, x.shape[0])

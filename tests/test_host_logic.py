@@ -638,13 +638,13 @@ def test_residual_additions_fold_into_the_projection_before_them():
 
 
 def test_few_row_kernel_routing_rule():
-    """17 to 64 rows against a weight of at least 2048 x 2048 elements go to the stream-K kernel; fewer rows, small
+    """17 to 128 rows against a weight of at least 2048 x 2048 elements go to the stream-K kernel; fewer rows, small
     weights, a K that is no multiple of 64 and rows that are not 16-byte aligned do not."""
     from kernl_amd.implementations.linear_layer import takes_few_row_kernel
 
     w = torch.zeros((2048, 2048), dtype=torch.float16)
     rows = lambda m, k=2048: torch.zeros((m, k), dtype=torch.float16)
-    assert [takes_few_row_kernel(rows(m), w) for m in (1, 16, 17, 64, 65)] == [False, False, True, True, False]
+    assert [takes_few_row_kernel(rows(m), w) for m in (1, 16, 17, 64, 128, 129)] == [False, False, True, True, True, False]
     assert not takes_few_row_kernel(rows(32, 1024), torch.zeros((2048, 1024), dtype=torch.float16))      # small weight
     assert not takes_few_row_kernel(rows(32, 4104), torch.zeros((2048, 4104), dtype=torch.float16))      # K % 64 != 0
     assert not takes_few_row_kernel(torch.zeros((32, 2052), dtype=torch.float16)[:, :2048], w)           # row stride

@@ -395,6 +395,9 @@ FEW_ROW_SHAPES = [
     (30, 26300, 256),    # 206 tiles: whole tiles per workgroup, the last one ragged
     (64, 40000, 256),    # more tiles than workgroups: runs of 5 units against 4 chunks per tile
     (18, 80000, 256),    # runs of 10 units: a workgroup finishes a tile, covers one whole and starts a third
+    (128, 1000, 320),    # eight 16-row blocks of x
+    (100, 5120, 1024),
+    (70, 26300, 256),    # whole tiles per workgroup with 128 rows of x
 ]
 
 
@@ -427,7 +430,8 @@ def test_linear_few_rows_stream_k(shape, dtype, close):
     "case",
     # batch, positions, K, heads (query + key + value), head size, rotated heads, bias, residual
     [(5, 4, 320, 6, 128, 4, True, True), (33, 1, 256, 10, 64, 10, False, False), (2, 32, 704, 12, 32, 8, True, True),
-     (40, 1, 4096, 96, 128, 64, False, False), (16, 1, 512, 4, 128, 2, False, True), (3, 7, 1024, 7, 64, 0, True, False)],
+     (40, 1, 4096, 96, 128, 64, False, False), (16, 1, 512, 4, 128, 2, False, True), (3, 7, 1024, 7, 64, 0, True, False),
+     (64, 2, 512, 6, 128, 4, True, True), (97, 1, 256, 10, 64, 6, False, True)],
     ids=lambda c: "x".join(str(int(v)) for v in c),
 )
 def test_few_rows_stream_k_with_norm_rotation_and_residual(case, dtype, close):
@@ -465,7 +469,8 @@ def test_few_rows_stream_k_with_norm_rotation_and_residual(case, dtype, close):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
 @pytest.mark.parametrize("with_norm", [False, True], ids=["plain", "rms"])
-@pytest.mark.parametrize("shape", [(20, 352, 320), (33, 96, 256), (64, 11008, 4096), (10, 14336, 256), (48, 1000, 512)],
+@pytest.mark.parametrize("shape", [(20, 352, 320), (33, 96, 256), (64, 11008, 4096), (10, 14336, 256), (48, 1000, 512),
+                                   (100, 352, 320), (128, 14336, 256)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_few_rows_stream_k_gated_and_normalised(shape, with_norm, dtype, close):
     """The gated linear unit on interleaved weights (the second launch multiplies act(gate) by the value two waves
@@ -499,7 +504,7 @@ def test_few_rows_stream_k_gated_and_normalised(shape, with_norm, dtype, close):
 
 
 def test_linear_few_rows_stream_k_is_what_the_operators_run(close, monkeypatch):
-    """17 to 64 rows against a large weight: `linear_layer` and the residual form of `decode_linear_layer` take the
+    """17 to 128 rows against a large weight: `linear_layer` and the residual form of `decode_linear_layer` take the
     stream-K kernel; fewer rows, small weights and a saved pre-activation keep the other kernels.  Strided rows of x
     and a 3-D input go through unchanged."""
     from kernl_amd.implementations.linear_layer import decode_linear_layer
@@ -511,7 +516,7 @@ def test_linear_few_rows_stream_k_is_what_the_operators_run(close, monkeypatch):
     N, K = 2304, 2048
     w = (torch.randn((N, K), generator=gen) * K ** -0.5).half()
     b = torch.randn((N,), generator=gen).half()
-    for rows, expected in ((16, 0), (17, 1), (64, 1), (65, 0)):
+    for rows, expected in ((16, 0), (17, 1), (64, 1), (65, 1), (128, 1), (129, 0)):
         calls.clear()
         x = torch.randn((rows, K), generator=gen).half()
         out = linear_layer(x.cuda(), w.cuda(), b.cuda(), "relu")
