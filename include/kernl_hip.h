@@ -237,6 +237,25 @@ int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float eps, const
                          int activation, int gated, int dtype, void *stream);
 
 /*
+ * kernl_linear_fwd for row counts between the two regimes (129 to a few hundred rows against a few thousand columns),
+ * where the 128-row tiles of the tiled kernels are too few to occupy the chip: every output tile is computed by up to
+ * four workgroups over disjoint ranges of K, and a second small launch adds their fp32 partial tiles in range order and
+ * runs the epilogue (same semantics and arguments as kernl_linear_fwd, reference src/kernl/implementations/
+ * linear_layer.py:92-210; the split over K is the `SPLIT_K` axis of the reference's configurations, which it leaves
+ * at 1, linear_layer.py:47-67).
+ *   kernl_linear_splitk_workspace_bytes(M, N, K) returns 0 when splitting does not pay (enough tiles, or a short K):
+ *   call kernl_linear_fwd then.  Otherwise pass a 16-byte aligned workspace of at least that many bytes (contents
+ *   irrelevant before and after the call; calls that overlap in time need workspaces of their own).
+ *   f16 / bf16, K % 64 == 0, x with unit feature stride and 16-byte aligned rows; anything else returns
+ *   KERNL_ERR_UNSUPPORTED.
+ */
+int64_t kernl_linear_splitk_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int kernl_linear_splitk_fwd(const void *x, const void *w, const void *bias, void *out, void *act_in, void *workspace,
+                            int64_t workspace_bytes, int64_t M, int64_t N, int64_t K, const int64_t x_strides[2],
+                            const int64_t out_strides[2], const int64_t act_in_strides[2], int activation, int dtype,
+                            void *stream);
+
+/*
  * The linear layer for a FEW rows of x with many columns and a long K (batched decoding steps: 17 to 128 rows, where
  * kernl_linear_fwd's weight-streaming kernel re-reads x once per 16 to 64 output columns and its tile kernels leave
  * most of their rows empty), with everything a decoder layer puts around its projections:

@@ -34,6 +34,8 @@ EXPORTED_SYMBOLS = (
     "kernl_linear_w8_fwd",
     "kernl_linear_rms_fwd",
     "kernl_linear_decode_fwd",
+    "kernl_linear_splitk_workspace_bytes",
+    "kernl_linear_splitk_fwd",
     "kernl_linear_fewrow_workspace_bytes",
     "kernl_linear_fewrow_fwd",
     "kernl_linear_glu_fwd",
@@ -111,6 +113,10 @@ def load() -> ctypes.CDLL:
         [_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp] + [_i64] * 3 + [_i64p] * 3 + [_vp, _vp] + [_i64] * 3
         + [_i64p, ctypes.c_int, ctypes.c_int, _vp]
     )
+    lib.kernl_linear_splitk_workspace_bytes.restype = _i64
+    lib.kernl_linear_splitk_workspace_bytes.argtypes = [_i64] * 3
+    lib.kernl_linear_splitk_fwd.restype = ctypes.c_int
+    lib.kernl_linear_splitk_fwd.argtypes = [_vp] * 6 + [_i64] * 4 + [_i64p] * 3 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_linear_fewrow_workspace_bytes.restype = _i64
     lib.kernl_linear_fewrow_workspace_bytes.argtypes = [_i64] * 3 + [ctypes.c_int] * 2
     lib.kernl_linear_fewrow_fwd.restype = ctypes.c_int
@@ -382,6 +388,34 @@ def linear_decode_fwd(x2d, rms_weight, eps: float, weight, bias, residual2d, out
             int(rows_per_batch), tstrides, tdtype, DTYPE_CODE[x2d.dtype], _stream(x2d),
         )
     _check(st, "kernl_linear_decode_fwd")
+
+
+def linear_splitk_workspace_bytes(x2d, weight) -> int:
+    """Bytes of workspace `linear_splitk_fwd` wants for this product; 0: splitting K does not pay (or the input is not
+    what the kernel takes) and `linear_fwd` is the call to make."""
+    M, K = x2d.shape
+    if not (
+        x2d.dtype in (torch.float16, torch.bfloat16) and weight.dtype == x2d.dtype and K % 64 == 0 and K < (1 << 22)
+        and x2d.stride(1) == 1 and x2d.stride(0) % 8 == 0 and x2d.stride(0) < (1 << 22) and x2d.data_ptr() % 16 == 0
+        and weight.is_contiguous() and weight.data_ptr() % 16 == 0
+    ):
+        return 0
+    return int(load().kernl_linear_splitk_workspace_bytes(M, weight.shape[0], K))
+
+
+def linear_splitk_fwd(x2d, weight, bias, out2d, act_in2d, activation: int, workspace) -> None:
+    _require_gpu(x2d, weight, bias, out2d, act_in2d, workspace)
+    M, K = x2d.shape
+    N = out2d.shape[1]
+    lib = load()
+    with torch.cuda.device(x2d.device):
+        st = lib.kernl_linear_splitk_fwd(
+            x2d.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(), out2d.data_ptr(),
+            None if act_in2d is None else act_in2d.data_ptr(), workspace.data_ptr(),
+            workspace.numel() * workspace.element_size(), M, N, K, _arr(x2d.stride()), _arr(out2d.stride()),
+            None if act_in2d is None else _arr(act_in2d.stride()), int(activation), DTYPE_CODE[x2d.dtype], _stream(x2d),
+        )
+    _check(st, "kernl_linear_splitk_fwd")
 
 
 def linear_fewrow_supported(x2d, weight) -> bool:

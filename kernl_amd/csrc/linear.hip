@@ -761,12 +761,27 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 // 16 KB (x) + 32 KB (w), k-tile T + 3 requested while k-tile T is multiplied, the wait in front of the second k-step
 // only for k-tile T + 1 (vmcnt(NL): the loads of T + 2 may still be in flight).  One workgroup per output tile.
 // ----------------------------------------------------------------------------------------------------
-template <typename T, int ACT, int NBN, bool W8 = false>
+// Tile t of the half-height kernels' grouped order (GROUP_M row tiles side by side) -> origin of the tile.
+__device__ __forceinline__ void half_tile_origin(int t, int tiles_m, int tiles_n, int BM, int BN, int &m0, int &n0) {
+    constexpr int GROUP_M = 8;
+    const int group_span = GROUP_M * tiles_n;
+    const int group = t / group_span;
+    const int first_m = group * GROUP_M;
+    const int gsize = min(tiles_m - first_m, GROUP_M);
+    const int in_group = t - group * group_span;
+    m0 = (first_m + in_group % gsize) * BM;
+    n0 = (in_group / gsize) * BN;
+}
+
+// SPLIT: blockIdx.y selects one of `splits` ranges of k-tiles; the workgroup leaves its fp32 partial tile in `part`
+// (slot blockIdx.y * tiles + t; per wave and 16 x 16 block 64 lanes x 16 bytes: coalesced, and the same lane reads it
+// back in linear_wide_half_reduce_kernel, which adds the ranges in order and runs the epilogue).
+template <typename T, int ACT, int NBN, bool W8 = false, bool SPLIT = false>
 __global__ void __launch_bounds__(256, 1)
 linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
                         T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs,
                         int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok,
-                        int ai_vec_ok, int bias_vec_ok) {
+                        int ai_vec_ok, int bias_vec_ok, float *__restrict__ part, int splits) {
     typedef typename Vec8<T>::type vec8;
     static_assert((ACT & kGluBit) == 0 && (NBN == 8 || NBN == 6), "plain epilogues, 256 or 192 columns");
     constexpr int NBM = 4, BM = 32 * NBM, BN = 32 * NBN, BK = 64, RB = BK * 2, CPR = BK / 8, KSTEPS = BK / 32;
@@ -776,19 +791,14 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     constexpr int WB = W8 ? 1 : 2, RBW = BK * WB, CPRW = RBW / 16;  // weight tile: bytes per element, row bytes, chunks per row
     constexpr int LOADS_X = BM * CPR / 256, LOADS_W = BN * CPRW / 256, NL = LOADS_X + LOADS_W;
     static_assert(LOADS_X == 4, "one group of four loads for the x tile");
-    constexpr int GROUP_M = 8;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) >> 3;
     const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
     if ((int)(blockIdx.x >> 3) >= per_xcd || t >= total) return;
-    const int group_span = GROUP_M * tiles_n;
-    const int group = t / group_span;
-    const int first_m = group * GROUP_M;
-    const int gsize = min(tiles_m - first_m, GROUP_M);
-    const int in_group = t - group * group_span;
-    const int m0 = (first_m + in_group % gsize) * BM, n0 = (in_group / gsize) * BN;
+    int m0, n0;
+    half_tile_origin(t, tiles_m, tiles_n, BM, BN, m0, n0);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -857,11 +867,16 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
 
     // Every k-tile slot issues its NL loads, so that the counter waits stay exact up to the end; requests past the
     // last k-tile fetch that tile again (into a stage nobody reads any more) instead of running past the row ends.
-    const int nk = K / BK;
+    int nk = K / BK, kb = 0;   // k-tiles of this workgroup: kb .. kb + nk - 1
+    if constexpr (SPLIT) {
+        const int per_split = (nk + splits - 1) / splits;
+        kb = (int)blockIdx.y * per_split;
+        nk = min(per_split, nk - kb);   // the host keeps every range non-empty
+    }
 #pragma unroll
     for (int s3 = 0; s3 < 3; ++s3)
 #pragma unroll
-        for (int l = 0; l < NL; ++l) tile_load(l, s3, min(s3, nk - 1) * BK);
+        for (int l = 0; l < NL; ++l) tile_load(l, s3, (kb + min(s3, nk - 1)) * BK);
     __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * NL) & 15) | (((2 * NL) >> 4) << 14));  // vmcnt(2 NL): k-tile 0 has landed
     __syncthreads();
 
@@ -903,7 +918,7 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     };
     auto k_tile = [&](auto cur_c, int kt) __attribute__((always_inline)) {
         constexpr int CUR = decltype(cur_c)::value, NXT = (CUR + 1) % 3;
-        const int k_next = min(kt + 3, nk - 1) * BK;
+        const int k_next = (kb + min(kt + 3, nk - 1)) * BK;
 #pragma unroll
         for (int st = 0; st < KSTEPS; ++st) {
             const int sn = st ^ 1;
@@ -951,6 +966,15 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     if (kt + 1 < nk) k_tile(IntC<1>(), kt + 1);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no load may still be writing LDS when the workgroup ends
 
+    if constexpr (SPLIT) {
+        float4 *dst = reinterpret_cast<float4 *>(part) + ((((int64_t)blockIdx.y * total + t) * 4 + wave) * (NBM * NBN)) * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < NBM; ++i)
+#pragma unroll
+            for (int j = 0; j < NBN; ++j)
+                dst[(i * NBN + j) * 64] = float4{acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+        return;
+    }
     const int n_wave = n0 + wave_n * (NBN * 16);
     constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB;
     u32x4 braw[NG][2];
@@ -967,6 +991,63 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     KERNL_HALF_EPILOGUE(2);
     KERNL_HALF_EPILOGUE(3);
 #undef KERNL_HALF_EPILOGUE
+}
+
+// Second launch of the split form: workgroup (t, I) adds the k ranges' partial sums of 16-row block I of every wave of
+// tile t, in range order, and runs the epilogue the unsplit kernel runs (same wave and lane geometry).
+template <typename T, int ACT, int NBN>
+__global__ void __launch_bounds__(256)
+linear_wide_half_reduce_kernel(const float *__restrict__ part, const T *__restrict__ bias, T *__restrict__ out,
+                               T *__restrict__ act_in, int M, int N, int64_t out_rs, int64_t out_cs, int64_t ai_rs,
+                               int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok, int ai_vec_ok, int bias_vec_ok,
+                               int splits) {
+    constexpr int NBM = 4, BM = 32 * NBM, BN = 32 * NBN;
+    const int t = (int)blockIdx.x, I = (int)blockIdx.y, total = tiles_m * tiles_n;
+    int m0, n0;
+    half_tile_origin(t, tiles_m, tiles_n, BM, BN, m0, n0);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave & 1, wave_n = wave >> 1;
+    const int l16 = lane & 15, g = lane >> 4;
+    f32x4_acc acc[NBM][NBN];
+#pragma unroll
+    for (int i = 0; i < NBM; ++i)
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+    const float4 *src = reinterpret_cast<const float4 *>(part) + (((int64_t)t * 4 + wave) * (NBM * NBN) + I * NBN) * 64 + lane;
+    const int64_t split_stride = (int64_t)total * 4 * (NBM * NBN) * 64;
+    for (int sp = 0; sp < splits; ++sp) {
+        float4 v[NBN];
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) v[j] = src[sp * split_stride + j * 64];
+#pragma unroll
+        for (int i = 0; i < NBM; ++i) {
+            if (i != I) continue;   // (the block index of the accumulators is a compile-time constant in the epilogue)
+#pragma unroll
+            for (int j = 0; j < NBN; ++j) {
+                acc[i][j][0] += v[j].x;
+                acc[i][j][1] += v[j].y;
+                acc[i][j][2] += v[j].z;
+                acc[i][j][3] += v[j].w;
+            }
+        }
+    }
+    const int n_wave = n0 + wave_n * (NBN * 16);
+    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB;
+    u32x4 braw[NG][2];
+#pragma unroll
+    for (int G = 0; G < NG; ++G)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0} : fetch8<T>(bias, n_wave + 16 * JB * G + 4 * JB * g + 8 * h, N, bias_vec_ok);
+#define KERNL_HALF_REDUCE_EPILOGUE(IB)                                                                                   \
+    if (I == IB)                                                                                                         \
+    wide_epilogue<T, ACT, IB, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, \
+                                        ai_rs, ai_cs, out_vec_ok, ai_vec_ok, braw)
+    KERNL_HALF_REDUCE_EPILOGUE(0);
+    KERNL_HALF_REDUCE_EPILOGUE(1);
+    KERNL_HALF_REDUCE_EPILOGUE(2);
+    KERNL_HALF_REDUCE_EPILOGUE(3);
+#undef KERNL_HALF_REDUCE_EPILOGUE
 }
 
 // ----------------------------------------------------------------------------------------------------
@@ -1430,7 +1511,67 @@ static void launch_wide_half_act(const LinearArgs &a) {
     const int bias_vec_ok = bias != nullptr && aligned16(bias);
     hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
-                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok);
+                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, static_cast<float *>(nullptr), 1);
+}
+
+// Split form of the 128 x 192 kernel for row counts that leave most CUs without a tile (129 to about 700 rows against
+// a few thousand columns): `splits` ranges of k-tiles per output tile, then the launch that adds them.
+struct HalfSplitPlan {
+    int tiles_m, tiles_n, splits;
+    int64_t bytes;
+};
+static HalfSplitPlan half_split_plan(int64_t M, int64_t N, int64_t K) {
+    HalfSplitPlan p;
+    p.tiles_m = (int)((M + 127) / 128);
+    p.tiles_n = (int)((N + 191) / 192);
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    const int nk = (int)(K / 64);
+    int64_t splits = 256 / tiles;           // one round of workgroups
+    if (splits > nk / 16) splits = nk / 16; // ranges of at least 16 k-tiles: with K = 768 two ranges cost more (14 us) than one tile pass (11)
+    if (splits > 4) splits = 4;             // partial tiles cost HBM traffic: rows x columns x 8 bytes per range
+    if (splits < 1) splits = 1;
+    // ranges of ceil(nk / splits) k-tiles: drop ranges that would be empty
+    const int per = (nk + (int)splits - 1) / (int)splits;
+    p.splits = (nk + per - 1) / per;
+    p.bytes = p.splits > 1 ? (int64_t)p.splits * tiles * 128 * 192 * 4 : 0;
+    return p;
+}
+
+template <typename T, int ACT>
+static void launch_half_split_act(const LinearArgs &a, const HalfSplitPlan &p, float *part) {
+    constexpr int NBN = 6;
+    auto kern = linear_wide_half_kernel<T, KERNL_ACT_NONE, NBN, false, true>;
+    constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768;
+    static bool attr_done = false;  // benign race: the attribute call is idempotent
+    if (!attr_done) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        attr_done = true;
+    }
+    const int per_xcd = (p.tiles_m * p.tiles_n + 7) / 8;
+    const T *bias = static_cast<const T *>(a.bias);
+    T *out = static_cast<T *>(a.out);
+    T *act_in = static_cast<T *>(a.act_in);
+    const int out_vec_ok = a.out_cs == 1 && a.out_rs % 8 == 0 && aligned16(out);
+    const int ai_vec_ok = act_in != nullptr && a.ai_cs == 1 && a.ai_rs % 8 == 0 && aligned16(act_in);
+    const int bias_vec_ok = bias != nullptr && aligned16(bias);
+    hipLaunchKernelGGL(kern, dim3(per_xcd * 8, p.splits), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
+                       static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
+                       a.ai_cs, p.tiles_m, p.tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, part, p.splits);
+    hipLaunchKernelGGL((linear_wide_half_reduce_kernel<T, ACT, NBN>), dim3(p.tiles_m * p.tiles_n, 4), dim3(256), 0, a.st,
+                       part, bias, out, act_in, a.M, a.N, a.out_rs, a.out_cs, a.ai_rs, a.ai_cs, p.tiles_m, p.tiles_n,
+                       out_vec_ok, ai_vec_ok, bias_vec_ok, p.splits);
+}
+
+template <typename T>
+static void launch_half_split(const LinearArgs &a, const HalfSplitPlan &p, float *part) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_half_split_act<T, KERNL_ACT_RELU>(a, p, part); break;
+        case KERNL_ACT_TANH: launch_half_split_act<T, KERNL_ACT_TANH>(a, p, part); break;
+        case KERNL_ACT_GELU_ERF: launch_half_split_act<T, KERNL_ACT_GELU_ERF>(a, p, part); break;
+        case KERNL_ACT_GELU_TANH: launch_half_split_act<T, KERNL_ACT_GELU_TANH>(a, p, part); break;
+        case KERNL_ACT_SILU: launch_half_split_act<T, KERNL_ACT_SILU>(a, p, part); break;
+        default: launch_half_split_act<T, KERNL_ACT_NONE>(a, p, part); break;
+    }
 }
 
 template <typename T, int NBN>
@@ -1712,6 +1853,53 @@ extern "C" int kernl_linear_fwd(const void *x, const void *w, const void *bias, 
         return linear_fma_dispatch<float>(a);
     }
     return set_error(KERNL_ERR_UNSUPPORTED, "linear: unknown dtype %d", dtype);
+}
+
+extern "C" int64_t kernl_linear_splitk_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    using namespace kernl;
+    if (M <= 0 || N <= 0 || K <= 0 || K % 64 != 0 || M > INT32_MAX || N > INT32_MAX || K >= (1 << 22)) return 0;
+    return half_split_plan(M, N, K).bytes;
+}
+
+extern "C" int kernl_linear_splitk_fwd(const void *x, const void *w, const void *bias, void *out, void *act_in,
+                                       void *workspace, int64_t workspace_bytes, int64_t M, int64_t N, int64_t K,
+                                       const int64_t x_strides[2], const int64_t out_strides[2],
+                                       const int64_t act_in_strides[2], int activation, int dtype, void *stream) {
+    using namespace kernl;
+    if (x == nullptr || w == nullptr || out == nullptr || x_strides == nullptr || out_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear (split K): x, w, out and their strides must not be NULL");
+    if (act_in != nullptr && act_in_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear (split K): act_in given without strides");
+    if (M <= 0 || N <= 0 || K <= 0 || workspace_bytes < 0)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear (split K): bad sizes M=%lld N=%lld K=%lld", (long long)M,
+                         (long long)N, (long long)K);
+    if (activation < KERNL_ACT_NONE || activation > KERNL_ACT_SILU)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear (split K): unknown activation %d", activation);
+    if (dtype != KERNL_F16 && dtype != KERNL_BF16)
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear (split K): only f16 and bf16 are supported, got dtype %d", dtype);
+    if (M > INT32_MAX || N > INT32_MAX || K % 64 != 0 || K >= (1 << 22) || x_strides[0] >= (1 << 22) ||
+        x_strides[1] != 1 || x_strides[0] % 8 != 0 || !aligned16(x) || !aligned16(w))
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear (split K): K must be a multiple of 64, x needs unit feature stride "
+                         "and 16-byte aligned rows, the weight a 16-byte aligned base");
+    const HalfSplitPlan p = half_split_plan(M, N, K);
+    if (p.splits < 2)
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear (split K): nothing to split for M=%lld N=%lld K=%lld "
+                         "(kernl_linear_splitk_workspace_bytes returns 0): use kernl_linear_fwd", (long long)M, (long long)N,
+                         (long long)K);
+    if (workspace == nullptr || workspace_bytes < p.bytes || !aligned16(workspace))
+        return set_error(KERNL_ERR_INVALID_ARG, "linear (split K): the workspace must hold %lld bytes, 16-byte aligned",
+                         (long long)p.bytes);
+    LinearArgs a;
+    a.x = x; a.w = w; a.bias = bias; a.out = out; a.act_in = act_in;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.x_rs = x_strides[0]; a.x_cs = x_strides[1];
+    a.out_rs = out_strides[0]; a.out_cs = out_strides[1];
+    a.ai_rs = act_in ? act_in_strides[0] : 0; a.ai_cs = act_in ? act_in_strides[1] : 0;
+    a.act = activation;
+    a.st = static_cast<hipStream_t>(stream);
+    if (dtype == KERNL_F16) launch_half_split<f16>(a, p, static_cast<float *>(workspace));
+    else launch_half_split<bf16>(a, p, static_cast<float *>(workspace));
+    return check_launch("linear (split K)");
 }
 
 extern "C" int kernl_linear_glu_fwd(const void *x, const void *w, const void *bias, void *out, int64_t M, int64_t N,

@@ -27,6 +27,7 @@ ONE_BYTE_WEIGHT_DTYPES = (torch.int8, torch.uint8, torch.float8_e5m2)
 
 FEW_ROW_MIN_ROWS = 17          # up to 16 rows the kernel that gives a workgroup 16 columns and all of K is as fast or faster
 FEW_ROW_MAX_ROWS = 128         # what `kernl_linear_fewrow_fwd` takes
+SPLIT_K_MAX_ROWS = 2048        # beyond that the tiled kernels always have tiles enough; the library decides below it
 FEW_ROW_MIN_WEIGHT = 1 << 22   # elements: below that (2048 x 2048) launch latency decides and one launch beats two
 
 
@@ -85,8 +86,13 @@ class LinearLayer(torch.autograd.Function):
         outputs = torch.empty((M, N), device=x.device, dtype=x.dtype)
         if act_inputs is not None:
             assert act_inputs.shape == (M, N) and act_inputs.dtype == x.dtype
+        split_bytes = _lib.linear_splitk_workspace_bytes(x_, weight) if FEW_ROW_MAX_ROWS < M <= SPLIT_K_MAX_ROWS else 0
         if act_inputs is None and takes_few_row_kernel(x_, weight):
             _lib.linear_fewrow_fwd(x_, weight, bias, None, outputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
+        elif split_bytes:
+            # too few 128-row tiles to occupy the chip: ranges of K per tile, added by a second launch
+            workspace = torch.empty(split_bytes, dtype=torch.uint8, device=x.device)
+            _lib.linear_splitk_fwd(x_, weight, bias, outputs, act_inputs, ACTIVATIONS.get(activation, _lib.ACT_NONE), workspace)
         else:
             _lib.linear_fwd(x_, weight, bias, outputs, act_inputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
         return outputs if x.ndim == 2 else outputs.reshape(*x.shape[:-1], N)

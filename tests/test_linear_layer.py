@@ -383,6 +383,48 @@ def test_decode_projection_rejections():
         _lib.linear_decode_fwd(x[:4], None, 0.0, w, None, None, out, t64, t64, 64, 64, 4)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("activation", ["", "fast_gelu"])
+@pytest.mark.parametrize("shape", [(129, 768, 3072), (200, 1000, 2048), (256, 4096, 4096), (300, 4100, 2112), (640, 400, 2112)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_linear_split_over_k(shape, activation, dtype, close):
+    """Row counts whose 128-row tiles are too few for the chip: `linear_layer` hands them to `kernl_linear_splitk_fwd`
+    (ranges of K per tile, partial tiles added by a second launch).  Ragged last tiles in both directions, ranges of
+    unequal length (33 k-tiles in 2), the saved pre-activation, and a workspace full of NaNs."""
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(71)
+    x, w, b = _inputs(M, N, K, dtype, gen, w_std=K ** -0.5)
+    xd, wd, bd = x.cuda(), w.cuda(), b.cuda()
+    need = _lib.linear_splitk_workspace_bytes(xd, wd)
+    assert need > 0, "the shape list is meant for the split form"
+    ws = torch.full((need // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    out = torch.empty((M, N), dtype=dtype, device="cuda")
+    act_in = torch.empty((M, N), dtype=dtype, device="cuda")
+    _lib.linear_splitk_fwd(xd, wd, bd, out, act_in, _lib.ACT_GELU_TANH if activation else _lib.ACT_NONE, ws)
+    routed = linear_layer(xd, wd, None, activation)
+    torch.cuda.synchronize()
+    ref, pre = linear_oracle(x, w, b, activation, return_act_inputs=True)
+    close(out, ref, dtype, what=f"split K {shape} {activation!r}")
+    close(act_in, pre, dtype, what=f"split K {shape} pre-activation")
+    close(routed, linear_oracle(x, w, None, activation), dtype, what=f"split K {shape} through linear_layer")
+
+
+def test_linear_split_over_k_rule():
+    """The library splits only where it pays: few tiles and a long K."""
+    rows = lambda m, k: torch.empty((m, k), dtype=torch.float16, device="cuda")
+    weight = lambda n, k: torch.empty((n, k), dtype=torch.float16, device="cuda")
+    assert _lib.linear_splitk_workspace_bytes(rows(256, 4096), weight(4096, 4096)) > 0
+    assert _lib.linear_splitk_workspace_bytes(rows(256, 768), weight(3072, 768)) == 0      # short K
+    assert _lib.linear_splitk_workspace_bytes(rows(2048, 4096), weight(4096, 4096)) == 0   # tiles enough
+    assert _lib.linear_splitk_workspace_bytes(rows(256, 4104), weight(4096, 4104)) == 0    # K % 64 != 0
+    with pytest.raises(_lib.KernlLibraryError, match="nothing to split"):
+        _lib.linear_splitk_fwd(rows(2048, 4096), weight(4096, 4096), None, rows(2048, 4096), None, _lib.ACT_NONE,
+                               torch.empty(1024, dtype=torch.uint8, device="cuda"))
+    with pytest.raises(_lib.KernlLibraryError, match="workspace"):
+        _lib.linear_splitk_fwd(rows(256, 4096), weight(4096, 4096), None, rows(256, 4096), None, _lib.ACT_NONE,
+                               torch.empty(1024, dtype=torch.uint8, device="cuda"))
+
+
 FEW_ROW_SHAPES = [
     (33, 200, 256),      # two tiles, the second ragged; a run is exactly one tile: no partial sums
     (17, 1000, 320),     # five chunks per tile, runs of four: every run crosses into the next tile
