@@ -1,0 +1,1768 @@
+// Kernels and launchers of the fused linear layer, shared by linear.hip (dispatch, entry points, the 8-wave, skinny
+// and FMA kernels), linear_wide.hip and linear_wide_half.hip.
+#pragma once
+
+// Fused linear layer for gfx950:  out[M,N] = act(x[M,K] · w[N,K]ᵀ + bias[N]).
+//
+// Semantics follow the reference kernel src/kernl/implementations/linear_layer.py:92-210: fp32 accumulation,
+// bias added in fp32, optional store of the pre-activation, activation applied to the fp32 accumulator, one
+// rounding to the output dtype.
+//
+// MFMA path (16-bit inputs, K-contiguous x): both operands are K-major, which is exactly what
+// v_mfma_f32_32x32x16 wants (each lane supplies 8 consecutive k of one row), so tiles go HBM -> VGPR -> LDS
+// with 16-byte accesses and no transposition.  The weight rows feed the MFMA "A" side and the activations the
+// "B" side, i.e. the instruction produces a 32(n) x 32(m) block of outᵀ; together with the row permutation
+// rowperm16 on the weight tile this leaves every lane holding 16 consecutive output columns of one output
+// row, so bias loads and output stores are 16-byte vectors without any shuffle through LDS.
+#include <type_traits>
+
+#include "activations.h"
+#include "common.h"
+
+namespace kernl {
+
+// The wide kernels are heavy to compile (dozens of fully unrolled instantiations): their launchers live in translation
+// units of their own (linear_wide.hip, linear_wide_half.hip) behind these functions, so that a build runs them in parallel.
+// dtype: KERNL_F16 / KERNL_BF16; cols: 256 or 192 output columns per tile.
+struct LinearArgs;
+struct HalfSplitPlan;
+void run_wide(const LinearArgs &a, int dtype, int cols);             // 256-row tiles; the gated epilogue when a.act says so
+void run_wide_w8(const LinearArgs &a);                               // fp8 e5m2 weights, fp16 activations
+void run_wide_half(const LinearArgs &a, int dtype, int cols);        // 128-row tiles
+void run_wide_half_w8(const LinearArgs &a);
+void run_half_split(const LinearArgs &a, const HalfSplitPlan &p, float *part, int dtype);
+
+
+// ----------------------------------------------------------------------------------------------------
+// Epilogue shared by the MFMA kernels: lane (lr, lh) holds, for 32x32 block (i, j) of its wave's tile, output row
+// m_wave + 32 i + lr and the 16 consecutive columns starting at n_wave + 32 j + 16 lh.  Bias add, optional store of
+// the pre-activation, activation, one rounding to the output dtype, 16-byte stores where the layout allows.
+//
+// Gated form (ACT has kGluBit set): the weight rows alternate in blocks of 32 between the gate and the value
+// projection, so blocks (i, 2p) and (i, 2p + 1) of a lane hold the gate and the value of the SAME 16 output elements;
+// out[m, n] = act(gate + bias_gate) * (value + bias_value) with N counting the interleaved rows (twice the output
+// width).  The same product as the reference's fused feed-forward kernel forms from two accumulators
+// (experimental/llama-v2/kernel/fused_kernel_ff.py:36-75).
+// ----------------------------------------------------------------------------------------------------
+static constexpr int kGluBit = 8;
+
+// Bias of a wave's TN column blocks as packed 16-bit values: raw[j] holds the 16 consecutive entries starting at
+// n_wave + 32 j + 16 lh.  Fetched ONCE per tile and ahead of time: with one or two waves per SIMD a load issued where
+// its value is needed stalls the whole epilogue for a memory round trip.
+template <typename T, int TN>
+__device__ __forceinline__ void bias_fetch(const T *__restrict__ bias, int n_wave, int lh, int N, int bias_vec_ok,
+                                           u32x4 (&raw)[TN][2]) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int n = n_wave + j * 32 + lh * 16;
+        if (bias == nullptr) {
+            raw[j][0] = u32x4{0, 0, 0, 0};
+            raw[j][1] = u32x4{0, 0, 0, 0};
+        } else if (bias_vec_ok && n + 16 <= N) {
+            raw[j][0] = *reinterpret_cast<const u32x4 *>(bias + n);
+            raw[j][1] = *reinterpret_cast<const u32x4 *>(bias + n + 8);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; v += 2) {
+                const uint32_t lo = n + v < N ? (uint32_t)__builtin_bit_cast(uint16_t, bias[n + v]) : 0u;
+                const uint32_t hi = n + v + 1 < N ? (uint32_t)__builtin_bit_cast(uint16_t, bias[n + v + 1]) : 0u;
+                raw[j][v >> 3][(v & 7) >> 1] = lo | (hi << 16);
+            }
+        }
+    }
+}
+template <typename T>
+__device__ __forceinline__ float bias_elem(const u32x4 (&raw)[2], int v) {
+    const uint32_t word = raw[v >> 3][(v & 7) >> 1];
+    const uint16_t bits = (uint16_t)((v & 1) ? (word >> 16) : (word & 0xFFFFu));
+    return to_float(__builtin_bit_cast(T, bits));
+}
+
+// ROW0 / ROWS select the 32-row blocks handled by one call (the wide kernel calls once per block so that each call
+// unrolls completely).  Waves whose blocks lie inside the matrix and whose output rows take 16-byte stores run a
+// straight-line path; edge tiles, strided outputs and the pre-activation side output run the general one.
+template <typename T, int ACT, int TM, int TN, int ROW0 = 0, int ROWS = TM>
+__device__ __forceinline__ void linear_epilogue(f32x16 (&acc)[TM][TN], int m_wave, int n_wave, int lr, int lh,
+                                                const T *__restrict__ bias, T *__restrict__ out,
+                                                T *__restrict__ act_in, int M, int N, int64_t out_rs, int64_t out_cs,
+                                                int64_t ai_rs, int64_t ai_cs, int out_vec_ok, int ai_vec_ok,
+                                                int bias_vec_ok, const u32x4 (&braw)[TN][2]) {
+    auto store16 = [&](T *p, const float (&r)[16]) __attribute__((always_inline)) {
+        u32x4 p0, p1;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            p0[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
+            p1[v] = pack2<T>(r[8 + 2 * v], r[8 + 2 * v + 1]);
+        }
+        *reinterpret_cast<u32x4 *>(p) = p0;
+        *reinterpret_cast<u32x4 *>(p + 8) = p1;
+    };
+    const bool rows_inside = m_wave + (ROW0 + ROWS) * 32 <= M;
+    if constexpr ((ACT & kGluBit) != 0) {
+        static_assert(TN % 2 == 0, "gated epilogue pairs neighbouring 32-column blocks");
+        constexpr int BASE = ACT & (kGluBit - 1);
+        const int n_total = N >> 1;
+        const bool interior = rows_inside && (n_wave >> 1) + TN * 16 <= n_total && out_vec_ok;
+        if (__builtin_amdgcn_readfirstlane((int)interior)) {
+#pragma unroll
+            for (int pr = 0; pr < TN / 2; ++pr) {
+                T *col = out + (int64_t)(m_wave + lr) * out_rs + (n_wave >> 1) + pr * 32 + lh * 16;
+#pragma unroll
+                for (int i = ROW0; i < ROW0 + ROWS; ++i) {
+                    float r[16];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        r[v] = apply_act16(acc[i][2 * pr][v] + bias_elem<T>(braw[2 * pr], v), BASE) *
+                               (acc[i][2 * pr + 1][v] + bias_elem<T>(braw[2 * pr + 1], v));
+                    store16(col + (int64_t)(i * 32) * out_rs, r);
+                }
+            }
+            return;
+        }
+#pragma unroll
+        for (int pr = 0; pr < TN / 2; ++pr) {
+            const int n = (n_wave >> 1) + pr * 32 + lh * 16;         // output column
+#pragma unroll
+            for (int i = ROW0; i < ROW0 + ROWS; ++i) {
+                const int m = m_wave + i * 32 + lr;
+                if (m >= M || n >= n_total) continue;  // n_total is a multiple of 32: a block is in or out as a whole
+                float r[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    r[v] = apply_act16(acc[i][2 * pr][v] + bias_elem<T>(braw[2 * pr], v), BASE) *
+                           (acc[i][2 * pr + 1][v] + bias_elem<T>(braw[2 * pr + 1], v));
+                if (out_vec_ok) {
+                    store16(out + (int64_t)m * out_rs + n, r);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
+                }
+            }
+        }
+        return;
+    }
+    const bool interior = rows_inside && n_wave + TN * 32 <= N && out_vec_ok && act_in == nullptr;
+    if (__builtin_amdgcn_readfirstlane((int)interior)) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            T *col = out + (int64_t)(m_wave + lr) * out_rs + n_wave + j * 32 + lh * 16;
+#pragma unroll
+            for (int i = ROW0; i < ROW0 + ROWS; ++i) {
+                float r[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) r[v] = apply_act16(acc[i][j][v] + bias_elem<T>(braw[j], v), ACT);
+                store16(col + (int64_t)(i * 32) * out_rs, r);
+            }
+        }
+        return;
+    }
+    const bool SAVE_ACT_IN = act_in != nullptr;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int n = n_wave + j * 32 + lh * 16;
+#pragma unroll
+        for (int i = ROW0; i < ROW0 + ROWS; ++i) {
+            const int m = m_wave + i * 32 + lr;
+            if (m >= M || n >= N) continue;
+            float r[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) r[v] = acc[i][j][v] + bias_elem<T>(braw[j], v);  // zeros without a bias
+            if (SAVE_ACT_IN) {
+                if (ai_vec_ok && n + 16 <= N) {
+                    store16(act_in + (int64_t)m * ai_rs + n, r);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        if (n + v < N) act_in[(int64_t)m * ai_rs + (int64_t)(n + v) * ai_cs] = from_float<T>(r[v]);
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) r[v] = apply_act16(r[v], ACT);
+            if (out_vec_ok && n + 16 <= N) {
+                store16(out + (int64_t)m * out_rs + n, r);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (n + v < N) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
+            }
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------------
+// MFMA kernel
+// ----------------------------------------------------------------------------------------------------
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int MIN_BLOCKS_>
+struct LinearTile {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int MIN_BLOCKS = MIN_BLOCKS_;
+    static constexpr int THREADS = 64 * WAVES_M * WAVES_N;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // per-wave output tile
+    static constexpr int TM = WM / 32, TN = WN / 32;            // 32x32 MFMA blocks per wave
+    static constexpr int ROW_BYTES = BK * 2;
+    static constexpr int CPR = BK / 8;  // 16-byte chunks per tile row
+    static constexpr int X_BYTES = BM * ROW_BYTES, W_BYTES = BN * ROW_BYTES;
+    static constexpr int STAGE_BYTES = X_BYTES + W_BYTES;
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+    static constexpr int XI = BM * CPR / THREADS, WI = BN * CPR / THREADS;  // chunks per thread per stage
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32 blocks");
+    static_assert(BM * CPR % THREADS == 0 && BN * CPR % THREADS == 0, "tile rows must split over threads");
+    static constexpr int GROUP_M = 4;  // m-tiles walked together so one XCD's L2 sees a compact block
+};
+
+// W8: the weight is stored as one byte per element (fp8 e5m2, the upper byte of the fp16 encoding); a thread fetches
+// 8 bytes where it would fetch a 16-byte chunk and widens them on the way into LDS, so everything after the LDS
+// store is the 16-bit kernel.
+template <typename T, typename Cfg, int ACT, bool W8 = false>
+__global__ void __launch_bounds__(Cfg::THREADS, Cfg::MIN_BLOCKS)
+linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
+                   T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx,
+                   int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n,
+                   int out_vec_ok, int ai_vec_ok, int bias_vec_ok) {
+    typedef typename Vec8<T>::type vec8;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, CPR = Cfg::CPR, RB = Cfg::ROW_BYTES;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    // ---- tile assignment: workgroup ids are dealt round-robin to the 8 XCDs, so give each XCD a
+    // contiguous run of the (grouped) tile order; its private L2 then sees neighbouring tiles.
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) >> 3;
+    const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || t >= total) return;
+    const int group_span = Cfg::GROUP_M * tiles_n;
+    const int group = t / group_span;
+    const int first_m = group * Cfg::GROUP_M;
+    const int gsize = min(tiles_m - first_m, Cfg::GROUP_M);
+    const int in_group = t - group * group_span;
+    const int tile_m = first_m + in_group % gsize;
+    const int tile_n = in_group / gsize;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave % Cfg::WAVES_M, wave_n = wave / Cfg::WAVES_M;
+    const int lr = lane & 31, lh = lane >> 5;
+
+    // ---- global -> register staging: thread owns chunks q = tid + THREADS*i, row q / CPR, chunk q % CPR.
+    // Loads are buffer loads: a wave-uniform resource (tile origin, extent up to the end of the last valid row),
+    // a loop-invariant per-thread 32-bit byte offset and the k position in a scalar register.  Anything past the
+    // extent — rows beyond M or N, k-tiles beyond K — reads as zero without touching memory, so the loop needs
+    // neither clamps nor branches; only a chunk that starts beyond K INSIDE a valid row is redirected by hand.
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    const int rows_x = min(BM, M - m0), rows_w = min(BN, N - n0);
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T *>(X + (int64_t)m0 * ldx), 0, (int)((((int64_t)rows_x - 1) * ldx + K) * 2), 0x00020000);
+    constexpr int WB = W8 ? 1 : 2;  // bytes per weight element in memory
+    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char *>(reinterpret_cast<const char *>(W) + (int64_t)n0 * K * WB), 0, (int)((int64_t)rows_w * K * WB),
+        0x00020000);
+    uint32_t xg[Cfg::XI], wg[Cfg::WI];  // byte offsets from the tile origins
+    int xl[Cfg::XI], wl[Cfg::WI];       // LDS byte offsets inside a stage
+#pragma unroll
+    for (int i = 0; i < Cfg::XI; ++i) {
+        const int q = tid + Cfg::THREADS * i;
+        const int row = q / CPR, c = q % CPR;
+        xg[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) : kOutOfRange;
+        xl[i] = swz_offset<RB>(row, c);
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::WI; ++i) {
+        const int q = tid + Cfg::THREADS * i;
+        const int row = q / CPR, c = q % CPR;
+        // LDS row `row` feeds MFMA row (row % 32) of its 32-block and carries weight row rowperm16(row % 32).
+        const int wrow = (row & ~31) + rowperm16(row & 31);
+        wg[i] = wrow < rows_w ? (uint32_t)(((int64_t)wrow * K + c * 8) * WB) : kOutOfRange;
+        wl[i] = Cfg::X_BYTES + swz_offset<RB>(row, c);
+    }
+    const int kchunk = (tid % CPR) * 8;  // same for every i because THREADS % CPR == 0
+
+    // ---- software pipeline over k-tiles of BK:
+    //   registers hold tile kt+1 (fetched from HBM/L2 during iteration kt-1), LDS stage kt&1 holds tile kt.
+    //   Iteration kt, k-step s:  read the operand fragments of step s+1 from LDS, store a quarter of tile kt+1
+    //   from registers into the other LDS stage, run the MFMAs of step s, and re-issue the global loads of the
+    //   same quarter for tile kt+2.  Global latency gets a whole iteration to hide, LDS stores ride under the
+    //   MFMAs, and there is one barrier per k-tile.  The loop body is branch-free (past the last k-tile the loads
+    //   return zeros and the stores fill a stage nobody reads), which keeps the number of loads in flight known
+    //   at compile time: the memory counters are waited on by count.
+    constexpr int KSTEPS = BK / 16;
+    vec8 xs[Cfg::XI], ws[Cfg::WI];
+    const int nk = (K + BK - 1) / BK;
+
+    auto gload_part = [&](int k0, int part) {  // chunks i with i % KSTEPS == part
+        const bool inside = k0 + kchunk < K;   // K % 8 == 0: a 16-byte chunk is entirely inside or outside
+#pragma unroll
+        for (int i = 0; i < Cfg::XI; ++i)
+            if (i % KSTEPS == part)
+                xs[i] = __builtin_bit_cast(
+                    vec8, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, inside ? xg[i] : kOutOfRange, k0 * 2, 0));
+#pragma unroll
+        for (int i = 0; i < Cfg::WI; ++i)
+            if (i % KSTEPS == part) {
+                if constexpr (W8) {
+                    const u32x2 raw = __builtin_amdgcn_raw_buffer_load_b64(wrsrc, inside ? wg[i] : kOutOfRange, k0, 0);
+                    const u32x4 wide = {__builtin_amdgcn_perm(0u, raw[0], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[0], 0x030c020cu),
+                                        __builtin_amdgcn_perm(0u, raw[1], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[1], 0x030c020cu)};
+                    ws[i] = __builtin_bit_cast(vec8, wide);
+                } else {
+                    ws[i] = __builtin_bit_cast(
+                        vec8, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, inside ? wg[i] : kOutOfRange, k0 * 2, 0));
+                }
+            }
+    };
+    auto lstore_part = [&](int stage, int part) {
+        unsigned char *base = smem + stage * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < Cfg::XI; ++i)
+            if (i % KSTEPS == part) *reinterpret_cast<vec8 *>(base + xl[i]) = xs[i];
+#pragma unroll
+        for (int i = 0; i < Cfg::WI; ++i)
+            if (i % KSTEPS == part) *reinterpret_cast<vec8 *>(base + wl[i]) = ws[i];
+    };
+
+    f32x16 acc[TM][TN];
+    // this wave's bias entries: in flight during the main loop where the tile shape leaves registers for them,
+    // fetched in one go after it otherwise
+    constexpr bool EARLY_BIAS = BM * BN < 256 * 256;
+    u32x4 braw[TN][2];
+    if (EARLY_BIAS) bias_fetch<T, TN>(bias, n0 + wave_n * Cfg::WN, lh, N, bias_vec_ok, braw);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // LDS byte offsets of this lane's operand fragments for k-step 0.  Chunk index 2*step + lh and the XOR swizzle
+    // only touch bits 4..6 of the offset, so step s is the same offset XOR 32*s.
+    static_assert(RB == 128 || RB == 64, "fragment addressing below assumes 64- or 32-element k-tiles");
+    int xoff[TM], woff[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) xoff[i] = swz_offset<RB>(wave_m * Cfg::WM + i * 32 + lr, lh);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) woff[j] = Cfg::X_BYTES + swz_offset<RB>(wave_n * Cfg::WN + j * 32 + lr, lh);
+
+#pragma unroll
+    for (int part = 0; part < KSTEPS; ++part) gload_part(0, part);
+#pragma unroll
+    for (int part = 0; part < KSTEPS; ++part) lstore_part(0, part);
+#pragma unroll
+    for (int part = 0; part < KSTEPS; ++part) gload_part(BK, part);
+    __syncthreads();
+
+    vec8 fa[2][TN], fb[2][TM];
+    for (int kt = 0; kt < nk; ++kt) {
+        const unsigned char *cur = smem + (kt & 1) * Cfg::STAGE_BYTES;
+        const int nxt = (kt + 1) & 1;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fa[0][j] = *reinterpret_cast<const vec8 *>(cur + woff[j]);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fb[0][i] = *reinterpret_cast<const vec8 *>(cur + xoff[i]);
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            if (st + 1 < KSTEPS) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    fa[(st + 1) & 1][j] = *reinterpret_cast<const vec8 *>(cur + (woff[j] ^ (32 * (st + 1))));
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    fb[(st + 1) & 1][i] = *reinterpret_cast<const vec8 *>(cur + (xoff[i] ^ (32 * (st + 1))));
+            }
+            lstore_part(nxt, st);
+            __builtin_amdgcn_sched_barrier(0);  // keep the order: fragment reads, LDS stores, MFMAs, global loads
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = mfma32(fa[st & 1][j], fb[st & 1][i], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
+            gload_part((kt + 2) * BK, st);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+    }
+
+    if (!EARLY_BIAS) bias_fetch<T, TN>(bias, n0 + wave_n * Cfg::WN, lh, N, bias_vec_ok, braw);
+    linear_epilogue<T, ACT, TM, TN>(acc, m0 + wave_m * Cfg::WM, n0 + wave_n * Cfg::WN, lr, lh, bias, out, act_in, M, N, out_rs,
+                                    out_cs, ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bias_vec_ok, braw);
+}
+
+// ----------------------------------------------------------------------------------------------------
+// Wide MFMA kernel for K % 64 == 0: 256x256 output tile, 4 waves, ONE wave per SIMD owning a 128x128 sub-tile as
+// 8x8 blocks of v_mfma_f32_16x16x32 (256 accumulator registers, kept in the accumulation half of the register file).
+// Per 32-wide k-step a wave runs 64 MFMAs on 16 operand fragments — half the LDS traffic per flop of the 8-wave
+// kernel above.  Operand tiles go HBM -> LDS directly (buffer loads with the LDS flag), two 64 KB stages.  With a
+// single wave per SIMD nothing else can fill a stall, so the instruction stream is laid out by hand: LDS reads and
+// tile loads issue in the shadow of the MFMAs (at most one every other MFMA), fragments are read one k-step (64
+// MFMAs) ahead, and the one barrier per k-tile sits in front of its second k-step, after which the stage just
+// consumed takes the next-but-one k-tile, one load every fourth MFMA.  (A burst of 16 loads followed by a wait for
+// all of them stalls a lone wave: 64 KB need >= 1024 cycles to pass the CU's 64 B/clk fill path.)
+//
+// Weight rows are placed in LDS so that a lane ends up with consecutive output columns: MFMA row r of block j in a
+// 64-row group carries weight row 16 (r/4) + 4 j + r%4, so lane group g = lane/16 holds the 16 columns 16 g .. 16 g+15
+// of the group across its four blocks.  Gated epilogues use 32 (j/2) + 8 (r/4) + 4 (j%2) + r%4 instead: the lane holds
+// gate AND value of the 8 output columns 8 g .. 8 g + 7.
+// ----------------------------------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ u32x4 fetch8(const T *__restrict__ p, int idx, int limit, int vec_ok) {
+    u32x4 r = {0, 0, 0, 0};
+    if (p == nullptr) return r;
+    if (vec_ok && idx + 8 <= limit) return *reinterpret_cast<const u32x4 *>(p + idx);
+#pragma unroll
+    for (int v = 0; v < 8; v += 2) {
+        const uint32_t lo = idx + v < limit ? (uint32_t)__builtin_bit_cast(uint16_t, p[idx + v]) : 0u;
+        const uint32_t hi = idx + v + 1 < limit ? (uint32_t)__builtin_bit_cast(uint16_t, p[idx + v + 1]) : 0u;
+        r[v >> 1] = lo | (hi << 16);
+    }
+    return r;
+}
+
+// Epilogue of m-block IB (16 rows) of a wave of the wide kernel: lane (l16, g) holds row m_wave + 16 IB + l16 and, in
+// every group of JB n-blocks, the 4 JB consecutive columns starting at 4 JB g (JB = 4: 64-column groups, 2: 32-column).
+template <typename T, int ACT, int IB, int NBN, int NBM = 8>
+__device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_wave, int n_wave, int l16, int g,
+                                              T *__restrict__ out, T *__restrict__ act_in, int M, int N,
+                                              int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs,
+                                              int out_vec_ok, int ai_vec_ok,
+                                              const u32x4 (&braw)[NBN == 8 ? 2 : 3][2]) {
+    const int m = m_wave + 16 * IB + l16;
+    const bool rows_inside = m_wave + 16 * IB + 16 <= M;
+    if constexpr ((ACT & kGluBit) != 0) {
+        static_assert(NBN == 8, "gated epilogues pair blocks inside 64-row groups");
+        constexpr int BASE = ACT & (kGluBit - 1);
+        const int n_total = N >> 1;
+        const bool interior = rows_inside && (n_wave >> 1) + 64 <= n_total && out_vec_ok;
+        const bool fast = __builtin_amdgcn_readfirstlane((int)interior) != 0;
+#pragma unroll
+        for (int G = 0; G < 2; ++G) {
+            const int n = (n_wave >> 1) + 32 * G + 8 * g;  // 8 consecutive output columns
+            if (!fast && (m >= M || n >= n_total)) continue;  // n_total is a multiple of 32 and n of 8
+            float r[8];
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const float gate = acc[IB][4 * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v);
+                const float value = acc[IB][4 * G + 2 + (v >> 2)][v & 3] + bias_elem<T>(braw[G], 8 + v);
+                r[v] = apply_act16(gate, BASE) * value;
+            }
+            if (fast || out_vec_ok) {
+                u32x4 p;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) p[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
+                *reinterpret_cast<u32x4 *>(out + (int64_t)m * out_rs + n) = p;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 8; ++v) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
+            }
+        }
+        return;
+    }
+    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB, VPG = 4 * JB;  // blocks per group, groups, values per lane and group
+    auto store_vec = [&](T *p, const float (&r)[VPG]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int h = 0; h < VPG / 8; ++h) {
+            u32x4 pk;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) pk[v] = pack2<T>(r[8 * h + 2 * v], r[8 * h + 2 * v + 1]);
+            *reinterpret_cast<u32x4 *>(p + 8 * h) = pk;
+        }
+    };
+    const bool interior = rows_inside && n_wave + NBN * 16 <= N && out_vec_ok && act_in == nullptr;
+    if (__builtin_amdgcn_readfirstlane((int)interior)) {
+#pragma unroll
+        for (int G = 0; G < NG; ++G) {
+            float r[VPG];
+#pragma unroll
+            for (int v = 0; v < VPG; ++v) r[v] = apply_act16(acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v), ACT);
+            store_vec(out + (int64_t)m * out_rs + n_wave + 16 * JB * G + VPG * g, r);
+        }
+        return;
+    }
+#pragma unroll
+    for (int G = 0; G < NG; ++G) {
+        const int n = n_wave + 16 * JB * G + VPG * g;
+        if (m >= M || n >= N) continue;
+        float r[VPG];
+#pragma unroll
+        for (int v = 0; v < VPG; ++v) r[v] = acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v);
+        if (act_in != nullptr) {
+            if (ai_vec_ok && n + VPG <= N) {
+                store_vec(act_in + (int64_t)m * ai_rs + n, r);
+            } else {
+#pragma unroll
+                for (int v = 0; v < VPG; ++v)
+                    if (n + v < N) act_in[(int64_t)m * ai_rs + (int64_t)(n + v) * ai_cs] = from_float<T>(r[v]);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < VPG; ++v) r[v] = apply_act16(r[v], ACT);
+        if (out_vec_ok && n + VPG <= N) {
+            store_vec(out + (int64_t)m * out_rs + n, r);
+        } else {
+#pragma unroll
+            for (int v = 0; v < VPG; ++v)
+                if (n + v < N) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
+        }
+    }
+}
+
+// W8: the weight is stored as one byte per element (fp8 e5m2, the upper byte of the fp16 encoding).  Its tile travels
+// HBM -> LDS as bytes (half the loads, 64-byte rows, chunks swizzled for 8-byte reads), a fragment is read as 8 bytes
+// and widened by four byte-permutes two read slots later, all in the shadow of the MFMAs; everything else is unchanged.
+template <typename T, int ACT, int NBN, bool W8 = false>
+__global__ void __launch_bounds__(256, 1)
+linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
+                   T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
+                   int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok, int ai_vec_ok,
+                   int bias_vec_ok) {
+    typedef typename Vec8<T>::type vec8;
+    constexpr bool GATED = (ACT & kGluBit) != 0;
+    static_assert(NBN == 8 || (NBN == 6 && !GATED), "256 or 192 columns per tile; gated epilogues need 256");
+    constexpr int BM = 256, BN = 32 * NBN, BK = 64, RB = BK * 2, CPR = BK / 8, NB = 8, KSTEPS = BK / 32;
+    // LDS: [x stage 0 | x stage 1 | w stage 0 | w stage 1], 32 KB each: every fragment address is one per-lane register
+    // plus an immediate of 0 or 32 KB for the stage (the immediate field of an LDS read ends at 64 KB - 1).
+    constexpr int X_BYTES = BM * RB, W_BYTES = 32768, W_BASE = 2 * X_BYTES;
+    static_assert(X_BYTES == 32768 && BN * RB <= W_BYTES, "stage immediates");
+    static_assert(!W8 || (std::is_same<T, f16>::value && NBN == 8 && !GATED), "one-byte weights: fp16, 256 columns, plain");
+    constexpr int WB = W8 ? 1 : 2;                                   // bytes per weight element in memory and in LDS
+    constexpr int RBW = BK * WB, CPRW = RBW / 16;                    // weight tile: row bytes, 16-byte chunks per row
+    constexpr int LOADS = BM * CPR / 256, LOADS_W = BN * CPRW / 256;  // 1 KB loads per wave for the x and the w tile
+    constexpr int NL = LOADS + LOADS_W;                             // tile loads per wave and k-tile
+    constexpr int GROUP_M = 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    // Persistent workgroups: one per CU (at most), each walking the output tiles  slot, slot + slots, ...  of its
+    // XCD's contiguous run of the grouped tile order.  The k-tile stream runs THROUGH tile boundaries: while the last
+    // k-tiles of one output tile are multiplied, the first two k-tiles of the next are already on their way into LDS,
+    // and the epilogue's stores drain under the next tile's main loop.
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) >> 3;
+    const int xcd = (int)(blockIdx.x & 7), slots = (int)(gridDim.x >> 3);
+    auto tile_origin = [&](int idx, int &m0, int &n0) __attribute__((always_inline)) -> bool {
+        const int t = xcd * per_xcd + idx;
+        if (idx >= per_xcd || t >= total) return false;
+        const int group_span = GROUP_M * tiles_n;
+        const int group = t / group_span;
+        const int first_m = group * GROUP_M;
+        const int gsize = min(tiles_m - first_m, GROUP_M);
+        const int in_group = t - group * group_span;
+        m0 = (first_m + in_group % gsize) * BM;
+        n0 = (in_group / gsize) * BN;
+        return true;
+    };
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave & 1, wave_n = wave >> 1;
+    const int l16 = lane & 15, g = lane >> 4;
+
+    // ---- tile loads: load i of a wave fills the 1 KB of 16-byte chunks [256 i + 64 wave, +64) of an operand tile;
+    // every lane fetches the chunk that belongs at its LDS position under the swizzle.  Rows beyond M / N lie outside
+    // the buffer resource and arrive as zeros.  A wave's loads of one operand tile land in one contiguous 8 KB block
+    // (load i at +1 KB i), so that groups of 4 loads share one write of the LDS base register and differ only in the
+    // instruction's immediate offset.  That immediate is added to the memory address too, hence it is subtracted from
+    // the per-lane offsets here.
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    u32x4 xrsrc = {0, 0, 0, 0x00020000u}, wrsrc = {0, 0, 0, 0x00020000u};
+    uint32_t xd[LOADS], wd[LOADS_W];
+    // points the tile loads at the output tile with origin (m0, n0); `valid` false switches them off
+    auto set_load_tile = [&](bool valid, int m0, int n0) __attribute__((always_inline)) {
+        const int rows_x = valid ? min(BM, M - m0) : 0, rows_w = valid ? min(BN, N - n0) : 0;
+        if (valid) {
+            const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx);
+            const uint64_t waddr = (uint64_t)(uintptr_t)(reinterpret_cast<const char *>(W) + (int64_t)n0 * K * WB);
+            xrsrc[0] = (uint32_t)xaddr;
+            xrsrc[1] = (uint32_t)(xaddr >> 32) & 0xFFFFu;
+            xrsrc[2] = (uint32_t)((((int64_t)rows_x - 1) * ldx + K) * 2);
+            wrsrc[0] = (uint32_t)waddr;
+            wrsrc[1] = (uint32_t)(waddr >> 32) & 0xFFFFu;
+            wrsrc[2] = (uint32_t)((int64_t)rows_w * K * WB);
+        }
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int q = (wave * LOADS + i) * 64 + lane;  // 16-byte chunk index inside the tile
+            const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+            xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
+        }
+#pragma unroll
+        for (int i = 0; i < LOADS_W; ++i) {
+            const int q = (wave * LOADS_W + i) * 64 + lane;
+            const int row = q / CPRW, c = swz_chunk<RBW>(row, q % CPRW);
+            // LDS row `row` is MFMA row r = row % 16 of n-block row / 16; see the placement rule above the kernel
+            const int wrow = wide_weight_row<GATED, NBN>(row);
+            wd[i] = wrow < rows_w ? (uint32_t)((int64_t)wrow * K * WB + c * 16) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
+        }
+    };
+    typedef __attribute__((address_space(3))) void lds_void;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
+    // inline assembly on purpose: the compiler would make every later LDS read wait for loads it sees writing LDS.
+    // `group` (0 or 1) selects loads 4 group .. 4 group + 3; its first load writes the LDS base register.
+    auto load4 = [&](const u32x4 &rsrc, uint32_t off, uint32_t lds, int group, int part, int kbytes) __attribute__((always_inline)) {
+        if (part == 0)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :: "s"(lds + group * 4096), "v"(off), "s"(rsrc), "s"(kbytes) : "memory", "m0");
+        else if (part == 1)
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
+        else if (part == 2)
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:2048 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
+        else
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
+    };
+    // load l (0 .. NL-1) of a k-tile: the x loads, then the w loads
+    auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
+        if (l < LOADS) load4(xrsrc, xd[l], lds_base + stage * X_BYTES + wave * (LOADS * 1024), l >> 2, l & 3, k0 * 2);
+        else load4(wrsrc, wd[l - LOADS], lds_base + W_BASE + stage * W_BYTES + wave * (LOADS_W * 1024), (l - LOADS) >> 2, (l - LOADS) & 3, k0 * WB);
+    };
+
+    // LDS addresses of this lane's operand fragments in stage 0, one register per (k-step, block): with a whole
+    // register file per wave there is room to keep them all, and no address arithmetic is left in the loop
+    typedef __attribute__((address_space(3))) const unsigned char *lds_bytes;
+    typedef __attribute__((address_space(3))) const vec8 *lds_frag;
+    const lds_bytes lds0 = (lds_bytes)smem;
+    lds_frag xfrag[KSTEPS][NB], wfrag[KSTEPS][NBN];
+#pragma unroll
+    for (int st = 0; st < KSTEPS; ++st) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) xfrag[st][i] = (lds_frag)(lds0 + swz_offset<RB>(wave_m * 128 + i * 16 + l16, 4 * st + g));
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) {
+            const int row = wave_n * (NBN * 16) + j * 16 + l16, unit = 4 * st + g;   // 8 k-values per unit
+            wfrag[st][j] = W8 ? (lds_frag)(lds0 + W_BASE + swz_offset<RBW>(row, unit >> 1) + (unit & 1) * 8)
+                              : (lds_frag)(lds0 + W_BASE + swz_offset<RBW>(row, unit));
+        }
+    }
+    constexpr int STAGE_FRAGS = X_BYTES / 16;  // pointer increment that selects stage 1
+    // one-byte weights: 8 bytes per fragment, widened (byte b of a dword becomes the 16-bit value b << 8)
+    typedef __attribute__((address_space(3))) const u32x2 *lds_frag8;
+    auto read8 = [&](lds_frag ptr) __attribute__((always_inline)) -> u32x2 { return *(lds_frag8)ptr; };
+    auto widen8 = [&](u32x2 raw) __attribute__((always_inline)) -> vec8 {
+        const u32x4 wide = {__builtin_amdgcn_perm(0u, raw[0], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[0], 0x030c020cu),
+                            __builtin_amdgcn_perm(0u, raw[1], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[1], 0x030c020cu)};
+        return __builtin_bit_cast(vec8, wide);
+    };
+    u32x2 wraw[W8 ? NBN : 1];
+
+    const int nk = K / BK;
+    int idx = (int)(blockIdx.x >> 3);  // position of the tile being multiplied in this XCD's run
+    int m0 = 0, n0 = 0;
+    if (!tile_origin(idx, m0, n0)) return;
+
+    // the load side runs ahead of the multiply side: (load_idx, load_kt) is the next k-tile to request
+    int load_idx = idx, load_kt = 0;
+    set_load_tile(true, m0, n0);
+    auto advance_load = [&]() __attribute__((always_inline)) {
+        if (++load_kt == nk) {
+            load_kt = 0;
+            load_idx += slots;
+            int lm0 = 0, ln0 = 0;
+            const bool more = tile_origin(load_idx, lm0, ln0);
+            set_load_tile(more, lm0, ln0);
+        }
+    };
+#pragma unroll
+    for (int l = 0; l < NL; ++l) tile_load(l, 0, load_kt * BK);
+    advance_load();
+#pragma unroll
+    for (int l = 0; l < NL; ++l) tile_load(l, 1, load_kt * BK);
+    advance_load();
+    // vmcnt(NL): the first k-tile has landed, the second may still be in flight
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (NL & 15) | ((NL >> 4) << 14));
+    __syncthreads();
+
+    vec8 fa[KSTEPS][NBN], fb[KSTEPS][NB];  // weight and activation fragments, one register set per k-step
+#pragma unroll
+    for (int j = 0; j < NBN; ++j) {
+        if constexpr (W8) fa[0][j] = widen8(read8(wfrag[0][j]));
+        else fa[0][j] = *wfrag[0][j];
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) fb[0][i] = *xfrag[0][i];
+
+    f32x4_acc acc[NB][NBN];  // [m-block][n-block]
+
+    // One k-tile held in stage CUR (a compile-time constant, so that stage offsets fold into instruction offsets).
+    // `landed`: the loads of the next k-tile are known to have arrived (a wait for later loads has been passed), and
+    // waiting for "everything outstanding" would only wait for the previous tile's output stores.
+    auto k_tile = [&](auto cur_c, bool landed) __attribute__((always_inline)) {
+        constexpr int CUR = decltype(cur_c)::value;
+        const int k0 = load_kt * BK;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            const int sn = st ^ 1;                               // k-step whose fragments are fetched now
+            const int src = (st == 0 ? CUR : CUR ^ 1) * STAGE_FRAGS;  // stage holding those fragments
+            if (st == 1) {
+                if (!landed) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads of the next k-tile are in
+                __syncthreads();                                  // ... everyone's are, and nobody reads stage CUR any more
+            }
+            constexpr int PERIOD = NBN == 8 ? 4 : 3;  // MFMAs per LDS read / tile load: 64 / 4 = 48 / 3 = 16 issue slots
+#pragma unroll
+            for (int m = 0; m < NB * NBN; ++m) {
+                const int i = m / NBN, j = m % NBN;
+                mfma16_inplace(fa[st][j], fb[st][i], acc[i][j]);
+                const int slot = m / PERIOD;
+                if (m % PERIOD == 0 && slot < NBN + NB) {
+                    // the weight fragments first: the first MFMAs of the next k-step need all of them
+                    if (slot < NBN) {
+                        // (stage offsets are in 16-byte units of the 16-bit layout: a byte-weight stage is W_BYTES further all the same)
+                        if constexpr (W8) wraw[slot] = read8(wfrag[sn][slot] + src);
+                        else fa[sn][slot] = *(wfrag[sn][slot] + src);
+                    } else {
+                        fb[sn][slot - NBN] = *(xfrag[sn][slot - NBN] + src);
+                    }
+                } else if (W8 && m % PERIOD == 1 && slot >= 2 && slot - 2 < NBN) {
+                    fa[sn][slot - 2] = widen8(wraw[slot - 2]);  // two read slots later: the bytes have arrived
+                } else if (m % PERIOD == PERIOD - 2 && st == 1 && slot < NL) {
+                    tile_load(slot, CUR, k0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    // Every output tile starts in stage 0: the host launches one workgroup per tile when the number of k-tiles is odd.
+    bool landed = false;
+    while (true) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+#pragma unroll
+            for (int j = 0; j < NBN; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+        int kt = 0;
+        for (; kt + 1 < nk; kt += 2) {
+            k_tile(IntC<0>(), landed);
+            advance_load();
+            landed = false;
+            k_tile(IntC<1>(), false);
+            advance_load();
+        }
+        if (kt < nk) {
+            k_tile(IntC<0>(), landed);
+            advance_load();
+        }
+
+        // all bias entries of the lane's columns in one go: one memory round trip per tile.  Its wait also covers the
+        // loads of the next k-tile, which were issued earlier.
+        const int n_wave = n0 + wave_n * (NBN * 16);
+        constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB;  // n-blocks per lane-contiguous group, groups per wave
+        u32x4 braw[NG][2];
+#pragma unroll
+        for (int G = 0; G < NG; ++G)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0}
+                             : fetch8<T>(bias, n_wave + 16 * JB * G + (GATED ? 32 * h + 8 * g : 4 * JB * g + 8 * h), N, bias_vec_ok);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        landed = true;
+        // one call per 16-row block: each stays small enough for the compiler to unroll completely, so the
+        // accumulators are only ever indexed by constants and never leave the register file
+#define KERNL_WIDE_EPILOGUE(I)                                                                                         \
+    wide_epilogue<T, ACT, I, NBN>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs, ai_cs,   \
+                             out_vec_ok, ai_vec_ok, braw)
+        KERNL_WIDE_EPILOGUE(0);
+        KERNL_WIDE_EPILOGUE(1);
+        KERNL_WIDE_EPILOGUE(2);
+        KERNL_WIDE_EPILOGUE(3);
+        KERNL_WIDE_EPILOGUE(4);
+        KERNL_WIDE_EPILOGUE(5);
+        KERNL_WIDE_EPILOGUE(6);
+        KERNL_WIDE_EPILOGUE(7);
+#undef KERNL_WIDE_EPILOGUE
+        idx += slots;
+        if (!tile_origin(idx, m0, n0)) break;
+    }
+}
+
+// ----------------------------------------------------------------------------------------------------
+// Half-height variant of the wide kernel for outputs that leave CUs idle with 256-row tiles (M = 2048 against
+// N = 4096 gives 128 tiles of 256x256 but 256 of 128x256): 128 x (256 | 192) tile, 4 waves as 2 x 2, a 64-row
+// sub-tile per wave (4 x NBN blocks of v_mfma_f32_16x16x32).  A k-tile is only 2 x 32 (24) MFMAs long here, too short
+// to cover the load latency with two stages, and the smaller x tile leaves room for a third: THREE stages of
+// 16 KB (x) + 32 KB (w), k-tile T + 3 requested while k-tile T is multiplied, the wait in front of the second k-step
+// only for k-tile T + 1 (vmcnt(NL): the loads of T + 2 may still be in flight).  One workgroup per output tile.
+// ----------------------------------------------------------------------------------------------------
+// Tile t of the half-height kernels' grouped order (GROUP_M row tiles side by side) -> origin of the tile.
+__device__ __forceinline__ void half_tile_origin(int t, int tiles_m, int tiles_n, int BM, int BN, int &m0, int &n0) {
+    constexpr int GROUP_M = 8;
+    const int group_span = GROUP_M * tiles_n;
+    const int group = t / group_span;
+    const int first_m = group * GROUP_M;
+    const int gsize = min(tiles_m - first_m, GROUP_M);
+    const int in_group = t - group * group_span;
+    m0 = (first_m + in_group % gsize) * BM;
+    n0 = (in_group / gsize) * BN;
+}
+
+// SPLIT: blockIdx.y selects one of `splits` ranges of k-tiles; the workgroup leaves its fp32 partial tile in `part`
+// (slot blockIdx.y * tiles + t; per wave and 16 x 16 block 64 lanes x 16 bytes: coalesced, and the same lane reads it
+// back in linear_wide_half_reduce_kernel, which adds the ranges in order and runs the epilogue).
+template <typename T, int ACT, int NBN, bool W8 = false, bool SPLIT = false>
+__global__ void __launch_bounds__(256, 1)
+linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
+                        T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs,
+                        int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok,
+                        int ai_vec_ok, int bias_vec_ok, float *__restrict__ part, int splits) {
+    typedef typename Vec8<T>::type vec8;
+    static_assert((ACT & kGluBit) == 0 && (NBN == 8 || NBN == 6), "plain epilogues, 256 or 192 columns");
+    constexpr int NBM = 4, BM = 32 * NBM, BN = 32 * NBN, BK = 64, RB = BK * 2, CPR = BK / 8, KSTEPS = BK / 32;
+    constexpr int X_STAGE = BM * RB, W_STAGE = 32768, W_BASE = 3 * X_STAGE;  // [x0|x1|x2|w0|w1|w2]
+    static_assert(X_STAGE == 16384 && BN * RB <= W_STAGE, "stage immediates");
+    static_assert(!W8 || (std::is_same<T, f16>::value && NBN == 8), "one-byte weights: fp16, 256 columns");
+    constexpr int WB = W8 ? 1 : 2, RBW = BK * WB, CPRW = RBW / 16;  // weight tile: bytes per element, row bytes, chunks per row
+    constexpr int LOADS_X = BM * CPR / 256, LOADS_W = BN * CPRW / 256, NL = LOADS_X + LOADS_W;
+    static_assert(LOADS_X == 4, "one group of four loads for the x tile");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) >> 3;
+    const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || t >= total) return;
+    int m0, n0;
+    half_tile_origin(t, tiles_m, tiles_n, BM, BN, m0, n0);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave & 1, wave_n = wave >> 1;
+    const int l16 = lane & 15, g = lane >> 4;
+
+    // tile loads, as in the wide kernel: every lane fetches the chunk that belongs at its LDS position
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    const int rows_x = min(BM, M - m0), rows_w = min(BN, N - n0);
+    const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx);
+    const uint64_t waddr = (uint64_t)(uintptr_t)(reinterpret_cast<const char *>(W) + (int64_t)n0 * K * WB);
+    const u32x4 xrsrc = {(uint32_t)xaddr, (uint32_t)(xaddr >> 32) & 0xFFFFu,
+                         (uint32_t)((((int64_t)rows_x - 1) * ldx + K) * 2), 0x00020000u};
+    const u32x4 wrsrc = {(uint32_t)waddr, (uint32_t)(waddr >> 32) & 0xFFFFu, (uint32_t)((int64_t)rows_w * K * WB),
+                         0x00020000u};
+    uint32_t xd[LOADS_X], wd[LOADS_W];
+#pragma unroll
+    for (int i = 0; i < LOADS_X; ++i) {
+        const int q = (wave * LOADS_X + i) * 64 + lane;
+        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
+    }
+#pragma unroll
+    for (int i = 0; i < LOADS_W; ++i) {
+        const int q = (wave * LOADS_W + i) * 64 + lane;
+        const int row = q / CPRW, c = swz_chunk<RBW>(row, q % CPRW);
+        const int wrow = wide_weight_row<false, NBN>(row);
+        wd[i] = wrow < rows_w ? (uint32_t)((int64_t)wrow * K * WB + c * 16) - (uint32_t)(i & 3) * 1024u : kOutOfRange;
+    }
+    typedef __attribute__((address_space(3))) void lds_void;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
+    auto load4 = [&](const u32x4 &rsrc, uint32_t off, uint32_t lds, int group4, int part, int kbytes) __attribute__((always_inline)) {
+        if (part == 0)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :: "s"(lds + group4 * 4096), "v"(off), "s"(rsrc), "s"(kbytes) : "memory", "m0");
+        else if (part == 1)
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
+        else if (part == 2)
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:2048 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
+        else
+            asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
+    };
+    auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
+        if (l < LOADS_X) load4(xrsrc, xd[l], lds_base + stage * X_STAGE + wave * (LOADS_X * 1024), 0, l, k0 * 2);
+        else load4(wrsrc, wd[l - LOADS_X], lds_base + W_BASE + stage * W_STAGE + wave * (LOADS_W * 1024), (l - LOADS_X) >> 2, (l - LOADS_X) & 3, k0 * WB);
+    };
+
+    // fragment addresses: x stages are 16 KB apart (immediates 0 / 16 K / 32 K); w stages 32 KB apart, and an LDS
+    // read's immediate ends at 64 KB - 1, so the third w stage has address registers of its own
+    typedef __attribute__((address_space(3))) const unsigned char *lds_bytes;
+    typedef __attribute__((address_space(3))) const vec8 *lds_frag;
+    const lds_bytes lds0 = (lds_bytes)smem;
+    lds_frag xfrag[KSTEPS][NBM], wfrag[KSTEPS][NBN], wfrag2[KSTEPS][NBN];
+#pragma unroll
+    for (int st = 0; st < KSTEPS; ++st) {
+#pragma unroll
+        for (int i = 0; i < NBM; ++i) xfrag[st][i] = (lds_frag)(lds0 + swz_offset<RB>(wave_m * (NBM * 16) + i * 16 + l16, 4 * st + g));
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) {
+            const int row = wave_n * (NBN * 16) + j * 16 + l16, unit = 4 * st + g;   // 8 k-values per unit
+            wfrag[st][j] = W8 ? (lds_frag)(lds0 + W_BASE + swz_offset<RBW>(row, unit >> 1) + (unit & 1) * 8)
+                              : (lds_frag)(lds0 + W_BASE + swz_offset<RBW>(row, unit));
+            wfrag2[st][j] = wfrag[st][j] + 2 * (W_STAGE / 16);
+        }
+    }
+
+    // Every k-tile slot issues its NL loads, so that the counter waits stay exact up to the end; requests past the
+    // last k-tile fetch that tile again (into a stage nobody reads any more) instead of running past the row ends.
+    int nk = K / BK, kb = 0;   // k-tiles of this workgroup: kb .. kb + nk - 1
+    if constexpr (SPLIT) {
+        const int per_split = (nk + splits - 1) / splits;
+        kb = (int)blockIdx.y * per_split;
+        nk = min(per_split, nk - kb);   // the host keeps every range non-empty
+    }
+#pragma unroll
+    for (int s3 = 0; s3 < 3; ++s3)
+#pragma unroll
+        for (int l = 0; l < NL; ++l) tile_load(l, s3, (kb + min(s3, nk - 1)) * BK);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * NL) & 15) | (((2 * NL) >> 4) << 14));  // vmcnt(2 NL): k-tile 0 has landed
+    __syncthreads();
+
+    // one-byte weights: 8 bytes per fragment, widened (byte b of a dword becomes the 16-bit value b << 8)
+    typedef __attribute__((address_space(3))) const u32x2 *lds_frag8;
+    auto widen8 = [&](u32x2 raw) __attribute__((always_inline)) -> vec8 {
+        const u32x4 wide = {__builtin_amdgcn_perm(0u, raw[0], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[0], 0x030c020cu),
+                            __builtin_amdgcn_perm(0u, raw[1], 0x010c000cu), __builtin_amdgcn_perm(0u, raw[1], 0x030c020cu)};
+        return __builtin_bit_cast(vec8, wide);
+    };
+    u32x2 wraw[W8 ? NBN : 1];
+    vec8 fa[KSTEPS][NBN], fb[KSTEPS][NBM];
+#pragma unroll
+    for (int j = 0; j < NBN; ++j) {
+        if constexpr (W8) fa[0][j] = widen8(*(lds_frag8)wfrag[0][j]);
+        else fa[0][j] = *wfrag[0][j];
+    }
+#pragma unroll
+    for (int i = 0; i < NBM; ++i) fb[0][i] = *xfrag[0][i];
+
+    f32x4_acc acc[NBM][NBN];
+#pragma unroll
+    for (int i = 0; i < NBM; ++i)
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // fragment reads of stage S3 for k-step st (compile-time stage: immediates, or the second register set)
+    auto read_w = [&](auto s3_c, int st, int j) __attribute__((always_inline)) -> vec8 {
+        constexpr int S3 = decltype(s3_c)::value;
+        return S3 == 2 ? *wfrag2[st][j] : *(wfrag[st][j] + S3 * (W_STAGE / 16));
+    };
+    auto read_w8 = [&](auto s3_c, int st, int j) __attribute__((always_inline)) -> u32x2 {
+        constexpr int S3 = decltype(s3_c)::value;
+        return S3 == 2 ? *(lds_frag8)wfrag2[st][j] : *(lds_frag8)(wfrag[st][j] + S3 * (W_STAGE / 16));
+    };
+    auto read_x = [&](auto s3_c, int st, int i) __attribute__((always_inline)) -> vec8 {
+        constexpr int S3 = decltype(s3_c)::value;
+        return *(xfrag[st][i] + S3 * (X_STAGE / 16));
+    };
+    auto k_tile = [&](auto cur_c, int kt) __attribute__((always_inline)) {
+        constexpr int CUR = decltype(cur_c)::value, NXT = (CUR + 1) % 3;
+        const int k_next = (kb + min(kt + 3, nk - 1)) * BK;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            const int sn = st ^ 1;
+            if (st == 1) {
+                __builtin_amdgcn_s_waitcnt(0x0F70 | (NL & 15) | ((NL >> 4) << 14));  // vmcnt(NL): k-tile kt + 1 has landed
+                __syncthreads();
+            }
+#pragma unroll
+            for (int m = 0; m < NBM * NBN; ++m) {
+                const int i = m / NBN, j = m % NBN;
+                mfma16_inplace(fa[st][j], fb[st][i], acc[i][j]);
+                const int slot = m >> 1;
+                if ((m & 1) == 0 && slot < NBN + NBM) {
+                    if (st == 0) {
+                        if (slot < NBN) {
+                            if constexpr (W8) wraw[slot] = read_w8(IntC<CUR>(), sn, slot);
+                            else fa[sn][slot] = read_w(IntC<CUR>(), sn, slot);
+                        } else {
+                            fb[sn][slot - NBN] = read_x(IntC<CUR>(), sn, slot - NBN);
+                        }
+                    } else {
+                        if (slot < NBN) {
+                            if constexpr (W8) wraw[slot] = read_w8(IntC<NXT>(), sn, slot);
+                            else fa[sn][slot] = read_w(IntC<NXT>(), sn, slot);
+                        } else {
+                            fb[sn][slot - NBN] = read_x(IntC<NXT>(), sn, slot - NBN);
+                        }
+                    }
+                } else if ((m & 1) == 1) {
+                    if (st == 1 && slot < NL) tile_load(slot, CUR, k_next);
+                    // one-byte weights: widened two read slots after the read, when the bytes have arrived
+                    if (W8 && slot >= 2 && slot - 2 < NBN) fa[sn][slot - 2] = widen8(wraw[slot - 2]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    int kt = 0;
+    for (; kt + 2 < nk; kt += 3) {
+        k_tile(IntC<0>(), kt);
+        k_tile(IntC<1>(), kt + 1);
+        k_tile(IntC<2>(), kt + 2);
+    }
+    if (kt < nk) k_tile(IntC<0>(), kt);
+    if (kt + 1 < nk) k_tile(IntC<1>(), kt + 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no load may still be writing LDS when the workgroup ends
+
+    if constexpr (SPLIT) {
+        float4 *dst = reinterpret_cast<float4 *>(part) + ((((int64_t)blockIdx.y * total + t) * 4 + wave) * (NBM * NBN)) * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < NBM; ++i)
+#pragma unroll
+            for (int j = 0; j < NBN; ++j)
+                dst[(i * NBN + j) * 64] = float4{acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+        return;
+    }
+    const int n_wave = n0 + wave_n * (NBN * 16);
+    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB;
+    u32x4 braw[NG][2];
+#pragma unroll
+    for (int G = 0; G < NG; ++G)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0} : fetch8<T>(bias, n_wave + 16 * JB * G + 4 * JB * g + 8 * h, N, bias_vec_ok);
+#define KERNL_HALF_EPILOGUE(I)                                                                                         \
+    wide_epilogue<T, ACT, I, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, \
+                                       ai_rs, ai_cs, out_vec_ok, ai_vec_ok, braw)
+    KERNL_HALF_EPILOGUE(0);
+    KERNL_HALF_EPILOGUE(1);
+    KERNL_HALF_EPILOGUE(2);
+    KERNL_HALF_EPILOGUE(3);
+#undef KERNL_HALF_EPILOGUE
+}
+
+// Second launch of the split form: workgroup (t, I) adds the k ranges' partial sums of 16-row block I of every wave of
+// tile t, in range order, and runs the epilogue the unsplit kernel runs (same wave and lane geometry).
+template <typename T, int ACT, int NBN>
+__global__ void __launch_bounds__(256)
+linear_wide_half_reduce_kernel(const float *__restrict__ part, const T *__restrict__ bias, T *__restrict__ out,
+                               T *__restrict__ act_in, int M, int N, int64_t out_rs, int64_t out_cs, int64_t ai_rs,
+                               int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok, int ai_vec_ok, int bias_vec_ok,
+                               int splits) {
+    constexpr int NBM = 4, BM = 32 * NBM, BN = 32 * NBN;
+    const int t = (int)blockIdx.x, I = (int)blockIdx.y, total = tiles_m * tiles_n;
+    int m0, n0;
+    half_tile_origin(t, tiles_m, tiles_n, BM, BN, m0, n0);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave & 1, wave_n = wave >> 1;
+    const int l16 = lane & 15, g = lane >> 4;
+    f32x4_acc acc[NBM][NBN];
+#pragma unroll
+    for (int i = 0; i < NBM; ++i)
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+    const float4 *src = reinterpret_cast<const float4 *>(part) + (((int64_t)t * 4 + wave) * (NBM * NBN) + I * NBN) * 64 + lane;
+    const int64_t split_stride = (int64_t)total * 4 * (NBM * NBN) * 64;
+    for (int sp = 0; sp < splits; ++sp) {
+        float4 v[NBN];
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) v[j] = src[sp * split_stride + j * 64];
+#pragma unroll
+        for (int i = 0; i < NBM; ++i) {
+            if (i != I) continue;   // (the block index of the accumulators is a compile-time constant in the epilogue)
+#pragma unroll
+            for (int j = 0; j < NBN; ++j) {
+                acc[i][j][0] += v[j].x;
+                acc[i][j][1] += v[j].y;
+                acc[i][j][2] += v[j].z;
+                acc[i][j][3] += v[j].w;
+            }
+        }
+    }
+    const int n_wave = n0 + wave_n * (NBN * 16);
+    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB;
+    u32x4 braw[NG][2];
+#pragma unroll
+    for (int G = 0; G < NG; ++G)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0} : fetch8<T>(bias, n_wave + 16 * JB * G + 4 * JB * g + 8 * h, N, bias_vec_ok);
+#define KERNL_HALF_REDUCE_EPILOGUE(IB)                                                                                   \
+    if (I == IB)                                                                                                         \
+    wide_epilogue<T, ACT, IB, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, \
+                                        ai_rs, ai_cs, out_vec_ok, ai_vec_ok, braw)
+    KERNL_HALF_REDUCE_EPILOGUE(0);
+    KERNL_HALF_REDUCE_EPILOGUE(1);
+    KERNL_HALF_REDUCE_EPILOGUE(2);
+    KERNL_HALF_REDUCE_EPILOGUE(3);
+#undef KERNL_HALF_REDUCE_EPILOGUE
+}
+
+// ----------------------------------------------------------------------------------------------------
+// Skinny kernel: at most 64 rows of x (decoding steps, pooled outputs).  The weight matrix is the only large operand
+// and the job is to stream it once at HBM speed with every CU: a workgroup owns 16 output columns (gated: their 16
+// gate and 16 value rows of the interleaved weight), its 4, 8 or 16 waves split K in interleaved 64-wide chunks (long
+// rows get many waves: the loop is bound by memory latency, and what counts is how many bytes a CU has in flight), every lane
+// fetches 32 contiguous bytes of its weight row per chunk (4 lanes cover a 128-byte line), and the fragments go from
+// global memory straight into v_mfma_f32_16x16x32 — weights on the A side, the few x rows on the B side.  The lane
+// of MFMA k-group g supplies k = 16 g + 8 s .. + 7 of the chunk in step s (s = 0, 1), on both sides, which is all
+// the instruction needs.  The waves' partial sums meet in LDS.  x is re-read by every workgroup, from L2.
+// ----------------------------------------------------------------------------------------------------
+// W8: the weight is stored as one byte per element, fp8 e5m2 — the upper byte of the fp16 encoding (reference:
+// `get_model_fp8`, experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84, read back with `.to(tl.float8e5,
+// bitcast=True).to(tl.float16)`, fused_kernel_ff.py:43-47).  A lane then fetches its 16 weights of a chunk as ONE
+// 16-byte load and byte-permutes them into the two fp16 fragments; fp16 activations only.
+// RMS: x is RMS-normalised on the way in (reference: `rms_matmul_rbe`, experimental/llama-v2/kernel/
+// fused_kernel_proj_qkv.py:116-183): the x fragments are multiplied by the norm's weight (rounded to 16 bit, as there),
+// every lane sums the squares of the x values that pass through it, and because the inverse root mean square is one
+// scalar per row it is applied to the finished sums: out = rsqrt(mean(x^2) + eps) * ((x * g) @ w^T) + bias.
+// Residual: out = act(...) + residual[m, n] when a residual pointer is given (the `hidden + projection(...)` of a
+// decoder layer; no counterpart in the reference, whose model adds in eager PyTorch).
+// ROPE: rotary position embedding applied to the output columns below `rope_cols`, in the half-split convention —
+// inside every head of `2 * half` columns, column d pairs with d + half:
+//     out[d] = y[d] cos[d] - y[d + half] sin[d],   out[d + half] = y[d + half] cos[d + half] + y[d] sin[d + half]
+// (reference: the rotation inside `rms_matmul_rbe_qkv`, experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:69-100
+// and :186-247, there on interleaved pairs with angles computed in the kernel; here from the cos / sin tables the
+// model computed, indexed by the row's batch entry and position).  A workgroup then owns the 16 columns d0 .. d0 + 15
+// of a head AND their partners (NR = 2 blocks, `half` columns apart), so both members of a pair meet in one lane.
+struct SkinnyExtra {
+    const void *residual;   // [M, N] of T, or null
+    int64_t res_rs, res_cs;
+    const void *cos, *sin;  // rotation tables, element (b, s, d) at b * t_bs + s * t_ss + d
+    int64_t t_bs, t_ss;
+    int table_dtype;        // KERNL_F16 / KERNL_BF16 / KERNL_F32
+    int half;               // half the head size
+    int rope_cols;          // columns [0, rope_cols) are rotated
+    int rows_per_batch;     // row m of x is position m % rows_per_batch of batch entry m / rows_per_batch
+};
+
+template <typename T, int MB, bool GATED, int WAVES, int NR, bool W8 = false, bool RMS = false, bool ROPE = false>
+__global__ void __launch_bounds__(64 * WAVES)
+linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
+                     T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
+                     int64_t ai_rs, int64_t ai_cs, int act, const T *__restrict__ rms_w, float eps, const SkinnyExtra ex) {
+    static_assert(!ROPE || (NR == 2 && !GATED && !W8), "the rotating form pairs two plain 16-column blocks");
+    typedef typename Vec8<T>::type vec8;
+    constexpr int NA = GATED ? 2 : 1;        // weight fragments per 16 output columns: plain, or gate and value
+    constexpr int NF = NA * NR;              // weight fragments per step (NR blocks of 16 output columns)
+    constexpr int U = (MB <= 2 && NF <= 2 && !RMS) ? 4 : 2;  // chunks requested together
+    static_assert(WAVES * NF * MB <= 64, "partial sums fit 64 KB of LDS");
+    __shared__ __attribute__((aligned(16))) float red[WAVES][NF * MB][64][4];
+    __shared__ float red_sq[RMS ? WAVES : 1][MB][16];
+
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    // first output column of this workgroup (N counts output columns) and the distance between its column blocks
+    const int blocks_per_half = ROPE ? ex.half / 16 : 1;
+    const int n0 = ROPE ? ((int)blockIdx.x / blocks_per_half) * (2 * ex.half) + ((int)blockIdx.x % blocks_per_half) * 16
+                        : (int)blockIdx.x * (16 * NR);
+    const int rb_stride = ROPE ? ex.half : 16;
+    // first interleaved row of the 16 output columns starting at nb (gated weights: 32 gate rows, 32 value rows, ...)
+    auto gated_row = [](int nb) -> int { return (nb >> 5) * 64 + (nb & 31); };
+    // rows of the weight this lane reads; columns beyond N repeat the last one and are never stored
+    static_assert(!W8 || std::is_same<T, f16>::value, "one-byte weights are decoded to fp16");
+    typedef typename std::conditional<W8, unsigned char, T>::type WT;  // what a weight element is stored as
+    const WT *wbase = reinterpret_cast<const WT *>(W);
+    const WT *wp[NF];
+#pragma unroll
+    for (int rb = 0; rb < NR; ++rb) {
+        const int nb = n0 + rb_stride * rb;
+        if (GATED) {
+            const int row = gated_row(min(nb, N - 16)) + r;
+            wp[rb * NA] = wbase + (int64_t)row * K + 16 * g;
+            wp[rb * NA + NA - 1] = wbase + (int64_t)(row + 32) * K + 16 * g;
+        } else {
+            wp[rb * NA] = wbase + (int64_t)min(nb + r, N - 1) * K + 16 * g;
+        }
+    }
+    const T *xp[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) xp[mb] = X + (int64_t)min(16 * mb + r, M - 1) * ldx + 16 * g;
+
+    f32x4_acc acc[NF][MB];
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[f][mb] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+
+    float sq[MB];  // sum of squares of the x values this lane has seen, per 16-row block (RMS)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) sq[mb] = 0.0f;
+    const int nchunks = K / 64;
+    const int rot = (int)((blockIdx.x * 13u) % (unsigned)nchunks);
+    for (int c0 = wave; c0 < nchunks; c0 += WAVES * U) {
+        vec8 wf[U][NF][2], xf[U][MB][2], gf[RMS ? U : 1][2];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            // chunks past the end are neither fetched nor multiplied (the test is uniform over the wave); only the
+            // 16-wave form with 128 fragment registers in flight, which has none to spare for the branches, fetches
+            // the last chunk again instead.  Workgroups walk the chunks from different starting points, so that they
+            // do not all ask L2 for the same lines of x at once.
+            constexpr bool kSkipTail = !(WAVES == 16 && U * (NF + MB) >= 16);
+            if (kSkipTail && c0 + WAVES * u >= nchunks) continue;
+            int cc = min(c0 + WAVES * u, nchunks - 1) + rot;
+            cc = cc >= nchunks ? cc - nchunks : cc;
+            const int k0 = cc * 64;
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+                if constexpr (W8) {
+                    const u32x4 raw = *reinterpret_cast<const u32x4 *>(wp[f] + k0);
+                    u32x4 lo, hi;  // bytes {0, b0, 0, b1} / {0, b2, 0, b3} of every word: fp16 pairs
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        lo[2 * j] = __builtin_amdgcn_perm(0u, raw[j], 0x010c000cu);
+                        lo[2 * j + 1] = __builtin_amdgcn_perm(0u, raw[j], 0x030c020cu);
+                        hi[2 * j] = __builtin_amdgcn_perm(0u, raw[2 + j], 0x010c000cu);
+                        hi[2 * j + 1] = __builtin_amdgcn_perm(0u, raw[2 + j], 0x030c020cu);
+                    }
+                    wf[u][f][0] = __builtin_bit_cast(vec8, lo);
+                    wf[u][f][1] = __builtin_bit_cast(vec8, hi);
+                } else {
+                    wf[u][f][0] = *reinterpret_cast<const vec8 *>(wp[f] + k0);
+                    wf[u][f][1] = *reinterpret_cast<const vec8 *>(wp[f] + k0 + 8);
+                }
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                xf[u][mb][0] = *reinterpret_cast<const vec8 *>(xp[mb] + k0);
+                xf[u][mb][1] = *reinterpret_cast<const vec8 *>(xp[mb] + k0 + 8);
+            }
+            if constexpr (RMS) {
+                gf[u][0] = *reinterpret_cast<const vec8 *>(rms_w + k0 + 16 * g);
+                gf[u][1] = *reinterpret_cast<const vec8 *>(rms_w + k0 + 16 * g + 8);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (c0 + WAVES * u < nchunks) {
+                if constexpr (RMS) {
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                const float xv = to_float(xf[u][mb][h][e]);
+                                sq[mb] = fmaf(xv, xv, sq[mb]);
+                            }
+                            xf[u][mb][h] = xf[u][mb][h] * gf[u][h];
+                        }
+                }
+#pragma unroll
+                for (int f = 0; f < NF; ++f)
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) {
+                        acc[f][mb] = mfma16(wf[u][f][0], xf[u][mb][0], acc[f][mb]);
+                        acc[f][mb] = mfma16(wf[u][f][1], xf[u][mb][1], acc[f][mb]);
+                    }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[wave][f * MB + mb][lane][e] = acc[f][mb][e];
+    if constexpr (RMS) {
+        // a row's squares are spread over the 4 lanes r, r + 16, r + 32, r + 48 of every wave
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            float t = sq[mb];
+            t += __shfl_xor(t, 16, 64);
+            t += __shfl_xor(t, 32, 64);
+            if (g == 0) red_sq[wave][mb][r] = t;
+        }
+    }
+    __syncthreads();
+
+    // the waves share the NR x MB blocks of 16 columns x 16 rows: element e of a lane is output column nb + 4 g + e
+    // of x row 16 mb + r
+    if constexpr (ROPE) {
+        // a wave takes both column blocks of a 16-row block: element e of a lane is column n0 + 4 g + e and its partner
+        for (int mb = wave; mb < MB; mb += WAVES) {
+            const int m = 16 * mb + r;
+            float rstd = 1.0f;
+            if constexpr (RMS) {
+                float t = 0.0f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) t += red_sq[w][mb][r];
+                rstd = 1.0f / sqrtf(t / (float)K + eps);
+            }
+            const int64_t trow = (int64_t)(min(m, M - 1) / ex.rows_per_batch) * ex.t_bs + (int64_t)(min(m, M - 1) % ex.rows_per_batch) * ex.t_ss;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = n0 + 4 * g + e;   // lower member of the pair; the upper one is `half` columns further
+                float v[2];
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    float t4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int w = 0; w < WAVES; ++w) t4[w & 3] += red[w][a * MB + mb][lane][e];
+                    v[a] = ((t4[0] + t4[1]) + (t4[2] + t4[3])) * rstd;
+                }
+                if (m >= M || n >= N) continue;
+                if (bias != nullptr) {
+                    v[0] += to_float(bias[n]);
+                    v[1] += to_float(bias[n + ex.half]);
+                }
+                float y0 = v[0], y1 = v[1];
+                if (n < ex.rope_cols) {
+                    const int d = n % (2 * ex.half);
+                    const float c0 = table_value(ex.cos, ex.table_dtype, trow + d), s0 = table_value(ex.sin, ex.table_dtype, trow + d);
+                    const float c1 = table_value(ex.cos, ex.table_dtype, trow + d + ex.half);
+                    const float s1 = table_value(ex.sin, ex.table_dtype, trow + d + ex.half);
+                    y0 = v[0] * c0 - v[1] * s0;
+                    y1 = v[1] * c1 + v[0] * s1;
+                }
+                if (ex.residual != nullptr) {
+                    const T *res = static_cast<const T *>(ex.residual) + (int64_t)m * ex.res_rs;
+                    y0 += to_float(res[(int64_t)n * ex.res_cs]);
+                    y1 += to_float(res[(int64_t)(n + ex.half) * ex.res_cs]);
+                }
+                out[(int64_t)m * out_rs + (int64_t)n * out_cs] = from_float<T>(y0);
+                out[(int64_t)m * out_rs + (int64_t)(n + ex.half) * out_cs] = from_float<T>(y1);
+            }
+        }
+        return;
+    }
+    for (int unit = wave; unit < NR * MB; unit += WAVES) {
+        const int rb = unit / MB, mb = unit % MB;
+        const int nb = n0 + 16 * rb;
+        const int m = 16 * mb + r;
+        float rstd = 1.0f;
+        if constexpr (RMS) {
+            float t = 0.0f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) t += red_sq[w][mb][r];
+            rstd = 1.0f / sqrtf(t / (float)K + eps);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int n = nb + 4 * g + e;
+            float v[NA];
+#pragma unroll
+            for (int a = 0; a < NA; ++a) {
+                float t4[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // fixed summation order: the result does not depend on timing
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) t4[w & 3] += red[w][(rb * NA + a) * MB + mb][lane][e];
+                v[a] = ((t4[0] + t4[1]) + (t4[2] + t4[3])) * rstd;
+            }
+            if (m >= M || n >= N) continue;
+            if (bias != nullptr) {
+                const int brow = GATED ? gated_row(nb) + 4 * g + e : n;
+                v[0] += to_float(bias[brow]);
+                if (GATED) v[NA - 1] += to_float(bias[brow + 32]);
+            }
+            if (!GATED && act_in != nullptr) act_in[(int64_t)m * ai_rs + (int64_t)n * ai_cs] = from_float<T>(v[0]);
+            float y = apply_act16(v[0], act);
+            if (GATED) y *= v[NA - 1];
+            if (ex.residual != nullptr)
+                y += to_float(static_cast<const T *>(ex.residual)[(int64_t)m * ex.res_rs + (int64_t)n * ex.res_cs]);
+            out[(int64_t)m * out_rs + (int64_t)n * out_cs] = from_float<T>(y);
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------------
+// FMA kernel: any dtype, any strides.  64x64 output tile, 16x16 threads, 4x4 outputs per thread, fp32 LDS tiles.
+// ----------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+linear_fma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
+                  T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t x_rs, int64_t x_cs,
+                  int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int act) {
+    __shared__ float xs[16][64 + 1];
+    __shared__ float ws[16][64 + 1];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        for (int e = threadIdx.x; e < 64 * 16; e += 256) {
+            const int r = e >> 4, kk = e & 15;
+            const int gm = m0 + r, gn = n0 + r, gk = k0 + kk;
+            xs[kk][r] = (gm < M && gk < K) ? to_float(X[(int64_t)gm * x_rs + (int64_t)gk * x_cs]) : 0.0f;
+            ws[kk][r] = (gn < N && gk < K) ? to_float(W[(int64_t)gn * K + gk]) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = xs[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = ws[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += a[i] * b[j];
+        }
+        __syncthreads();
+    }
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= N) continue;
+            float r = acc[i][j];
+            if (bias != nullptr) r += to_float(bias[n]);
+            if (act_in != nullptr) act_in[(int64_t)m * ai_rs + (int64_t)n * ai_cs] = from_float<T>(r);
+            out[(int64_t)m * out_rs + (int64_t)n * out_cs] = from_float<T>(apply_act(r, act));
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------------
+// host dispatch
+// ----------------------------------------------------------------------------------------------------
+struct LinearArgs {
+    const void *x, *w, *bias;
+    void *out, *act_in;
+    int M, N, K;
+    int64_t x_rs, x_cs, out_rs, out_cs, ai_rs, ai_cs;
+    int act;
+    hipStream_t st;
+    const SkinnyExtra *extra = nullptr;  // residual / rotation of the few-row kernel (decoding steps)
+};
+
+template <typename T, typename Cfg, int ACT, bool W8 = false>
+static void launch_mfma_act(const LinearArgs &a) {
+    auto kern = linear_mfma_kernel<T, Cfg, ACT, W8>;
+    static bool attr_done = false;  // benign race: the attribute call is idempotent
+    if (!attr_done) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+        attr_done = true;
+    }
+    const int tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
+    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+    const T *x = static_cast<const T *>(a.x);
+    const T *w = static_cast<const T *>(a.w);
+    const T *bias = static_cast<const T *>(a.bias);
+    T *out = static_cast<T *>(a.out);
+    T *act_in = static_cast<T *>(a.act_in);
+    const int out_vec_ok = a.out_cs == 1 && a.out_rs % 8 == 0 && aligned16(out);
+    const int ai_vec_ok = act_in != nullptr && a.ai_cs == 1 && a.ai_rs % 8 == 0 && aligned16(act_in);
+    const int bias_vec_ok = bias != nullptr && aligned16(bias);
+    hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(Cfg::THREADS), Cfg::LDS_BYTES, a.st, x, w, bias, out,
+                       act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs, a.ai_cs, tiles_m, tiles_n,
+                       out_vec_ok, ai_vec_ok, bias_vec_ok);
+}
+
+template <typename T, typename Cfg>
+static void launch_mfma_cfg(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_mfma_act<T, Cfg, KERNL_ACT_RELU>(a); break;
+        case KERNL_ACT_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_TANH>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_ERF>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_mfma_act<T, Cfg, KERNL_ACT_GELU_TANH>(a); break;
+        case KERNL_ACT_SILU: launch_mfma_act<T, Cfg, KERNL_ACT_SILU>(a); break;
+        default: launch_mfma_act<T, Cfg, KERNL_ACT_NONE>(a); break;
+    }
+}
+
+// one-byte weights (fp16 activations)
+template <typename Cfg>
+static void launch_mfma_w8(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_mfma_act<f16, Cfg, KERNL_ACT_RELU, true>(a); break;
+        case KERNL_ACT_TANH: launch_mfma_act<f16, Cfg, KERNL_ACT_TANH, true>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_mfma_act<f16, Cfg, KERNL_ACT_GELU_ERF, true>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_mfma_act<f16, Cfg, KERNL_ACT_GELU_TANH, true>(a); break;
+        case KERNL_ACT_SILU: launch_mfma_act<f16, Cfg, KERNL_ACT_SILU, true>(a); break;
+        default: launch_mfma_act<f16, Cfg, KERNL_ACT_NONE, true>(a); break;
+    }
+}
+
+// gated epilogues: tiles whose waves span an even number of 32-column blocks
+template <typename T, typename Cfg>
+static void launch_mfma_glu(const LinearArgs &a) {
+    switch (a.act & (kGluBit - 1)) {
+        case KERNL_ACT_GELU_ERF: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_GELU_ERF>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_GELU_TANH>(a); break;
+        case KERNL_ACT_RELU: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_RELU>(a); break;
+        case KERNL_ACT_NONE: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_NONE>(a); break;
+        case KERNL_ACT_TANH: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_TANH>(a); break;
+        default: launch_mfma_act<T, Cfg, kGluBit | KERNL_ACT_SILU>(a); break;
+    }
+}
+
+template <typename T, int ACT, int NBN = 8, bool W8 = false>
+static void launch_wide_act(const LinearArgs &a) {
+    auto kern = linear_wide_kernel<T, ACT, NBN, W8>;
+    constexpr int LDS_BYTES = 2 * (256 + 256) * 128;
+    static bool attr_done = false;  // benign race: the attribute call is idempotent
+    if (!attr_done) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        attr_done = true;
+    }
+    const int tiles_m = (a.M + 255) / 256, tiles_n = (a.N + 32 * NBN - 1) / (32 * NBN);
+    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+    const T *bias = static_cast<const T *>(a.bias);
+    T *out = static_cast<T *>(a.out);
+    T *act_in = static_cast<T *>(a.act_in);
+    const int out_vec_ok = a.out_cs == 1 && a.out_rs % 8 == 0 && aligned16(out);
+    const int ai_vec_ok = act_in != nullptr && a.ai_cs == 1 && a.ai_rs % 8 == 0 && aligned16(act_in);
+    const int bias_vec_ok = bias != nullptr && aligned16(bias);
+    // persistent: at most one workgroup per CU (32 per XCD), each walks its share of the XCD's tiles.  The kernel
+    // needs every tile to start in LDS stage 0: with an odd number of k-tiles each workgroup gets a single tile.
+    const int slots = (per_xcd < 32 || (a.K / 64) % 2 != 0) ? per_xcd : 32;
+    hipLaunchKernelGGL(kern, dim3(slots * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
+                       static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
+                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok);
+}
+
+template <typename T, int ACT, int NBN, bool W8>
+static void launch_wide_half_act(const LinearArgs &a);
+
+template <typename T, int ACT, int NBN, bool W8 = false>
+static void launch_wide_half_act(const LinearArgs &a) {
+    auto kern = linear_wide_half_kernel<T, ACT, NBN, W8>;
+    constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768;
+    static bool attr_done = false;  // benign race: the attribute call is idempotent
+    if (!attr_done) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        attr_done = true;
+    }
+    const int tiles_m = (a.M + 127) / 128, tiles_n = (a.N + 32 * NBN - 1) / (32 * NBN);
+    const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+    const T *bias = static_cast<const T *>(a.bias);
+    T *out = static_cast<T *>(a.out);
+    T *act_in = static_cast<T *>(a.act_in);
+    const int out_vec_ok = a.out_cs == 1 && a.out_rs % 8 == 0 && aligned16(out);
+    const int ai_vec_ok = act_in != nullptr && a.ai_cs == 1 && a.ai_rs % 8 == 0 && aligned16(act_in);
+    const int bias_vec_ok = bias != nullptr && aligned16(bias);
+    hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
+                       static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
+                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, static_cast<float *>(nullptr), 1);
+}
+
+// Split form of the 128 x 192 kernel for row counts that leave most CUs without a tile (129 to about 700 rows against
+// a few thousand columns): `splits` ranges of k-tiles per output tile, then the launch that adds them.
+struct HalfSplitPlan {
+    int tiles_m, tiles_n, splits;
+    int64_t bytes;
+};
+static HalfSplitPlan half_split_plan(int64_t M, int64_t N, int64_t K) {
+    HalfSplitPlan p;
+    p.tiles_m = (int)((M + 127) / 128);
+    p.tiles_n = (int)((N + 191) / 192);
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    const int nk = (int)(K / 64);
+    int64_t splits = 256 / tiles;           // one round of workgroups
+    if (splits > nk / 16) splits = nk / 16; // ranges of at least 16 k-tiles: with K = 768 two ranges cost more (14 us) than one tile pass (11)
+    if (splits > 4) splits = 4;             // partial tiles cost HBM traffic: rows x columns x 8 bytes per range
+    if (splits < 1) splits = 1;
+    // ranges of ceil(nk / splits) k-tiles: drop ranges that would be empty
+    const int per = (nk + (int)splits - 1) / (int)splits;
+    p.splits = (nk + per - 1) / per;
+    p.bytes = p.splits > 1 ? (int64_t)p.splits * tiles * 128 * 192 * 4 : 0;
+    return p;
+}
+
+template <typename T, int ACT>
+static void launch_half_split_act(const LinearArgs &a, const HalfSplitPlan &p, float *part) {
+    constexpr int NBN = 6;
+    auto kern = linear_wide_half_kernel<T, KERNL_ACT_NONE, NBN, false, true>;
+    constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768;
+    static bool attr_done = false;  // benign race: the attribute call is idempotent
+    if (!attr_done) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        attr_done = true;
+    }
+    const int per_xcd = (p.tiles_m * p.tiles_n + 7) / 8;
+    const T *bias = static_cast<const T *>(a.bias);
+    T *out = static_cast<T *>(a.out);
+    T *act_in = static_cast<T *>(a.act_in);
+    const int out_vec_ok = a.out_cs == 1 && a.out_rs % 8 == 0 && aligned16(out);
+    const int ai_vec_ok = act_in != nullptr && a.ai_cs == 1 && a.ai_rs % 8 == 0 && aligned16(act_in);
+    const int bias_vec_ok = bias != nullptr && aligned16(bias);
+    hipLaunchKernelGGL(kern, dim3(per_xcd * 8, p.splits), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
+                       static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
+                       a.ai_cs, p.tiles_m, p.tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, part, p.splits);
+    hipLaunchKernelGGL((linear_wide_half_reduce_kernel<T, ACT, NBN>), dim3(p.tiles_m * p.tiles_n, 4), dim3(256), 0, a.st,
+                       part, bias, out, act_in, a.M, a.N, a.out_rs, a.out_cs, a.ai_rs, a.ai_cs, p.tiles_m, p.tiles_n,
+                       out_vec_ok, ai_vec_ok, bias_vec_ok, p.splits);
+}
+
+template <typename T>
+static void launch_half_split(const LinearArgs &a, const HalfSplitPlan &p, float *part) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_half_split_act<T, KERNL_ACT_RELU>(a, p, part); break;
+        case KERNL_ACT_TANH: launch_half_split_act<T, KERNL_ACT_TANH>(a, p, part); break;
+        case KERNL_ACT_GELU_ERF: launch_half_split_act<T, KERNL_ACT_GELU_ERF>(a, p, part); break;
+        case KERNL_ACT_GELU_TANH: launch_half_split_act<T, KERNL_ACT_GELU_TANH>(a, p, part); break;
+        case KERNL_ACT_SILU: launch_half_split_act<T, KERNL_ACT_SILU>(a, p, part); break;
+        default: launch_half_split_act<T, KERNL_ACT_NONE>(a, p, part); break;
+    }
+}
+
+template <typename T, int NBN>
+static void launch_wide_half(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_wide_half_act<T, KERNL_ACT_RELU, NBN>(a); break;
+        case KERNL_ACT_TANH: launch_wide_half_act<T, KERNL_ACT_TANH, NBN>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_wide_half_act<T, KERNL_ACT_GELU_ERF, NBN>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_wide_half_act<T, KERNL_ACT_GELU_TANH, NBN>(a); break;
+        case KERNL_ACT_SILU: launch_wide_half_act<T, KERNL_ACT_SILU, NBN>(a); break;
+        default: launch_wide_half_act<T, KERNL_ACT_NONE, NBN>(a); break;
+    }
+}
+
+template <typename T>
+static void launch_wide192(const LinearArgs &a) {
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_wide_act<T, KERNL_ACT_RELU, 6>(a); break;
+        case KERNL_ACT_TANH: launch_wide_act<T, KERNL_ACT_TANH, 6>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_wide_act<T, KERNL_ACT_GELU_ERF, 6>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_wide_act<T, KERNL_ACT_GELU_TANH, 6>(a); break;
+        case KERNL_ACT_SILU: launch_wide_act<T, KERNL_ACT_SILU, 6>(a); break;
+        default: launch_wide_act<T, KERNL_ACT_NONE, 6>(a); break;
+    }
+}
+
+template <typename T>
+static void launch_wide(const LinearArgs &a) {
+    if (a.act & kGluBit) {
+        switch (a.act & (kGluBit - 1)) {
+            case KERNL_ACT_GELU_ERF: launch_wide_act<T, kGluBit | KERNL_ACT_GELU_ERF>(a); break;
+            case KERNL_ACT_GELU_TANH: launch_wide_act<T, kGluBit | KERNL_ACT_GELU_TANH>(a); break;
+            case KERNL_ACT_RELU: launch_wide_act<T, kGluBit | KERNL_ACT_RELU>(a); break;
+            case KERNL_ACT_NONE: launch_wide_act<T, kGluBit | KERNL_ACT_NONE>(a); break;
+            case KERNL_ACT_TANH: launch_wide_act<T, kGluBit | KERNL_ACT_TANH>(a); break;
+            default: launch_wide_act<T, kGluBit | KERNL_ACT_SILU>(a); break;
+        }
+        return;
+    }
+    switch (a.act) {
+        case KERNL_ACT_RELU: launch_wide_act<T, KERNL_ACT_RELU>(a); break;
+        case KERNL_ACT_TANH: launch_wide_act<T, KERNL_ACT_TANH>(a); break;
+        case KERNL_ACT_GELU_ERF: launch_wide_act<T, KERNL_ACT_GELU_ERF>(a); break;
+        case KERNL_ACT_GELU_TANH: launch_wide_act<T, KERNL_ACT_GELU_TANH>(a); break;
+        case KERNL_ACT_SILU: launch_wide_act<T, KERNL_ACT_SILU>(a); break;
+        default: launch_wide_act<T, KERNL_ACT_NONE>(a); break;
+    }
+}
+
+//                         BM   BN  BK  WAVES_M WAVES_N  MIN_BLOCKS
+typedef LinearTile<256, 256, 64, 2, 4, 1> Tile256x256;
+typedef LinearTile<256, 192, 64, 4, 2, 1> Tile256x192;
+typedef LinearTile<128, 128, 64, 2, 2, 2> Tile128x128;
+typedef LinearTile<256, 128, 32, 2, 2, 2> Tile256x128k32;  // 48 KB of LDS: two workgroups per CU
+
+// Run-time proxy of a tile shape: tiles one CU has to work through, times the tile's area relative to 256x256, times
+// a speed factor of the kernel that runs it (measured on the Llama-7B and BERT-base shapes: the wide kernel's k-loop is
+// the fastest, and the longer K is the more the 8-wave kernels fall behind it).
+static double tile_cost(int M, int N, int K, int bm, int bn, double base, double per_k) {
+    const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    const int64_t per_cu = (tiles + 255) / 256;
+    const double kf = (double)K / ((double)K + 1500.0);
+    return (double)per_cu * ((double)bm * bn / 65536.0) * (base + per_k * kf);
+}
+// which: 1 = 256x256, 2 = 256x192, 3 = 128x128 (8-wave kernel), 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192 (K % 64 == 0)
+static int pick_tile(int M, int N, int K, bool gated) {
+    int pick = 1;
+    double best = tile_cost(M, N, K, 256, 256, 1.15, 0.3);
+    if (K % 64 == 0) {
+        best = tile_cost(M, N, K, 256, 256, 1.0, 0.0);
+        pick = 5;
+        const double c6 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.04, 0.0);
+        if (c6 < best) { best = c6; pick = 6; }
+        // half-height tiles: a quarter slower per output element at long K (more operand traffic per MFMA), and a
+        // prologue per tile that weighs more the shorter K is; they win where 256-row tiles leave CUs idle
+        const double c7 = gated ? 1e30 : tile_cost(M, N, K, 128, 256, 1.5, -0.35);
+        if (c7 < best) { best = c7; pick = 7; }
+        const double c8 = gated ? 1e30 : tile_cost(M, N, K, 128, 192, 1.65, -0.35);
+        if (c8 < best) { best = c8; pick = 8; }
+    }
+    // 256x192 gives a wave an odd number of column blocks: not usable for gate/value pairs
+    const double c2 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.2, 0.3);
+    const double c3 = tile_cost(M, N, K, 128, 128, 1.9, 0.4);
+    if (c2 < best) { best = c2; pick = 2; }
+    if (c3 < best) { best = c3; pick = 3; }
+    return pick;
+}
+
+extern int g_linear_force_tile;  // test / tuning hook (defined in linear.hip): 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192
+
+template <typename T, bool GATED, int MB, int NR, bool W8, bool RMS = false, bool ROPE = false>
+static void launch_skinny_blocks(const LinearArgs &a, const void *rms_w = nullptr, float eps = 0.0f,
+                                 const SkinnyExtra *extra = nullptr) {
+    const int n_out = GATED ? a.N / 2 : a.N;
+    const dim3 grid((unsigned)((n_out + 16 * NR - 1) / (16 * NR)));  // the rotating form: N is a multiple of the head size
+    SkinnyExtra ex = {};
+    if (extra != nullptr) ex = *extra;
+    else if (a.extra != nullptr) ex = *a.extra;
+    const int act = a.act & (kGluBit - 1);
+    // waves per workgroup: enough to have a whole block of weight rows in flight when K is long, never more than
+    // there are chunks, and no more than the LDS for their partial sums allows
+    const int nchunks = a.K / 64;
+    // (the normalising form also keeps a few more loads per chunk in flight: half the waves for it)
+    constexpr int kUnits = (GATED ? 2 : 1) * NR * MB * (RMS ? 2 : 1);
+    constexpr int kMaxWaves = kUnits > 8 ? 4 : kUnits > 4 ? 8 : 16;
+    // ... and few enough that the workgroups one CU gets (256 CUs) are resident together: a 1024-thread workgroup
+    // fills half a CU, and 344 of them would leave a third of the chip idle
+    const int per_cu = ((int)grid.x + 255) / 256;
+    int waves = nchunks >= 64 ? 16 : nchunks >= 24 ? 8 : 4;
+    if (per_cu >= 3) waves = 4;
+    else if (per_cu == 2 && waves > 8) waves = 8;
+#define KERNL_SKINNY(WV)                                                                                                \
+    hipLaunchKernelGGL((linear_skinny_kernel<T, MB, GATED, WV, NR, W8, RMS, ROPE>), grid, dim3(64 * WV), 0, a.st,                \
+                       static_cast<const T *>(a.x), static_cast<const T *>(a.w), static_cast<const T *>(a.bias),       \
+                       static_cast<T *>(a.out), static_cast<T *>(a.act_in), a.M, n_out, a.K, a.x_rs, a.out_rs, a.out_cs, \
+                       a.ai_rs, a.ai_cs, act, static_cast<const T *>(rms_w), eps, ex)
+    if constexpr (kMaxWaves >= 16) {
+        if (waves >= 16) { KERNL_SKINNY(16); return; }
+    }
+    if constexpr (kMaxWaves >= 8) {
+        if (waves >= 8) { KERNL_SKINNY(8); return; }
+    }
+    KERNL_SKINNY(4);
+#undef KERNL_SKINNY
+}
+
+template <typename T, bool GATED, bool W8 = false>
+static void launch_skinny(const LinearArgs &a) {
+    const int n_out = GATED ? a.N / 2 : a.N;
+    const int mb = (a.M + 15) / 16;
+    // every workgroup reads all of x (from L2), so more output columns per workgroup mean less of that traffic.
+    // Gated and one-byte weights: with more than 16 rows of x and enough output columns to fill the chip twice over,
+    // a workgroup takes 32 columns
+    const bool two = n_out >= 8192 && mb >= 2;
+    if constexpr (!W8 && !GATED) {
+        // 16-bit plain weights, 8 rows of x or more (measured at 8..64 rows, 4096..32000 columns): as few 16-column
+        // blocks per workgroup as put the whole grid on the chip at once, one workgroup per CU — 11008 columns in
+        // blocks of 48 are 230 workgroups, where blocks of 32 leave 88 CUs with two workgroups and the rest with one;
+        // grids that do not fit either way take 32 columns, 64 with more than 48 rows
+        int nr = 1;
+        if (a.M >= 8) {
+            nr = (n_out + 16 * 256 - 1) / (16 * 256);
+            if (nr > 4) nr = mb >= 4 ? 4 : 2;
+        }
+#define KERNL_SKINNY_NR(NRV)                                            \
+    do {                                                                \
+        if (mb <= 1) launch_skinny_blocks<T, GATED, 1, NRV, W8>(a);      \
+        else if (mb <= 2) launch_skinny_blocks<T, GATED, 2, NRV, W8>(a); \
+        else launch_skinny_blocks<T, GATED, 4, NRV, W8>(a);              \
+    } while (0)
+        if (nr == 1) KERNL_SKINNY_NR(1);
+        else if (nr == 2) KERNL_SKINNY_NR(2);
+        else if (nr == 3) KERNL_SKINNY_NR(3);
+        else KERNL_SKINNY_NR(4);
+#undef KERNL_SKINNY_NR
+        return;
+    }
+    if constexpr (GATED && !W8) {
+        // gated 16-bit weights, 8..32 rows of x: the same rule (measured: 11008 gate/value pairs against K = 4096 at
+        // 32 rows 48 -> 34 us, 13824 against 5120 65 -> 56 us); more rows do not leave the LDS for 48 columns
+        const int nr = (n_out + 16 * 256 - 1) / (16 * 256);
+        if (a.M >= 8 && mb <= 2 && nr >= 3 && nr <= 4) {
+            if (nr == 3) { if (mb <= 1) launch_skinny_blocks<T, GATED, 1, 3, W8>(a); else launch_skinny_blocks<T, GATED, 2, 3, W8>(a); }
+            else { if (mb <= 1) launch_skinny_blocks<T, GATED, 1, 4, W8>(a); else launch_skinny_blocks<T, GATED, 2, 4, W8>(a); }
+            return;
+        }
+    }
+    if (mb <= 1) { if (two) launch_skinny_blocks<T, GATED, 1, 2, W8>(a); else launch_skinny_blocks<T, GATED, 1, 1, W8>(a); }
+    else if (mb <= 2) { if (two) launch_skinny_blocks<T, GATED, 2, 2, W8>(a); else launch_skinny_blocks<T, GATED, 2, 1, W8>(a); }
+    else { if (two) launch_skinny_blocks<T, GATED, 4, 2, W8>(a); else launch_skinny_blocks<T, GATED, 4, 1, W8>(a); }
+}
+
+// RMS-normalised input: 16 output columns per workgroup, 16-bit weights
+template <typename T, bool GATED>
+static void launch_skinny_rms(const LinearArgs &a, const void *rms_w, float eps) {
+    const int mb = (a.M + 15) / 16;
+    if (mb <= 1) launch_skinny_blocks<T, GATED, 1, 1, false, true>(a, rms_w, eps);
+    else if (mb <= 2) launch_skinny_blocks<T, GATED, 2, 1, false, true>(a, rms_w, eps);
+    else launch_skinny_blocks<T, GATED, 4, 1, false, true>(a, rms_w, eps);
+}
+
+// decoding-step projection with optional RMSNorm prologue, rotary epilogue and residual (plain 16-bit weights)
+template <typename T>
+static void launch_skinny_decode(const LinearArgs &a, const void *rms_w, float eps, const SkinnyExtra &ex) {
+    const int mb = (a.M + 15) / 16;
+    if (ex.half > 0) {  // rotating form: two column blocks per workgroup, always with the normalising prologue
+        if (mb <= 1) launch_skinny_blocks<T, false, 1, 2, false, true, true>(a, rms_w, eps, &ex);
+        else if (mb <= 2) launch_skinny_blocks<T, false, 2, 2, false, true, true>(a, rms_w, eps, &ex);
+        else launch_skinny_blocks<T, false, 4, 2, false, true, true>(a, rms_w, eps, &ex);
+    } else if (rms_w != nullptr) {
+        if (mb <= 1) launch_skinny_blocks<T, false, 1, 1, false, true>(a, rms_w, eps, &ex);
+        else if (mb <= 2) launch_skinny_blocks<T, false, 2, 1, false, true>(a, rms_w, eps, &ex);
+        else launch_skinny_blocks<T, false, 4, 1, false, true>(a, rms_w, eps, &ex);
+    } else {
+        LinearArgs b = a;  // the plain kernel with its own grid rule; the residual travels in the arguments
+        b.extra = &ex;
+        launch_skinny<T, false>(b);
+    }
+}
+
+}  // namespace kernl

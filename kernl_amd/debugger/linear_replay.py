@@ -1,4 +1,4 @@
-"""Checks of the wide linear kernel's weight placement (csrc/linear.hip, `wide_weight_row`): LDS row `row` of a weight
+"""Checks of the wide linear kernel's weight placement (csrc/linear_kernels.h; `wide_weight_row` in csrc/index_math.h): LDS row `row` of a weight
 tile feeds MFMA row row % 16 of 16-row block row / 16, and carries a weight row chosen so that the four-element
 results of a lane line up as consecutive output columns."""
 from typing import Dict, List
