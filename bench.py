@@ -116,6 +116,14 @@ def main():
         "each, every launch after a 256 MB cache flush, and exit: the workload of the rocprofv3 --kernel-trace run "
         "behind the *_cold_us figures (profiles/bench_cold_kernel_trace.txt)",
     )
+    ap.add_argument(
+        "--decode-probe",
+        action="store_true",
+        help="launch the four projections of a Llama-7B layer's batched decoding step (32 and 64 sequences; norm + QKV + "
+        "rotation, output + residual, norm + gate/up, down + residual) and a 256 x 4096 x 4096 product 20 times each "
+        "over rotating weights, and exit: the workload of the rocprofv3 --kernel-trace run behind "
+        "profiles/linear_batched_decode_kernel_trace.txt",
+    )
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU per process and ships no multi-GPU path; run with --gpus 1")
@@ -152,6 +160,34 @@ def main():
         dst = torch.empty_like(src)
         for _ in range(3):
             dst.copy_(src)
+        torch.cuda.synchronize()
+        return
+
+    if args.decode_probe:
+        from kernl_amd.implementations.linear_layer import decode_linear_layer, rms_linear_layer
+
+        gen = torch.Generator().manual_seed(0)
+        heads, hd, width, ffn = 32, 128, 4096, 11008
+
+        def weights(n, k, count):
+            return [(torch.randn((n, k), generator=gen) * k ** -0.5).half().to(dev) for _ in range(count)]
+
+        w_qkv, w_o, w_gu, w_dn = weights(3 * width, width, 4), weights(width, width, 8), weights(2 * ffn, width, 3), weights(width, ffn, 4)
+        norm_w = torch.ones(width, dtype=torch.half, device=dev)
+        for batch in (32, 64):
+            x = torch.randn((batch, 1, width), generator=gen).half().to(dev)
+            xf = torch.randn((batch, 1, ffn), generator=gen).half().to(dev)
+            res = torch.randn((batch, 1, width), generator=gen).half().to(dev)
+            ang = torch.rand((batch, 1, hd), generator=gen) * 6.28
+            cos, sin = ang.cos().half().to(dev), ang.sin().half().to(dev)
+            for i in range(20):
+                decode_linear_layer(x, w_qkv[i % 4], None, norm_w, 1e-5, None, cos, sin, head_dim=hd, rope_cols=2 * heads * hd)
+                decode_linear_layer(x, w_o[i % 8], None, residual=res)
+                rms_linear_layer(x, norm_w, 1e-5, w_gu[i % 3], None, "silu", gated=True)
+                decode_linear_layer(xf, w_dn[i % 4], None, residual=res)
+        x256 = torch.randn((256, width), generator=gen).half().to(dev)
+        for i in range(20):
+            linear_layer(x256, w_o[i % 8], None, "")
         torch.cuda.synchronize()
         return
 

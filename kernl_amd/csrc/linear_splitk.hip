@@ -355,43 +355,85 @@ __global__ void __launch_bounds__(256) linear_fewrow_reduce_kernel(const FewRowA
     const int w_first = (tile * nch) / run, w_last = ((tile + 1) * nch - 1) / run;   // units fit 31 bits
     const int n_slots = w_last - w_first + 1;
     const float4 *theirs = reinterpret_cast<const float4 *>(a.part) + ((int64_t)w_first + tile) * TILE_ELEMS + e0;
-    auto slot_sum = [&](const float4 *src) __attribute__((always_inline)) -> f32x4_acc {
-        f32x4_acc acc = {0.0f, 0.0f, 0.0f, 0.0f};
-        int s = 0;
-        for (; s + 4 <= n_slots; s += 4) {   // four loads in flight, added in workgroup order
-            float4 v[4];
+    // Every load of this thread is requested before the first one is used: the kernel is a chain of memory round trips
+    // otherwise (partial tiles, the norm's row sums, tables), and it is all latency.
+    const float4 *partner = theirs + pair_waves * MB * 64;
+    f32x4_acc acc = {0.0f, 0.0f, 0.0f, 0.0f}, other = {0.0f, 0.0f, 0.0f, 0.0f};
+    float4 pv[4], qv[4];
+    const int first = min(n_slots, 4);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = src[(int64_t)(s + u) * TILE_ELEMS];
+    for (int u = 0; u < 4; ++u) {   // (slots past the last one fetch it again: no branch around a load)
+        const int64_t slot = (int64_t)min(u, n_slots - 1) * TILE_ELEMS;
+        pv[u] = theirs[slot];
+        if (MODE != kFewRowPlain) qv[u] = partner[slot];
+    }
+    float sq_sum = 0.0f;
+    if (a.rms_w != nullptr) {
+        const int w_sq_last = (nch - 1) / run;
+        for (int w = 0; w <= w_sq_last; ++w) sq_sum += a.sqpart[(int64_t)w * kFewRowMaxRows + m];
+    }
+    const bool rotate = MODE == kFewRowRope && n < a.rope_cols;   // rope_cols is a multiple of the head size, n of 4
+    float tc[2][4], ts[2][4];   // cos / sin of the four columns and of their partners
+    if (MODE == kFewRowRope && rotate) {
+        const int d = n % (2 * a.half);
+        const int64_t trow = (int64_t)(m / a.rows_per_batch) * a.t_bs + (int64_t)(m % a.rows_per_batch) * a.t_ss + d;
+        const bool vec = ((a.t_bs | a.t_ss) & 3) == 0 && ((reinterpret_cast<uintptr_t>(a.cos) | reinterpret_cast<uintptr_t>(a.sin)) & 15) == 0;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                acc[0] += v[u].x;
-                acc[1] += v[u].y;
-                acc[2] += v[u].z;
-                acc[3] += v[u].w;
+        for (int h = 0; h < 2; ++h) {
+            const int64_t off = trow + h * a.half;
+            if (vec && a.table_dtype == KERNL_F32) {
+                const float4 c = *reinterpret_cast<const float4 *>(static_cast<const float *>(a.cos) + off);
+                const float4 sn = *reinterpret_cast<const float4 *>(static_cast<const float *>(a.sin) + off);
+                tc[h][0] = c.x; tc[h][1] = c.y; tc[h][2] = c.z; tc[h][3] = c.w;
+                ts[h][0] = sn.x; ts[h][1] = sn.y; ts[h][2] = sn.z; ts[h][3] = sn.w;
+            } else if (vec && a.table_dtype == KERNL_F16) {
+                const f16x4 c = *reinterpret_cast<const f16x4 *>(static_cast<const f16 *>(a.cos) + off);
+                const f16x4 sn = *reinterpret_cast<const f16x4 *>(static_cast<const f16 *>(a.sin) + off);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    tc[h][e] = (float)c[e];
+                    ts[h][e] = (float)sn[e];
+                }
+            } else if (vec && a.table_dtype == KERNL_BF16) {
+                const bf16x4 c = *reinterpret_cast<const bf16x4 *>(static_cast<const bf16 *>(a.cos) + off);
+                const bf16x4 sn = *reinterpret_cast<const bf16x4 *>(static_cast<const bf16 *>(a.sin) + off);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    tc[h][e] = (float)c[e];
+                    ts[h][e] = (float)sn[e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    tc[h][e] = table_value(a.cos, a.table_dtype, off + e);
+                    ts[h][e] = table_value(a.sin, a.table_dtype, off + e);
+                }
             }
         }
-        for (; s < n_slots; ++s) {
-            const float4 v = src[(int64_t)s * TILE_ELEMS];
-            acc[0] += v.x;
-            acc[1] += v.y;
-            acc[2] += v.z;
-            acc[3] += v.w;
-        }
-        return acc;
-    };
-    f32x4_acc acc = slot_sum(theirs);
-    float rstd = 1.0f;
-    if (a.rms_w != nullptr) {
-        float t = 0.0f;
-        const int w_sq_last = (nch - 1) / run;
-        for (int w = 0; w <= w_sq_last; ++w) t += a.sqpart[(int64_t)w * kFewRowMaxRows + m];
-        rstd = 1.0f / sqrtf(t / (float)a.K + a.eps);
     }
+    // add in workgroup order: the slots requested above, then any further ones four at a time
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        if (u < first) {
+            acc[0] += pv[u].x; acc[1] += pv[u].y; acc[2] += pv[u].z; acc[3] += pv[u].w;
+            if (MODE != kFewRowPlain) {
+                other[0] += qv[u].x; other[1] += qv[u].y; other[2] += qv[u].z; other[3] += qv[u].w;
+            }
+        }
+    }
+    for (int s = 4; s < n_slots; ++s) {
+        const float4 v = theirs[(int64_t)s * TILE_ELEMS];
+        acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+        if (MODE != kFewRowPlain) {
+            const float4 o = partner[(int64_t)s * TILE_ELEMS];
+            other[0] += o.x; other[1] += o.y; other[2] += o.z; other[3] += o.w;
+        }
+    }
+    const float rstd = a.rms_w != nullptr ? 1.0f / sqrtf(sq_sum / (float)a.K + a.eps) : 1.0f;
     if (MODE == kFewRowPlain) {
         fewrow_epilogue<T>(acc, rstd, m, n, a);
         return;
     }
-    const f32x4_acc other = slot_sum(theirs + pair_waves * MB * 64);
     const T *bias = static_cast<const T *>(a.bias);
     T *out = static_cast<T *>(a.out);
     const T *residual = static_cast<const T *>(a.residual);
@@ -410,8 +452,6 @@ __global__ void __launch_bounds__(256) linear_fewrow_reduce_kernel(const FewRowA
     }
     // rope: columns n .. n + 3 and their partners `half` further on
     float lo[4], hi[4];
-    const int d = n % (2 * a.half);
-    const int64_t trow = (int64_t)(m / a.rows_per_batch) * a.t_bs + (int64_t)(m % a.rows_per_batch) * a.t_ss;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float v0 = acc[e] * rstd, v1 = other[e] * rstd;
@@ -419,15 +459,8 @@ __global__ void __launch_bounds__(256) linear_fewrow_reduce_kernel(const FewRowA
             v0 += to_float(bias[min(n + e, a.N - 1)]);
             v1 += to_float(bias[min(n + e + a.half, a.N - 1)]);
         }
-        lo[e] = v0;
-        hi[e] = v1;
-        if (n + e < a.rope_cols) {
-            const float c0 = table_value(a.cos, a.table_dtype, trow + d + e), s0 = table_value(a.sin, a.table_dtype, trow + d + e);
-            const float c1 = table_value(a.cos, a.table_dtype, trow + d + e + a.half);
-            const float s1 = table_value(a.sin, a.table_dtype, trow + d + e + a.half);
-            lo[e] = v0 * c0 - v1 * s0;
-            hi[e] = v1 * c1 + v0 * s1;
-        }
+        lo[e] = rotate ? v0 * tc[0][e] - v1 * ts[0][e] : v0;
+        hi[e] = rotate ? v1 * tc[1][e] + v0 * ts[1][e] : v1;
     }
     fewrow_store<T>(lo, m, n, out, a.N, a.out_rs, a.out_cs, residual, a.res_rs, a.res_cs);
     fewrow_store<T>(hi, m, n + a.half, out, a.N, a.out_rs, a.out_cs, residual, a.res_rs, a.res_cs);
