@@ -286,6 +286,15 @@ int kernl_linear_fewrow_fwd(const void *x, const void *rms_weight, float eps, co
                             const int64_t residual_strides[2], const void *cos, const void *sin, int64_t head_dim,
                             int64_t rope_cols, int64_t rows_per_batch, const int64_t table_strides[3], int table_dtype,
                             int activation, int gated, int dtype, void *stream);
+/* The same with the weight stored as fp8 e5m2 bytes (w8 [N, K] or [2N, K] of one byte per element, decoded to fp16 on
+ * its way into the MFMA as in kernl_linear_w8_fwd; reference experimental/llama-v2/kernel/fused_kernel_fp8.py:75-84,
+ * fused_kernel_ff.py:43-47); f16 activations only. */
+int kernl_linear_fewrow_w8_fwd(const void *x, const void *rms_weight, float eps, const void *w8, const void *bias,
+                               const void *residual, void *out, void *workspace, int64_t workspace_bytes, int64_t M,
+                               int64_t N, int64_t K, const int64_t x_strides[2], const int64_t out_strides[2],
+                               const int64_t residual_strides[2], const void *cos, const void *sin, int64_t head_dim,
+                               int64_t rope_cols, int64_t rows_per_batch, const int64_t table_strides[3],
+                               int table_dtype, int activation, int gated, int dtype, void *stream);
 
 /*
  * A decoding step's projection with everything around it in ONE launch (at most 64 rows of x, K % 64 == 0, f16 / bf16,

@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "kernl_linear_splitk_fwd",
     "kernl_linear_fewrow_workspace_bytes",
     "kernl_linear_fewrow_fwd",
+    "kernl_linear_fewrow_w8_fwd",
     "kernl_linear_glu_fwd",
     "kernl_layernorm_fwd",
     "kernl_add_layernorm_fwd",
@@ -124,6 +125,8 @@ def load() -> ctypes.CDLL:
         [_vp, _vp, ctypes.c_float] + [_vp] * 5 + [_i64] * 4 + [_i64p] * 3 + [_vp, _vp] + [_i64] * 3
         + [_i64p] + [ctypes.c_int] * 4 + [_vp]
     )
+    lib.kernl_linear_fewrow_w8_fwd.restype = ctypes.c_int
+    lib.kernl_linear_fewrow_w8_fwd.argtypes = lib.kernl_linear_fewrow_fwd.argtypes
     lib.kernl_linear_rms_fwd.restype = ctypes.c_int
     lib.kernl_linear_rms_fwd.argtypes = (
         [_vp, _vp, ctypes.c_float, _vp, _vp, _vp] + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int] * 3 + [_vp]
@@ -419,10 +422,13 @@ def linear_splitk_fwd(x2d, weight, bias, out2d, act_in2d, activation: int, works
 
 
 def linear_fewrow_supported(x2d, weight) -> bool:
-    """What `kernl_linear_fewrow_fwd` takes: 16-bit rows, at most 64 of them, K a multiple of 64 from 256 on."""
+    """What `kernl_linear_fewrow_fwd` / `_w8_fwd` take: 16-bit rows, at most 128 of them, K a multiple of 64 from 256 on,
+    a weight of the same type or — fp16 rows only — fp8 e5m2 bytes."""
     M, K = x2d.shape
+    one_byte = weight.dtype in (torch.int8, torch.uint8, torch.float8_e5m2)
     return (
-        x2d.dtype in (torch.float16, torch.bfloat16) and weight.dtype == x2d.dtype and 0 < M <= 128
+        x2d.dtype in (torch.float16, torch.bfloat16) and 0 < M <= 128
+        and (weight.dtype == x2d.dtype or (one_byte and x2d.dtype == torch.float16))
         and K % 64 == 0 and K >= 256 and x2d.stride(1) == 1 and x2d.stride(0) % 8 == 0 and x2d.data_ptr() % 16 == 0
         and weight.is_contiguous() and weight.data_ptr() % 16 == 0
     )
@@ -454,8 +460,9 @@ def linear_fewrow_fwd(x2d, weight, bias, residual2d, out2d, activation: int, wor
         tdtype, cptr, sptr = DTYPE_CODE[cos.dtype], cos.data_ptr(), sin.data_ptr()
     else:
         tstrides, tdtype, cptr, sptr = None, KERNL_F32, None, None
+    entry = lib.kernl_linear_fewrow_fwd if weight.element_size() == 2 else lib.kernl_linear_fewrow_w8_fwd
     with torch.cuda.device(x2d.device):
-        st = lib.kernl_linear_fewrow_fwd(
+        st = entry(
             x2d.data_ptr(), None if rms_weight is None else rms_weight.data_ptr(), float(eps), weight.data_ptr(),
             None if bias is None else bias.data_ptr(), None if residual2d is None else residual2d.data_ptr(),
             out2d.data_ptr(), ws_ptr, ws_bytes, M, N, K, _arr(x2d.stride()), _arr(out2d.stride()),

@@ -127,7 +127,9 @@ __device__ __forceinline__ void fewrow_epilogue(const f32x4_acc &acc, float rstd
                     a.res_cs);
 }
 
-template <typename T, int MB, int WAVES, int GC, int RING, bool RMS>
+// W8: the weight is stored as one byte per element, fp8 e5m2 — the upper byte of the fp16 encoding (as in the other
+// linear kernels' W8 forms): a lane's 16 weights of a unit are one 16-byte load, byte-permuted into its two fragments.
+template <typename T, int MB, int WAVES, int GC, int RING, bool RMS, bool W8 = false>
 __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowArgs a) {
     typedef typename Vec8<T>::type vec8;
     static_assert(RING % (2 * GC) == 0, "a round of RING units is a whole number of stage pairs");
@@ -141,7 +143,10 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
     __shared__ __attribute__((aligned(16))) unsigned char xs[2][GC * CHUNK_BYTES];
     __shared__ float rstd_s[MP];
 
-    const T *X = static_cast<const T *>(a.x), *W = static_cast<const T *>(a.w);
+    static_assert(!W8 || std::is_same<T, f16>::value, "one-byte weights are decoded to fp16");
+    typedef typename std::conditional<W8, unsigned char, T>::type WT;   // what a weight element is stored as
+    const T *X = static_cast<const T *>(a.x);
+    const WT *W = static_cast<const WT *>(a.w);
     const int M = a.M, N = a.N, K = a.K, tiles = a.tiles, run = a.run, direct = a.direct;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
@@ -154,17 +159,22 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
     // ---- weights: a ring of RING units per wave.  The request cursor walks the run and stops at its last unit
     // (requests past the end fetch that unit again and are never used): no branch around a load, so the compiler's
     // wait counts are exact and the ring really is in flight.  Columns beyond N repeat the last weight row.
-    vec8 wf[RING][2];
+    vec8 wf[W8 ? 1 : RING][2];
+    u32x4 wraw[W8 ? RING : 1];
     int rq_left = n_units - 1;                  // units the cursor may still advance by
     int rq_tile = first_tile, rq_chunk = first_chunk;
-    auto weight_row = [&](int tile) __attribute__((always_inline)) -> const T * {
+    auto weight_row = [&](int tile) __attribute__((always_inline)) -> const WT * {
         return W + (int64_t)min(tile * (16 * WAVES) + 16 * wave + r, N - 1) * K + 16 * g;
     };
-    const T *wrow = weight_row(rq_tile);
+    const WT *wrow = weight_row(rq_tile);
     auto request_w = [&](int slot) __attribute__((always_inline)) {
-        const T *src = wrow + (int64_t)rq_chunk * 64;
-        wf[slot][0] = *reinterpret_cast<const vec8 *>(src);
-        wf[slot][1] = *reinterpret_cast<const vec8 *>(src + 8);
+        const WT *src = wrow + (int64_t)rq_chunk * 64;
+        if constexpr (W8) {
+            wraw[slot] = *reinterpret_cast<const u32x4 *>(src);
+        } else {
+            wf[slot][0] = *reinterpret_cast<const vec8 *>(src);
+            wf[slot][1] = *reinterpret_cast<const vec8 *>(src + 8);
+        }
         if (rq_left > 0) {      // uniform; address arithmetic only
             --rq_left;
             if (++rq_chunk == nch) {
@@ -256,12 +266,29 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
     auto unit_step = [&](int i, int slot) __attribute__((always_inline)) {
         if (i < n_units) {   // uniform over the workgroup; no load of global memory inside
             const unsigned char *chunk = xs[(slot / GC) & 1] + (slot % GC) * CHUNK_BYTES;
+            vec8 w0, w1;
+            if constexpr (W8) {
+                const u32x4 raw = wraw[slot];
+                u32x4 lo, hi;  // bytes {0, b0, 0, b1} / {0, b2, 0, b3} of every word: fp16 pairs
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+                    lo[2 * jj] = __builtin_amdgcn_perm(0u, raw[jj], 0x010c000cu);
+                    lo[2 * jj + 1] = __builtin_amdgcn_perm(0u, raw[jj], 0x030c020cu);
+                    hi[2 * jj] = __builtin_amdgcn_perm(0u, raw[2 + jj], 0x010c000cu);
+                    hi[2 * jj + 1] = __builtin_amdgcn_perm(0u, raw[2 + jj], 0x030c020cu);
+                }
+                w0 = __builtin_bit_cast(vec8, lo);
+                w1 = __builtin_bit_cast(vec8, hi);
+            } else {
+                w0 = wf[slot][0];
+                w1 = wf[slot][1];
+            }
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
                 const vec8 x0 = *reinterpret_cast<const vec8 *>(chunk + xoff[mb][0]);
                 const vec8 x1 = *reinterpret_cast<const vec8 *>(chunk + xoff[mb][1]);
-                acc[mb] = mfma16(wf[slot][0], x0, acc[mb]);
-                acc[mb] = mfma16(wf[slot][1], x1, acc[mb]);
+                acc[mb] = mfma16(w0, x0, acc[mb]);
+                acc[mb] = mfma16(w1, x1, acc[mb]);
             }
             if (++c_chunk == nch || i == n_units - 1) {
                 if (!direct) flush_partial(c_tile);
@@ -466,7 +493,7 @@ __global__ void __launch_bounds__(256) linear_fewrow_reduce_kernel(const FewRowA
     fewrow_store<T>(hi, m, n + a.half, out, a.N, a.out_rs, a.out_cs, residual, a.res_rs, a.res_cs);
 }
 
-template <typename T>
+template <typename T, bool W8 = false>
 static void launch_fewrow(FewRowArgs a, const FewRowPlan &p, int mode, hipStream_t st) {
     const int mb = fewrow_row_blocks(a.M);
     const dim3 grid((unsigned)p.grid), block(64 * kFewRowWaves);
@@ -475,8 +502,8 @@ static void launch_fewrow(FewRowArgs a, const FewRowPlan &p, int mode, hipStream
     // x groups of 2 units and a ring of 4 measured best (by 0.5 to 1.4 us against 4 and 8); 16 rows of x are too few
     // pieces for 512 threads to stage 2 units at a time
 #define KERNL_FEWROW_MAIN(MBV, RMSV)                                                                                   \
-    hipLaunchKernelGGL((linear_fewrow_kernel<T, MBV, kFewRowWaves, (MBV == 1 ? 4 : 2), (MBV == 1 ? 8 : 4), RMSV>), grid, \
-                       block, 0, st, a)
+    hipLaunchKernelGGL((linear_fewrow_kernel<T, MBV, kFewRowWaves, (MBV == 1 ? 4 : 2), (MBV == 1 ? 8 : 4), RMSV, W8>), \
+                       grid, block, 0, st, a)
 #define KERNL_FEWROW_REDUCE(MBV, MODEV)                                                                                \
     hipLaunchKernelGGL((linear_fewrow_reduce_kernel<T, MBV, kFewRowWaves, MODEV>), rgrid, dim3(256), 0, st, a)
 #define KERNL_FEWROW(MBV)                                                                                              \
@@ -507,14 +534,13 @@ extern "C" int64_t kernl_linear_fewrow_workspace_bytes(int64_t M, int64_t N, int
     return p.partial_bytes + p.sq_bytes;
 }
 
-extern "C" int kernl_linear_fewrow_fwd(const void *x, const void *rms_weight, float eps, const void *w, const void *bias,
-                                       const void *residual, void *out, void *workspace, int64_t workspace_bytes,
-                                       int64_t M, int64_t N, int64_t K, const int64_t x_strides[2],
-                                       const int64_t out_strides[2], const int64_t residual_strides[2], const void *cos,
-                                       const void *sin, int64_t head_dim, int64_t rope_cols, int64_t rows_per_batch,
-                                       const int64_t table_strides[3], int table_dtype, int activation, int gated,
-                                       int dtype, void *stream) {
-    using namespace kernl;
+namespace kernl {
+static int fewrow_entry(const void *x, const void *rms_weight, float eps, const void *w, const void *bias,
+                        const void *residual, void *out, void *workspace, int64_t workspace_bytes, int64_t M, int64_t N,
+                        int64_t K, const int64_t x_strides[2], const int64_t out_strides[2],
+                        const int64_t residual_strides[2], const void *cos, const void *sin, int64_t head_dim,
+                        int64_t rope_cols, int64_t rows_per_batch, const int64_t table_strides[3], int table_dtype,
+                        int activation, int gated, int dtype, void *stream, bool w8) {
     if (x == nullptr || w == nullptr || out == nullptr || x_strides == nullptr || out_strides == nullptr)
         return set_error(KERNL_ERR_INVALID_ARG, "few-row linear: x, w, out and their strides must not be NULL");
     if (residual != nullptr && residual_strides == nullptr)
@@ -576,7 +602,36 @@ extern "C" int kernl_linear_fewrow_fwd(const void *x, const void *rms_weight, fl
     a.eps = eps;
     const int mode = gated ? kFewRowGated : rope ? kFewRowRope : kFewRowPlain;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (dtype == KERNL_F16) launch_fewrow<f16>(a, p, mode, st);
+    if (w8) launch_fewrow<f16, true>(a, p, mode, st);
+    else if (dtype == KERNL_F16) launch_fewrow<f16>(a, p, mode, st);
     else launch_fewrow<bf16>(a, p, mode, st);
     return check_launch("linear (few rows, stream-K)");
+}
+}  // namespace kernl
+
+extern "C" int kernl_linear_fewrow_fwd(const void *x, const void *rms_weight, float eps, const void *w, const void *bias,
+                                       const void *residual, void *out, void *workspace, int64_t workspace_bytes,
+                                       int64_t M, int64_t N, int64_t K, const int64_t x_strides[2],
+                                       const int64_t out_strides[2], const int64_t residual_strides[2], const void *cos,
+                                       const void *sin, int64_t head_dim, int64_t rope_cols, int64_t rows_per_batch,
+                                       const int64_t table_strides[3], int table_dtype, int activation, int gated,
+                                       int dtype, void *stream) {
+    return kernl::fewrow_entry(x, rms_weight, eps, w, bias, residual, out, workspace, workspace_bytes, M, N, K, x_strides,
+                               out_strides, residual_strides, cos, sin, head_dim, rope_cols, rows_per_batch, table_strides,
+                               table_dtype, activation, gated, dtype, stream, false);
+}
+
+extern "C" int kernl_linear_fewrow_w8_fwd(const void *x, const void *rms_weight, float eps, const void *w8,
+                                          const void *bias, const void *residual, void *out, void *workspace,
+                                          int64_t workspace_bytes, int64_t M, int64_t N, int64_t K,
+                                          const int64_t x_strides[2], const int64_t out_strides[2],
+                                          const int64_t residual_strides[2], const void *cos, const void *sin,
+                                          int64_t head_dim, int64_t rope_cols, int64_t rows_per_batch,
+                                          const int64_t table_strides[3], int table_dtype, int activation, int gated,
+                                          int dtype, void *stream) {
+    if (dtype != KERNL_F16)
+        return kernl::set_error(KERNL_ERR_UNSUPPORTED, "few-row linear (fp8 weight): activations must be f16, got dtype %d", dtype);
+    return kernl::fewrow_entry(x, rms_weight, eps, w8, bias, residual, out, workspace, workspace_bytes, M, N, K, x_strides,
+                               out_strides, residual_strides, cos, sin, head_dim, rope_cols, rows_per_batch, table_strides,
+                               table_dtype, activation, gated, dtype, stream, true);
 }

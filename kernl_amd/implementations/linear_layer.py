@@ -68,7 +68,10 @@ class LinearLayer(torch.autograd.Function):
             if _lib.linear_w8_supported(x_, weight):
                 M, N = x_.shape[0], weight.shape[0]
                 outputs = torch.empty((M, N), device=x.device, dtype=x.dtype)
-                _lib.linear_w8_fwd(x_, weight, bias, outputs, act_inputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
+                if act_inputs is None and takes_few_row_kernel(x_, weight):
+                    _lib.linear_fewrow_fwd(x_, weight, bias, None, outputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
+                else:
+                    _lib.linear_w8_fwd(x_, weight, bias, outputs, act_inputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
                 return outputs if x.ndim == 2 else outputs.reshape(*x.shape[:-1], N)
             weight = weight.view(torch.float8_e5m2).to(torch.float16)
 

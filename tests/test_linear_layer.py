@@ -171,6 +171,41 @@ def test_linear_fp8_weight_storage(shape, activation, close):
     close(act_in, pre, what=f"fp8 weight {shape} pre-activation")
 
 
+@pytest.mark.parametrize("shape", [(20, 1000, 320), (33, 2304, 2048), (128, 4096, 1024), (64, 26300, 256)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_linear_fp8_weight_stream_k(shape, close, monkeypatch):
+    """fp8 e5m2 weights on the stream-K few-row kernel (a lane's 16 weight bytes of a unit are one load, widened by byte
+    permutes): plain with bias + activation and the gated form with the RMSNorm prologue, against the oracle on the
+    decoded weight; 17 to 128 rows against a large weight reach it through `linear_layer`."""
+    from kernl_amd.implementations.linear_layer import interleave_glu_rows
+    from oracle import e5m2_decode_oracle, glu_oracle, rms_norm_oracle
+
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(73)
+    x, w, b = _inputs(M, N, K, torch.float16, gen, w_std=K ** -0.5)
+    w8 = w.to(torch.float8_e5m2).view(torch.int8)
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    _lib.linear_fewrow_fwd(x.cuda(), w8.cuda(), b.cuda(), None, out, _lib.ACT_GELU_TANH)
+    torch.cuda.synchronize()
+    close(out, linear_oracle(x, e5m2_decode_oracle(w8), b, "fast_gelu"), what=f"stream-K fp8 weight {shape}")
+    calls = []
+    real = _lib.linear_fewrow_fwd
+    monkeypatch.setattr(_lib, "linear_fewrow_fwd", lambda *a, **k: (calls.append(a[1].dtype), real(*a, **k))[1])
+    routed = linear_layer(x.cuda(), w8.cuda(), b.cuda(), "fast_gelu")
+    assert calls == ([torch.int8] if N * K >= (1 << 22) else [])
+    close(routed, linear_oracle(x, e5m2_decode_oracle(w8), b, "fast_gelu"), what=f"fp8 weight {shape} through linear_layer")
+    if N % 32 == 0:
+        wv = (torch.randn((N, K), generator=gen) * K ** -0.5).half()
+        g = (1.0 + 0.2 * torch.randn((K,), generator=gen)).half()
+        wi8 = interleave_glu_rows(w, wv).to(torch.float8_e5m2).view(torch.int8)
+        dec = e5m2_decode_oracle(wi8).reshape(N // 32, 2, 32, K)
+        out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+        real(x.cuda(), wi8.cuda(), None, None, out, _lib.ACT_SILU, rms_weight=g.cuda(), eps=1.6e-5, gated=True)
+        torch.cuda.synchronize()
+        ref = glu_oracle(rms_norm_oracle(x, g, 1.6e-5), dec[:, 0].reshape(N, K), None, dec[:, 1].reshape(N, K), None, "silu")
+        close(out, ref, scale="magnitude", what=f"stream-K fp8 gated + norm {shape}")
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
 @pytest.mark.parametrize("kind", ["plain", "plain_bias_silu", "gated"])
 @pytest.mark.parametrize("shape", [(1, 4096, 4096), (5, 96, 64), (16, 1024, 192), (33, 2304, 768), (64, 512, 1024),
