@@ -103,4 +103,25 @@ KERNL_HD int wide_weight_row(int row) {
     return (row & ~31) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3);
 }
 
+// ----------------------------------------------------------------------------------------------------
+// Stream-K few-row linear kernel: a stage of x holds GC units (64-wide chunks of K), unit j at byte j * CHUNK_BYTES, as
+// MP = 16 MB rows of 128 bytes whose eight 16-byte pieces are XOR-swizzled.
+//   staging   piece i of thread tid is 16-byte piece piece_index(tid) of row piece_row(tid, i) of the group's unit
+//             piece_unit(tid, i) (q = tid + THREADS i walks unit, row, piece), stored at piece_dst(tid, i)
+//   reads     lane (r = lane % 16, g = lane / 16) takes, for 16-row block mb and k-step s, the 16 bytes at
+//             frag_offset(mb, r, g, s) of the unit: k = 16 g + 8 s .. + 7 of x row 16 mb + r
+// ----------------------------------------------------------------------------------------------------
+template <int MB, int GC, int THREADS>
+struct FewRowStageMap {
+    static constexpr int MP = 16 * MB, CHUNK_BYTES = MP * 128, XP = GC * MP * 8 / THREADS;
+    static_assert(GC * MP * 8 % THREADS == 0 && XP >= 1, "every thread stages the same number of pieces");
+    static KERNL_HD int piece_unit(int tid, int i) { return (tid + THREADS * i) / (MP * 8); }
+    static KERNL_HD int piece_row(int tid, int i) { return ((tid + THREADS * i) >> 3) % MP; }
+    static KERNL_HD int piece_index(int tid) { return tid & 7; }
+    static KERNL_HD int piece_dst(int tid, int i) {
+        return piece_unit(tid, i) * CHUNK_BYTES + swz_offset<128>(piece_row(tid, i), piece_index(tid));
+    }
+    static KERNL_HD int frag_offset(int mb, int r, int g, int s) { return swz_offset<128>(16 * mb + r, 2 * g + s); }
+};
+
 }  // namespace kernl

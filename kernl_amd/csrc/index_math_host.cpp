@@ -4,7 +4,25 @@
 
 using namespace kernl;
 
+// Stream-K few-row linear kernel, 512 threads; (row blocks, units per stage) as the kernel is built: (1, 4), (2, 2),
+// (4, 2), (8, 2).  which: 0 piece_unit(tid=a, i=b), 1 piece_row(tid=a, i=b), 2 piece_index(tid=a), 3 piece_dst(tid=a, i=b),
+//        4 frag_offset(mb=a, r=b, g=c, s=d), 5 pieces per thread, 6 bytes per unit
+template <int MB, int GC>
+static int fewrow_index(int which, int a, int b, int c, int d) {
+    typedef FewRowStageMap<MB, GC, 512> M;
+    switch (which) {
+        case 0: return M::piece_unit(a, b);
+        case 1: return M::piece_row(a, b);
+        case 2: return M::piece_index(a);
+        case 3: return M::piece_dst(a, b);
+        case 4: return M::frag_offset(a, b, c, d);
+        case 5: return M::XP;
+        case 6: return M::CHUNK_BYTES;
+    }
+    return -1;
+}
 extern "C" {
+
 
 int kernl_idx_rowperm16(int i) { return rowperm16(i); }
 
@@ -65,6 +83,14 @@ int kernl_idx_wide_weight_row(int layout, int row) {
     if (layout == 0) return wide_weight_row<false, 8>(row);
     if (layout == 1) return wide_weight_row<false, 6>(row);
     if (layout == 2) return wide_weight_row<true, 8>(row);
+    return -1;
+}
+
+int kernl_idx_fewrow(int row_blocks, int units_per_stage, int which, int a, int b, int c, int d) {
+    if (row_blocks == 1 && units_per_stage == 4) return fewrow_index<1, 4>(which, a, b, c, d);
+    if (row_blocks == 2 && units_per_stage == 2) return fewrow_index<2, 2>(which, a, b, c, d);
+    if (row_blocks == 4 && units_per_stage == 2) return fewrow_index<4, 2>(which, a, b, c, d);
+    if (row_blocks == 8 && units_per_stage == 2) return fewrow_index<8, 2>(which, a, b, c, d);
     return -1;
 }
 

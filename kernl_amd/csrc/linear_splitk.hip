@@ -134,10 +134,10 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
     typedef typename Vec8<T>::type vec8;
     static_assert(RING % (2 * GC) == 0, "a round of RING units is a whole number of stage pairs");
     constexpr int THREADS = 64 * WAVES;
-    constexpr int MP = 16 * MB;                 // rows of x, padded to whole MFMA blocks
-    constexpr int CHUNK_BYTES = MP * 128;       // one staged chunk of x
-    constexpr int XP = GC * MP * 8 / THREADS;   // 16-byte pieces of a group of x per thread
-    static_assert(GC * MP * 8 % THREADS == 0 && XP >= 1, "every thread stages the same number of pieces");
+    typedef FewRowStageMap<MB, GC, THREADS> StageMap;   // index_math.h: shared with the host-side replay
+    constexpr int MP = StageMap::MP;                    // rows of x, padded to whole MFMA blocks
+    constexpr int CHUNK_BYTES = StageMap::CHUNK_BYTES;  // one staged chunk of x
+    constexpr int XP = StageMap::XP;                    // 16-byte pieces of a group of x per thread
     constexpr int RPT = MP * 8 > THREADS ? MP * 8 / THREADS : 1;   // rows of x a thread stages pieces of
     static_assert(2 * GC * CHUNK_BYTES >= RPT * THREADS * 4, "the stages double as the buffer of the row sums");
     __shared__ __attribute__((aligned(16))) unsigned char xs[2][GC * CHUNK_BYTES];
@@ -199,10 +199,9 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
     for (int t = 0; t < RPT; ++t) sq[t] = 0.0f;
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
-        const int q = tid + THREADS * i, j = q / (MP * 8), row = (q >> 3) % MP, piece = q & 7;
-        xrow[i] = X + (int64_t)min(row, M - 1) * a.ldx + piece * 8;
-        xunit[i] = __builtin_amdgcn_readfirstlane(j);   // a wave's 64 pieces belong to one unit
-        xdst[i] = j * CHUNK_BYTES + swz_offset<128>(row, piece);
+        xrow[i] = X + (int64_t)min(StageMap::piece_row(tid, i), M - 1) * a.ldx + StageMap::piece_index(tid) * 8;
+        xunit[i] = __builtin_amdgcn_readfirstlane(StageMap::piece_unit(tid, i));   // a wave's 64 pieces belong to one unit
+        xdst[i] = StageMap::piece_dst(tid, i);
     }
     const T *grow = static_cast<const T *>(a.rms_w) + (tid & 7) * 8;
     // (the chunk of a group's first unit is kept as a running value: no division in the loop)
@@ -243,7 +242,7 @@ __global__ void __launch_bounds__(64 * WAVES) linear_fewrow_kernel(const FewRowA
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int s = 0; s < 2; ++s) xoff[mb][s] = swz_offset<128>(16 * mb + r, 2 * g + s);
+        for (int s = 0; s < 2; ++s) xoff[mb][s] = StageMap::frag_offset(mb, r, g, s);
 
     f32x4_acc acc[MB];
 #pragma unroll

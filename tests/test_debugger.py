@@ -122,3 +122,16 @@ def test_index_functions_known_values():
         ix.swz_offset(96, 0, 0)
     with pytest.raises(ValueError):
         ix.attention(80, "stage_row", 0)
+
+
+@pytest.mark.parametrize("row_blocks, units_per_stage", [(1, 4), (2, 2), (4, 2), (8, 2)])
+def test_few_row_stage_of_x_is_written_once_and_read_without_conflicts(row_blocks, units_per_stage):
+    """The stream-K few-row linear kernel's x stage, replayed from the kernel's own index functions: the 512 threads'
+    16-byte stores cover a stage exactly once, every lane's fragment reads return k = 16 g + 8 s .. + 7 of row
+    16 mb + r of the unit (what `v_mfma_f32_16x16x32` expects on its B side), and no store or read conflicts on banks."""
+    from kernl_amd.debugger.fewrow_replay import replay_stage
+
+    writes, reads = replay_stage(row_blocks, units_per_stage)
+    assert writes.conflict_free, (writes.passes, writes.cycles)
+    assert reads.conflict_free, (reads.passes, reads.cycles)
+    assert reads.instructions == units_per_stage * row_blocks * 2
