@@ -28,19 +28,25 @@ ONE_BYTE_WEIGHT_DTYPES = (torch.int8, torch.uint8, torch.float8_e5m2)
 FEW_ROW_MIN_ROWS = 17          # up to 16 rows the kernel that gives a workgroup 16 columns and all of K is as fast or faster
 FEW_ROW_MAX_ROWS = 128         # what `kernl_linear_fewrow_fwd` takes
 SPLIT_K_MAX_ROWS = 2048        # beyond that the tiled kernels always have tiles enough; the library decides below it
-FEW_ROW_MIN_WEIGHT = 1 << 22   # elements: below that (2048 x 2048) launch latency decides and one launch beats two
+FEW_ROW_MIN_WEIGHT = 1 << 22   # elements: below that (2048 x 2048) launch latency decides and one launch beats two ...
+
+
+FEW_ROW_LONG_K = 1536          # ... unless K is long and there are more than 32 rows
+
+
+def few_row_rule(rows: int, n: int, k: int) -> bool:
+    """Where the stream-K kernel is the faster one (measured, graph replay): 17 to 128 rows against a weight of 4 M
+    elements or more (5120 x 5120 at 32 / 64 rows: 18 / 21 us against 34 / 35 on the weight-streaming kernel of
+    `kernl_linear_fwd`; 4096 x 11008: 25 / 30 against 35 / 53; at 128 rows 28 against 63 and 38 against 130 on its tile
+    kernels), and 33 rows or more against smaller weights with a long K (768 x 3072 at 48 / 128 rows: 11 / 14 us against
+    15 / 27).  Short K and few rows stay where they were (3072 x 768 at 48 rows: 8.9 against 7.2)."""
+    if not FEW_ROW_MIN_ROWS <= rows <= FEW_ROW_MAX_ROWS or k < 256 or k % 64 != 0:
+        return False
+    return n * k >= FEW_ROW_MIN_WEIGHT or (k >= FEW_ROW_LONG_K and rows > 32)
 
 
 def takes_few_row_kernel(x2d: torch.Tensor, weight: torch.Tensor) -> bool:
-    """17 to 128 rows against a large 16-bit weight run the stream-K kernel (`kernl_linear_fewrow_fwd`): measured against
-    the weight-streaming kernel of `kernl_linear_fwd` at 32 / 64 rows, 5120 x 5120: 18 / 21 us against 34 / 35;
-    4096 x 11008: 25 / 30 against 35 / 53; 12288 x 4096: 27 / 32 against 28 / 37 — and against its tile kernels at 128
-    rows: 28 against 63, 38 against 130, 39 against 52."""
-    return (
-        FEW_ROW_MIN_ROWS <= x2d.shape[0] <= FEW_ROW_MAX_ROWS
-        and weight.shape[0] * weight.shape[1] >= FEW_ROW_MIN_WEIGHT
-        and _lib.linear_fewrow_supported(x2d, weight)
-    )
+    return few_row_rule(x2d.shape[0], weight.shape[0], weight.shape[1]) and _lib.linear_fewrow_supported(x2d, weight)
 
 
 class LinearLayer(torch.autograd.Function):
@@ -211,10 +217,7 @@ def decode_linear_supported(x: torch.Tensor, weight: torch.Tensor, head_dim: Opt
         return False
     if 0 < rows <= 64:
         return True
-    return (
-        rows <= FEW_ROW_MAX_ROWS and weight.shape[0] * weight.shape[1] >= FEW_ROW_MIN_WEIGHT and x.shape[-1] >= 256
-        and (head_dim is None or head_dim in (32, 64, 128))
-    )
+    return few_row_rule(rows, weight.shape[0], weight.shape[1]) and (head_dim is None or head_dim in (32, 64, 128))
 
 
 def decode_linear_layer(

@@ -646,6 +646,9 @@ def test_few_row_kernel_routing_rule():
     rows = lambda m, k=2048: torch.zeros((m, k), dtype=torch.float16)
     assert [takes_few_row_kernel(rows(m), w) for m in (1, 16, 17, 64, 128, 129)] == [False, False, True, True, True, False]
     assert not takes_few_row_kernel(rows(32, 1024), torch.zeros((2048, 1024), dtype=torch.float16))      # small weight
+    assert not takes_few_row_kernel(rows(32, 3072), torch.zeros((768, 3072), dtype=torch.float16))       # ... few rows
+    assert takes_few_row_kernel(rows(33, 3072), torch.zeros((768, 3072), dtype=torch.float16))           # long K
+    assert not takes_few_row_kernel(rows(64, 768), torch.zeros((3072, 768), dtype=torch.float16))        # short K
     assert not takes_few_row_kernel(rows(32, 4104), torch.zeros((2048, 4104), dtype=torch.float16))      # K % 64 != 0
     assert not takes_few_row_kernel(torch.zeros((32, 2052), dtype=torch.float16)[:, :2048], w)           # row stride
     assert not takes_few_row_kernel(rows(32).to(torch.float32), w.to(torch.float32))
