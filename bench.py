@@ -496,7 +496,18 @@ def main():
             t = graph_time_ms(batched_down, reps=4) / len(w_dn)
             extra["decode_down_residual_32x4096x11008_us_graph_replay"] = round(t * 1e3, 2)
             extra["decode_down_residual_32x4096x11008_gbps"] = round(w_dn[0].numel() * 2 / (t * 1e-3) / 1e9, 1)
-            del w_dn, x32, x32f, res32
+            # 256 rows against 4096 x 4096 (a short prompt's projections): too few 128-row tiles for the chip, K split
+            x256 = torch.randn((256, 4096), generator=gen).half().to(dev)
+            w_sq = [(torch.randn((4096, 4096), generator=gen) * 0.02).half().to(dev) for _ in range(12)]
+
+            def mid_linears():
+                for w_i in w_sq:
+                    linear_layer(x256, w_i, None)
+
+            t = graph_time_ms(mid_linears, reps=4) / len(w_sq)
+            extra["linear_256x4096x4096_us_graph_replay"] = round(t * 1e3, 2)
+            extra["linear_256x4096x4096_tflops"] = round(2.0 * 256 * 4096 * 4096 / (t * 1e-3) / 1e12, 1)
+            del w_dn, w_sq, x32, x32f, res32, x256
         except Exception as exc:  # the headline must still be printed
             extra["decoder_kernels_error"] = f"{type(exc).__name__}: {exc}"[:300]
 
