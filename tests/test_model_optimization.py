@@ -455,18 +455,28 @@ def test_llama_generation_runs_the_decode_projection_kernel(batch, hidden, heads
     torch.manual_seed(0)
     layers, steps = 2, 12
     cfg = LlamaConfig(num_hidden_layers=layers, hidden_size=hidden, num_attention_heads=heads, num_key_value_heads=heads,
-                      intermediate_size=inter, vocab_size=1000, rms_norm_eps=1.6e-5, max_position_embeddings=512,
+                      intermediate_size=inter, vocab_size=1000, rms_norm_eps=1e-5, max_position_embeddings=512,
                       pad_token_id=0, bos_token_id=1, eos_token_id=2)
-    # (eps 1.6e-5: the value the fp16 RMSNorm operator clamps smaller ones to — reference layer_norm.py:295-296 — so that
-    # the eager model and the operators normalise alike; what the clamp does is measured in the Llama-shaped tests above)
     cfg._attn_implementation = "sdpa"
     model = LlamaForCausalLM(cfg).eval().half().cuda()
     gen = torch.Generator().manual_seed(1)
     ids = torch.randint(3, 1000, (batch, 20), generator=gen).cuda()
     kwargs = dict(input_ids=ids, attention_mask=torch.ones_like(ids), min_new_tokens=steps, max_new_tokens=steps,
                   do_sample=False, output_scores=True, return_dict_in_generate=True)
+    # The model under test keeps the config's eps (1e-5).  The fp16 RMSNorm operator clamps eps to 1.6e-5 (reference
+    # layer_norm.py:295-296): with N(0, 0.02) weights that alone moves the first step's scores by about 1 % of their
+    # range, printed below.  The per-step bound is therefore taken against the eager model run with the clamped eps.
+    norms = [m for m in model.modules() if type(m).__name__ == "LlamaRMSNorm"]
     with torch.inference_mode():
+        config_eps = model.generate(**kwargs)
+        for m in norms:
+            m.variance_epsilon = 1.6e-5
         ref = model.generate(**kwargs)
+        for m in norms:
+            m.variance_epsilon = 1e-5
+    first = torch.isfinite(ref.scores[0])
+    clamp_effect = (ref.scores[0].float() - config_eps.scores[0].float())[first].abs().max().item()
+    print(f"eps clamp alone moves the first scores by {clamp_effect:.4f} (range {ref.scores[0][first].abs().max().item():.2f})", flush=True)
 
     calls = {"rotated": 0, "residual": 0, "gated": 0}
     real, real_few = _lib.linear_decode_fwd, _lib.linear_fewrow_fwd
