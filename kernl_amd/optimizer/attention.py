@@ -76,6 +76,16 @@ def attention_wrapper(
     return output
 
 
+def additive_mask(mask: torch.Tensor) -> torch.Tensor:
+    """A boolean attention mask (True = attend) as the additive 0 / -inf mask the kernels take, one value per key
+    where the query dimension was only `expand`ed.  Any other mask passes through."""
+    if mask.dtype != torch.bool:
+        return mask
+    while mask.dim() < 4:
+        mask = mask.unsqueeze(0)
+    return torch.where(_per_key_view(mask), 0.0, float("-inf"))
+
+
 def sdpa_wrapper(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -93,15 +103,14 @@ def sdpa_wrapper(
     if mask is not None:
         while mask.dim() < 4:
             mask = mask.unsqueeze(0)
-        mask = _per_key_view(mask)
-        if mask.dtype == torch.bool:
-            mask = torch.zeros(mask.shape, dtype=torch.float32, device=mask.device).masked_fill_(~mask, float("-inf"))
+        mask = _per_key_view(additive_mask(mask))
     output = torch.empty_like(q)
     return attention_wrapper(q, k, v, output, float(scale), bool(is_causal) or assume_causal, mask)
 
 
 torch.fx.wrap("attention_wrapper")
 torch.fx.wrap("sdpa_wrapper")
+torch.fx.wrap("additive_mask")
 
 
 def fuse_attention_pattern_1(gm: torch.fx.GraphModule, is_causal: bool):
@@ -252,3 +261,25 @@ def fuse_attention_sdpa(gm: torch.fx.GraphModule, is_causal: bool):
         gm.graph.erase_node(node)
     gm.graph.lint()
     gm.recompile()
+
+
+def share_mask_conversion(gm: torch.fx.GraphModule):
+    """Every layer of an encoder receives the same mask node; converting a boolean mask inside each fused call costs
+    a few small kernels per layer, which is most of a short sequence's forward.  One `additive_mask` node per
+    distinct mask feeds all the calls that use it."""
+    converted = {}
+    for node in list(gm.graph.nodes):
+        if node.op != "call_function" or node.target is not sdpa_wrapper:
+            continue
+        mask = node.args[3]
+        if not isinstance(mask, torch.fx.Node) or (mask.op == "call_function" and mask.target is additive_mask):
+            continue
+        if mask not in converted:
+            with gm.graph.inserting_after(mask):
+                converted[mask] = gm.graph.call_function(additive_mask, (mask,))
+        args = list(node.args)
+        args[3] = converted[mask]
+        node.args = tuple(args)
+    if converted:
+        gm.graph.lint()
+        gm.recompile()

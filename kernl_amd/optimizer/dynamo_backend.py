@@ -8,6 +8,7 @@ from kernl_amd.optimizer.attention import (
     fuse_attention_pattern_3,
     fuse_attention_scaled,
     fuse_attention_sdpa,
+    share_mask_conversion,
 )
 from kernl_amd.optimizer.dropout import remove_dropout
 from kernl_amd.optimizer.kv_cache import drop_empty_cat_operands
@@ -45,6 +46,7 @@ def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
     fuse_attention_scaled(gm, assume_causal)
     fuse_attention_sdpa(gm, assume_causal)
     constant_causal_masks_to_flag(gm)
+    share_mask_conversion(gm)
     replace_all_linear(gm)
     replace_layer_norm(gm)
     replace_layer_norm_fn(gm)

@@ -273,9 +273,27 @@ def test_backend_rewrites_dynamo_graph_of_bert():
         # the padding mask reaches the kernel as a broadcast of a per-key tensor, not as a [B,1,S,S] matrix
         attn = next(n for n in graphs[0].graph.nodes if n.op == "call_function" and n.target.__name__ == fused)
         mask_node = attn.args[6] if fused == "attention_wrapper" else attn.args[3]
+        if fused == "sdpa_wrapper":
+            # the boolean mask is turned into an additive one once, for every layer
+            assert mask_node.target.__name__ == "additive_mask" and t.count("additive_mask") == 1
+            assert len(mask_node.users) == 2
+            mask_node = mask_node.args[0]
         assert mask_node.op == "call_method" and mask_node.target == "expand"
         assert "and_" not in t
     torch._dynamo.reset()
+
+
+def test_boolean_masks_become_additive_per_key():
+    from kernl_amd.optimizer.attention import additive_mask
+
+    keep = torch.tensor([[True, True, False, True]])
+    m = additive_mask(keep[:, None, None, :].expand(1, 1, 4, 4))
+    assert m.shape == (1, 1, 1, 4) and m.dtype == torch.float32
+    assert m.flatten().tolist() == [0.0, 0.0, float("-inf"), 0.0]
+    m = additive_mask(torch.tril(torch.ones(3, 3, dtype=torch.bool)))
+    assert m.shape == (1, 1, 3, 3) and m[0, 0, 0].tolist() == [0.0, float("-inf"), float("-inf")]
+    f = torch.zeros(1, 1, 1, 4)
+    assert additive_mask(f) is f
 
 
 def test_rms_norm_and_swiglu_patterns():
