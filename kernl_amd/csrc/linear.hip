@@ -17,15 +17,15 @@ static int linear_mfma_dispatch(const LinearArgs &a) {
     }
     if (pick == 0 || pick == 9) pick = pick_tile(a.M, a.N, a.K, (a.act & kGluBit) != 0);
     if (a.act & kGluBit) {
-        if (pick == 5 && a.K % 64 == 0) run_wide(a, kDtype, 256);
+        if (pick == 5) run_wide(a, kDtype, 256);
         else if (pick == 3) launch_mfma_glu<T, Tile128x128>(a);
         else launch_mfma_glu<T, Tile256x256>(a);
         return check_launch("gated linear (mfma)");
     }
-    if (pick == 5 && a.K % 64 == 0) run_wide(a, kDtype, 256);
-    else if (pick == 6 && a.K % 64 == 0) run_wide(a, kDtype, 192);
-    else if (pick == 7 && a.K % 64 == 0) run_wide_half(a, kDtype, 256);
-    else if (pick == 8 && a.K % 64 == 0) run_wide_half(a, kDtype, 192);
+    if (pick == 5) run_wide(a, kDtype, 256);
+    else if (pick == 6) run_wide(a, kDtype, 192);
+    else if (pick == 7) run_wide_half(a, kDtype, 256);
+    else if (pick == 8) run_wide_half(a, kDtype, 192);
     else if (pick == 1) launch_mfma_cfg<T, Tile256x256>(a);
     else if (pick == 2) launch_mfma_cfg<T, Tile256x192>(a);
     else if (pick == 4) launch_mfma_cfg<T, Tile256x128k32>(a);

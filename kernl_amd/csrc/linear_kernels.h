@@ -387,7 +387,7 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 }
 
 // ----------------------------------------------------------------------------------------------------
-// Wide MFMA kernel for K % 64 == 0: 256x256 output tile, 4 waves, ONE wave per SIMD owning a 128x128 sub-tile as
+// Wide MFMA kernel for K % 8 == 0 (K % 64 == 0 with one-byte weights): 256x256 output tile, 4 waves, ONE wave per SIMD owning a 128x128 sub-tile as
 // 8x8 blocks of v_mfma_f32_16x16x32 (256 accumulator registers, kept in the accumulation half of the register file).
 // Per 32-wide k-step a wave runs 64 MFMAs on 16 operand fragments — half the LDS traffic per flop of the 8-wave
 // kernel above.  Operand tiles go HBM -> LDS directly (buffer loads with the LDS flag), two 64 KB stages.  With a
@@ -606,10 +606,30 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         else
             asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
     };
+    // K % 64 != 0: the last k-tile of every output tile is ragged.  Bit l of `tail_bits` says whether the chunk that
+    // load l of this lane fetches starts below K in that k-tile; the others are pointed out of range and arrive as
+    // zeros, in BOTH operands (a zero weight against whatever follows a row of x would still turn an infinity there
+    // into a NaN here).  The chunk a (lane, load) pair fetches is the same for every tile.
+    const int nk = (K + BK - 1) / BK;
+    const int k_last = K - (nk - 1) * BK;  // 8 .. 64 valid k in the last k-tile
+    uint32_t tail_bits = 0;
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int q = (wave * LOADS + i) * 64 + lane;
+        if (swz_chunk<RB>(q / CPR, q % CPR) * 8 < k_last) tail_bits |= 1u << i;
+    }
+#pragma unroll
+    for (int i = 0; i < LOADS_W; ++i) {
+        const int q = (wave * LOADS_W + i) * 64 + lane;
+        if (swz_chunk<RBW>(q / CPRW, q % CPRW) * (16 / WB) < k_last) tail_bits |= 1u << (LOADS + i);
+    }
     // load l (0 .. NL-1) of a k-tile: the x loads, then the w loads
-    auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
-        if (l < LOADS) load4(xrsrc, xd[l], lds_base + stage * X_BYTES + wave * (LOADS * 1024), l >> 2, l & 3, k0 * 2);
-        else load4(wrsrc, wd[l - LOADS], lds_base + W_BASE + stage * W_BYTES + wave * (LOADS_W * 1024), (l - LOADS) >> 2, (l - LOADS) & 3, k0 * WB);
+    // `keep`: bit l clear sends load l out of range (all ones for a whole k-tile, `tail_bits` for the ragged one)
+    auto tile_load = [&](int l, int stage, int k0, uint32_t keep) __attribute__((always_inline)) {
+        uint32_t off = l < LOADS ? xd[l] : wd[l - LOADS];
+        off = ((keep >> l) & 1u) != 0 ? off : kOutOfRange;
+        if (l < LOADS) load4(xrsrc, off, lds_base + stage * X_BYTES + wave * (LOADS * 1024), l >> 2, l & 3, k0 * 2);
+        else load4(wrsrc, off, lds_base + W_BASE + stage * W_BYTES + wave * (LOADS_W * 1024), (l - LOADS) >> 2, (l - LOADS) & 3, k0 * WB);
     };
 
     // LDS addresses of this lane's operand fragments in stage 0, one register per (k-step, block): with a whole
@@ -640,7 +660,6 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     };
     u32x2 wraw[W8 ? NBN : 1];
 
-    const int nk = K / BK;
     int idx = (int)(blockIdx.x >> 3);  // position of the tile being multiplied in this XCD's run
     int m0 = 0, n0 = 0;
     if (!tile_origin(idx, m0, n0)) return;
@@ -658,10 +677,10 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         }
     };
 #pragma unroll
-    for (int l = 0; l < NL; ++l) tile_load(l, 0, load_kt * BK);
+    for (int l = 0; l < NL; ++l) tile_load(l, 0, load_kt * BK, load_kt == nk - 1 ? tail_bits : ~0u);
     advance_load();
 #pragma unroll
-    for (int l = 0; l < NL; ++l) tile_load(l, 1, load_kt * BK);
+    for (int l = 0; l < NL; ++l) tile_load(l, 1, load_kt * BK, load_kt == nk - 1 ? tail_bits : ~0u);
     advance_load();
     // vmcnt(NL): the first k-tile has landed, the second may still be in flight
     __builtin_amdgcn_s_waitcnt(0x0F70 | (NL & 15) | ((NL >> 4) << 14));
@@ -683,6 +702,7 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     // waiting for "everything outstanding" would only wait for the previous tile's output stores.
     auto k_tile = [&](auto cur_c, bool landed) __attribute__((always_inline)) {
         constexpr int CUR = decltype(cur_c)::value;
+        const uint32_t keep = load_kt == nk - 1 ? tail_bits : ~0u;  // the k-tile requested during this one may be the ragged one
         const int k0 = load_kt * BK;
 #pragma unroll
         for (int st = 0; st < KSTEPS; ++st) {
@@ -710,7 +730,7 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
                 } else if (W8 && m % PERIOD == 1 && slot >= 2 && slot - 2 < NBN) {
                     fa[sn][slot - 2] = widen8(wraw[slot - 2]);  // two read slots later: the bytes have arrived
                 } else if (m % PERIOD == PERIOD - 2 && st == 1 && slot < NL) {
-                    tile_load(slot, CUR, k0);
+                    tile_load(slot, CUR, k0, keep);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -857,9 +877,27 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
         else
             asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:3072 lds" :: "v"(off), "s"(rsrc), "s"(kbytes) : "memory");
     };
+    // K % 64 != 0: chunks of the last k-tile that start at or beyond K are pointed out of range and arrive as zeros,
+    // in both operands (as in the wide kernel); bit l of `tail_bits`: load l of this lane stays inside
+    const int nk_all = (K + BK - 1) / BK;
+    const int k_last = K - (nk_all - 1) * BK;
+    uint32_t tail_bits = 0;
+#pragma unroll
+    for (int i = 0; i < LOADS_X; ++i) {
+        const int q = (wave * LOADS_X + i) * 64 + lane;
+        if (swz_chunk<RB>(q / CPR, q % CPR) * 8 < k_last) tail_bits |= 1u << i;
+    }
+#pragma unroll
+    for (int i = 0; i < LOADS_W; ++i) {
+        const int q = (wave * LOADS_W + i) * 64 + lane;
+        if (swz_chunk<RBW>(q / CPRW, q % CPRW) * (16 / WB) < k_last) tail_bits |= 1u << (LOADS_X + i);
+    }
     auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
-        if (l < LOADS_X) load4(xrsrc, xd[l], lds_base + stage * X_STAGE + wave * (LOADS_X * 1024), 0, l, k0 * 2);
-        else load4(wrsrc, wd[l - LOADS_X], lds_base + W_BASE + stage * W_STAGE + wave * (LOADS_W * 1024), (l - LOADS_X) >> 2, (l - LOADS_X) & 3, k0 * WB);
+        const uint32_t keep = k0 == (nk_all - 1) * BK ? tail_bits : ~0u;
+        uint32_t off = l < LOADS_X ? xd[l] : wd[l - LOADS_X];
+        off = ((keep >> l) & 1u) != 0 ? off : kOutOfRange;
+        if (l < LOADS_X) load4(xrsrc, off, lds_base + stage * X_STAGE + wave * (LOADS_X * 1024), 0, l, k0 * 2);
+        else load4(wrsrc, off, lds_base + W_BASE + stage * W_STAGE + wave * (LOADS_W * 1024), (l - LOADS_X) >> 2, (l - LOADS_X) & 3, k0 * WB);
     };
 
     // fragment addresses: x stages are 16 KB apart (immediates 0 / 16 K / 32 K); w stages 32 KB apart, and an LDS
@@ -883,7 +921,7 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
 
     // Every k-tile slot issues its NL loads, so that the counter waits stay exact up to the end; requests past the
     // last k-tile fetch that tile again (into a stage nobody reads any more) instead of running past the row ends.
-    int nk = K / BK, kb = 0;   // k-tiles of this workgroup: kb .. kb + nk - 1
+    int nk = nk_all, kb = 0;   // k-tiles of this workgroup: kb .. kb + nk - 1
     if constexpr (SPLIT) {
         const int per_split = (nk + splits - 1) / splits;
         kb = (int)blockIdx.y * per_split;
@@ -1476,7 +1514,7 @@ static void launch_wide_act(const LinearArgs &a) {
     const int bias_vec_ok = bias != nullptr && aligned16(bias);
     // persistent: at most one workgroup per CU (32 per XCD), each walks its share of the XCD's tiles.  The kernel
     // needs every tile to start in LDS stage 0: with an odd number of k-tiles each workgroup gets a single tile.
-    const int slots = (per_xcd < 32 || (a.K / 64) % 2 != 0) ? per_xcd : 32;
+    const int slots = (per_xcd < 32 || ((a.K + 63) / 64) % 2 != 0) ? per_xcd : 32;
     hipLaunchKernelGGL(kern, dim3(slots * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
                        a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok);
@@ -1629,22 +1667,19 @@ static double tile_cost(int M, int N, int K, int bm, int bn, double base, double
     const double kf = (double)K / ((double)K + 1500.0);
     return (double)per_cu * ((double)bm * bn / 65536.0) * (base + per_k * kf);
 }
-// which: 1 = 256x256, 2 = 256x192, 3 = 128x128 (8-wave kernel), 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192 (K % 64 == 0)
+// which: 1 = 256x256, 2 = 256x192, 3 = 128x128 (8-wave kernel), 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192
 static int pick_tile(int M, int N, int K, bool gated) {
-    int pick = 1;
-    double best = tile_cost(M, N, K, 256, 256, 1.15, 0.3);
-    if (K % 64 == 0) {
-        best = tile_cost(M, N, K, 256, 256, 1.0, 0.0);
-        pick = 5;
-        const double c6 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.04, 0.0);
-        if (c6 < best) { best = c6; pick = 6; }
-        // half-height tiles: a quarter slower per output element at long K (more operand traffic per MFMA), and a
-        // prologue per tile that weighs more the shorter K is; they win where 256-row tiles leave CUs idle
-        const double c7 = gated ? 1e30 : tile_cost(M, N, K, 128, 256, 1.5, -0.35);
-        if (c7 < best) { best = c7; pick = 7; }
-        const double c8 = gated ? 1e30 : tile_cost(M, N, K, 128, 192, 1.65, -0.35);
-        if (c8 < best) { best = c8; pick = 8; }
-    }
+    // (the wide kernels take any K the MFMA path takes, with a zero-filled last k-tile)
+    int pick = 5;
+    double best = tile_cost(M, N, K, 256, 256, 1.0, 0.0);
+    const double c6 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.04, 0.0);
+    if (c6 < best) { best = c6; pick = 6; }
+    // half-height tiles: a quarter slower per output element at long K (more operand traffic per MFMA), and a
+    // prologue per tile that weighs more the shorter K is; they win where 256-row tiles leave CUs idle
+    const double c7 = gated ? 1e30 : tile_cost(M, N, K, 128, 256, 1.5, -0.35);
+    if (c7 < best) { best = c7; pick = 7; }
+    const double c8 = gated ? 1e30 : tile_cost(M, N, K, 128, 192, 1.65, -0.35);
+    if (c8 < best) { best = c8; pick = 8; }
     // 256x192 gives a wave an odd number of column blocks: not usable for gate/value pairs
     const double c2 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.2, 0.3);
     const double c3 = tile_cost(M, N, K, 128, 128, 1.9, 0.4);

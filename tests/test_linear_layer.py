@@ -65,6 +65,33 @@ def test_linear_every_tile_shape(shape, tile, close):
     close(out, linear_oracle(x, w, b, "gelu"), what=f"linear tile {tile} {shape}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("tile", [0, 5, 6, 7, 8], ids=["heuristic"] + TILE_IDS[4:])
+@pytest.mark.parametrize("shape", [(300, 520, 8), (300, 520, 40), (513, 385, 72), (700, 520, 136), (1000, 600, 520),
+                                   (2050, 1030, 776), (4352, 4300, 1992)], ids=lambda s: "x".join(map(str, s)))
+def test_linear_ragged_last_k_tile(shape, tile, dtype, close):
+    """K a multiple of 8 but not of 64 on the wide kernels: the last k-tile of every output tile is partly
+    outside the rows.  One, two, an odd and an even number of k-tiles; more output tiles than compute units, so the
+    stream of k-tiles crosses tile boundaries.  What follows a row in memory must not leak into it: the row after
+    row 4 starts with infinities, and row 4 (like every other row) still has to match the oracle."""
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(31)
+    x, w, b = _inputs(M, N, K, dtype, gen, w_std=K ** -0.5)
+    x[5, :8] = float("inf")
+    lib = _lib.load()
+    lib.kernl_linear_force_tile(tile)
+    try:
+        out = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation="tanh")
+        torch.cuda.synchronize()
+    finally:
+        lib.kernl_linear_force_tile(0)
+    keep = torch.arange(M) != 5
+    assert torch.isfinite(out[keep.cuda()].float()).all(), "a neighbouring row leaked into the ragged k-tile"
+    x[5, :8] = 0.0
+    ref = linear_oracle(x, w, b, "tanh")
+    close(out[keep.cuda()], ref[keep], dtype, what=f"ragged K {shape} tile {tile}")
+
+
 def test_linear_non_contiguous_input(close):
     # reference test/test_linear_layer.py:73-78: x.mT of a contiguous [K, M] matrix
     gen = torch.Generator().manual_seed(2)
