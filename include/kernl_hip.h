@@ -370,7 +370,9 @@ int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, 
  *                                2 = 256x192, 3 = 128x128, 4 = 256x128 with 32-wide k-tiles; persistent kernel with one
  *                                wave per SIMD: 5 = 256x256, 6 = 256x192; its one-tile-per-workgroup variant with
  *                                three LDS stages: 7 = 128x256, 8 = 128x192 (5..8 take any K the MFMA path takes, with
- *                                a zero-filled last k-tile when K % 64 != 0; gated epilogues take 1, 3 or 5).  With the heuristic, inputs of at most
+ *                                a zero-filled last k-tile when K % 64 != 0; gated epilogues take 1, 3 or 5);
+ *                                10 / 11 = the small-tile kernel (32 x 64 / 64 x 64 tiles over the whole K, one launch),
+ *                                which the heuristic takes for 65+ rows, K < 1536 and at most 256 such tiles.  With the heuristic, inputs of at most
  *                                64 rows and K % 64 == 0 go to a kernel that streams the weight once (16 output
  *                                columns per workgroup); 9 = that kernel where it applies, the heuristic elsewhere;
  *                                1..8 keep such inputs on the tile kernels.

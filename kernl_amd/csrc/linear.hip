@@ -15,6 +15,15 @@ static int linear_mfma_dispatch(const LinearArgs &a) {
         else launch_skinny<T, false>(a);
         return check_launch("linear (skinny)");
     }
+    // small problems: one launch of small tiles over the whole K (10 / 11 force its 32- / 64-row form)
+    if (pick == 0 && !(a.act & kGluBit)) {
+        const int rows = small_tile_rows(a.M, a.N, a.K);
+        if (rows != 0) pick = rows == 32 ? 10 : 11;
+    }
+    if ((pick == 10 || pick == 11) && !(a.act & kGluBit)) {
+        run_small(a, kDtype, pick == 10 ? 32 : 64);
+        return check_launch("linear (small tiles)");
+    }
     if (pick == 0 || pick == 9) pick = pick_tile(a.M, a.N, a.K, (a.act & kGluBit) != 0);
     if (a.act & kGluBit) {
         if (pick == 5) run_wide(a, kDtype, 256);

@@ -31,6 +31,7 @@ void run_wide_w8(const LinearArgs &a);                               // fp8 e5m2
 void run_wide_half(const LinearArgs &a, int dtype, int cols);        // 128-row tiles
 void run_wide_half_w8(const LinearArgs &a);
 void run_half_split(const LinearArgs &a, const HalfSplitPlan &p, float *part, int dtype);
+void run_small(const LinearArgs &a, int dtype, int rows);            // 32- or 64-row tiles over the whole K (linear_small.hip)
 
 
 // ----------------------------------------------------------------------------------------------------
@@ -1688,7 +1689,21 @@ static int pick_tile(int M, int N, int K, bool gated) {
     return pick;
 }
 
-extern int g_linear_force_tile;  // test / tuning hook (defined in linear.hip): 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192
+// Rows per tile of the small-tile kernel (linear_small.hip), or 0 when the problem is not its kind: more than 64 rows
+// (fewer stream the weight), a short K (from 1536 on the stream-K / split-K kernels or the big tiles are ahead), and
+// one round of workgroups — 32-row tiles where they make at most 256 workgroups, else 64-row tiles on the same
+// condition.  Measured against the tile kernels it replaces there (graph replay, us): 128 x 768 x 768 10.7 -> 7.3,
+// 128 x 2304 x 768 11.7 -> 7.7, 128 x 3072 x 768 11.7 -> 8.3, 512 x 768 x 768 11.0 -> 7.6, 512 x 1024 x 1024 13.0 ->
+// 8.6, 128 x 4096 x 1024 14.4 -> 10.0; 64-row tiles: 256 x 3072 x 768 11.8 -> 11.2, 1024 x 1024 x 1024 14.0 -> 12.2.
+static int small_tile_rows(int M, int N, int K) {
+    if (M <= 64 || K >= 1536) return 0;
+    const int64_t cols = (N + 63) / 64;
+    if ((int64_t)((M + 31) / 32) * cols <= 256) return 32;
+    if ((int64_t)((M + 63) / 64) * cols <= 256) return 64;
+    return 0;
+}
+
+extern int g_linear_force_tile;  // test / tuning hook (defined in linear.hip): 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192, 10 / 11 = small tiles of 32 / 64 rows
 
 template <typename T, bool GATED, int MB, int NR, bool W8, bool RMS = false, bool ROPE = false>
 static void launch_skinny_blocks(const LinearArgs &a, const void *rms_w = nullptr, float eps = 0.0f,

@@ -42,9 +42,11 @@ def test_linear_vs_oracle(shape, bias, activation, dtype, close):
 
 
 TILE_IDS = ["256x256", "256x192", "128x128", "256x128k32", "wide256x256", "wide256x192", "wide128x256", "wide128x192"]
+SMALL_TILES = [10, 11]  # 32 x 64 and 64 x 64 tiles over the whole K
+SMALL_IDS = ["small32x64", "small64x64"]
 
 
-@pytest.mark.parametrize("tile", list(range(1, 9)), ids=TILE_IDS)
+@pytest.mark.parametrize("tile", list(range(1, 9)) + SMALL_TILES, ids=TILE_IDS + SMALL_IDS)
 @pytest.mark.parametrize(
     "shape",
     [(1000, 600, 776), (256, 256, 64), (513, 385, 1032), (700, 520, 1024), (300, 260, 32), (257, 513, 96), (640, 512, 160),
@@ -66,7 +68,7 @@ def test_linear_every_tile_shape(shape, tile, close):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("tile", [0, 5, 6, 7, 8], ids=["heuristic"] + TILE_IDS[4:])
+@pytest.mark.parametrize("tile", [0, 5, 6, 7, 8] + SMALL_TILES, ids=["heuristic"] + TILE_IDS[4:] + SMALL_IDS)
 @pytest.mark.parametrize("shape", [(300, 520, 8), (300, 520, 40), (513, 385, 72), (700, 520, 136), (1000, 600, 520),
                                    (2050, 1030, 776), (4352, 4300, 1992)], ids=lambda s: "x".join(map(str, s)))
 def test_linear_ragged_last_k_tile(shape, tile, dtype, close):
@@ -90,6 +92,40 @@ def test_linear_ragged_last_k_tile(shape, tile, dtype, close):
     x[5, :8] = 0.0
     ref = linear_oracle(x, w, b, "tanh")
     close(out[keep.cuda()], ref[keep], dtype, what=f"ragged K {shape} tile {tile}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("activation", ["", "fast_gelu"])
+@pytest.mark.parametrize("shape", [(65, 768, 768), (128, 2304, 768), (128, 3072, 768), (200, 1000, 448), (500, 520, 64),
+                                   (512, 1024, 1024), (1024, 700, 1480), (1000, 960, 520), (130, 70, 8)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_linear_small_tiles_are_what_small_problems_run(shape, activation, dtype, close):
+    """65 rows and more against a short K with at most 256 small tiles: the library's own choice is the small-tile
+    kernel (one launch, whole K per workgroup).  Forcing either of its tile heights must give the same bits as the
+    heuristic for the height it picks, and all three must match the oracle: tiles ragged in rows, columns and K, fewer
+    k-tiles than ring stages, strided output."""
+    M, N, K = shape
+    gen = torch.Generator().manual_seed(57)
+    x, w, b = _inputs(M, N, K, dtype, gen, w_std=K ** -0.5)
+    ref = linear_oracle(x, w, b, activation)
+    lib = _lib.load()
+    outs = {}
+    for tile in (0, 10, 11):
+        lib.kernl_linear_force_tile(tile)
+        try:
+            outs[tile] = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation=activation)
+            torch.cuda.synchronize()
+        finally:
+            lib.kernl_linear_force_tile(0)
+        close(outs[tile], ref, dtype, what=f"small tiles {shape} {activation!r} tile {tile}")
+    picked = 10 if -(-M // 32) * -(-N // 64) <= 256 else 11
+    assert torch.equal(outs[0], outs[picked]), "the heuristic did not run the small-tile kernel"
+    # a column slice of a wider buffer as the output's home: row stride != N
+    wide = torch.zeros((M, N + 24), dtype=dtype, device="cuda")
+    _lib.linear_fwd(x.cuda(), w.cuda(), b.cuda(), wide[:, 8:8 + N], None, _lib.ACT_NONE)
+    torch.cuda.synchronize()
+    close(wide[:, 8:8 + N], linear_oracle(x, w, b, ""), dtype, what=f"small tiles {shape} strided output")
+    assert (wide[:, :8] == 0).all() and (wide[:, 8 + N:] == 0).all()
 
 
 def test_linear_non_contiguous_input(close):
@@ -125,7 +161,7 @@ def test_linear_saves_activation_inputs(close):
     close(act_in, pre, what="linear act_inputs")
 
 
-@pytest.mark.parametrize("tile", [5, 6, 7, 8], ids=TILE_IDS[4:])
+@pytest.mark.parametrize("tile", [5, 6, 7, 8] + SMALL_TILES, ids=TILE_IDS[4:] + SMALL_IDS)
 def test_linear_wide_tiles_save_activation_inputs(tile, close):
     gen = torch.Generator().manual_seed(13)
     M, N, K = 300, 520, 448
