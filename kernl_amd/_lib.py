@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "kernl_attention_skinny_static_fwd",
     "kernl_rope_fwd",
     "kernl_linear_fwd",
+    "kernl_linear_small_kind",
     "kernl_linear_w8_fwd",
     "kernl_linear_rms_fwd",
     "kernl_linear_decode_fwd",
@@ -131,6 +132,8 @@ def load() -> ctypes.CDLL:
     lib.kernl_linear_rms_fwd.argtypes = (
         [_vp, _vp, ctypes.c_float, _vp, _vp, _vp] + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int] * 3 + [_vp]
     )
+    lib.kernl_linear_small_kind.restype = ctypes.c_int
+    lib.kernl_linear_small_kind.argtypes = [_i64] * 3
     lib.kernl_linear_glu_fwd.restype = ctypes.c_int
     lib.kernl_linear_glu_fwd.argtypes = [_vp] * 4 + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_layernorm_fwd.restype = ctypes.c_int
@@ -290,6 +293,11 @@ def rope_fwd(x, cos, sin, out) -> None:
             DTYPE_CODE[cos.dtype], DTYPE_CODE[x.dtype], _stream(x),
         )
     _check(st, "kernl_rope_fwd")
+
+
+def linear_small_kind(M: int, N: int, K: int) -> int:
+    """Non-zero when `kernl_linear_fwd` runs an M x N x K problem on one of its small-problem kernels."""
+    return int(load().kernl_linear_small_kind(int(M), int(N), int(K)))
 
 
 def linear_fwd(x2d, weight, bias, out2d, act_in2d, activation: int) -> None:

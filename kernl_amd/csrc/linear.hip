@@ -10,15 +10,17 @@ static int linear_mfma_dispatch(const LinearArgs &a) {
     constexpr int kDtype = std::is_same<T, f16>::value ? KERNL_F16 : KERNL_BF16;
     int pick = g_linear_force_tile;
     // few rows of x: stream the weight once with every CU (9 forces this kernel where it applies)
-    if ((pick == 0 || pick == 9) && a.M <= 64 && a.K % 64 == 0) {
+    const bool small_first = pick == 0 && !(a.act & kGluBit) && small_problem_kind(a.M, a.N, a.K) != 0;
+    if ((pick == 0 || pick == 9) && !small_first && a.M <= 64 && a.K % 64 == 0) {
         if (a.act & kGluBit) launch_skinny<T, true>(a);
         else launch_skinny<T, false>(a);
         return check_launch("linear (skinny)");
     }
     // small problems: one launch of small tiles over the whole K (10 / 11 force its 32- / 64-row form)
-    if (pick == 0 && !(a.act & kGluBit)) {
-        const int rows = small_tile_rows(a.M, a.N, a.K);
-        if (rows != 0) pick = rows == 32 ? 10 : 11;
+    if (pick == 0 && !(a.act & kGluBit)) pick = small_problem_kind(a.M, a.N, a.K);
+    if ((pick == 12 || pick == 13) && !(a.act & kGluBit)) {
+        run_small_dealt(a, kDtype, pick == 12 ? 16 : 32);
+        return check_launch("linear (small tiles, dealt k-tiles)");
     }
     if ((pick == 10 || pick == 11) && !(a.act & kGluBit)) {
         run_small(a, kDtype, pick == 10 ? 32 : 64);
@@ -53,6 +55,11 @@ static int linear_fma_dispatch(const LinearArgs &a) {
 }
 
 }  // namespace kernl
+
+extern "C" int kernl_linear_small_kind(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % 8 != 0) return 0;
+    return kernl::small_problem_kind(M, N, K);
+}
 
 // Tuning hook used by the sweep tests: force a tile shape (0 restores the heuristic).
 extern "C" void kernl_linear_force_tile(int which) { kernl::g_linear_force_tile = which; }

@@ -175,6 +175,189 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
     }
 }
 
+// The same problem class with a LONG K (BERT-base's feed-forward down projection at batch 1: 128 x 768 x 3072): time per
+// workgroup is latency x (bytes the workgroup pulls) / (bytes the CU keeps in flight), so the tiles get smaller still
+// — 32 x 32 or 16 x 32, up to 256 workgroups — and the four waves no longer share a tile's k-tiles but deal them out:
+// wave w multiplies k-tiles w, w + 4, ... of the WHOLE tile out of a ring of its own (no barrier in the loop, program
+// order and the load counter are all the synchronisation), and the four partial tiles meet in LDS at the end.
+template <typename T, int BM, int BN>
+__global__ void __launch_bounds__(256, 1)
+linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
+                          T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs,
+                          int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int act, int tiles_m) {
+    typedef typename Vec8<T>::type vec8;
+    constexpr int BK = 64, RB = BK * 2, CPR = BK / 8, WAVES = 4;
+    constexpr int X_BYTES = BM * RB, W_BYTES = BN * RB, STAGE = X_BYTES + W_BYTES;
+    constexpr int S = (32 * 1024) / STAGE;                          // stages of a wave's 32 KB ring
+    constexpr int LX = BM * CPR / 64, LW = BN * CPR / 64, L = LX + LW;  // 1 KB loads per wave and stage
+    constexpr int NBM = BM / 16, NBN = BN / 16;
+    static_assert(S >= 3 && (S - 2) * L <= 63, "ring depth and wait count");
+    static_assert(WAVES * NBM * NBN * 1024 <= WAVES * 32 * 1024, "the partial tiles fit the rings");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int m0 = ((int)blockIdx.x % tiles_m) * BM, n0 = ((int)blockIdx.x / tiles_m) * BN;
+
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    const int rows_x = min(BM, M - m0), rows_w = min(BN, N - n0);
+    const uint64_t xaddr = (uint64_t)(uintptr_t)(X + (int64_t)m0 * ldx);
+    const uint64_t waddr = (uint64_t)(uintptr_t)(W + (int64_t)n0 * K);
+    const u32x4 xrsrc = {(uint32_t)xaddr, (uint32_t)(xaddr >> 32) & 0xFFFFu,
+                         (uint32_t)((((int64_t)rows_x - 1) * ldx + K) * 2), 0x00020000u};
+    const u32x4 wrsrc = {(uint32_t)waddr, (uint32_t)(waddr >> 32) & 0xFFFFu, (uint32_t)((int64_t)rows_w * K * 2),
+                         0x00020000u};
+    // load i of the wave fills the 1 KB of 16-byte chunks [64 i, 64 i + 64) of an operand tile (the whole tile is the wave's)
+    const int nk = (K + BK - 1) / BK;
+    const int k_last = K - (nk - 1) * BK;
+    uint32_t xd[LX], wd[LW], tail_bits = 0;
+#pragma unroll
+    for (int i = 0; i < LX; ++i) {
+        const int q = i * 64 + lane;
+        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) : kOutOfRange;
+        if (c * 8 < k_last) tail_bits |= 1u << i;
+    }
+#pragma unroll
+    for (int i = 0; i < LW; ++i) {
+        const int q = i * 64 + lane;
+        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        wd[i] = row < rows_w ? (uint32_t)(((int64_t)row * K + c * 8) * 2) : kOutOfRange;
+        if (c * 8 < k_last) tail_bits |= 1u << (LX + i);
+    }
+    typedef __attribute__((address_space(3))) void lds_void;
+    const uint32_t ring = (uint32_t)(uintptr_t)(lds_void *)smem + (uint32_t)wave * (32 * 1024);
+    auto load1 = [&](const u32x4 &rsrc, uint32_t off, uint32_t lds, int kbytes) __attribute__((always_inline)) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :: "s"(lds), "v"(off), "s"(rsrc), "s"(kbytes) : "memory", "m0");
+    };
+    // the wave's j-th k-tile (k-tile wave + 4 j of the problem) into stage `stage` of its ring
+    auto request = [&](int j, int stage) __attribute__((always_inline)) {
+        const int kt = wave + WAVES * j;
+        const uint32_t keep = kt < nk - 1 ? ~0u : kt == nk - 1 ? tail_bits : 0u;
+        const uint32_t base = ring + (uint32_t)stage * STAGE;
+        const int kbytes = kt < nk ? kt * BK * 2 : 0;
+#pragma unroll
+        for (int i = 0; i < LX; ++i) load1(xrsrc, ((keep >> i) & 1u) != 0 ? xd[i] : kOutOfRange, base + i * 1024, kbytes);
+#pragma unroll
+        for (int i = 0; i < LW; ++i)
+            load1(wrsrc, ((keep >> (LX + i)) & 1u) != 0 ? wd[i] : kOutOfRange, base + X_BYTES + i * 1024, kbytes);
+    };
+    int xoff[2][NBM], woff[2][NBN];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+        for (int i = 0; i < NBM; ++i) xoff[st][i] = swz_offset<RB>(16 * i + r, 4 * st + g);
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) woff[st][j] = X_BYTES + swz_offset<RB>(16 * j + r, 4 * st + g);
+    }
+    f32x4_acc acc[NBM][NBN];
+#pragma unroll
+    for (int i = 0; i < NBM; ++i)
+#pragma unroll
+        for (int j = 0; j < NBN; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const int mine = nk > wave ? (nk - wave + WAVES - 1) / WAVES : 0;  // k-tiles of this wave
+#pragma unroll
+    for (int j = 0; j < S - 1; ++j) request(j, j);
+    int stage = 0;
+    const unsigned char *my = smem + wave * (32 * 1024);
+    for (int j = 0; j < mine; ++j) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (((S - 2) * L) & 15) | ((((S - 2) * L) >> 4) << 14));
+        const unsigned char *sb = my + stage * STAGE;
+        vec8 xf[2][NBM], wf[2][NBN];
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+#pragma unroll
+            for (int i = 0; i < NBM; ++i) xf[st][i] = *reinterpret_cast<const vec8 *>(sb + xoff[st][i]);
+#pragma unroll
+            for (int jj = 0; jj < NBN; ++jj) wf[st][jj] = *reinterpret_cast<const vec8 *>(sb + woff[st][jj]);
+        }
+        // the fragments are in registers before the stage is handed back to the loads
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        request(j + S - 1, stage == 0 ? S - 1 : stage - 1);
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int i = 0; i < NBM; ++i)
+#pragma unroll
+                for (int jj = 0; jj < NBN; ++jj) acc[i][jj] = mfma16(wf[st][jj], xf[st][i], acc[i][jj]);
+        stage = stage == S - 1 ? 0 : stage + 1;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // the out-of-range requests of the last rounds are done with
+    __syncthreads();                     // every ring is free: the partial tiles take their place
+
+    float *red = reinterpret_cast<float *>(smem);  // [wave][block][lane][4]
+#pragma unroll
+    for (int i = 0; i < NBM; ++i)
+#pragma unroll
+        for (int j = 0; j < NBN; ++j)
+            *reinterpret_cast<f32x4_acc *>(red + ((wave * (NBM * NBN) + i * NBN + j) * 64 + lane) * 4) = acc[i][j];
+    __syncthreads();
+
+    const bool out_vec = out_cs == 1 && (out_rs & 3) == 0 && ((uintptr_t)out & 7) == 0;
+    const bool ai_vec = act_in != nullptr && ai_cs == 1 && (ai_rs & 3) == 0 && ((uintptr_t)act_in & 7) == 0;
+    for (int b = wave; b < NBM * NBN; b += WAVES) {
+        const int i = b / NBN, j = b % NBN;
+        const int m = m0 + 16 * i + r, n = n0 + 16 * j + 4 * g;
+        f32x4_acc t = *reinterpret_cast<const f32x4_acc *>(red + (b * 64 + lane) * 4);
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) t += *reinterpret_cast<const f32x4_acc *>(red + ((w * (NBM * NBN) + b) * 64 + lane) * 4);
+        if (m >= M || n >= N) continue;
+        float v[4], y[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[e] = t[e] + ((bias != nullptr && n + e < N) ? to_float(bias[n + e]) : 0.0f);
+            y[e] = apply_act16(v[e], act);
+        }
+        if (n + 4 <= N && out_vec) {
+            const u32x2 p = {pack2<T>(y[0], y[1]), pack2<T>(y[2], y[3])};
+            *reinterpret_cast<u32x2 *>(out + (int64_t)m * out_rs + n) = p;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (n + e < N) out[(int64_t)m * out_rs + (int64_t)(n + e) * out_cs] = from_float<T>(y[e]);
+        }
+        if (act_in != nullptr) {
+            if (n + 4 <= N && ai_vec) {
+                const u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+                *reinterpret_cast<u32x2 *>(act_in + (int64_t)m * ai_rs + n) = p;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) act_in[(int64_t)m * ai_rs + (int64_t)(n + e) * ai_cs] = from_float<T>(v[e]);
+            }
+        }
+    }
+}
+
+template <typename T, int BM, int BN>
+static void launch_small_dealt(const LinearArgs &a) {
+    auto kern = linear_small_dealt_kernel<T, BM, BN>;
+    constexpr int LDS_BYTES = 4 * 32 * 1024;
+    static bool attr_done = false;  // benign race: the attribute call is idempotent
+    if (!attr_done) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        attr_done = true;
+    }
+    const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
+                       static_cast<const T *>(a.w), static_cast<const T *>(a.bias), static_cast<T *>(a.out),
+                       static_cast<T *>(a.act_in), a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs, a.ai_cs, a.act,
+                       tiles_m);
+}
+
+// rows: 16 or 32 per tile (32 columns)
+void run_small_dealt(const LinearArgs &a, int dtype, int rows) {
+    if (dtype == KERNL_F16) {
+        if (rows == 16) launch_small_dealt<f16, 16, 32>(a);
+        else launch_small_dealt<f16, 32, 32>(a);
+    } else {
+        if (rows == 16) launch_small_dealt<bf16, 16, 32>(a);
+        else launch_small_dealt<bf16, 32, 32>(a);
+    }
+}
+
 template <typename T, int BM>
 static void launch_small(const LinearArgs &a) {
     auto kern = linear_small_kernel<T, BM>;

@@ -45,6 +45,22 @@ def few_row_rule(rows: int, n: int, k: int) -> bool:
     return n * k >= FEW_ROW_MIN_WEIGHT or (k >= FEW_ROW_LONG_K and rows > 32)
 
 
+SMALL_PROBLEM_KERNELS = True   # tuning hook: False keeps such shapes on the stream-K / split-K / tile kernels
+
+
+def takes_small_problem_kernel(x2d: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether `kernl_linear_fwd` runs this product on one of its small-problem kernels (one launch of small tiles over
+    the whole K: a few hundred rows at most against a weight of a few million elements) — such shapes are not handed
+    to the stream-K or split-K entry points, which they would otherwise qualify for."""
+    M, K = x2d.shape
+    return (
+        SMALL_PROBLEM_KERNELS
+        and x2d.dtype in (torch.float16, torch.bfloat16) and weight.dtype == x2d.dtype
+        and x2d.stride(1) == 1 and x2d.stride(0) % 8 == 0 and x2d.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
+        and _lib.linear_small_kind(M, weight.shape[0], K) != 0
+    )
+
+
 def takes_few_row_kernel(x2d: torch.Tensor, weight: torch.Tensor) -> bool:
     return few_row_rule(x2d.shape[0], weight.shape[0], weight.shape[1]) and _lib.linear_fewrow_supported(x2d, weight)
 
@@ -95,8 +111,13 @@ class LinearLayer(torch.autograd.Function):
         outputs = torch.empty((M, N), device=x.device, dtype=x.dtype)
         if act_inputs is not None:
             assert act_inputs.shape == (M, N) and act_inputs.dtype == x.dtype
-        split_bytes = _lib.linear_splitk_workspace_bytes(x_, weight) if FEW_ROW_MAX_ROWS < M <= SPLIT_K_MAX_ROWS else 0
-        if act_inputs is None and takes_few_row_kernel(x_, weight):
+        small = takes_small_problem_kernel(x_, weight)
+        split_bytes = 0
+        if not small and FEW_ROW_MAX_ROWS < M <= SPLIT_K_MAX_ROWS:
+            split_bytes = _lib.linear_splitk_workspace_bytes(x_, weight)
+        if small:
+            _lib.linear_fwd(x_, weight, bias, outputs, act_inputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
+        elif act_inputs is None and takes_few_row_kernel(x_, weight):
             _lib.linear_fewrow_fwd(x_, weight, bias, None, outputs, ACTIVATIONS.get(activation, _lib.ACT_NONE))
         elif split_bytes:
             # too few 128-row tiles to occupy the chip: ranges of K per tile, added by a second launch

@@ -42,8 +42,8 @@ def test_linear_vs_oracle(shape, bias, activation, dtype, close):
 
 
 TILE_IDS = ["256x256", "256x192", "128x128", "256x128k32", "wide256x256", "wide256x192", "wide128x256", "wide128x192"]
-SMALL_TILES = [10, 11]  # 32 x 64 and 64 x 64 tiles over the whole K
-SMALL_IDS = ["small32x64", "small64x64"]
+SMALL_TILES = [10, 11, 12, 13]  # tiles over the whole K: 32 x 64, 64 x 64 (shared by the waves), 16 x 32, 32 x 32 (k-tiles dealt)
+SMALL_IDS = ["small32x64", "small64x64", "dealt16x32", "dealt32x32"]
 
 
 @pytest.mark.parametrize("tile", list(range(1, 9)) + SMALL_TILES, ids=TILE_IDS + SMALL_IDS)
@@ -97,34 +97,41 @@ def test_linear_ragged_last_k_tile(shape, tile, dtype, close):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
 @pytest.mark.parametrize("activation", ["", "fast_gelu"])
 @pytest.mark.parametrize("shape", [(65, 768, 768), (128, 2304, 768), (128, 3072, 768), (200, 1000, 448), (500, 520, 64),
-                                   (512, 1024, 1024), (1024, 700, 1480), (1000, 960, 520), (130, 70, 8)],
+                                   (512, 1024, 1024), (1024, 700, 1480), (1000, 960, 520), (130, 70, 8),
+                                   (8, 768, 3072), (16, 2304, 768), (16, 8192, 1024), (33, 768, 3080), (128, 768, 3072),
+                                   (256, 1024, 4096), (100, 2048, 2048), (20, 1000, 8192), (40, 96, 72)],
                          ids=lambda s: "x".join(map(str, s)))
-def test_linear_small_tiles_are_what_small_problems_run(shape, activation, dtype, close):
-    """65 rows and more against a short K with at most 256 small tiles: the library's own choice is the small-tile
-    kernel (one launch, whole K per workgroup).  Forcing either of its tile heights must give the same bits as the
-    heuristic for the height it picks, and all three must match the oracle: tiles ragged in rows, columns and K, fewer
-    k-tiles than ring stages, strided output."""
+def test_linear_small_problem_kernels_are_what_small_problems_run(shape, activation, dtype, close):
+    """A few hundred rows at most against a weight of a few million elements: the library's own choice is one of the
+    small-problem kernels (one launch, whole K per workgroup; `kernl_linear_small_kind` names it).  Forcing that kernel
+    must give the same bits as the heuristic, every one of the four must match the oracle, and so must the operator,
+    which must not hand such a shape to the stream-K or split-K entry points.  Tiles ragged in rows, columns and K, fewer
+    k-tiles than ring stages or waves, strided output."""
     M, N, K = shape
     gen = torch.Generator().manual_seed(57)
     x, w, b = _inputs(M, N, K, dtype, gen, w_std=K ** -0.5)
     ref = linear_oracle(x, w, b, activation)
     lib = _lib.load()
+    picked = _lib.linear_small_kind(M, N, K)
+    assert picked in SMALL_TILES
     outs = {}
-    for tile in (0, 10, 11):
+    for tile in [0] + SMALL_TILES:
+        out = torch.empty((M, N), dtype=dtype, device="cuda")
         lib.kernl_linear_force_tile(tile)
         try:
-            outs[tile] = linear_layer(x.cuda(), w.cuda(), b.cuda(), activation=activation)
+            _lib.linear_fwd(x.cuda(), w.cuda(), b.cuda(), out, None, {"": _lib.ACT_NONE, "fast_gelu": _lib.ACT_GELU_TANH}[activation])
             torch.cuda.synchronize()
         finally:
             lib.kernl_linear_force_tile(0)
-        close(outs[tile], ref, dtype, what=f"small tiles {shape} {activation!r} tile {tile}")
-    picked = 10 if -(-M // 32) * -(-N // 64) <= 256 else 11
-    assert torch.equal(outs[0], outs[picked]), "the heuristic did not run the small-tile kernel"
+        outs[tile] = out
+        close(out, ref, dtype, what=f"small problem {shape} {activation!r} tile {tile}")
+    assert torch.equal(outs[0], outs[picked]), "the heuristic did not run the kernel kernl_linear_small_kind names"
+    assert torch.equal(linear_layer(x.cuda(), w.cuda(), b.cuda(), activation=activation), outs[0])
     # a column slice of a wider buffer as the output's home: row stride != N
     wide = torch.zeros((M, N + 24), dtype=dtype, device="cuda")
     _lib.linear_fwd(x.cuda(), w.cuda(), b.cuda(), wide[:, 8:8 + N], None, _lib.ACT_NONE)
     torch.cuda.synchronize()
-    close(wide[:, 8:8 + N], linear_oracle(x, w, b, ""), dtype, what=f"small tiles {shape} strided output")
+    close(wide[:, 8:8 + N], linear_oracle(x, w, b, ""), dtype, what=f"small problem {shape} strided output")
     assert (wide[:, :8] == 0).all() and (wide[:, 8 + N:] == 0).all()
 
 
@@ -653,7 +660,7 @@ def test_linear_few_rows_stream_k_is_what_the_operators_run(close, monkeypatch):
     real = _lib.linear_fewrow_fwd
     monkeypatch.setattr(_lib, "linear_fewrow_fwd", lambda *a, **k: (calls.append(a[0].shape[0]), real(*a, **k))[1])
     gen = torch.Generator().manual_seed(59)
-    N, K = 2304, 2048
+    N, K = 4608, 2048   # 9.4 M weights: beyond what the small-problem kernels take
     w = (torch.randn((N, K), generator=gen) * K ** -0.5).half()
     b = torch.randn((N,), generator=gen).half()
     for rows, expected in ((16, 0), (17, 1), (64, 1), (65, 1), (128, 1), (129, 0)):
