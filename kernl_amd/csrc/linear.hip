@@ -18,8 +18,8 @@ static int linear_mfma_dispatch(const LinearArgs &a) {
     }
     // small problems: one launch of small tiles over the whole K (10 / 11 force its 32- / 64-row form)
     if (pick == 0 && !(a.act & kGluBit)) pick = small_problem_kind(a.M, a.N, a.K);
-    if ((pick == 12 || pick == 13) && !(a.act & kGluBit)) {
-        run_small_dealt(a, kDtype, pick == 12 ? 16 : 32);
+    if ((pick == 12 || pick == 13 || pick == 14) && !(a.act & kGluBit)) {
+        run_small_dealt(a, kDtype, pick == 12 ? 16 : pick == 13 ? 32 : 64);
         return check_launch("linear (small tiles, dealt k-tiles)");
     }
     if ((pick == 10 || pick == 11) && !(a.act & kGluBit)) {

@@ -31,8 +31,8 @@ void run_wide_w8(const LinearArgs &a);                               // fp8 e5m2
 void run_wide_half(const LinearArgs &a, int dtype, int cols);        // 128-row tiles
 void run_wide_half_w8(const LinearArgs &a);
 void run_half_split(const LinearArgs &a, const HalfSplitPlan &p, float *part, int dtype);
-void run_small(const LinearArgs &a, int dtype, int rows);            // 32- or 64-row tiles over the whole K (linear_small.hip)
-void run_small_dealt(const LinearArgs &a, int dtype, int rows);      // 16- or 32-row, 32-column tiles, k-tiles dealt to the waves
+void run_small(const LinearArgs &a, int dtype, int rows);            // 32 x 64 or 64 x 64 tiles over the whole K (linear_small.hip)
+void run_small_dealt(const LinearArgs &a, int dtype, int rows);      // 16-, 32- or 64-row, 32-column tiles, k-tiles dealt to the waves
 
 
 // ----------------------------------------------------------------------------------------------------
@@ -1691,29 +1691,29 @@ static int pick_tile(int M, int N, int K, bool gated) {
 }
 
 // Which of the small-problem kernels (linear_small.hip) takes M x N x K, as the value of the tile hook that forces it
-// (10 / 11: 32 x 64 / 64 x 64 tiles shared by the waves; 12 / 13: 16 x 32 / 32 x 32 tiles with the k-tiles dealt to the
-// waves), or 0 when the problem is not their kind.  One round of workgroups is the condition for all of them.
+// (10 / 11: 32 x 64 / 64 x 64 tiles shared by the waves; 12 / 13 / 14: 16 x 32 / 32 x 32 / 64 x 32 tiles with the k-tiles
+// dealt to the waves), or 0 when the problem is not their kind.  One round of workgroups is the condition for all of them.
 //  - dealt k-tiles: weights of up to 8 M elements, 8 rows or more (fewer stream the weight faster), at most 256 tiles.
 //    Graph replay, us, against what ran before: 16 x 768 x 3072 6.7 (9.0), 64 x 768 x 3072 8.0 (11.6), 128 x 768 x 3072
 //    8.4 (14.3), 256 x 768 x 3072 9.8 (15.8), 128 x 768 x 768 5.1 (7.3), 64 x 2304 x 768 5.4 (7.6), 128 x 2048 x 2048 9.0
-//    (15.2), 128 x 1024 x 8192 15.3 (25.3), 32 x 8192 x 1024 6.5 (10.1); 4096 x 4096 and larger stay where they were.
+//    (15.2), 128 x 1024 x 8192 15.3 (25.3), 32 x 8192 x 1024 6.5 (10.1); 64 x 32 tiles where 32 x 32 need a second round:
+//    512 x 768 x 3072 12.4 (18.3), 384 x 1024 x 4096 14.8 (18.7), 256 x 2048 x 2048 10.9 (17.1), 512 x 768 x 768 7.4 (7.6);
+//    4096 x 4096 and larger stay where they were.
 //  - shared tiles: more than 64 rows and K < 1536 (from there on the stream-K / split-K kernels or the big tiles are
 //    ahead): 128 x 2304 x 768 7.7 (11.7), 128 x 3072 x 768 8.3 (11.7), 512 x 768 x 768 7.6 (11.0), 512 x 1024 x 1024 8.6
 //    (13.0), 128 x 4096 x 1024 10.0 (14.4); 64-row tiles: 256 x 3072 x 768 11.2 (11.8), 1024 x 1024 x 1024 12.2 (14.0).
 static int small_problem_kind(int64_t M, int64_t N, int64_t K) {
     const int64_t cols32 = (N + 31) / 32, cols64 = (N + 63) / 64;
-    if (N * K <= ((int64_t)1 << 23)) {
-        if (M >= 8 && M <= 16 && cols32 <= 256) return 12;
-        if (M > 16 && ((M + 31) / 32) * cols32 <= 256) return 13;
-    }
-    if (M > 64 && K < 1536) {
-        if (((M + 31) / 32) * cols64 <= 256) return 10;
-        if (((M + 63) / 64) * cols64 <= 256) return 11;
-    }
+    const bool small_weight = N * K <= ((int64_t)1 << 23), short_k = M > 64 && K < 1536;
+    if (small_weight && M >= 8 && M <= 16 && cols32 <= 256) return 12;
+    if (small_weight && M > 16 && ((M + 31) / 32) * cols32 <= 256) return 13;
+    if (short_k && ((M + 31) / 32) * cols64 <= 256) return 10;
+    if (small_weight && M > 16 && ((M + 63) / 64) * cols32 <= 256) return 14;
+    if (short_k && ((M + 63) / 64) * cols64 <= 256) return 11;
     return 0;
 }
 
-extern int g_linear_force_tile;  // test / tuning hook (defined in linear.hip): 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192, 10 .. 13 = the small-problem kernels
+extern int g_linear_force_tile;  // test / tuning hook (defined in linear.hip): 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192, 10 .. 14 = the small-problem kernels
 
 template <typename T, bool GATED, int MB, int NR, bool W8, bool RMS = false, bool ROPE = false>
 static void launch_skinny_blocks(const LinearArgs &a, const void *rms_w = nullptr, float eps = 0.0f,

@@ -15,20 +15,22 @@
 
 namespace kernl {
 
-constexpr int kSmallStages = 8, kSmallBK = 64;  // measured against 128-wide k-tiles in 6 / 4 stages: 5-10 % faster
+constexpr int kSmallBK = 64;  // measured against 128-wide k-tiles in 6 / 4 stages: 5-10 % faster
+// ring stages of the shared-tile kernel: 8 of them, or as many as fit 144 KB
+constexpr int small_stages(int bm, int bn) { return (bm + bn) * kSmallBK * 2 * 8 <= 144 * 1024 ? 8 : (144 * 1024) / ((bm + bn) * kSmallBK * 2); }
 
-template <typename T, int BM>
+template <typename T, int BM, int BN>
 __global__ void __launch_bounds__(256, 1)
 linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
                     T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
                     int64_t ai_rs, int64_t ai_cs, int act, int tiles_m) {
     typedef typename Vec8<T>::type vec8;
-    constexpr int BN = 64, BK = kSmallBK, RB = BK * 2, CPR = BK / 8, S = kSmallStages, KSTEPS = BK / 32;
+    constexpr int BK = kSmallBK, RB = BK * 2, CPR = BK / 8, S = small_stages(BM, BN), KSTEPS = BK / 32;
     constexpr int X_BYTES = BM * RB, W_BYTES = BN * RB, STAGE = X_BYTES + W_BYTES;
     constexpr int LX = BM * CPR / 256, LW = BN * CPR / 256, L = LX + LW;  // 1 KB loads per wave... per thread and stage
     constexpr int NBM = BM / 32, NBN = BN / 32;                            // 16 x 16 blocks per wave: rows of x, rows of w
-    static_assert(BM == 32 || BM == 64, "tile heights");
-    static_assert((S - 2) * L <= 63, "the wait count must be encodable");
+    static_assert((BM == 32 || BM == 64) && (BN == 64 || BN == 128), "tile shapes");
+    static_assert(S >= 3 && (S - 2) * L <= 63, "ring depth; the wait count must be encodable");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -180,6 +182,9 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
 // — 32 x 32 or 16 x 32, up to 256 workgroups — and the four waves no longer share a tile's k-tiles but deal them out:
 // wave w multiplies k-tiles w, w + 4, ... of the WHOLE tile out of a ring of its own (no barrier in the loop, program
 // order and the load counter are all the synchronisation), and the four partial tiles meet in LDS at the end.
+// a wave's ring: 32 KB, 36 KB for the 12 KB stages of 64 x 32 tiles (three of them)
+constexpr int small_ring_bytes(int bm, int bn) { return (bm + bn) == 96 ? 36 * 1024 : 32 * 1024; }
+
 template <typename T, int BM, int BN>
 __global__ void __launch_bounds__(256, 1)
 linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
@@ -188,11 +193,11 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
     typedef typename Vec8<T>::type vec8;
     constexpr int BK = 64, RB = BK * 2, CPR = BK / 8, WAVES = 4;
     constexpr int X_BYTES = BM * RB, W_BYTES = BN * RB, STAGE = X_BYTES + W_BYTES;
-    constexpr int S = (32 * 1024) / STAGE;                          // stages of a wave's 32 KB ring
+    constexpr int RING = small_ring_bytes(BM, BN), S = RING / STAGE;  // a wave's ring and its stages
     constexpr int LX = BM * CPR / 64, LW = BN * CPR / 64, L = LX + LW;  // 1 KB loads per wave and stage
     constexpr int NBM = BM / 16, NBN = BN / 16;
     static_assert(S >= 3 && (S - 2) * L <= 63, "ring depth and wait count");
-    static_assert(WAVES * NBM * NBN * 1024 <= WAVES * 32 * 1024, "the partial tiles fit the rings");
+    static_assert(NBM * NBN * 1024 <= RING, "the partial tiles fit the rings");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -226,7 +231,7 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
         if (c * 8 < k_last) tail_bits |= 1u << (LX + i);
     }
     typedef __attribute__((address_space(3))) void lds_void;
-    const uint32_t ring = (uint32_t)(uintptr_t)(lds_void *)smem + (uint32_t)wave * (32 * 1024);
+    const uint32_t ring = (uint32_t)(uintptr_t)(lds_void *)smem + (uint32_t)wave * RING;
     auto load1 = [&](const u32x4 &rsrc, uint32_t off, uint32_t lds, int kbytes) __attribute__((always_inline)) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                      :: "s"(lds), "v"(off), "s"(rsrc), "s"(kbytes) : "memory", "m0");
@@ -261,7 +266,7 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
 #pragma unroll
     for (int j = 0; j < S - 1; ++j) request(j, j);
     int stage = 0;
-    const unsigned char *my = smem + wave * (32 * 1024);
+    const unsigned char *my = smem + wave * RING;
     for (int j = 0; j < mine; ++j) {
         __builtin_amdgcn_s_waitcnt(0x0F70 | (((S - 2) * L) & 15) | ((((S - 2) * L) >> 4) << 14));
         const unsigned char *sb = my + stage * STAGE;
@@ -334,7 +339,7 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
 template <typename T, int BM, int BN>
 static void launch_small_dealt(const LinearArgs &a) {
     auto kern = linear_small_dealt_kernel<T, BM, BN>;
-    constexpr int LDS_BYTES = 4 * 32 * 1024;
+    constexpr int LDS_BYTES = 4 * small_ring_bytes(BM, BN);
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
@@ -347,41 +352,43 @@ static void launch_small_dealt(const LinearArgs &a) {
                        tiles_m);
 }
 
-// rows: 16 or 32 per tile (32 columns)
+// rows: 16, 32 or 64 per tile (32 columns)
 void run_small_dealt(const LinearArgs &a, int dtype, int rows) {
     if (dtype == KERNL_F16) {
         if (rows == 16) launch_small_dealt<f16, 16, 32>(a);
-        else launch_small_dealt<f16, 32, 32>(a);
+        else if (rows == 32) launch_small_dealt<f16, 32, 32>(a);
+        else launch_small_dealt<f16, 64, 32>(a);
     } else {
         if (rows == 16) launch_small_dealt<bf16, 16, 32>(a);
-        else launch_small_dealt<bf16, 32, 32>(a);
+        else if (rows == 32) launch_small_dealt<bf16, 32, 32>(a);
+        else launch_small_dealt<bf16, 64, 32>(a);
     }
 }
 
-template <typename T, int BM>
+template <typename T, int BM, int BN>
 static void launch_small(const LinearArgs &a) {
-    auto kern = linear_small_kernel<T, BM>;
-    constexpr int LDS_BYTES = kSmallStages * (BM + 64) * kSmallBK * 2;
+    auto kern = linear_small_kernel<T, BM, BN>;
+    constexpr int LDS_BYTES = small_stages(BM, BN) * (BM + BN) * kSmallBK * 2;
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         attr_done = true;
     }
-    const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + 63) / 64;
+    const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), static_cast<const T *>(a.bias), static_cast<T *>(a.out),
                        static_cast<T *>(a.act_in), a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs, a.ai_cs, a.act,
                        tiles_m);
 }
 
-// rows: 32 or 64 per tile
+// rows of a tile: 32 or 64 (64 columns; 64 x 128 tiles in a ring of 6 stages were measured too and never won)
 void run_small(const LinearArgs &a, int dtype, int rows) {
     if (dtype == KERNL_F16) {
-        if (rows == 32) launch_small<f16, 32>(a);
-        else launch_small<f16, 64>(a);
+        if (rows == 32) launch_small<f16, 32, 64>(a);
+        else launch_small<f16, 64, 64>(a);
     } else {
-        if (rows == 32) launch_small<bf16, 32>(a);
-        else launch_small<bf16, 64>(a);
+        if (rows == 32) launch_small<bf16, 32, 64>(a);
+        else launch_small<bf16, 64, 64>(a);
     }
 }
 
