@@ -124,6 +124,12 @@ def main():
         "over rotating weights, and exit: the workload of the rocprofv3 --kernel-trace run behind "
         "profiles/linear_batched_decode_kernel_trace.txt",
     )
+    ap.add_argument(
+        "--small-probe",
+        action="store_true",
+        help="run BERT-base fp16 through optimize_model at batch 1 with 16, 128 and 512 tokens (30 hipGraph replays each) "
+        "and exit: the workload of the rocprofv3 --kernel-trace run behind profiles/bert_base_batch1_kernel_trace.txt",
+    )
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU per process and ships no multi-GPU path; run with --gpus 1")
@@ -161,6 +167,28 @@ def main():
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
+        return
+
+    if args.small_probe:
+        import torch._dynamo
+        from transformers import BertConfig, BertModel
+
+        from kernl_amd.model_optimization import optimize_model
+
+        torch.manual_seed(0)
+        cfg = BertConfig()
+        cfg._attn_implementation = "sdpa"
+        model = BertModel(cfg).eval().half().to(dev)
+        optimize_model(model)
+        gen = torch.Generator().manual_seed(0)
+        for seq in (16, 128, 512):
+            torch._dynamo.reset()
+            ids = torch.randint(0, 30522, (1, seq), generator=gen).to(dev)
+            mask = torch.ones_like(ids)
+            with torch.inference_mode():
+                for _ in range(33):
+                    model(input_ids=ids, attention_mask=mask)
+            torch.cuda.synchronize()
         return
 
     if args.decode_probe:
@@ -507,6 +535,18 @@ def main():
             t = graph_time_ms(mid_linears, reps=4) / len(w_sq)
             extra["linear_256x4096x4096_us_graph_replay"] = round(t * 1e3, 2)
             extra["linear_256x4096x4096_tflops"] = round(2.0 * 256 * 4096 * 4096 / (t * 1e-3) / 1e12, 1)
+            # small problems (BERT-base at batch 1 with 128 tokens): one launch of small tiles over the whole K
+            for (m_s, n_s, k_s) in ((128, 768, 3072), (128, 2304, 768), (512, 768, 3072)):
+                x_s = torch.randn((m_s, k_s), generator=gen).half().to(dev)
+                w_s = [(torch.randn((n_s, k_s), generator=gen) * k_s ** -0.5).half().to(dev) for _ in range(8)]
+                b_s = torch.randn((n_s,), generator=gen).half().to(dev)
+
+                def small_linears():
+                    for w_i in w_s:
+                        linear_layer(x_s, w_i, b_s, "gelu")
+
+                t = graph_time_ms(small_linears, reps=4) / len(w_s)
+                extra[f"linear_{m_s}x{n_s}x{k_s}_gelu_us_graph_replay"] = round(t * 1e3, 2)
             del w_dn, w_sq, x32, x32f, res32, x256
         except Exception as exc:  # the headline must still be printed
             extra["decoder_kernels_error"] = f"{type(exc).__name__}: {exc}"[:300]
