@@ -1697,7 +1697,8 @@ static int pick_tile(int M, int N, int K, bool gated) {
 //    Graph replay, us, against what ran before: 16 x 768 x 3072 6.7 (9.0), 64 x 768 x 3072 8.0 (11.6), 128 x 768 x 3072
 //    8.4 (14.3), 256 x 768 x 3072 9.8 (15.8), 128 x 768 x 768 5.1 (7.3), 64 x 2304 x 768 5.4 (7.6), 128 x 2048 x 2048 9.0
 //    (15.2), 128 x 1024 x 8192 15.3 (25.3), 32 x 8192 x 1024 6.5 (10.1); 64 x 32 tiles where 32 x 32 need a second round:
-//    512 x 768 x 3072 12.4 (18.3), 384 x 1024 x 4096 14.8 (18.7), 256 x 2048 x 2048 10.9 (17.1), 512 x 768 x 768 7.4 (7.6);
+//    512 x 768 x 3072 12.4 (18.3), 384 x 1024 x 4096 14.8 (18.7), 256 x 2048 x 2048 10.9 (17.1), 128 x 3072 x 768 7.1 (shared
+//    32 x 64 tiles: 7.9);
 //    4096 x 4096 and larger stay where they were.
 //  - shared tiles: more than 64 rows and K < 1536 (from there on the stream-K / split-K kernels or the big tiles are
 //    ahead): 128 x 2304 x 768 7.7 (11.7), 128 x 3072 x 768 8.3 (11.7), 512 x 768 x 768 7.6 (11.0), 512 x 1024 x 1024 8.6
@@ -1707,8 +1708,8 @@ static int small_problem_kind(int64_t M, int64_t N, int64_t K) {
     const bool small_weight = N * K <= ((int64_t)1 << 23), short_k = M > 64 && K < 1536;
     if (small_weight && M >= 8 && M <= 16 && cols32 <= 256) return 12;
     if (small_weight && M > 16 && ((M + 31) / 32) * cols32 <= 256) return 13;
-    if (short_k && ((M + 31) / 32) * cols64 <= 256) return 10;
     if (small_weight && M > 16 && ((M + 63) / 64) * cols32 <= 256) return 14;
+    if (short_k && ((M + 31) / 32) * cols64 <= 256) return 10;
     if (short_k && ((M + 63) / 64) * cols64 <= 256) return 11;
     return 0;
 }

@@ -110,6 +110,16 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
     for (int i = 0; i < NBM; ++i)
 #pragma unroll
         for (int j = 0; j < NBN; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+    // the bias of the lane's columns, requested before anything else: fetched where it is used, every block of the
+    // epilogue would cost the wave a memory round trip of its own
+    float bz[NBN][4];
+#pragma unroll
+    for (int j = 0; j < NBN; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int n = n0 + wave_n * (BN / 2) + 16 * j + 4 * g + e;
+            bz[j][e] = (bias != nullptr && n < N) ? to_float(bias[n]) : 0.0f;
+        }
 
 #pragma unroll
     for (int kt = 0; kt < S - 1; ++kt) request(kt, kt);
@@ -152,7 +162,7 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
             float v[4], y[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                v[e] = acc[i][j][e] + ((bias != nullptr && n + e < N) ? to_float(bias[n + e]) : 0.0f);
+                v[e] = acc[i][j][e] + bz[j][e];
                 y[e] = apply_act16(v[e], act);
             }
             if (n + 4 <= N && out_vec) {
@@ -262,6 +272,16 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
 #pragma unroll
         for (int j = 0; j < NBN; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
 
+    // the bias of the columns this wave finishes in the epilogue, requested before anything else
+    constexpr int OWN = (NBM * NBN + WAVES - 1) / WAVES;  // blocks per wave in the epilogue: wave, wave + 4, ...
+    float bz[OWN][4];
+#pragma unroll
+    for (int t = 0; t < OWN; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int n = n0 + 16 * ((wave + WAVES * t) % NBN) + 4 * g + e;
+            bz[t][e] = (bias != nullptr && n < N) ? to_float(bias[n]) : 0.0f;
+        }
     const int mine = nk > wave ? (nk - wave + WAVES - 1) / WAVES : 0;  // k-tiles of this wave
 #pragma unroll
     for (int j = 0; j < S - 1; ++j) request(j, j);
@@ -302,17 +322,20 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
 
     const bool out_vec = out_cs == 1 && (out_rs & 3) == 0 && ((uintptr_t)out & 7) == 0;
     const bool ai_vec = act_in != nullptr && ai_cs == 1 && (ai_rs & 3) == 0 && ((uintptr_t)act_in & 7) == 0;
-    for (int b = wave; b < NBM * NBN; b += WAVES) {
+#pragma unroll
+    for (int t = 0; t < OWN; ++t) {
+        const int b = wave + WAVES * t;
+        if (b >= NBM * NBN) break;
         const int i = b / NBN, j = b % NBN;
         const int m = m0 + 16 * i + r, n = n0 + 16 * j + 4 * g;
-        f32x4_acc t = *reinterpret_cast<const f32x4_acc *>(red + (b * 64 + lane) * 4);
+        f32x4_acc sum = *reinterpret_cast<const f32x4_acc *>(red + (b * 64 + lane) * 4);
 #pragma unroll
-        for (int w = 1; w < WAVES; ++w) t += *reinterpret_cast<const f32x4_acc *>(red + ((w * (NBM * NBN) + b) * 64 + lane) * 4);
+        for (int w = 1; w < WAVES; ++w) sum += *reinterpret_cast<const f32x4_acc *>(red + ((w * (NBM * NBN) + b) * 64 + lane) * 4);
         if (m >= M || n >= N) continue;
         float v[4], y[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            v[e] = t[e] + ((bias != nullptr && n + e < N) ? to_float(bias[n + e]) : 0.0f);
+            v[e] = sum[e] + bz[t][e];
             y[e] = apply_act16(v[e], act);
         }
         if (n + 4 <= N && out_vec) {

@@ -684,9 +684,8 @@ def test_small_problem_rule_of_the_library():
     assert kind(8, 8224, 1024) == 0 and kind(7, 768, 3072) == 0 and kind(1, 768, 768) == 0
     assert kind(128, 768, 3072) == 13 and kind(64, 2304, 768) == 13     # 32 x 32 tiles, k-tiles dealt to the waves
     assert kind(256, 1024, 4096) == 13 and kind(288, 1024, 4096) == 14  # 8 x 32 tiles of 32 rows fit, 9 x 32 do not: 64 rows
-    assert kind(512, 768, 3072) == 14 and kind(256, 2048, 2048) == 14   # 64 x 32 tiles, k-tiles dealt
-    assert kind(512, 768, 768) == 10                                    # ... but 32 x 64 shared tiles first when K is short
-    assert kind(128, 2304, 768) == 10 and kind(384, 2304, 768) == 11    # 32 x 64 tiles where 32 x 32 need a second round
+    assert kind(512, 768, 3072) == 14 and kind(128, 2304, 768) == 14    # 64 x 32 tiles, k-tiles dealt
+    assert kind(96, 5440, 768) == 10 and kind(384, 2304, 768) == 11     # shared 32 x 64 / 64 x 64 tiles where those need a second round
     assert kind(256, 3072, 768) == 11 and kind(1024, 1024, 1024) == 11  # 64 x 64 tiles
     assert kind(512, 3072, 768) == 0 and kind(2048, 768, 768) == 0      # more than 256 tiles either way
     assert kind(32, 4096, 4096) == 0 and kind(128, 11008, 4096) == 0    # big weights stay with the streaming kernels

@@ -99,7 +99,7 @@ def test_linear_ragged_last_k_tile(shape, tile, dtype, close):
 @pytest.mark.parametrize("shape", [(65, 768, 768), (128, 2304, 768), (128, 3072, 768), (200, 1000, 448), (500, 520, 64),
                                    (512, 1024, 1024), (1024, 700, 1480), (1000, 960, 520), (130, 70, 8),
                                    (8, 768, 3072), (16, 2304, 768), (16, 8192, 1024), (33, 768, 3080), (128, 768, 3072),
-                                   (256, 1024, 4096), (100, 2048, 2048), (20, 1000, 8192), (40, 96, 72), (512, 768, 3072), (300, 1000, 2056)],
+                                   (256, 1024, 4096), (100, 2048, 2048), (20, 1000, 8192), (40, 96, 72), (512, 768, 3072), (300, 1000, 2056), (96, 5440, 768)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_linear_small_problem_kernels_are_what_small_problems_run(shape, activation, dtype, close):
     """A few hundred rows at most against a weight of a few million elements: the library's own choice is one of the
