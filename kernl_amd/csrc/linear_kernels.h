@@ -1196,6 +1196,24 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
     float sq[MB];  // sum of squares of the x values this lane has seen, per 16-row block (RMS)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) sq[mb] = 0.0f;
+    // Bias and residual of the block this wave finishes first (unit `wave` of the epilogue), requested before the weight
+    // stream: fetched where they are used they cost the wave one more memory round trip at the very end of a kernel whose
+    // whole life is a few of them.
+    float pre_bias[NA][4], pre_res[4];
+    if constexpr (!ROPE) {
+        const int rb = wave / MB, mb = wave % MB;
+        const int nb = n0 + 16 * rb, m = 16 * mb + r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int n = nb + 4 * g + e;
+            const bool live = wave < NR * MB && m < M && n < N;
+            const int brow = GATED ? gated_row(nb) + 4 * g + e : n;
+            pre_bias[0][e] = (live && bias != nullptr) ? to_float(bias[brow]) : 0.0f;
+            if (GATED) pre_bias[NA - 1][e] = (live && bias != nullptr) ? to_float(bias[brow + 32]) : 0.0f;
+            pre_res[e] = (live && ex.residual != nullptr)
+                             ? to_float(static_cast<const T *>(ex.residual)[(int64_t)m * ex.res_rs + (int64_t)n * ex.res_cs]) : 0.0f;
+        }
+    }
     const int nchunks = K / 64;
     const int rot = (int)((blockIdx.x * 13u) % (unsigned)nchunks);
     for (int c0 = wave; c0 < nchunks; c0 += WAVES * U) {
@@ -1358,7 +1376,11 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
                 v[a] = ((t4[0] + t4[1]) + (t4[2] + t4[3])) * rstd;
             }
             if (m >= M || n >= N) continue;
-            if (bias != nullptr) {
+            const bool first = unit == wave;  // what this block needs from memory is here already
+            if (first) {
+                v[0] += pre_bias[0][e];
+                if (GATED) v[NA - 1] += pre_bias[NA - 1][e];
+            } else if (bias != nullptr) {
                 const int brow = GATED ? gated_row(nb) + 4 * g + e : n;
                 v[0] += to_float(bias[brow]);
                 if (GATED) v[NA - 1] += to_float(bias[brow + 32]);
@@ -1366,7 +1388,8 @@ linear_skinny_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *
             if (!GATED && act_in != nullptr) act_in[(int64_t)m * ai_rs + (int64_t)n * ai_cs] = from_float<T>(v[0]);
             float y = apply_act16(v[0], act);
             if (GATED) y *= v[NA - 1];
-            if (ex.residual != nullptr)
+            if (first) y += pre_res[e];
+            else if (ex.residual != nullptr)
                 y += to_float(static_cast<const T *>(ex.residual)[(int64_t)m * ex.res_rs + (int64_t)n * ex.res_cs]);
             out[(int64_t)m * out_rs + (int64_t)n * out_cs] = from_float<T>(y);
         }
