@@ -15,6 +15,21 @@
 
 namespace kernl {
 
+// bias[n .. n + 3] as floats (zeros past N or without a bias): one 8-byte load where the four are inside and aligned
+template <typename T>
+__device__ __forceinline__ void load_bias4(const T *__restrict__ bias, int n, int N, bool vec_ok, float (&dst)[4]) {
+    if (bias != nullptr && vec_ok && n + 4 <= N) {
+        const u32x2 raw = *reinterpret_cast<const u32x2 *>(bias + n);
+        typedef T pair_t __attribute__((ext_vector_type(2)));
+        const uint32_t r0 = raw[0], r1 = raw[1];  // (a bit cast straight from a vector ELEMENT reads the vector's first one)
+        const pair_t lo = __builtin_bit_cast(pair_t, r0), hi = __builtin_bit_cast(pair_t, r1);
+        dst[0] = to_float(lo[0]); dst[1] = to_float(lo[1]); dst[2] = to_float(hi[0]); dst[3] = to_float(hi[1]);
+        return;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[e] = (bias != nullptr && n + e < N) ? to_float(bias[n + e]) : 0.0f;
+}
+
 constexpr int kSmallBK = 64;  // measured against 128-wide k-tiles in 6 / 4 stages: 5-10 % faster
 // ring stages of the shared-tile kernel: 8 of them, or as many as fit 144 KB
 constexpr int small_stages(int bm, int bn) { return (bm + bn) * kSmallBK * 2 * 8 <= 144 * 1024 ? 8 : (144 * 1024) / ((bm + bn) * kSmallBK * 2); }
@@ -113,13 +128,12 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
     // the bias of the lane's columns, requested before anything else: fetched where it is used, every block of the
     // epilogue would cost the wave a memory round trip of its own
     float bz[NBN][4];
+    const bool bias_vec = ((uintptr_t)bias & 7) == 0;
 #pragma unroll
-    for (int j = 0; j < NBN; ++j)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int n = n0 + wave_n * (BN / 2) + 16 * j + 4 * g + e;
-            bz[j][e] = (bias != nullptr && n < N) ? to_float(bias[n]) : 0.0f;
-        }
+    for (int j = 0; j < NBN; ++j) {
+        const int n = n0 + wave_n * (BN / 2) + 16 * j + 4 * g;
+        load_bias4<T>(bias, n, N, bias_vec, bz[j]);
+    }
 
 #pragma unroll
     for (int kt = 0; kt < S - 1; ++kt) request(kt, kt);
@@ -275,13 +289,12 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
     // the bias of the columns this wave finishes in the epilogue, requested before anything else
     constexpr int OWN = (NBM * NBN + WAVES - 1) / WAVES;  // blocks per wave in the epilogue: wave, wave + 4, ...
     float bz[OWN][4];
+    const bool bias_vec = ((uintptr_t)bias & 7) == 0;
 #pragma unroll
-    for (int t = 0; t < OWN; ++t)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int n = n0 + 16 * ((wave + WAVES * t) % NBN) + 4 * g + e;
-            bz[t][e] = (bias != nullptr && n < N) ? to_float(bias[n]) : 0.0f;
-        }
+    for (int t = 0; t < OWN; ++t) {
+        const int n = n0 + 16 * ((wave + WAVES * t) % NBN) + 4 * g;
+        load_bias4<T>(bias, n, N, bias_vec, bz[t]);
+    }
     const int mine = nk > wave ? (nk - wave + WAVES - 1) / WAVES : 0;  // k-tiles of this wave
 #pragma unroll
     for (int j = 0; j < S - 1; ++j) request(j, j);

@@ -135,6 +135,27 @@ def test_linear_small_problem_kernels_are_what_small_problems_run(shape, activat
     assert (wide[:, :8] == 0).all() and (wide[:, 8 + N:] == 0).all()
 
 
+@pytest.mark.parametrize("tile", SMALL_TILES, ids=SMALL_IDS)
+def test_linear_small_problem_kernels_take_any_bias_alignment(tile, close):
+    """The small-problem kernels fetch a lane's four bias values as one 8-byte load where they can: a bias that starts 2
+    bytes into an allocation, and one whose last group of four crosses N, take the element-wise route."""
+    gen = torch.Generator().manual_seed(61)
+    M, N, K = 70, 330, 200
+    x, w, _ = _inputs(M, N, K, torch.float16, gen, w_std=K ** -0.5)
+    holder = torch.randn((N + 1,), generator=gen).half().cuda()
+    lib = _lib.load()
+    for b in (holder[1:], holder[:N].clone()):
+        assert b.is_contiguous() and b.shape == (N,)
+        out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+        lib.kernl_linear_force_tile(tile)
+        try:
+            _lib.linear_fwd(x.cuda(), w.cuda(), b, out, None, _lib.ACT_NONE)
+            torch.cuda.synchronize()
+        finally:
+            lib.kernl_linear_force_tile(0)
+        close(out, linear_oracle(x, w, b.cpu(), ""), what=f"tile {tile}, bias at offset {b.data_ptr() % 8}")
+
+
 def test_linear_non_contiguous_input(close):
     # reference test/test_linear_layer.py:73-78: x.mT of a contiguous [K, M] matrix
     gen = torch.Generator().manual_seed(2)
