@@ -53,6 +53,8 @@ __device__ __forceinline__ float act_gelu_erf_fast(float x) {
 
 // activation of the MFMA kernels, whose outputs are fp16 / bf16
 __device__ __forceinline__ float apply_act16(float x, int act) {
+    // (with a run-time `act` the switch becomes a tree of scalar branches per element: the common case leaves first)
+    if (act == KERNL_ACT_NONE) return x;
     switch (act) {
         case KERNL_ACT_RELU: return fmaxf(x, 0.0f);
         case KERNL_ACT_TANH: return act_tanh(x);

@@ -166,6 +166,9 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
     // ---- epilogue: bias, optional pre-activation, activation, one rounding; 4 consecutive columns per lane and block
     const bool out_vec = out_cs == 1 && (out_rs & 3) == 0 && ((uintptr_t)out & 7) == 0;
     const bool ai_vec = act_in != nullptr && ai_cs == 1 && (ai_rs & 3) == 0 && ((uintptr_t)act_in & 7) == 0;
+    // (the activation is chosen once, outside: a switch per element is a tree of scalar branches per element)
+    auto finish = [&](auto act_c) __attribute__((always_inline)) {
+    constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
     for (int i = 0; i < NBM; ++i) {
         const int m = m0 + wave_m * (BM / 2) + 16 * i + r;
@@ -177,7 +180,7 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 v[e] = acc[i][j][e] + bz[j][e];
-                y[e] = apply_act16(v[e], act);
+                y[e] = apply_act16(v[e], ACT);
             }
             if (n + 4 <= N && out_vec) {
                 const u32x2 p = {pack2<T>(y[0], y[1]), pack2<T>(y[2], y[3])};
@@ -198,6 +201,15 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
                 }
             }
         }
+    }
+    };
+    switch (act) {
+        case KERNL_ACT_RELU: finish(IntC<KERNL_ACT_RELU>()); break;
+        case KERNL_ACT_TANH: finish(IntC<KERNL_ACT_TANH>()); break;
+        case KERNL_ACT_GELU_ERF: finish(IntC<KERNL_ACT_GELU_ERF>()); break;
+        case KERNL_ACT_GELU_TANH: finish(IntC<KERNL_ACT_GELU_TANH>()); break;
+        case KERNL_ACT_SILU: finish(IntC<KERNL_ACT_SILU>()); break;
+        default: finish(IntC<KERNL_ACT_NONE>()); break;
     }
 }
 
@@ -335,6 +347,8 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
 
     const bool out_vec = out_cs == 1 && (out_rs & 3) == 0 && ((uintptr_t)out & 7) == 0;
     const bool ai_vec = act_in != nullptr && ai_cs == 1 && (ai_rs & 3) == 0 && ((uintptr_t)act_in & 7) == 0;
+    auto finish = [&](auto act_c) __attribute__((always_inline)) {
+    constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
     for (int t = 0; t < OWN; ++t) {
         const int b = wave + WAVES * t;
@@ -349,7 +363,7 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             v[e] = sum[e] + bz[t][e];
-            y[e] = apply_act16(v[e], act);
+            y[e] = apply_act16(v[e], ACT);
         }
         if (n + 4 <= N && out_vec) {
             const u32x2 p = {pack2<T>(y[0], y[1]), pack2<T>(y[2], y[3])};
@@ -369,6 +383,15 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
                     if (n + e < N) act_in[(int64_t)m * ai_rs + (int64_t)(n + e) * ai_cs] = from_float<T>(v[e]);
             }
         }
+    }
+    };
+    switch (act) {
+        case KERNL_ACT_RELU: finish(IntC<KERNL_ACT_RELU>()); break;
+        case KERNL_ACT_TANH: finish(IntC<KERNL_ACT_TANH>()); break;
+        case KERNL_ACT_GELU_ERF: finish(IntC<KERNL_ACT_GELU_ERF>()); break;
+        case KERNL_ACT_GELU_TANH: finish(IntC<KERNL_ACT_GELU_TANH>()); break;
+        case KERNL_ACT_SILU: finish(IntC<KERNL_ACT_SILU>()); break;
+        default: finish(IntC<KERNL_ACT_NONE>()); break;
     }
 }
 
