@@ -124,4 +124,19 @@ struct FewRowStageMap {
     static KERNL_HD int frag_offset(int mb, int r, int g, int s) { return swz_offset<128>(16 * mb + r, 2 * g + s); }
 };
 
+// ----------------------------------------------------------------------------------------------------
+// Small-problem linear kernels (linear_small.hip): an operand tile of a k-tile is ROWS rows of 128 bytes (64 k-values)
+// whose eight 16-byte chunks are XOR-swizzled.  Tile loads write LDS directly, a wave's load filling 1 KB of consecutive
+// LDS: the lane that writes LDS chunk q (byte 16 q of the tile) fetches from memory what belongs there.
+//   loads     LDS chunk q holds chunk load_chunk(q) (k = 8 load_chunk(q) .. + 7) of tile row load_row(q)
+//   reads     lane (r = lane % 16, g = lane / 16) takes, for 16-row block b and k-step s, the 16 bytes at
+//             frag_offset(16 b + r, s, g): k = 32 s + 8 g .. + 7 of that row
+// ----------------------------------------------------------------------------------------------------
+struct SmallTileMap {
+    static constexpr int ROW_BYTES = 128, CHUNKS_PER_ROW = 8;
+    static KERNL_HD int load_row(int q) { return q / CHUNKS_PER_ROW; }
+    static KERNL_HD int load_chunk(int q) { return swz_chunk<ROW_BYTES>(q / CHUNKS_PER_ROW, q % CHUNKS_PER_ROW); }
+    static KERNL_HD int frag_offset(int row, int kstep, int g) { return swz_offset<ROW_BYTES>(row, 4 * kstep + g); }
+};
+
 }  // namespace kernl

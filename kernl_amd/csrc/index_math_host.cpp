@@ -86,6 +86,16 @@ int kernl_idx_wide_weight_row(int layout, int row) {
     return -1;
 }
 
+// which: 0 load_row(q=a), 1 load_chunk(q=a), 2 frag_offset(row=a, kstep=b, g=c)
+int kernl_idx_small_tile(int which, int a, int b, int c) {
+    switch (which) {
+        case 0: return SmallTileMap::load_row(a);
+        case 1: return SmallTileMap::load_chunk(a);
+        case 2: return SmallTileMap::frag_offset(a, b, c);
+    }
+    return -1;
+}
+
 int kernl_idx_fewrow(int row_blocks, int units_per_stage, int which, int a, int b, int c, int d) {
     if (row_blocks == 1 && units_per_stage == 4) return fewrow_index<1, 4>(which, a, b, c, d);
     if (row_blocks == 2 && units_per_stage == 2) return fewrow_index<2, 2>(which, a, b, c, d);

@@ -41,6 +41,7 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
                     int64_t ai_rs, int64_t ai_cs, int act, int tiles_m) {
     typedef typename Vec8<T>::type vec8;
     constexpr int BK = kSmallBK, RB = BK * 2, CPR = BK / 8, S = small_stages(BM, BN), KSTEPS = BK / 32;
+    static_assert(RB == SmallTileMap::ROW_BYTES && CPR == SmallTileMap::CHUNKS_PER_ROW, "tile rows as the tile map lays them out");
     constexpr int X_BYTES = BM * RB, W_BYTES = BN * RB, STAGE = X_BYTES + W_BYTES;
     constexpr int LX = BM * CPR / 256, LW = BN * CPR / 256, L = LX + LW;  // 1 KB loads per wave... per thread and stage
     constexpr int NBM = BM / 32, NBN = BN / 32;                            // 16 x 16 blocks per wave: rows of x, rows of w
@@ -67,13 +68,13 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
 #pragma unroll
     for (int i = 0; i < LX; ++i) {
         const int q = (wave * LX + i) * 64 + lane;
-        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        const int row = SmallTileMap::load_row(q), c = SmallTileMap::load_chunk(q);
         xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) : kOutOfRange;
     }
 #pragma unroll
     for (int i = 0; i < LW; ++i) {
         const int q = (wave * LW + i) * 64 + lane;
-        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        const int row = SmallTileMap::load_row(q), c = SmallTileMap::load_chunk(q);
         wd[i] = row < rows_w ? (uint32_t)(((int64_t)row * K + c * 8) * 2) : kOutOfRange;
     }
     // bit l of tail_bits: the chunk load l of this lane fetches starts below K in the last k-tile
@@ -83,12 +84,12 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
 #pragma unroll
     for (int i = 0; i < LX; ++i) {
         const int q = (wave * LX + i) * 64 + lane;
-        if (swz_chunk<RB>(q / CPR, q % CPR) * 8 < k_last) tail_bits |= 1u << i;
+        if (SmallTileMap::load_chunk(q) * 8 < k_last) tail_bits |= 1u << i;
     }
 #pragma unroll
     for (int i = 0; i < LW; ++i) {
         const int q = (wave * LW + i) * 64 + lane;
-        if (swz_chunk<RB>(q / CPR, q % CPR) * 8 < k_last) tail_bits |= 1u << (LX + i);
+        if (SmallTileMap::load_chunk(q) * 8 < k_last) tail_bits |= 1u << (LX + i);
     }
     typedef __attribute__((address_space(3))) void lds_void;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
@@ -115,9 +116,9 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st) {
 #pragma unroll
-        for (int i = 0; i < NBM; ++i) xoff[st][i] = swz_offset<RB>(wave_m * (BM / 2) + 16 * i + r, 4 * st + g);
+        for (int i = 0; i < NBM; ++i) xoff[st][i] = SmallTileMap::frag_offset(wave_m * (BM / 2) + 16 * i + r, st, g);
 #pragma unroll
-        for (int j = 0; j < NBN; ++j) woff[st][j] = X_BYTES + swz_offset<RB>(wave_n * (BN / 2) + 16 * j + r, 4 * st + g);
+        for (int j = 0; j < NBN; ++j) woff[st][j] = X_BYTES + SmallTileMap::frag_offset(wave_n * (BN / 2) + 16 * j + r, st, g);
     }
 
     f32x4_acc acc[NBM][NBN];  // block (i, j): lane (r, g) holds x row 16 i + r, output columns 16 j + 4 g .. + 3
@@ -228,6 +229,7 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
                           int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int act, int tiles_m) {
     typedef typename Vec8<T>::type vec8;
     constexpr int BK = 64, RB = BK * 2, CPR = BK / 8, WAVES = 4;
+    static_assert(RB == SmallTileMap::ROW_BYTES && CPR == SmallTileMap::CHUNKS_PER_ROW, "tile rows as the tile map lays them out");
     constexpr int X_BYTES = BM * RB, W_BYTES = BN * RB, STAGE = X_BYTES + W_BYTES;
     constexpr int RING = small_ring_bytes(BM, BN), S = RING / STAGE;  // a wave's ring and its stages
     constexpr int LX = BM * CPR / 64, LW = BN * CPR / 64, L = LX + LW;  // 1 KB loads per wave and stage
@@ -255,14 +257,14 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
 #pragma unroll
     for (int i = 0; i < LX; ++i) {
         const int q = i * 64 + lane;
-        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        const int row = SmallTileMap::load_row(q), c = SmallTileMap::load_chunk(q);
         xd[i] = row < rows_x ? (uint32_t)(((int64_t)row * ldx + c * 8) * 2) : kOutOfRange;
         if (c * 8 < k_last) tail_bits |= 1u << i;
     }
 #pragma unroll
     for (int i = 0; i < LW; ++i) {
         const int q = i * 64 + lane;
-        const int row = q / CPR, c = swz_chunk<RB>(row, q % CPR);
+        const int row = SmallTileMap::load_row(q), c = SmallTileMap::load_chunk(q);
         wd[i] = row < rows_w ? (uint32_t)(((int64_t)row * K + c * 8) * 2) : kOutOfRange;
         if (c * 8 < k_last) tail_bits |= 1u << (LX + i);
     }
@@ -288,9 +290,9 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
 #pragma unroll
-        for (int i = 0; i < NBM; ++i) xoff[st][i] = swz_offset<RB>(16 * i + r, 4 * st + g);
+        for (int i = 0; i < NBM; ++i) xoff[st][i] = SmallTileMap::frag_offset(16 * i + r, st, g);
 #pragma unroll
-        for (int j = 0; j < NBN; ++j) woff[st][j] = X_BYTES + swz_offset<RB>(16 * j + r, 4 * st + g);
+        for (int j = 0; j < NBN; ++j) woff[st][j] = X_BYTES + SmallTileMap::frag_offset(16 * j + r, st, g);
     }
     f32x4_acc acc[NBM][NBN];
 #pragma unroll

@@ -16,13 +16,15 @@ class IndexLib:
     ATTN = {"stage_row": 0, "k_stage_chunk": 1, "v_stage_chunk": 2, "k_frag_offset": 3, "v_frag_offset": 4}
     MASK = {"stage_row": 0, "stage_chunk": 1, "read_offset": 2}
     WIDE = {"256": 0, "192": 1, "gated": 2}
+    SMALL = {"load_row": 0, "load_chunk": 1, "frag_offset": 2}
     FEWROW = {"piece_unit": 0, "piece_row": 1, "piece_index": 2, "piece_dst": 3, "frag_offset": 4, "pieces_per_thread": 5,
               "unit_bytes": 6}
 
     def __init__(self, cdll):
         self._c = cdll
         for name, n in (("kernl_idx_rowperm16", 1), ("kernl_idx_swz_offset", 3), ("kernl_idx_attention", 5),
-                        ("kernl_idx_mask", 5), ("kernl_idx_wide_weight_row", 2), ("kernl_idx_fewrow", 7)):
+                        ("kernl_idx_mask", 5), ("kernl_idx_wide_weight_row", 2), ("kernl_idx_fewrow", 7),
+                        ("kernl_idx_small_tile", 4)):
             fn = getattr(cdll, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.c_int] * n
@@ -44,6 +46,9 @@ class IndexLib:
 
     def fewrow(self, row_blocks: int, units_per_stage: int, what: str, a: int = 0, b: int = 0, c: int = 0, d: int = 0) -> int:
         return self._checked(self._c.kernl_idx_fewrow(row_blocks, units_per_stage, self.FEWROW[what], a, b, c, d))
+
+    def small_tile(self, what: str, a: int, b: int = 0, c: int = 0) -> int:
+        return self._checked(self._c.kernl_idx_small_tile(self.SMALL[what], a, b, c))
 
     @staticmethod
     def _checked(v: int) -> int:

@@ -135,3 +135,16 @@ def test_few_row_stage_of_x_is_written_once_and_read_without_conflicts(row_block
     assert writes.conflict_free, (writes.passes, writes.cycles)
     assert reads.conflict_free, (reads.passes, reads.cycles)
     assert reads.instructions == units_per_stage * row_blocks * 2
+
+
+@pytest.mark.parametrize("rows", [16, 32, 64])
+def test_small_problem_tile_is_loaded_once_and_read_without_conflicts(rows):
+    """An operand tile of the small-problem linear kernels, replayed from the kernels' own index functions: the direct-to-LDS
+    loads bring every (row, chunk) of the tile exactly once, every lane's fragment reads return k = 32 s + 8 g .. + 7 of
+    row 16 b + r (what `v_mfma_f32_16x16x32` expects of either operand), and no read conflicts on banks."""
+    from kernl_amd.debugger.small_replay import replay_tile
+
+    reads = replay_tile(rows)
+    assert reads.conflict_free, (reads.passes, reads.cycles)
+    assert reads.instructions == rows // 16 * 2
+
