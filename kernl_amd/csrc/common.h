@@ -82,6 +82,20 @@ __device__ __forceinline__ void mfma16_inplace(f16x8 a, f16x8 b, f32x4_acc &c) {
 __device__ __forceinline__ void mfma16_inplace(bf16x8 a, bf16x8 b, f32x4_acc &c) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
+// To the compiler the instruction above is opaque text: it inserts none of the wait states that a read of a matrix
+// instruction's result needs (11 after an 8-pass instruction), so the copies out of the accumulation registers with
+// which an epilogue begins could follow the last MFMA directly and see registers that some lanes' results have not
+// reached yet.  Call this between the last mfma16_inplace and the first use of the accumulators: 16 wait states, then
+// every accumulator passes through an empty statement that the copies depend on (volatile statements keep their
+// order, and a copy cannot move above the statement that produces its source).
+template <int NA, int NB_>
+__device__ __forceinline__ void mfma16_inplace_results_landed(f32x4_acc (&acc)[NA][NB_]) {
+    asm volatile("s_nop 15");
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+#pragma unroll
+        for (int j = 0; j < NB_; ++j) asm volatile("" : "+a"(acc[i][j]));
+}
 
 // ----------------------------------------------------------------------------------------------------
 // conversions

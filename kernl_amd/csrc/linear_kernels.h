@@ -625,11 +625,20 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         const int q = (wave * LOADS_W + i) * 64 + lane;
         if (swz_chunk<RBW>(q / CPRW, q % CPRW) * (16 / WB) < k_last) tail_bits |= 1u << (LOADS + i);
     }
+    // The offsets are clipped IN PLACE when the ragged k-tile is the next one to request (it is the last k-tile of its
+    // output tile: the next tile's offsets are computed afresh) — a branch taken once per output tile, and never when
+    // K % 64 == 0; a select per load would put three VALU instructions per load into every k-tile of every shape.
+    const int tail_kt = (K % BK) != 0 ? nk - 1 : -1;
+    auto clip_tail = [&]() __attribute__((always_inline)) {
+        asm volatile("" ::: "memory");  // keeps this a branch: without it the compiler turns the block into selects
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) xd[i] = ((tail_bits >> i) & 1u) != 0 ? xd[i] : kOutOfRange;
+#pragma unroll
+        for (int i = 0; i < LOADS_W; ++i) wd[i] = ((tail_bits >> (LOADS + i)) & 1u) != 0 ? wd[i] : kOutOfRange;
+    };
     // load l (0 .. NL-1) of a k-tile: the x loads, then the w loads
-    // `keep`: bit l clear sends load l out of range (all ones for a whole k-tile, `tail_bits` for the ragged one)
-    auto tile_load = [&](int l, int stage, int k0, uint32_t keep) __attribute__((always_inline)) {
-        uint32_t off = l < LOADS ? xd[l] : wd[l - LOADS];
-        off = ((keep >> l) & 1u) != 0 ? off : kOutOfRange;
+    auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
+        const uint32_t off = l < LOADS ? xd[l] : wd[l - LOADS];
         if (l < LOADS) load4(xrsrc, off, lds_base + stage * X_BYTES + wave * (LOADS * 1024), l >> 2, l & 3, k0 * 2);
         else load4(wrsrc, off, lds_base + W_BASE + stage * W_BYTES + wave * (LOADS_W * 1024), (l - LOADS) >> 2, (l - LOADS) & 3, k0 * WB);
     };
@@ -669,6 +678,7 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     // the load side runs ahead of the multiply side: (load_idx, load_kt) is the next k-tile to request
     int load_idx = idx, load_kt = 0;
     set_load_tile(true, m0, n0);
+    if (tail_kt == 0) clip_tail();
     auto advance_load = [&]() __attribute__((always_inline)) {
         if (++load_kt == nk) {
             load_kt = 0;
@@ -677,12 +687,13 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
             const bool more = tile_origin(load_idx, lm0, ln0);
             set_load_tile(more, lm0, ln0);
         }
+        if (load_kt == tail_kt) clip_tail();
     };
 #pragma unroll
-    for (int l = 0; l < NL; ++l) tile_load(l, 0, load_kt * BK, load_kt == nk - 1 ? tail_bits : ~0u);
+    for (int l = 0; l < NL; ++l) tile_load(l, 0, load_kt * BK);
     advance_load();
 #pragma unroll
-    for (int l = 0; l < NL; ++l) tile_load(l, 1, load_kt * BK, load_kt == nk - 1 ? tail_bits : ~0u);
+    for (int l = 0; l < NL; ++l) tile_load(l, 1, load_kt * BK);
     advance_load();
     // vmcnt(NL): the first k-tile has landed, the second may still be in flight
     __builtin_amdgcn_s_waitcnt(0x0F70 | (NL & 15) | ((NL >> 4) << 14));
@@ -704,7 +715,6 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     // waiting for "everything outstanding" would only wait for the previous tile's output stores.
     auto k_tile = [&](auto cur_c, bool landed) __attribute__((always_inline)) {
         constexpr int CUR = decltype(cur_c)::value;
-        const uint32_t keep = load_kt == nk - 1 ? tail_bits : ~0u;  // the k-tile requested during this one may be the ragged one
         const int k0 = load_kt * BK;
 #pragma unroll
         for (int st = 0; st < KSTEPS; ++st) {
@@ -732,7 +742,7 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
                 } else if (W8 && m % PERIOD == 1 && slot >= 2 && slot - 2 < NBN) {
                     fa[sn][slot - 2] = widen8(wraw[slot - 2]);  // two read slots later: the bytes have arrived
                 } else if (m % PERIOD == PERIOD - 2 && st == 1 && slot < NL) {
-                    tile_load(slot, CUR, k0, keep);
+                    tile_load(slot, CUR, k0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -758,6 +768,7 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
             k_tile(IntC<0>(), landed);
             advance_load();
         }
+        mfma16_inplace_results_landed(acc);
 
         // all bias entries of the lane's columns in one go: one memory round trip per tile.  Its wait also covers the
         // loads of the next k-tile, which were issued earlier.
@@ -894,10 +905,18 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
         const int q = (wave * LOADS_W + i) * 64 + lane;
         if (swz_chunk<RBW>(q / CPRW, q % CPRW) * (16 / WB) < k_last) tail_bits |= 1u << (LOADS_X + i);
     }
+    // clipped in place when the ragged k-tile is the next one to request: every request after it is for that k-tile
+    // again.  A branch that K % 64 == 0 never takes; a select per load would cost every k-tile of every shape.
+    const int tail_k0 = (K % BK) != 0 ? (nk_all - 1) * BK : -1;
+    auto clip_tail = [&]() __attribute__((always_inline)) {
+        asm volatile("" ::: "memory");  // keeps this a branch: without it the compiler turns the block into selects
+#pragma unroll
+        for (int i = 0; i < LOADS_X; ++i) xd[i] = ((tail_bits >> i) & 1u) != 0 ? xd[i] : kOutOfRange;
+#pragma unroll
+        for (int i = 0; i < LOADS_W; ++i) wd[i] = ((tail_bits >> (LOADS_X + i)) & 1u) != 0 ? wd[i] : kOutOfRange;
+    };
     auto tile_load = [&](int l, int stage, int k0) __attribute__((always_inline)) {
-        const uint32_t keep = k0 == (nk_all - 1) * BK ? tail_bits : ~0u;
-        uint32_t off = l < LOADS_X ? xd[l] : wd[l - LOADS_X];
-        off = ((keep >> l) & 1u) != 0 ? off : kOutOfRange;
+        const uint32_t off = l < LOADS_X ? xd[l] : wd[l - LOADS_X];
         if (l < LOADS_X) load4(xrsrc, off, lds_base + stage * X_STAGE + wave * (LOADS_X * 1024), 0, l, k0 * 2);
         else load4(wrsrc, off, lds_base + W_BASE + stage * W_STAGE + wave * (LOADS_W * 1024), (l - LOADS_X) >> 2, (l - LOADS_X) & 3, k0 * WB);
     };
@@ -930,9 +949,12 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
         nk = min(per_split, nk - kb);   // the host keeps every range non-empty
     }
 #pragma unroll
-    for (int s3 = 0; s3 < 3; ++s3)
+    for (int s3 = 0; s3 < 3; ++s3) {
+        const int k0 = (kb + min(s3, nk - 1)) * BK;
+        if (k0 == tail_k0) clip_tail();   // (clipping twice changes nothing)
 #pragma unroll
-        for (int l = 0; l < NL; ++l) tile_load(l, s3, (kb + min(s3, nk - 1)) * BK);
+        for (int l = 0; l < NL; ++l) tile_load(l, s3, k0);
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * NL) & 15) | (((2 * NL) >> 4) << 14));  // vmcnt(2 NL): k-tile 0 has landed
     __syncthreads();
 
@@ -975,6 +997,7 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     auto k_tile = [&](auto cur_c, int kt) __attribute__((always_inline)) {
         constexpr int CUR = decltype(cur_c)::value, NXT = (CUR + 1) % 3;
         const int k_next = (kb + min(kt + 3, nk - 1)) * BK;
+        if (k_next == tail_k0 && kt + 3 == nk - 1) clip_tail();   // once: later requests are for this k-tile again
 #pragma unroll
         for (int st = 0; st < KSTEPS; ++st) {
             const int sn = st ^ 1;
@@ -1020,6 +1043,7 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     }
     if (kt < nk) k_tile(IntC<0>(), kt);
     if (kt + 1 < nk) k_tile(IntC<1>(), kt + 1);
+    mfma16_inplace_results_landed(acc);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no load may still be writing LDS when the workgroup ends
 
     if constexpr (SPLIT) {
