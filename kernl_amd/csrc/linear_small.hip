@@ -98,17 +98,25 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                      :: "s"(lds), "v"(off), "s"(rsrc), "s"(kbytes) : "memory", "m0");
     };
-    // k-tile kt into stage `stage`; past the last k-tile the loads are pointed out of range (the counts stay exact)
+    // The offsets are clipped in place, under a branch taken twice per workgroup: to the chunks below K when the last
+    // k-tile is requested, to nothing at the first request past it (the counts stay exact: every slot issues its loads).
+    // A select per load would put three VALU instructions per load into every k-tile.
+    auto clip = [&](uint32_t keep) __attribute__((always_inline)) {
+        asm volatile("" ::: "memory");  // keeps this a branch: without it the compiler turns the block into selects
+#pragma unroll
+        for (int i = 0; i < LX; ++i) xd[i] = ((keep >> i) & 1u) != 0 ? xd[i] : kOutOfRange;
+#pragma unroll
+        for (int i = 0; i < LW; ++i) wd[i] = ((keep >> (LX + i)) & 1u) != 0 ? wd[i] : kOutOfRange;
+    };
+    // k-tile kt into stage `stage`
     auto request = [&](int kt, int stage) __attribute__((always_inline)) {
-        const uint32_t keep = kt < nk - 1 ? ~0u : kt == nk - 1 ? tail_bits : 0u;
+        if (kt == nk - 1 || kt == nk) clip(kt == nk ? 0u : tail_bits);
         const uint32_t base = lds_base + (uint32_t)stage * STAGE;
         const int kbytes = kt < nk ? kt * BK * 2 : 0;
 #pragma unroll
-        for (int i = 0; i < LX; ++i)
-            load1(xrsrc, ((keep >> i) & 1u) != 0 ? xd[i] : kOutOfRange, base + (wave * LX + i) * 1024, kbytes);
+        for (int i = 0; i < LX; ++i) load1(xrsrc, xd[i], base + (wave * LX + i) * 1024, kbytes);
 #pragma unroll
-        for (int i = 0; i < LW; ++i)
-            load1(wrsrc, ((keep >> (LX + i)) & 1u) != 0 ? wd[i] : kOutOfRange, base + X_BYTES + (wave * LW + i) * 1024, kbytes);
+        for (int i = 0; i < LW; ++i) load1(wrsrc, wd[i], base + X_BYTES + (wave * LW + i) * 1024, kbytes);
     };
 
     // LDS byte offsets of this lane's fragments inside a stage: block rows, k-step st, 8 k-values per 16-byte unit
@@ -275,16 +283,24 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
                      :: "s"(lds), "v"(off), "s"(rsrc), "s"(kbytes) : "memory", "m0");
     };
     // the wave's j-th k-tile (k-tile wave + 4 j of the problem) into stage `stage` of its ring
+    // offsets clipped in place under a branch (as in the shared-tile kernel): to the chunks below K for the last k-tile
+    // of the problem, to nothing at the wave's first request past it
+    auto clip = [&](uint32_t keep) __attribute__((always_inline)) {
+        asm volatile("" ::: "memory");  // keeps this a branch: without it the compiler turns the block into selects
+#pragma unroll
+        for (int i = 0; i < LX; ++i) xd[i] = ((keep >> i) & 1u) != 0 ? xd[i] : kOutOfRange;
+#pragma unroll
+        for (int i = 0; i < LW; ++i) wd[i] = ((keep >> (LX + i)) & 1u) != 0 ? wd[i] : kOutOfRange;
+    };
     auto request = [&](int j, int stage) __attribute__((always_inline)) {
         const int kt = wave + WAVES * j;
-        const uint32_t keep = kt < nk - 1 ? ~0u : kt == nk - 1 ? tail_bits : 0u;
+        if (kt >= nk - 1 && kt < nk + WAVES) clip(kt >= nk ? 0u : tail_bits);
         const uint32_t base = ring + (uint32_t)stage * STAGE;
         const int kbytes = kt < nk ? kt * BK * 2 : 0;
 #pragma unroll
-        for (int i = 0; i < LX; ++i) load1(xrsrc, ((keep >> i) & 1u) != 0 ? xd[i] : kOutOfRange, base + i * 1024, kbytes);
+        for (int i = 0; i < LX; ++i) load1(xrsrc, xd[i], base + i * 1024, kbytes);
 #pragma unroll
-        for (int i = 0; i < LW; ++i)
-            load1(wrsrc, ((keep >> (LX + i)) & 1u) != 0 ? wd[i] : kOutOfRange, base + X_BYTES + i * 1024, kbytes);
+        for (int i = 0; i < LW; ++i) load1(wrsrc, wd[i], base + X_BYTES + i * 1024, kbytes);
     };
     int xoff[2][NBM], woff[2][NBN];
 #pragma unroll
