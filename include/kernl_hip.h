@@ -238,7 +238,7 @@ int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float eps, const
 
 /*
  * Whether kernl_linear_fwd runs M x N x K (16-bit, plain epilogue, x with unit feature stride) on one of its
- * small-problem kernels, and which: 0 = no; otherwise the kernl_linear_force_tile value of the kernel (10 .. 14).  A
+ * small-problem kernels, and which: 0 = no; otherwise the kernl_linear_force_tile value of the kernel (10 .. 15).  A
  * caller that would otherwise route such a shape to the stream-K or split-K entry points (kernl_linear_fewrow_fwd,
  * kernl_linear_splitk_fwd) should call kernl_linear_fwd instead: a few hundred rows against a weight of a few million
  * elements run faster as one launch of small tiles.  No counterpart in the reference, which has one kernel and an
@@ -381,9 +381,9 @@ int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, 
  *                                wave per SIMD: 5 = 256x256, 6 = 256x192; its one-tile-per-workgroup variant with
  *                                three LDS stages: 7 = 128x256, 8 = 128x192 (5..8 take any K the MFMA path takes, with
  *                                a zero-filled last k-tile when K % 64 != 0; gated epilogues take 1, 3 or 5);
- *                                10 .. 14 = the small-problem kernels (one launch of small tiles over the whole K:
+ *                                10 .. 15 = the small-problem kernels (one launch of small tiles over the whole K:
  *                                32 x 64 / 64 x 64 tiles shared by the waves, 16 x 32 / 32 x 32 / 64 x 32 tiles with the
- *                                k-tiles dealt to the waves); the heuristic takes them where kernl_linear_small_kind
+ *                                k-tiles dealt to the waves, 15 = 64 x 128 shared tiles); the heuristic takes them where kernl_linear_small_kind
  *                                says so.  With the heuristic, inputs of at most
  *                                64 rows and K % 64 == 0 go to a kernel that streams the weight once (16 output
  *                                columns per workgroup); 9 = that kernel where it applies, the heuristic elsewhere;

@@ -132,6 +132,15 @@ struct FewRowStageMap {
 //   reads     lane (r = lane % 16, g = lane / 16) takes, for 16-row block b and k-step s, the 16 bytes at
 //             frag_offset(16 b + r, s, g): k = 32 s + 8 g .. + 7 of that row
 // ----------------------------------------------------------------------------------------------------
+// Workgroups of a launch are dealt to the 8 XCDs in turn (workgroup b runs on XCD b % 8), and each XCD has an L2 of its
+// own.  This maps workgroup b of n to a tile index such that every XCD works on ONE contiguous run of indices: with the
+// row tile running fastest in the index, the workgroups that share a weight tile then sit on one XCD at the same time
+// and all but the first of them find it in that L2.  A bijection of 0 .. n-1 for every n.
+KERNL_HD int xcd_contiguous_index(int b, int n) {
+    const int xcd = b % 8, slot = b / 8, base = n / 8, rem = n % 8;
+    return xcd * base + (xcd < rem ? xcd : rem) + slot;
+}
+
 struct SmallTileMap {
     static constexpr int ROW_BYTES = 128, CHUNKS_PER_ROW = 8;
     static KERNL_HD int load_row(int q) { return q / CHUNKS_PER_ROW; }

@@ -86,6 +86,8 @@ int kernl_idx_wide_weight_row(int layout, int row) {
     return -1;
 }
 
+int kernl_idx_xcd_contiguous(int b, int n) { return xcd_contiguous_index(b, n); }
+
 // which: 0 load_row(q=a), 1 load_chunk(q=a), 2 frag_offset(row=a, kstep=b, g=c)
 int kernl_idx_small_tile(int which, int a, int b, int c) {
     switch (which) {

@@ -16,14 +16,14 @@ static int linear_mfma_dispatch(const LinearArgs &a) {
         else launch_skinny<T, false>(a);
         return check_launch("linear (skinny)");
     }
-    // small problems: one launch of small tiles over the whole K (10 / 11 force its 32- / 64-row form)
+    // small problems: one launch of small tiles over the whole K (10 / 11 / 15 force its 32 x 64 / 64 x 64 / 64 x 128 form)
     if (pick == 0 && !(a.act & kGluBit)) pick = small_problem_kind(a.M, a.N, a.K);
     if ((pick == 12 || pick == 13 || pick == 14) && !(a.act & kGluBit)) {
         run_small_dealt(a, kDtype, pick == 12 ? 16 : pick == 13 ? 32 : 64);
         return check_launch("linear (small tiles, dealt k-tiles)");
     }
-    if ((pick == 10 || pick == 11) && !(a.act & kGluBit)) {
-        run_small(a, kDtype, pick == 10 ? 32 : 64);
+    if ((pick == 10 || pick == 11 || pick == 15) && !(a.act & kGluBit)) {
+        run_small(a, kDtype, pick == 10 ? 32 : 64, pick == 15 ? 128 : 64);
         return check_launch("linear (small tiles)");
     }
     if (pick == 0 || pick == 9) pick = pick_tile(a.M, a.N, a.K, (a.act & kGluBit) != 0);

@@ -31,7 +31,7 @@ void run_wide_w8(const LinearArgs &a);                               // fp8 e5m2
 void run_wide_half(const LinearArgs &a, int dtype, int cols);        // 128-row tiles
 void run_wide_half_w8(const LinearArgs &a);
 void run_half_split(const LinearArgs &a, const HalfSplitPlan &p, float *part, int dtype);
-void run_small(const LinearArgs &a, int dtype, int rows);            // 32 x 64 or 64 x 64 tiles over the whole K (linear_small.hip)
+void run_small(const LinearArgs &a, int dtype, int rows, int cols);  // 32 x 64, 64 x 64 or 64 x 128 tiles over the whole K (linear_small.hip)
 void run_small_dealt(const LinearArgs &a, int dtype, int rows);      // 16-, 32- or 64-row, 32-column tiles, k-tiles dealt to the waves
 
 
@@ -1738,8 +1738,8 @@ static int pick_tile(int M, int N, int K, bool gated) {
 }
 
 // Which of the small-problem kernels (linear_small.hip) takes M x N x K, as the value of the tile hook that forces it
-// (10 / 11: 32 x 64 / 64 x 64 tiles shared by the waves; 12 / 13 / 14: 16 x 32 / 32 x 32 / 64 x 32 tiles with the k-tiles
-// dealt to the waves), or 0 when the problem is not their kind.  One round of workgroups is the condition for all of them.
+// (10 / 11 / 15: 32 x 64 / 64 x 64 / 64 x 128 tiles shared by the waves; 12 / 13 / 14: 16 x 32 / 32 x 32 / 64 x 32 tiles with
+// the k-tiles dealt to the waves), or 0 when the problem is not their kind.  One round of workgroups is the condition for all of them.
 //  - dealt k-tiles: weights of up to 8 M elements, 8 rows or more (fewer stream the weight faster), at most 256 tiles.
 //    Graph replay, us, against what ran before: 16 x 768 x 3072 6.7 (9.0), 64 x 768 x 3072 8.0 (11.6), 128 x 768 x 3072
 //    8.4 (14.3), 256 x 768 x 3072 9.8 (15.8), 128 x 768 x 768 5.1 (7.3), 64 x 2304 x 768 5.4 (7.6), 128 x 2048 x 2048 9.0
@@ -1750,6 +1750,10 @@ static int pick_tile(int M, int N, int K, bool gated) {
 //  - shared tiles: more than 64 rows and K < 1536 (from there on the stream-K / split-K kernels or the big tiles are
 //    ahead): 128 x 2304 x 768 7.7 (11.7), 128 x 3072 x 768 8.3 (11.7), 512 x 768 x 768 7.6 (11.0), 512 x 1024 x 1024 8.6
 //    (13.0), 128 x 4096 x 1024 10.0 (14.4); 64-row tiles: 256 x 3072 x 768 11.2 (11.8), 1024 x 1024 x 1024 12.2 (14.0).
+//    With the tiles that share a weight tile on one XCD, one round of 64 x 64 tiles also wins over a long K where the
+//    dealt tiles need two (1024 x 768 x 1536 10.8 against 18.5, 512 x 2048 x 2048 13.0 (19.2), 1024 x 768 x 3072 16.8
+//    (18.9)), and one round of 64 x 128 tiles over a short K where 64 x 64 need two (512 x 3072 x 768 10.3 (12.3),
+//    512 x 2304 x 768 10.1 (11.9), 2048 x 768 x 768 10.7 (12.2), 512 x 4096 x 1024 12.3 (14.7)).
 static int small_problem_kind(int64_t M, int64_t N, int64_t K) {
     const int64_t cols32 = (N + 31) / 32, cols64 = (N + 63) / 64;
     const bool small_weight = N * K <= ((int64_t)1 << 23), short_k = M > 64 && K < 1536;
@@ -1758,6 +1762,10 @@ static int small_problem_kind(int64_t M, int64_t N, int64_t K) {
     if (small_weight && M > 16 && ((M + 63) / 64) * cols32 <= 256) return 14;
     if (short_k && ((M + 31) / 32) * cols64 <= 256) return 10;
     if (short_k && ((M + 63) / 64) * cols64 <= 256) return 11;
+    // one round of 64 x 64 tiles over a long K where the dealt tiles would need a second one
+    if (small_weight && M > 64 && ((M + 63) / 64) * cols64 <= 256) return 11;
+    // short K, one round of 64 x 128 tiles where 64 x 64 would need two
+    if (short_k && ((M + 63) / 64) * ((N + 127) / 128) <= 256) return 15;
     return 0;
 }
 

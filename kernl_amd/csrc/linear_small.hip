@@ -52,7 +52,9 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave & 1, wave_n = wave >> 1;
     const int r = lane & 15, g = lane >> 4;
-    const int m0 = ((int)blockIdx.x % tiles_m) * BM, n0 = ((int)blockIdx.x / tiles_m) * BN;
+    // tiles that share a weight tile (consecutive indices, the row tile running fastest) go to one XCD
+    const int tile = xcd_contiguous_index((int)blockIdx.x, (int)gridDim.x);
+    const int m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
 
     // ---- tile loads: load i of a wave fills the 1 KB of 16-byte chunks [(wave * loads + i) * 64, +64) of an operand
     // tile.  Rows beyond M / N are pointed out of the buffer's range and arrive as zeros.
@@ -248,7 +250,9 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
-    const int m0 = ((int)blockIdx.x % tiles_m) * BM, n0 = ((int)blockIdx.x / tiles_m) * BN;
+    // tiles that share a weight tile (consecutive indices, the row tile running fastest) go to one XCD
+    const int tile = xcd_contiguous_index((int)blockIdx.x, (int)gridDim.x);
+    const int m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
 
     constexpr uint32_t kOutOfRange = 0x80000000u;
     const int rows_x = min(BM, M - m0), rows_w = min(BN, N - n0);
@@ -458,13 +462,15 @@ static void launch_small(const LinearArgs &a) {
                        tiles_m);
 }
 
-// rows of a tile: 32 or 64 (64 columns; 64 x 128 tiles in a ring of 6 stages were measured too and never won)
-void run_small(const LinearArgs &a, int dtype, int rows) {
+// tile shapes: 32 x 64, 64 x 64, 64 x 128 (rows x columns; the last in a ring of 6 stages)
+void run_small(const LinearArgs &a, int dtype, int rows, int cols) {
     if (dtype == KERNL_F16) {
-        if (rows == 32) launch_small<f16, 32, 64>(a);
+        if (cols == 128) launch_small<f16, 64, 128>(a);
+        else if (rows == 32) launch_small<f16, 32, 64>(a);
         else launch_small<f16, 64, 64>(a);
     } else {
-        if (rows == 32) launch_small<bf16, 32, 64>(a);
+        if (cols == 128) launch_small<bf16, 64, 128>(a);
+        else if (rows == 32) launch_small<bf16, 32, 64>(a);
         else launch_small<bf16, 64, 64>(a);
     }
 }

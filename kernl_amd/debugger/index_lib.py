@@ -24,7 +24,7 @@ class IndexLib:
         self._c = cdll
         for name, n in (("kernl_idx_rowperm16", 1), ("kernl_idx_swz_offset", 3), ("kernl_idx_attention", 5),
                         ("kernl_idx_mask", 5), ("kernl_idx_wide_weight_row", 2), ("kernl_idx_fewrow", 7),
-                        ("kernl_idx_small_tile", 4)):
+                        ("kernl_idx_small_tile", 4), ("kernl_idx_xcd_contiguous", 2)):
             fn = getattr(cdll, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.c_int] * n
@@ -46,6 +46,9 @@ class IndexLib:
 
     def fewrow(self, row_blocks: int, units_per_stage: int, what: str, a: int = 0, b: int = 0, c: int = 0, d: int = 0) -> int:
         return self._checked(self._c.kernl_idx_fewrow(row_blocks, units_per_stage, self.FEWROW[what], a, b, c, d))
+
+    def xcd_contiguous(self, b: int, n: int) -> int:
+        return self._checked(self._c.kernl_idx_xcd_contiguous(b, n))
 
     def small_tile(self, what: str, a: int, b: int = 0, c: int = 0) -> int:
         return self._checked(self._c.kernl_idx_small_tile(self.SMALL[what], a, b, c))

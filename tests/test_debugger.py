@@ -148,3 +148,19 @@ def test_small_problem_tile_is_loaded_once_and_read_without_conflicts(rows):
     assert reads.conflict_free, (reads.passes, reads.cycles)
     assert reads.instructions == rows // 16 * 2
 
+
+@pytest.mark.parametrize("n", [1, 7, 8, 9, 50, 192, 255, 256])
+def test_small_problem_tiles_of_an_xcd_are_one_contiguous_run(n):
+    """Workgroup b runs on XCD b % 8.  The small-problem kernels' workgroup -> tile map is a bijection, and the tiles of
+    the workgroups of one XCD, taken in launch order, are consecutive indices — so the tiles that share a weight tile
+    (consecutive indices) meet in one L2."""
+    from kernl_amd.debugger.index_lib import index_lib
+
+    ix = index_lib()
+    tiles = [ix.xcd_contiguous(b, n) for b in range(n)]
+    assert sorted(tiles) == list(range(n))
+    runs = [[tiles[b] for b in range(x, n, 8)] for x in range(8)]
+    assert all(run == list(range(run[0], run[0] + len(run))) for run in runs if run)
+    starts = [run[0] for run in runs if run]
+    assert starts == sorted(starts)
+

@@ -687,7 +687,9 @@ def test_small_problem_rule_of_the_library():
     assert kind(512, 768, 3072) == 14 and kind(128, 2304, 768) == 14    # 64 x 32 tiles, k-tiles dealt
     assert kind(96, 5440, 768) == 10 and kind(384, 2304, 768) == 11     # shared 32 x 64 / 64 x 64 tiles where those need a second round
     assert kind(256, 3072, 768) == 11 and kind(1024, 1024, 1024) == 11  # 64 x 64 tiles
-    assert kind(512, 3072, 768) == 0 and kind(2048, 768, 768) == 0      # more than 256 tiles either way
+    assert kind(512, 3072, 768) == 15 and kind(2048, 768, 768) == 15    # short K: 64 x 128 tiles where 64 x 64 need a second round
+    assert kind(768, 3072, 768) == 0 and kind(1024, 3072, 768) == 0     # more than 256 tiles of any kind
     assert kind(32, 4096, 4096) == 0 and kind(128, 11008, 4096) == 0    # big weights stay with the streaming kernels
-    assert kind(768, 768, 3072) == 0                                    # long K with many rows: split-K
+    assert kind(768, 768, 3072) == 11 and kind(1024, 768, 1536) == 11   # long K: one round of 64 x 64 tiles where the dealt ones need two
+    assert kind(2048, 1024, 4096) == 0                                  # long K and more than 256 tiles of 64 x 64: split-K
     assert kind(128, 768, 3076) == 0 and kind(0, 768, 768) == 0         # K no multiple of 8: not the MFMA path at all

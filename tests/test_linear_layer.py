@@ -42,8 +42,9 @@ def test_linear_vs_oracle(shape, bias, activation, dtype, close):
 
 
 TILE_IDS = ["256x256", "256x192", "128x128", "256x128k32", "wide256x256", "wide256x192", "wide128x256", "wide128x192"]
-SMALL_TILES = [10, 11, 12, 13, 14]  # tiles over the whole K: 32 x 64, 64 x 64 (shared by the waves), 16 / 32 / 64 x 32 (k-tiles dealt)
-SMALL_IDS = ["small32x64", "small64x64", "dealt16x32", "dealt32x32", "dealt64x32"]
+# tiles over the whole K: 32 x 64, 64 x 64 (shared by the waves), 16 / 32 / 64 x 32 (k-tiles dealt), 64 x 128 (shared)
+SMALL_TILES = [10, 11, 12, 13, 14, 15]
+SMALL_IDS = ["small32x64", "small64x64", "dealt16x32", "dealt32x32", "dealt64x32", "small64x128"]
 
 
 @pytest.mark.parametrize("tile", list(range(1, 9)) + SMALL_TILES, ids=TILE_IDS + SMALL_IDS)
@@ -99,12 +100,13 @@ def test_linear_ragged_last_k_tile(shape, tile, dtype, close):
 @pytest.mark.parametrize("shape", [(65, 768, 768), (128, 2304, 768), (128, 3072, 768), (200, 1000, 448), (500, 520, 64),
                                    (512, 1024, 1024), (1024, 700, 1480), (1000, 960, 520), (130, 70, 8),
                                    (8, 768, 3072), (16, 2304, 768), (16, 8192, 1024), (33, 768, 3080), (128, 768, 3072),
-                                   (256, 1024, 4096), (100, 2048, 2048), (20, 1000, 8192), (40, 96, 72), (512, 768, 3072), (300, 1000, 2056), (96, 5440, 768)],
+                                   (256, 1024, 4096), (100, 2048, 2048), (20, 1000, 8192), (40, 96, 72), (512, 768, 3072), (300, 1000, 2056), (96, 5440, 768),
+                                   (512, 3072, 768), (500, 2300, 776), (1024, 768, 1536), (700, 1000, 2056)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_linear_small_problem_kernels_are_what_small_problems_run(shape, activation, dtype, close):
     """A few hundred rows at most against a weight of a few million elements: the library's own choice is one of the
     small-problem kernels (one launch, whole K per workgroup; `kernl_linear_small_kind` names it).  Forcing that kernel
-    must give the same bits as the heuristic, every one of the five must match the oracle, and so must the operator,
+    must give the same bits as the heuristic, every one of the six must match the oracle, and so must the operator,
     which must not hand such a shape to the stream-K or split-K entry points.  Tiles ragged in rows, columns and K, fewer
     k-tiles than ring stages or waves, strided output."""
     M, N, K = shape
