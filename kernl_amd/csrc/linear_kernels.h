@@ -1769,7 +1769,7 @@ static int small_problem_kind(int64_t M, int64_t N, int64_t K) {
     return 0;
 }
 
-extern int g_linear_force_tile;  // test / tuning hook (defined in linear.hip): 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192, 10 .. 14 = the small-problem kernels
+extern int g_linear_force_tile;  // test / tuning hook (defined in linear.hip): 0 = heuristic, 1 = 256x256, 2 = 256x192, 3 = 128x128, 4 = 256x128 k32, 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192, 10 .. 15 = the small-problem kernels
 
 template <typename T, bool GATED, int MB, int NR, bool W8, bool RMS = false, bool ROPE = false>
 static void launch_skinny_blocks(const LinearArgs &a, const void *rms_w = nullptr, float eps = 0.0f,
