@@ -52,8 +52,9 @@ linear_small_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *_
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave & 1, wave_n = wave >> 1;
     const int r = lane & 15, g = lane >> 4;
-    // tiles that share a weight tile (consecutive indices, the row tile running fastest) go to one XCD
-    const int tile = xcd_contiguous_index((int)blockIdx.x, (int)gridDim.x);
+    // tiles that share a weight tile (consecutive indices, the row tile running fastest) go to one XCD; with a single
+    // row tile nothing is shared, and workgroups that run side by side had better read neighbouring weight rows
+    const int tile = tiles_m > 1 ? xcd_contiguous_index((int)blockIdx.x, (int)gridDim.x) : (int)blockIdx.x;
     const int m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
 
     // ---- tile loads: load i of a wave fills the 1 KB of 16-byte chunks [(wave * loads + i) * 64, +64) of an operand
@@ -250,8 +251,9 @@ linear_small_dealt_kernel(const T *__restrict__ X, const T *__restrict__ W, cons
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
-    // tiles that share a weight tile (consecutive indices, the row tile running fastest) go to one XCD
-    const int tile = xcd_contiguous_index((int)blockIdx.x, (int)gridDim.x);
+    // tiles that share a weight tile (consecutive indices, the row tile running fastest) go to one XCD; with a single
+    // row tile nothing is shared, and workgroups that run side by side had better read neighbouring weight rows
+    const int tile = tiles_m > 1 ? xcd_contiguous_index((int)blockIdx.x, (int)gridDim.x) : (int)blockIdx.x;
     const int m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
 
     constexpr uint32_t kOutOfRange = 0x80000000u;
