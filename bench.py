@@ -536,7 +536,7 @@ def main():
             extra["linear_256x4096x4096_us_graph_replay"] = round(t * 1e3, 2)
             extra["linear_256x4096x4096_tflops"] = round(2.0 * 256 * 4096 * 4096 / (t * 1e-3) / 1e12, 1)
             # small problems (BERT-base at batch 1 with 128 tokens): one launch of small tiles over the whole K
-            for (m_s, n_s, k_s) in ((128, 768, 3072), (128, 2304, 768), (512, 768, 3072)):
+            for (m_s, n_s, k_s) in ((128, 768, 3072), (128, 2304, 768), (512, 768, 3072), (512, 3072, 768), (1024, 768, 1536)):
                 x_s = torch.randn((m_s, k_s), generator=gen).half().to(dev)
                 w_s = [(torch.randn((n_s, k_s), generator=gen) * k_s ** -0.5).half().to(dev) for _ in range(8)]
                 b_s = torch.randn((n_s,), generator=gen).half().to(dev)
