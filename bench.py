@@ -63,6 +63,64 @@ def traffic_from_profile():
     return None
 
 
+def measured_peaks(dev, reps=3, ms_target=20.0):
+    """What this GPU sustains on register-only MFMA loops and plain streaming passes (kernl_probe_rate, compiled into the
+    library: kernl_amd/csrc/peak_probe.hip), each with the shader clock its loop ran at (shader-clock ticks over
+    100 MHz wall-clock ticks, read inside the kernel by every workgroup).  The last of `reps` launches of about
+    `ms_target` ms each is reported.  These are the ceilings a kernel can be compared with on THIS box; roofline
+    fractions are still divided by the published 2.5 PFLOP/s and 8 TB/s."""
+    import torch
+
+    from kernl_amd import _lib
+
+    lib = _lib.load()
+    n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
+    gen = torch.Generator().manual_seed(0)
+    table = (torch.rand((256 * 16 * 256 * 8,), generator=gen) * 2 - 1).half().to(dev)  # 16 MiB of fp16 in (-1, 1)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run(kind, iters, wgs, src, dst, nbytes):
+        stats = torch.zeros((wgs, 2), dtype=torch.int64, device=dev)
+        sink = torch.empty((max(wgs, 512) * 256,), dtype=torch.float32, device=dev)
+        best = None
+        for _ in range(reps):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            st = lib.kernl_probe_rate(kind, iters, wgs, src.data_ptr(), 0 if dst is None else dst.data_ptr(), nbytes,
+                                      stats.data_ptr(), sink.data_ptr(), stream)
+            e.record()
+            _lib._check(st, "kernl_probe_rate")
+            e.synchronize()
+            ticks = stats.cpu().double()
+            best = (s.elapsed_time(e), float((ticks[:, 0] / ticks[:, 1].clamp_min(1)).mean()) * 0.1)  # ms, GHz
+        return best
+
+    out = {"compute_units": n_cu}
+    flop_per_trip = {0: 32 * 32768.0, 1: 64 * 16384.0, 2: 32 * 32768.0, 3: 16 * 32768.0}
+    for label, kind, wgs in (("mfma_32x32x16_f16", 0, n_cu), ("mfma_16x16x32_f16", 1, n_cu), ("mfma_32x32x16_f16_zero_operands", 2, n_cu),
+                             ("attention_mix_1mfma_2exp_4fma_1wave_per_simd", 3, n_cu), ("attention_mix_1mfma_2exp_4fma_2waves_per_simd", 3, 2 * n_cu)):
+        per_trip = flop_per_trip[kind] * wgs * 4
+        iters = 2000
+        ms, _ = run(kind, iters, wgs, table, None, table.numel() * 2)
+        iters = max(1000, int(iters * ms_target / ms))
+        ms, ghz = run(kind, iters, wgs, table, None, table.numel() * 2)
+        out[f"measured_peak_{label}_tflops"] = round(per_trip * iters / (ms * 1e-3) / 1e12, 1)
+        out[f"measured_peak_{label}_clock_ghz"] = round(ghz, 3)
+    nbytes = 1 << 30
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_()
+    dst = torch.empty_like(src)
+    for label, kind, moved in (("hbm_read_1gib", 4, nbytes), ("hbm_copy_1gib", 5, 2 * nbytes)):
+        best_rate, best_wgs = 0.0, 0
+        for wgs in (8 * n_cu, 16 * n_cu, 32 * n_cu):
+            ms, _ = run(kind, 0, wgs, src, dst, nbytes)
+            rate = moved / (ms * 1e-3) / 1e9
+            if rate > best_rate:
+                best_rate, best_wgs = rate, wgs
+        out[f"measured_peak_{label}_gbps"] = round(best_rate, 1)
+        out[f"measured_peak_{label}_workgroups"] = best_wgs
+    return out
+
+
 def config1_inputs():
     import torch
 
@@ -130,6 +188,14 @@ def main():
         help="run BERT-base fp16 through optimize_model at batch 1 with 16, 128 and 512 tokens (30 hipGraph replays each) "
         "and exit: the workload of the rocprofv3 --kernel-trace run behind profiles/bert_base_batch1_kernel_trace.txt",
     )
+    ap.add_argument(
+        "--peak-probe",
+        action="store_true",
+        help="run only the rate probes (register-only MFMA loops of both shapes, the attention loop's instruction mix, a "
+        "1 GiB read-only pass and a 1 GiB copy, each with its in-kernel clock reading), print them as one JSON line and "
+        "exit: the workload behind profiles/peak_probe_kernel_trace.txt; every ordinary run carries the same figures as "
+        "extra.measured_peak_*",
+    )
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU per process and ships no multi-GPU path; run with --gpus 1")
@@ -145,6 +211,10 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.peak_probe:
+        print(json.dumps(measured_peaks(dev)), flush=True)
+        return
 
     # ------------------------------------------------------------------ headline: fused attention, config 1
     q, k, v, mask, lengths = config1_inputs()
@@ -671,6 +741,15 @@ def main():
             del llama
         except Exception as exc:
             extra["llama7b_width_error"] = f"{type(exc).__name__}: {exc}"[:300]
+
+    # ------------------------------------------------------------------ what this box sustains (rate probes)
+    if not args.skip_extra:
+        try:
+            extra.update(measured_peaks(dev))
+            extra["attention_frac_of_measured_mix_rate"] = round(
+                achieved / max(extra["measured_peak_attention_mix_1mfma_2exp_4fma_2waves_per_simd_tflops"], 1e-9), 4)
+        except Exception as exc:
+            extra["measured_peak_error"] = f"{type(exc).__name__}: {exc}"[:300]
 
     result["extra"] = extra
     print(json.dumps(result), flush=True)

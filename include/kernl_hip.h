@@ -151,7 +151,10 @@ int kernl_attention_skinny_kv8_fwd(const void *q, const void *k, const void *v, 
  * partial maxima / sums / products with torch on every call (src/kernl/implementations/attention_skinny.py:416-441).
  * The partial results of the key ranges live in a device array of kernl_attention_skinny_static_max_bytes() bytes
  * (512 KiB) that is part of the library image: every GPU the library runs on holds it until the process ends.  The call
- * itself performs no hipMalloc / hipFree; the first call on a device looks the array's address up once.
+ * itself performs no hipMalloc / hipFree; the first call on a device looks the array's address up once
+ * (hipGetSymbolAddress, which may load the code object): that first call must happen OUTSIDE any stream capture.
+ * kernl_attention_skinny_static_init() performs just that lookup for the current device and launches nothing — call
+ * it (or make one eager call) per device before capturing a graph that holds kernl_attention_skinny_static_fwd.
  *
  *   - 16-bit keys and values only; arguments as kernl_attention_skinny_fwd without the workspace pair.
  *   - Problems with kernl_attention_skinny_workspace_bytes(B,H,M,N,D) above the array's size (the largest workspace
@@ -163,6 +166,7 @@ int kernl_attention_skinny_kv8_fwd(const void *q, const void *k, const void *v, 
  *     threads) race.  Calls on one stream are ordered and safe.
  */
 int64_t kernl_attention_skinny_static_max_bytes(void);
+int kernl_attention_skinny_static_init(void);
 int kernl_attention_skinny_static_fwd(const void *q, const void *k, const void *v, void *out, const void *mask,
                                       int64_t B, int64_t H, int64_t M, int64_t N, int64_t D,
                                       const int64_t q_strides[4], const int64_t k_strides[4],
@@ -374,29 +378,7 @@ int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, 
                             int64_t res_col_stride, int64_t out_row_stride, int64_t out_col_stride,
                             float eps, int is_rms, int dtype, void *stream);
 
-/*
- * Test and tuning hooks (process-wide, not thread-safe; no counterpart in the reference).
- *   kernl_linear_force_tile      0 = heuristic (default); output tile of the MFMA linear kernel: 1 = 256x256,
- *                                2 = 256x192, 3 = 128x128, 4 = 256x128 with 32-wide k-tiles; persistent kernel with one
- *                                wave per SIMD: 5 = 256x256, 6 = 256x192; its one-tile-per-workgroup variant with
- *                                three LDS stages: 7 = 128x256, 8 = 128x192 (5..8 take any K the MFMA path takes, with
- *                                a zero-filled last k-tile when K % 64 != 0; gated epilogues take 1, 3 or 5);
- *                                10 .. 15 = the small-problem kernels (one launch of small tiles over the whole K:
- *                                32 x 64 / 64 x 64 tiles shared by the waves, 16 x 32 / 32 x 32 / 64 x 32 tiles with the
- *                                k-tiles dealt to the waves, 15 = 64 x 128 shared tiles); the heuristic takes them where kernl_linear_small_kind
- *                                says so.  With the heuristic, inputs of at most
- *                                64 rows and K % 64 == 0 go to a kernel that streams the weight once (16 output
- *                                columns per workgroup); 9 = that kernel where it applies, the heuristic elsewhere;
- *                                1..8 keep such inputs on the tile kernels.
- *   kernl_attention_force_scalar non-zero routes every attention call through the strided scalar kernel.
- *   kernl_attention_set_variant  0 = heuristic; register budget of the head-size-64 streaming attention kernel: 1 = built
- *                                for 3 waves/SIMD, 2 = built for 2 waves/SIMD; 3 = streaming kernel for every shape,
- *                                4 = software-pipelined kernel wherever it applies (head size 64; no mask, a per-key
- *                                mask of at most 2048 keys, or causal), also below 1024 keys.
- */
-void kernl_linear_force_tile(int which);
-void kernl_attention_force_scalar(int on);
-void kernl_attention_set_variant(int which);
+/* The process-wide test and tuning hooks are not part of this interface: they are declared in kernl_hip_test.h. */
 
 #ifdef __cplusplus
 }

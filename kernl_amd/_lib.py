@@ -28,6 +28,7 @@ EXPORTED_SYMBOLS = (
     "kernl_attention_skinny_kv8_fwd",
     "kernl_attention_kv8_fwd",
     "kernl_attention_skinny_static_max_bytes",
+    "kernl_attention_skinny_static_init",
     "kernl_attention_skinny_static_fwd",
     "kernl_rope_fwd",
     "kernl_linear_fwd",
@@ -43,9 +44,14 @@ EXPORTED_SYMBOLS = (
     "kernl_linear_glu_fwd",
     "kernl_layernorm_fwd",
     "kernl_add_layernorm_fwd",
+)
+
+# the process-wide test and tuning hooks of include/kernl_hip_test.h (bound for the tests and benchmarks only)
+TEST_HOOK_SYMBOLS = (
     "kernl_linear_force_tile",
     "kernl_attention_force_scalar",
     "kernl_attention_set_variant",
+    "kernl_probe_rate",
 )
 
 _i64 = ctypes.c_int64
@@ -100,6 +106,8 @@ def load() -> ctypes.CDLL:
     )
     lib.kernl_attention_skinny_static_max_bytes.restype = _i64
     lib.kernl_attention_skinny_static_max_bytes.argtypes = []
+    lib.kernl_attention_skinny_static_init.restype = ctypes.c_int
+    lib.kernl_attention_skinny_static_init.argtypes = []
     lib.kernl_attention_skinny_static_fwd.restype = ctypes.c_int
     lib.kernl_attention_skinny_static_fwd.argtypes = (
         [_vp] * 5 + [_i64] * 5 + [_i64p] * 6 + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_float, ctypes.c_int, _vp]
@@ -146,6 +154,8 @@ def load() -> ctypes.CDLL:
     lib.kernl_attention_force_scalar.argtypes = [ctypes.c_int]
     lib.kernl_attention_set_variant.restype = None
     lib.kernl_attention_set_variant.argtypes = [ctypes.c_int]
+    lib.kernl_probe_rate.restype = ctypes.c_int
+    lib.kernl_probe_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _i64, _vp, _vp, _vp]
     _lib = lib
     return lib
 
@@ -258,6 +268,15 @@ def attention_skinny_fwd(q, k, v, out, mask, workspace, sm_scale: float, is_caus
             float(sm_scale), int(bool(is_causal)), float(mask_min_clamp), DTYPE_CODE[q.dtype], _stream(q),
         )
     _check(st, "kernl_attention_skinny_fwd")
+
+
+def attention_skinny_static_init(device=None) -> None:
+    """Look up the static partial-result buffer of `device` (default: the current one): to be called outside graph
+    capture before `attention_skinny_static_fwd` is captured for the first time on that device."""
+    lib = load()
+    with torch.cuda.device(device):
+        st = lib.kernl_attention_skinny_static_init()
+    _check(st, "kernl_attention_skinny_static_init")
 
 
 def attention_skinny_static_fwd(q, k, v, out, mask, sm_scale: float, is_causal: bool, mask_min_clamp: float) -> None:

@@ -456,6 +456,13 @@ static int skinny_scratch(void **ptr_out) {
 
 extern "C" int64_t kernl_attention_skinny_static_max_bytes(void) { return kernl::kSkScratchBytes; }
 
+// The once-per-device address lookup on its own, for callers whose first use of the static entry point would fall
+// inside a stream capture: a symbol lookup may load the code object, which a capturing stream does not allow.
+extern "C" int kernl_attention_skinny_static_init(void) {
+    void *ptr = nullptr;
+    return kernl::skinny_scratch(&ptr);
+}
+
 extern "C" int kernl_attention_skinny_static_fwd(const void *q, const void *k, const void *v, void *out,
                                                  const void *mask, int64_t B, int64_t H, int64_t M, int64_t N,
                                                  int64_t D, const int64_t q_strides[4], const int64_t k_strides[4],

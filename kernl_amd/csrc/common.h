@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "../../include/kernl_hip.h"
+#include "../../include/kernl_hip_test.h"
 #include "index_math.h"
 
 namespace kernl {

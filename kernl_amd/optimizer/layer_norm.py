@@ -51,10 +51,11 @@ def layer_norm_wrapper_functional(v: torch.Tensor, normalized_shape, weight, bia
 
 
 def add_layer_norm_wrapper_functional(a: torch.Tensor, b: torch.Tensor, normalized_shape, weight, bias, eps: float):
-    _half_params_once(a, weight, bias)
     if not isinstance(a, torch.Tensor) or not isinstance(b, torch.Tensor) or a.shape != b.shape or a.dtype != b.dtype:
-        # a python scalar or a broadcast operand: add first (one element-wise kernel), then the LayerNorm kernel
+        # a python scalar (on either side) or a broadcast operand: add first (one element-wise kernel), then the
+        # LayerNorm kernel, which also casts the parameters once to the dtype of the sum
         return layer_norm_wrapper_functional(a + b, normalized_shape, weight, bias, eps)
+    _half_params_once(a, weight, bias)
     if len(normalized_shape) == 1 and weight is not None:
         return add_layer_norm(a, b, weight, bias, eps)
     lead, n, w, bb = _flat_affine(a, normalized_shape, weight, bias)

@@ -278,15 +278,41 @@ def _concatenated_params(v: torch.Tensor, weights, biases):
             bias = torch.cat(
                 [torch.zeros(w.shape[0], dtype=w.dtype, device=w.device) if b is None else b.detach() for w, b in zip(weights, biases)]
             ).contiguous()
-        row = 0
-        for w, b, n in zip(weights, biases, sizes):
-            w.data = weight[row : row + n]
-            if b is not None:
-                b.data = bias[row : row + n]
-            row += n
         cached = (weight, bias, sizes)
-        _fused_params.put(originals, cached)  # keyed by the addresses the parameters now have inside the fused buffers
+        if any(_is_view_of_larger_storage(p) for p in originals):
+            # Some parameter is already a slice of a larger buffer — the fused weight of ANOTHER group it belongs to
+            # (tied or shared projections), or a flat parameter buffer.  Re-pointing it a second time would move it out
+            # of the first group's buffer, whose entry would then be dropped and its memory freed under graphs that
+            # still read it.  This group keeps a copy instead, rewritten in place when a parameter's version moves.
+            _fused_params.put(originals, cached, rebuild=_rebuild_concatenated)
+        else:
+            row = 0
+            for w, b, n in zip(weights, biases, sizes):
+                w.data = weight[row : row + n]
+                if b is not None:
+                    b.data = bias[row : row + n]
+                row += n
+            _fused_params.put(originals, cached)  # keyed by the addresses the parameters now have inside the fused buffers
     return cached
+
+
+def _is_view_of_larger_storage(p) -> bool:
+    return p is not None and p.untyped_storage().nbytes() != p.numel() * p.element_size()
+
+
+def _rebuild_concatenated(value, originals):
+    """In-place refresh of a COPIED concatenation (see `_concatenated_params`) from its live parameters."""
+    weight, bias, sizes = value
+    count = len(sizes)
+    row = 0
+    for w, b, n in zip(originals[:count], originals[count:], sizes):
+        weight[row : row + n].copy_(w.detach())
+        if bias is not None:
+            if b is None:
+                bias[row : row + n].zero_()
+            else:
+                bias[row : row + n].copy_(b.detach())
+        row += n
 
 
 torch.fx.wrap("fused_linear_wrapper")
@@ -507,14 +533,18 @@ def linear_residual_wrapper(v: torch.Tensor, weight: torch.Tensor, bias, residua
     the addition that follows them.  Decoding steps (at most 64 rows) run it as one launch; larger inputs as the linear
     kernel and the addition they were.  No counterpart in the reference, whose model adds in eager PyTorch
     (experimental/llama-v2/llama/model.py:262-264)."""
-    from kernl_amd.implementations.linear_layer import decode_linear_layer, decode_linear_supported
+    from kernl_amd.implementations.linear_layer import decode_linear_layer, decode_linear_supported, takes_small_problem_kernel
 
     if weight.dtype == torch.float32 and (v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")):
         weight.data = weight.data.half()
     if bias is not None and bias.dtype == torch.float32 and (v.dtype == torch.float16 or torch.is_autocast_enabled("cuda")):
         bias.data = bias.data.half()
+    x2d = v if v.dim() == 2 else v.reshape(-1, v.shape[-1])
     if (
         decode_linear_supported(v, weight)
+        # small weights: the one-launch small-tile kernels beat the weight-streaming kernel by more than the separate
+        # addition costs (64 x 768 x 3072: 8.0 us against 11.6), so such shapes keep the addition
+        and not takes_small_problem_kernel(x2d, weight)
         and residual.dtype == v.dtype
         and residual.shape[:-1] == v.shape[:-1]
         and residual.shape[-1] == weight.shape[0]

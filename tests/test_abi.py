@@ -12,20 +12,23 @@ from kernl_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "kernl_hip.h")).read()
+def _declared_symbols(header="kernl_hip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(kernl_[a-z_0-9]+)\s*\(", text)))
 
 
 def test_header_and_binding_agree():
     assert _declared_symbols() == sorted(_lib.EXPORTED_SYMBOLS)
+    # the process-wide tuning hooks live in a header of their own, outside the re-entrant interface
+    assert _declared_symbols("kernl_hip_test.h") == sorted(_lib.TEST_HOOK_SYMBOLS)
+    assert not set(_lib.TEST_HOOK_SYMBOLS) & set(_declared_symbols())
 
 
 def test_library_exports_every_declared_symbol():
     lib = _lib.load()
-    for name in _declared_symbols():
-        assert hasattr(lib, name), f"{name} declared in include/kernl_hip.h but not exported"
+    for name in _declared_symbols() + _declared_symbols("kernl_hip_test.h"):
+        assert hasattr(lib, name), f"{name} declared under include/ but not exported"
     assert lib.kernl_version() == 100
 
 

@@ -6,6 +6,7 @@ docs/how-to-guides/support-new-model.md:139-246.
 """
 import operator
 
+import pytest
 import torch
 
 from kernl_amd.implementations.attention import closest_power_of_2
@@ -575,6 +576,49 @@ def test_concatenated_projection_weights_alias_their_parameters():
     assert torch.equal(b2[:8], torch.zeros(8)) and lin_b.bias.data_ptr() == b2[8:].data_ptr()
 
 
+def test_overlapping_projection_groups_do_not_move_each_others_parameters():
+    """A weight that belongs to two sibling groups (shared or tied projections): the first group's fused buffer keeps
+    its address and values — a captured graph reads it —, the second group keeps a copy that follows the parameters'
+    version counters in place."""
+    from kernl_amd.optimizer.linear import _concatenated_params, _fused_params
+
+    torch.manual_seed(0)
+    q, k, v = (torch.nn.Linear(16, 8) for _ in range(3))
+    x = torch.zeros(2, 16)
+    first = _concatenated_params(x, [q.weight, k.weight, v.weight], [q.bias, k.bias, v.bias])
+    ptr, snapshot = first[0].data_ptr(), first[0].clone()
+    second = _concatenated_params(x, [k.weight, v.weight], [k.bias, v.bias])
+    # the second group did not re-point k and v: they still live in the first group's buffer
+    assert k.weight.data_ptr() == first[0][8].data_ptr() and v.weight.data_ptr() == first[0][16].data_ptr()
+    assert second[0].data_ptr() != k.weight.data_ptr() and torch.equal(second[0], first[0][8:])
+    again = _concatenated_params(x, [q.weight, k.weight, v.weight], [q.bias, k.bias, v.bias])
+    assert again[0] is first[0] and again[0].data_ptr() == ptr and torch.equal(again[0], snapshot)
+    assert _concatenated_params(x, [k.weight, v.weight], [k.bias, v.bias])[0] is second[0]
+    # a version-counted write reaches both: the aliased buffer directly, the copy on its next lookup, in place
+    with torch.no_grad():
+        k.weight.fill_(2.0)
+        v.bias.fill_(-1.0)
+    assert torch.equal(first[0][8:16], torch.full((8, 16), 2.0))
+    refreshed = _concatenated_params(x, [k.weight, v.weight], [k.bias, v.bias])
+    assert refreshed[0] is second[0] and torch.equal(second[0][:8], torch.full((8, 16), 2.0))
+    assert torch.equal(second[1][8:], torch.full((8,), -1.0))
+    assert len(_fused_params) >= 2
+
+
+def test_add_layer_norm_with_a_scalar_on_either_side_reaches_the_kernel():
+    """`layer_norm(1.0 + x)` traces to add(scalar, tensor): the wrapper must add first and call the LayerNorm kernel
+    (which refuses CPU tensors here), not look for a dtype on the scalar."""
+    from kernl_amd._lib import KernlLibraryError
+    from kernl_amd.optimizer.layer_norm import add_layer_norm_wrapper_functional
+
+    x = torch.zeros(2, 8, dtype=torch.float16)
+    w, b = torch.ones(8), torch.zeros(8)
+    for a, c in ((1.0, x), (x, 1.0), (x[:1], x)):
+        with pytest.raises(KernlLibraryError):
+            add_layer_norm_wrapper_functional(a, c, (8,), w, b, 1e-5)
+    assert w.dtype == torch.float16  # parameters were cast once on the way
+
+
 def test_interleaved_gate_weights_are_refreshed_in_place():
     """The block-interleaved weight of a gated linear unit is a copy: version-counted writes refresh it on the next
     lookup, other writes through `refresh_fused_parameters()`, always at the same address."""
@@ -653,6 +697,24 @@ def test_residual_additions_fold_into_the_projection_before_them():
     assert t.count("linear_residual_wrapper") == 2 and t.count("add") == 2
     nodes = [n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "linear_residual_wrapper"]
     assert [n.args[3].name for n in nodes] == ["r", nodes[0].name]       # the residual operand of each
+
+
+def test_residual_projection_keeps_the_addition_where_the_small_tile_kernels_are_faster(monkeypatch):
+    """A residual projection of a decoding step runs as one launch of the weight-streaming kernel — except against a
+    small weight, where `kernl_linear_fwd`'s one-launch small-tile kernels win by more than the addition costs."""
+    import kernl_amd.implementations.linear_layer as impl
+    import kernl_amd.optimizer.linear as opt
+
+    taken = []
+    monkeypatch.setattr(impl, "decode_linear_layer", lambda v, w, b, residual=None: taken.append("fused") or residual)
+    monkeypatch.setattr(opt, "linear_wrapper_functional", lambda v, w, b: taken.append("separate") or torch.zeros(v.shape[0], w.shape[0], dtype=v.dtype))
+    for rows, n, k in ((64, 768, 3072), (1, 4096, 4096), (32, 4096, 4096), (1, 768, 768)):
+        x = torch.zeros((rows, k), dtype=torch.float16)
+        w = torch.zeros((n, k), dtype=torch.float16)
+        opt.linear_residual_wrapper(x, w, None, torch.zeros((rows, n), dtype=torch.float16))
+        small = impl.takes_small_problem_kernel(x, w)
+        assert taken[-1] == ("separate" if small else "fused"), (rows, n, k)
+    assert taken[0] == "separate" and taken[1] == "fused"
 
 
 def test_few_row_kernel_routing_rule():

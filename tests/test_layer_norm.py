@@ -25,7 +25,7 @@ def test_layer_norm_vs_oracle(shape, dtype, close):
     out = layer_norm(x.cuda(), w.cuda(), b.cuda(), eps)
     torch.cuda.synchronize()
     ref = layer_norm_oracle(x, w, b, effective_eps(eps, dtype))
-    close(out, ref, torch.float16 if dtype == torch.float32 else dtype, scale="magnitude", what=f"layernorm {shape}")
+    close(out, ref, dtype, scale="magnitude", what=f"layernorm {shape}")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
@@ -99,7 +99,7 @@ def test_rows_that_share_a_wave(dtype, n, close):
         w = (1 + 0.1 * torch.randn((n,), generator=gen)).to(dtype)
         b = (0.1 * torch.randn((n,), generator=gen)).to(dtype)
         eps = effective_eps(1e-5, dtype)
-        tol = torch.float16 if dtype == torch.float32 else dtype
+        tol = dtype
         print(f"case rows={rows} n={n} {dtype}", flush=True)
         out = layer_norm(x.cuda(), w.cuda(), b.cuda(), 1e-5)
         close(out, layer_norm_oracle(x, w, b, eps), tol, scale="magnitude", what=f"layernorm {rows}x{n}")

@@ -36,7 +36,7 @@ def test_rotary_vs_oracle(shape, dtype, close):
     out = rotary_forward(x.cuda(), cos.cuda(), sin.cuda())
     torch.cuda.synchronize()
     assert out.dtype == dtype and out.stride() == x.stride()
-    close(out, rotary_oracle(x, cos, sin), torch.float16 if dtype == torch.float32 else dtype, scale="magnitude", what=f"rotary {shape}")
+    close(out, rotary_oracle(x, cos, sin), dtype, scale="magnitude", what=f"rotary {shape}")
 
 
 @pytest.mark.parametrize("table_dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["t-fp32", "t-fp16", "t-bf16"])

@@ -46,6 +46,46 @@ def test_static_buffer_entry_matches_workspace_entry_twice_in_a_row():
     _both((2, 8, 1, 128), 4096, seed=2, causal=True)
 
 
+def test_static_buffer_entry_allocates_nothing_and_replays_from_a_graph():
+    """The use the entry point is for: captured in a hipGraph (after the once-per-device lookup outside capture) and
+    replayed on changed inputs, with torch's allocator untouched by the call; every replay is compared with the
+    workspace entry on the same inputs, with eager work and synchronisations between the replays."""
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(7)
+    B, H, N, D = 2, 8, 2048, 128
+    q = torch.randn((B, H, 1, D), generator=gen).half().to(dev)
+    k = torch.randn((B, H, N, D), generator=gen).half().to(dev)
+    v = torch.randn((B, H, N, D), generator=gen).half().to(dev)
+    out = torch.empty_like(q)
+    ref = torch.empty_like(q)
+    nbytes = _lib.attention_skinny_workspace_bytes(B, H, 1, N, D)
+    assert 0 < nbytes <= _lib.load().kernl_attention_skinny_static_max_bytes()
+    ws = torch.empty((nbytes // 4,), dtype=torch.float32, device=dev)
+    _lib.attention_skinny_static_init(dev)  # the address lookup, outside capture
+    torch.cuda.synchronize()
+    before = (torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev))
+    _lib.attention_skinny_static_fwd(q, k, v, out, None, D ** -0.5, False, 0.0)
+    torch.cuda.synchronize()
+    assert (torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev)) == before
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=side):
+        _lib.attention_skinny_static_fwd(q, k, v, out, None, D ** -0.5, False, 0.0)
+    torch.cuda.synchronize()
+    for r in range(3):
+        q.copy_(torch.randn(q.shape, generator=gen).half())
+        k[:, :, r::3].mul_(-0.5)
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        _lib.attention_skinny_fwd(q, k, v, ref, None, ws, D ** -0.5, False, 0.0)
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), f"replay {r} differs from the workspace entry"
+        check_close(out, attention_oracle(q.cpu(), k.cpu(), v.cpu(), D ** -0.5, False, None), torch.float16, what=f"skinny static replay {r}")
+
+
 def test_static_buffer_entry_refuses_what_does_not_fit():
     lib = _lib.load()
     B, H, M, N, D = 5, 80, 1, 4096, 256
