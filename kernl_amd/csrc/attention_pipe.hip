@@ -29,14 +29,18 @@
 // those of attention.hip.
 //
 // The grid is persistent (two workgroups per CU, each walking a fixed list of (batch, head, query tile) items): the
-// next item's query rows, first K / V tiles and mask row are requested as soon as the ring is free and arrive while
-// the finished item is normalised and stored.
+// next item's query rows, first K / V tiles and mask row are requested as soon as the ring is free — all of them
+// into LDS (the query and mask rows into ring slots that are idle between two items) — and arrive while the finished
+// item is normalised and stored.
 //
-// Where it is used: the chip is power-limited on this loop (about 1.0 PFLOP/s at head size 64 whatever the
-// instruction order: fewer stall cycles are answered by a lower clock), so what the pipelined stream gains is the
-// energy of the instructions it no longer executes — 4..16 % from 1024 keys on.  Below that the fixed cost of an
-// item (tile classification, the first tile's serial chain, the epilogue: about half of an item's life at 512 keys)
-// weighs more with two workgroups per CU than it does in the streaming kernel with three, and that kernel is faster.
+// Where it is used: from 1024 keys on, where the pipelined stream is 4..16 % ahead of the streaming kernel.  Below that
+// the fixed cost of an item weighs as much as its tile loop.  Cycle stamps at 512 keys (8 tiles, two workgroups per CU):
+// about 18 000 cycles per item, of which the tile loop takes 9 700; the rest is the first tile's serial chain (2 800),
+// the request of the next item (2 000 .. 3 000: some 180 scalar instructions of address arithmetic and 14 .. 22
+// tile-sized loads, executed by all eight waves of the CU at once), the tile classification of a per-key mask (2 500),
+// the store (1 200), the overflow vote (700) and waits.  Every wave runs such serial code at about ten cycles per
+// instruction, so the count of instructions outside the loop is what is left to cut; running one item per workgroup
+// under the hardware's own dispatch measures the same as the persistent grid (36.8 us either way at [32,12,512,64]).
 #include "attention_common.h"
 
 #ifndef KERNL_ATTN_PIPE_LOOKAHEAD
@@ -66,7 +70,20 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
     constexpr int PER = VEC ? BIAS_KEYS / 256 : 1;       // keys of a mask row per thread
     static_assert(!(VEC && CAUSAL), "per-key masks with causal masking take the streaming kernel");
     static_assert(KI * 4096 == K_BYTES && K_BYTES == V_BYTES, "a tile is KI loads of 1 KB per wave");
-    static_assert(!VEC || PER == 8, "item_loads_landed names the eight mask registers");
+    // What an item needs before its first tile is PREFETCHED INTO LDS, into ring slots that are idle between two items
+    // (the next item's first tiles only take K slots 0..2 and V slots 0..1):
+    //   query rows   V ring slots 2 and 3: wave w keeps its 32 rows at Q_STAGE + w * KS KB, lane l's fragment s at
+    //                + s KB + 16 l — every lane reads back exactly what its own load wrote;
+    //   mask row     K ring slot 3, one dword per key (16-bit masks: the value in the low half).  Rows of up to
+    //                64 * PER keys are fetched by EVERY wave into a quarter of the slot of its own; longer rows once,
+    //                shared out over the four waves.
+    // Nothing the compiler knows as a register is pending between request and use (an earlier form kept these loads'
+    // destination registers live across the previous item's epilogue; the register allocator was free to copy them
+    // before the wait that made them valid, and one build did).
+    constexpr int Q_STAGE = V_RING + 2 * V_BYTES, MASK_STAGE = 3 * K_BYTES;
+    constexpr int WAVE_ROW_KEYS = 64 * PER;  // 512: longest mask row a single wave classifies by itself
+    static_assert(KS * 1024 * 4 <= 2 * V_BYTES, "the four waves' query rows fit two V ring slots");
+    static_assert(!VEC || (kPipeMaxMaskKeys * 4 <= K_BYTES && WAVE_ROW_KEYS * 4 * 4 <= K_BYTES), "a mask row fits K ring slot 3");
     typedef BoolC<true> Yes;
     typedef BoolC<false> No;
 
@@ -75,14 +92,14 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
     __shared__ __attribute__((aligned(16))) unsigned char smem_fixed[D == 64 ? LDS_BYTES : 16];
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_dynamic[];
     unsigned char *const smem = D == 64 ? smem_fixed : smem_dynamic;
-    float *bias_lds = reinterpret_cast<float *>(smem + BIAS_OFF);
-    float *red_lds = bias_lds + BIAS_KEYS;                                   // 4 floats: per-wave maxima of a mask row
+    float *bias_lds = reinterpret_cast<float *>(smem + BIAS_OFF);  // additive terms of the item's keys (see the classification)
     int *vote_lds = reinterpret_cast<int *>(smem + BIAS_OFF + BIAS_KEYS * 4 + 16);  // 4 ints: per-wave overflow votes
-    uint32_t *cls_lds = reinterpret_cast<uint32_t *>(smem + BIAS_OFF + BIAS_KEYS * 4 + 32);  // 4 x 3 words: per-wave tile classes
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 31, lh = lane >> 5;
     const int M = p.M, N = p.N;
+    const bool wave_rows = VEC && N <= WAVE_ROW_KEYS;
+    const int bias_wave = wave_rows ? wave * WAVE_ROW_KEYS : 0;  // short rows: every wave keeps the terms in a copy of its own
     auto uniform = [](uint32_t x) __attribute__((always_inline)) -> uint32_t { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); };
 
     // ---- the work of this workgroup.  The grid is persistent: 8 W workgroups, W per XCD (workgroup ids are dealt
@@ -148,8 +165,6 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
     // every later one while the previous item finishes): the query rows, the first K and V tiles in natural order
     // (what a mask that pads on the right ends up with; another order re-requests them), the mask row.
     //   ring requests:  K(0), V(0), K(1), K(2), V(1)   — step t then requests K(t+3) and V(t+2)
-    vec8 q_raw[KS];
-    float mask_raw[PER];
     uint64_t kaddr = 0, vaddr = 0;  // of the item whose tiles are being requested
     // (batch, head, first query row, key tiles up to the causal bound) of the item being computed and of the requested one
     int cur_b = 0, cur_h = 0, cur_q0 = 0, cur_nt_all = 0, req_b = 0, req_h = 0, req_q0 = 0, req_nt_all = 0;
@@ -170,32 +185,20 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
         dma_k(t2, 2);
         dma_v(t1, 1);
     };
-    // The loads of the query rows and of the mask row are issued from inline assembly as well: the compiler makes every
-    // barrier wait for the vector-memory loads it knows of, and these are meant to stay in flight across the barriers
-    // of the previous item's epilogue.  `item_loads_landed` is the wait that ties their registers.  Between the two the
-    // compiler believes the registers hold their values: were it to SPILL one of them there, it would store what the
-    // load has not delivered yet.  The registers are therefore only ever named by those two statements, and the
-    // build is checked for it: the per-key-mask form of head size 64 has 5-6 spilled registers, none of them these (a
-    // build that moved the LDS rings of that form to dynamic LDS spilled 26 and read garbage mask values).
-    auto request_item = [&](int idx) __attribute__((always_inline)) {
-        const int bh = 8 * (idx / p.nq_tiles) + xcd, qt = idx % p.nq_tiles;
-        req_b = bh / p.H;
-        req_h = bh % p.H;
-        req_q0 = (CAUSAL ? p.nq_tiles - 1 - qt : qt) * BM;
-        const int n_end = CAUSAL ? min(N, req_q0 + BM + p.causal_off) : N;
-        req_nt_all = (n_end + BN - 1) / BN;
-        set_kv(req_b, req_h);
+    // Query rows and mask row of the requested item -> their LDS staging areas (direct-to-LDS loads from inline assembly,
+    // like the tile loads: the compiler would make every barrier wait for loads it knows of, and these are meant to stay
+    // in flight across the barriers of the previous item's epilogue).
+    auto request_staged = [&]() __attribute__((always_inline)) {
         const int my_m = req_q0 + wave * 32 + lr;
-        const T *qrow = static_cast<const T *>(p.q) + req_b * p.qs[0] + req_h * p.qs[1] + (int64_t)min(my_m, M - 1) * p.qs[2] + lh * 8;
-        asm volatile("global_load_dwordx4 %0, %4, off\n\tglobal_load_dwordx4 %1, %4, off offset:32\n\t"
-                     "global_load_dwordx4 %2, %4, off offset:64\n\tglobal_load_dwordx4 %3, %4, off offset:96"
-                     : "=&v"(q_raw[0]), "=&v"(q_raw[1]), "=&v"(q_raw[2]), "=&v"(q_raw[3]) : "v"(qrow) : "memory");
-        if constexpr (KS == 8)
-            asm volatile("global_load_dwordx4 %0, %4, off offset:128\n\tglobal_load_dwordx4 %1, %4, off offset:160\n\t"
-                         "global_load_dwordx4 %2, %4, off offset:192\n\tglobal_load_dwordx4 %3, %4, off offset:224"
-                         : "=&v"(q_raw[KS - 4]), "=&v"(q_raw[KS - 3]), "=&v"(q_raw[KS - 2]), "=&v"(q_raw[KS - 1]) : "v"(qrow) : "memory");
-        const int last = req_nt_all - 1;
-        request_first_tiles(0, min(1, last), min(2, last));
+        const uint64_t qaddr = (uint64_t)(uintptr_t)(static_cast<const T *>(p.q) + req_b * p.qs[0] + req_h * p.qs[1]);
+        const u32x4 qrsrc = {uniform((uint32_t)qaddr), uniform((uint32_t)(qaddr >> 32) & 0xFFFFu),
+                             uniform((uint32_t)((((int64_t)M - 1) * p.qs[2] + D) * 2)), 0x00020000u};
+        const uint32_t qoff = (uint32_t)(((int64_t)min(my_m, M - 1) * p.qs[2] + lh * 8) * 2);
+        const uint32_t qdst = uniform(lds_base + Q_STAGE + wave * (KS * 1024));
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :: "s"(qdst + s * 1024), "v"(qoff), "s"(qrsrc), "s"(32 * s) : "memory", "m0");
         if (VEC) {
             // one value per key; keys past the end read as 0 through the bounds of the buffer resource and are set
             // to -inf afterwards
@@ -204,27 +207,43 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
             const u32x4 mrsrc = {uniform((uint32_t)maddr), uniform((uint32_t)(maddr >> 32) & 0xFFFFu),
                                  uniform((uint32_t)(((int64_t)(N - 1) * p.ms[3] + 1) * es)), 0x00020000u};
             const int step_bytes = (int)p.ms[3] * es;
-            if (p.mask_dtype == KERNL_F32) {
+            // load i of a wave covers 64 consecutive keys, lane l the key first + l, written to LDS as dword first + l
+            const int first = wave_rows ? 0 : 64 * wave, step = wave_rows ? 64 : 256;
+            const uint32_t mdst = uniform(lds_base + MASK_STAGE + (wave_rows ? wave * (WAVE_ROW_KEYS * 4) : 64 * 4 * wave));
 #pragma unroll
-                for (int i = 0; i < PER; ++i)
-                    asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(mask_raw[i]) : "v"((tid + 256 * i) * step_bytes), "s"(mrsrc) : "memory");
-            } else {
-#pragma unroll
-                for (int i = 0; i < PER; ++i)
-                    asm volatile("buffer_load_ushort %0, %1, %2, 0 offen" : "=v"(mask_raw[i]) : "v"((tid + 256 * i) * step_bytes), "s"(mrsrc) : "memory");
+            for (int i = 0; i < PER; ++i) {
+                if (first + step * i < N) {  // wave-uniform
+                    if (p.mask_dtype == KERNL_F32)
+                        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
+                                     :: "s"(mdst + step * 4 * i), "v"((first + step * i + lane) * step_bytes), "s"(mrsrc) : "memory", "m0");
+                    else
+                        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ushort %1, %2, 0 offen lds"
+                                     :: "s"(mdst + step * 4 * i), "v"((first + step * i + lane) * step_bytes), "s"(mrsrc) : "memory", "m0");
+                }
             }
         }
     };
-    auto item_loads_landed = [&]() __attribute__((always_inline)) {
-        if (VEC) {
-            asm volatile("s_waitcnt vmcnt(0)" : "+v"(q_raw[0]), "+v"(q_raw[1]), "+v"(q_raw[2]), "+v"(q_raw[3]), "+v"(mask_raw[0]), "+v"(mask_raw[1]),
-                         "+v"(mask_raw[2]), "+v"(mask_raw[3]), "+v"(mask_raw[4]), "+v"(mask_raw[5]), "+v"(mask_raw[6]), "+v"(mask_raw[7]) :: "memory");
-        } else {
-            asm volatile("s_waitcnt vmcnt(0)" : "+v"(q_raw[0]), "+v"(q_raw[1]), "+v"(q_raw[2]), "+v"(q_raw[3]) :: "memory");
+    auto request_item = [&](int idx) __attribute__((always_inline)) {
+        const int bh = 8 * (idx / p.nq_tiles) + xcd, qt = idx % p.nq_tiles;
+        req_b = bh / p.H;
+        req_h = bh % p.H;
+        req_q0 = (CAUSAL ? p.nq_tiles - 1 - qt : qt) * BM;
+        const int n_end = CAUSAL ? min(N, req_q0 + BM + p.causal_off) : N;
+        req_nt_all = (n_end + BN - 1) / BN;
+        set_kv(req_b, req_h);
+        const int last = req_nt_all - 1;
+        request_first_tiles(0, min(1, last), min(2, last));
+        request_staged();
+    };
+    // one mask value as the classification sees it: the staged dword of key n decoded, scaled to the log2 domain with
+    // -inf replaced by the clamp value, -inf past the last key
+    auto staged_mask_value = [&](uint32_t raw, int n) __attribute__((always_inline)) -> float {
+        float mv = __builtin_bit_cast(float, raw);
+        if (p.mask_dtype != KERNL_F32) {
+            const uint16_t bits = (uint16_t)raw;
+            mv = p.mask_dtype == KERNL_F16 ? (float)__builtin_bit_cast(f16, bits) : (float)__builtin_bit_cast(bf16, bits);
         }
-        // (the wait above is for everything outstanding; this one only ties the other four query registers to it)
-        if constexpr (KS == 8)
-            asm volatile("s_waitcnt vmcnt(0)" : "+v"(q_raw[KS - 4]), "+v"(q_raw[KS - 3]), "+v"(q_raw[KS - 2]), "+v"(q_raw[KS - 1]) :: "memory");
+        return n < N ? scale_mask(mv, p.clamp) : -INFINITY;
     };
     request_item(item);
     auto lds_barrier = []() __attribute__((always_inline)) {  // LDS writes of this wave are done, then the workgroup barrier
@@ -262,7 +281,7 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
         gen_bits = 0;
         for (int g = 0; g * 64 < npad; ++g) {
             const int n = g * 64 + lane;
-            const float v = bias_lds[n];
+            const float v = bias_lds[bias_wave + n];
             const bool valid = n < N;
             const bool any_nz = __ballot(valid && v != 0.0f) != 0, any_nm = __ballot(valid && v > kNegBig) != 0,
                        any_ord = __ballot(valid && v == 0.0f) != 0;
@@ -304,7 +323,7 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
         const int v0 = 2 * e;
         const int c0 = 32 * half + 8 * (v0 / 4) + (v0 % 4);  // key of the first score of the pair, relative to n0 + 4 lh
         if (VEC) {
-            const f32x2 cb = *reinterpret_cast<const f32x2 *>(bias_lds + n0 + c0 + lh * 4);
+            const f32x2 cb = *reinterpret_cast<const f32x2 *>(bias_lds + bias_wave + n0 + c0 + lh * 4);
             Sc[v0] += cb[0];
             Sc[v0 + 1] += cb[1];
         } else {
@@ -407,65 +426,90 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
         cur_h = req_h;
         cur_q0 = req_q0;
         cur_nt_all = req_nt_all;
-        item_loads_landed();
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of everything requested for the item has landed
+        // this wave's query rows (and, for short mask rows, its copy of the mask row) leave the staging areas before the
+        // barrier: after it any wave may request tiles into those ring slots
+        vec8 q_raw[KS];
+        {
+            const unsigned char *qs = smem + Q_STAGE + wave * (KS * 1024) + lane * 16;
+#pragma unroll
+            for (int s = 0; s < KS; ++s) q_raw[s] = *reinterpret_cast<const vec8 *>(qs + s * 1024);
+        }
+        uint32_t mraw[PER];
+        if (VEC && wave_rows) {
+            const uint32_t *ms = reinterpret_cast<const uint32_t *>(smem + MASK_STAGE) + wave * WAVE_ROW_KEYS + lane;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) mraw[i] = ms[64 * i];
+#pragma unroll
+            for (int i = 0; i < PER; ++i) asm volatile("" : "+v"(mraw[i]));  // the reads are done with before the barrier
+        }
+#pragma unroll
+        for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(q_raw[s]));
+        // all four waves' parts of the first tiles (and of a shared mask row) have landed: every wave waited for
+        // everything it had requested
+        lds_barrier();
         nt = cur_nt_all;
         n_clean = 0;
         first_tile = 0;
         order_pos = 1;
         bool zero_q = false;
-        if (VEC) {
-            // additive terms of all keys (log2 domain, -inf past the last key), relative to the largest one: softmax
-            // does not change when every key's term moves by the same amount, and this way some key is always
-            // "ordinary" (term 0), so the exponent reference set by the first tile is an ordinary score.  When even the
-            // largest term is a clamped -inf, fp32 scores would have absorbed q·k entirely: q is dropped, which gives
-            // the plain average of V over those keys, as the reference does.
+        // Per-key masks.  Additive terms of all keys (log2 domain, -inf past the last key), relative to the largest one:
+        // softmax does not change when every key's term moves by the same amount, and this way some key is always
+        // "ordinary" (term 0), so the exponent reference set by the first tile is an ordinary score.  When even the
+        // largest term is a clamped -inf, fp32 scores would have absorbed q·k entirely: q is dropped, which gives the
+        // plain average of V over those keys, as the reference does.
+        // Tile classes from two ballots per tile (lane l looks at key 64 i + l of tile i): clean = full and all zero,
+        // general = needs the masked body, neither = so negative everywhere that the tile contributes exactly 0.  Keys
+        // past the end carry -inf: neither zero nor above the "contributes nothing" bound, so a tile that holds one
+        // counts as non-zero — which is what a ragged tile must be — and a tile beyond the row sets no bit at all.
+        if (VEC && wave_rows) {
+            // every wave for itself, from registers: no exchange, no further barrier; the terms go to a copy of the
+            // wave's own
+            float mv[PER];
             float lmax = -INFINITY;
 #pragma unroll
             for (int i = 0; i < PER; ++i) {
-                const int n = tid + 256 * i;
-                float mv = mask_raw[i];
-                if (p.mask_dtype != KERNL_F32) {
-                    const uint16_t bits = (uint16_t)__builtin_bit_cast(uint32_t, mv);
-                    mv = p.mask_dtype == KERNL_F16 ? (float)__builtin_bit_cast(f16, bits) : (float)__builtin_bit_cast(bf16, bits);
-                }
-                mask_raw[i] = n < N ? scale_mask(mv, p.clamp) : -INFINITY;
-                lmax = fmaxf(lmax, mask_raw[i]);
+                mv[i] = staged_mask_value(mraw[i], lane + 64 * i);
+                lmax = fmaxf(lmax, mv[i]);
             }
-            lmax = wave_max(lmax);
-            if (lane == 0) red_lds[wave] = lmax;
-            lds_barrier();
-            const float bmax = fmaxf(fmaxf(red_lds[0], red_lds[1]), fmaxf(red_lds[2], red_lds[3]));
+            const float bmax = wave_max(lmax);
             zero_q = bmax < kNegBig;
-            // The 64 keys tid + 256 i of wave w are exactly tile w + 4 i: every wave classifies its own tiles with
-            // three ballots each — clean = full and all zero, general = needs the masked body, neither = so negative
-            // everywhere that the tile contributes exactly 0 — and the four waves exchange their bit sets through LDS.
-            uint32_t my_clean = 0, my_gen = 0, my_ord = 0;
+            uint32_t all_ord = 0;
+            clean_bits = 0;
+            gen_bits = 0;
 #pragma unroll
             for (int i = 0; i < PER; ++i) {
-                const int n = tid + 256 * i, tile = wave + 4 * i;
-                if (tile < cur_nt_all) {
-                    const float v = mask_raw[i] - bmax;
-                    bias_lds[n] = v;
-                    const bool valid = n < N;
-                    const bool any_nz = __ballot(valid && v != 0.0f) != 0, any_nm = __ballot(valid && v > kNegBig) != 0,
-                               any_ord = __ballot(valid && v == 0.0f) != 0;
-                    const bool full = tile * BN + BN <= N;
-                    if (any_nm) {
-                        if (any_nz || !full) my_gen |= 1u << tile;
-                        else my_clean |= 1u << tile;
-                    }
-                    if (any_ord) my_ord |= 1u << tile;
-                }
+                const float v = mv[i] - bmax;
+                bias_lds[bias_wave + lane + 64 * i] = v;
+                const uint64_t nz = __ballot(v != 0.0f), nm = __ballot(v > kNegBig);
+                const uint32_t bit = 1u << i;
+                gen_bits |= (nm != 0 && nz != 0) ? bit : 0u;
+                clean_bits |= (nm != 0 && nz == 0) ? bit : 0u;
+                all_ord |= (nz != ~0ull) ? bit : 0u;
             }
-            if (lane == 0) {
-                cls_lds[3 * wave] = my_clean;
-                cls_lds[3 * wave + 1] = my_gen;
-                cls_lds[3 * wave + 2] = my_ord;
+            pick_first(all_ord);
+        } else if (VEC) {
+            // long rows: every wave walks the whole staged row twice (maximum, then terms and classes); tile i's terms
+            // are written by wave i % 4, and a second barrier publishes them
+            const uint32_t *ms = reinterpret_cast<const uint32_t *>(smem + MASK_STAGE) + lane;
+            float lmax = -INFINITY;
+            for (int i = 0; i < cur_nt_all; ++i) lmax = fmaxf(lmax, staged_mask_value(ms[64 * i], lane + 64 * i));
+            const float bmax = wave_max(lmax);
+            zero_q = bmax < kNegBig;
+            uint32_t all_ord = 0;
+            clean_bits = 0;
+            gen_bits = 0;
+            for (int i = 0; i < cur_nt_all; ++i) {
+                const float v = staged_mask_value(ms[64 * i], lane + 64 * i) - bmax;
+                if ((i & 3) == wave) bias_lds[lane + 64 * i] = v;
+                const uint64_t nz = __ballot(v != 0.0f), nm = __ballot(v > kNegBig);
+                const uint32_t bit = 1u << i;
+                gen_bits |= (nm != 0 && nz != 0) ? bit : 0u;
+                clean_bits |= (nm != 0 && nz == 0) ? bit : 0u;
+                all_ord |= (nz != ~0ull) ? bit : 0u;
             }
-            lds_barrier();
-            clean_bits = cls_lds[0] | cls_lds[3] | cls_lds[6] | cls_lds[9];
-            gen_bits = cls_lds[1] | cls_lds[4] | cls_lds[7] | cls_lds[10];
-            pick_first(cls_lds[2] | cls_lds[5] | cls_lds[8] | cls_lds[11]);
+            pick_first(all_ord);
+            lds_barrier();  // the terms are in LDS, and nobody reads the staged row any more
         } else {
             n_clean = CAUSAL ? min(N / BN, (cur_q0 + p.causal_off + 1) / BN) : N / BN;
             n_clean = min(n_clean, nt);
@@ -476,10 +520,10 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
         {
             const int last = cur_nt_all - 1;
             const bool natural = tq[0] == 0 && tq[1] == min(1, last) && tq[2] == min(2, last);
-            if (!natural) {  // wave-uniform, and the same in every wave
-                __builtin_amdgcn_s_barrier();  // nobody's natural-order request is still in flight (all landed above)
+            if (!natural) {  // wave-uniform, and the same in every wave; nobody's natural-order request is still in flight
                 request_first_tiles(tq[0], tq[1], tq[2]);
                 __builtin_amdgcn_s_waitcnt(0x0F70);
+                __builtin_amdgcn_s_barrier();
             }
         }
         key_limit = (CAUSAL ? min(N - 1, cur_q0 + wave * 32 + lr + p.causal_off) : N - 1) - lh * 4;
@@ -511,7 +555,6 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
 
         // ================= position 0: K(0) has landed -> scores (against a reference of 0), row maximum = the
         // row's reference, probabilities of the lower half; then the unit-B half of a step =================
-        __builtin_amdgcn_s_barrier();  // all four waves' parts of the first tiles have landed (item_loads_landed waits for everything)
         {
             vec8 fa[KS], fb[KS];
 #pragma unroll
@@ -631,6 +674,10 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
                 // Plain loop over the same tiles in the same order: one tile at a time through ring slot 3 (the
                 // next item's first tiles sit in slots 0..2), running maximum as the reference, everything rescaled
                 // when it moves.  Runs with the finished item's addresses, mask terms (still in LDS) and rows.
+                // (the next item's staged rows are on their way into ring slot 3, which this loop uses: they must have
+                // landed everywhere before the first tile is requested; they are requested again afterwards)
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+                __syncthreads();
                 set_kv(cur_b, cur_h);
                 if (VEC) classify_tiles();
                 order_pos = 1;
@@ -691,7 +738,13 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
                     tile = next_tile(tile);
                 }
                 l_tot = halves32_sum(l_i);
-                if (next_item >= 0) set_kv(req_b, req_h);
+                if (next_item >= 0) {
+                    // the plain loop went through ring slot 3 of K and of V, where the next item's mask row and half of
+                    // its query rows were waiting: request them again
+                    set_kv(req_b, req_h);
+                    __syncthreads();
+                    request_staged();
+                }
             }
         }
         // ---- normalise and store: lane holds features 32 d + 16 lh + (0..15) of its row
@@ -750,6 +803,7 @@ bool launch_attention_pipe(const AttnParams &p, int D, int dtype, int mask_mode,
     if (D != 64 && D != 128) return false;
     if (mask_mode == MASK_MATRIX) return false;
     if (mask_mode == MASK_VECTOR && (causal || p.N > kPipeMaxMaskKeys)) return false;
+    if (((int64_t)p.M + 128) * p.qs[2] >= (1ll << 30)) return false;  // the query rows are fetched through 32-bit byte offsets
     if (!force && p.N < kPipeMinKeys) return false;
     // Head size 128 runs one workgroup per CU here and is no faster per tile than the streaming kernel (both sit at the
     // chip's power limit); what it wins is BALANCE when a causal problem has few (batch, head) pairs: a persistent

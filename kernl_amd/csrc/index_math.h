@@ -90,8 +90,10 @@ struct MaskTileMap {
 // ----------------------------------------------------------------------------------------------------
 // Wide linear kernel: which weight row (inside the tile) LDS row `row` of the weight tile carries.  LDS row `row` is
 // MFMA row r = row % 16 of 16-row block row / 16; the placement makes a lane end up with consecutive output columns:
-//   256 columns    in a 64-row group, block j row r carries weight row 16 (r/4) + 4 j + r%4: lane group g = lane / 16
-//                  holds the 16 columns 16 g .. 16 g + 15 of the group across its four blocks
+//   256 columns    in a 128-row group (the sub-tile of one wave), block j row r carries weight row 32 (r/4) + 4 j + r%4:
+//                  lane group g = lane / 16 holds the 32 columns 32 g .. 32 g + 31 across its eight blocks — 64
+//                  contiguous bytes of an output row, which a transposition inside each quad of lanes turns into
+//                  stores where four adjacent lanes cover those 64 bytes
 //   192 columns    32-row groups of two blocks: 8 (r/4) + 4 (j%2) + r%4 (8 consecutive columns per lane and group)
 //   gated          32 (j/2) + 8 (r/4) + 4 (j%2) + r%4: the lane holds gate AND value of the 8 output columns 8 g .. 8 g + 7
 // ----------------------------------------------------------------------------------------------------
@@ -99,7 +101,7 @@ template <bool GATED, int NBN>
 KERNL_HD int wide_weight_row(int row) {
     const int r = row & 15, j = (row >> 4) & 3;
     if (GATED) return (row & ~63) + 32 * (j >> 1) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3);
-    if (NBN == 8) return (row & ~63) + 16 * (r >> 2) + 4 * j + (r & 3);
+    if (NBN == 8) return (row & ~127) + 32 * (r >> 2) + 4 * ((row >> 4) & 7) + (r & 3);
     return (row & ~31) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3);
 }
 

@@ -399,9 +399,9 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 // consumed takes the next-but-one k-tile, one load every fourth MFMA.  (A burst of 16 loads followed by a wait for
 // all of them stalls a lone wave: 64 KB need >= 1024 cycles to pass the CU's 64 B/clk fill path.)
 //
-// Weight rows are placed in LDS so that a lane ends up with consecutive output columns: MFMA row r of block j in a
-// 64-row group carries weight row 16 (r/4) + 4 j + r%4, so lane group g = lane/16 holds the 16 columns 16 g .. 16 g+15
-// of the group across its four blocks.  Gated epilogues use 32 (j/2) + 8 (r/4) + 4 (j%2) + r%4 instead: the lane holds
+// Weight rows are placed in LDS so that a lane ends up with consecutive output columns: MFMA row r of block j of a
+// wave's 128 weight rows carries weight row 32 (r/4) + 4 j + r%4, so lane group g = lane/16 holds the 32 columns
+// 32 g .. 32 g+31 across its eight blocks (192-column tiles: 8 columns per lane and pair of blocks).  Gated epilogues use 32 (j/2) + 8 (r/4) + 4 (j%2) + r%4 instead: the lane holds
 // gate AND value of the 8 output columns 8 g .. 8 g + 7.
 // ----------------------------------------------------------------------------------------------------
 template <typename T>
@@ -418,8 +418,57 @@ __device__ __forceinline__ u32x4 fetch8(const T *__restrict__ p, int idx, int li
     return r;
 }
 
-// Epilogue of m-block IB (16 rows) of a wave of the wide kernel: lane (l16, g) holds row m_wave + 16 IB + l16 and, in
-// every group of JB n-blocks, the 4 JB consecutive columns starting at 4 JB g (JB = 4: 64-column groups, 2: 32-column).
+// Epilogue of m-block IB (16 rows) of a wave of the wide kernel.  Lane (l16, g) holds row m_wave + 16 IB + l16 and
+//   256-column tiles: the 32 consecutive columns 32 g .. 32 g + 31 of the wave's 128 (group G = blocks 4 G .. 4 G + 3:
+//                     columns 32 g + 16 G .. + 15),
+//   192-column tiles: in every 32-column group G (two blocks) the 8 consecutive columns 32 G + 8 g .. + 7.
+// Adjacent lanes hold DIFFERENT ROWS, so a 16-byte store per lane reaches memory as 64 separate 16-byte pieces.  Interior
+// blocks of 256-column tiles therefore transpose inside every quad of lanes first (two butterfly steps of
+// quad-permuting DPP moves and selects on the packed 16-bit results): afterwards lane i of a quad holds 16-byte chunk i
+// of each of the quad's four rows, and every store instruction has four adjacent lanes covering 64 contiguous bytes.
+// Measured on 16384 x 3072 x 768 without activation: 78 -> 72 us; covering whole 256-byte rows with 16 adjacent lanes
+// (through LDS) measured no better than the 64-byte form and costs LDS bandwidth that all four waves want at once.
+template <int NBN>
+__device__ __forceinline__ int wide_lane_col(int G, int g) {
+    return NBN == 8 ? 32 * g + 16 * G : 32 * G + 8 * g;
+}
+// quad_perm DPP move of every dword of a 16-byte value
+template <int CTRL>
+__device__ __forceinline__ u32x4 quad_perm4(u32x4 v) {
+    u32x4 r;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) r[d] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v[d], CTRL, 0xF, 0xF, true);
+    return r;
+}
+// 4 x 4 transposition inside every quad of lanes: on entry lane i holds P[c] = chunk c of ITS row, on return P[k] =
+// chunk i of the row of the quad's lane k.
+__device__ __forceinline__ void quad_transpose4(u32x4 (&P)[4], int lane_in_quad) {
+    const bool odd = (lane_in_quad & 1) != 0, upper = (lane_in_quad & 2) != 0;
+    u32x4 A[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const u32x4 other = quad_perm4<0xB1>(P[c ^ 1]);  // quad_perm [1,0,3,2]: the neighbour's other chunk of the pair
+        const bool keep = ((c & 1) != 0) == odd;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) A[c][d] = keep ? P[c][d] : other[d];
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const u32x4 other = quad_perm4<0x4E>(A[c ^ 2]);  // quad_perm [2,3,0,1]
+        const bool keep = ((c & 2) != 0) == upper;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) P[c][d] = keep ? A[c][d] : other[d];
+    }
+}
+
+// Row-padded LDS layout of the 192-column tiles' store transposition (see wide_epilogue_transposed): 16 rows of 192
+// bytes, 208 bytes apart
+template <int NBN>
+__device__ __forceinline__ int xpose_offset(int row, int chunk) {
+    static_assert(NBN == 6, "only the 192-column tiles transpose through LDS");
+    return row * 208 + (chunk << 4);
+}
+
 template <typename T, int ACT, int IB, int NBN, int NBM = 8>
 __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_wave, int n_wave, int l16, int g,
                                               T *__restrict__ out, T *__restrict__ act_in, int M, int N,
@@ -469,18 +518,36 @@ __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_
     };
     const bool interior = rows_inside && n_wave + NBN * 16 <= N && out_vec_ok && act_in == nullptr;
     if (__builtin_amdgcn_readfirstlane((int)interior)) {
+        if constexpr (NBN == 8) {
+            u32x4 P[4];  // chunk c = 2 G + h: columns 32 g + 8 c .. + 7 of this lane's row
+#pragma unroll
+            for (int G = 0; G < NG; ++G) {
+                float r[VPG];
+#pragma unroll
+                for (int v = 0; v < VPG; ++v) r[v] = apply_act16(acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v), ACT);
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) P[2 * G + h][v] = pack2<T>(r[8 * h + 2 * v], r[8 * h + 2 * v + 1]);
+            }
+            quad_transpose4(P, l16 & 3);
+            T *p = out + (int64_t)(m_wave + 16 * IB + (l16 & ~3)) * out_rs + n_wave + 32 * g + 8 * (l16 & 3);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) *reinterpret_cast<u32x4 *>(p + k * out_rs) = P[k];
+            return;
+        }
 #pragma unroll
         for (int G = 0; G < NG; ++G) {
             float r[VPG];
 #pragma unroll
             for (int v = 0; v < VPG; ++v) r[v] = apply_act16(acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v), ACT);
-            store_vec(out + (int64_t)m * out_rs + n_wave + 16 * JB * G + VPG * g, r);
+            store_vec(out + (int64_t)m * out_rs + n_wave + wide_lane_col<NBN>(G, g), r);
         }
         return;
     }
 #pragma unroll
     for (int G = 0; G < NG; ++G) {
-        const int n = n_wave + 16 * JB * G + VPG * g;
+        const int n = n_wave + wide_lane_col<NBN>(G, g);
         if (m >= M || n >= N) continue;
         float r[VPG];
 #pragma unroll
@@ -503,6 +570,73 @@ __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_
             for (int v = 0; v < VPG; ++v)
                 if (n + v < N) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
         }
+    }
+}
+
+// 192-column tiles: the whole epilogue of a wave whose sub-tile lies inside the matrix (plain activations, 16-byte
+// aligned contiguous output rows, no pre-activation side output).  A lane holds only 16 contiguous bytes of a row per
+// 32-column group here, so the transposition inside a quad of lanes that the 256-column tiles use has nothing to join;
+// the packed results go through a 4 KB LDS region of the wave's own instead (rows padded to 208 bytes: no bank
+// conflicts), and come back so that 12 adjacent lanes cover the 192 contiguous bytes of a row.  Only the wave itself
+// touches its region and LDS operations of one wave execute in program order: no barrier.  Software-pipelined by hand
+// over the 16-row blocks, because with one wave per SIMD nothing else hides the LDS round trip:
+//   values of block b (bias, activation, rounding)  ->  global stores of block b - 1 (its LDS reads were issued before
+//   those values were computed)  ->  LDS writes of block b  ->  LDS reads of block b.
+// Measured, graph replay: 16384 x 2304 x 768 60.3 -> 58.2 us, 16384 x 768 x 768 23.7 -> 23.0, 16384 x 768 x 3072 65.2 ->
+// 64.6 (direct stores with runs of 48 bytes per quad, the best a transposition inside quads can do here: 59.0 / 23.4 /
+// 65.0).
+template <typename T, int ACT, int NBN, int NBM>
+__device__ __forceinline__ void wide_epilogue_transposed(f32x4_acc (&acc)[NBM][NBN], int m_wave, int n_wave, int l16, int g,
+                                                         T *__restrict__ out, int64_t out_rs,
+                                                         const u32x4 (&braw)[NBN == 8 ? 2 : 3][2], unsigned char *xpose) {
+    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB, VPG = 4 * JB;
+    constexpr int CPR = NBN * 2, NK = CPR / 4;  // 16-byte chunks per row of the sub-tile; stores per lane and block
+    const int lane = 16 * g + l16;
+    int rd_off[NK];
+    int64_t st_off[NK];
+#pragma unroll
+    for (int k = 0; k < NK; ++k) {
+        const int idx = k * 64 + lane, row = idx / CPR, chunk = idx % CPR;
+        rd_off[k] = xpose_offset<NBN>(row, chunk);
+        st_off[k] = (int64_t)row * out_rs + 8 * chunk;
+    }
+    int wr_off[NG][VPG / 8];
+#pragma unroll
+    for (int G = 0; G < NG; ++G)
+#pragma unroll
+        for (int h = 0; h < VPG / 8; ++h) wr_off[G][h] = xpose_offset<NBN>(l16, 2 * JB * G + (VPG / 8) * g + h);
+    T *base = out + (int64_t)m_wave * out_rs + n_wave;
+    u32x4 rd[NK];
+#pragma unroll
+    for (int IB = 0; IB <= NBM; ++IB) {
+        u32x4 pk[NG][VPG / 8];
+        if (IB < NBM) {
+#pragma unroll
+            for (int G = 0; G < NG; ++G) {
+                float r[VPG];
+#pragma unroll
+                for (int v = 0; v < VPG; ++v) r[v] = apply_act16(acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v), ACT);
+#pragma unroll
+                for (int h = 0; h < VPG / 8; ++h)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) pk[G][h][v] = pack2<T>(r[8 * h + 2 * v], r[8 * h + 2 * v + 1]);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (IB > 0) {
+#pragma unroll
+            for (int k = 0; k < NK; ++k) *reinterpret_cast<u32x4 *>(base + (int64_t)(16 * (IB - 1)) * out_rs + st_off[k]) = rd[k];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (IB < NBM) {
+#pragma unroll
+            for (int G = 0; G < NG; ++G)
+#pragma unroll
+                for (int h = 0; h < VPG / 8; ++h) *reinterpret_cast<u32x4 *>(xpose + wr_off[G][h]) = pk[G][h];
+#pragma unroll
+            for (int k = 0; k < NK; ++k) rd[k] = *reinterpret_cast<const u32x4 *>(xpose + rd_off[k]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -780,23 +914,32 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 #pragma unroll
             for (int h = 0; h < 2; ++h)
                 braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0}
-                             : fetch8<T>(bias, n_wave + 16 * JB * G + (GATED ? 32 * h + 8 * g : 4 * JB * g + 8 * h), N, bias_vec_ok);
+                             : fetch8<T>(bias, n_wave + (GATED ? 64 * G + 32 * h + 8 * g : wide_lane_col<NBN>(G, g) + 8 * h), N, bias_vec_ok);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         landed = true;
         // one call per 16-row block: each stays small enough for the compiler to unroll completely, so the
         // accumulators are only ever indexed by constants and never leave the register file
+        bool whole_inside = false;
+        if constexpr (!GATED && NBN == 6)
+            whole_inside = m0 + wave_m * 128 + 128 <= M && n_wave + NBN * 16 <= N && out_vec_ok && act_in == nullptr;
+        if (__builtin_amdgcn_readfirstlane((int)whole_inside)) {
+            if constexpr (!GATED && NBN == 6)
+                wide_epilogue_transposed<T, ACT, NBN, 8>(acc, m0 + wave_m * 128, n_wave, l16, g, out, out_rs, braw,
+                                                         smem + 2 * (X_BYTES + W_BYTES) + wave * 4096);
+        } else {
 #define KERNL_WIDE_EPILOGUE(I)                                                                                         \
     wide_epilogue<T, ACT, I, NBN>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs, ai_cs,   \
                              out_vec_ok, ai_vec_ok, braw)
-        KERNL_WIDE_EPILOGUE(0);
-        KERNL_WIDE_EPILOGUE(1);
-        KERNL_WIDE_EPILOGUE(2);
-        KERNL_WIDE_EPILOGUE(3);
-        KERNL_WIDE_EPILOGUE(4);
-        KERNL_WIDE_EPILOGUE(5);
-        KERNL_WIDE_EPILOGUE(6);
-        KERNL_WIDE_EPILOGUE(7);
+            KERNL_WIDE_EPILOGUE(0);
+            KERNL_WIDE_EPILOGUE(1);
+            KERNL_WIDE_EPILOGUE(2);
+            KERNL_WIDE_EPILOGUE(3);
+            KERNL_WIDE_EPILOGUE(4);
+            KERNL_WIDE_EPILOGUE(5);
+            KERNL_WIDE_EPILOGUE(6);
+            KERNL_WIDE_EPILOGUE(7);
 #undef KERNL_WIDE_EPILOGUE
+        }
         idx += slots;
         if (!tile_origin(idx, m0, n0)) break;
     }
@@ -1062,7 +1205,15 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     for (int G = 0; G < NG; ++G)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
-            braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0} : fetch8<T>(bias, n_wave + 16 * JB * G + 4 * JB * g + 8 * h, N, bias_vec_ok);
+            braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0} : fetch8<T>(bias, n_wave + wide_lane_col<NBN>(G, g) + 8 * h, N, bias_vec_ok);
+    if constexpr (NBN == 6) {
+        const bool whole_inside = m0 + wave_m * (NBM * 16) + NBM * 16 <= M && n_wave + NBN * 16 <= N && out_vec_ok && act_in == nullptr;
+        if (__builtin_amdgcn_readfirstlane((int)whole_inside)) {
+            wide_epilogue_transposed<T, ACT, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, out_rs, braw,
+                                                       smem + 3 * 16384 + 3 * 32768 + wave * 4096);
+            return;
+        }
+    }
 #define KERNL_HALF_EPILOGUE(I)                                                                                         \
     wide_epilogue<T, ACT, I, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, \
                                        ai_rs, ai_cs, out_vec_ok, ai_vec_ok, braw)
@@ -1118,7 +1269,7 @@ linear_wide_half_reduce_kernel(const float *__restrict__ part, const T *__restri
     for (int G = 0; G < NG; ++G)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
-            braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0} : fetch8<T>(bias, n_wave + 16 * JB * G + 4 * JB * g + 8 * h, N, bias_vec_ok);
+            braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0} : fetch8<T>(bias, n_wave + wide_lane_col<NBN>(G, g) + 8 * h, N, bias_vec_ok);
 #define KERNL_HALF_REDUCE_EPILOGUE(IB)                                                                                   \
     if (I == IB)                                                                                                         \
     wide_epilogue<T, ACT, IB, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, \
@@ -1547,7 +1698,7 @@ static void launch_mfma_glu(const LinearArgs &a) {
 template <typename T, int ACT, int NBN = 8, bool W8 = false>
 static void launch_wide_act(const LinearArgs &a) {
     auto kern = linear_wide_kernel<T, ACT, NBN, W8>;
-    constexpr int LDS_BYTES = 2 * (256 + 256) * 128;
+    constexpr int LDS_BYTES = 2 * (256 + 256) * 128 + (NBN == 6 ? 4 * 4096 : 0);  // two stages (+ a 4 KB store-transposition region per wave)
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
@@ -1575,7 +1726,7 @@ static void launch_wide_half_act(const LinearArgs &a);
 template <typename T, int ACT, int NBN, bool W8 = false>
 static void launch_wide_half_act(const LinearArgs &a) {
     auto kern = linear_wide_half_kernel<T, ACT, NBN, W8>;
-    constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768;
+    constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768 + (NBN == 6 ? 4 * 4096 : 0);  // three stages (+ a 4 KB store-transposition region per wave: all 160 KB)
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);

@@ -42,3 +42,9 @@ def check_weight_placement(layout: str) -> None:
                     raise AssertionError(f"gated: lane group {g} holds {cols}, not 8 gate columns and their value columns")
             elif cols != list(range(cols[0], cols[0] + len(cols))) or cols[0] % len(cols) != 0:
                 raise AssertionError(f"{layout}: lane group {g} holds {cols}, not consecutive output columns")
+        if layout == "256":
+            # the two groups of a wave's eight blocks follow each other: 32 consecutive columns, 64-byte aligned
+            for first in range(0, len(groups), 2):
+                both = groups[first] + groups[first + 1]
+                if both != list(range(both[0], both[0] + 32)) or both[0] % 32 != 0:
+                    raise AssertionError(f"256: lane group {g} holds {both}, not 32 consecutive output columns")

@@ -70,6 +70,36 @@ def test_attention_vs_oracle(shape, mask_kind, causal, dtype, close):
     close(out, ref, dtype, what=f"attention {shape} {mask_kind} causal={causal}")
 
 
+@pytest.mark.parametrize("mask_dtype", ["fp32", "same"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("keys", [200, 512, 1500])
+def test_per_key_mask_of_every_dtype_and_length(keys, dtype, mask_dtype, close):
+    """Per-key masks with ordinary values, a -inf tail and a fully masked batch entry, as fp32 and in the inputs' 16-bit
+    type, on rows that one wave classifies by itself (up to 512 keys) and on longer ones, with enough (batch, head) pairs
+    that the persistent kernel walks several items per workgroup (its next item's query and mask rows are prefetched
+    into LDS while the current one finishes)."""
+    B, H, D = 9, 16, 64
+    gen = torch.Generator().manual_seed(keys)
+    q, k, v = (_mk((B, H, keys, D), dtype, gen) for _ in range(3))
+    mask = torch.randn((B, 1, 1, keys), generator=gen)
+    lengths = torch.randint(1, keys + 1, (B,), generator=gen)
+    for b in range(B):
+        if b % 3 != 0:
+            mask[b, :, :, : lengths[b]] = 0.0          # a plain padding mask: zeros, then -inf
+        mask[b, :, :, lengths[b]:] = float("-inf")
+    mask[4] = float("-inf")                            # nothing visible: the plain average of V
+    mask = mask.to(torch.float32 if mask_dtype == "fp32" else dtype)
+    print(f"case keys={keys} dtype={dtype} mask={mask.dtype}", flush=True)
+    out = _run(q, k, v, 0.125, False, mask)
+    ref = attention_oracle(q, k, v, 0.125, False, mask)
+    # every key at -inf: the reference kernel replaces -inf by the most negative finite value of the MASK's dtype
+    # (attention.py:380,516) and adds that to the fp32 scores — an fp32 minimum absorbs them (uniform softmax), a
+    # half-precision one (-65504) leaves them their weight; the closed form above has no such row
+    floor = torch.full((1, 1, 1, keys), torch.finfo(mask.dtype).min, dtype=torch.float32)
+    ref[4] = attention_oracle(q[4:5], k[4:5], v[4:5], 0.125, False, floor)[0]
+    close(out, ref, dtype, what=f"per-key mask {keys} {mask.dtype}")
+
+
 def test_attention_u02_inputs_like_reference(close):
     # reference draws q, k, v from U(0, 2) with sm_scale 0.3 (test/test_attention.py:91-99): large positive logits
     gen = torch.Generator().manual_seed(1)

@@ -105,7 +105,9 @@ def test_wide_linear_weight_placement(layout):
     check_weight_placement(layout)
     cols = lane_columns(layout, 192 if layout == "192" else 256)
     if layout == "256":
-        assert cols[0][0] == list(range(16)) and cols[3][0] == list(range(48, 64)) and cols[1][1] == list(range(80, 96))
+        # lane group g: columns 32 g .. 32 g + 31 of each wave's 128 (64 contiguous bytes of an output row), eight blocks
+        assert cols[0][0] + cols[0][1] == list(range(32)) and cols[3][0] + cols[3][1] == list(range(96, 128))
+        assert cols[1][2] + cols[1][3] == list(range(160, 192))
     if layout == "192":
         assert cols[0][0] == list(range(8)) and cols[2][1] == list(range(48, 56))
     if layout == "gated":
