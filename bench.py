@@ -34,12 +34,13 @@ PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E
 
 
 def _event_times(fn, n, flush=None):
+    """HIP-event time of each of `n` calls of `fn`; `flush` (a callable) runs untimed before every call."""
     import torch
 
     times = []
     for _ in range(n):
         if flush is not None:
-            flush.zero_()
+            flush()
         s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         s.record()
         fn()
@@ -49,18 +50,72 @@ def _event_times(fn, n, flush=None):
     return times
 
 
+ATTENTION_KERNEL_SOURCES = ("attention.hip", "attention_pipe.hip", "attention_common.h", "index_math.h", "common.h")
+
+
+def attention_sources_digest():
+    """sha256 over the sources the headline kernel is compiled from: ties a counter summary under profiles/ to the
+    kernel it was taken from."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in ATTENTION_KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "kernl_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def traffic_from_profile():
     """HBM bytes per launch of the headline kernel as measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE runs,
     each scaled by the same counter's reading for a copy of known size): the line `traffic_bytes_per_launch: <number>`
-    of profiles/attention_config1_pmc_traffic.txt, or None when the file is not there."""
+    of profiles/attention_config1_pmc_traffic.txt.  None when the file is not there, or when its line
+    `kernel_sources_sha256:` does not match the attention sources in the tree (the summary is of another kernel)."""
     path = os.path.join(ROOT, "profiles", "attention_config1_pmc_traffic.txt")
+    value, digest = None, None
     try:
         for line in open(path):
             if line.startswith("traffic_bytes_per_launch:"):
-                return float(line.split(":", 1)[1].split()[0])
+                value = float(line.split(":", 1)[1].split()[0])
+            if line.startswith("kernel_sources_sha256:"):
+                digest = line.split(":", 1)[1].strip()
     except OSError:
-        pass
-    return None
+        return None
+    try:
+        return value if digest == attention_sources_digest() else None
+    except OSError:
+        return None
+
+
+class CacheFlush:
+    """The two ways of emptying the caches in front of a timed launch.
+
+    dirty()  rewrites a 256 MB buffer (what the reference's benchmark fixture does, benchmark_fixture.py:71-90, written
+             for a 6 MB L2).  On this chip it leaves up to 256 MB of DIRTY lines in the memory-side cache, which the
+             measured kernel's own traffic then has to write back: its time includes that write-back.
+    clean()  READS a 512 MB buffer that was zeroed once (kernl_probe_rate kind 4): the caches end up full of clean lines
+             that are dropped for free — the measured kernel pays for its own bytes only.  This is the figure the
+             `*_cold_clean_us` fields and the LayerNorm fraction of the HBM peak are put on."""
+
+    def __init__(self, dev):
+        import torch
+
+        from kernl_amd import _lib
+
+        self._lib, self._torch = _lib, torch
+        self.dirty_buf = torch.empty(256 * 1024 * 1024, dtype=torch.int8, device=dev)
+        self.clean_buf = torch.zeros(512 * 1024 * 1024, dtype=torch.int8, device=dev)
+        self.stats = torch.zeros((4096, 2), dtype=torch.int64, device=dev)
+        self.sink = torch.empty((4096 * 256,), dtype=torch.float32, device=dev)
+        torch.cuda.synchronize()
+
+    def dirty(self):
+        self.dirty_buf.zero_()
+
+    def clean(self):
+        st = self._lib.load().kernl_probe_rate(4, 0, 4096, self.clean_buf.data_ptr(), 0, self.clean_buf.numel(),
+                                              self.stats.data_ptr(), self.sink.data_ptr(),
+                                              self._torch.cuda.current_stream().cuda_stream)
+        self._lib._check(st, "kernl_probe_rate")
 
 
 def measured_peaks(dev, reps=3, ms_target=20.0):
@@ -121,6 +176,78 @@ def measured_peaks(dev, reps=3, ms_target=20.0):
     return out
 
 
+LLAMA7B_PREFILL_FLOP = 28.16e12  # 32 x (828.93 G linear + 34.36 G causal attention) + 536.9 G output head, b1 s2048
+
+
+def llama7b_prefill(dev, layers=32, seq=2048):
+    """BASELINE configs[4]: a Llama-2-7B-shaped decoder (hidden 4096, 32 heads of 128, SwiGLU 11008, RMSNorm eps 1e-5,
+    RoPE base 10000, vocabulary 32000), random N(0, 0.02) fp16 weights created on the GPU, batch 1, `seq` tokens, causal
+    prefill of the decoder stack + output head through optimize_model (hipGraph replay, median wall clock of 5).  The
+    hidden states are checked to be finite and compared with eager fp16 PyTorch on the same weights."""
+    import torch
+    import torch._dynamo
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from kernl_amd.model_optimization import optimize_model
+
+    torch._dynamo.reset()
+    cfg = LlamaConfig(num_hidden_layers=layers, hidden_size=4096, num_attention_heads=32, num_key_value_heads=32,
+                      intermediate_size=11008, vocab_size=32000, rms_norm_eps=1e-5, max_position_embeddings=4096,
+                      rope_theta=10000.0, initializer_range=0.02, tie_word_embeddings=False)
+    cfg._attn_implementation = "sdpa"
+    old_dtype = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float16)
+    try:
+        torch.manual_seed(0)
+        with torch.device(dev):
+            model = LlamaForCausalLM(cfg).eval()
+    finally:
+        torch.set_default_dtype(old_dtype)
+    gen = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, 32000, (1, seq), generator=gen).to(dev)
+    out = {}
+    with torch.inference_mode():
+        eager = model(input_ids=ids, use_cache=False).logits.float()
+        # the fp16 operators clamp the norms' epsilon to 1.6e-5 as the reference does (layer_norm.py:295-296); an eager
+        # run with that epsilon separates the clamp's effect — which 65 norms over N(0, 0.02) weights compound — from
+        # the kernels' own error
+        norms = [m for m in model.modules() if hasattr(m, "variance_epsilon")]
+        for m in norms:
+            m.variance_epsilon = max(m.variance_epsilon, 1.6e-5)
+        eager_clamped = model(input_ids=ids, use_cache=False).logits.float()
+        for m in norms:
+            m.variance_epsilon = cfg.rms_norm_eps
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        optimize_model(model)
+        for _ in range(3):
+            got = model(input_ids=ids, use_cache=False).logits
+        torch.cuda.synchronize()
+        out["llama7b_b1_s2048_compile_and_capture_s"] = round(time.perf_counter() - t0, 1)
+        times = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            model(input_ids=ids, use_cache=False)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+    assert torch.isfinite(got).all(), "Llama-7B-shaped prefill: non-finite logits"
+    ms = statistics.median(times)
+    tag = "llama7b_b1_s2048" if (layers, seq) == (32, 2048) else f"llama7b_width_{layers}_layers_s{seq}"
+    out[f"{tag}_fwd_ms"] = round(ms, 3)
+    if (layers, seq) == (32, 2048):
+        out[f"{tag}_tflops"] = round(LLAMA7B_PREFILL_FLOP / (ms * 1e-3) / 1e12, 1)
+        out[f"{tag}_frac_of_mfma_peak"] = round(LLAMA7B_PREFILL_FLOP / (ms * 1e-3) / 1e12 / PEAK_MFMA_F16_TFLOPS, 4)
+    out[f"{tag}_mean_rel_diff_vs_fp16_eager"] = round(((got.float() - eager).abs().mean() / eager.abs().mean()).item(), 5)
+    out[f"{tag}_max_abs_diff_vs_fp16_eager"] = round((got.float() - eager).abs().max().item(), 5)
+    out[f"{tag}_mean_rel_diff_vs_fp16_eager_with_clamped_eps"] = round(
+        ((got.float() - eager_clamped).abs().mean() / eager_clamped.abs().mean()).item(), 5)
+    out[f"{tag}_mean_rel_diff_of_the_eps_clamp_alone"] = round(
+        ((eager_clamped - eager).abs().mean() / eager.abs().mean()).item(), 5)
+    del model, eager, eager_clamped, got
+    torch.cuda.empty_cache()
+    return out
+
+
 def config1_inputs():
     import torch
 
@@ -161,6 +288,9 @@ def main():
     ap.add_argument("--skip-e2e", action="store_true", help="skip the BERT-base forward latency")
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline timings")
     ap.add_argument("--skip-extra", action="store_true", help="only the headline attention numbers")
+    ap.add_argument("--skip-llama32", action="store_true", help="skip the 32-layer Llama-7B-shaped prefill (configs[4])")
+    ap.add_argument("--llama-probe", action="store_true",
+                    help="run only the 32-layer Llama-7B-shaped prefill (configs[4]) and print its figures as one JSON line")
     ap.add_argument(
         "--pmc-probe",
         action="store_true",
@@ -189,6 +319,26 @@ def main():
         "and exit: the workload of the rocprofv3 --kernel-trace run behind profiles/bert_base_batch1_kernel_trace.txt",
     )
     ap.add_argument(
+        "--pmc-probe-linear",
+        action="store_true",
+        help="launch the config-2 up projection (tanh-GELU), its erf-GELU form and the down projection 3 times each, then "
+        "copy a 64 MiB tensor 3 times, and exit: the workload of the rocprofv3 --pmc runs behind "
+        "profiles/linear_config2_pmc_sq.txt",
+    )
+    ap.add_argument(
+        "--pmc-probe-layernorm",
+        action="store_true",
+        help="launch the config-2 LayerNorm and a LayerNorm of 16 times the rows 3 times each, then copy a 64 MiB tensor 3 "
+        "times, and exit: the workload of the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs behind "
+        "profiles/layernorm_config2_pmc_traffic.txt",
+    )
+    ap.add_argument(
+        "--e2e-probe",
+        action="store_true",
+        help="run BERT-base fp16 b32 s512 (BASELINE config 3) through optimize_model, 12 hipGraph replays, and exit: the "
+        "workload of the rocprofv3 --kernel-trace run behind profiles/bert_base_b32_s512_kernel_trace.txt",
+    )
+    ap.add_argument(
         "--peak-probe",
         action="store_true",
         help="run only the rate probes (register-only MFMA loops of both shapes, the attention loop's instruction mix, a "
@@ -215,6 +365,9 @@ def main():
     if args.peak_probe:
         print(json.dumps(measured_peaks(dev)), flush=True)
         return
+    if args.llama_probe:
+        print(json.dumps(llama7b_prefill(dev)), flush=True)
+        return
 
     # ------------------------------------------------------------------ headline: fused attention, config 1
     q, k, v, mask, lengths = config1_inputs()
@@ -228,14 +381,59 @@ def main():
     def step():
         attention_forward(qd, kd, vd, out, 0.125, False, md)
 
+    def copy_64mib(times=3):
+        src = torch.empty(32 * 1024 * 1024, dtype=torch.half, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(times):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
     if args.pmc_probe:
         for _ in range(3):
             step()
         torch.cuda.synchronize()
-        src = torch.empty(32 * 1024 * 1024, dtype=torch.half, device=dev).normal_()
-        dst = torch.empty_like(src)
+        copy_64mib()
+        return
+
+    if args.pmc_probe_linear:
+        c2 = config2_tensors(dev)
+        for act in ("fast_gelu", "gelu"):
+            for _ in range(3):
+                linear_layer(c2["x_up"], c2["w_up"], c2["b_up"], act)
         for _ in range(3):
-            dst.copy_(src)
+            linear_layer(c2["x_dn"], c2["w_dn"], c2["b_dn"], "")
+        torch.cuda.synchronize()
+        copy_64mib()
+        return
+
+    if args.pmc_probe_layernorm:
+        c2 = config2_tensors(dev)
+        x16 = torch.randn((16 * c2["M"], c2["K"]), generator=c2["gen"]).half().to(dev)
+        for _ in range(3):
+            layer_norm(c2["x_ln"], c2["g_ln"], c2["be_ln"], 1e-12)
+        for _ in range(3):
+            layer_norm(x16, c2["g_ln"], c2["be_ln"], 1e-12)
+        torch.cuda.synchronize()
+        copy_64mib()
+        return
+
+    if args.e2e_probe:
+        from transformers import BertConfig, BertModel
+
+        from kernl_amd.model_optimization import optimize_model
+
+        torch.manual_seed(0)
+        cfg = BertConfig()
+        cfg._attn_implementation = "eager"
+        model = BertModel(cfg).eval().half().to(dev)
+        gen = torch.Generator().manual_seed(0)
+        ids = torch.randint(0, 30522, (32, 512), generator=gen).to(dev)
+        lens = torch.randint(256, 513, (32,), generator=gen)
+        amask = (torch.arange(512)[None, :] < lens[:, None]).long().to(dev)
+        optimize_model(model)
+        with torch.inference_mode():
+            for _ in range(15):  # 3 warm-up / capture calls, then 12 replays
+                model(input_ids=ids, attention_mask=amask)
         torch.cuda.synchronize()
         return
 
@@ -291,7 +489,7 @@ def main():
 
     if args.cold_probe:
         c2 = config2_tensors(dev)
-        flush = torch.empty(256 * 1024 * 1024, dtype=torch.int8, device=dev)
+        flusher = CacheFlush(dev)
         cp_dst = torch.empty_like(c2["x_ln"])
         probes = [
             step,
@@ -300,10 +498,11 @@ def main():
             lambda: layer_norm(c2["x_ln"], c2["g_ln"], c2["be_ln"], 1e-12),
             lambda: cp_dst.copy_(c2["x_ln"]),
         ]
-        for fn in probes:
-            for _ in range(20):
-                flush.zero_()
-                fn()
+        for flush in (flusher.dirty, flusher.clean):  # per kernel: 20 launches after a rewrite, then 20 after a read
+            for fn in probes:
+                for _ in range(20):
+                    flush()
+                    fn()
         torch.cuda.synchronize()
         return
 
@@ -413,7 +612,7 @@ def main():
 
     # ------------------------------------------------------------------ the other kernels of the metric (config 2)
     if not args.skip_extra:
-        flush = torch.empty(256 * 1024 * 1024, dtype=torch.int8, device=dev)
+        flusher = CacheFlush(dev)
         c2 = config2_tensors(dev)
         gen = c2["gen"]
         M, Kd, N = c2["M"], c2["K"], c2["N"]
@@ -438,22 +637,27 @@ def main():
             torch.cuda.synchronize()
             return statistics.median(_event_times(g.replay, 20)) / reps
 
-        def cold_us(fn):
-            """Median of 30 single launches, each after the 256 MB flush buffer has been rewritten (memory-side cache
-            and L2 hold none of the operands), timed with an event pair around the launch."""
-            return statistics.median(_event_times(fn, 30, flush)) * 1e3
+        def cold_us(fn, clean=False):
+            """Median of 30 single launches, each timed with an event pair after the caches have been emptied: by
+            rewriting 256 MB (the reference fixture's way; leaves dirty lines the launch has to write back) or, with
+            `clean`, by reading 512 MB of zeros (clean lines; see CacheFlush)."""
+            return statistics.median(_event_times(fn, 30, flusher.clean if clean else flusher.dirty)) * 1e3
 
         def measure(fn, label, work, unit_scale, peak):
             warm = graph_time_ms(fn)
             cold = cold_us(fn)
             extra[f"{label}_us_graph_replay"] = round(warm * 1e3, 2)
             extra[f"{label}_cold_us"] = round(cold, 2)
+            extra[f"{label}_cold_clean_us"] = round(cold_us(fn, clean=True), 2)
             rate = work / (warm * 1e-3) / unit_scale
             extra[f"{label}_tflops_graph_replay"] = round(rate, 1)
             extra[f"{label}_frac_of_peak"] = round(rate / peak, 4)
             extra[f"{label}_cold_frac_of_peak"] = round(work / (cold * 1e-6) / unit_scale / peak, 4)
+            extra[f"{label}_cold_clean_frac_of_peak"] = round(
+                work / (extra[f"{label}_cold_clean_us"] * 1e-6) / unit_scale / peak, 4)
 
         extra["attention_cold_us"] = round(cold_us(step), 2)
+        extra["attention_cold_clean_us"] = round(cold_us(step, clean=True), 2)
         # the same problem with one additive value per (query, key): a mask broadcast over heads (fp32), and a
         # position bias broadcast over the batch, in the model's dtype
         for label, mshape, mdt in (("attention_mask_b1ss_fp32", (B, 1, S, S), torch.float32),
@@ -476,26 +680,45 @@ def main():
 
         t = graph_time_ms(ln_once, reps=20)
         cold = cold_us(ln_once)
+        cold_clean = cold_us(ln_once, clean=True)
         extra["layernorm_us_graph_replay"] = round(t * 1e3, 2)
         extra["layernorm_gbps_graph_replay"] = round(ln_bytes / (t * 1e-3) / 1e9, 1)
         extra["layernorm_cold_us"] = round(cold, 2)
         extra["layernorm_cold_gbps"] = round(ln_bytes / (cold * 1e-6) / 1e9, 1)
-        extra["layernorm_frac_of_hbm_peak"] = round(ln_bytes / (cold * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4)
+        extra["layernorm_cold_clean_us"] = round(cold_clean, 2)
+        extra["layernorm_cold_clean_gbps"] = round(ln_bytes / (cold_clean * 1e-6) / 1e9, 1)
+        # the fraction of the HBM peak is put on the launch after a CLEAN flush: operands come from HBM, and nobody
+        # else's dirty lines are written back inside the timed region (the dirty figure stays beside it)
+        extra["layernorm_frac_of_hbm_peak"] = round(ln_bytes / (cold_clean * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4)
+        extra["layernorm_cold_dirty_frac_of_hbm_peak"] = round(ln_bytes / (cold * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4)
         extra["layernorm_warm_frac_of_hbm_peak"] = round(ln_bytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
-        # four times the rows: ramp and drain weigh less
-        x_ln4 = torch.randn((4 * M, Kd), generator=gen).half().to(dev)
-        cold4 = cold_us(lambda: layer_norm(x_ln4, g_ln, be_ln, 1e-12))
-        extra["layernorm_65536x768_cold_us"] = round(cold4, 2)
-        extra["layernorm_65536x768_cold_gbps"] = round(4 * ln_bytes / (cold4 * 1e-6) / 1e9, 1)
-        del x_ln4
+        # four and sixteen times the rows (201 MB and 805 MB of traffic: more than the memory-side cache holds, so the
+        # graph-replayed figure is an HBM figure too): ramp and drain weigh less
+        for mult in (4, 16):
+            x_big = torch.randn((mult * M, Kd), generator=gen).half().to(dev)
+            fn_big = lambda: layer_norm(x_big, g_ln, be_ln, 1e-12)  # noqa: E731
+            c_d, c_c = cold_us(fn_big), cold_us(fn_big, clean=True)
+            w_big = graph_time_ms(fn_big, reps=5)
+            tag = f"layernorm_{mult * M}x{Kd}"
+            extra[f"{tag}_cold_us"] = round(c_d, 2)
+            extra[f"{tag}_cold_gbps"] = round(mult * ln_bytes / (c_d * 1e-6) / 1e9, 1)
+            extra[f"{tag}_cold_clean_us"] = round(c_c, 2)
+            extra[f"{tag}_cold_clean_gbps"] = round(mult * ln_bytes / (c_c * 1e-6) / 1e9, 1)
+            extra[f"{tag}_us_graph_replay"] = round(w_big * 1e3, 2)
+            extra[f"{tag}_frac_of_hbm_peak_graph_replay"] = round(mult * ln_bytes / (w_big * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
+            extra[f"{tag}_frac_of_hbm_peak_cold_clean"] = round(mult * ln_bytes / (c_c * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4)
+            del x_big, fn_big
         # what a plain device-to-device copy of the same 2 x 25 MB reaches on this box (the practical HBM ceiling)
         cp_src, cp_dst = x_ln, torch.empty_like(x_ln)
         t = graph_time_ms(lambda: cp_dst.copy_(cp_src), reps=20)
         cold = cold_us(lambda: cp_dst.copy_(cp_src))
+        cold_clean = cold_us(lambda: cp_dst.copy_(cp_src), clean=True)
         extra["copy_same_bytes_gbps_graph_replay"] = round(2 * x_ln.numel() * 2 / (t * 1e-3) / 1e9, 1)
         extra["copy_same_bytes_cold_us"] = round(cold, 2)
         extra["copy_same_bytes_cold_gbps"] = round(2 * x_ln.numel() * 2 / (cold * 1e-6) / 1e9, 1)
-        del flush
+        extra["copy_same_bytes_cold_clean_us"] = round(cold_clean, 2)
+        extra["copy_same_bytes_cold_clean_gbps"] = round(2 * x_ln.numel() * 2 / (cold_clean * 1e-6) / 1e9, 1)
+        del flusher
 
         # ---- the decoder-side kernels (Llama-7B prefill / decode shapes), graph-replayed
         try:
@@ -741,6 +964,14 @@ def main():
             del llama
         except Exception as exc:
             extra["llama7b_width_error"] = f"{type(exc).__name__}: {exc}"[:300]
+
+        # configs[4] at its stated depth: 32 decoder layers (6.6 G parameters, 13.5 GB in fp16) built directly on the GPU
+        # in fp16 with N(0, 0.02) weights, batch 1, 2048 tokens, causal prefill through optimize_model + hipGraph
+        if not args.skip_llama32:
+            try:
+                extra.update(llama7b_prefill(dev))
+            except Exception as exc:
+                extra["llama7b_32_layers_error"] = f"{type(exc).__name__}: {exc}"[:300]
 
     # ------------------------------------------------------------------ what this box sustains (rate probes)
     if not args.skip_extra:

@@ -21,7 +21,12 @@ struct Row16 {  // one 16-byte chunk of a row
 // before it reduces the current one, so that loads of one row overlap the arithmetic and the stores of another.
 // HALF (single-wave groups only): a group is half a wave, so that a wave works on two rows at once — rows of 32·k
 // chunks with odd k (768 fp16 values are 96 chunks) then keep every lane busy.
-template <typename T, int CHUNKS, bool RMS, bool HAS_RES, int GROUP_WAVES, bool HALF = false>
+// FULL: the row is exactly CHUNKS chunks per thread of the group, so no chunk needs a bounds test, gamma / beta are
+// converted to fp32 once per group instead of once per row, and a group whose row lies beyond M (the upper half of
+// the last wave) computes on the last row again and skips the store — the per-element selects of the general form
+// are gone.  BASELINE config 2 (768 fp16 values = 3 chunks per lane of a half wave) went from about 450 to about 250
+// instructions per row pair: on such inputs the vector ALU work is of the order of the memory time.
+template <typename T, int CHUNKS, bool RMS, bool HAS_RES, int GROUP_WAVES, bool HALF = false, bool FULL = false>
 __global__ void __launch_bounds__(256)
 layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const T *__restrict__ w,
                       const T *__restrict__ b, T *__restrict__ out, float *__restrict__ mean_out,
@@ -55,37 +60,49 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
         return (red[slot][0] + red[slot][1]) + (red[slot][2] + red[slot][3]);
     };
 
-    // gamma / beta stay in registers (as 16-bit values) for every row this group visits.
+    // gamma / beta stay in registers (as 16-bit values; FULL: as fp32) for every row this group visits.
     chunk_t wv[CHUNKS], bv[CHUNKS];
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int ci = t + c * G;
-        if (ci < nchunks) {
+        if (FULL || ci < nchunks) {
             wv[c] = *reinterpret_cast<const chunk_t *>(w + (int64_t)ci * E);
             if (b != nullptr) bv[c] = *reinterpret_cast<const chunk_t *>(b + (int64_t)ci * E);
         }
+    }
+    constexpr int CF = FULL ? CHUNKS : 1;
+    float wf[CF][E], bf[CF][E];
+    if (FULL) {
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                wf[c][e] = to_float(wv[c].v[e]);
+                bf[c][e] = b != nullptr ? to_float(bv[c].v[e]) : 0.0f;
+            }
     }
 
     const int row_step = gridDim.x * groups_per_block;
     int row = blockIdx.x * groups_per_block + group;
     chunk_t xn[CHUNKS], rn[HAS_RES ? CHUNKS : 1];
     auto fetch = [&](int r) {
+        if (FULL) r = min(r, M - 1);  // a group beyond the last row reads the last row again (and stores nothing)
         const T *xr = x + (int64_t)r * x_rs;
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
             const int ci = t + c * G;
-            if (ci < nchunks) xn[c] = *reinterpret_cast<const chunk_t *>(xr + (int64_t)ci * E);
+            if (FULL || ci < nchunks) xn[c] = *reinterpret_cast<const chunk_t *>(xr + (int64_t)ci * E);
         }
         if (HAS_RES) {
             const T *rr = res + (int64_t)r * res_rs;
 #pragma unroll
             for (int c = 0; c < CHUNKS; ++c) {
                 const int ci = t + c * G;
-                if (ci < nchunks) rn[c] = *reinterpret_cast<const chunk_t *>(rr + (int64_t)ci * E);
+                if (FULL || ci < nchunks) rn[c] = *reinterpret_cast<const chunk_t *>(rr + (int64_t)ci * E);
             }
         }
     };
-    if (row < M) fetch(row);
+    if (FULL || row < M) fetch(row);
 
     // with half-wave groups the wave stays together while its lower half has a row; the upper half's last row may
     // lie beyond M, then it computes on zeros and stores nothing
@@ -98,14 +115,14 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 float a = 0.0f;
-                if (ci < nchunks && live) {
+                if (FULL || (ci < nchunks && live)) {
                     a = to_float(xn[c].v[e]);
                     if (HAS_RES) a += to_float(rn[c].v[e]);
                 }
                 v[c][e] = a;
             }
         }
-        if (row + row_step < M) fetch(row + row_step);
+        if (FULL ? lead + row_step < M : row + row_step < M) fetch(row + row_step);
 
         float mean = 0.0f, var;
         if (RMS) {
@@ -126,7 +143,7 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
 #pragma unroll
             for (int c = 0; c < CHUNKS; ++c) {
                 const int ci = t + c * G;
-                if (ci < nchunks) {
+                if (FULL || ci < nchunks) {
 #pragma unroll
                     for (int e = 0; e < E; ++e) {
                         const float d = v[c][e] - mean;
@@ -143,15 +160,21 @@ layernorm_rows_kernel(const T *__restrict__ x, const T *__restrict__ res, const 
         }
 
         T *orow = out + (int64_t)row * out_rs;
+        const float shift = -mean * rstd;  // (v - mean) * rstd = v * rstd + shift
 #pragma unroll
         for (int c = 0; c < CHUNKS; ++c) {
             const int ci = t + c * G;
-            if (ci < nchunks && live) {
+            if (FULL ? live : (ci < nchunks && live)) {
                 chunk_t o;
 #pragma unroll
                 for (int e = 0; e < E; ++e) {
-                    float y = (v[c][e] - mean) * rstd * to_float(wv[c].v[e]);
-                    if (b != nullptr) y += to_float(bv[c].v[e]);
+                    float y;
+                    if (FULL) {
+                        y = fmaf(fmaf(v[c][e], rstd, shift), wf[c][e], bf[c][e]);
+                    } else {
+                        y = (v[c][e] - mean) * rstd * to_float(wv[c].v[e]);
+                        if (b != nullptr) y += to_float(bv[c].v[e]);
+                    }
                     o.v[e] = from_float<T>(y);
                 }
                 // Outputs too large to stay cached until their consumer runs are written with streaming stores
@@ -217,12 +240,21 @@ layernorm_strided_kernel(const T *__restrict__ x, const T *__restrict__ res, con
     }
 }
 
-template <typename T, int CHUNKS, int GROUP_WAVES, bool HALF = false>
+template <typename T, int CHUNKS, int GROUP_WAVES, bool HALF = false, bool FULL = false>
 static void launch_rows(bool rms, bool has_res, dim3 grid, hipStream_t st, const T *x, const T *res,
                         const T *w, const T *b, T *out, float *mean, float *rstd, int M, int N, int64_t x_rs,
                         int64_t res_rs, int64_t out_rs, float eps) {
+    // rows that fill every lane's chunks exactly take the form without bounds tests (single-wave groups of up to 4
+    // chunks: gamma and beta are kept as fp32 there)
+    if constexpr (!FULL && GROUP_WAVES == 1 && CHUNKS <= 4) {
+        if (N == CHUNKS * (HALF ? 32 : 64) * (int)(16 / sizeof(T))) {
+            launch_rows<T, CHUNKS, GROUP_WAVES, HALF, true>(rms, has_res, grid, st, x, res, w, b, out, mean, rstd, M, N, x_rs,
+                                                            res_rs, out_rs, eps);
+            return;
+        }
+    }
 #define KERNL_LN_LAUNCH(R, H)                                                                                       \
-    hipLaunchKernelGGL((layernorm_rows_kernel<T, CHUNKS, R, H, GROUP_WAVES, HALF>), grid, dim3(256), 0, st, x, res, w, b, \
+    hipLaunchKernelGGL((layernorm_rows_kernel<T, CHUNKS, R, H, GROUP_WAVES, HALF, FULL>), grid, dim3(256), 0, st, x, res, w, b, \
                        out, mean, rstd, M, N, x_rs, res_rs, out_rs, eps, stream_out)
     const int stream_out = (int64_t)M * N * (int64_t)sizeof(T) > (128ll << 20);
     if (rms) {
