@@ -83,6 +83,14 @@ __device__ __forceinline__ void mfma16_inplace(f16x8 a, f16x8 b, f32x4_acc &c) {
 __device__ __forceinline__ void mfma16_inplace(bf16x8 a, bf16x8 b, f32x4_acc &c) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
+// First product of an output tile: the accumulator is WRITTEN as a * b + 0 (the inline constant), so a tile never
+// zeroes its 256 accumulator registers.
+__device__ __forceinline__ void mfma16_start(f16x8 a, f16x8 b, f32x4_acc &c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma16_start(bf16x8 a, bf16x8 b, f32x4_acc &c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+}
 // To the compiler the instruction above is opaque text: it inserts none of the wait states that a read of a matrix
 // instruction's result needs (11 after an 8-pass instruction), so the copies out of the accumulation registers with
 // which an epilogue begins could follow the last MFMA directly and see registers that some lanes' results have not

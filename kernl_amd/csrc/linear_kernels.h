@@ -847,8 +847,9 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     // One k-tile held in stage CUR (a compile-time constant, so that stage offsets fold into instruction offsets).
     // `landed`: the loads of the next k-tile are known to have arrived (a wait for later loads has been passed), and
     // waiting for "everything outstanding" would only wait for the previous tile's output stores.
-    auto k_tile = [&](auto cur_c, bool landed) __attribute__((always_inline)) {
+    auto k_tile = [&](auto cur_c, bool landed, auto first_c) __attribute__((always_inline)) {
         constexpr int CUR = decltype(cur_c)::value;
+        constexpr bool FIRST = decltype(first_c)::value;  // the first k-tile of an output tile: its first k-step starts the sums
         const int k0 = load_kt * BK;
 #pragma unroll
         for (int st = 0; st < KSTEPS; ++st) {
@@ -862,7 +863,8 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 #pragma unroll
             for (int m = 0; m < NB * NBN; ++m) {
                 const int i = m / NBN, j = m % NBN;
-                mfma16_inplace(fa[st][j], fb[st][i], acc[i][j]);
+                if (FIRST && st == 0) mfma16_start(fa[st][j], fb[st][i], acc[i][j]);
+                else mfma16_inplace(fa[st][j], fb[st][i], acc[i][j]);
                 const int slot = m / PERIOD;
                 if (m % PERIOD == 0 && slot < NBN + NB) {
                     // the weight fragments first: the first MFMAs of the next k-step need all of them
@@ -886,20 +888,19 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     // Every output tile starts in stage 0: the host launches one workgroup per tile when the number of k-tiles is odd.
     bool landed = false;
     while (true) {
-#pragma unroll
-        for (int i = 0; i < NB; ++i)
-#pragma unroll
-            for (int j = 0; j < NBN; ++j) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
-        int kt = 0;
+        // (no zeroing of the accumulators: the first k-step of the tile writes them)
+        k_tile(IntC<0>(), landed, BoolC<true>());
+        advance_load();
+        landed = false;
+        int kt = 1;
         for (; kt + 1 < nk; kt += 2) {
-            k_tile(IntC<0>(), landed);
+            k_tile(IntC<1>(), false, BoolC<false>());
             advance_load();
-            landed = false;
-            k_tile(IntC<1>(), false);
+            k_tile(IntC<0>(), false, BoolC<false>());
             advance_load();
         }
         if (kt < nk) {
-            k_tile(IntC<0>(), landed);
+            k_tile(IntC<1>(), false, BoolC<false>());
             advance_load();
         }
         mfma16_inplace_results_landed(acc);
