@@ -88,21 +88,24 @@ struct MaskTileMap {
 };
 
 // ----------------------------------------------------------------------------------------------------
-// Wide linear kernel: which weight row (inside the tile) LDS row `row` of the weight tile carries.  LDS row `row` is
-// MFMA row r = row % 16 of 16-row block row / 16; the placement makes a lane end up with consecutive output columns:
-//   256 columns    in a 128-row group (the sub-tile of one wave), block j row r carries weight row 32 (r/4) + 4 j + r%4:
-//                  lane group g = lane / 16 holds the 32 columns 32 g .. 32 g + 31 across its eight blocks — 64
-//                  contiguous bytes of an output row, which a transposition inside each quad of lanes turns into
-//                  stores where four adjacent lanes cover those 64 bytes
-//   192 columns    32-row groups of two blocks: 8 (r/4) + 4 (j%2) + r%4 (8 consecutive columns per lane and group)
-//   gated          32 (j/2) + 8 (r/4) + 4 (j%2) + r%4: the lane holds gate AND value of the 8 output columns 8 g .. 8 g + 7
+// Wide linear kernels: which weight row (inside the tile) LDS row `row` of the weight tile carries.  LDS row `row` is
+// row r = row % 16 of 16-row block j of a wave's weight rows (128 per wave in 256-column tiles, 96 in 192-column tiles),
+// and lane l16 of the wave receives the results of row r = l16 of every block.  The placement gives that lane
+// consecutive output columns:
+//   plain    block j row r carries weight row NBN r + j of the wave's rows: lane l16 holds columns NBN l16 .. + NBN - 1
+//   gated    the fused weight holds 32 gate rows, then the 32 value rows of the same 32 output columns, and so on; blocks
+//            0 .. 3 carry the gate rows and blocks 4 .. 7 the value rows of output columns c = 4 r + j % 4 (of the wave's
+//            64): fused row 64 (c / 32) + 32 (j / 4) + c % 32
 // ----------------------------------------------------------------------------------------------------
 template <bool GATED, int NBN>
 KERNL_HD int wide_weight_row(int row) {
-    const int r = row & 15, j = (row >> 4) & 3;
-    if (GATED) return (row & ~63) + 32 * (j >> 1) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3);
-    if (NBN == 8) return (row & ~127) + 32 * (r >> 2) + 4 * ((row >> 4) & 7) + (r & 3);
-    return (row & ~31) + 8 * (r >> 2) + 4 * (j & 1) + (r & 3);
+    const int r = row & 15;
+    if (GATED) {
+        const int j = (row >> 4) & 7, c = 4 * r + (j & 3);
+        return (row & ~127) + 64 * (c >> 5) + 32 * (j >> 2) + (c & 31);
+    }
+    const int per_wave = 16 * NBN, first = (row / per_wave) * per_wave;
+    return first + NBN * r + ((row - first) >> 4);
 }
 
 // ----------------------------------------------------------------------------------------------------

@@ -399,244 +399,150 @@ linear_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 // consumed takes the next-but-one k-tile, one load every fourth MFMA.  (A burst of 16 loads followed by a wait for
 // all of them stalls a lone wave: 64 KB need >= 1024 cycles to pass the CU's 64 B/clk fill path.)
 //
-// Weight rows are placed in LDS so that a lane ends up with consecutive output columns: MFMA row r of block j of a
-// wave's 128 weight rows carries weight row 32 (r/4) + 4 j + r%4, so lane group g = lane/16 holds the 32 columns
-// 32 g .. 32 g+31 across its eight blocks (192-column tiles: 8 columns per lane and pair of blocks).  Gated epilogues use 32 (j/2) + 8 (r/4) + 4 (j%2) + r%4 instead: the lane holds
-// gate AND value of the 8 output columns 8 g .. 8 g + 7.
+// Weight rows are placed in LDS so that a lane ends up with consecutive output columns of a row (see WideLane below and
+// wide_weight_row): stores need no regrouping and 16 adjacent lanes cover a whole row of the wave's sub-tile.
 // ----------------------------------------------------------------------------------------------------
-template <typename T>
-__device__ __forceinline__ u32x4 fetch8(const T *__restrict__ p, int idx, int limit, int vec_ok) {
-    u32x4 r = {0, 0, 0, 0};
-    if (p == nullptr) return r;
-    if (vec_ok && idx + 8 <= limit) return *reinterpret_cast<const u32x4 *>(p + idx);
+// Lane geometry of the wide kernels' results.  The x fragment is the matrix instruction's A operand and the weight
+// fragment its B operand: element v of accumulator [i][j] in lane (l16 = lane % 16, g = lane / 16) is output row
+// 16 i + 4 g + v of the wave's sub-tile and the output column whose weight row sits in LDS row 16 j + l16 of the wave's
+// weight rows.  The placement of weight rows in LDS (wide_weight_row) makes those the lane's CONSECUTIVE columns:
+//   plain   LDS row 16 j + r carries weight row NBN r + j: lane l16 holds columns NBN l16 .. NBN l16 + NBN - 1 of each
+//           of its four rows — one 16-byte (256-column tiles) or 12-byte (192-column tiles) store per row, and the 16
+//           lanes of a group cover the 256 (192) contiguous bytes of the row: a store instruction writes four whole
+//           rows of the sub-tile
+//   gated   blocks 0 .. 3 carry the gate rows and blocks 4 .. 7 the value rows of output columns 4 l16 .. 4 l16 + 3 (of
+//           the wave's 64): one 8-byte store per row
+// With the operands the other way round (weights on the A side) adjacent lanes hold different ROWS and every 16-byte
+// store reaches memory as 64 separate pieces; regrouping the packed results so that adjacent lanes write contiguous
+// bytes (inside quads of lanes with DPP moves, or through LDS) cost 64 vector instructions per 16-row block or the LDS
+// bandwidth all four waves want at once.  Here the epilogue of a block is: read, add bias, activate, round, store.
+template <bool GATED, int NBN>
+struct WideLane {
+    static constexpr int NV = GATED ? 4 : NBN;  // output values per lane and row
+    // first output column of lane l16 in a wave whose weight rows start at fused row n_wave
+    static __device__ __forceinline__ int col(int n_wave, int l16) { return GATED ? (n_wave >> 1) + 4 * l16 : n_wave + NBN * l16; }
+};
+
+// The lane's bias entries, fetched as packed 16-bit values (`raw`: entry j of accumulator block j in half j % 2 of dword
+// j / 2; zeros without a bias and beyond N) and converted to fp32 once per output tile.  The fetch is issued in front of
+// a tile's main loop and the conversion after it, so that no wave waits for a memory round trip between its last
+// product and its epilogue.  `N` is the number of weight rows (gated: gate and value rows together; the fused weight
+// holds 32 gate rows, then the 32 value rows of the same output columns, and so on).
+template <typename T, bool GATED, int NBN>
+__device__ __forceinline__ void wide_bias_fetch(const T *__restrict__ bias, int n_wave, int l16, int N, int bias_vec_ok,
+                                                uint32_t (&raw)[NBN / 2]) {
 #pragma unroll
-    for (int v = 0; v < 8; v += 2) {
-        const uint32_t lo = idx + v < limit ? (uint32_t)__builtin_bit_cast(uint16_t, p[idx + v]) : 0u;
-        const uint32_t hi = idx + v + 1 < limit ? (uint32_t)__builtin_bit_cast(uint16_t, p[idx + v + 1]) : 0u;
-        r[v >> 1] = lo | (hi << 16);
+    for (int e = 0; e < NBN / 2; ++e) raw[e] = 0u;
+    if (bias == nullptr) return;
+    auto entry = [&](int row) __attribute__((always_inline)) -> uint32_t {
+        return row < N ? (uint32_t)__builtin_bit_cast(uint16_t, bias[row]) : 0u;
+    };
+    if constexpr (GATED) {
+        const int c = 4 * l16;                              // first of the lane's 4 output columns inside the wave's 64
+        const int row = n_wave + 64 * (c >> 5) + (c & 31);  // its gate row; the value row is 32 further
+        if (bias_vec_ok && row + 36 <= N) {
+            const u32x2 gt = *reinterpret_cast<const u32x2 *>(bias + row), vl = *reinterpret_cast<const u32x2 *>(bias + row + 32);
+            raw[0] = gt[0], raw[1] = gt[1], raw[2] = vl[0], raw[3] = vl[1];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                raw[e] = entry(row + 2 * e) | (entry(row + 2 * e + 1) << 16);
+                raw[2 + e] = entry(row + 32 + 2 * e) | (entry(row + 33 + 2 * e) << 16);
+            }
+        }
+    } else {
+        const int n = n_wave + NBN * l16;
+        if (bias_vec_ok && n + NBN <= N) {
+            if constexpr (NBN == 8) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(bias + n);
+                raw[0] = v[0], raw[1] = v[1], raw[2] = v[2], raw[3] = v[3];
+            } else {
+#pragma unroll
+                for (int e = 0; e < NBN / 2; ++e) raw[e] = reinterpret_cast<const uint32_t *>(bias + n)[e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < NBN / 2; ++e) raw[e] = entry(n + 2 * e) | (entry(n + 2 * e + 1) << 16);
+        }
     }
-    return r;
+}
+template <typename T, int NBN>
+__device__ __forceinline__ void wide_bias_unpack(const uint32_t (&raw)[NBN / 2], float (&bf)[NBN]) {
+#pragma unroll
+    for (int j = 0; j < NBN; ++j) bf[j] = to_float(__builtin_bit_cast(T, (uint16_t)(raw[j >> 1] >> (16 * (j & 1)))));
 }
 
-// Epilogue of m-block IB (16 rows) of a wave of the wide kernel.  Lane (l16, g) holds row m_wave + 16 IB + l16 and
-//   256-column tiles: the 32 consecutive columns 32 g .. 32 g + 31 of the wave's 128 (group G = blocks 4 G .. 4 G + 3:
-//                     columns 32 g + 16 G .. + 15),
-//   192-column tiles: in every 32-column group G (two blocks) the 8 consecutive columns 32 G + 8 g .. + 7.
-// Adjacent lanes hold DIFFERENT ROWS, so a 16-byte store per lane reaches memory as 64 separate 16-byte pieces.  Interior
-// blocks of 256-column tiles therefore transpose inside every quad of lanes first (two butterfly steps of
-// quad-permuting DPP moves and selects on the packed 16-bit results): afterwards lane i of a quad holds 16-byte chunk i
-// of each of the quad's four rows, and every store instruction has four adjacent lanes covering 64 contiguous bytes.
-// Measured on 16384 x 3072 x 768 without activation: 78 -> 72 us; covering whole 256-byte rows with 16 adjacent lanes
-// (through LDS) measured no better than the 64-byte form and costs LDS bandwidth that all four waves want at once.
-template <int NBN>
-__device__ __forceinline__ int wide_lane_col(int G, int g) {
-    return NBN == 8 ? 32 * g + 16 * G : 32 * G + 8 * g;
-}
-// quad_perm DPP move of every dword of a 16-byte value
-template <int CTRL>
-__device__ __forceinline__ u32x4 quad_perm4(u32x4 v) {
-    u32x4 r;
+// NV rounded values of one row -> one 16-, 12- or 8-byte store
+template <typename T, int NV>
+__device__ __forceinline__ void wide_store_row(T *p, const float (&r)[NV]) {
+    static_assert(NV == 8 || NV == 6 || NV == 4, "values per lane and row");
+    uint32_t w[NV / 2];
 #pragma unroll
-    for (int d = 0; d < 4; ++d) r[d] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v[d], CTRL, 0xF, 0xF, true);
-    return r;
-}
-// 4 x 4 transposition inside every quad of lanes: on entry lane i holds P[c] = chunk c of ITS row, on return P[k] =
-// chunk i of the row of the quad's lane k.
-__device__ __forceinline__ void quad_transpose4(u32x4 (&P)[4], int lane_in_quad) {
-    const bool odd = (lane_in_quad & 1) != 0, upper = (lane_in_quad & 2) != 0;
-    u32x4 A[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const u32x4 other = quad_perm4<0xB1>(P[c ^ 1]);  // quad_perm [1,0,3,2]: the neighbour's other chunk of the pair
-        const bool keep = ((c & 1) != 0) == odd;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) A[c][d] = keep ? P[c][d] : other[d];
-    }
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const u32x4 other = quad_perm4<0x4E>(A[c ^ 2]);  // quad_perm [2,3,0,1]
-        const bool keep = ((c & 2) != 0) == upper;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) P[c][d] = keep ? A[c][d] : other[d];
-    }
+    for (int e = 0; e < NV / 2; ++e) w[e] = pack2<T>(r[2 * e], r[2 * e + 1]);
+    if constexpr (NV == 8) *reinterpret_cast<u32x4 *>(p) = u32x4{w[0], w[1], w[2], w[3]};
+    else if constexpr (NV == 6) *reinterpret_cast<u32x3 *>(p) = u32x3{w[0], w[1], w[2]};
+    else *reinterpret_cast<u32x2 *>(p) = u32x2{w[0], w[1]};
 }
 
-// Row-padded LDS layout of the 192-column tiles' store transposition (see wide_epilogue_transposed): 16 rows of 192
-// bytes, 208 bytes apart
-template <int NBN>
-__device__ __forceinline__ int xpose_offset(int row, int chunk) {
-    static_assert(NBN == 6, "only the 192-column tiles transpose through LDS");
-    return row * 208 + (chunk << 4);
-}
-
+// Epilogue of m-block IB (16 rows) of a wave of the wide kernels.  Blocks that lie inside the matrix, with contiguous
+// 16-byte aligned output rows and no pre-activation side output, run a straight-line path.
 template <typename T, int ACT, int IB, int NBN, int NBM = 8>
 __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_wave, int n_wave, int l16, int g,
                                               T *__restrict__ out, T *__restrict__ act_in, int M, int N,
                                               int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs,
-                                              int out_vec_ok, int ai_vec_ok,
-                                              const u32x4 (&braw)[NBN == 8 ? 2 : 3][2]) {
-    const int m = m_wave + 16 * IB + l16;
-    const bool rows_inside = m_wave + 16 * IB + 16 <= M;
-    if constexpr ((ACT & kGluBit) != 0) {
-        static_assert(NBN == 8, "gated epilogues pair blocks inside 64-row groups");
-        constexpr int BASE = ACT & (kGluBit - 1);
-        const int n_total = N >> 1;
-        const bool interior = rows_inside && (n_wave >> 1) + 64 <= n_total && out_vec_ok;
-        const bool fast = __builtin_amdgcn_readfirstlane((int)interior) != 0;
+                                              int out_vec_ok, int ai_vec_ok, const float (&bf)[NBN]) {
+    constexpr bool GATED = (ACT & kGluBit) != 0;
+    static_assert(!GATED || NBN == 8, "gated epilogues: four gate and four value blocks");
+    constexpr int BASE = ACT & (kGluBit - 1), NV = WideLane<GATED, NBN>::NV;
+    const int n = WideLane<GATED, NBN>::col(n_wave, l16);
+    const int n_total = GATED ? N >> 1 : N;  // output columns
+    const int m_first = m_wave + 16 * IB + 4 * g;
+    // pre-activation values of row 4 g + v (gated: the gate; `value` then holds what it is multiplied with)
+    auto sums = [&](int v, float (&r)[NV], float (&value)[NV]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int G = 0; G < 2; ++G) {
-            const int n = (n_wave >> 1) + 32 * G + 8 * g;  // 8 consecutive output columns
-            if (!fast && (m >= M || n >= n_total)) continue;  // n_total is a multiple of 32 and n of 8
-            float r[8];
-#pragma unroll
-            for (int v = 0; v < 8; ++v) {
-                const float gate = acc[IB][4 * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v);
-                const float value = acc[IB][4 * G + 2 + (v >> 2)][v & 3] + bias_elem<T>(braw[G], 8 + v);
-                r[v] = apply_act16(gate, BASE) * value;
-            }
-            if (fast || out_vec_ok) {
-                u32x4 p;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) p[v] = pack2<T>(r[2 * v], r[2 * v + 1]);
-                *reinterpret_cast<u32x4 *>(out + (int64_t)m * out_rs + n) = p;
-            } else {
-#pragma unroll
-                for (int v = 0; v < 8; ++v) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
-            }
-        }
-        return;
-    }
-    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB, VPG = 4 * JB;  // blocks per group, groups, values per lane and group
-    auto store_vec = [&](T *p, const float (&r)[VPG]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int h = 0; h < VPG / 8; ++h) {
-            u32x4 pk;
-#pragma unroll
-            for (int v = 0; v < 4; ++v) pk[v] = pack2<T>(r[8 * h + 2 * v], r[8 * h + 2 * v + 1]);
-            *reinterpret_cast<u32x4 *>(p + 8 * h) = pk;
+        for (int c = 0; c < NV; ++c) {
+            r[c] = acc[IB][c][v] + bf[c];
+            value[c] = GATED ? acc[IB][(4 + c) % NBN][v] + bf[(4 + c) % NBN] : 1.0f;
         }
     };
-    const bool interior = rows_inside && n_wave + NBN * 16 <= N && out_vec_ok && act_in == nullptr;
+    const bool interior = m_wave + 16 * IB + 16 <= M && (GATED ? (n_wave >> 1) + 64 <= n_total : n_wave + NBN * 16 <= N) &&
+                          out_vec_ok && (GATED || act_in == nullptr);
     if (__builtin_amdgcn_readfirstlane((int)interior)) {
-        if constexpr (NBN == 8) {
-            u32x4 P[4];  // chunk c = 2 G + h: columns 32 g + 8 c .. + 7 of this lane's row
+        T *p = out + (int64_t)m_first * out_rs + n;
 #pragma unroll
-            for (int G = 0; G < NG; ++G) {
-                float r[VPG];
+        for (int v = 0; v < 4; ++v) {
+            float r[NV], value[NV];
+            sums(v, r, value);
 #pragma unroll
-                for (int v = 0; v < VPG; ++v) r[v] = apply_act16(acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v), ACT);
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) P[2 * G + h][v] = pack2<T>(r[8 * h + 2 * v], r[8 * h + 2 * v + 1]);
-            }
-            quad_transpose4(P, l16 & 3);
-            T *p = out + (int64_t)(m_wave + 16 * IB + (l16 & ~3)) * out_rs + n_wave + 32 * g + 8 * (l16 & 3);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) *reinterpret_cast<u32x4 *>(p + k * out_rs) = P[k];
-            return;
-        }
-#pragma unroll
-        for (int G = 0; G < NG; ++G) {
-            float r[VPG];
-#pragma unroll
-            for (int v = 0; v < VPG; ++v) r[v] = apply_act16(acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v), ACT);
-            store_vec(out + (int64_t)m * out_rs + n_wave + wide_lane_col<NBN>(G, g), r);
+            for (int c = 0; c < NV; ++c) r[c] = GATED ? apply_act16(r[c], BASE) * value[c] : apply_act16(r[c], ACT);
+            wide_store_row<T, NV>(p + v * out_rs, r);
         }
         return;
     }
 #pragma unroll
-    for (int G = 0; G < NG; ++G) {
-        const int n = n_wave + wide_lane_col<NBN>(G, g);
-        if (m >= M || n >= N) continue;
-        float r[VPG];
-#pragma unroll
-        for (int v = 0; v < VPG; ++v) r[v] = acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v);
-        if (act_in != nullptr) {
-            if (ai_vec_ok && n + VPG <= N) {
-                store_vec(act_in + (int64_t)m * ai_rs + n, r);
+    for (int v = 0; v < 4; ++v) {
+        const int m = m_first + v;
+        if (m >= M || n >= n_total) continue;
+        float r[NV], value[NV];
+        sums(v, r, value);
+        if (!GATED && act_in != nullptr) {
+            if (ai_vec_ok && n + NV <= n_total) {
+                wide_store_row<T, NV>(act_in + (int64_t)m * ai_rs + n, r);
             } else {
 #pragma unroll
-                for (int v = 0; v < VPG; ++v)
-                    if (n + v < N) act_in[(int64_t)m * ai_rs + (int64_t)(n + v) * ai_cs] = from_float<T>(r[v]);
+                for (int c = 0; c < NV; ++c)
+                    if (n + c < n_total) act_in[(int64_t)m * ai_rs + (int64_t)(n + c) * ai_cs] = from_float<T>(r[c]);
             }
         }
 #pragma unroll
-        for (int v = 0; v < VPG; ++v) r[v] = apply_act16(r[v], ACT);
-        if (out_vec_ok && n + VPG <= N) {
-            store_vec(out + (int64_t)m * out_rs + n, r);
+        for (int c = 0; c < NV; ++c) r[c] = GATED ? apply_act16(r[c], BASE) * value[c] : apply_act16(r[c], ACT);
+        if (out_vec_ok && n + NV <= n_total) {
+            wide_store_row<T, NV>(out + (int64_t)m * out_rs + n, r);
         } else {
 #pragma unroll
-            for (int v = 0; v < VPG; ++v)
-                if (n + v < N) out[(int64_t)m * out_rs + (int64_t)(n + v) * out_cs] = from_float<T>(r[v]);
+            for (int c = 0; c < NV; ++c)
+                if (n + c < n_total) out[(int64_t)m * out_rs + (int64_t)(n + c) * out_cs] = from_float<T>(r[c]);
         }
-    }
-}
-
-// 192-column tiles: the whole epilogue of a wave whose sub-tile lies inside the matrix (plain activations, 16-byte
-// aligned contiguous output rows, no pre-activation side output).  A lane holds only 16 contiguous bytes of a row per
-// 32-column group here, so the transposition inside a quad of lanes that the 256-column tiles use has nothing to join;
-// the packed results go through a 4 KB LDS region of the wave's own instead (rows padded to 208 bytes: no bank
-// conflicts), and come back so that 12 adjacent lanes cover the 192 contiguous bytes of a row.  Only the wave itself
-// touches its region and LDS operations of one wave execute in program order: no barrier.  Software-pipelined by hand
-// over the 16-row blocks, because with one wave per SIMD nothing else hides the LDS round trip:
-//   values of block b (bias, activation, rounding)  ->  global stores of block b - 1 (its LDS reads were issued before
-//   those values were computed)  ->  LDS writes of block b  ->  LDS reads of block b.
-// Measured, graph replay: 16384 x 2304 x 768 60.3 -> 58.2 us, 16384 x 768 x 768 23.7 -> 23.0, 16384 x 768 x 3072 65.2 ->
-// 64.6 (direct stores with runs of 48 bytes per quad, the best a transposition inside quads can do here: 59.0 / 23.4 /
-// 65.0).
-template <typename T, int ACT, int NBN, int NBM>
-__device__ __forceinline__ void wide_epilogue_transposed(f32x4_acc (&acc)[NBM][NBN], int m_wave, int n_wave, int l16, int g,
-                                                         T *__restrict__ out, int64_t out_rs,
-                                                         const u32x4 (&braw)[NBN == 8 ? 2 : 3][2], unsigned char *xpose) {
-    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB, VPG = 4 * JB;
-    constexpr int CPR = NBN * 2, NK = CPR / 4;  // 16-byte chunks per row of the sub-tile; stores per lane and block
-    const int lane = 16 * g + l16;
-    int rd_off[NK];
-    int64_t st_off[NK];
-#pragma unroll
-    for (int k = 0; k < NK; ++k) {
-        const int idx = k * 64 + lane, row = idx / CPR, chunk = idx % CPR;
-        rd_off[k] = xpose_offset<NBN>(row, chunk);
-        st_off[k] = (int64_t)row * out_rs + 8 * chunk;
-    }
-    int wr_off[NG][VPG / 8];
-#pragma unroll
-    for (int G = 0; G < NG; ++G)
-#pragma unroll
-        for (int h = 0; h < VPG / 8; ++h) wr_off[G][h] = xpose_offset<NBN>(l16, 2 * JB * G + (VPG / 8) * g + h);
-    T *base = out + (int64_t)m_wave * out_rs + n_wave;
-    u32x4 rd[NK];
-#pragma unroll
-    for (int IB = 0; IB <= NBM; ++IB) {
-        u32x4 pk[NG][VPG / 8];
-        if (IB < NBM) {
-#pragma unroll
-            for (int G = 0; G < NG; ++G) {
-                float r[VPG];
-#pragma unroll
-                for (int v = 0; v < VPG; ++v) r[v] = apply_act16(acc[IB][JB * G + (v >> 2)][v & 3] + bias_elem<T>(braw[G], v), ACT);
-#pragma unroll
-                for (int h = 0; h < VPG / 8; ++h)
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) pk[G][h][v] = pack2<T>(r[8 * h + 2 * v], r[8 * h + 2 * v + 1]);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (IB > 0) {
-#pragma unroll
-            for (int k = 0; k < NK; ++k) *reinterpret_cast<u32x4 *>(base + (int64_t)(16 * (IB - 1)) * out_rs + st_off[k]) = rd[k];
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (IB < NBM) {
-#pragma unroll
-            for (int G = 0; G < NG; ++G)
-#pragma unroll
-                for (int h = 0; h < VPG / 8; ++h) *reinterpret_cast<u32x4 *>(xpose + wr_off[G][h]) = pk[G][h];
-#pragma unroll
-            for (int k = 0; k < NK; ++k) rd[k] = *reinterpret_cast<const u32x4 *>(xpose + rd_off[k]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -863,8 +769,9 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
 #pragma unroll
             for (int m = 0; m < NB * NBN; ++m) {
                 const int i = m / NBN, j = m % NBN;
-                if (FIRST && st == 0) mfma16_start(fa[st][j], fb[st][i], acc[i][j]);
-                else mfma16_inplace(fa[st][j], fb[st][i], acc[i][j]);
+                // x on the A side: rows of the result are rows of x
+                if (FIRST && st == 0) mfma16_start(fb[st][i], fa[st][j], acc[i][j]);
+                else mfma16_inplace(fb[st][i], fa[st][j], acc[i][j]);
                 const int slot = m / PERIOD;
                 if (m % PERIOD == 0 && slot < NBN + NB) {
                     // the weight fragments first: the first MFMAs of the next k-step need all of them
@@ -888,6 +795,10 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
     // Every output tile starts in stage 0: the host launches one workgroup per tile when the number of k-tiles is odd.
     bool landed = false;
     while (true) {
+        // the tile's bias entries travel under its main loop
+        const int n_wave = n0 + wave_n * (NBN * 16);
+        uint32_t braw[NBN / 2];
+        wide_bias_fetch<T, GATED, NBN>(bias, n_wave, l16, N, bias_vec_ok, braw);
         // (no zeroing of the accumulators: the first k-step of the tile writes them)
         k_tile(IntC<0>(), landed, BoolC<true>());
         advance_load();
@@ -905,42 +816,25 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         }
         mfma16_inplace_results_landed(acc);
 
-        // all bias entries of the lane's columns in one go: one memory round trip per tile.  Its wait also covers the
-        // loads of the next k-tile, which were issued earlier.
-        const int n_wave = n0 + wave_n * (NBN * 16);
-        constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB;  // n-blocks per lane-contiguous group, groups per wave
-        u32x4 braw[NG][2];
-#pragma unroll
-        for (int G = 0; G < NG; ++G)
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-                braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0}
-                             : fetch8<T>(bias, n_wave + (GATED ? 64 * G + 32 * h + 8 * g : wide_lane_col<NBN>(G, g) + 8 * h), N, bias_vec_ok);
+        // the loads of the next k-tile were issued earlier: after this wait they are known to have landed
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         landed = true;
+        float bf[NBN];
+        wide_bias_unpack<T, NBN>(braw, bf);
         // one call per 16-row block: each stays small enough for the compiler to unroll completely, so the
         // accumulators are only ever indexed by constants and never leave the register file
-        bool whole_inside = false;
-        if constexpr (!GATED && NBN == 6)
-            whole_inside = m0 + wave_m * 128 + 128 <= M && n_wave + NBN * 16 <= N && out_vec_ok && act_in == nullptr;
-        if (__builtin_amdgcn_readfirstlane((int)whole_inside)) {
-            if constexpr (!GATED && NBN == 6)
-                wide_epilogue_transposed<T, ACT, NBN, 8>(acc, m0 + wave_m * 128, n_wave, l16, g, out, out_rs, braw,
-                                                         smem + 2 * (X_BYTES + W_BYTES) + wave * 4096);
-        } else {
 #define KERNL_WIDE_EPILOGUE(I)                                                                                         \
     wide_epilogue<T, ACT, I, NBN>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs, ai_cs,   \
-                             out_vec_ok, ai_vec_ok, braw)
-            KERNL_WIDE_EPILOGUE(0);
-            KERNL_WIDE_EPILOGUE(1);
-            KERNL_WIDE_EPILOGUE(2);
-            KERNL_WIDE_EPILOGUE(3);
-            KERNL_WIDE_EPILOGUE(4);
-            KERNL_WIDE_EPILOGUE(5);
-            KERNL_WIDE_EPILOGUE(6);
-            KERNL_WIDE_EPILOGUE(7);
+                             out_vec_ok, ai_vec_ok, bf)
+        KERNL_WIDE_EPILOGUE(0);
+        KERNL_WIDE_EPILOGUE(1);
+        KERNL_WIDE_EPILOGUE(2);
+        KERNL_WIDE_EPILOGUE(3);
+        KERNL_WIDE_EPILOGUE(4);
+        KERNL_WIDE_EPILOGUE(5);
+        KERNL_WIDE_EPILOGUE(6);
+        KERNL_WIDE_EPILOGUE(7);
 #undef KERNL_WIDE_EPILOGUE
-        }
         idx += slots;
         if (!tile_origin(idx, m0, n0)) break;
     }
@@ -1152,7 +1046,7 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
 #pragma unroll
             for (int m = 0; m < NBM * NBN; ++m) {
                 const int i = m / NBN, j = m % NBN;
-                mfma16_inplace(fa[st][j], fb[st][i], acc[i][j]);
+                mfma16_inplace(fb[st][i], fa[st][j], acc[i][j]);  // x on the A side
                 const int slot = m >> 1;
                 if ((m & 1) == 0 && slot < NBN + NBM) {
                     if (st == 0) {
@@ -1200,24 +1094,13 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
         return;
     }
     const int n_wave = n0 + wave_n * (NBN * 16);
-    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB;
-    u32x4 braw[NG][2];
-#pragma unroll
-    for (int G = 0; G < NG; ++G)
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-            braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0} : fetch8<T>(bias, n_wave + wide_lane_col<NBN>(G, g) + 8 * h, N, bias_vec_ok);
-    if constexpr (NBN == 6) {
-        const bool whole_inside = m0 + wave_m * (NBM * 16) + NBM * 16 <= M && n_wave + NBN * 16 <= N && out_vec_ok && act_in == nullptr;
-        if (__builtin_amdgcn_readfirstlane((int)whole_inside)) {
-            wide_epilogue_transposed<T, ACT, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, out_rs, braw,
-                                                       smem + 3 * 16384 + 3 * 32768 + wave * 4096);
-            return;
-        }
-    }
+    uint32_t braw[NBN / 2];
+    float bf[NBN];
+    wide_bias_fetch<T, false, NBN>(bias, n_wave, l16, N, bias_vec_ok, braw);
+    wide_bias_unpack<T, NBN>(braw, bf);
 #define KERNL_HALF_EPILOGUE(I)                                                                                         \
     wide_epilogue<T, ACT, I, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, \
-                                       ai_rs, ai_cs, out_vec_ok, ai_vec_ok, braw)
+                                       ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bf)
     KERNL_HALF_EPILOGUE(0);
     KERNL_HALF_EPILOGUE(1);
     KERNL_HALF_EPILOGUE(2);
@@ -1264,17 +1147,14 @@ linear_wide_half_reduce_kernel(const float *__restrict__ part, const T *__restri
         }
     }
     const int n_wave = n0 + wave_n * (NBN * 16);
-    constexpr int JB = NBN == 8 ? 4 : 2, NG = NBN / JB;
-    u32x4 braw[NG][2];
-#pragma unroll
-    for (int G = 0; G < NG; ++G)
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-            braw[G][h] = (JB == 2 && h == 1) ? u32x4{0, 0, 0, 0} : fetch8<T>(bias, n_wave + wide_lane_col<NBN>(G, g) + 8 * h, N, bias_vec_ok);
+    uint32_t braw[NBN / 2];
+    float bf[NBN];
+    wide_bias_fetch<T, false, NBN>(bias, n_wave, l16, N, bias_vec_ok, braw);
+    wide_bias_unpack<T, NBN>(braw, bf);
 #define KERNL_HALF_REDUCE_EPILOGUE(IB)                                                                                   \
     if (I == IB)                                                                                                         \
     wide_epilogue<T, ACT, IB, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, \
-                                        ai_rs, ai_cs, out_vec_ok, ai_vec_ok, braw)
+                                        ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bf)
     KERNL_HALF_REDUCE_EPILOGUE(0);
     KERNL_HALF_REDUCE_EPILOGUE(1);
     KERNL_HALF_REDUCE_EPILOGUE(2);
@@ -1699,7 +1579,7 @@ static void launch_mfma_glu(const LinearArgs &a) {
 template <typename T, int ACT, int NBN = 8, bool W8 = false>
 static void launch_wide_act(const LinearArgs &a) {
     auto kern = linear_wide_kernel<T, ACT, NBN, W8>;
-    constexpr int LDS_BYTES = 2 * (256 + 256) * 128 + (NBN == 6 ? 4 * 4096 : 0);  // two stages (+ a 4 KB store-transposition region per wave)
+    constexpr int LDS_BYTES = 2 * (256 + 256) * 128;  // two stages
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
@@ -1727,7 +1607,7 @@ static void launch_wide_half_act(const LinearArgs &a);
 template <typename T, int ACT, int NBN, bool W8 = false>
 static void launch_wide_half_act(const LinearArgs &a) {
     auto kern = linear_wide_half_kernel<T, ACT, NBN, W8>;
-    constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768 + (NBN == 6 ? 4 * 4096 : 0);  // three stages (+ a 4 KB store-transposition region per wave: all 160 KB)
+    constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768;  // three stages
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);

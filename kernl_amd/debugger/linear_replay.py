@@ -1,50 +1,47 @@
-"""Checks of the wide linear kernel's weight placement (csrc/linear_kernels.h; `wide_weight_row` in csrc/index_math.h): LDS row `row` of a weight
-tile feeds MFMA row row % 16 of 16-row block row / 16, and carries a weight row chosen so that the four-element
-results of a lane line up as consecutive output columns."""
+"""Checks of the wide linear kernels' weight placement (csrc/linear_kernels.h; `wide_weight_row` in csrc/index_math.h).
+
+The x fragment is the matrix instruction's A operand and the weight fragment its B operand, so lane l of a wave receives
+column l % 16 of every 16 x 16 result block: the output column whose weight row sits in LDS row 16 j + l % 16 of the
+wave's weight rows (block j).  The placement picks that weight row so that the lane's blocks line up as consecutive
+output columns of one row."""
 from typing import Dict, List
 
 from kernl_amd.debugger.index_lib import index_lib
 from kernl_amd.debugger.wave_ops import mfma16_result_position
 
+ROWS_PER_WAVE = {"256": 128, "192": 96, "gated": 128}
+
 
 def lane_columns(layout: str, tile_rows: int) -> Dict[int, List[List[int]]]:
-    """For every lane group g = lane / 16: the weight rows (= output columns inside the tile) its accumulators hold,
-    one list per lane-contiguous group of blocks, in register order (block by block, element by element)."""
+    """For every lane l16 = 0 .. 15: the weight rows (= columns inside the tile; gated: rows of the fused weight) its
+    accumulators hold, one list per wave of the tile's column split, in block order."""
     ix = index_lib()
-    blocks_per_group = 2 if layout == "192" else 4
+    per_wave = ROWS_PER_WAVE[layout]
     out: Dict[int, List[List[int]]] = {}
-    for g in range(4):
-        lane = 16 * g
-        groups = []
-        for first in range(0, tile_rows // 16, blocks_per_group):
-            cols = []
-            for j in range(first, first + blocks_per_group):
-                for e in range(4):
-                    r, _ = mfma16_result_position(lane, e)       # MFMA row inside block j
-                    cols.append(ix.wide_weight_row(layout, 16 * j + r))
-            groups.append(cols)
-        out[g] = groups
+    for l16 in range(16):
+        _, col = mfma16_result_position(l16, 0)   # column of the result block = row of the B operand = LDS row in block
+        out[l16] = [[ix.wide_weight_row(layout, first + 16 * j + col) for j in range(per_wave // 16)]
+                    for first in range(0, tile_rows, per_wave)]
     return out
 
 
 def check_weight_placement(layout: str) -> None:
     ix = index_lib()
     tile_rows = 192 if layout == "192" else 256
+    per_wave = ROWS_PER_WAVE[layout]
     rows = [ix.wide_weight_row(layout, r) for r in range(tile_rows)]
     if sorted(rows) != list(range(tile_rows)):
         raise AssertionError(f"{layout}: the placement is not a permutation of the tile's weight rows")
-    for g, groups in lane_columns(layout, tile_rows).items():
-        for cols in groups:
+    for l16, waves in lane_columns(layout, tile_rows).items():
+        for w, cols in enumerate(waves):
             if layout == "gated":
-                # gate columns 8 g' .. + 7 and the value columns 32 further on, g' within the 64-row group
-                gate, value = cols[0:4] + cols[4:8], cols[8:12] + cols[12:16]
-                if gate != list(range(gate[0], gate[0] + 8)) or value != [c + 32 for c in gate] or gate[0] % 8 != 0:
-                    raise AssertionError(f"gated: lane group {g} holds {cols}, not 8 gate columns and their value columns")
-            elif cols != list(range(cols[0], cols[0] + len(cols))) or cols[0] % len(cols) != 0:
-                raise AssertionError(f"{layout}: lane group {g} holds {cols}, not consecutive output columns")
-        if layout == "256":
-            # the two groups of a wave's eight blocks follow each other: 32 consecutive columns, 64-byte aligned
-            for first in range(0, len(groups), 2):
-                both = groups[first] + groups[first + 1]
-                if both != list(range(both[0], both[0] + 32)) or both[0] % 32 != 0:
-                    raise AssertionError(f"256: lane group {g} holds {both}, not 32 consecutive output columns")
+                # output columns c .. c + 3 of the wave's 64, c = 4 l16: their gate rows (32 gate rows, then the 32 value
+                # rows of the same columns, and so on), then their value rows 32 further on
+                c = 4 * l16
+                gate = [per_wave * w + 64 * (c // 32) + c % 32 + e for e in range(4)]
+                if cols != gate + [r + 32 for r in gate]:
+                    raise AssertionError(f"gated: lane {l16} holds {cols}, not 4 gate rows and their value rows")
+            else:
+                n = per_wave // 16
+                if cols != list(range(per_wave * w + n * l16, per_wave * w + n * l16 + n)):
+                    raise AssertionError(f"{layout}: lane {l16} holds {cols}, not {n} consecutive output columns")

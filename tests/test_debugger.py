@@ -105,13 +105,13 @@ def test_wide_linear_weight_placement(layout):
     check_weight_placement(layout)
     cols = lane_columns(layout, 192 if layout == "192" else 256)
     if layout == "256":
-        # lane group g: columns 32 g .. 32 g + 31 of each wave's 128 (64 contiguous bytes of an output row), eight blocks
-        assert cols[0][0] + cols[0][1] == list(range(32)) and cols[3][0] + cols[3][1] == list(range(96, 128))
-        assert cols[1][2] + cols[1][3] == list(range(160, 192))
+        # lane l16: columns 8 l16 .. 8 l16 + 7 of each wave's 128 — 16 lanes cover the 256 contiguous bytes of a row
+        assert cols[0] == [list(range(8)), list(range(128, 136))] and cols[15][1] == list(range(248, 256))
     if layout == "192":
-        assert cols[0][0] == list(range(8)) and cols[2][1] == list(range(48, 56))
+        assert cols[0] == [list(range(6)), list(range(96, 102))] and cols[3][0] == list(range(18, 24))
     if layout == "gated":
-        assert cols[1][0] == [8, 9, 10, 11, 12, 13, 14, 15, 40, 41, 42, 43, 44, 45, 46, 47]
+        # lane 9: output columns 36 .. 39 of the wave's 64 = second 32-column group: gate rows 64 + 4 .., value rows 96 + 4 ..
+        assert cols[9][0] == [68, 69, 70, 71, 100, 101, 102, 103]
 
 
 def test_index_functions_known_values():
