@@ -301,8 +301,9 @@ def main():
         "--cold-probe",
         action="store_true",
         help="launch attention (config 1), both config-2 linears, LayerNorm and a copy of the LayerNorm bytes 20 times "
-        "each, every launch after a 256 MB cache flush, and exit: the workload of the rocprofv3 --kernel-trace run "
-        "behind the *_cold_us figures (profiles/bench_cold_kernel_trace.txt)",
+        "each after the cache flush that rewrites 256 MB and 20 times each after the one that reads 512 MB of zeros, and "
+        "exit: the workload of the rocprofv3 --kernel-trace run behind the *_cold_us and *_cold_clean_us figures "
+        "(profiles/bench_cold_kernel_trace.txt)",
     )
     ap.add_argument(
         "--decode-probe",
