@@ -241,6 +241,25 @@ int kernl_linear_rms_fwd(const void *x, const void *rms_weight, float eps, const
                          int activation, int gated, int dtype, void *stream);
 
 /*
+ * The linear layer behind an RMSNorm for MANY rows (a prompt), with the norm folded away:
+ *     rmsnorm(x) @ w^T  =  rstd[m] * (x @ (w * norm_weight)^T),   rstd[m] = 1 / sqrt(mean(x[m]^2) + eps)
+ * so the caller multiplies the norm's weight into the columns of w once, obtains rstd from whoever produced x
+ * (kernl_add_rms_stats_fwd below) and this entry point computes
+ *     out = (x @ w^T) * row_scale[:, None] + bias                                    plain:  activation KERNL_ACT_NONE
+ *     out = silu(y_gate * row_scale + b_gate) * (y_value * row_scale + b_value)      gated != 0, activation KERNL_ACT_SILU:
+ *                                                                                     w [2N, K], bias [2N] interleaved as
+ *                                                                                     for kernl_linear_glu_fwd
+ * in the epilogue of the wide tile kernels: the normalised tensor is never written or read.  Replaces, for prompts, what
+ * the reference's `rms_matmul_rbe` (experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:116-183) and `ff_llama`
+ * (fused_kernel_ff.py:10-79) do for decoding steps — normalise inside the product — where those kernels re-compute the
+ * row statistics in every program.  row_scale: fp32 [M], 16-byte aligned.  f16 / bf16, K % 8 == 0, x with unit feature
+ * stride and 16-byte aligned rows; other activations return KERNL_ERR_UNSUPPORTED.
+ */
+int kernl_linear_scaled_fwd(const void *x, const void *w, const void *bias, const float *row_scale, void *out, int64_t M,
+                            int64_t N, int64_t K, const int64_t x_strides[2], const int64_t out_strides[2],
+                            int activation, int gated, int dtype, void *stream);
+
+/*
  * Whether kernl_linear_fwd runs M x N x K (16-bit, plain epilogue, x with unit feature stride) on one of its
  * small-problem kernels, and which: 0 = no; otherwise the kernl_linear_force_tile value of the kernel (10 .. 15).  A
  * caller that would otherwise route such a shape to the stream-K or split-K entry points (kernl_linear_fewrow_fwd,
@@ -377,6 +396,18 @@ int kernl_add_layernorm_fwd(const void *x, const void *residual, const void *w, 
                             int64_t x_row_stride, int64_t x_col_stride, int64_t res_row_stride,
                             int64_t res_col_stride, int64_t out_row_stride, int64_t out_col_stride,
                             float eps, int is_rms, int dtype, void *stream);
+
+/*
+ * sum = a + b, rounded to the tensors' dtype, and rstd[m] = 1 / sqrt(mean(sum[m]^2) + eps) of the ROUNDED sum — the
+ * residual addition of a decoder layer together with the row statistics of the RMSNorm that follows it
+ * (kernl_linear_scaled_fwd takes them).  b == NULL (then sum is not written): the statistics of `a` alone.  a, b, sum
+ * [M, N] with unit feature stride, 16-byte aligned rows, N % 8 == 0, f16 / bf16; rstd fp32 [M].  No counterpart in the
+ * reference, whose model adds in eager PyTorch (experimental/llama-v2/llama/model.py:262-264) and normalises inside its
+ * projection kernels.
+ */
+int kernl_add_rms_stats_fwd(const void *a, const void *b, void *sum, float *rstd, int64_t M, int64_t N,
+                            int64_t a_row_stride, int64_t b_row_stride, int64_t sum_row_stride, float eps, int dtype,
+                            void *stream);
 
 /* The process-wide test and tuning hooks are not part of this interface: they are declared in kernl_hip_test.h. */
 

@@ -35,6 +35,7 @@ EXPORTED_SYMBOLS = (
     "kernl_linear_small_kind",
     "kernl_linear_w8_fwd",
     "kernl_linear_rms_fwd",
+    "kernl_linear_scaled_fwd",
     "kernl_linear_decode_fwd",
     "kernl_linear_splitk_workspace_bytes",
     "kernl_linear_splitk_fwd",
@@ -44,6 +45,7 @@ EXPORTED_SYMBOLS = (
     "kernl_linear_glu_fwd",
     "kernl_layernorm_fwd",
     "kernl_add_layernorm_fwd",
+    "kernl_add_rms_stats_fwd",
 )
 
 # the process-wide test and tuning hooks of include/kernl_hip_test.h (bound for the tests and benchmarks only)
@@ -140,6 +142,10 @@ def load() -> ctypes.CDLL:
     lib.kernl_linear_rms_fwd.argtypes = (
         [_vp, _vp, ctypes.c_float, _vp, _vp, _vp] + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int] * 3 + [_vp]
     )
+    lib.kernl_linear_scaled_fwd.restype = ctypes.c_int
+    lib.kernl_linear_scaled_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int] * 3 + [_vp]
+    lib.kernl_add_rms_stats_fwd.restype = ctypes.c_int
+    lib.kernl_add_rms_stats_fwd.argtypes = [_vp] * 4 + [_i64] * 5 + [ctypes.c_float, ctypes.c_int, _vp]
     lib.kernl_linear_small_kind.restype = ctypes.c_int
     lib.kernl_linear_small_kind.argtypes = [_i64] * 3
     lib.kernl_linear_glu_fwd.restype = ctypes.c_int
@@ -384,6 +390,51 @@ def linear_rms_fwd(x2d, rms_weight, eps: float, weight, bias, out2d, activation:
             _stream(x2d),
         )
     _check(st, "kernl_linear_rms_fwd")
+
+
+def linear_scaled_supported(x2d, weight) -> bool:
+    """What `kernl_linear_scaled_fwd` takes: 16-bit rows with unit feature stride, 16-byte aligned, K a multiple of 8."""
+    M, K = x2d.shape
+    return (
+        x2d.dtype in (torch.float16, torch.bfloat16) and weight.dtype == x2d.dtype and K % 8 == 0 and x2d.stride(1) == 1
+        and x2d.stride(0) % 8 == 0 and x2d.stride(0) < (1 << 22) and K < (1 << 22) and x2d.data_ptr() % 16 == 0
+        and weight.is_contiguous() and weight.data_ptr() % 16 == 0
+    )
+
+
+def linear_scaled_fwd(x2d, weight, bias, row_scale, out2d, activation: int, gated: bool) -> None:
+    """out = act((x @ w^T) * row_scale[:, None] + bias); gated: w and bias interleaved as for `linear_glu_fwd`."""
+    _require_gpu(x2d, weight, bias, row_scale, out2d)
+    M, K = x2d.shape
+    N = out2d.shape[1]
+    if row_scale.dtype != torch.float32 or row_scale.numel() != M or not row_scale.is_contiguous():
+        raise ValueError("row_scale must be a contiguous fp32 vector with one entry per row of x")
+    lib = load()
+    with torch.cuda.device(x2d.device):
+        st = lib.kernl_linear_scaled_fwd(
+            x2d.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(), row_scale.data_ptr(),
+            out2d.data_ptr(), M, N, K, _arr(x2d.stride()), _arr(out2d.stride()), int(activation), int(bool(gated)),
+            DTYPE_CODE[x2d.dtype], _stream(x2d),
+        )
+    _check(st, "kernl_linear_scaled_fwd")
+
+
+def add_rms_stats_fwd(a2d, b2d, sum2d, rstd, eps: float) -> None:
+    """sum = a + b (b and sum may be None: statistics of `a` alone), rstd[m] = 1 / sqrt(mean(sum[m]^2) + eps)."""
+    _require_gpu(a2d, b2d, sum2d, rstd)
+    M, N = a2d.shape
+    if rstd.dtype != torch.float32 or rstd.numel() != M or not rstd.is_contiguous():
+        raise ValueError("rstd must be a contiguous fp32 vector with one entry per row")
+    if a2d.stride(1) != 1 or (b2d is not None and (b2d.stride(1) != 1 or sum2d.stride(1) != 1)):
+        raise ValueError("add_rms_stats needs unit feature strides")
+    lib = load()
+    with torch.cuda.device(a2d.device):
+        st = lib.kernl_add_rms_stats_fwd(
+            a2d.data_ptr(), None if b2d is None else b2d.data_ptr(), None if sum2d is None else sum2d.data_ptr(),
+            rstd.data_ptr(), M, N, a2d.stride(0), 0 if b2d is None else b2d.stride(0),
+            0 if sum2d is None else sum2d.stride(0), float(eps), DTYPE_CODE[a2d.dtype], _stream(a2d),
+        )
+    _check(st, "kernl_add_rms_stats_fwd")
 
 
 def linear_decode_supported(x2d, weight) -> bool:

@@ -336,6 +336,37 @@ static int layernorm_dispatch(const void *x_, const void *res_, const void *w_, 
     return check_launch("layernorm");
 }
 
+// sum = a + b rounded to T (b may be NULL: then nothing is written), rstd[row] = 1 / sqrt(mean(sum^2) + eps) of the ROUNDED
+// sum — what an RMSNorm applied to the stored tensor would compute.  One wave per row, 16-byte chunks.
+template <typename T>
+__global__ void __launch_bounds__(256) add_rms_stats_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ sum,
+                                                            float *__restrict__ rstd, int M, int N, int64_t a_rs, int64_t b_rs,
+                                                            int64_t sum_rs, float eps) {
+    typedef typename Vec8<T>::type vec8;
+    const int lane = threadIdx.x & 63, row = (int)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const vec8 *ap = reinterpret_cast<const vec8 *>(a + (int64_t)row * a_rs);
+    const vec8 *bp = b != nullptr ? reinterpret_cast<const vec8 *>(b + (int64_t)row * b_rs) : nullptr;
+    vec8 *sp = b != nullptr ? reinterpret_cast<vec8 *>(sum + (int64_t)row * sum_rs) : nullptr;
+    float sq = 0.0f;
+    for (int c = lane; c < N / 8; c += 64) {
+        vec8 v = ap[c];
+        if (bp != nullptr) {
+            const vec8 w = bp[c];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = from_float<T>(to_float(v[e]) + to_float(w[e]));
+            sp[c] = v;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float f = to_float(v[e]);
+            sq = fmaf(f, f, sq);
+        }
+    }
+    sq = wave_sum(sq);
+    if (lane == 0) rstd[row] = rsqrtf(sq / (float)N + eps);
+}
+
 static int layernorm_entry(const void *x, const void *res, const void *w, const void *b, void *out,
                            float *mean, float *rstd, int64_t M, int64_t N, int64_t x_rs, int64_t x_cs,
                            int64_t res_rs, int64_t res_cs, int64_t out_rs, int64_t out_cs, float eps,
@@ -384,4 +415,29 @@ extern "C" int kernl_add_layernorm_fwd(const void *x, const void *residual, cons
     return kernl::layernorm_entry(x, residual, w, bias, out, mean, rstd, M, N, x_row_stride, x_col_stride,
                                   res_row_stride, res_col_stride, out_row_stride, out_col_stride, eps,
                                   is_rms, dtype, stream);
+}
+
+extern "C" int kernl_add_rms_stats_fwd(const void *a, const void *b, void *sum, float *rstd, int64_t M, int64_t N,
+                                       int64_t a_row_stride, int64_t b_row_stride, int64_t sum_row_stride, float eps,
+                                       int dtype, void *stream) {
+    using namespace kernl;
+    if (a == nullptr || rstd == nullptr) return set_error(KERNL_ERR_INVALID_ARG, "add_rms_stats: a and rstd must not be NULL");
+    if (b != nullptr && sum == nullptr) return set_error(KERNL_ERR_INVALID_ARG, "add_rms_stats: b given without sum");
+    if (M < 0 || N <= 0) return set_error(KERNL_ERR_INVALID_ARG, "add_rms_stats: bad sizes M=%lld N=%lld", (long long)M, (long long)N);
+    if (dtype != KERNL_F16 && dtype != KERNL_BF16)
+        return set_error(KERNL_ERR_UNSUPPORTED, "add_rms_stats: only f16 and bf16 are supported, got dtype %d", dtype);
+    if (N % 8 != 0 || N > (1 << 20) || M > INT32_MAX - 4 || !aligned16(a) || a_row_stride % 8 != 0 ||
+        (b != nullptr && (!aligned16(b) || !aligned16(sum) || b_row_stride % 8 != 0 || sum_row_stride % 8 != 0)))
+        return set_error(KERNL_ERR_UNSUPPORTED, "add_rms_stats: rows must be contiguous, 16-byte aligned and a multiple of 8 "
+                         "elements long");
+    if (M == 0) return KERNL_OK;
+    const dim3 grid((unsigned)((M + 3) / 4)), block(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == KERNL_F16)
+        hipLaunchKernelGGL((add_rms_stats_kernel<f16>), grid, block, 0, st, static_cast<const f16 *>(a), static_cast<const f16 *>(b),
+                           static_cast<f16 *>(sum), rstd, (int)M, (int)N, a_row_stride, b_row_stride, sum_row_stride, eps);
+    else
+        hipLaunchKernelGGL((add_rms_stats_kernel<bf16>), grid, block, 0, st, static_cast<const bf16 *>(a), static_cast<const bf16 *>(b),
+                           static_cast<bf16 *>(sum), rstd, (int)M, (int)N, a_row_stride, b_row_stride, sum_row_stride, eps);
+    return check_launch("add_rms_stats");
 }

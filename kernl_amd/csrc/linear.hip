@@ -186,6 +186,52 @@ extern "C" int kernl_linear_glu_fwd(const void *x, const void *w, const void *bi
     return dtype == KERNL_F16 ? linear_mfma_dispatch<f16>(a) : linear_mfma_dispatch<bf16>(a);
 }
 
+extern "C" int kernl_linear_scaled_fwd(const void *x, const void *w, const void *bias, const float *row_scale, void *out,
+                                       int64_t M, int64_t N, int64_t K, const int64_t x_strides[2],
+                                       const int64_t out_strides[2], int activation, int gated, int dtype, void *stream) {
+    using namespace kernl;
+    if (x == nullptr || w == nullptr || out == nullptr || row_scale == nullptr || x_strides == nullptr || out_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "scaled linear: x, w, row_scale, out and their strides must not be NULL");
+    if (M < 0 || N <= 0 || K <= 0)
+        return set_error(KERNL_ERR_INVALID_ARG, "scaled linear: bad sizes M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+                         (long long)K);
+    const int64_t rows_w = gated ? 2 * N : N;  // the kernels see the interleaved weight of the gated form
+    if (M > INT32_MAX || rows_w > INT32_MAX || K > INT32_MAX)
+        return set_error(KERNL_ERR_UNSUPPORTED, "scaled linear: sizes must fit in 31 bits");
+    if (gated && N % 32 != 0)
+        return set_error(KERNL_ERR_UNSUPPORTED, "scaled linear: gated output width %lld must be a multiple of 32 (the "
+                         "interleaving block)", (long long)N);
+    if (activation < KERNL_ACT_NONE || activation > KERNL_ACT_SILU)
+        return set_error(KERNL_ERR_INVALID_ARG, "scaled linear: unknown activation %d", activation);
+    if (activation != (gated ? KERNL_ACT_SILU : KERNL_ACT_NONE))
+        return set_error(KERNL_ERR_UNSUPPORTED, "scaled linear: built for plain sums without activation and for SiLU gates "
+                         "(the projections an RMSNorm feeds in a SwiGLU decoder), got activation %d, gated %d", activation, gated);
+    if (dtype != KERNL_F16 && dtype != KERNL_BF16)
+        return set_error(KERNL_ERR_UNSUPPORTED, "scaled linear: only f16 and bf16 are supported, got dtype %d", dtype);
+    if (x_strides[1] != 1 || K % 8 != 0 || x_strides[0] % 8 != 0 || !aligned16(x) || !aligned16(w) || !aligned16(row_scale) ||
+        x_strides[0] >= (1 << 22) || K >= (1 << 22))
+        return set_error(KERNL_ERR_UNSUPPORTED, "scaled linear: x must have unit feature stride, 16-byte aligned rows and K a "
+                         "multiple of 8; w and row_scale 16-byte aligned bases");
+    if (M == 0) return KERNL_OK;
+    LinearArgs a;
+    a.x = x; a.w = w; a.bias = bias; a.out = out; a.act_in = nullptr;
+    a.M = (int)M; a.N = (int)rows_w; a.K = (int)K;
+    a.x_rs = x_strides[0]; a.x_cs = x_strides[1];
+    a.out_rs = out_strides[0]; a.out_cs = out_strides[1];
+    a.ai_rs = 0; a.ai_cs = 0;
+    a.act = gated ? (kGluBit | activation) : activation;
+    a.st = static_cast<hipStream_t>(stream);
+    a.row_scale = row_scale;
+    // only the wide kernels take per-row factors (5 / 6: 256-row tiles, 7 / 8: 128-row tiles; gated: 256 x 256 only)
+    int pick = g_linear_force_tile >= 5 && g_linear_force_tile <= 8 ? g_linear_force_tile : pick_tile(a.M, a.N, a.K, gated != 0, true);
+    if (gated) pick = 5;
+    if (pick == 5) run_wide(a, dtype, 256);
+    else if (pick == 6) run_wide(a, dtype, 192);
+    else if (pick == 7) run_wide_half(a, dtype, 256);
+    else run_wide_half(a, dtype, 192);
+    return check_launch("scaled linear");
+}
+
 extern "C" int kernl_linear_w8_fwd(const void *x, const void *w8, const void *bias, void *out, void *act_in, int64_t M,
                                    int64_t N, int64_t K, const int64_t x_strides[2], const int64_t out_strides[2],
                                    const int64_t act_in_strides[2], int activation, int dtype, void *stream) {

@@ -472,6 +472,30 @@ __device__ __forceinline__ void wide_bias_unpack(const uint32_t (&raw)[NBN / 2],
     for (int j = 0; j < NBN; ++j) bf[j] = to_float(__builtin_bit_cast(T, (uint16_t)(raw[j >> 1] >> (16 * (j & 1)))));
 }
 
+// Optional per-row factors of the finished sums (fp32, one per row of x: the inverse root mean square when an RMSNorm
+// has been folded into the weight): rs[i][v] belongs to row 16 i + 4 g + v of the wave's sub-tile, 1 without factors and
+// beyond M.  Fetched in front of a tile's main loop, like the bias.
+template <int NBM>
+__device__ __forceinline__ void wide_row_scale_fetch(const float *__restrict__ row_scale, int m_lane, int M, float (&rs)[NBM][4]) {
+#pragma unroll
+    for (int i = 0; i < NBM; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) rs[i][v] = 1.0f;
+    if (row_scale == nullptr) return;
+#pragma unroll
+    for (int i = 0; i < NBM; ++i) {
+        const int m = m_lane + 16 * i;  // a multiple of 4: 16-byte aligned in an aligned vector
+        if (m + 4 <= M) {
+            const float4 v4 = *reinterpret_cast<const float4 *>(row_scale + m);
+            rs[i][0] = v4.x, rs[i][1] = v4.y, rs[i][2] = v4.z, rs[i][3] = v4.w;
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (m + v < M) rs[i][v] = row_scale[m + v];
+        }
+    }
+}
+
 // NV rounded values of one row -> one 16-, 12- or 8-byte store
 template <typename T, int NV>
 __device__ __forceinline__ void wide_store_row(T *p, const float (&r)[NV]) {
@@ -484,13 +508,13 @@ __device__ __forceinline__ void wide_store_row(T *p, const float (&r)[NV]) {
     else *reinterpret_cast<u32x2 *>(p) = u32x2{w[0], w[1]};
 }
 
-// Epilogue of m-block IB (16 rows) of a wave of the wide kernels.  Blocks that lie inside the matrix, with contiguous
+// Epilogue of m-block IB (16 rows) of a wave of the wide kernels: out = act(sum * row factor + bias).  Blocks that lie inside the matrix, with contiguous
 // 16-byte aligned output rows and no pre-activation side output, run a straight-line path.
-template <typename T, int ACT, int IB, int NBN, int NBM = 8>
+template <typename T, int ACT, int IB, int NBN, int NBM = 8, bool SCALED = false>
 __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_wave, int n_wave, int l16, int g,
                                               T *__restrict__ out, T *__restrict__ act_in, int M, int N,
                                               int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs,
-                                              int out_vec_ok, int ai_vec_ok, const float (&bf)[NBN]) {
+                                              int out_vec_ok, int ai_vec_ok, const float (&bf)[NBN], const float (&rs)[4]) {
     constexpr bool GATED = (ACT & kGluBit) != 0;
     static_assert(!GATED || NBN == 8, "gated epilogues: four gate and four value blocks");
     constexpr int BASE = ACT & (kGluBit - 1), NV = WideLane<GATED, NBN>::NV;
@@ -501,8 +525,9 @@ __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_
     auto sums = [&](int v, float (&r)[NV], float (&value)[NV]) __attribute__((always_inline)) {
 #pragma unroll
         for (int c = 0; c < NV; ++c) {
-            r[c] = acc[IB][c][v] + bf[c];
-            value[c] = GATED ? acc[IB][(4 + c) % NBN][v] + bf[(4 + c) % NBN] : 1.0f;
+            r[c] = SCALED ? fmaf(acc[IB][c][v], rs[v], bf[c]) : acc[IB][c][v] + bf[c];
+            if (GATED) value[c] = SCALED ? fmaf(acc[IB][(4 + c) % NBN][v], rs[v], bf[(4 + c) % NBN]) : acc[IB][(4 + c) % NBN][v] + bf[(4 + c) % NBN];
+            else value[c] = 1.0f;
         }
     };
     const bool interior = m_wave + 16 * IB + 16 <= M && (GATED ? (n_wave >> 1) + 64 <= n_total : n_wave + NBN * 16 <= N) &&
@@ -549,12 +574,13 @@ __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_
 // W8: the weight is stored as one byte per element (fp8 e5m2, the upper byte of the fp16 encoding).  Its tile travels
 // HBM -> LDS as bytes (half the loads, 64-byte rows, chunks swizzled for 8-byte reads), a fragment is read as 8 bytes
 // and widened by four byte-permutes two read slots later, all in the shadow of the MFMAs; everything else is unchanged.
-template <typename T, int ACT, int NBN, bool W8 = false>
+// SCALED: the finished sums are multiplied by a factor per row of x (row_scale, fp32 [M]) before the bias is added.
+template <typename T, int ACT, int NBN, bool W8 = false, bool SCALED = false>
 __global__ void __launch_bounds__(256, 1)
 linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
                    T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
                    int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok, int ai_vec_ok,
-                   int bias_vec_ok) {
+                   int bias_vec_ok, const float *__restrict__ row_scale) {
     typedef typename Vec8<T>::type vec8;
     constexpr bool GATED = (ACT & kGluBit) != 0;
     static_assert(NBN == 8 || (NBN == 6 && !GATED), "256 or 192 columns per tile; gated epilogues need 256");
@@ -799,6 +825,8 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         const int n_wave = n0 + wave_n * (NBN * 16);
         uint32_t braw[NBN / 2];
         wide_bias_fetch<T, GATED, NBN>(bias, n_wave, l16, N, bias_vec_ok, braw);
+        float rsc[SCALED ? NB : 1][4];
+        if constexpr (SCALED) wide_row_scale_fetch<NB>(row_scale, m0 + wave_m * 128 + 4 * g, M, rsc);
         // (no zeroing of the accumulators: the first k-step of the tile writes them)
         k_tile(IntC<0>(), landed, BoolC<true>());
         advance_load();
@@ -824,8 +852,8 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         // one call per 16-row block: each stays small enough for the compiler to unroll completely, so the
         // accumulators are only ever indexed by constants and never leave the register file
 #define KERNL_WIDE_EPILOGUE(I)                                                                                         \
-    wide_epilogue<T, ACT, I, NBN>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs, ai_cs,   \
-                             out_vec_ok, ai_vec_ok, bf)
+    wide_epilogue<T, ACT, I, NBN, 8, SCALED>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs,  \
+                                             ai_cs, out_vec_ok, ai_vec_ok, bf, rsc[SCALED ? I : 0])
         KERNL_WIDE_EPILOGUE(0);
         KERNL_WIDE_EPILOGUE(1);
         KERNL_WIDE_EPILOGUE(2);
@@ -863,12 +891,13 @@ __device__ __forceinline__ void half_tile_origin(int t, int tiles_m, int tiles_n
 // SPLIT: blockIdx.y selects one of `splits` ranges of k-tiles; the workgroup leaves its fp32 partial tile in `part`
 // (slot blockIdx.y * tiles + t; per wave and 16 x 16 block 64 lanes x 16 bytes: coalesced, and the same lane reads it
 // back in linear_wide_half_reduce_kernel, which adds the ranges in order and runs the epilogue).
-template <typename T, int ACT, int NBN, bool W8 = false, bool SPLIT = false>
+template <typename T, int ACT, int NBN, bool W8 = false, bool SPLIT = false, bool SCALED = false>
 __global__ void __launch_bounds__(256, 1)
 linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
                         T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs,
                         int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok,
-                        int ai_vec_ok, int bias_vec_ok, float *__restrict__ part, int splits) {
+                        int ai_vec_ok, int bias_vec_ok, float *__restrict__ part, int splits,
+                        const float *__restrict__ row_scale) {
     typedef typename Vec8<T>::type vec8;
     static_assert((ACT & kGluBit) == 0 && (NBN == 8 || NBN == 6), "plain epilogues, 256 or 192 columns");
     constexpr int NBM = 4, BM = 32 * NBM, BN = 32 * NBN, BK = 64, RB = BK * 2, CPR = BK / 8, KSTEPS = BK / 32;
@@ -891,6 +920,9 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave & 1, wave_n = wave >> 1;
     const int l16 = lane & 15, g = lane >> 4;
+    // per-row factors of the finished sums, if any: they travel under the main loop
+    float rsc[SCALED ? NBM : 1][4];
+    if constexpr (SCALED) wide_row_scale_fetch<NBM>(row_scale, m0 + wave_m * (NBM * 16) + 4 * g, M, rsc);
 
     // tile loads, as in the wide kernel: every lane fetches the chunk that belongs at its LDS position
     constexpr uint32_t kOutOfRange = 0x80000000u;
@@ -1099,8 +1131,8 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     wide_bias_fetch<T, false, NBN>(bias, n_wave, l16, N, bias_vec_ok, braw);
     wide_bias_unpack<T, NBN>(braw, bf);
 #define KERNL_HALF_EPILOGUE(I)                                                                                         \
-    wide_epilogue<T, ACT, I, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, \
-                                       ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bf)
+    wide_epilogue<T, ACT, I, NBN, NBM, SCALED>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs,  \
+                                               out_cs, ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bf, rsc[SCALED ? I : 0])
     KERNL_HALF_EPILOGUE(0);
     KERNL_HALF_EPILOGUE(1);
     KERNL_HALF_EPILOGUE(2);
@@ -1151,10 +1183,11 @@ linear_wide_half_reduce_kernel(const float *__restrict__ part, const T *__restri
     float bf[NBN];
     wide_bias_fetch<T, false, NBN>(bias, n_wave, l16, N, bias_vec_ok, braw);
     wide_bias_unpack<T, NBN>(braw, bf);
+    const float ones[4] = {1.0f, 1.0f, 1.0f, 1.0f};  // (the split form takes no per-row factors)
 #define KERNL_HALF_REDUCE_EPILOGUE(IB)                                                                                   \
     if (I == IB)                                                                                                         \
     wide_epilogue<T, ACT, IB, NBN, NBM>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, \
-                                        ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bf)
+                                        ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bf, ones)
     KERNL_HALF_REDUCE_EPILOGUE(0);
     KERNL_HALF_REDUCE_EPILOGUE(1);
     KERNL_HALF_REDUCE_EPILOGUE(2);
@@ -1512,6 +1545,7 @@ struct LinearArgs {
     int act;
     hipStream_t st;
     const SkinnyExtra *extra = nullptr;  // residual / rotation of the few-row kernel (decoding steps)
+    const float *row_scale = nullptr;    // fp32 [M] factors of the finished sums (wide kernels only)
 };
 
 template <typename T, typename Cfg, int ACT, bool W8 = false>
@@ -1576,9 +1610,9 @@ static void launch_mfma_glu(const LinearArgs &a) {
     }
 }
 
-template <typename T, int ACT, int NBN = 8, bool W8 = false>
+template <typename T, int ACT, int NBN = 8, bool W8 = false, bool SCALED = false>
 static void launch_wide_act(const LinearArgs &a) {
-    auto kern = linear_wide_kernel<T, ACT, NBN, W8>;
+    auto kern = linear_wide_kernel<T, ACT, NBN, W8, SCALED>;
     constexpr int LDS_BYTES = 2 * (256 + 256) * 128;  // two stages
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
@@ -1598,15 +1632,12 @@ static void launch_wide_act(const LinearArgs &a) {
     const int slots = (per_xcd < 32 || ((a.K + 63) / 64) % 2 != 0) ? per_xcd : 32;
     hipLaunchKernelGGL(kern, dim3(slots * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
-                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok);
+                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, a.row_scale);
 }
 
-template <typename T, int ACT, int NBN, bool W8>
-static void launch_wide_half_act(const LinearArgs &a);
-
-template <typename T, int ACT, int NBN, bool W8 = false>
+template <typename T, int ACT, int NBN, bool W8 = false, bool SCALED = false>
 static void launch_wide_half_act(const LinearArgs &a) {
-    auto kern = linear_wide_half_kernel<T, ACT, NBN, W8>;
+    auto kern = linear_wide_half_kernel<T, ACT, NBN, W8, false, SCALED>;
     constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768;  // three stages
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
@@ -1623,7 +1654,7 @@ static void launch_wide_half_act(const LinearArgs &a) {
     const int bias_vec_ok = bias != nullptr && aligned16(bias);
     hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
-                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, static_cast<float *>(nullptr), 1);
+                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, static_cast<float *>(nullptr), 1, a.row_scale);
 }
 
 // Split form of the 128 x 192 kernel for row counts that leave most CUs without a tile (129 to about 700 rows against
@@ -1668,7 +1699,7 @@ static void launch_half_split_act(const LinearArgs &a, const HalfSplitPlan &p, f
     const int bias_vec_ok = bias != nullptr && aligned16(bias);
     hipLaunchKernelGGL(kern, dim3(per_xcd * 8, p.splits), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
-                       a.ai_cs, p.tiles_m, p.tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, part, p.splits);
+                       a.ai_cs, p.tiles_m, p.tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, part, p.splits, static_cast<const float *>(nullptr));
     hipLaunchKernelGGL((linear_wide_half_reduce_kernel<T, ACT, NBN>), dim3(p.tiles_m * p.tiles_n, 4), dim3(256), 0, a.st,
                        part, bias, out, act_in, a.M, a.N, a.out_rs, a.out_cs, a.ai_rs, a.ai_cs, p.tiles_m, p.tiles_n,
                        out_vec_ok, ai_vec_ok, bias_vec_ok, p.splits);
@@ -1688,6 +1719,10 @@ static void launch_half_split(const LinearArgs &a, const HalfSplitPlan &p, float
 
 template <typename T, int NBN>
 static void launch_wide_half(const LinearArgs &a) {
+    if (a.row_scale != nullptr) {  // (the entry point admits no activation with per-row factors here)
+        launch_wide_half_act<T, KERNL_ACT_NONE, NBN, false, true>(a);
+        return;
+    }
     switch (a.act) {
         case KERNL_ACT_RELU: launch_wide_half_act<T, KERNL_ACT_RELU, NBN>(a); break;
         case KERNL_ACT_TANH: launch_wide_half_act<T, KERNL_ACT_TANH, NBN>(a); break;
@@ -1700,6 +1735,10 @@ static void launch_wide_half(const LinearArgs &a) {
 
 template <typename T>
 static void launch_wide192(const LinearArgs &a) {
+    if (a.row_scale != nullptr) {
+        launch_wide_act<T, KERNL_ACT_NONE, 6, false, true>(a);
+        return;
+    }
     switch (a.act) {
         case KERNL_ACT_RELU: launch_wide_act<T, KERNL_ACT_RELU, 6>(a); break;
         case KERNL_ACT_TANH: launch_wide_act<T, KERNL_ACT_TANH, 6>(a); break;
@@ -1712,6 +1751,11 @@ static void launch_wide192(const LinearArgs &a) {
 
 template <typename T>
 static void launch_wide(const LinearArgs &a) {
+    if (a.row_scale != nullptr) {  // (the entry point admits SiLU gates and plain sums with per-row factors)
+        if (a.act & kGluBit) launch_wide_act<T, kGluBit | KERNL_ACT_SILU, 8, false, true>(a);
+        else launch_wide_act<T, KERNL_ACT_NONE, 8, false, true>(a);
+        return;
+    }
     if (a.act & kGluBit) {
         switch (a.act & (kGluBit - 1)) {
             case KERNL_ACT_GELU_ERF: launch_wide_act<T, kGluBit | KERNL_ACT_GELU_ERF>(a); break;
@@ -1749,7 +1793,7 @@ static double tile_cost(int M, int N, int K, int bm, int bn, double base, double
     return (double)per_cu * ((double)bm * bn / 65536.0) * (base + per_k * kf);
 }
 // which: 1 = 256x256, 2 = 256x192, 3 = 128x128 (8-wave kernel), 5 = wide 256x256, 6 = wide 256x192, 7 = wide 128x256, 8 = wide 128x192
-static int pick_tile(int M, int N, int K, bool gated) {
+static int pick_tile(int M, int N, int K, bool gated, bool wide_only = false) {
     // (the wide kernels take any K the MFMA path takes, with a zero-filled last k-tile)
     int pick = 5;
     double best = tile_cost(M, N, K, 256, 256, 1.0, 0.0);
@@ -1762,8 +1806,9 @@ static int pick_tile(int M, int N, int K, bool gated) {
     const double c8 = gated ? 1e30 : tile_cost(M, N, K, 128, 192, 1.65, -0.35);
     if (c8 < best) { best = c8; pick = 8; }
     // 256x192 gives a wave an odd number of column blocks: not usable for gate/value pairs
-    const double c2 = gated ? 1e30 : tile_cost(M, N, K, 256, 192, 1.2, 0.3);
-    const double c3 = tile_cost(M, N, K, 128, 128, 1.9, 0.4);
+    // (wide_only: the caller needs an epilogue only the wide kernels have)
+    const double c2 = gated || wide_only ? 1e30 : tile_cost(M, N, K, 256, 192, 1.2, 0.3);
+    const double c3 = wide_only ? 1e30 : tile_cost(M, N, K, 128, 128, 1.9, 0.4);
     if (c2 < best) { best = c2; pick = 2; }
     if (c3 < best) { best = c3; pick = 3; }
     return pick;

@@ -195,9 +195,19 @@ def rms_linear_layer(
     bias: Optional[torch.Tensor] = None,
     activation: str = "",
     gated: bool = False,
+    folded_weight: Optional[torch.Tensor] = None,
+    rstd: Optional[torch.Tensor] = None,
+    unfolded=None,
 ) -> torch.Tensor:
     """activation(linear(rms_norm(x, rms_weight, eps), weight, bias)) — or, with `gated`, the gated linear unit of the
     normalised input (weight and bias interleaved by `interleave_glu_rows`) — in one launch for decoding steps.
+
+    Prompts (more rows than the few-row kernels take) run the norm folded away when the caller hands in `folded_weight`
+    = weight * rms_weight[None, :]: rms_norm(x) @ w^T = rstd[:, None] * (x @ folded_weight^T), the factor applied in the
+    tile kernels' epilogue (`scaled_linear_layer`).  `rstd` [rows] fp32 = 1 / sqrt(mean(x^2) + eps) comes from whoever
+    produced x (`add_rms_stats`) or is computed here in one pass over x.  A caller that passes the folded weight as
+    `weight` too (it keeps no other arrangement) gives `unfolded`, a function returning the plain one, for the shapes that
+    end up on the two-launch path.
 
     Reference: `rms_matmul_rbe_wrapper` without the rotary epilogue (experimental/llama-v2/kernel/
     fused_kernel_proj_qkv.py:186-213) and `kernel_ff` (fused_kernel_ff.py:82-117), whose kernels normalise inside the
@@ -222,10 +232,77 @@ def rms_linear_layer(
         out = torch.empty((x_.shape[0], n_out), device=x.device, dtype=x.dtype)
         _lib.linear_rms_fwd(x_, rms_weight, eps, weight, bias, out, ACTIVATIONS.get(activation, _lib.ACT_NONE), gated)
         return out if x.ndim == 2 else out.reshape(*x.shape[:-1], n_out)
+    if (
+        folded_weight is not None
+        and activation == ("silu" if gated else "")
+        and (not gated or n_out % GLU_BLOCK == 0)
+        and x_.shape[0] > FEW_ROW_MAX_ROWS
+        and _lib.linear_scaled_supported(x_, folded_weight)
+        and (bias is None or bias.dtype == x.dtype)
+        # only where the plain product would run the wide tile kernels anyway (not the small-tile or split-K forms)
+        and not takes_small_problem_kernel(x_, folded_weight)
+        and (x_.shape[0] > SPLIT_K_MAX_ROWS or _lib.linear_splitk_workspace_bytes(x_, folded_weight) == 0)
+    ):
+        if rstd is None:
+            rstd = rms_stats(x_, eps, clamp=False)
+        out = scaled_linear_layer(x_, folded_weight, bias, rstd, activation, gated)
+        return out if x.ndim == 2 else out.reshape(*x.shape[:-1], n_out)
     normed = layer_norm(x, rms_weight, None, eps, use_rms_norm=True)
+    if unfolded is not None:
+        weight = unfolded()
     if gated:
         return linear_glu_layer(normed, weight, bias, activation)
     return linear_layer(normed, weight, bias, activation)
+
+
+def rms_eps(dtype: torch.dtype, eps: float) -> float:
+    """The eps the RMSNorm operator uses for `dtype`: fp16 inputs clamp it to 1.6e-5 (reference: layer_norm.py:295-296)."""
+    return max(eps, 1.6e-5) if dtype == torch.float16 else eps
+
+
+def rms_stats(x: torch.Tensor, eps: float, clamp: bool = True) -> torch.Tensor:
+    """rstd [rows] fp32 = 1 / sqrt(mean(x^2, -1) + eps) of a 16-bit tensor, one pass over x."""
+    x_ = x if x.ndim == 2 else x.reshape(-1, x.shape[-1])
+    if x_.stride(-1) != 1 or x_.stride(0) % 8 != 0 or x_.data_ptr() % 16 != 0:
+        x_ = x_.contiguous()
+    rstd = torch.empty((x_.shape[0],), device=x.device, dtype=torch.float32)
+    _lib.add_rms_stats_fwd(x_, None, None, rstd, rms_eps(x.dtype, eps) if clamp else eps)
+    return rstd
+
+
+def add_rms_stats_supported(a: torch.Tensor, b: torch.Tensor) -> bool:
+    return (
+        a.is_cuda and a.dtype in (torch.float16, torch.bfloat16) and b.dtype == a.dtype and a.shape == b.shape
+        and a.ndim >= 2 and a.shape[-1] % 8 == 0 and a.numel() > 0
+    )
+
+
+def add_rms_stats(a: torch.Tensor, b: torch.Tensor, eps: float):
+    """(a + b, rstd): the sum rounded to the inputs' dtype and, per row, 1 / sqrt(mean(sum^2) + eps) of the rounded sum
+    in fp32 — a residual addition together with the row statistics of the RMSNorm that follows it, in one pass.
+    `eps` is used as given (`rms_eps` holds the operator's fp16 policy)."""
+    assert add_rms_stats_supported(a, b)
+    rows = a.numel() // a.shape[-1]
+
+    def rows_of(t):
+        t2 = t.reshape(rows, t.shape[-1])
+        return t2 if t2.stride(-1) == 1 and t2.stride(0) % 8 == 0 and t2.data_ptr() % 16 == 0 else t2.contiguous()
+
+    out = torch.empty(a.shape, device=a.device, dtype=a.dtype)
+    rstd = torch.empty((rows,), device=a.device, dtype=torch.float32)
+    _lib.add_rms_stats_fwd(rows_of(a), rows_of(b), out.view(rows, a.shape[-1]), rstd, eps)
+    return out, rstd
+
+
+def scaled_linear_layer(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], row_scale: torch.Tensor,
+                        activation: str = "", gated: bool = False) -> torch.Tensor:
+    """act((x @ weight^T) * row_scale[:, None] + bias) for 2-D x; gated: silu(gate) * value of the interleaved weight.
+    The tile kernels' epilogue applies the factor: see `kernl_linear_scaled_fwd`."""
+    assert x.ndim == 2 and row_scale.dtype == torch.float32 and row_scale.numel() == x.shape[0]
+    n_out = weight.shape[0] // 2 if gated else weight.shape[0]
+    out = torch.empty((x.shape[0], n_out), device=x.device, dtype=x.dtype)
+    _lib.linear_scaled_fwd(x, weight, bias, row_scale, out, ACTIVATIONS.get(activation, _lib.ACT_NONE), gated)
+    return out
 
 
 def decode_linear_supported(x: torch.Tensor, weight: torch.Tensor, head_dim: Optional[int] = None) -> bool:

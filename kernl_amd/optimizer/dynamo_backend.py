@@ -16,6 +16,7 @@ from kernl_amd.optimizer.layer_norm import replace_layer_norm, replace_layer_nor
 from kernl_amd.optimizer.linear import (
     fuse_residual_into_linears,
     fuse_rms_norm_into_linears,
+    fuse_rms_stats_into_residual_adds,
     fuse_rotary_into_projections,
     replace_all_linear,
 )
@@ -54,4 +55,5 @@ def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
     fuse_rms_norm_into_linears(gm)
     fuse_rotary_into_projections(gm)
     fuse_residual_into_linears(gm)
+    fuse_rms_stats_into_residual_adds(gm)
     return gm

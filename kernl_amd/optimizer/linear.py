@@ -478,13 +478,90 @@ def _rms_weight_like(x: torch.Tensor, rms_weight: torch.Tensor) -> torch.Tensor:
     return rms_weight if rms_weight.dtype == x.dtype else rms_weight.to(x.dtype)
 
 
-def rms_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, weight, bias, activation=""):
+RMS_PROMPT_FOLDING = True   # tuning hook: False keeps prompts on the RMSNorm kernel followed by the plain products
+
+
+def _rms_prompt_foldable(x: torch.Tensor, rms_weight: torch.Tensor) -> bool:
+    """Prompts: more rows than the few-row kernels take, 16-bit, no autocast — the norm is folded into the weight and
+    the row statistics into the product's epilogue (`rms_linear_layer` decides whether the shape runs that way)."""
+    from kernl_amd.implementations.linear_layer import FEW_ROW_MAX_ROWS
+
+    rows = x.numel() // x.shape[-1] if x.numel() else 0
+    return (
+        RMS_PROMPT_FOLDING
+        and x.is_cuda
+        and x.dtype in (torch.float16, torch.bfloat16)
+        and rows > FEW_ROW_MAX_ROWS
+        and x.shape[-1] % 8 == 0
+        and rms_weight.shape == (x.shape[-1],)
+        and not torch.is_autocast_enabled("cuda")
+    )
+
+
+def _folded(weight: torch.Tensor, rms_weight: torch.Tensor) -> torch.Tensor:
+    # the product is formed in fp32 and rounded once
+    return (weight.float() * rms_weight.float()[None, :]).to(weight.dtype)
+
+
+def _folded_weight(weight: torch.Tensor, rms_weight: torch.Tensor) -> torch.Tensor:
+    """weight * rms_weight[None, :] of ONE parameter (a copy, rewritten in place when either version counter moves)."""
+    params = (weight, rms_weight)
+    cached = _fused_params.get(params)
+    if cached is None:
+        cached = _folded(weight.detach(), rms_weight.detach()).contiguous()
+        _fused_params.put(params, cached, lambda value, originals: value.copy_(_folded(originals[0].detach(), originals[1].detach())))
+    return cached
+
+
+def _folded_concatenated_weight(weights, rms_weight: torch.Tensor) -> torch.Tensor:
+    """Row-concatenated weights of sibling projections with the norm's weight multiplied into their columns: a second
+    copy beside the concatenation the parameters alias (which decoding steps keep using), rewritten in place when a
+    version counter moves."""
+    params = tuple(weights) + (rms_weight,)
+    cached = _fused_params.get(params)
+    if cached is None:
+        def build(originals):
+            return _folded(torch.cat([w.detach() for w in originals[:-1]], dim=0), originals[-1].detach())
+
+        cached = build(params).contiguous()
+        _fused_params.put(params, cached, lambda value, originals: value.copy_(build(originals)))
+    return cached
+
+
+def _folded_interleaved_params(half: bool, w_gate, b_gate, w_value, b_value, rms_weight: torch.Tensor):
+    """`_interleaved_params` with the norm's weight multiplied into the columns of both weights."""
+    params = (w_gate, w_value, rms_weight) + (() if b_gate is None else (b_gate, b_value))
+    cached = _fused_params.get(params)
+    if cached is None:
+        for p in params:
+            if p.dtype == torch.float32 and half:
+                p.data = p.data.half()
+
+        def build_weight(originals):
+            g = originals[2].detach()
+            return interleave_glu_rows(_folded(originals[0].detach(), g), _folded(originals[1].detach(), g))
+
+        weight = build_weight(params)
+        bias = None if b_gate is None else interleave_glu_rows(b_gate.detach(), b_value.detach())
+        cached = (weight, bias)
+
+        def rebuild(value, originals):
+            value[0].copy_(build_weight(originals))
+            if value[1] is not None:
+                value[1].copy_(interleave_glu_rows(originals[3].detach(), originals[4].detach()))
+
+        _fused_params.put(params, cached, rebuild)
+    return cached
+
+
+def rms_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, weight, bias, activation="", rstd=None):
     """linear_wrapper_functional(layer_norm_rms_wrapper(x, rms_weight, eps), weight, bias, activation) — one launch
     for decoding steps (reference: `rms_matmul_rbe_wrapper`, experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:186-213)."""
     from kernl_amd.implementations.linear_layer import rms_linear_layer
     from kernl_amd.optimizer.layer_norm import layer_norm_rms_wrapper
 
-    if not _rms_fusable(x, rms_weight) or weight.dtype not in (x.dtype, torch.float32):
+    prompt = activation == "" and _rms_prompt_foldable(x, rms_weight)
+    if not (_rms_fusable(x, rms_weight) or prompt) or weight.dtype not in (x.dtype, torch.float32):
         return linear_wrapper_functional(layer_norm_rms_wrapper(x, rms_weight, eps), weight, bias, activation=activation)
     if weight.dtype == torch.float32:
         weight.data = weight.data.half()
@@ -493,26 +570,31 @@ def rms_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, weight, bias, ac
     if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
         return linear_wrapper_functional(layer_norm_rms_wrapper(x, rms_weight, eps), weight, bias, activation=activation)
     w = weight if weight.is_contiguous() else weight.contiguous()
-    return rms_linear_layer(x, _rms_weight_like(x, rms_weight), eps, w, bias, activation)
+    g = _rms_weight_like(x, rms_weight)
+    return rms_linear_layer(x, g, eps, w, bias, activation, folded_weight=_folded_weight(w, g) if prompt else None,
+                            rstd=rstd if prompt else None)
 
 
-def rms_fused_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, weights, biases):
+def rms_fused_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, weights, biases, rstd=None):
     """fused_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), weights, biases): the query / key / value
     projections of a decoder layer with the RMSNorm in front of them (reference: `rms_matmul_rbe_qkv_wrapper`,
     experimental/llama-v2/kernel/fused_kernel_proj_qkv.py:289-344, without its rotary epilogue)."""
     from kernl_amd.implementations.linear_layer import rms_linear_layer
     from kernl_amd.optimizer.layer_norm import layer_norm_rms_wrapper
 
-    if not _rms_fusable(x, rms_weight):
+    prompt = _rms_prompt_foldable(x, rms_weight)
+    if not (_rms_fusable(x, rms_weight) or prompt):
         return fused_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), weights, biases)
     weight, bias, sizes = _concatenated_params(x, weights, biases)
     if weight.dtype != x.dtype:
         return fused_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), weights, biases)
-    out = rms_linear_layer(x, _rms_weight_like(x, rms_weight), eps, weight, bias, "")
+    g = _rms_weight_like(x, rms_weight)
+    out = rms_linear_layer(x, g, eps, weight, bias, "", folded_weight=_folded_concatenated_weight(weights, g) if prompt else None,
+                           rstd=rstd if prompt else None)
     return tuple(torch.split(out, sizes, dim=-1))
 
 
-def rms_glu_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, w_gate, b_gate, w_value, b_value, activation: str):
+def rms_glu_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, w_gate, b_gate, w_value, b_value, activation: str, rstd=None):
     """glu_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), ...): the feed-forward entry of a SwiGLU decoder
     with its RMSNorm (reference: `kernel_ff`, experimental/llama-v2/kernel/fused_kernel_ff.py:82-117, whose kernel
     normalises inside the product, :10-79)."""
@@ -520,12 +602,21 @@ def rms_glu_linear_wrapper(x: torch.Tensor, rms_weight, eps: float, w_gate, b_ga
     from kernl_amd.optimizer.layer_norm import layer_norm_rms_wrapper
 
     usable, half = _glu_usable(x, w_gate, b_gate, w_value, b_value)
-    if not usable or not _rms_fusable(x, rms_weight):
+    prompt = activation == "silu" and _rms_prompt_foldable(x, rms_weight)
+    if not usable or not (_rms_fusable(x, rms_weight) or prompt):
         return glu_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), w_gate, b_gate, w_value, b_value, activation)
+    g = _rms_weight_like(x, rms_weight)
+    if prompt:
+        # prompts read the weight with the norm's weight folded in: the un-folded arrangement is only built if decoding
+        # steps (which apply the norm's weight to x) ever run through this layer
+        folded, bias = _folded_interleaved_params(half, w_gate, b_gate, w_value, b_value, g)
+        if folded.dtype == x.dtype:
+            return rms_linear_layer(x, g, eps, folded, bias, activation, gated=True, folded_weight=folded, rstd=rstd,
+                                    unfolded=lambda: _interleaved_params(half, w_gate, b_gate, w_value, b_value)[0])
     weight, bias = _interleaved_params(half, w_gate, b_gate, w_value, b_value)
     if weight.dtype != x.dtype:
         return glu_linear_wrapper(layer_norm_rms_wrapper(x, rms_weight, eps), w_gate, b_gate, w_value, b_value, activation)
-    return rms_linear_layer(x, _rms_weight_like(x, rms_weight), eps, weight, bias, activation, gated=True)
+    return rms_linear_layer(x, g, eps, weight, bias, activation, gated=True)
 
 
 def linear_residual_wrapper(v: torch.Tensor, weight: torch.Tensor, bias, residual: torch.Tensor):
@@ -555,7 +646,31 @@ def linear_residual_wrapper(v: torch.Tensor, weight: torch.Tensor, bias, residua
     return residual + linear_wrapper_functional(v, weight, bias)
 
 
-def rms_fused_linear_rope_wrapper(x: torch.Tensor, rms_weight, eps: float, weights, biases, cos, sin, n_rotated: int, head_dim: int):
+def linear_residual_stats_wrapper(v: torch.Tensor, weight: torch.Tensor, bias, residual: torch.Tensor, eps: float):
+    """(residual + linear(v, weight, bias), rstd): `linear_residual_wrapper` whose addition also leaves, for prompts, the
+    row statistics 1 / sqrt(mean(sum^2) + eps) of the RMSNorm that follows — the projections behind that norm take them
+    (`rstd=` of the `rms_*` wrappers) and never see a normalised tensor.  rstd is None where the statistics are not
+    wanted (decoding steps, whose one-launch kernels normalise inside the product; dtypes the kernel does not take)."""
+    from kernl_amd.implementations.linear_layer import add_rms_stats, add_rms_stats_supported, rms_eps
+
+    from kernl_amd.implementations.linear_layer import FEW_ROW_MAX_ROWS
+
+    rows = v.numel() // v.shape[-1] if v.numel() else 0
+    prompt = (
+        RMS_PROMPT_FOLDING and residual.is_cuda and rows > FEW_ROW_MAX_ROWS and not torch.is_autocast_enabled("cuda")
+        and residual.dtype in (torch.float16, torch.bfloat16) and residual.dtype == v.dtype
+        and residual.shape[:-1] == v.shape[:-1] and residual.shape[-1] == weight.shape[0] and weight.shape[0] % 8 == 0
+    )
+    if not prompt:
+        return linear_residual_wrapper(v, weight, bias, residual), None
+    y = linear_wrapper_functional(v, weight, bias)
+    if y.dtype != residual.dtype or not add_rms_stats_supported(residual, y):
+        return residual + y, None
+    return add_rms_stats(residual, y, rms_eps(residual.dtype, eps))
+
+
+def rms_fused_linear_rope_wrapper(x: torch.Tensor, rms_weight, eps: float, weights, biases, cos, sin, n_rotated: int, head_dim: int,
+                                  rstd=None):
     """rms_fused_linear_wrapper(x, ...) with the rotary embedding of its first `n_rotated` outputs (query and key) applied
     head by head: outputs [.., heads_i * head_dim] as before, the rotated ones already rotated.  A decoding step runs
     norm, product and rotation as ONE launch (reference: `rms_matmul_rbe_qkv_wrapper`,
@@ -580,7 +695,7 @@ def rms_fused_linear_rope_wrapper(x: torch.Tensor, rms_weight, eps: float, weigh
         out = decode_linear_layer(x, weight, bias, _rms_weight_like(x, rms_weight), eps, None, cos.squeeze(1), sin.squeeze(1),
                                   head_dim=head_dim, rope_cols=sum(sizes[:n_rotated]))
         return tuple(torch.split(out, sizes, dim=-1))
-    outs = list(rms_fused_linear_wrapper(x, rms_weight, eps, weights, biases))
+    outs = list(rms_fused_linear_wrapper(x, rms_weight, eps, weights, biases, rstd=rstd))
     first = outs[0]
     rot_cols = sum(sizes[:n_rotated])
     adjacent = (
@@ -607,6 +722,7 @@ torch.fx.wrap("rms_linear_wrapper")
 torch.fx.wrap("rms_fused_linear_wrapper")
 torch.fx.wrap("rms_glu_linear_wrapper")
 torch.fx.wrap("linear_residual_wrapper")
+torch.fx.wrap("linear_residual_stats_wrapper")
 torch.fx.wrap("rms_fused_linear_rope_wrapper")
 
 
@@ -636,6 +752,39 @@ def fuse_residual_into_linears(gm: torch.fx.GraphModule):
             gm.graph.erase_node(lin)
             changed = True
             break
+    if changed:
+        gm.graph.lint()
+        gm.recompile()
+
+
+def fuse_rms_stats_into_residual_adds(gm: torch.fx.GraphModule):
+    """A `linear_residual_wrapper` whose sum feeds `rms_*` projections (the residual stream of a decoder layer in front
+    of the next RMSNorm) becomes `linear_residual_stats_wrapper`: element 0 replaces the sum everywhere, element 1 — the
+    row statistics of that norm — goes to those projections as `rstd=`.  All of them must use the same eps.  Runs after
+    the residual, RMSNorm and rotary passes."""
+    import operator
+
+    rms_forms = (rms_linear_wrapper, rms_fused_linear_wrapper, rms_glu_linear_wrapper, rms_fused_linear_rope_wrapper)
+    changed = False
+    for node in list(gm.graph.nodes):
+        if not (node.op == "call_function" and node.target is linear_residual_wrapper and len(node.args) == 4 and not node.kwargs):
+            continue
+        takers = [u for u in node.users if u.op == "call_function" and u.target in rms_forms and len(u.args) >= 3
+                  and u.args[0] is node and "rstd" not in u.kwargs and isinstance(u.args[2], (int, float))]
+        if not takers or len({float(u.args[2]) for u in takers}) != 1:
+            continue
+        with gm.graph.inserting_after(node):
+            both = gm.graph.call_function(linear_residual_stats_wrapper, tuple(node.args) + (float(takers[0].args[2]),))
+        with gm.graph.inserting_after(both):
+            total = gm.graph.call_function(operator.getitem, (both, 0))
+        with gm.graph.inserting_after(total):
+            rstd = gm.graph.call_function(operator.getitem, (both, 1))
+        total.meta = dict(node.meta)
+        node.replace_all_uses_with(total)
+        gm.graph.erase_node(node)
+        for u in takers:
+            u.kwargs = {**u.kwargs, "rstd": rstd}
+        changed = True
     if changed:
         gm.graph.lint()
         gm.recompile()

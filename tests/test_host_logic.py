@@ -382,8 +382,20 @@ def test_llama_graph_rewrite_and_constant_causal_mask():
         # nothing left of rotate_half nor of a rotation kernel of its own
         assert t.count("rms_fused_linear_rope_wrapper") == 2 and "rms_fused_linear_wrapper" not in t
         assert "rotary_wrapper" not in t and "neg" not in t
-        # the additions after the attention-output and feed-forward-down projections ride in those projections
-        assert t.count("linear_residual_wrapper") == 2 * 2 and "linear_wrapper_functional" not in t
+        # the additions after the attention-output and feed-forward-down projections ride in those projections; the
+        # three whose sum feeds the projections behind the next RMSNorm also leave that norm's row statistics (the
+        # last one feeds the final norm, which stays a kernel of its own)
+        assert t.count("linear_residual_stats_wrapper") == 3 and t.count("linear_residual_wrapper") == 1
+        assert "linear_wrapper_functional" not in t
+        for node in graphs[0].graph.nodes:
+            if node.op == "call_function" and node.target.__name__ in ("rms_glu_linear_wrapper", "rms_fused_linear_rope_wrapper"):
+                fed_by_sum = node.args[0].target.__name__ == "getitem" and node.args[0].args[1] == 0
+                if fed_by_sum:
+                    rstd = node.kwargs["rstd"]
+                    assert rstd.target.__name__ == "getitem" and rstd.args == (node.args[0].args[0], 1)
+                    assert rstd.args[0].target.__name__ == "linear_residual_stats_wrapper" and rstd.args[0].args[4] == 1e-5
+                else:
+                    assert "rstd" not in node.kwargs            # the first layer reads the embeddings
         assert t.count("add") == 1                      # position ids; no residual addition is left
         # the fresh key/value cache no longer copies: the only cat left builds the angle table
         assert t.count("cat") == 1
@@ -697,6 +709,72 @@ def test_residual_additions_fold_into_the_projection_before_them():
     assert t.count("linear_residual_wrapper") == 2 and t.count("add") == 2
     nodes = [n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "linear_residual_wrapper"]
     assert [n.args[3].name for n in nodes] == ["r", nodes[0].name]       # the residual operand of each
+
+
+def test_row_statistics_ride_in_the_residual_addition_only_where_every_taker_agrees():
+    """`fuse_rms_stats_into_residual_adds`: the sum of a residual projection that feeds `rms_*` projections becomes
+    element 0 of `linear_residual_stats_wrapper` for ALL its users and element 1 goes to those projections as `rstd=`;
+    takers with different eps leave the graph alone; a sum no `rms_*` projection reads keeps its plain wrapper."""
+    import operator
+
+    from kernl_amd.optimizer.linear import (fuse_rms_stats_into_residual_adds, linear_residual_wrapper, rms_glu_linear_wrapper,
+                                            rms_linear_wrapper)
+
+    def graph(eps_a, eps_b):
+        g = torch.fx.Graph()
+        x, r, w, gam = (g.placeholder(n) for n in ("x", "r", "w", "gam"))
+        h = g.call_function(linear_residual_wrapper, (x, w, None, r))
+        a = g.call_function(rms_linear_wrapper, (h, gam, eps_a, w, None))
+        b = g.call_function(rms_glu_linear_wrapper, (h, gam, eps_b, w, None, w, None, "silu"))
+        plain = g.call_function(linear_residual_wrapper, (a, w, None, h))      # reads the sum as its residual; feeds no norm
+        g.output((plain, b))
+        return torch.fx.GraphModule(torch.nn.Module(), g)
+
+    gm = graph(1e-6, 1e-6)
+    fuse_rms_stats_into_residual_adds(gm)
+    nodes = {n.name: n for n in gm.graph.nodes}
+    stats = [n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "linear_residual_stats_wrapper"]
+    assert len(stats) == 1 and stats[0].args[4] == 1e-6
+    total, rstd = [n for n in gm.graph.nodes if n.op == "call_function" and n.target is operator.getitem]
+    assert total.args == (stats[0], 0) and rstd.args == (stats[0], 1)
+    takers = [n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ in ("rms_linear_wrapper", "rms_glu_linear_wrapper")]
+    assert all(n.args[0] is total and n.kwargs["rstd"] is rstd for n in takers) and len(takers) == 2
+    plain = [n for n in gm.graph.nodes if n.op == "call_function" and n.target.__name__ == "linear_residual_wrapper"]
+    assert len(plain) == 1 and plain[0].args[3] is total
+    assert nodes  # (graph still lints)
+    gm.graph.lint()
+
+    gm = graph(1e-6, 1e-5)
+    fuse_rms_stats_into_residual_adds(gm)
+    assert "linear_residual_stats_wrapper" not in _targets(gm)
+
+
+def test_folded_norm_weights_follow_their_parameters():
+    """The prompt path's weights with the RMSNorm weight multiplied into their columns are copies: built once, rewritten
+    in place when the projection weight OR the norm weight changes, and dropped with their parameters."""
+    from kernl_amd.optimizer.linear import _folded_concatenated_weight, _folded_weight, _fused_params
+
+    w = torch.nn.Parameter(torch.randn(6, 4))
+    w2 = torch.nn.Parameter(torch.randn(2, 4))
+    g = torch.nn.Parameter(torch.rand(4) + 0.5)
+    f1 = _folded_weight(w, g)
+    assert torch.equal(f1, w.detach() * g.detach()[None, :]) and _folded_weight(w, g) is f1
+    fc = _folded_concatenated_weight([w, w2], g)
+    assert fc.shape == (8, 4) and torch.equal(fc, torch.cat([w, w2]).detach() * g.detach()[None, :])
+    with torch.no_grad():
+        g.mul_(2.0)
+    assert _folded_weight(w, g) is f1 and torch.equal(f1, w.detach() * g.detach()[None, :])
+    with torch.no_grad():
+        w2.add_(1.0)
+    assert _folded_concatenated_weight([w, w2], g) is fc and torch.equal(fc, torch.cat([w, w2]).detach() * g.detach()[None, :])
+    keys = [_fused_params.key_of((w, g)), _fused_params.key_of((w, w2, g))]
+    assert all(k in _fused_params._entries for k in keys)
+    del w, w2, g
+    import gc
+
+    gc.collect()
+    _fused_params._drop_dead()
+    assert not any(k in _fused_params._entries for k in keys)
 
 
 def test_residual_projection_keeps_the_addition_where_the_small_tile_kernels_are_faster(monkeypatch):

@@ -298,6 +298,97 @@ def test_linear_fp8_weight_stream_k(shape, close, monkeypatch):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("kind", ["plain", "plain_bias", "gated", "gated_bias"])
+@pytest.mark.parametrize("shape", [(2048, 12288, 4096), (2048, 11008, 4096), (300, 768, 512), (1000, 1056, 776), (129, 256, 264),
+                                   (4100, 192, 64)], ids=lambda s: "x".join(map(str, s)))
+def test_rms_norm_folded_into_the_weight_for_prompts(shape, kind, dtype, close):
+    """Prompts: rms_norm(x) @ w^T as rstd * (x @ (w * g)^T) with the row factor applied in the wide kernels' epilogue
+    (`kernl_linear_scaled_fwd`) and the statistics from `kernl_add_rms_stats_fwd` — against the composition of the RMSNorm
+    and linear / gated oracles on the UNFOLDED weights.  2048 x 4096 -> 12288 and -> 2 x 11008 are a Llama-7B prompt's
+    query/key/value and feed-forward entry projections (oracle on a sample of rows there); the others put ragged rows,
+    ragged columns, a ragged last k-tile and every tile shape of the wide kernels behind the same epilogue."""
+    from kernl_amd.implementations.linear_layer import interleave_glu_rows, rms_linear_layer, rms_stats
+    from oracle import glu_oracle, rms_norm_oracle
+
+    M, N, K = shape
+    gated, with_bias = kind.startswith("gated"), kind.endswith("bias")
+    if gated and N % 32 != 0:
+        pytest.skip("gated outputs come in blocks of 32")
+    gen = torch.Generator().manual_seed(43)
+    x = (torch.randn((M, K), generator=gen) * 3.0 + 0.5).to(dtype)       # rows far from unit RMS
+    x[::7] *= 0.05                                                       # and far from each other
+    g = (1.0 + 0.2 * torch.randn((K,), generator=gen)).to(dtype)
+    eps = 1e-5 if dtype == torch.bfloat16 else 1.6e-5
+    rows = torch.arange(0, M, 37 if M >= 2048 else 1)
+    normed = rms_norm_oracle(x[rows], g, eps)
+
+    def fold(w):
+        return (w.float() * g.float()[None, :]).to(dtype)
+
+    rstd = rms_stats(x.cuda(), eps, clamp=False)
+    torch.testing.assert_close(rstd.cpu(), torch.rsqrt(x.float().pow(2).mean(-1) + eps), rtol=2e-6, atol=0)
+    if gated:
+        wg = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+        wv = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+        bg, bv = ((0.5 * torch.randn((N,), generator=gen)).to(dtype) for _ in range(2)) if with_bias else (None, None)
+        bias = interleave_glu_rows(bg, bv).cuda() if with_bias else None
+        out = rms_linear_layer(x.cuda(), g.cuda(), eps, interleave_glu_rows(wg, wv).cuda(), bias, "silu", gated=True,
+                               folded_weight=interleave_glu_rows(fold(wg), fold(wv)).cuda(), rstd=rstd)
+        ref = glu_oracle(normed, wg, bg, wv, bv, "silu")
+    else:
+        w = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+        b = (0.5 * torch.randn((N,), generator=gen)).to(dtype) if with_bias else None
+        out = rms_linear_layer(x.cuda(), g.cuda(), eps, w.cuda(), None if b is None else b.cuda(), "",
+                               folded_weight=fold(w).cuda(), rstd=None if M == 300 else rstd)   # one case computes them itself
+        ref = linear_oracle(normed, w, b, "")
+    torch.cuda.synchronize()
+    assert out.shape == (M, N) and out.dtype == dtype
+    close(out[rows.cuda()], ref, dtype, scale="magnitude", what=f"folded rms + linear {shape} {kind}")
+
+
+def test_prompt_route_of_the_rms_projections_calls_the_scaled_kernel(monkeypatch):
+    """Which shapes take the folded route: more rows than the few-row kernels take, where the plain product would run the
+    wide tile kernels; fewer rows, or a missing folded weight, keep the kernels they had."""
+    from kernl_amd.implementations import linear_layer as ll
+
+    calls = []
+    real = _lib.linear_scaled_fwd
+    monkeypatch.setattr(_lib, "linear_scaled_fwd", lambda *a, **k: (calls.append(a[0].shape[0]), real(*a, **k))[1])
+    gen = torch.Generator().manual_seed(3)
+    w = (torch.randn((4096, 2048), generator=gen) * 0.02).half().cuda()
+    g = torch.ones(2048).half().cuda()
+    # (256 rows: too few tiles for the chip, the plain product splits K instead)
+    for rows, expect in ((2048, True), (4096, True), (256, False), (100, False), (16, False)):
+        x = torch.randn((rows, 2048), generator=gen).half().cuda()
+        n = len(calls)
+        a = ll.rms_linear_layer(x, g, 1e-5, w, None, "", folded_weight=w)
+        b = ll.rms_linear_layer(x, g, 1e-5, w, None, "")
+        assert (len(calls) > n) == expect, (rows, calls)
+        assert len(calls) <= n + 1            # never without the folded weight
+        torch.testing.assert_close(a.float(), b.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_residual_addition_with_row_statistics(close):
+    """`add_rms_stats`: the sum is the fp16 / bf16 rounding of the fp32 sum (what `a + b` gives), the statistics are those
+    of the ROUNDED sum; ragged row counts, 3-D inputs, non-contiguous operands."""
+    from kernl_amd.implementations.linear_layer import add_rms_stats
+
+    gen = torch.Generator().manual_seed(5)
+    for dtype in (torch.float16, torch.bfloat16):
+        for shape in ((3, 701, 1024), (2050, 4096), (130, 8), (5, 33, 776)):
+            a = (torch.randn(shape, generator=gen) * 4).to(dtype)
+            b = (torch.randn(shape, generator=gen) * 0.3).to(dtype)
+            total, rstd = add_rms_stats(a.cuda(), b.cuda(), 1e-5)
+            want = (a.float() + b.float()).to(dtype)
+            assert torch.equal(total.cpu(), want), (dtype, shape)
+            torch.testing.assert_close(rstd.cpu(), torch.rsqrt(want.float().pow(2).mean(-1) + 1e-5).reshape(-1), rtol=3e-6, atol=0)
+    a = torch.randn((400, 2048), generator=gen).half().cuda()[:, ::2]          # strided rows: copied before the launch
+    b = torch.randn((400, 1024), generator=gen).half().cuda()
+    total, rstd = add_rms_stats(a, b, 1e-5)
+    assert torch.equal(total, a + b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
 @pytest.mark.parametrize("kind", ["plain", "plain_bias_silu", "gated"])
 @pytest.mark.parametrize("shape", [(1, 4096, 4096), (5, 96, 64), (16, 1024, 192), (33, 2304, 768), (64, 512, 1024),
                                    (100, 256, 128), (4, 96, 72)], ids=lambda s: "x".join(map(str, s)))
