@@ -29,6 +29,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# torch.compile's worker pool (a child process per compile thread) is of no use here — the backend of optimize_model
+# compiles nothing — and would outlive the run: keep compilation in this process.  Must be set before torch is imported.
+os.environ.setdefault("TORCHINDUCTOR_COMPILE_THREADS", "1")
+
 PEAK_MFMA_F16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E
 
@@ -51,6 +55,22 @@ def _event_times(fn, n, flush=None):
 
 
 ATTENTION_KERNEL_SOURCES = ("attention.hip", "attention_pipe.hip", "attention_common.h", "index_math.h", "common.h")
+
+
+def reap_children():
+    """Ends whatever child processes are still alive (none are expected) and returns how many there were."""
+    try:
+        import psutil
+    except ImportError:
+        return None
+    children = psutil.Process().children(recursive=True)
+    for c in children:
+        try:
+            c.terminate()
+        except psutil.Error:
+            pass
+    psutil.wait_procs(children, timeout=5)
+    return len(children)
 
 
 def attention_sources_digest():
@@ -984,6 +1004,7 @@ def main():
             extra["measured_peak_error"] = f"{type(exc).__name__}: {exc}"[:300]
 
     result["extra"] = extra
+    result["extra"]["child_processes_at_exit"] = reap_children()
     print(json.dumps(result), flush=True)
 
 

@@ -34,21 +34,28 @@ namespace kernl {
 // tiles cannot be written to LDS by the load itself then: a thread fetches the 8 bytes of each of its 16-byte LDS
 // chunks into registers while the current tile is processed, widens them and stores them before the barrier that
 // publishes the stage.  Everything that reads LDS is the 16-bit kernel.
-template <typename T, int D, int WPE, int MASK_MODE, bool CAUSAL, bool KV8 = false>
+// WSPLIT (small grids: a few (batch, head) pairs, a few hundred keys or more): a workgroup owns 32 query rows instead of
+// 128 and its four waves split the KEY tiles of those rows — wave w takes tiles w, w + 4, ... through a double buffer of
+// its own, no barrier in the loop — and merge their (reference, row sum, accumulator) triples through LDS at the end.
+// Four times the workgroups, a quarter of the serial tile chain per wave.  Head size 64, no mask or a per-key mask,
+// non-causal, at most 64 key tiles; 8 stages of dynamic LDS.
+template <typename T, int D, int WPE, int MASK_MODE, bool CAUSAL, bool KV8 = false, bool WSPLIT = false>
 __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnParams p) {
+    static_assert(!WSPLIT || (D == 64 && !CAUSAL && !KV8 && MASK_MODE != MASK_MATRIX), "key tiles split over the waves: plain forms only");
     typedef typename Vec8<T>::type vec8;
     typedef __attribute__((address_space(3))) void lds_void;
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef short s16x8 __attribute__((ext_vector_type(8)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
     typedef AttnTileMap<D> TileMap;                       // staging and fragment addresses of a K / V stage
-    constexpr int BM = 128, BN = 64;
+    constexpr int BM = WSPLIT ? 32 : 128, BN = 64;
     constexpr int KROW = D * 2, VP = D * 2;               // LDS row bytes of the K tile [key][D] and V tile [key][D]
     constexpr int K_BYTES = BN * KROW, V_BYTES = BN * VP;
     constexpr int STAGE = K_BYTES + V_BYTES + BN * 4;     // + per-key additive term (fp32)
     constexpr int NBS = BN / 32, DB = D / 32, KS = D / 16;
     constexpr int DC = D / 8;                             // 16-byte chunks per K/V row
-    constexpr int KI = BN * DC / 256;                     // 1 KB loads per wave for each of K and V
+    constexpr int KI = BN * DC / (WSPLIT ? 64 : 256);     // 1 KB loads per wave for each of K and V
+    constexpr int DMA_STRIDE = WSPLIT ? 1024 : 4096;      // LDS distance between a wave's consecutive loads of a tile
 
     // head size 64 stages matrix masks through LDS: every wave keeps the 32 rows x 64 keys it needs of the current
     // key tile (8 KB as fp32) in a region of its own
@@ -56,14 +63,23 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     constexpr int MASK_WAVE_BYTES = 32 * BN * 4;
     constexpr int MASK_LDS = MASK_VIA_LDS ? 4 * MASK_WAVE_BYTES : 0;
 
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE + MASK_LDS];
+    __shared__ __attribute__((aligned(16))) unsigned char static_smem[WSPLIT ? 16 : 2 * STAGE + MASK_LDS];
+    extern __shared__ __attribute__((aligned(16))) unsigned char dynamic_smem[];  // WSPLIT: 4 waves x 2 stages
+    unsigned char *const smem = WSPLIT ? dynamic_smem : static_smem;
 
     // Workgroup ids are dealt round-robin to the 8 XCDs.  Normally the query tiles of one (batch, head) share an XCD
     // and with it the L2 that holds their keys and values; with a matrix mask that is broadcast over heads the
     // workgroups of one batch entry — all heads — share it, so that the mask, the larger operand, is fetched once.
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     int b, h, qt;
-    if (MASK_MODE == MASK_MATRIX && p.xcd_by_batch) {
+    if (WSPLIT) {
+        // small grids: workgroups are dealt to the XCDs one by one (the keys and values of a head are small, every XCD
+        // may fetch them), so that a grid of up to 256 workgroups is one round whatever the number of heads
+        const int bh = (int)blockIdx.x / p.nq_tiles;
+        qt = (int)blockIdx.x % p.nq_tiles;
+        b = bh / p.H;
+        h = bh % p.H;
+    } else if (MASK_MODE == MASK_MATRIX && p.xcd_by_batch) {
         const int per_batch = p.H * p.nq_tiles;
         b = (slot / per_batch) * 8 + xcd;
         h = (slot % per_batch) / p.nq_tiles;
@@ -81,7 +97,9 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 31, lh = lane >> 5;
     const int q0 = qt * BM;
-    const int m_wave0 = q0 + wave * 32;
+    const int m_wave0 = WSPLIT ? q0 : q0 + wave * 32;
+    const int wave_lds = WSPLIT ? wave * (2 * STAGE) : 0;  // WSPLIT: the wave's private pair of stages
+    const int ktid = WSPLIT ? lane : tid;                  // the thread's index among those that stage a tile together
     const int my_m = m_wave0 + lr;
     const int M = p.M, N = p.N;
 
@@ -114,13 +132,13 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     uint32_t kdma[KI], vdma[KI];
 #pragma unroll
     for (int i = 0; i < KI; ++i) {
-        const int qd = tid + 256 * i;
+        const int qd = ktid + (WSPLIT ? 64 : 256) * i;
         const int row = TileMap::stage_row(qd);
         kdma[i] = (uint32_t)(((int64_t)row * p.ks[2] + TileMap::k_stage_chunk(qd) * 8) * KVB);
         vdma[i] = (uint32_t)(((int64_t)row * p.vs[2] + TileMap::v_stage_chunk(qd) * 8) * KVB);
     }
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void *)smem;
-    const uint32_t dma_base = lds_base + wave * 1024;
+    const uint32_t dma_base = lds_base + (WSPLIT ? wave_lds : wave * 1024);
     const uint64_t kaddr = (uint64_t)(uintptr_t)kp, vaddr = (uint64_t)(uintptr_t)vp;
     const u32x4 krsrc = {(uint32_t)kaddr, (uint32_t)(kaddr >> 32) & 0xFFFFu,
                          (uint32_t)((((int64_t)N - 1) * p.ks[2] + D) * KVB), 0x00020000u};
@@ -155,11 +173,11 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 #pragma unroll
         for (int i = 0; i < KI; ++i)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :: "s"(sb + i * 4096), "v"(kdma[i]), "s"(kr), "s"(k_soff) : "memory", "m0");
+                         :: "s"(sb + i * DMA_STRIDE), "v"(kdma[i]), "s"(kr), "s"(k_soff) : "memory", "m0");
 #pragma unroll
         for (int i = 0; i < KI; ++i)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :: "s"(sb + K_BYTES + i * 4096), "v"(vdma[i]), "s"(vr), "s"(v_soff) : "memory", "m0");
+                         :: "s"(sb + K_BYTES + i * DMA_STRIDE), "v"(vdma[i]), "s"(vr), "s"(v_soff) : "memory", "m0");
     };
     // one-byte keys and values: the fetched bytes, widened (byte b of a dword becomes the 16-bit value b << 8), go to
     // the LDS positions the direct loads of the 16-bit kernel would have written
@@ -180,7 +198,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     // per-key additive term of a general tile (mask value in the log2 domain, -inf past the last key); thread tid
     // < 64 owns key tid of the tile
     auto key_bias = [&](int tile) __attribute__((always_inline)) -> float {
-        const int n = tile * BN + tid;
+        const int n = tile * BN + ktid;
         float bv = 0.0f;
         if (MASK_MODE == MASK_VECTOR)
             bv = scale_mask(load_mask_value(p.mask, p.mask_dtype, mask_base + min(n, N - 1) * p.ms[3]), p.clamp);
@@ -192,17 +210,19 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     const int n_end = CAUSAL ? min(N, q0 + BM + p.causal_off) : N;
     const int nt_all = (n_end + BN - 1) / BN;
     constexpr bool MAY_LIST = (MASK_MODE == MASK_VECTOR && !CAUSAL);
-    const bool use_list = MAY_LIST && nt_all <= 64;
+    const bool use_list = WSPLIT || (MAY_LIST && nt_all <= 64);  // (the host hands WSPLIT at most 64 tiles)
     int nt = nt_all, n_clean = 0;
     if (MASK_MODE == MASK_NONE) n_clean = CAUSAL ? min(N / BN, (q0 + p.causal_off + 1) / BN) : N / BN;
     // the first tile is fetched before the mask has been looked at: tile 0 almost always comes first
-    if (nt_all > 0) dma(0, 0);
+    // (WSPLIT: wave w's tiles are w, w + 4, ...)
+    const int t_first = WSPLIT ? wave : 0;
+    if (t_first < nt_all) dma(t_first, 0);
     // With a per-key mask every wave classifies all key tiles by itself (the mask row is a few KB, and this way no
     // barrier or LDS table is needed): bit t of clean_bits = tile t is all zero and full, of gen_bits = it needs
     // the general body; tiles in neither set are so negative everywhere that they contribute exactly 0 and are
     // dropped.  Both sets are wave-uniform scalars; tiles are taken from them lowest index first.
     uint64_t clean_bits = 0, gen_bits = 0;
-    if (use_list) {
+    if (use_list && MASK_MODE == MASK_VECTOR) {
         // lane l looks at key 64 t + l of tile t; 32-bit offsets (the host checks that a mask row fits them)
         auto classify = [&](auto *mrow) __attribute__((always_inline)) {
             const int ms3 = (int)p.ms[3];
@@ -237,9 +257,9 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
             typedef typename std::remove_cv<typename std::remove_pointer<decltype(mrow)>::type>::type MT;
             const __amdgpu_buffer_rsrc_t mrsrc =
                 __builtin_amdgcn_make_buffer_rsrc(const_cast<MT *>(mrow), 0, N * (int)sizeof(MT), 0x00020000);
-            for (int j = 0; j * 256 < N; ++j) {
-                const int e0 = (64 * j + lane) * 4;
-                float mv[4];
+            // two loads (512 keys) in flight per step: the loop is a chain of memory round trips otherwise
+            auto fetch = [&](int j, float (&mv)[4]) __attribute__((always_inline)) {
+                const int e0 = (64 * j + lane) * 4;  // (beyond the row the buffer returns zeros; `valid` below ignores them)
                 if constexpr (sizeof(MT) == 4) {
                     const f32x4 raw = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(mrsrc, e0 * 4, 0, 0));
 #pragma unroll
@@ -250,6 +270,9 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
 #pragma unroll
                     for (int r = 0; r < 4; ++r) mv[r] = (float)raw[r];
                 }
+            };
+            auto judge = [&](int j, const float (&mv)[4]) __attribute__((always_inline)) {
+                const int e0 = (64 * j + lane) * 4;
                 bool nz = false, nm = false;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -265,6 +288,13 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                 const bool general = any_nz || t * BN + BN > N;
                 clean_bits |= (__ballot(mine && !general) & 0xFull) << (4 * j);
                 gen_bits |= (__ballot(mine && general) & 0xFull) << (4 * j);
+            };
+            for (int j = 0; j * 256 < N; j += 2) {
+                float mv0[4], mv1[4];
+                fetch(j, mv0);
+                fetch(j + 1, mv1);
+                judge(j, mv0);
+                if ((j + 1) * 256 < N) judge(j + 1, mv1);
             }
         };
         const bool rows_vectorizable = p.ms[3] == 1;
@@ -283,6 +313,18 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         }
         // every key masked: keep all tiles, the result is the (finite) uniform average
         if ((clean_bits | gen_bits) == 0) gen_bits = (nt_all >= 64) ? ~0ull : ((1ull << nt_all) - 1ull);
+        n_clean = __popcll(clean_bits);
+        nt = n_clean + __popcll(gen_bits);
+    }
+    if constexpr (WSPLIT) {
+        if (MASK_MODE == MASK_NONE) {  // the full tiles, then the ragged one
+            const int full = N / BN;
+            clean_bits = full >= 64 ? ~0ull : ((1ull << full) - 1ull);
+            gen_bits = (N % BN) != 0 ? 1ull << full : 0ull;
+        }
+        const uint64_t mine = 0x1111111111111111ull << wave;  // tiles t with t % 4 == wave
+        clean_bits &= mine;
+        gen_bits &= mine;
         n_clean = __popcll(clean_bits);
         nt = n_clean + __popcll(gen_bits);
     }
@@ -429,6 +471,12 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     // ROUTE: how a matrix mask is read (0 = element by element, 1 = prefetched 16-bit vectors, 2 = prefetched fp32
     // vectors); a compile-time choice so that the tile body carries no branches for it
     // EDGE: the tile may hold keys past the last one or beyond the causal diagonal of some row of the workgroup
+    // publishes a stage: to the workgroup, or — WSPLIT, where a stage belongs to one wave, whose LDS operations execute in
+    // program order — only to the compiler
+    auto stage_sync = [&]() __attribute__((always_inline)) {
+        if constexpr (WSPLIT) __builtin_amdgcn_wave_barrier();
+        else __syncthreads();
+    };
     auto tile_step = [&](auto general_c, auto stage_c, auto route_c, auto edge_c) __attribute__((always_inline)) {
         constexpr bool GENERAL = decltype(general_c)::value;
         constexpr int ST = decltype(stage_c)::value;
@@ -442,9 +490,9 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         constexpr bool LATE_DMA = GENERAL && (MASK_MODE == MASK_MATRIX) && ROUTE < 3;
         if (!LATE_DMA) dma(tile_next, ST ^ 1);
         float bias_next = 0.0f;
-        if (GENERAL && tid < BN) bias_next = key_bias(tile_next);
+        if (GENERAL && ktid < BN) bias_next = key_bias(tile_next);
 
-        const unsigned char *sb = smem + ST * STAGE;
+        const unsigned char *sb = smem + wave_lds + ST * STAGE;
         // a wave whose 32 rows all lie above a causal tile has nothing to compute in it
         if (!(GENERAL && CAUSAL && n0 > m_wave0 + 31 + p.causal_off)) {
             // ---- Sᵀ = K · Qᵀ, relative to the row's reference
@@ -620,20 +668,21 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
             if (ROUTE >= 3) mask_take(route_c, min(tile_next + 1, nt - 1));  // matrix masks walk the tiles in order
             else mask_issue(route_c, tile_next);
         }
-        if (GENERAL && tid < BN)
-            *reinterpret_cast<float *>(smem + (ST ^ 1) * STAGE + K_BYTES + V_BYTES + tid * 4) = bias_next;
-        __syncthreads();
+        if (GENERAL && ktid < BN)
+            *reinterpret_cast<float *>(smem + wave_lds + (ST ^ 1) * STAGE + K_BYTES + V_BYTES + ktid * 4) = bias_next;
+        stage_sync();
         t_cur = t_nxt;
         t_nxt = next_tile(t_nxt);
     };
 
     if (nt > 0) {
-        if (t_cur != 0) dma(t_cur, 0);
-        if (n_clean == 0 && tid < BN) *reinterpret_cast<float *>(smem + K_BYTES + V_BYTES + tid * 4) = key_bias(t_cur);
+        if (t_cur != t_first) dma(t_cur, 0);
+        if (n_clean == 0 && ktid < BN)
+            *reinterpret_cast<float *>(smem + wave_lds + K_BYTES + V_BYTES + ktid * 4) = key_bias(t_cur);
         kv8_commit(0);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // everything issued so far (Q fragments included) has landed
-    __syncthreads();
+    stage_sync();
 
     // clean tiles in pairs over the two stages; an odd one leaves the general tiles starting in stage 1
     int idx = 0;
@@ -648,9 +697,9 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     }
     if (idx < nt) {
         if (n_clean > 0) {  // the additive terms of the first general tile
-            if (tid < BN)
-                *reinterpret_cast<float *>(smem + (odd_clean ? STAGE : 0) + K_BYTES + V_BYTES + tid * 4) = key_bias(t_cur);
-            __syncthreads();
+            if (ktid < BN)
+                *reinterpret_cast<float *>(smem + wave_lds + (odd_clean ? STAGE : 0) + K_BYTES + V_BYTES + ktid * 4) = key_bias(t_cur);
+            stage_sync();
         }
         auto general_tiles = [&](auto route_c) __attribute__((always_inline)) {
             constexpr int ROUTE = decltype(route_c)::value;
@@ -695,6 +744,61 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
         else general_tiles(IntC<0>());
     }
 
+    if constexpr (WSPLIT) {
+        // ---- the four waves hold partial results for the SAME 32 rows, each relative to a reference of its own: the
+        // row's exponent reference if the wave has seen an ordinary score (class 2), the reference of its masked scores
+        // if it has only seen those (class 1), nothing (class 0).  As inside a wave, ordinary keys discard masked ones.
+        // Every wave leaves its triple in its own (now idle) stages; wave w then merges accumulator registers
+        // 8 w .. 8 w + 7 of all four — 8 consecutive features of the row — and stores them.
+        constexpr int XO = 32 * 64;  // floats of an accumulator image: [register][lane]
+        float *mine = reinterpret_cast<float *>(smem + wave_lds);
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) mine[(d * 16 + v) * 64 + lane] = o_acc[d][v];
+        mine[XO + lane] = fresh ? m_masked : m_i;
+        mine[XO + 64 + lane] = halves32_sum(l_i);
+        mine[XO + 128 + lane] = !fresh ? 2.0f : (m_masked > -INFINITY ? 1.0f : 0.0f);
+        __syncthreads();
+        float ref[4], sum[4], cls[4];
+        float top = 0.0f;
+#pragma unroll
+        for (int z = 0; z < 4; ++z) {
+            const float *part = reinterpret_cast<const float *>(smem + z * (2 * STAGE));
+            ref[z] = part[XO + lane];
+            sum[z] = part[XO + 64 + lane];
+            cls[z] = part[XO + 128 + lane];
+            top = fmaxf(top, cls[z]);
+        }
+        float m_all = -INFINITY;
+#pragma unroll
+        for (int z = 0; z < 4; ++z)
+            if (cls[z] == top) m_all = fmaxf(m_all, ref[z]);
+        float wgt[4], l_all = 0.0f;
+#pragma unroll
+        for (int z = 0; z < 4; ++z) {
+            wgt[z] = (cls[z] == top && top > 0.0f) ? __builtin_amdgcn_exp2f(ref[z] - m_all) : 0.0f;
+            l_all = fmaf(wgt[z], sum[z], l_all);
+        }
+        const float inv = 1.0f / l_all;
+        float r[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float a = 0.0f;
+#pragma unroll
+            for (int z = 0; z < 4; ++z)
+                a = fmaf(wgt[z], reinterpret_cast<const float *>(smem + z * (2 * STAGE))[(8 * wave + e) * 64 + lane], a);
+            r[e] = a * inv;
+        }
+        if (my_m < M) {
+            // registers 8 w .. 8 w + 7 = block d = w / 2, elements 8 (w % 2) ..: features 32 d + 16 lh + 8 (w % 2) .. + 7
+            u32x4 pk;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) pk[j] = pack2<T>(r[2 * j], r[2 * j + 1]);
+            *reinterpret_cast<u32x4 *>(op + (int64_t)my_m * p.os[2] + (wave >> 1) * 32 + lh * 16 + (wave & 1) * 8) = pk;
+        }
+        return;
+    }
     // ---- normalise and store: lane holds features 32 d + 16 lh + (0..15) of row my_m
     const float l_tot = halves32_sum(l_i);
     const float inv_l = 1.0f / l_tot;
@@ -797,6 +901,24 @@ static void launch_stream(const AttnParams &p, int mask_mode, bool causal, hipSt
         else KERNL_ATTN_LAUNCH(MASK_MATRIX, false);
     }
 #undef KERNL_ATTN_LAUNCH
+}
+
+// small grids, head size 64: 32-row workgroups whose waves split the key tiles (the kernel's WSPLIT form)
+template <typename T>
+static void launch_stream_wsplit(AttnParams p, int mask_mode, hipStream_t st) {
+    constexpr int LDS_BYTES = 8 * (2 * 64 * 128 + 64 * 4);  // 4 waves x 2 stages of a K tile, a V tile and 64 per-key terms
+    p.nq_tiles = (p.M + 31) / 32;
+    dim3 grid((unsigned)(p.B * p.H * p.nq_tiles)), block(256);
+    auto k_none = attention_stream_kernel<T, 64, 1, MASK_NONE, false, false, true>;
+    auto k_vec = attention_stream_kernel<T, 64, 1, MASK_VECTOR, false, false, true>;
+    static bool attr_done = false;  // benign race: the attribute calls are idempotent
+    if (!attr_done) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(k_none), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(k_vec), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        attr_done = true;
+    }
+    if (mask_mode == MASK_NONE) hipLaunchKernelGGL(k_none, grid, block, LDS_BYTES, st, p);
+    else hipLaunchKernelGGL(k_vec, grid, block, LDS_BYTES, st, p);
 }
 
 // one-byte keys and values: fp16 queries, no mask or a per-key mask
@@ -915,6 +1037,21 @@ static int attention_entry(const void *q, const void *k, const void *v, void *ou
         if (D == 64) launch_stream_kv8<64>(p, mask_mode, causal, st);
         else launch_stream_kv8<128>(p, mask_mode, causal, st);
         return check_launch("attention (mfma, fp8 keys/values)");
+    }
+    // Small grids (BERT-base at batch 1: 12 heads x 4 query tiles on 256 CUs, each walking all key tiles): 32-row
+    // workgroups whose four waves split the key tiles, where that still is a single round of workgroups (one per CU:
+    // 130 KB of LDS) and every wave gets a tile.  Measured over 4 .. 64 heads x 64 .. 1536 rows x 256 .. 2048 keys: ahead of
+    // both other kernels wherever the grid is at most 256 workgroups ([1,12,512,64]: 9.8 -> 7.5 us, [1,16,512,2048]:
+    // 28.0 -> 15.1), behind from the second round on.  (Hook: variant 5 takes this form wherever it applies, 3 and 4 never.)
+    {
+        const int64_t wgs32 = B * H * ((M + 31) / 32);
+        const bool applies = mfma_ok && D == 64 && !causal && mask_mode != MASK_MATRIX && N <= 64 * 64;
+        const bool pays = N >= 256 && wgs32 <= 224;  // (at 256 the pipelined kernel, which takes such grids next, draws level)
+        if (applies && g_attention_variant != 3 && g_attention_variant != 4 && (pays || g_attention_variant == 5)) {
+            if (dtype == KERNL_F16) launch_stream_wsplit<f16>(p, mask_mode, st);
+            else launch_stream_wsplit<bf16>(p, mask_mode, st);
+            return check_launch("attention (mfma, key tiles split over waves)");
+        }
     }
     // the software-pipelined kernel takes long key sequences of what it covers (hook: variant 3 keeps everything on the
     // streaming kernel, variant 4 sends everything the pipelined kernel covers to it)

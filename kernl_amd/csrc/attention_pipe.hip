@@ -804,7 +804,12 @@ bool launch_attention_pipe(const AttnParams &p, int D, int dtype, int mask_mode,
     if (mask_mode == MASK_MATRIX) return false;
     if (mask_mode == MASK_VECTOR && (causal || p.N > kPipeMaxMaskKeys)) return false;
     if (((int64_t)p.M + 128) * p.qs[2] >= (1ll << 30)) return false;  // the query rows are fetched through 32-bit byte offsets
-    if (!force && p.N < kPipeMinKeys) return false;
+    // From kPipeMinKeys keys on, and for SMALL grids (at most one 128-query item per CU) from 256 keys on: there the
+    // streaming kernel has no other workgroup on the CU to fill a wave's dependent phases with, and this kernel's own
+    // overlap is worth 10-16 % (head size 64, [1,64,512,64]: 10.6 -> 9.3 us, [1,32,512,768]: 13.0 -> 10.2; with 512 items 4 %,
+    // beyond that it ties or loses, as at BASELINE config 1).
+    const bool small_grid = D == 64 && !causal && p.N >= 256 && (int64_t)p.B * p.H * ((p.M + 127) / 128) <= 256;
+    if (!force && p.N < kPipeMinKeys && !small_grid) return false;
     // Head size 128 runs one workgroup per CU here and is no faster per tile than the streaming kernel (both sit at the
     // chip's power limit); what it wins is BALANCE when a causal problem has few (batch, head) pairs: a persistent
     // workgroup pairs long and short query tiles, where the streaming kernel's grid is one round of unequal workgroups

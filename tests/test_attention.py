@@ -14,13 +14,16 @@ from oracle import attention_oracle
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["auto", "streaming", "pipelined"])
+@pytest.fixture(autouse=True, params=["auto", "streaming", "pipelined", "split"])
 def attention_kernel(request):
-    """Every case runs three times: with the library's own choice between its two MFMA kernels, with the streaming
-    kernel forced, and with the software-pipelined kernel forced wherever it applies (head size 64; no mask, per-key
-    mask or causal) — by default that kernel only takes 1024 keys or more, which few of the shapes here have."""
+    """Every case runs four times: with the library's own choice between its MFMA kernels, with the streaming kernel
+    forced, with the software-pipelined kernel forced wherever it applies (head size 64; no mask, per-key mask or
+    causal) — by default that kernel only takes 1024 keys or more, which few of the shapes here have — and with the
+    streaming kernel's small-grid form (32-row workgroups whose waves split the key tiles) forced wherever it applies
+    (head size 64, non-causal, no mask or a per-key mask, up to 4096 keys), whatever the grid: one tile for four waves,
+    ragged tiles, rows beyond M, fully masked rows and tiles all go through its merge."""
     lib = _lib.load()
-    lib.kernl_attention_set_variant({"auto": 0, "streaming": 3, "pipelined": 4}[request.param])
+    lib.kernl_attention_set_variant({"auto": 0, "streaming": 3, "pipelined": 4, "split": 5}[request.param])
     yield request.param
     lib.kernl_attention_set_variant(0)
 
