@@ -31,7 +31,10 @@ extern "C" {
  *   kernl_attention_set_variant  0 = heuristic; register budget of the head-size-64 streaming attention kernel: 1 = built
  *                                for 3 waves/SIMD, 2 = built for 2 waves/SIMD; 3 = streaming kernel for every shape,
  *                                4 = software-pipelined kernel wherever it applies (head size 64; no mask, a per-key
- *                                mask of at most 2048 keys, or causal), also below 1024 keys.
+ *                                mask of at most 2048 keys, or causal), also below 1024 keys and on large grids;
+ *                                5 = the small-grid form of the streaming kernel (32-row workgroups whose waves split
+ *                                the key tiles) wherever it applies (head size 64, non-causal, no mask or a per-key
+ *                                mask, at most 4096 keys), whatever the grid.
  */
 void kernl_linear_force_tile(int which);
 void kernl_attention_force_scalar(int on);
