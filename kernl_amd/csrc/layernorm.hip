@@ -349,10 +349,9 @@ __global__ void __launch_bounds__(256) add_rms_stats_kernel(const T *__restrict_
     const vec8 *bp = b != nullptr ? reinterpret_cast<const vec8 *>(b + (int64_t)row * b_rs) : nullptr;
     vec8 *sp = b != nullptr ? reinterpret_cast<vec8 *>(sum + (int64_t)row * sum_rs) : nullptr;
     float sq = 0.0f;
-    for (int c = lane; c < N / 8; c += 64) {
-        vec8 v = ap[c];
+    const int chunks = N / 8;
+    auto take = [&](int c, vec8 v, vec8 w) __attribute__((always_inline)) {
         if (bp != nullptr) {
-            const vec8 w = bp[c];
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] = from_float<T>(to_float(v[e]) + to_float(w[e]));
             sp[c] = v;
@@ -362,7 +361,21 @@ __global__ void __launch_bounds__(256) add_rms_stats_kernel(const T *__restrict_
             const float f = to_float(v[e]);
             sq = fmaf(f, f, sq);
         }
+    };
+    // four chunks of either operand in flight per lane (a 4096-wide row is two such rounds)
+    int c = lane;
+    for (; c + 192 < chunks; c += 256) {
+        vec8 v[4], w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = ap[c + 64 * i];
+        if (bp != nullptr) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w[i] = bp[c + 64 * i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) take(c + 64 * i, v[i], w[i]);
     }
+    for (; c < chunks; c += 64) take(c, ap[c], bp != nullptr ? bp[c] : vec8{});
     sq = wave_sum(sq);
     if (lane == 0) rstd[row] = rsqrtf(sq / (float)N + eps);
 }
