@@ -186,7 +186,7 @@ def test_fully_masked_row_is_finite_uniform_average():
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("kind", ["all_very_negative", "growing", "shrinking", "first_tiles_masked", "huge_then_small",
+@pytest.mark.parametrize("kind", ["all_very_negative", "growing", "shrinking", "first_tiles_masked", "huge_then_small", "small_then_huge",
                                   "half_min_bias"])
 def test_softmax_reference_moves_with_the_scores(kind, dtype, close):
     """The kernel keeps scores relative to a per-row exponent reference that moves lazily: up when a score exceeds it
@@ -220,6 +220,11 @@ def test_softmax_reference_moves_with_the_scores(kind, dtype, close):
         mask[:, :, 7::16, :] = -65504.0
     elif kind == "huge_then_small":
         k[:, :, 5, :] = q[:, :, 40, :] * 4.0      # one dominant key in the first tile for row 40 (and large for others)
+    elif kind == "small_then_huge":
+        # a dominant key in the LAST tile (a later clean tile of its wave in the small-grid form too): row 40's score there
+        # is ~46 octaves above everything in its first tile, so steps that trust the first tile's reference overflow 16
+        # bits and the tiles have to be walked again in full
+        k[:, :, 300, :] = q[:, :, 40, :] * 4.0
     q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
     out = _run(q, k, v, 0.125, False, mask)
     ref = attention_oracle(q, k, v, 0.125, False, mask)
