@@ -333,15 +333,14 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     auto next_tile = [&](int last) __attribute__((always_inline)) -> int {
         int t;
         if (use_list) {
-            if (clean_bits != 0) {
-                t = __builtin_ctzll(clean_bits);
-                clean_bits &= clean_bits - 1;
-            } else if (gen_bits != 0) {
-                t = __builtin_ctzll(gen_bits);
-                gen_bits &= gen_bits - 1;
-            } else {
-                t = last;
-            }
+            // (value selects on purpose: written as "clear the lowest bit of whichever set is not empty" the two sets end
+            // up behind a selected address, i.e. in scratch memory)
+            const bool from_clean = clean_bits != 0;
+            const uint64_t set = from_clean ? clean_bits : gen_bits;
+            const uint64_t rest = set & (set - 1);
+            t = set != 0 ? __builtin_ctzll(set) : last;
+            clean_bits = from_clean ? rest : clean_bits;
+            gen_bits = from_clean ? gen_bits : rest;
         } else {
             t = min(order_pos, nt - 1);
         }
