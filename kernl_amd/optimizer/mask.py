@@ -54,8 +54,12 @@ _FOLDABLE_FUNCTIONS = {
     operator.add, operator.sub, operator.mul, operator.and_, operator.or_, operator.getitem,
     operator.ge, operator.gt, operator.le, operator.lt, operator.eq, operator.ne,
     torch.add, torch.sub, torch.mul, torch.bitwise_and, torch.bitwise_or,
+    # (the packed-sequence test transformers makes on position ids when no key/value cache is in use: position
+    # differences, a running count of restarts, and a comparison of the counts of query and key)
+    torch.diff, torch.cumsum, torch.eq, torch.ne,
 }
-_FOLDABLE_METHODS = {"new_ones", "new_zeros", "to", "expand", "view", "reshape", "unsqueeze", "squeeze", "bool", "long", "int"}
+_FOLDABLE_METHODS = {"new_ones", "new_zeros", "to", "expand", "view", "reshape", "unsqueeze", "squeeze", "bool", "long", "int",
+                     "cumsum", "diff", "__eq__", "__ne__", "__and__", "__or__", "__ge__", "__gt__", "__le__", "__lt__"}
 _FOLD_LIMIT = 1 << 22  # elements
 
 

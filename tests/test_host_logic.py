@@ -350,7 +350,9 @@ def test_llama_graph_rewrite_and_constant_causal_mask():
     into one GEMM, and the constant causal mask replaced by the kernel's is_causal flag."""
     from transformers import LlamaConfig, LlamaModel
 
-    for attn_impl, fused, mask_idx in (("eager", "attention_wrapper", 6), ("sdpa", "sdpa_wrapper", 3)):
+    # (without a key/value cache transformers also derives a packed-sequence mask from the position ids: constants too)
+    for attn_impl, fused, mask_idx, call_kwargs in (("eager", "attention_wrapper", 6, {}), ("sdpa", "sdpa_wrapper", 3, {}),
+                                                    ("sdpa", "sdpa_wrapper", 3, {"use_cache": False})):
         torch.manual_seed(0)
         cfg = LlamaConfig(num_hidden_layers=2, hidden_size=128, num_attention_heads=2, num_key_value_heads=2,
                           intermediate_size=256, vocab_size=100, rms_norm_eps=1e-5)
@@ -366,7 +368,7 @@ def test_llama_graph_rewrite_and_constant_causal_mask():
         torch._dynamo.reset()
         try:
             with torch.inference_mode():
-                torch._dynamo.optimize(backend, dynamic=False)(model.forward)(input_ids=torch.randint(0, 100, (1, 16)))
+                torch._dynamo.optimize(backend, dynamic=False)(model.forward)(input_ids=torch.randint(0, 100, (1, 16)), **call_kwargs)
         except Exception:
             pass
         assert len(graphs) == 1
