@@ -260,6 +260,21 @@ int kernl_linear_scaled_fwd(const void *x, const void *w, const void *bias, cons
                             int activation, int gated, int dtype, void *stream);
 
 /*
+ * The linear layer of MANY rows with the residual addition that follows it in a transformer layer:
+ *     out = round(x @ w^T + bias) + residual
+ * (the projection is rounded to the 16-bit type first and the sum once more: bit for bit what kernl_linear_fwd followed
+ * by an addition of the two 16-bit tensors gives).  The reference's fused linear kernel (src/kernl/implementations/
+ * linear_layer.py:92-210) has no residual operand: its models add in eager PyTorch (`hidden_states + input_tensor` in
+ * front of every LayerNorm of the graph in docs/how-to-guides/support-new-model.md:481-520; experimental/llama-v2/llama/
+ * model.py:262-264).  Here the wide tile kernels fetch the residual one 16-row block ahead of the epilogue that adds it,
+ * so the addition costs no pass over memory.  residual: [M, N] of the same dtype with its strides; it must not overlap
+ * out.  No activation.  f16 / bf16, K % 8 == 0, x with unit feature stride and 16-byte aligned rows.
+ */
+int kernl_linear_residual_fwd(const void *x, const void *w, const void *bias, const void *residual, void *out, int64_t M,
+                              int64_t N, int64_t K, const int64_t x_strides[2], const int64_t out_strides[2],
+                              const int64_t residual_strides[2], int dtype, void *stream);
+
+/*
  * Whether kernl_linear_fwd runs M x N x K (16-bit, plain epilogue, x with unit feature stride) on one of its
  * small-problem kernels, and which: 0 = no; otherwise the kernl_linear_force_tile value of the kernel (10 .. 15).  A
  * caller that would otherwise route such a shape to the stream-K or split-K entry points (kernl_linear_fewrow_fwd,
@@ -268,6 +283,15 @@ int kernl_linear_scaled_fwd(const void *x, const void *w, const void *bias, cons
  * autotuner (src/kernl/implementations/linear_layer.py:47-91).
  */
 int kernl_linear_small_kind(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Whether kernl_linear_fwd runs M x N x K (16-bit, plain epilogue) on one of its wide tile kernels, and which: 0 = no,
+ * otherwise the kernl_linear_force_tile value of the kernel (5 .. 8).  kernl_linear_residual_fwd and
+ * kernl_linear_scaled_fwd exist on those kernels only and run them whatever the shape: a caller asks here first and
+ * keeps the separate addition (or normalisation) where another kernel is the faster one.  No counterpart in the
+ * reference (one kernel and an autotuner, src/kernl/implementations/linear_layer.py:47-91).
+ */
+int kernl_linear_wide_kind(int64_t M, int64_t N, int64_t K);
 
 /*
  * kernl_linear_fwd for row counts between the two regimes (129 to a few hundred rows against a few thousand columns),

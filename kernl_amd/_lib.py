@@ -36,6 +36,8 @@ EXPORTED_SYMBOLS = (
     "kernl_linear_w8_fwd",
     "kernl_linear_rms_fwd",
     "kernl_linear_scaled_fwd",
+    "kernl_linear_residual_fwd",
+    "kernl_linear_wide_kind",
     "kernl_linear_decode_fwd",
     "kernl_linear_splitk_workspace_bytes",
     "kernl_linear_splitk_fwd",
@@ -144,10 +146,14 @@ def load() -> ctypes.CDLL:
     )
     lib.kernl_linear_scaled_fwd.restype = ctypes.c_int
     lib.kernl_linear_scaled_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int] * 3 + [_vp]
+    lib.kernl_linear_residual_fwd.restype = ctypes.c_int
+    lib.kernl_linear_residual_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, _vp]
     lib.kernl_add_rms_stats_fwd.restype = ctypes.c_int
     lib.kernl_add_rms_stats_fwd.argtypes = [_vp] * 4 + [_i64] * 5 + [ctypes.c_float, ctypes.c_int, _vp]
     lib.kernl_linear_small_kind.restype = ctypes.c_int
     lib.kernl_linear_small_kind.argtypes = [_i64] * 3
+    lib.kernl_linear_wide_kind.restype = ctypes.c_int
+    lib.kernl_linear_wide_kind.argtypes = [_i64] * 3
     lib.kernl_linear_glu_fwd.restype = ctypes.c_int
     lib.kernl_linear_glu_fwd.argtypes = [_vp] * 4 + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int, ctypes.c_int, _vp]
     lib.kernl_layernorm_fwd.restype = ctypes.c_int
@@ -325,6 +331,11 @@ def linear_small_kind(M: int, N: int, K: int) -> int:
     return int(load().kernl_linear_small_kind(int(M), int(N), int(K)))
 
 
+def linear_wide_kind(M: int, N: int, K: int) -> int:
+    """Non-zero when `kernl_linear_fwd` runs a plain 16-bit M x N x K problem on one of its wide tile kernels."""
+    return int(load().kernl_linear_wide_kind(int(M), int(N), int(K)))
+
+
 def linear_fwd(x2d, weight, bias, out2d, act_in2d, activation: int) -> None:
     _require_gpu(x2d, weight, bias, out2d, act_in2d)
     M, K = x2d.shape
@@ -417,6 +428,24 @@ def linear_scaled_fwd(x2d, weight, bias, row_scale, out2d, activation: int, gate
             DTYPE_CODE[x2d.dtype], _stream(x2d),
         )
     _check(st, "kernl_linear_scaled_fwd")
+
+
+def linear_residual_fwd(x2d, weight, bias, residual2d, out2d) -> None:
+    """out = round(x @ w^T + bias) + residual in the epilogue of the wide tile kernels (`linear_scaled_supported` says
+    which x and w they take; residual and out are [M, N] of x's dtype and must not overlap)."""
+    _require_gpu(x2d, weight, bias, residual2d, out2d)
+    M, K = x2d.shape
+    N = out2d.shape[1]
+    if residual2d.shape != out2d.shape or residual2d.dtype != x2d.dtype or out2d.dtype != x2d.dtype:
+        raise ValueError("residual and out must have shape [M, N] and the dtype of x")
+    lib = load()
+    with torch.cuda.device(x2d.device):
+        st = lib.kernl_linear_residual_fwd(
+            x2d.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(), residual2d.data_ptr(),
+            out2d.data_ptr(), M, N, K, _arr(x2d.stride()), _arr(out2d.stride()), _arr(residual2d.stride()),
+            DTYPE_CODE[x2d.dtype], _stream(x2d),
+        )
+    _check(st, "kernl_linear_residual_fwd")
 
 
 def add_rms_stats_fwd(a2d, b2d, sum2d, rstd, eps: float) -> None:

@@ -61,6 +61,14 @@ extern "C" int kernl_linear_small_kind(int64_t M, int64_t N, int64_t K) {
     return kernl::small_problem_kind(M, N, K);
 }
 
+extern "C" int kernl_linear_wide_kind(int64_t M, int64_t N, int64_t K) {
+    using namespace kernl;
+    if (M <= 64 || N <= 0 || K <= 0 || K % 8 != 0 || M > INT32_MAX || N > INT32_MAX || K >= (1 << 22)) return 0;
+    if (small_problem_kind(M, N, K) != 0) return 0;
+    const int pick = pick_tile((int)M, (int)N, (int)K, false);
+    return pick >= 5 && pick <= 8 ? pick : 0;
+}
+
 // Tuning hook used by the sweep tests: force a tile shape (0 restores the heuristic).
 extern "C" void kernl_linear_force_tile(int which) { kernl::g_linear_force_tile = which; }
 
@@ -230,6 +238,45 @@ extern "C" int kernl_linear_scaled_fwd(const void *x, const void *w, const void 
     else if (pick == 7) run_wide_half(a, dtype, 256);
     else run_wide_half(a, dtype, 192);
     return check_launch("scaled linear");
+}
+
+extern "C" int kernl_linear_residual_fwd(const void *x, const void *w, const void *bias, const void *residual, void *out,
+                                         int64_t M, int64_t N, int64_t K, const int64_t x_strides[2],
+                                         const int64_t out_strides[2], const int64_t residual_strides[2], int dtype,
+                                         void *stream) {
+    using namespace kernl;
+    if (x == nullptr || w == nullptr || out == nullptr || residual == nullptr || x_strides == nullptr ||
+        out_strides == nullptr || residual_strides == nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear + residual: x, w, residual, out and their strides must not be NULL");
+    if (M < 0 || N <= 0 || K <= 0)
+        return set_error(KERNL_ERR_INVALID_ARG, "linear + residual: bad sizes M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+                         (long long)K);
+    if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear + residual: sizes must fit in 31 bits");
+    if (dtype != KERNL_F16 && dtype != KERNL_BF16)
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear + residual: only f16 and bf16 are supported, got dtype %d", dtype);
+    if (x_strides[1] != 1 || K % 8 != 0 || x_strides[0] % 8 != 0 || !aligned16(x) || !aligned16(w) ||
+        x_strides[0] >= (1 << 22) || K >= (1 << 22))
+        return set_error(KERNL_ERR_UNSUPPORTED, "linear + residual: x must have unit feature stride, 16-byte aligned rows and K "
+                         "a multiple of 8; w a 16-byte aligned base");
+    if (M == 0) return KERNL_OK;
+    LinearArgs a;
+    a.x = x; a.w = w; a.bias = bias; a.out = out; a.act_in = nullptr;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.x_rs = x_strides[0]; a.x_cs = x_strides[1];
+    a.out_rs = out_strides[0]; a.out_cs = out_strides[1];
+    a.ai_rs = 0; a.ai_cs = 0;
+    a.act = KERNL_ACT_NONE;
+    a.st = static_cast<hipStream_t>(stream);
+    a.residual = residual;
+    a.res_rs = residual_strides[0]; a.res_cs = residual_strides[1];
+    // only the wide kernels add a residual (5 / 6: 256-row tiles, 7 / 8: 128-row tiles)
+    const int pick = g_linear_force_tile >= 5 && g_linear_force_tile <= 8 ? g_linear_force_tile : pick_tile(a.M, a.N, a.K, false, true);
+    if (pick == 5) run_wide(a, dtype, 256);
+    else if (pick == 6) run_wide(a, dtype, 192);
+    else if (pick == 7) run_wide_half(a, dtype, 256);
+    else run_wide_half(a, dtype, 192);
+    return check_launch("linear + residual");
 }
 
 extern "C" int kernl_linear_w8_fwd(const void *x, const void *w8, const void *bias, void *out, void *act_in, int64_t M,

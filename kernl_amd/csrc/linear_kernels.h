@@ -497,26 +497,94 @@ __device__ __forceinline__ void wide_row_scale_fetch(const float *__restrict__ r
 }
 
 // NV rounded values of one row -> one 16-, 12- or 8-byte store
-template <typename T, int NV>
-__device__ __forceinline__ void wide_store_row(T *p, const float (&r)[NV]) {
+// (RES: `res` holds the packed residual entries of the same elements; they are added to the ROUNDED values and the sum
+// is rounded again — what `round(linear) + residual` gives as an addition of two 16-bit tensors)
+template <typename T, int NV, bool RES = false, bool PACKED = true>
+__device__ __forceinline__ void wide_store_row(T *p, const float (&r)[NV], const uint32_t (&res)[NV / 2]) {
     static_assert(NV == 8 || NV == 6 || NV == 4, "values per lane and row");
     uint32_t w[NV / 2];
 #pragma unroll
-    for (int e = 0; e < NV / 2; ++e) w[e] = pack2<T>(r[2 * e], r[2 * e + 1]);
+    for (int e = 0; e < NV / 2; ++e) {
+        w[e] = pack2<T>(r[2 * e], r[2 * e + 1]);
+        if constexpr (RES) {
+            if constexpr (std::is_same<T, f16>::value && PACKED) {
+                typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+                w[e] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, w[e]) + __builtin_bit_cast(half2_t, res[e]));
+            } else if constexpr (std::is_same<T, f16>::value) {
+                typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+                const half2_t a = __builtin_bit_cast(half2_t, w[e]), b = __builtin_bit_cast(half2_t, res[e]);
+                w[e] = pack2<T>((float)a[0] + (float)b[0], (float)a[1] + (float)b[1]);
+            } else {
+                // bf16 -> fp32 is a shift
+                const float lo = __builtin_bit_cast(float, w[e] << 16) + __builtin_bit_cast(float, res[e] << 16);
+                const float hi = __builtin_bit_cast(float, w[e] & 0xFFFF0000u) + __builtin_bit_cast(float, res[e] & 0xFFFF0000u);
+                w[e] = pack2<T>(lo, hi);
+            }
+        }
+    }
     if constexpr (NV == 8) *reinterpret_cast<u32x4 *>(p) = u32x4{w[0], w[1], w[2], w[3]};
     else if constexpr (NV == 6) *reinterpret_cast<u32x3 *>(p) = u32x3{w[0], w[1], w[2]};
     else *reinterpret_cast<u32x2 *>(p) = u32x2{w[0], w[1]};
 }
 
-// Epilogue of m-block IB (16 rows) of a wave of the wide kernels: out = act(sum * row factor + bias).  Blocks that lie inside the matrix, with contiguous
-// 16-byte aligned output rows and no pre-activation side output, run a straight-line path.
-template <typename T, int ACT, int IB, int NBN, int NBM = 8, bool SCALED = false>
+// Optional residual of the plain wide kernels: out = act(...) + residual[m, n], a matrix of the output's shape and dtype
+// (the `hidden + projection(...)` of a transformer layer; no counterpart in the reference, whose models add in eager
+// PyTorch).  `vec_ok`: unit column stride, rows that keep the lane's 16- or 12-byte pieces aligned.
+struct WideResidual {
+    const void *ptr = nullptr;
+    int64_t rs = 0, cs = 0;
+    int vec_ok = 0;
+};
+// The lane's residual entries of one 16-row block — rows m_first .. m_first + 3, its NBN consecutive columns from n on —
+// as packed 16-bit values (zeros outside the matrix).  Issued one block ahead of the epilogue that adds them (block 0:
+// in front of the tile's main loop, like the bias), so that no epilogue waits for a memory round trip.
+template <typename T, int NBN>
+__device__ __forceinline__ void wide_residual_fetch(const WideResidual &res, int m_first, int n, int M, int N,
+                                                    uint32_t (&raw)[4][NBN / 2]) {
+    const T *base = static_cast<const T *>(res.ptr);
+    if (res.vec_ok && m_first + 4 <= M && n + NBN <= N) {
+        const T *p = base + (int64_t)m_first * res.rs + n;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            if constexpr (NBN == 8) {
+                const u32x4 t = *reinterpret_cast<const u32x4 *>(p + v * res.rs);
+                raw[v][0] = t[0], raw[v][1] = t[1], raw[v][2] = t[2], raw[v][3] = t[3];
+            } else {
+                const u32x3 t = *reinterpret_cast<const u32x3 *>(p + v * res.rs);
+                raw[v][0] = t[0], raw[v][1] = t[1], raw[v][2] = t[2];
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+#pragma unroll
+        for (int e = 0; e < NBN / 2; ++e) raw[v][e] = 0u;
+#pragma unroll
+        for (int c = 0; c < NBN; ++c)
+            if (m_first + v < M && n + c < N)
+                raw[v][c >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, base[(int64_t)(m_first + v) * res.rs + (int64_t)(n + c) * res.cs]) << (16 * (c & 1));
+    }
+}
+
+template <typename T, int NV>
+__device__ __forceinline__ void wide_store_row(T *p, const float (&r)[NV]) {
+    const uint32_t none[NV / 2] = {};
+    wide_store_row<T, NV, false>(p, r, none);
+}
+
+// Epilogue of m-block IB (16 rows) of a wave of the wide kernels: out = act(sum * row factor + bias) (+ residual, RES:
+// added to the ROUNDED value and rounded again, as a separate addition of two 16-bit tensors would).  Blocks that lie
+// inside the matrix, with contiguous 16-byte aligned output rows and no pre-activation side output, run a straight-line path.
+template <typename T, int ACT, int IB, int NBN, int NBM = 8, bool SCALED = false, bool RES = false>
 __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_wave, int n_wave, int l16, int g,
                                               T *__restrict__ out, T *__restrict__ act_in, int M, int N,
                                               int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs,
-                                              int out_vec_ok, int ai_vec_ok, const float (&bf)[NBN], const float (&rs)[4]) {
+                                              int out_vec_ok, int ai_vec_ok, const float (&bf)[NBN], const float (&rs)[4],
+                                              const uint32_t (&rres)[4][NBN / 2]) {
     constexpr bool GATED = (ACT & kGluBit) != 0;
     static_assert(!GATED || NBN == 8, "gated epilogues: four gate and four value blocks");
+    static_assert(!RES || !GATED, "the residual form is for plain epilogues");
     constexpr int BASE = ACT & (kGluBit - 1), NV = WideLane<GATED, NBN>::NV;
     const int n = WideLane<GATED, NBN>::col(n_wave, l16);
     const int n_total = GATED ? N >> 1 : N;  // output columns
@@ -540,7 +608,8 @@ __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_
             sums(v, r, value);
 #pragma unroll
             for (int c = 0; c < NV; ++c) r[c] = GATED ? apply_act16(r[c], BASE) * value[c] : apply_act16(r[c], ACT);
-            wide_store_row<T, NV>(p + v * out_rs, r);
+            if constexpr (RES) wide_store_row<T, NV, true>(p + v * out_rs, r, rres[v]);
+            else wide_store_row<T, NV>(p + v * out_rs, r);
         }
         return;
     }
@@ -562,25 +631,41 @@ __device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_
 #pragma unroll
         for (int c = 0; c < NV; ++c) r[c] = GATED ? apply_act16(r[c], BASE) * value[c] : apply_act16(r[c], ACT);
         if (out_vec_ok && n + NV <= n_total) {
-            wide_store_row<T, NV>(out + (int64_t)m * out_rs + n, r);
+            if constexpr (RES) wide_store_row<T, NV, true>(out + (int64_t)m * out_rs + n, r, rres[v]);
+            else wide_store_row<T, NV>(out + (int64_t)m * out_rs + n, r);
         } else {
 #pragma unroll
-            for (int c = 0; c < NV; ++c)
-                if (n + c < n_total) out[(int64_t)m * out_rs + (int64_t)(n + c) * out_cs] = from_float<T>(r[c]);
+            for (int c = 0; c < NV; ++c) {
+                if (n + c >= n_total) continue;
+                T o = from_float<T>(r[c]);
+                if constexpr (RES) o = from_float<T>(to_float(o) + to_float(__builtin_bit_cast(T, (uint16_t)(rres[v][c >> 1] >> (16 * (c & 1))))));
+                out[(int64_t)m * out_rs + (int64_t)(n + c) * out_cs] = o;
+            }
         }
     }
+}
+
+template <typename T, int ACT, int IB, int NBN, int NBM = 8, bool SCALED = false>
+__device__ __forceinline__ void wide_epilogue(f32x4_acc (&acc)[NBM][NBN], int m_wave, int n_wave, int l16, int g,
+                                              T *__restrict__ out, T *__restrict__ act_in, int M, int N,
+                                              int64_t out_rs, int64_t out_cs, int64_t ai_rs, int64_t ai_cs,
+                                              int out_vec_ok, int ai_vec_ok, const float (&bf)[NBN], const float (&rs)[4]) {
+    const uint32_t none[4][NBN / 2] = {};
+    wide_epilogue<T, ACT, IB, NBN, NBM, SCALED, false>(acc, m_wave, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs,
+                                                       ai_cs, out_vec_ok, ai_vec_ok, bf, rs, none);
 }
 
 // W8: the weight is stored as one byte per element (fp8 e5m2, the upper byte of the fp16 encoding).  Its tile travels
 // HBM -> LDS as bytes (half the loads, 64-byte rows, chunks swizzled for 8-byte reads), a fragment is read as 8 bytes
 // and widened by four byte-permutes two read slots later, all in the shadow of the MFMAs; everything else is unchanged.
 // SCALED: the finished sums are multiplied by a factor per row of x (row_scale, fp32 [M]) before the bias is added.
-template <typename T, int ACT, int NBN, bool W8 = false, bool SCALED = false>
+// RES: a residual matrix is added to the rounded results (plain epilogues only).
+template <typename T, int ACT, int NBN, bool W8 = false, bool SCALED = false, bool RES = false>
 __global__ void __launch_bounds__(256, 1)
 linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias, T *__restrict__ out,
                    T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs, int64_t out_cs,
                    int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok, int ai_vec_ok,
-                   int bias_vec_ok, const float *__restrict__ row_scale) {
+                   int bias_vec_ok, const float *__restrict__ row_scale, const WideResidual residual) {
     typedef typename Vec8<T>::type vec8;
     constexpr bool GATED = (ACT & kGluBit) != 0;
     static_assert(NBN == 8 || (NBN == 6 && !GATED), "256 or 192 columns per tile; gated epilogues need 256");
@@ -827,6 +912,17 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         wide_bias_fetch<T, GATED, NBN>(bias, n_wave, l16, N, bias_vec_ok, braw);
         float rsc[SCALED ? NB : 1][4];
         if constexpr (SCALED) wide_row_scale_fetch<NB>(row_scale, m0 + wave_m * 128 + 4 * g, M, rsc);
+        // the residual entries of the first 16-row blocks too; those of block I + RD - 1 are requested in front of block
+        // I's epilogue (a ring of RD blocks: inside a model the residual was written several hundred MB of traffic ago
+        // and comes from HBM, two or three block epilogues away)
+        constexpr int RD = RES ? (NBN == 6 ? 4 : 3) : 1;
+        uint32_t rres[RD][4][NBN / 2];
+        const int n_lane = WideLane<GATED, NBN>::col(n_wave, l16);
+        if constexpr (RES) {
+#pragma unroll
+            for (int i = 0; i < RD - 1; ++i)
+                wide_residual_fetch<T, NBN>(residual, m0 + wave_m * 128 + 16 * i + 4 * g, n_lane, M, N, rres[i]);
+        }
         // (no zeroing of the accumulators: the first k-step of the tile writes them)
         k_tile(IntC<0>(), landed, BoolC<true>());
         advance_load();
@@ -852,8 +948,10 @@ linear_wide_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__
         // one call per 16-row block: each stays small enough for the compiler to unroll completely, so the
         // accumulators are only ever indexed by constants and never leave the register file
 #define KERNL_WIDE_EPILOGUE(I)                                                                                         \
-    wide_epilogue<T, ACT, I, NBN, 8, SCALED>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs, ai_rs,  \
-                                             ai_cs, out_vec_ok, ai_vec_ok, bf, rsc[SCALED ? I : 0])
+    if constexpr (RES && I + RD - 1 < 8)                                                                               \
+        wide_residual_fetch<T, NBN>(residual, m0 + wave_m * 128 + 16 * (I + RD - 1) + 4 * g, n_lane, M, N, rres[(I + RD - 1) % RD]); \
+    wide_epilogue<T, ACT, I, NBN, 8, SCALED, RES>(acc, m0 + wave_m * 128, n_wave, l16, g, out, act_in, M, N, out_rs, out_cs,   \
+                                                  ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bf, rsc[SCALED ? I : 0], rres[I % RD])
         KERNL_WIDE_EPILOGUE(0);
         KERNL_WIDE_EPILOGUE(1);
         KERNL_WIDE_EPILOGUE(2);
@@ -891,13 +989,14 @@ __device__ __forceinline__ void half_tile_origin(int t, int tiles_m, int tiles_n
 // SPLIT: blockIdx.y selects one of `splits` ranges of k-tiles; the workgroup leaves its fp32 partial tile in `part`
 // (slot blockIdx.y * tiles + t; per wave and 16 x 16 block 64 lanes x 16 bytes: coalesced, and the same lane reads it
 // back in linear_wide_half_reduce_kernel, which adds the ranges in order and runs the epilogue).
-template <typename T, int ACT, int NBN, bool W8 = false, bool SPLIT = false, bool SCALED = false>
+template <typename T, int ACT, int NBN, bool W8 = false, bool SPLIT = false, bool SCALED = false, bool RES = false>
 __global__ void __launch_bounds__(256, 1)
 linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const T *__restrict__ bias,
                         T *__restrict__ out, T *__restrict__ act_in, int M, int N, int K, int64_t ldx, int64_t out_rs,
                         int64_t out_cs, int64_t ai_rs, int64_t ai_cs, int tiles_m, int tiles_n, int out_vec_ok,
                         int ai_vec_ok, int bias_vec_ok, float *__restrict__ part, int splits,
-                        const float *__restrict__ row_scale) {
+                        const float *__restrict__ row_scale, const WideResidual residual) {
+    static_assert(!RES || !SPLIT, "the split form leaves its epilogue to the reduction launch");
     typedef typename Vec8<T>::type vec8;
     static_assert((ACT & kGluBit) == 0 && (NBN == 8 || NBN == 6), "plain epilogues, 256 or 192 columns");
     constexpr int NBM = 4, BM = 32 * NBM, BN = 32 * NBN, BK = 64, RB = BK * 2, CPR = BK / 8, KSTEPS = BK / 32;
@@ -1114,6 +1213,16 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     if (kt < nk) k_tile(IntC<0>(), kt);
     if (kt + 1 < nk) k_tile(IntC<1>(), kt + 1);
     mfma16_inplace_results_landed(acc);
+    // the residual entries of the wave's four 16-row blocks (one tile per workgroup and a long K: this one round trip
+    // is not worth registers held through the main loop)
+    uint32_t rres_a[4][NBN / 2] = {}, rres_b[4][NBN / 2] = {}, rres_c[4][NBN / 2] = {}, rres_d[4][NBN / 2] = {};
+    const int n_lane = n0 + wave_n * (NBN * 16) + NBN * l16;
+    if constexpr (RES) {
+        wide_residual_fetch<T, NBN>(residual, m0 + wave_m * (NBM * 16) + 4 * g, n_lane, M, N, rres_a);
+        wide_residual_fetch<T, NBN>(residual, m0 + wave_m * (NBM * 16) + 16 + 4 * g, n_lane, M, N, rres_b);
+        wide_residual_fetch<T, NBN>(residual, m0 + wave_m * (NBM * 16) + 32 + 4 * g, n_lane, M, N, rres_c);
+        wide_residual_fetch<T, NBN>(residual, m0 + wave_m * (NBM * 16) + 48 + 4 * g, n_lane, M, N, rres_d);
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): no load may still be writing LDS when the workgroup ends
 
     if constexpr (SPLIT) {
@@ -1131,8 +1240,9 @@ linear_wide_half_kernel(const T *__restrict__ X, const T *__restrict__ W, const 
     wide_bias_fetch<T, false, NBN>(bias, n_wave, l16, N, bias_vec_ok, braw);
     wide_bias_unpack<T, NBN>(braw, bf);
 #define KERNL_HALF_EPILOGUE(I)                                                                                         \
-    wide_epilogue<T, ACT, I, NBN, NBM, SCALED>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs,  \
-                                               out_cs, ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bf, rsc[SCALED ? I : 0])
+    wide_epilogue<T, ACT, I, NBN, NBM, SCALED, RES>(acc, m0 + wave_m * (NBM * 16), n_wave, l16, g, out, act_in, M, N, out_rs, \
+                                                    out_cs, ai_rs, ai_cs, out_vec_ok, ai_vec_ok, bf, rsc[SCALED ? I : 0],  \
+                                                    I == 0 ? rres_a : I == 1 ? rres_b : I == 2 ? rres_c : rres_d)
     KERNL_HALF_EPILOGUE(0);
     KERNL_HALF_EPILOGUE(1);
     KERNL_HALF_EPILOGUE(2);
@@ -1546,7 +1656,21 @@ struct LinearArgs {
     hipStream_t st;
     const SkinnyExtra *extra = nullptr;  // residual / rotation of the few-row kernel (decoding steps)
     const float *row_scale = nullptr;    // fp32 [M] factors of the finished sums (wide kernels only)
+    const void *residual = nullptr;      // [M, N] matrix added to the rounded results (wide kernels, plain epilogue, no activation)
+    int64_t res_rs = 0, res_cs = 0;
 };
+
+template <typename T, int NBN>
+static WideResidual wide_residual_of(const LinearArgs &a) {
+    WideResidual r;
+    r.ptr = a.residual;
+    r.rs = a.res_rs;
+    r.cs = a.res_cs;
+    // 16-byte pieces at columns that are multiples of 8, or 12-byte pieces (4-byte aligned) at multiples of 6
+    r.vec_ok = a.residual != nullptr && a.res_cs == 1 &&
+               (NBN == 8 ? (a.res_rs % 8 == 0 && aligned16(a.residual)) : (a.res_rs % 2 == 0 && (reinterpret_cast<uintptr_t>(a.residual) & 3) == 0));
+    return r;
+}
 
 template <typename T, typename Cfg, int ACT, bool W8 = false>
 static void launch_mfma_act(const LinearArgs &a) {
@@ -1610,9 +1734,9 @@ static void launch_mfma_glu(const LinearArgs &a) {
     }
 }
 
-template <typename T, int ACT, int NBN = 8, bool W8 = false, bool SCALED = false>
+template <typename T, int ACT, int NBN = 8, bool W8 = false, bool SCALED = false, bool RES = false>
 static void launch_wide_act(const LinearArgs &a) {
-    auto kern = linear_wide_kernel<T, ACT, NBN, W8, SCALED>;
+    auto kern = linear_wide_kernel<T, ACT, NBN, W8, SCALED, RES>;
     constexpr int LDS_BYTES = 2 * (256 + 256) * 128;  // two stages
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
@@ -1632,12 +1756,12 @@ static void launch_wide_act(const LinearArgs &a) {
     const int slots = (per_xcd < 32 || ((a.K + 63) / 64) % 2 != 0) ? per_xcd : 32;
     hipLaunchKernelGGL(kern, dim3(slots * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
-                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, a.row_scale);
+                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, a.row_scale, wide_residual_of<T, NBN>(a));
 }
 
-template <typename T, int ACT, int NBN, bool W8 = false, bool SCALED = false>
+template <typename T, int ACT, int NBN, bool W8 = false, bool SCALED = false, bool RES = false>
 static void launch_wide_half_act(const LinearArgs &a) {
-    auto kern = linear_wide_half_kernel<T, ACT, NBN, W8, false, SCALED>;
+    auto kern = linear_wide_half_kernel<T, ACT, NBN, W8, false, SCALED, RES>;
     constexpr int LDS_BYTES = 3 * 16384 + 3 * 32768;  // three stages
     static bool attr_done = false;  // benign race: the attribute call is idempotent
     if (!attr_done) {
@@ -1654,7 +1778,8 @@ static void launch_wide_half_act(const LinearArgs &a) {
     const int bias_vec_ok = bias != nullptr && aligned16(bias);
     hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
-                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, static_cast<float *>(nullptr), 1, a.row_scale);
+                       a.ai_cs, tiles_m, tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, static_cast<float *>(nullptr), 1, a.row_scale,
+                       wide_residual_of<T, NBN>(a));
 }
 
 // Split form of the 128 x 192 kernel for row counts that leave most CUs without a tile (129 to about 700 rows against
@@ -1699,7 +1824,8 @@ static void launch_half_split_act(const LinearArgs &a, const HalfSplitPlan &p, f
     const int bias_vec_ok = bias != nullptr && aligned16(bias);
     hipLaunchKernelGGL(kern, dim3(per_xcd * 8, p.splits), dim3(256), LDS_BYTES, a.st, static_cast<const T *>(a.x),
                        static_cast<const T *>(a.w), bias, out, act_in, a.M, a.N, a.K, a.x_rs, a.out_rs, a.out_cs, a.ai_rs,
-                       a.ai_cs, p.tiles_m, p.tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, part, p.splits, static_cast<const float *>(nullptr));
+                       a.ai_cs, p.tiles_m, p.tiles_n, out_vec_ok, ai_vec_ok, bias_vec_ok, part, p.splits, static_cast<const float *>(nullptr),
+                       WideResidual());
     hipLaunchKernelGGL((linear_wide_half_reduce_kernel<T, ACT, NBN>), dim3(p.tiles_m * p.tiles_n, 4), dim3(256), 0, a.st,
                        part, bias, out, act_in, a.M, a.N, a.out_rs, a.out_cs, a.ai_rs, a.ai_cs, p.tiles_m, p.tiles_n,
                        out_vec_ok, ai_vec_ok, bias_vec_ok, p.splits);
@@ -1719,6 +1845,10 @@ static void launch_half_split(const LinearArgs &a, const HalfSplitPlan &p, float
 
 template <typename T, int NBN>
 static void launch_wide_half(const LinearArgs &a) {
+    if (a.residual != nullptr) {   // (the entry point admits no activation and no per-row factors with a residual)
+        launch_wide_half_act<T, KERNL_ACT_NONE, NBN, false, false, true>(a);
+        return;
+    }
     if (a.row_scale != nullptr) {  // (the entry point admits no activation with per-row factors here)
         launch_wide_half_act<T, KERNL_ACT_NONE, NBN, false, true>(a);
         return;
@@ -1735,6 +1865,10 @@ static void launch_wide_half(const LinearArgs &a) {
 
 template <typename T>
 static void launch_wide192(const LinearArgs &a) {
+    if (a.residual != nullptr) {
+        launch_wide_act<T, KERNL_ACT_NONE, 6, false, false, true>(a);
+        return;
+    }
     if (a.row_scale != nullptr) {
         launch_wide_act<T, KERNL_ACT_NONE, 6, false, true>(a);
         return;
@@ -1751,6 +1885,10 @@ static void launch_wide192(const LinearArgs &a) {
 
 template <typename T>
 static void launch_wide(const LinearArgs &a) {
+    if (a.residual != nullptr) {
+        launch_wide_act<T, KERNL_ACT_NONE, 8, false, false, true>(a);
+        return;
+    }
     if (a.row_scale != nullptr) {  // (the entry point admits SiLU gates and plain sums with per-row factors)
         if (a.act & kGluBit) launch_wide_act<T, kGluBit | KERNL_ACT_SILU, 8, false, true>(a);
         else launch_wide_act<T, KERNL_ACT_NONE, 8, false, true>(a);

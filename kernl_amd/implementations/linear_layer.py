@@ -305,6 +305,38 @@ def scaled_linear_layer(x: torch.Tensor, weight: torch.Tensor, bias: Optional[to
     return out
 
 
+def residual_linear_supported(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], residual: torch.Tensor) -> bool:
+    """Whether `residual_linear_layer` takes this input: a 16-bit problem that `linear_layer` would run on the wide tile
+    kernels (they alone add a residual in their epilogue), a residual of the output's shape and dtype."""
+    if not (x.is_cuda and x.dtype in (torch.float16, torch.bfloat16) and weight.dtype == x.dtype and residual.dtype == x.dtype):
+        return False
+    if bias is not None and bias.dtype != x.dtype:
+        return False
+    if x.numel() == 0 or residual.shape != (*x.shape[:-1], weight.shape[0]) or torch.is_autocast_enabled("cuda"):
+        return False
+    rows = x.numel() // x.shape[-1]
+    if rows <= FEW_ROW_MAX_ROWS or weight.shape[0] % 8 != 0:
+        return False
+    x_ = x if x.ndim == 2 else x.reshape(-1, x.shape[-1])
+    if not _lib.linear_scaled_supported(x_, weight):
+        return False
+    if rows <= SPLIT_K_MAX_ROWS and _lib.linear_splitk_workspace_bytes(x_, weight) != 0:
+        return False
+    return _lib.linear_wide_kind(rows, weight.shape[0], weight.shape[1]) != 0
+
+
+def residual_linear_layer(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], residual: torch.Tensor) -> torch.Tensor:
+    """residual + linear(x, weight, bias) in one launch: the addition happens in the tile kernels' epilogue, on the rounded
+    projection (bit for bit the two-step result).  See `kernl_linear_residual_fwd`; no counterpart in the reference."""
+    assert residual_linear_supported(x, weight, bias, residual)
+    rows, n_out = x.numel() // x.shape[-1], weight.shape[0]
+    x_ = x if x.ndim == 2 else x.reshape(rows, x.shape[-1])
+    res_ = residual.reshape(rows, n_out)
+    out = torch.empty((rows, n_out), device=x.device, dtype=x.dtype)
+    _lib.linear_residual_fwd(x_, weight, bias, res_, out)
+    return out.reshape(residual.shape)
+
+
 def decode_linear_supported(x: torch.Tensor, weight: torch.Tensor, head_dim: Optional[int] = None) -> bool:
     """Whether `decode_linear_layer` takes this input: 16-bit, K a multiple of 64, at most 64 rows in all — or up to 128
     against a weight large enough for the stream-K kernel (whose rotation wants a head size of 32, 64 or 128)."""

@@ -14,6 +14,7 @@ from kernl_amd.optimizer.dropout import remove_dropout
 from kernl_amd.optimizer.kv_cache import drop_empty_cat_operands
 from kernl_amd.optimizer.layer_norm import replace_layer_norm, replace_layer_norm_fn, replace_layer_norm_rms
 from kernl_amd.optimizer.linear import (
+    fuse_linears_into_add_layer_norms,
     fuse_residual_into_linears,
     fuse_rms_norm_into_linears,
     fuse_rms_stats_into_residual_adds,
@@ -55,5 +56,6 @@ def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
     fuse_rms_norm_into_linears(gm)
     fuse_rotary_into_projections(gm)
     fuse_residual_into_linears(gm)
+    fuse_linears_into_add_layer_norms(gm)
     fuse_rms_stats_into_residual_adds(gm)
     return gm

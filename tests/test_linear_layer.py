@@ -368,6 +368,67 @@ def test_prompt_route_of_the_rms_projections_calls_the_scaled_kernel(monkeypatch
         torch.testing.assert_close(a.float(), b.float(), rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("tile", [0, 5, 6, 7, 8], ids=["heuristic", "wide256x256", "wide256x192", "wide128x256", "wide128x192"])
+@pytest.mark.parametrize("shape", [(16384, 768, 768), (2048, 4096, 4096), (1000, 1056, 776), (513, 390, 264), (300, 768, 3072),
+                                   (129, 200, 72)], ids=lambda s: "x".join(map(str, s)))
+def test_linear_with_the_residual_added_in_the_epilogue(shape, tile, dtype, close):
+    """`kernl_linear_residual_fwd`: round(x @ w^T + bias) + residual from the wide kernels' epilogue — bit for bit the
+    linear kernel followed by an addition of the two 16-bit tensors, and the oracle's product plus the residual within
+    tolerance.  16384 x 768 -> 768 is BERT-base's attention-output projection at batch 32 x 512 and 2048 x 4096 -> 4096 a
+    Llama-7B prompt's; the others put ragged rows, ragged columns (scalar residual reads), a ragged last k-tile and a
+    residual with padded rows behind every tile shape."""
+    M, N, K = shape
+    if tile == 0 and M * N * K > 2 ** 33:
+        pytest.skip("the large shapes run once per forced tile")
+    gen = torch.Generator().manual_seed(11)
+    x, w, b = _inputs(M, N, K, dtype, gen, w_std=K ** -0.5, bias=(N % 2 == 0))
+    res_full = (torch.randn((M, N + 24), generator=gen) * 2.0).to(dtype).cuda()
+    res = res_full[:, 8:8 + N] if M < 1000 else res_full[:, :N].contiguous()    # (padded rows; 16-byte aligned only if N % 8 == 0)
+    xd, wd, bd = x.cuda(), w.cuda(), None if b is None else b.cuda()
+    out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+    lib = _lib.load()
+    lib.kernl_linear_force_tile(tile)
+    try:
+        _lib.linear_residual_fwd(xd, wd, bd, res, out)
+        plain = torch.empty_like(out)
+        _lib.linear_fwd(xd, wd, bd, plain, None, _lib.ACT_NONE)
+        torch.cuda.synchronize()
+    finally:
+        lib.kernl_linear_force_tile(0)
+    # (left to the heuristic the plain product may run another kernel, whose sums differ in the last bit)
+    if tile != 0 or _lib.linear_wide_kind(M, N, K) != 0:
+        assert torch.equal(out, plain + res), f"linear + residual {shape} tile {tile}: differs from product, then addition"
+    rows = torch.arange(0, M, 29 if M >= 2048 else 1)
+    ref = linear_oracle(x[rows], w, b, "") + res.cpu()[rows].float()
+    close(out[rows.cuda()], ref, dtype, scale="magnitude", what=f"linear + residual {shape} tile {tile}")
+
+
+def test_which_shapes_add_the_residual_in_the_epilogue():
+    """`residual_linear_supported`: 16-bit problems that the plain product runs on the wide tile kernels — encoder batches
+    and prompts — and nothing else (few rows, small problems, split K, fp32, mismatched residuals)."""
+    from kernl_amd.implementations.linear_layer import residual_linear_layer, residual_linear_supported
+
+    def case(rows, n, k, dtype=torch.float16, res_shape=None, res_dtype=None):
+        x = torch.zeros((rows, k), dtype=dtype, device="cuda")
+        w = torch.zeros((n, k), dtype=dtype, device="cuda")
+        r = torch.zeros(res_shape or (rows, n), dtype=res_dtype or dtype, device="cuda")
+        return residual_linear_supported(x, w, None, r)
+
+    assert case(16384, 768, 768) and case(16384, 768, 3072) and case(2048, 4096, 4096) and case(2048, 4096, 11008)
+    assert case(8192, 768, 768, torch.bfloat16)
+    assert not case(64, 4096, 4096) and not case(128, 768, 768)          # decoding steps: the few-row kernels
+    assert not case(512, 768, 768) and not case(256, 768, 3072)          # small problems / split K
+    assert not case(16384, 768, 768, torch.float32)
+    assert not case(16384, 768, 768, res_dtype=torch.float32) and not case(16384, 768, 768, res_shape=(16384, 1))
+    gen = torch.Generator().manual_seed(2)
+    x = torch.randn((8, 1024, 768), generator=gen).half().cuda()
+    w = (torch.randn((768, 768), generator=gen) * 0.03).half().cuda()
+    r = torch.randn((8, 1024, 768), generator=gen).half().cuda()
+    out = residual_linear_layer(x, w, None, r)
+    assert out.shape == r.shape and torch.equal(out, linear_layer(x, w, None) + r)
+
+
 def test_residual_addition_with_row_statistics(close):
     """`add_rms_stats`: the sum is the fp16 / bf16 rounding of the fp32 sum (what `a + b` gives), the statistics are those
     of the ROUNDED sum; ragged row counts, 3-D inputs, non-contiguous operands."""
