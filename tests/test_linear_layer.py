@@ -429,6 +429,40 @@ def test_which_shapes_add_the_residual_in_the_epilogue():
     assert out.shape == r.shape and torch.equal(out, linear_layer(x, w, None) + r)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [(8, 1024, 768, 768), (4, 2048, 768, 3072), (2, 128, 768, 768), (1, 16, 264, 520)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_projection_with_the_addition_and_layer_norm_behind_it(shape, dtype, close, monkeypatch):
+    """`linear_add_layer_norm_wrapper` = layer_norm(residual + linear(v)), an encoder layer's attention-output and
+    feed-forward-down projections: against the composition of the oracles, whichever kernel the addition ends up in (the
+    projection's epilogue for the first two shapes, the add + LayerNorm kernel for the others), and the two routes agree."""
+    from kernl_amd.optimizer import linear as ol
+    from oracle import effective_eps, layer_norm_oracle
+
+    bs, M, N, K = shape
+    gen = torch.Generator().manual_seed(17)
+    v = torch.randn((bs, M, K), generator=gen).to(dtype)
+    w = (torch.randn((N, K), generator=gen) * K ** -0.5).to(dtype)
+    b = (0.3 * torch.randn((N,), generator=gen)).to(dtype)
+    res = (2.0 * torch.randn((bs, M, N), generator=gen)).to(dtype)
+    g = (1.0 + 0.2 * torch.randn((N,), generator=gen)).to(dtype)
+    be = (0.1 * torch.randn((N,), generator=gen)).to(dtype)
+    calls = []
+    real = _lib.linear_residual_fwd
+    monkeypatch.setattr(_lib, "linear_residual_fwd", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    args = (v.cuda(), w.cuda(), b.cuda(), res.cuda(), (N,), g.cuda(), be.cuda(), 1e-12)
+    out = ol.linear_add_layer_norm_wrapper(*args)
+    assert len(calls) == (1 if bs * M >= 8192 else 0)
+    monkeypatch.setattr(ol, "WIDE_RESIDUAL_EPILOGUE", False)
+    other = ol.linear_add_layer_norm_wrapper(*args)
+    torch.cuda.synchronize()
+    assert len(calls) <= 1 and out.shape == res.shape and out.dtype == dtype
+    summed = res.float() + linear_oracle(v, w, b, "").to(dtype).float()   # the projection is rounded before the addition
+    ref = layer_norm_oracle(summed, g, be, effective_eps(1e-12, dtype))
+    close(out, ref, dtype, scale="magnitude", what=f"projection + add + layernorm {shape}")
+    close(other, ref, dtype, scale="magnitude", what=f"projection, then add + layernorm {shape}")
+
+
 def test_residual_addition_with_row_statistics(close):
     """`add_rms_stats`: the sum is the fp16 / bf16 rounding of the fp32 sum (what `a + b` gives), the statistics are those
     of the ROUNDED sum; ragged row counts, 3-D inputs, non-contiguous operands."""
