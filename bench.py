@@ -252,6 +252,13 @@ def llama7b_prefill(dev, layers=32, seq=2048):
         for m in norms:
             m.variance_epsilon = max(m.variance_epsilon, 1.6e-5)
         eager_clamped = model(input_ids=ids, use_cache=False).logits.float()
+        # ... and the same weights in fp32 (clamped epsilon too) give the logits both fp16 runs are approximations of
+        import copy
+
+        ref_model = copy.deepcopy(model).float()
+        ref32 = ref_model(input_ids=ids, use_cache=False).logits.float()
+        del ref_model
+        torch.cuda.empty_cache()
         for m in norms:
             m.variance_epsilon = cfg.rms_norm_eps
         torch.cuda.synchronize()
@@ -281,7 +288,11 @@ def llama7b_prefill(dev, layers=32, seq=2048):
         ((got.float() - eager_clamped).abs().mean() / eager_clamped.abs().mean()).item(), 5)
     out[f"{tag}_mean_rel_diff_of_the_eps_clamp_alone"] = round(
         ((eager_clamped - eager).abs().mean() / eager.abs().mean()).item(), 5)
-    del model, eager, eager_clamped, got
+    out[f"{tag}_mean_rel_err_vs_fp32_model_with_clamped_eps"] = round(
+        ((got.float() - ref32).abs().mean() / ref32.abs().mean()).item(), 5)
+    out[f"{tag}_fp16_eager_mean_rel_err_vs_fp32_model_with_clamped_eps"] = round(
+        ((eager_clamped - ref32).abs().mean() / ref32.abs().mean()).item(), 5)
+    del model, eager, eager_clamped, got, ref32
     torch.cuda.empty_cache()
     return out
 
