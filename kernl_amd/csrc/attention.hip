@@ -222,6 +222,8 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     // the general body; tiles in neither set are so negative everywhere that they contribute exactly 0 and are
     // dropped.  Both sets are wave-uniform scalars; tiles are taken from them lowest index first.
     uint64_t clean_bits = 0, gen_bits = 0;
+    constexpr bool SHARED = !WSPLIT;
+    __shared__ uint64_t tile_sets[4][2];
     if (use_list && MASK_MODE == MASK_VECTOR) {
         // lane l looks at key 64 t + l of tile t; 32-bit offsets (the host checks that a mask row fits them)
         auto classify = [&](auto *mrow) __attribute__((always_inline)) {
@@ -289,27 +291,46 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                 clean_bits |= (__ballot(mine && !general) & 0xFull) << (4 * j);
                 gen_bits |= (__ballot(mine && general) & 0xFull) << (4 * j);
             };
-            for (int j = 0; j * 256 < N; j += 2) {
+            // SHARED: the four waves of a workgroup want the same two sets, so wave w judges the loads j = w, w + 4, ...
+            // only and the sets are put together through LDS below (WSPLIT waves synchronise among themselves only:
+            // each judges everything)
+            constexpr int FIRST_STEP = SHARED ? 4 : 1;
+            for (int j = SHARED ? wave : 0; j * 256 < N; j += 2 * FIRST_STEP) {
                 float mv0[4], mv1[4];
                 fetch(j, mv0);
-                fetch(j + 1, mv1);
+                fetch(j + FIRST_STEP, mv1);
                 judge(j, mv0);
-                if ((j + 1) * 256 < N) judge(j + 1, mv1);
+                if ((j + FIRST_STEP) * 256 < N) judge(j + FIRST_STEP, mv1);
             }
         };
         const bool rows_vectorizable = p.ms[3] == 1;
+        bool shared_sets = false;
         if (p.mask_dtype == KERNL_F32) {
             const float *mrow = static_cast<const float *>(p.mask) + mask_base;
-            if (rows_vectorizable && aligned16(mrow)) classify4(mrow);
+            if (rows_vectorizable && aligned16(mrow)) classify4(mrow), shared_sets = SHARED;
             else classify(mrow);
         } else if (p.mask_dtype == KERNL_F16) {
             const f16 *mrow = static_cast<const f16 *>(p.mask) + mask_base;
-            if (rows_vectorizable && aligned16(mrow)) classify4(mrow);
+            if (rows_vectorizable && aligned16(mrow)) classify4(mrow), shared_sets = SHARED;
             else classify(mrow);
         } else {
             const bf16 *mrow = static_cast<const bf16 *>(p.mask) + mask_base;
-            if (rows_vectorizable && aligned16(mrow)) classify4(mrow);
+            if (rows_vectorizable && aligned16(mrow)) classify4(mrow), shared_sets = SHARED;
             else classify(mrow);
+        }
+        if constexpr (SHARED) {
+            if (shared_sets) {  // (workgroup-uniform: the mask row's layout decides)
+                if (lane == 0) {
+                    tile_sets[wave][0] = clean_bits;
+                    tile_sets[wave][1] = gen_bits;
+                }
+                __syncthreads();
+                const uint64_t c = tile_sets[0][0] | tile_sets[1][0] | tile_sets[2][0] | tile_sets[3][0];
+                const uint64_t g = tile_sets[0][1] | tile_sets[1][1] | tile_sets[2][1] | tile_sets[3][1];
+                // (every lane read the same words: back into scalar registers, where the tile order is computed)
+                clean_bits = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(c >> 32)) << 32) | (uint32_t)__builtin_amdgcn_readfirstlane((int)c);
+                gen_bits = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(g >> 32)) << 32) | (uint32_t)__builtin_amdgcn_readfirstlane((int)g);
+            }
         }
         // every key masked: keep all tiles, the result is the (finite) uniform average
         if ((clean_bits | gen_bits) == 0) gen_bits = (nt_all >= 64) ? ~0ull : ((1ull << nt_all) - 1ull);
