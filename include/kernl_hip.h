@@ -433,6 +433,24 @@ int kernl_add_rms_stats_fwd(const void *a, const void *b, void *sum, float *rstd
                             int64_t a_row_stride, int64_t b_row_stride, int64_t sum_row_stride, float eps, int dtype,
                             void *stream);
 
+/*
+ * The embedding stage of an encoder in one launch: up to three lookups summed in the tensors' dtype, one addition after
+ * the other, and the LayerNorm behind them,
+ *     out[b, s, :] = LayerNorm(round(round(table0[ids0[b, s]] + table1[ids1[b, s]]) + table2[ids2[b, s]])) * w + bias
+ * (BERT: word, token-type and position embeddings).  The reference leaves this stage to PyTorch — three gathers, two
+ * additions and its LayerNorm kernel (src/kernl/implementations/layer_norm.py:115-205, whose statistics and eps handling
+ * this kernel keeps); at batch 1 those launches are a tenth of a BERT-base forward.  tables [rows_i, N] contiguous
+ * (table1 / table2 may be NULL, in that order), ids int64 with entry (b, s) at b * batch_stride + s * seq_stride
+ * (a stride of 0 broadcasts: position ids shared by all sequences); an id outside its table is clamped into it.
+ * f16 / bf16, N % 8 == 0, N <= 2048, 16-byte aligned tables, w, bias (or NULL) and out [batch * seq, N] contiguous.
+ */
+int kernl_embedding_layernorm_fwd(const void *table0, const int64_t *ids0, int64_t ids0_batch_stride, int64_t ids0_seq_stride,
+                                  int64_t rows0, const void *table1, const int64_t *ids1, int64_t ids1_batch_stride,
+                                  int64_t ids1_seq_stride, int64_t rows1, const void *table2, const int64_t *ids2,
+                                  int64_t ids2_batch_stride, int64_t ids2_seq_stride, int64_t rows2, const void *w,
+                                  const void *bias, void *out, int64_t batch, int64_t seq, int64_t N, float eps, int dtype,
+                                  void *stream);
+
 /* The process-wide test and tuning hooks are not part of this interface: they are declared in kernl_hip_test.h. */
 
 #ifdef __cplusplus

@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "kernl_linear_scaled_fwd",
     "kernl_linear_residual_fwd",
     "kernl_linear_wide_kind",
+    "kernl_embedding_layernorm_fwd",
     "kernl_linear_decode_fwd",
     "kernl_linear_splitk_workspace_bytes",
     "kernl_linear_splitk_fwd",
@@ -148,6 +149,9 @@ def load() -> ctypes.CDLL:
     lib.kernl_linear_scaled_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 2 + [ctypes.c_int] * 3 + [_vp]
     lib.kernl_linear_residual_fwd.restype = ctypes.c_int
     lib.kernl_linear_residual_fwd.argtypes = [_vp] * 5 + [_i64] * 3 + [_i64p] * 3 + [ctypes.c_int, _vp]
+    lib.kernl_embedding_layernorm_fwd.restype = ctypes.c_int
+    lib.kernl_embedding_layernorm_fwd.argtypes = [_vp, _vp, _i64, _i64, _i64] * 3 + [_vp, _vp, _vp, _i64, _i64, _i64,
+                                                                                      ctypes.c_float, ctypes.c_int, _vp]
     lib.kernl_add_rms_stats_fwd.restype = ctypes.c_int
     lib.kernl_add_rms_stats_fwd.argtypes = [_vp] * 4 + [_i64] * 5 + [ctypes.c_float, ctypes.c_int, _vp]
     lib.kernl_linear_small_kind.restype = ctypes.c_int
@@ -446,6 +450,30 @@ def linear_residual_fwd(x2d, weight, bias, residual2d, out2d) -> None:
             DTYPE_CODE[x2d.dtype], _stream(x2d),
         )
     _check(st, "kernl_linear_residual_fwd")
+
+
+def embedding_layernorm_fwd(tables, ids, weight, bias, out, eps: float) -> None:
+    """out[b, s] = LayerNorm(sum of tables[i][ids[i][b, s]]) (rows added one after the other in the tables' dtype).
+    tables: 1 to 3 contiguous [rows, N] matrices; ids: int64 [batch, seq] views (stride 0 allowed); out [batch, seq, N]."""
+    _require_gpu(*tables, *ids, weight, bias, out)
+    batch, seq, n = out.shape
+    if not 1 <= len(tables) <= 3 or len(ids) != len(tables):
+        raise ValueError("one to three tables, each with its ids")
+    if not out.is_contiguous() or any(not t.is_contiguous() or t.shape[1] != n or t.dtype != out.dtype for t in tables):
+        raise ValueError("tables and out must be contiguous, of one dtype and one width")
+    if any(i.dtype != torch.int64 or tuple(i.shape) != (batch, seq) for i in ids):
+        raise ValueError("ids must be int64 [batch, seq] (expanded views are fine)")
+    args = []
+    for k in range(3):
+        if k < len(tables):
+            args += [tables[k].data_ptr(), ids[k].data_ptr(), ids[k].stride(0), ids[k].stride(1), tables[k].shape[0]]
+        else:
+            args += [None, None, 0, 0, 0]
+    lib = load()
+    with torch.cuda.device(out.device):
+        st = lib.kernl_embedding_layernorm_fwd(*args, weight.data_ptr(), None if bias is None else bias.data_ptr(), out.data_ptr(),
+                                               batch, seq, n, float(eps), DTYPE_CODE[out.dtype], _stream(out))
+    _check(st, "kernl_embedding_layernorm_fwd")
 
 
 def add_rms_stats_fwd(a2d, b2d, sum2d, rstd, eps: float) -> None:

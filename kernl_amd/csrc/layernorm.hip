@@ -380,6 +380,82 @@ __global__ void __launch_bounds__(256) add_rms_stats_kernel(const T *__restrict_
     if (lane == 0) rstd[row] = rsqrtf(sq / (float)N + eps);
 }
 
+// Embedding lookups summed and normalised: out[m] = LayerNorm(round(round(t0[i0[m]] + t1[i1[m]]) + t2[i2[m]])) — the
+// rows are added in the tensors' dtype, one addition after the other, as the eager model adds them.  One wave per output
+// row, a lane keeps up to 4 chunks of 8 values (N <= 2048); an index outside its table is clamped into it.
+struct EmbedTable {
+    const void *table;   // [rows, N] contiguous, or null
+    const int64_t *ids;  // entry (b, s) at b * ids_bs + s * ids_ss
+    int64_t ids_bs, ids_ss, rows;
+};
+template <typename T>
+__global__ void __launch_bounds__(256) embedding_layernorm_kernel(EmbedTable t0, EmbedTable t1, EmbedTable t2,
+                                                                  const T *__restrict__ w, const T *__restrict__ b,
+                                                                  T *__restrict__ out, int M, int S, int N, float eps) {
+    typedef typename Vec8<T>::type vec8;
+    const int lane = threadIdx.x & 63, row = (int)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const int bi = row / S, si = row % S;
+    auto row_of = [&](const EmbedTable &t) __attribute__((always_inline)) -> const vec8 * {
+        int64_t id = t.ids[bi * t.ids_bs + si * t.ids_ss];
+        id = id < 0 ? 0 : (id >= t.rows ? t.rows - 1 : id);
+        return reinterpret_cast<const vec8 *>(static_cast<const T *>(t.table) + id * N);
+    };
+    const vec8 *r0 = row_of(t0);
+    const vec8 *r1 = t1.table != nullptr ? row_of(t1) : nullptr;
+    const vec8 *r2 = t2.table != nullptr ? row_of(t2) : nullptr;
+    const int chunks = N / 8;
+    float v[4][8];
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = lane + 64 * i;
+        const bool in = c < chunks;
+        vec8 a = in ? r0[c] : vec8{};
+        if (r1 != nullptr && in) {
+            const vec8 o = r1[c];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[e] = from_float<T>(to_float(a[e]) + to_float(o[e]));
+        }
+        if (r2 != nullptr && in) {
+            const vec8 o = r2[c];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[e] = from_float<T>(to_float(a[e]) + to_float(o[e]));
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            v[i][e] = to_float(a[e]);
+            sum += v[i][e];
+        }
+    }
+    const float mean = wave_sum(sum) / (float)N;
+    float sq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (lane + 64 * i < chunks) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float d = v[i][e] - mean;
+                sq = fmaf(d, d, sq);
+            }
+        }
+    }
+    const float rstd = rsqrtf(wave_sum(sq) / (float)N + eps);
+    vec8 *op = reinterpret_cast<vec8 *>(out + (int64_t)row * N);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = lane + 64 * i;
+        if (c < chunks) {
+            const vec8 g = reinterpret_cast<const vec8 *>(w)[c];
+            const vec8 be = b != nullptr ? reinterpret_cast<const vec8 *>(b)[c] : vec8{};
+            vec8 o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = from_float<T>(fmaf((v[i][e] - mean) * rstd, to_float(g[e]), b != nullptr ? to_float(be[e]) : 0.0f));
+            op[c] = o;
+        }
+    }
+}
+
 static int layernorm_entry(const void *x, const void *res, const void *w, const void *b, void *out,
                            float *mean, float *rstd, int64_t M, int64_t N, int64_t x_rs, int64_t x_cs,
                            int64_t res_rs, int64_t res_cs, int64_t out_rs, int64_t out_cs, float eps,
@@ -453,4 +529,41 @@ extern "C" int kernl_add_rms_stats_fwd(const void *a, const void *b, void *sum, 
         hipLaunchKernelGGL((add_rms_stats_kernel<bf16>), grid, block, 0, st, static_cast<const bf16 *>(a), static_cast<const bf16 *>(b),
                            static_cast<bf16 *>(sum), rstd, (int)M, (int)N, a_row_stride, b_row_stride, sum_row_stride, eps);
     return check_launch("add_rms_stats");
+}
+
+extern "C" int kernl_embedding_layernorm_fwd(const void *table0, const int64_t *ids0, int64_t ids0_batch_stride,
+                                             int64_t ids0_seq_stride, int64_t rows0, const void *table1, const int64_t *ids1,
+                                             int64_t ids1_batch_stride, int64_t ids1_seq_stride, int64_t rows1,
+                                             const void *table2, const int64_t *ids2, int64_t ids2_batch_stride,
+                                             int64_t ids2_seq_stride, int64_t rows2, const void *w, const void *bias, void *out,
+                                             int64_t batch, int64_t seq, int64_t N, float eps, int dtype, void *stream) {
+    using namespace kernl;
+    if (table0 == nullptr || ids0 == nullptr || w == nullptr || out == nullptr || (table1 != nullptr && ids1 == nullptr) ||
+        (table2 != nullptr && ids2 == nullptr))
+        return set_error(KERNL_ERR_INVALID_ARG, "embedding + layernorm: table0, its ids, w and out must not be NULL, and every table needs ids");
+    if (table1 == nullptr && table2 != nullptr)
+        return set_error(KERNL_ERR_INVALID_ARG, "embedding + layernorm: tables are given in order (table2 without table1)");
+    if (batch < 0 || seq < 0 || N <= 0 || rows0 <= 0 || (table1 != nullptr && rows1 <= 0) || (table2 != nullptr && rows2 <= 0))
+        return set_error(KERNL_ERR_INVALID_ARG, "embedding + layernorm: bad sizes batch=%lld seq=%lld N=%lld", (long long)batch,
+                         (long long)seq, (long long)N);
+    if (dtype != KERNL_F16 && dtype != KERNL_BF16)
+        return set_error(KERNL_ERR_UNSUPPORTED, "embedding + layernorm: only f16 and bf16 are supported, got dtype %d", dtype);
+    if (N % 8 != 0 || N > 2048 || batch * seq > INT32_MAX || !aligned16(table0) || !aligned16(out) || !aligned16(w) ||
+        (bias != nullptr && !aligned16(bias)) || (table1 != nullptr && !aligned16(table1)) || (table2 != nullptr && !aligned16(table2)))
+        return set_error(KERNL_ERR_UNSUPPORTED, "embedding + layernorm: N must be a multiple of 8 and at most 2048, tables, w, bias "
+                         "and out 16-byte aligned and contiguous");
+    if (batch == 0 || seq == 0) return KERNL_OK;
+    const EmbedTable t0 = {table0, ids0, ids0_batch_stride, ids0_seq_stride, rows0};
+    const EmbedTable t1 = {table1, ids1, ids1_batch_stride, ids1_seq_stride, rows1};
+    const EmbedTable t2 = {table2, ids2, ids2_batch_stride, ids2_seq_stride, rows2};
+    const int M = (int)(batch * seq);
+    const dim3 grid((unsigned)((M + 3) / 4)), block(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == KERNL_F16)
+        hipLaunchKernelGGL((embedding_layernorm_kernel<f16>), grid, block, 0, st, t0, t1, t2, static_cast<const f16 *>(w),
+                           static_cast<const f16 *>(bias), static_cast<f16 *>(out), M, (int)seq, (int)N, eps);
+    else
+        hipLaunchKernelGGL((embedding_layernorm_kernel<bf16>), grid, block, 0, st, t0, t1, t2, static_cast<const bf16 *>(w),
+                           static_cast<const bf16 *>(bias), static_cast<bf16 *>(out), M, (int)seq, (int)N, eps);
+    return check_launch("embedding + layernorm");
 }

@@ -82,3 +82,40 @@ def add_layer_norm(
     """LayerNorm(x + residual) in one pass over HBM.  No reference counterpart: there the add is a separate
     eager op in front of every LayerNorm."""
     return LayerNorm.apply(x, weight, bias, eps, None, use_rms_norm, residual)
+
+
+def embedding_layer_norm_supported(tables, ids, weight, bias) -> bool:
+    """What `embedding_layer_norm` takes: 1 to 3 fp16 / bf16 tables of one width (a multiple of 8, at most 2048) on the
+    GPU, int64 ids that broadcast to one [batch, seq] shape, LayerNorm parameters of the tables' dtype."""
+    if not 1 <= len(tables) <= 3 or len(ids) != len(tables):
+        return False
+    t0 = tables[0]
+    if not (t0.is_cuda and t0.dtype in (torch.float16, torch.bfloat16) and t0.dim() == 2 and t0.shape[1] % 8 == 0 and t0.shape[1] <= 2048):
+        return False
+    if any(t.dim() != 2 or t.dtype != t0.dtype or t.shape[1] != t0.shape[1] or not t.is_contiguous() or t.data_ptr() % 16 != 0 for t in tables):
+        return False
+    if any(i.dtype != torch.int64 or i.dim() > 2 or not i.is_cuda for i in ids):
+        return False
+    try:
+        shape = torch.broadcast_shapes(*[tuple(i.shape) for i in ids])
+    except RuntimeError:
+        return False
+    if len(shape) != 2 or shape[0] * shape[1] == 0:
+        return False
+    params_ok = weight is not None and weight.dtype == t0.dtype and weight.is_contiguous() and weight.numel() == t0.shape[1]
+    return bool(params_ok and (bias is None or (bias.dtype == t0.dtype and bias.is_contiguous() and bias.numel() == t0.shape[1])))
+
+
+def embedding_layer_norm(tables, ids, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+    """LayerNorm(tables[0][ids[0]] + tables[1][ids[1]] + tables[2][ids[2]]) in one launch: the embedding stage of an
+    encoder (word, token-type and position embeddings; the rows are added in the tables' dtype, in that order, as the
+    eager model adds them).  The fp16 eps policy is the LayerNorm operator's.  No counterpart in the reference, which
+    leaves the lookups and additions to PyTorch in front of its LayerNorm kernel (implementations/layer_norm.py:279-335)."""
+    assert embedding_layer_norm_supported(tables, ids, weight, bias)
+    shape = torch.broadcast_shapes(*[tuple(i.shape) for i in ids])
+    t0 = tables[0]
+    if t0.dtype == torch.float16:
+        eps = max(eps, 1.6e-5)
+    out = torch.empty((shape[0], shape[1], t0.shape[1]), device=t0.device, dtype=t0.dtype)
+    _lib.embedding_layernorm_fwd(list(tables), [i.expand(shape) for i in ids], weight, bias, out, eps)
+    return out

@@ -12,7 +12,12 @@ from kernl_amd.optimizer.attention import (
 )
 from kernl_amd.optimizer.dropout import remove_dropout
 from kernl_amd.optimizer.kv_cache import drop_empty_cat_operands
-from kernl_amd.optimizer.layer_norm import replace_layer_norm, replace_layer_norm_fn, replace_layer_norm_rms
+from kernl_amd.optimizer.layer_norm import (
+    fuse_embeddings_into_layer_norm,
+    replace_layer_norm,
+    replace_layer_norm_fn,
+    replace_layer_norm_rms,
+)
 from kernl_amd.optimizer.linear import (
     fuse_linears_into_add_layer_norms,
     fuse_residual_into_linears,
@@ -24,6 +29,7 @@ from kernl_amd.optimizer.linear import (
 from kernl_amd.optimizer.mask import (
     constant_causal_masks_to_flag,
     drop_all_true_conjuncts,
+    full_range_index_to_view,
     merge_nested_expands,
     scalar_tensors_to_full,
     sink_expand_below_where,
@@ -39,6 +45,7 @@ def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
     fuse_rotary_embedding(gm)
     scalar_tensors_to_full(gm)
     drop_all_true_conjuncts(gm)
+    full_range_index_to_view(gm)
     merge_nested_expands(gm)
     sink_expand_below_where(gm)
     merge_nested_expands(gm)
@@ -53,6 +60,7 @@ def dynamo_backend_ofi(gm: torch.fx.GraphModule, assume_causal=False):
     replace_layer_norm(gm)
     replace_layer_norm_fn(gm)
     replace_layer_norm_rms(gm)
+    fuse_embeddings_into_layer_norm(gm)
     fuse_rms_norm_into_linears(gm)
     fuse_rotary_into_projections(gm)
     fuse_residual_into_linears(gm)

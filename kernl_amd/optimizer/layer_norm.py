@@ -68,6 +68,25 @@ def layer_norm_rms_wrapper(v: torch.Tensor, weight: torch.Tensor, eps: float):
     return layer_norm(v, weight, None, eps, None, use_rms_norm=True)
 
 
+def embedding_layer_norm_wrapper(ids0, table0, ids1, table1, ids2, table2, normalized_shape, weight, bias, eps: float):
+    """layer_norm((embedding(ids0, table0) + embedding(ids1, table1)) + embedding(ids2, table2)) — the third pair may be
+    None — as one launch where the kernel takes the operands (`embedding_layer_norm`), as the lookups, additions and the
+    LayerNorm kernel they were otherwise."""
+    from kernl_amd.implementations.layer_norm import embedding_layer_norm, embedding_layer_norm_supported
+
+    pairs = [(i, t) for i, t in ((ids0, table0), (ids1, table1), (ids2, table2)) if t is not None]
+    tables, ids = [t for _, t in pairs], [i for i, _ in pairs]
+    if all(t.dtype == torch.float16 for t in tables):
+        _half_params_once(tables[0], weight, bias)
+    if len(normalized_shape) == 1 and not torch.is_autocast_enabled("cuda") and embedding_layer_norm_supported(tables, ids, weight, bias):
+        return embedding_layer_norm(tables, ids, weight, bias, eps)
+    total = torch.nn.functional.embedding(ids[0], tables[0])
+    for i, t in zip(ids[1:-1], tables[1:-1]):
+        total = total + torch.nn.functional.embedding(i, t)
+    return add_layer_norm_wrapper_functional(total, torch.nn.functional.embedding(ids[-1], tables[-1]), normalized_shape, weight, bias, eps)
+
+
+torch.fx.wrap("embedding_layer_norm_wrapper")
 torch.fx.wrap("layer_norm_wrapper")
 torch.fx.wrap("layer_norm_wrapper_functional")
 torch.fx.wrap("add_layer_norm_wrapper_functional")
@@ -135,3 +154,47 @@ def replace_layer_norm_rms(gm: torch.fx.GraphModule):
             return pattern_llama
 
         replace_pattern(gm, make(dtype), replace)
+
+
+def fuse_embeddings_into_layer_norm(gm: torch.fx.GraphModule):
+    """`add_layer_norm_wrapper_functional(embedding(i0, t0) + embedding(i1, t1), embedding(i2, t2), ...)` — or two lookups —
+    becomes one `embedding_layer_norm_wrapper` call (BertEmbeddings: word + token type, + position, LayerNorm).  Only sums
+    taken left to right are rewritten (the kernel adds in that order, rounding after each addition as the model does), and
+    only lookups and partial sums nothing else reads.  Runs after the LayerNorm passes."""
+    import operator
+
+    def lookup(n):
+        if not (isinstance(n, torch.fx.Node) and n.op == "call_function" and n.target is torch.nn.functional.embedding and len(n.users) == 1):
+            return None
+        args = list(n.args) + [None] * 7
+        max_norm = n.kwargs.get("max_norm", args[3])
+        if max_norm is not None or len(n.args) < 2:
+            return None
+        return (n.args[0], n.args[1])
+
+    changed = False
+    for node in list(gm.graph.nodes):
+        if not (node.op == "call_function" and node.target is add_layer_norm_wrapper_functional and len(node.args) == 6 and not node.kwargs):
+            continue
+        a, b = node.args[:2]
+        last = lookup(b)
+        if last is None:
+            continue
+        first = lookup(a)
+        if first is not None:
+            pairs = [first, last]
+        elif (isinstance(a, torch.fx.Node) and a.op == "call_function" and a.target in (operator.add, torch.add) and len(a.args) == 2
+              and not a.kwargs and len(a.users) == 1 and lookup(a.args[0]) is not None and lookup(a.args[1]) is not None):
+            pairs = [lookup(a.args[0]), lookup(a.args[1]), last]
+        else:
+            continue
+        flat = [x for pair in pairs for x in pair] + [None, None] * (3 - len(pairs))
+        with gm.graph.inserting_before(node):
+            fused = gm.graph.call_function(embedding_layer_norm_wrapper, tuple(flat) + tuple(node.args[2:]))
+        node.replace_all_uses_with(fused)
+        gm.graph.erase_node(node)
+        changed = True
+    if changed:
+        gm.graph.eliminate_dead_code()
+        gm.graph.lint()
+        gm.recompile()

@@ -71,6 +71,12 @@ def _fold_constants(gm: torch.fx.GraphModule):
         return torch.fx.node.map_arg(arg, lambda n: values[n])
 
     for node in gm.graph.nodes:
+        if node.op == "get_attr" and str(node.target).startswith("_tensor_constant"):
+            # literal tensors the tracer lifted into attributes of the graph module
+            const = getattr(gm, node.target, None)
+            if isinstance(const, torch.Tensor) and const.numel() <= _FOLD_LIMIT:
+                values[node] = const
+            continue
         if node.op == "call_function" and node.target in _FOLDABLE_FUNCTIONS:
             pass
         elif node.op == "call_method" and node.target in _FOLDABLE_METHODS:
@@ -125,6 +131,54 @@ def drop_all_true_conjuncts(gm: torch.fx.GraphModule):
             gm.graph.erase_node(node)
             changed = True
             break
+    if changed:
+        gm.graph.eliminate_dead_code()
+        gm.graph.lint()
+        gm.recompile()
+
+
+def full_range_index_to_view(gm: torch.fx.GraphModule):
+    """`x[i0, i1, ...]` with one constant index tensor per dimension of x, each an `arange` over the whole dimension laid
+    along an axis of its own (`padding[batch_idx[:, None, None, None], kv_idx[None, None, None, :]]`, what transformers'
+    mask builders index the [B, S] padding mask with), is `x` reshaped with those axes in place and ones elsewhere: a view
+    instead of two aranges, an addition and a gather launch per forward."""
+    values = _fold_constants(gm)
+    changed = False
+    for node in list(gm.graph.nodes):
+        if node.op != "call_function" or node.target is not operator.getitem or len(node.args) != 2:
+            continue
+        x, index = node.args
+        if not (isinstance(x, Node) and isinstance(index, tuple) and index and all(isinstance(i, Node) and i in values for i in index)):
+            continue
+        xv = x.meta.get("example_value")
+        if x in values or not isinstance(xv, torch.Tensor) or xv.dim() != len(index) or not all(isinstance(d, int) for d in xv.shape):
+            continue
+        idx = [values[i] for i in index]
+        rank = max(t.dim() for t in idx)
+        if rank == 0 or any(t.dtype not in (torch.int64, torch.int32) for t in idx):
+            continue
+        target, last_axis, ok = [1] * rank, -1, True
+        for k, t in enumerate(idx):
+            shape = (1,) * (rank - t.dim()) + tuple(t.shape)
+            axes = [a for a, d in enumerate(shape) if d != 1]
+            if xv.shape[k] == 1 and not axes:
+                axes = [last_axis + 1] if last_axis + 1 < rank else []
+            if len(axes) != 1 or axes[0] <= last_axis or shape[axes[0]] != xv.shape[k]:
+                ok = False
+                break
+            if not torch.equal(t.reshape(-1).cpu().long(), torch.arange(xv.shape[k])):
+                ok = False
+                break
+            last_axis = axes[0]
+            target[last_axis] = xv.shape[k]
+        if not ok:
+            continue
+        with gm.graph.inserting_before(node):
+            view = gm.graph.call_method("reshape", (x,) + tuple(target))
+        view.meta["example_value"] = xv.reshape(target)
+        node.replace_all_uses_with(view)
+        gm.graph.erase_node(node)
+        changed = True
     if changed:
         gm.graph.eliminate_dead_code()
         gm.graph.lint()

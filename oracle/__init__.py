@@ -10,6 +10,7 @@ from oracle.ops import (  # noqa: F401
     attention_tiled_oracle,
     e5m2_decode_oracle,
     effective_eps,
+    embedding_layer_norm_oracle,
     glu_oracle,
     layer_norm_oracle,
     layer_norm_welford_oracle,

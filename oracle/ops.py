@@ -214,6 +214,20 @@ def layer_norm_oracle(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
     return out
 
 
+def embedding_layer_norm_oracle(tables, ids, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+    """LayerNorm of the sum of embedding lookups, the rows added in the tables' dtype one after the other as an eager
+    model adds them (`word + token_type`, then `+ position`: transformers' BertEmbeddings.forward; the reference runs
+    these as PyTorch ops in front of its LayerNorm kernel, implementations/layer_norm.py:115-205).  ids broadcast
+    against each other; the result is fp32."""
+    dtype = tables[0].dtype
+    shape = torch.broadcast_shapes(*[tuple(i.shape) for i in ids])
+    total = None
+    for table, index in zip(tables, ids):
+        rows = table.detach().cpu()[index.detach().cpu().expand(shape)]
+        total = rows if total is None else (total.float() + rows.float()).to(dtype)
+    return layer_norm_oracle(total, weight, bias, eps)
+
+
 def rms_norm_oracle(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """x·rsqrt(mean(x²)+eps)·w, fp32 (implementations/layer_norm.py:41-57 and the IS_RMSNORM branch :169-170,:182-183)."""
     x32 = x.detach().float().cpu()

@@ -273,7 +273,16 @@ def test_backend_rewrites_dynamo_graph_of_bert():
         # pooler stay on their own, and so does the add + LayerNorm of the embeddings
         assert t.count("linear_add_layer_norm_wrapper") == 2 * 2
         assert t.count("linear_wrapper_functional") == 2 * 1 + 1
-        assert t.count("add_layer_norm_wrapper_functional") == 1
+        assert t.count("add_layer_norm_wrapper_functional") == 0
+        # the three embedding lookups, their two additions and the LayerNorm behind them are one call
+        assert t.count("embedding_layer_norm_wrapper") == 1 and "embedding" not in t
+        emb = next(n for n in graphs[0].graph.nodes if n.op == "call_function" and n.target.__name__ == "embedding_layer_norm_wrapper")
+        assert [a.name for a in emb.args[1:6:2]] == [
+            "l_self_modules_embeddings_modules_word_embeddings_parameters_weight_",
+            "l_self_modules_embeddings_modules_token_type_embeddings_parameters_weight_",
+            "l_self_modules_embeddings_modules_position_embeddings_parameters_weight_"]
+        # the padding mask is reshaped, not gathered with index grids
+        assert "arange" not in t
         assert "softmax" not in t and "dropout" not in t and "gelu" not in t and "layer_norm" not in t and "linear" not in t
         # the padding mask reaches the kernel as a broadcast of a per-key tensor, not as a [B,1,S,S] matrix
         attn = next(n for n in graphs[0].graph.nodes if n.op == "call_function" and n.target.__name__ == fused)
@@ -839,3 +848,57 @@ def test_small_problem_rule_of_the_library():
     assert kind(768, 768, 3072) == 11 and kind(1024, 768, 1536) == 11   # long K: one round of 64 x 64 tiles where the dealt ones need two
     assert kind(2048, 1024, 4096) == 0                                  # long K and more than 256 tiles of 64 x 64: split-K
     assert kind(128, 768, 3076) == 0 and kind(0, 768, 768) == 0         # K no multiple of 8: not the MFMA path at all
+
+
+def test_full_range_index_grids_become_a_view():
+    """`x[arange(B)[:, None, None, None], arange(S)[None, None, None, :]]` is x reshaped to [B, 1, 1, S]; partial ranges,
+    permuted axes and shifted grids stay gathers."""
+    from kernl_amd.optimizer.mask import full_range_index_to_view
+
+    def build(fn):
+        gm = torch.fx.symbolic_trace(fn)
+        for n in gm.graph.nodes:
+            if n.op == "placeholder":
+                n.meta["example_value"] = torch.zeros(3, 5, dtype=torch.bool)
+        full_range_index_to_view(gm)
+        return gm
+
+    def whole(x):
+        return x[torch.arange(3)[:, None, None, None], (torch.arange(5) + 0)[None, None, None, :]]
+
+    def partial(x):
+        return x[torch.arange(2)[:, None, None, None], torch.arange(5)[None, None, None, :]]
+
+    def swapped(x):
+        return x[torch.arange(3)[None, None, None, :], torch.arange(5)[:, None, None, None]]
+
+    def shifted(x):
+        return x[torch.arange(3)[:, None], (torch.arange(5) + 1).clamp(max=4)[None, :]]
+
+    x = torch.rand(3, 5) > 0.5
+    gm = build(whole)
+    assert "reshape" in _targets(gm) and "arange" not in _targets(gm)
+    assert torch.equal(gm(x), whole(x)) and gm(x).shape == (3, 1, 1, 5)
+    for fn in (partial, swapped, shifted):
+        gm = build(fn)
+        assert "reshape" not in _targets(gm)
+        assert torch.equal(gm(x), fn(x))
+
+
+def test_embedding_oracle_against_the_library_routines():
+    """The oracle of the fused embedding stage is gathers, additions and the LayerNorm oracle: with fp32 tables (no
+    rounding between the additions) it must equal F.embedding + F.layer_norm; with fp16 tables the additions round."""
+    from oracle import embedding_layer_norm_oracle
+
+    gen = torch.Generator().manual_seed(4)
+    tables = [torch.randn((r, 24), generator=gen) for r in (50, 2, 16)]
+    ids = [torch.randint(0, 50, (3, 16), generator=gen), torch.randint(0, 2, (3, 16), generator=gen), torch.arange(16)[None, :]]
+    w, b = torch.randn(24, generator=gen), torch.randn(24, generator=gen)
+    want = torch.nn.functional.layer_norm(sum(torch.nn.functional.embedding(i, t) for i, t in zip(ids, tables)), (24,), w, b, 1e-5)
+    torch.testing.assert_close(embedding_layer_norm_oracle(tables, ids, w, b, 1e-5), want, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(embedding_layer_norm_oracle(tables[:1], ids[:1], w, None, 1e-5),
+                               torch.nn.functional.layer_norm(tables[0][ids[0]], (24,), w, None, 1e-5), rtol=1e-5, atol=1e-5)
+    half = [t.half() for t in tables]
+    rounded = ((half[0][ids[0]] + half[1][ids[1]]) + half[2][ids[2].expand(3, 16)]).float()   # fp16 additions round each time
+    torch.testing.assert_close(embedding_layer_norm_oracle(half, ids, w, b, 1e-5),
+                               torch.nn.functional.layer_norm(rounded, (24,), w, b, 1e-5), rtol=1e-5, atol=1e-5)

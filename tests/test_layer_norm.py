@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from kernl_amd.implementations.layer_norm import add_layer_norm, layer_norm
-from oracle import effective_eps, layer_norm_oracle, rms_norm_oracle
+from oracle import effective_eps, embedding_layer_norm_oracle, layer_norm_oracle, rms_norm_oracle
 
 pytestmark = pytest.mark.gpu
 
@@ -184,3 +184,43 @@ def test_functional_layer_norm_forms_all_reach_the_kernel(form, close, monkeypat
     ref = layer_norm_oracle(flat, wf, bf, eps).reshape(x.shape)
     assert out.shape == x.shape and out.dtype == torch.half
     close(out, ref, scale="magnitude", what=f"functional layer norm, {form}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("case", [(32, 512, 768, 3), (1, 16, 768, 3), (3, 77, 264, 2), (2, 5, 2048, 1), (5, 130, 1024, 3)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_embedding_lookups_summed_and_normalised(case, dtype, close):
+    """`embedding_layer_norm`: word + token-type + position rows and their LayerNorm in one launch, against the oracle
+    (gathers, additions rounded to the tables' dtype, fp32 LayerNorm).  32 x 512 x 768 is BERT-base's embedding stage at
+    BASELINE config 3; the others put ragged widths, one and two tables, broadcast position ids (stride 0) and a
+    token-type view with stride 0 in both dimensions behind the same kernel."""
+    from kernl_amd.implementations.layer_norm import embedding_layer_norm
+
+    batch, seq, n, n_tables = case
+    gen = torch.Generator().manual_seed(9)
+    rows = (1000, 2, 600)[:n_tables]
+    tables = [(torch.randn((r, n), generator=gen) * (0.5, 0.1, 0.2)[k]).to(dtype) for k, r in enumerate(rows)]
+    ids = [torch.randint(0, 1000, (batch, seq), generator=gen)]
+    if n_tables > 1:
+        ids.append(torch.zeros((1, 1), dtype=torch.int64).expand(batch, seq) if batch == 1 else torch.randint(0, 2, (batch, seq), generator=gen))
+    if n_tables > 2:
+        ids.append(torch.arange(seq)[None, :])                      # shared by all sequences
+    w = (1.0 + 0.2 * torch.randn((n,), generator=gen)).to(dtype)
+    b = (0.1 * torch.randn((n,), generator=gen)).to(dtype) if n != 264 else None
+    out = embedding_layer_norm([t.cuda() for t in tables], [i.cuda() for i in ids], w.cuda(), None if b is None else b.cuda(), 1e-12)
+    torch.cuda.synchronize()
+    assert out.shape == (batch, seq, n) and out.dtype == dtype
+    ref = embedding_layer_norm_oracle(tables, ids, w, b, effective_eps(1e-12, dtype))
+    close(out, ref, dtype, scale="magnitude", what=f"embedding + layernorm {case}")
+
+
+def test_embedding_ids_outside_the_table_are_clamped():
+    from kernl_amd.implementations.layer_norm import embedding_layer_norm
+
+    gen = torch.Generator().manual_seed(1)
+    table = torch.randn((10, 64), generator=gen).half().cuda()
+    w = torch.ones(64).half().cuda()
+    ids = torch.tensor([[0, 9, 10, 12345, -1, -99]]).cuda()
+    out = embedding_layer_norm([table], [ids], w, None, 1e-5)
+    want = embedding_layer_norm([table], [ids.clamp(0, 9)], w, None, 1e-5)
+    assert torch.equal(out, want)
