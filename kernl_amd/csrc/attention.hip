@@ -243,7 +243,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                         const bool valid = t * BN + lane < N;
                         const float sm = scale_mask(mv[j], p.clamp);
                         const bool any_nonzero = __ballot(valid && (sm != 0.0f)) != 0;
-                        const bool any_normal = __ballot(valid && (sm > kNegBig)) != 0;
+                        const bool any_normal = __ballot(valid && (sm > kDeadMask)) != 0;
                         if (any_normal) {
                             if (any_nonzero || t * BN + BN > N) gen_bits |= 1ull << t;
                             else clean_bits |= 1ull << t;
@@ -281,7 +281,7 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                     const float sm = scale_mask(mv[r], p.clamp);
                     const bool valid = e0 + r < N;
                     nz |= valid && (sm != 0.0f);
-                    nm |= valid && (sm > kNegBig);
+                    nm |= valid && (sm > kDeadMask);
                 }
                 const uint64_t bz = __ballot(nz), bn = __ballot(nm);
                 const int k = lane & 3, t = 4 * j + k;

@@ -14,6 +14,11 @@ static constexpr float kNegBig = -1.0e30f;            // anything below: exp2(x 
 static constexpr float kClampFloor = -1.7014118e38f;  // scaled mask values are kept finite (-FLT_MAX / 2)
 static constexpr float kRescaleThreshold = 8.0f;  // log2 units
 static constexpr float kMaskedScore = -32768.0f;  // base-2 scores below this are mask values, not scores
+// A mask value (base-2 domain) at or below this marks a dead key: added to any score a 16-bit model produces it stays
+// below kMaskedScore, so the key weighs exactly 0 in every row that has an ordinary key, and a key tile of dead keys only
+// is not visited at all.  -inf and the fp32 / bf16 "minimum" masks are far below it, and so is the fp16 one that models
+// build in their own dtype (finfo(float16).min = -65504, -94505 in the base-2 domain) — which kNegBig does not catch.
+static constexpr float kDeadMask = 2.0f * kMaskedScore;
 
 enum { MASK_NONE = 0, MASK_VECTOR = 1, MASK_MATRIX = 2 };
 

@@ -283,7 +283,7 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
             const int n = g * 64 + lane;
             const float v = bias_lds[bias_wave + n];
             const bool valid = n < N;
-            const bool any_nz = __ballot(valid && v != 0.0f) != 0, any_nm = __ballot(valid && v > kNegBig) != 0,
+            const bool any_nz = __ballot(valid && v != 0.0f) != 0, any_nm = __ballot(valid && v > kDeadMask) != 0,
                        any_ord = __ballot(valid && v == 0.0f) != 0;
             const bool full = g * 64 + 64 <= N;
             if (any_nm) {
@@ -481,7 +481,7 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
             for (int i = 0; i < PER; ++i) {
                 const float v = mv[i] - bmax;
                 bias_lds[bias_wave + lane + 64 * i] = v;
-                const uint64_t nz = __ballot(v != 0.0f), nm = __ballot(v > kNegBig);
+                const uint64_t nz = __ballot(v != 0.0f), nm = __ballot(v > kDeadMask);
                 const uint32_t bit = 1u << i;
                 gen_bits |= (nm != 0 && nz != 0) ? bit : 0u;
                 clean_bits |= (nm != 0 && nz == 0) ? bit : 0u;
@@ -502,7 +502,7 @@ __global__ void __launch_bounds__(256, D == 64 ? 2 : 1) attention_pipe_kernel(co
             for (int i = 0; i < cur_nt_all; ++i) {
                 const float v = staged_mask_value(ms[64 * i], lane + 64 * i) - bmax;
                 if ((i & 3) == wave) bias_lds[lane + 64 * i] = v;
-                const uint64_t nz = __ballot(v != 0.0f), nm = __ballot(v > kNegBig);
+                const uint64_t nz = __ballot(v != 0.0f), nm = __ballot(v > kDeadMask);
                 const uint32_t bit = 1u << i;
                 gen_bits |= (nm != 0 && nz != 0) ? bit : 0u;
                 clean_bits |= (nm != 0 && nz == 0) ? bit : 0u;

@@ -103,6 +103,25 @@ def test_per_key_mask_of_every_dtype_and_length(keys, dtype, mask_dtype, close):
     close(out, ref, dtype, what=f"per-key mask {keys} {mask.dtype}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("keys", [512, 1536])
+def test_padding_masks_in_the_model_dtype_drop_the_same_tiles(keys, dtype, close):
+    """A padding mask built in the model's dtype with `finfo(dtype).min` beyond the length (what transformers' mask
+    builders produce: -65504 for fp16) marks dead keys just as -inf in fp32 does: the key tiles it covers entirely are
+    not visited, and the result is bit for bit the one the fp32 -inf mask gives (and close to the oracle's)."""
+    B, H, D = 6, 12, 64
+    gen = torch.Generator().manual_seed(keys + 1)
+    q, k, v = (_mk((B, H, keys, D), dtype, gen) for _ in range(3))
+    lengths = torch.tensor([keys, keys // 2 + 3, 64, 65, keys - 1, 200])
+    visible = torch.arange(keys)[None, :] < lengths[:, None]
+    m32 = torch.where(visible, 0.0, float("-inf"))[:, None, None, :]
+    m16 = torch.where(visible, 0.0, torch.finfo(dtype).min).to(dtype)[:, None, None, :]
+    out32 = _run(q, k, v, 0.125, False, m32)
+    out16 = _run(q, k, v, 0.125, False, m16)
+    assert torch.equal(out32, out16)
+    close(out16, attention_oracle(q, k, v, 0.125, False, m16), dtype, what=f"model-dtype padding mask {keys} {dtype}")
+
+
 def test_attention_u02_inputs_like_reference(close):
     # reference draws q, k, v from U(0, 2) with sm_scale 0.3 (test/test_attention.py:91-99): large positive logits
     gen = torch.Generator().manual_seed(1)
