@@ -24,6 +24,9 @@ How each function is pinned (tests/test_oracle.py):
   rotary_oracle           equals rotary_complex_oracle (the reference's complex product) under the even/odd <-> half
                           permutation; zero angle = identity; angles add; quarter turn of a unit vector; norms kept
   rotary_complex_oracle   torch.view_as_complex product as in the reference; pinned by the same known answers
+  embedding_layer_norm_oracle  F.embedding + F.layer_norm with fp32 tables (nothing rounds between the additions); with
+                          fp16 tables, F.layer_norm of the sum formed by fp16 tensor additions; one table = plain lookup
+                          (tests/test_host_logic.py::test_embedding_oracle_against_the_library_routines)
 Nothing here is "parity unpinned".
 """
 import math
