@@ -209,7 +209,9 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
     // ---- key tiles: [0, n_clean) of the processing order need no masking, [n_clean, nt) take the general body
     const int n_end = CAUSAL ? min(N, q0 + BM + p.causal_off) : N;
     const int nt_all = (n_end + BN - 1) / BN;
-    constexpr bool MAY_LIST = (MASK_MODE == MASK_VECTOR && !CAUSAL);
+    // (causal with a per-key mask: tiles that reach beyond the diagonal of the workgroup's first row are never clean)
+    constexpr bool MAY_LIST = (MASK_MODE == MASK_VECTOR);
+    const int first_diag_key = CAUSAL ? q0 + p.causal_off : 0x7fffffff;  // keys above it are hidden from some row
     const bool use_list = WSPLIT || (MAY_LIST && nt_all <= 64);  // (the host hands WSPLIT at most 64 tiles)
     int nt = nt_all, n_clean = 0;
     if (MASK_MODE == MASK_NONE) n_clean = CAUSAL ? min(N / BN, (q0 + p.causal_off + 1) / BN) : N / BN;
@@ -244,8 +246,8 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                         const float sm = scale_mask(mv[j], p.clamp);
                         const bool any_nonzero = __ballot(valid && (sm != 0.0f)) != 0;
                         const bool any_normal = __ballot(valid && (sm > kDeadMask)) != 0;
-                        if (any_normal) {
-                            if (any_nonzero || t * BN + BN > N) gen_bits |= 1ull << t;
+                        if (any_normal || CAUSAL) {  // (causal: a row may see dead keys only — they are visited)
+                            if (any_nonzero || t * BN + BN > N || t * BN + BN - 1 > first_diag_key) gen_bits |= 1ull << t;
                             else clean_bits |= 1ull << t;
                         }
                     }
@@ -286,8 +288,8 @@ __global__ void __launch_bounds__(256, WPE) attention_stream_kernel(const AttnPa
                 const uint64_t bz = __ballot(nz), bn = __ballot(nm);
                 const int k = lane & 3, t = 4 * j + k;
                 const bool any_nz = ((bz >> (16 * k)) & 0xFFFFull) != 0, any_nm = ((bn >> (16 * k)) & 0xFFFFull) != 0;
-                const bool mine = lane < 4 && t < nt_all && any_nm;
-                const bool general = any_nz || t * BN + BN > N;
+                const bool mine = lane < 4 && t < nt_all && (any_nm || CAUSAL);  // (causal: a row may see dead keys only — they are visited)
+                const bool general = any_nz || t * BN + BN > N || t * BN + BN - 1 > first_diag_key;
                 clean_bits |= (__ballot(mine && !general) & 0xFull) << (4 * j);
                 gen_bits |= (__ballot(mine && general) & 0xFull) << (4 * j);
             };

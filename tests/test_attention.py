@@ -122,6 +122,24 @@ def test_padding_masks_in_the_model_dtype_drop_the_same_tiles(keys, dtype, close
     close(out16, attention_oracle(q, k, v, 0.125, False, m16), dtype, what=f"model-dtype padding mask {keys} {dtype}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+def test_causal_attention_with_left_padding(dtype, close):
+    """The causal flag together with a per-key padding mask whose hidden keys come FIRST (left-padded prompts): the rows
+    inside the padding see hidden keys only and get their plain average of V (the mask holds the most negative fp32
+    value, which absorbs every score), the rows behind it see the visible keys of their causal prefix — key tiles that
+    hold hidden keys only are still visited wherever a row depends on them."""
+    B, H, S, D = 4, 3, 512, 64
+    gen = torch.Generator().manual_seed(21)
+    q, k, v = (_mk((B, H, S, D), dtype, gen) for _ in range(3))
+    pad = torch.tensor([0, 70, 130, 511])
+    hidden = torch.arange(S)[None, :] < pad[:, None]
+    mask = torch.where(hidden, torch.finfo(torch.float32).min, 0.0)[:, None, None, :]
+    out = _run(q, k, v, 0.125, True, mask)
+    ref = attention_oracle(q, k, v, 0.125, True, mask)
+    assert torch.isfinite(out).all()
+    close(out, ref, dtype, what=f"causal + left padding {dtype}")
+
+
 def test_attention_u02_inputs_like_reference(close):
     # reference draws q, k, v from U(0, 2) with sm_scale 0.3 (test/test_attention.py:91-99): large positive logits
     gen = torch.Generator().manual_seed(1)
