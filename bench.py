@@ -564,8 +564,8 @@ def main():
     torch.cuda.synchronize()
     # The K timed steps are replayed from ONE hipGraph holding K launches (this is how the product path runs the
     # kernels — optimize_model replays a hipGraph — and it keeps the ~40 us of Python/ctypes work per eager call out
-    # of a ~40 us kernel's timing).  The replay is bracketed by a host clock (value) and by a HIP event pair on the
-    # stream the replay is launched on (average launch duration for the roofline).
+    # of a ~40 us kernel's timing).  One replay is bracketed by the host clock between two synchronisations (value), a
+    # second one by a HIP event pair on the stream the replay is launched on (average launch duration for the roofline).
     graph = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -584,14 +584,19 @@ def main():
     from_idle_launch_ms = evi0.elapsed_time(evi1) / args.steps
     # ... and, for the figures of the JSON line, after the power management has settled under this very load
     settle(graph.replay, args.settle_ms)
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # the K timed steps, by the host clock between two synchronisations ...
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    # ... and the same replay once more between two HIP events on the replay's stream (the kernel's average duration)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     ev0.record()
     graph.replay()
     ev1.record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
     avg_launch_ms = ev0.elapsed_time(ev1) / args.steps
     # eager launches with an event pair each, for comparison: these include the gap the host leaves between launches
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
